@@ -1,0 +1,133 @@
+/* khan_aev.h -- C ABI of libkhan_aev.so: the ANI-1 featurization path of proteneer/khan on one
+ * AMD MI355X (gfx950).
+ *
+ * Each entry point replaces one TensorFlow custom op of the reference's ani.so.  Arguments keep the
+ * reference's order, meaning and layout: every tensor is a flat, contiguous, rank-1 array; float
+ * tensors are float32 (_f32) or float64 (_f64); every index tensor is int32.  All pointers are
+ * DEVICE pointers unless the name ends in _host.  Work is enqueued on `stream` (a hipStream_t passed
+ * as void*; NULL is the default stream) and the call returns without synchronising.  The library
+ * keeps no state between calls, never frees or retains caller memory, and writes every element of
+ * every output (outputs need not be zeroed by the caller).
+ *
+ * Return value: KHAN_OK, or a KHAN_ERR_* code; khan_status_string() describes it.  Nothing here
+ * calls exit().  An empty batch (0 atoms, 0 molecules) is a successful no-op: the reference trainer
+ * feeds such batches (khan/training/trainer_multi_tower.py:795-817).
+ *
+ * Atom types are 0=H 1=C 2=N 3=O.  As in the reference (kernel_cpu.cpp:439-447) any other value is
+ * treated as O.
+ */
+#ifndef KHAN_AEV_H_
+#define KHAN_AEV_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KHAN_OK 0
+#define KHAN_ERR_INVALID_ARG 1   /* null pointer with non-empty input, negative size */
+#define KHAN_ERR_HIP 2           /* a HIP runtime call or kernel launch failed */
+#define KHAN_ERR_TOO_LARGE 3     /* size exceeds what int32 indices can address */
+
+typedef void *khan_stream_t;     /* hipStream_t */
+
+/* Width of one atomic-environment vector: 64 radial + 320 angular = 384.
+ * Replaces the `feature_size` attr of the Featurize op (gpu_featurizer/ani_op.cpp:108). */
+int32_t khan_feature_size(void);
+
+const char *khan_status_string(int status);
+
+/* Text of the last HIP error seen by the calling thread inside this library ("" if none). */
+const char *khan_last_hip_error(void);
+
+/* Featurization parameters for introspection (gpu_featurizer/parameters.h:61-114), host arrays:
+ * r_rs[16], a_thetas[8], a_rs[4], scalars[6] = {R_eta, R_Rc, A_Rc, A_eta, A_zeta, CHARGE_CONSTANT}. */
+void khan_get_parameters(float *r_rs_host, float *a_thetas_host, float *a_rs_host, float *scalars_host);
+
+/* mol_atom_counts = segment_sum(ones_like(mol_idxs), mol_idxs); mol_offsets = cumsum(exclusive).
+ * Replaces the two TensorFlow ops the reference trainer runs before AniSort
+ * (khan/training/trainer_multi_tower.py:302-303; gpu_featurizer/test_kernel.py:300-301).
+ * mol_idxs[n_atoms] must be sorted ascending with values in [0, n_mols). Outputs: macs[n_mols], mos[n_mols]. */
+int khan_mol_offsets(const int32_t *mol_idxs, int64_t n_atoms, int32_t n_mols, int32_t *macs,
+                     int32_t *mos, khan_stream_t stream);
+
+/* AniSort (gpu_featurizer/ani_sort.cpp:27-31 registration, 71-115 Compute).
+ * in : atomic_numbers[n_atoms]
+ * out: scatter_idxs[n_atoms]  rank of each atom among atoms of its own type
+ *      gather_idxs[n_atoms]   position of each atom under a stable sort by type
+ *      atom_counts[4]         atoms per type (DEVICE memory here; the reference op is host-only)
+ * Bit-identical to the reference's host algorithm. Allocates a small stream-ordered workspace. */
+int khan_ani_sort(const int32_t *atomic_numbers, int64_t n_atoms, int32_t *scatter_idxs,
+                  int32_t *gather_idxs, int32_t *atom_counts, khan_stream_t stream);
+
+/* Featurize (op: gpu_featurizer/ani_op.cpp:95-117; functor: functor_op.h:8-25, functor_op_gpu.cu:57-88;
+ * kernel: kernel_cpu.cpp:406-537 / kernel.cu:72-268).
+ * in : xs, ys, zs [n_atoms]; as [n_atoms]; mos, macs [n_mols]; sis = scatter_idxs [n_atoms];
+ *      acs_host[4] = atom_counts in HOST memory (the reference declares it HostMemory, ani_op.cpp:333)
+ * out: h_feat[acs[0]*384], c_feat[acs[1]*384], n_feat[acs[2]*384], o_feat[acs[3]*384], row-major;
+ *      the row of atom g is bucket[as[g]] + sis[g]*384. */
+int khan_featurize_f32(const float *xs, const float *ys, const float *zs, const int32_t *as,
+                       const int32_t *mos, const int32_t *macs, int32_t n_mols, const int32_t *sis,
+                       float *h_feat, float *c_feat, float *n_feat, float *o_feat,
+                       const int32_t *acs_host, khan_stream_t stream);
+int khan_featurize_f64(const double *xs, const double *ys, const double *zs, const int32_t *as,
+                       const int32_t *mos, const int32_t *macs, int32_t n_mols, const int32_t *sis,
+                       double *h_feat, double *c_feat, double *n_feat, double *o_feat,
+                       const int32_t *acs_host, khan_stream_t stream);
+
+/* FeaturizeGrad (op: gpu_featurizer/ani_op.cpp:200-221; functor: functor_op.h:27-47,
+ * functor_op_cpu.cpp:46-83; kernel: kernel_cpu.cpp:217-366 -- CPU-only in the reference).
+ * in : the Featurize inputs, then the upstream gradients h_grads..o_grads laid out like its outputs
+ * out: x_grads, y_grads, z_grads [sum(acs_host)] in original atom order. */
+int khan_featurize_grad_f32(const float *xs, const float *ys, const float *zs, const int32_t *as,
+                            const int32_t *mos, const int32_t *macs, int32_t n_mols,
+                            const int32_t *sis, const float *h_grads, const float *c_grads,
+                            const float *n_grads, const float *o_grads, float *x_grads,
+                            float *y_grads, float *z_grads, const int32_t *acs_host,
+                            khan_stream_t stream);
+int khan_featurize_grad_f64(const double *xs, const double *ys, const double *zs, const int32_t *as,
+                            const int32_t *mos, const int32_t *macs, int32_t n_mols,
+                            const int32_t *sis, const double *h_grads, const double *c_grads,
+                            const double *n_grads, const double *o_grads, double *x_grads,
+                            double *y_grads, double *z_grads, const int32_t *acs_host,
+                            khan_stream_t stream);
+
+/* AniCharge (gpu_featurizer/ani_charges.cpp:45-52 registration, 58-71 charge_energy, 81-119 Compute;
+ * CUDA twin ani_charges_gpu.cu:70-128).
+ * in : xs, ys, zs, qs [n_atoms]; mos, macs [n_mols]      out: charge_energies[n_mols] */
+int khan_ani_charge_f32(const float *xs, const float *ys, const float *zs, const float *qs,
+                        const int32_t *mos, const int32_t *macs, int32_t n_mols,
+                        float *charge_energies, khan_stream_t stream);
+int khan_ani_charge_f64(const double *xs, const double *ys, const double *zs, const double *qs,
+                        const int32_t *mos, const int32_t *macs, int32_t n_mols,
+                        double *charge_energies, khan_stream_t stream);
+
+/* AniChargeGrad (gpu_featurizer/ani_charges.cpp:123-131 registration, 138-160 charge_grads,
+ * 170-217 Compute; CUDA twin ani_charges_gpu.cu:197-260).
+ * in : the AniCharge inputs, then grads[n_mols] (upstream gradient per molecule)
+ * out: q_grads[n_atoms].  Atoms not covered by any molecule are left untouched. */
+int khan_ani_charge_grad_f32(const float *xs, const float *ys, const float *zs, const float *qs,
+                             const int32_t *mos, const int32_t *macs, int32_t n_mols,
+                             const float *grads, float *q_grads, khan_stream_t stream);
+int khan_ani_charge_grad_f64(const double *xs, const double *ys, const double *zs, const double *qs,
+                             const int32_t *mos, const int32_t *macs, int32_t n_mols,
+                             const double *grads, double *q_grads, khan_stream_t stream);
+
+/* Coordinate gradient of the charge energy.  No reference counterpart: the reference's registered
+ * gradient returns None for xs, ys, zs (khan/training/trainer_multi_tower.py:112-119).  Same inputs
+ * as AniChargeGrad; out: x_grads, y_grads, z_grads [n_atoms]; q_grads may be NULL to skip it. */
+int khan_ani_charge_grad_xyz_f32(const float *xs, const float *ys, const float *zs, const float *qs,
+                                 const int32_t *mos, const int32_t *macs, int32_t n_mols,
+                                 const float *grads, float *q_grads, float *x_grads, float *y_grads,
+                                 float *z_grads, khan_stream_t stream);
+int khan_ani_charge_grad_xyz_f64(const double *xs, const double *ys, const double *zs,
+                                 const double *qs, const int32_t *mos, const int32_t *macs,
+                                 int32_t n_mols, const double *grads, double *q_grads,
+                                 double *x_grads, double *y_grads, double *z_grads,
+                                 khan_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KHAN_AEV_H_ */

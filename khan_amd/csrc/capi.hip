@@ -1,0 +1,217 @@
+// extern "C" surface of libkhan_aev.so: argument checks and dispatch to the kernel launchers.
+#include <string>
+
+#include "../../include/khan_aev.h"
+#include "khan_internal.h"
+#include "khan_params.h"
+
+namespace {
+
+thread_local std::string g_last_hip_error;
+
+int hip_status(hipError_t e)
+{
+    if (e == hipSuccess) return KHAN_OK;
+    g_last_hip_error = hipGetErrorString(e);
+    return KHAN_ERR_HIP;
+}
+
+inline hipStream_t as_stream(khan_stream_t s) { return static_cast<hipStream_t>(s); }
+
+template <typename T>
+int featurize_impl(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
+                   const int32_t* macs, int32_t n_mols, const int32_t* sis, T* h, T* c, T* n, T* o,
+                   const int32_t* acs_host, khan_stream_t stream)
+{
+    if (n_mols < 0 || !acs_host) return KHAN_ERR_INVALID_ARG;
+    if (n_mols == 0) return KHAN_OK;
+    const int64_t n_atoms = static_cast<int64_t>(acs_host[0]) + acs_host[1] + acs_host[2] + acs_host[3];
+    if (acs_host[0] < 0 || acs_host[1] < 0 || acs_host[2] < 0 || acs_host[3] < 0) return KHAN_ERR_INVALID_ARG;
+    if (n_atoms == 0) return KHAN_OK;
+    if (!xs || !ys || !zs || !as || !mos || !macs || !sis) return KHAN_ERR_INVALID_ARG;
+    if ((acs_host[0] && !h) || (acs_host[1] && !c) || (acs_host[2] && !n) || (acs_host[3] && !o))
+        return KHAN_ERR_INVALID_ARG;
+    khan::Buckets<T> out{{h, c, n, o}};
+    return hip_status(khan::launch_fwd_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out, as_stream(stream)));
+}
+
+template <typename T>
+int featurize_grad_impl(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
+                        const int32_t* macs, int32_t n_mols, const int32_t* sis, const T* gh,
+                        const T* gc, const T* gn, const T* go, T* gx, T* gy, T* gz,
+                        const int32_t* acs_host, khan_stream_t stream)
+{
+    if (n_mols < 0 || !acs_host) return KHAN_ERR_INVALID_ARG;
+    if (acs_host[0] < 0 || acs_host[1] < 0 || acs_host[2] < 0 || acs_host[3] < 0) return KHAN_ERR_INVALID_ARG;
+    const int64_t n_atoms = static_cast<int64_t>(acs_host[0]) + acs_host[1] + acs_host[2] + acs_host[3];
+    if (n_atoms == 0) return KHAN_OK;
+    if (n_atoms > INT32_MAX) return KHAN_ERR_TOO_LARGE;
+    if (!gx || !gy || !gz) return KHAN_ERR_INVALID_ARG;
+    if (n_mols > 0 && (!xs || !ys || !zs || !as || !mos || !macs || !sis)) return KHAN_ERR_INVALID_ARG;
+    if ((acs_host[0] && !gh) || (acs_host[1] && !gc) || (acs_host[2] && !gn) || (acs_host[3] && !go))
+        return KHAN_ERR_INVALID_ARG;
+    khan::Buckets<const T> g{{gh, gc, gn, go}};
+    return hip_status(khan::launch_bwd_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                  n_atoms, as_stream(stream)));
+}
+
+template <typename T>
+int charge_impl(const T* xs, const T* ys, const T* zs, const T* qs, const int32_t* mos,
+                const int32_t* macs, int32_t n_mols, T* e, khan_stream_t stream)
+{
+    if (n_mols < 0) return KHAN_ERR_INVALID_ARG;
+    if (n_mols == 0) return KHAN_OK;
+    if (!xs || !ys || !zs || !qs || !mos || !macs || !e) return KHAN_ERR_INVALID_ARG;
+    return hip_status(khan::launch_charge_energy<T>(xs, ys, zs, qs, mos, macs, n_mols, e, as_stream(stream)));
+}
+
+template <typename T>
+int charge_grad_impl(const T* xs, const T* ys, const T* zs, const T* qs, const int32_t* mos,
+                     const int32_t* macs, int32_t n_mols, const T* grads, T* qg, T* gx, T* gy, T* gz,
+                     bool want_xyz, khan_stream_t stream)
+{
+    if (n_mols < 0) return KHAN_ERR_INVALID_ARG;
+    if (n_mols == 0) return KHAN_OK;
+    if (!xs || !ys || !zs || !qs || !mos || !macs || !grads) return KHAN_ERR_INVALID_ARG;
+    if (want_xyz ? (!gx || !gy || !gz) : !qg) return KHAN_ERR_INVALID_ARG;
+    return hip_status(khan::launch_charge_grad<T>(xs, ys, zs, qs, mos, macs, n_mols, grads, qg,
+                                                  want_xyz ? gx : nullptr, gy, gz, as_stream(stream)));
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t khan_feature_size(void) { return khan::kFeats; }
+
+const char* khan_status_string(int status)
+{
+    switch (status) {
+        case KHAN_OK: return "ok";
+        case KHAN_ERR_INVALID_ARG: return "invalid argument";
+        case KHAN_ERR_HIP: return "HIP runtime error";
+        case KHAN_ERR_TOO_LARGE: return "input too large for int32 indexing";
+        default: return "unknown status";
+    }
+}
+
+const char* khan_last_hip_error(void) { return g_last_hip_error.c_str(); }
+
+void khan_get_parameters(float* r_rs, float* a_thetas, float* a_rs, float* scalars)
+{
+    static const float rrs[16] = {5.0000000e-01f, 7.5625000e-01f, 1.0125000e+00f, 1.2687500e+00f,
+                                  1.5250000e+00f, 1.7812500e+00f, 2.0375000e+00f, 2.2937500e+00f,
+                                  2.5500000e+00f, 2.8062500e+00f, 3.0625000e+00f, 3.3187500e+00f,
+                                  3.5750000e+00f, 3.8312500e+00f, 4.0875000e+00f, 4.3437500e+00f};
+    static const float ath[8] = {0.0000000e+00f, 7.8539816e-01f, 1.5707963e+00f, 2.3561945e+00f,
+                                 3.1415927e+00f, 3.9269908e+00f, 4.7123890e+00f, 5.4977871e+00f};
+    static const float ars[4] = {5.0000000e-01f, 1.1500000e+00f, 1.8000000e+00f, 2.4500000e+00f};
+    for (int i = 0; i < 16; ++i) r_rs[i] = rrs[i];
+    for (int i = 0; i < 8; ++i) a_thetas[i] = ath[i];
+    for (int i = 0; i < 4; ++i) a_rs[i] = ars[i];
+    scalars[0] = khan::kR_eta_f;
+    scalars[1] = khan::kR_Rc_f;
+    scalars[2] = khan::kA_Rc_f;
+    scalars[3] = khan::kA_eta_f;
+    scalars[4] = 8.0f;
+    scalars[5] = khan::kChargeK_f;
+}
+
+int khan_mol_offsets(const int32_t* mol_idxs, int64_t n_atoms, int32_t n_mols, int32_t* macs,
+                     int32_t* mos, khan_stream_t stream)
+{
+    if (n_atoms < 0 || n_mols < 0) return KHAN_ERR_INVALID_ARG;
+    if (n_atoms > INT32_MAX) return KHAN_ERR_TOO_LARGE;
+    if (n_mols == 0) return KHAN_OK;
+    if (!macs || !mos || (n_atoms > 0 && !mol_idxs)) return KHAN_ERR_INVALID_ARG;
+    return hip_status(khan::launch_mol_offsets(mol_idxs, n_atoms, n_mols, macs, mos, as_stream(stream)));
+}
+
+int khan_ani_sort(const int32_t* atomic_numbers, int64_t n_atoms, int32_t* scatter_idxs,
+                  int32_t* gather_idxs, int32_t* atom_counts, khan_stream_t stream)
+{
+    if (n_atoms < 0 || !atom_counts) return KHAN_ERR_INVALID_ARG;
+    if (n_atoms > INT32_MAX) return KHAN_ERR_TOO_LARGE;
+    if (n_atoms > 0 && (!atomic_numbers || !scatter_idxs || !gather_idxs)) return KHAN_ERR_INVALID_ARG;
+    return hip_status(khan::launch_ani_sort(atomic_numbers, n_atoms, scatter_idxs, gather_idxs, atom_counts,
+                                            as_stream(stream)));
+}
+
+int khan_featurize_f32(const float* xs, const float* ys, const float* zs, const int32_t* as,
+                       const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
+                       float* h, float* c, float* n, float* o, const int32_t* acs_host,
+                       khan_stream_t stream)
+{
+    return featurize_impl<float>(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, stream);
+}
+int khan_featurize_f64(const double* xs, const double* ys, const double* zs, const int32_t* as,
+                       const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
+                       double* h, double* c, double* n, double* o, const int32_t* acs_host,
+                       khan_stream_t stream)
+{
+    return featurize_impl<double>(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, stream);
+}
+
+int khan_featurize_grad_f32(const float* xs, const float* ys, const float* zs, const int32_t* as,
+                            const int32_t* mos, const int32_t* macs, int32_t n_mols,
+                            const int32_t* sis, const float* gh, const float* gc, const float* gn,
+                            const float* go, float* gx, float* gy, float* gz,
+                            const int32_t* acs_host, khan_stream_t stream)
+{
+    return featurize_grad_impl<float>(xs, ys, zs, as, mos, macs, n_mols, sis, gh, gc, gn, go, gx, gy, gz,
+                                      acs_host, stream);
+}
+int khan_featurize_grad_f64(const double* xs, const double* ys, const double* zs, const int32_t* as,
+                            const int32_t* mos, const int32_t* macs, int32_t n_mols,
+                            const int32_t* sis, const double* gh, const double* gc, const double* gn,
+                            const double* go, double* gx, double* gy, double* gz,
+                            const int32_t* acs_host, khan_stream_t stream)
+{
+    return featurize_grad_impl<double>(xs, ys, zs, as, mos, macs, n_mols, sis, gh, gc, gn, go, gx, gy, gz,
+                                       acs_host, stream);
+}
+
+int khan_ani_charge_f32(const float* xs, const float* ys, const float* zs, const float* qs,
+                        const int32_t* mos, const int32_t* macs, int32_t n_mols, float* e,
+                        khan_stream_t stream)
+{
+    return charge_impl<float>(xs, ys, zs, qs, mos, macs, n_mols, e, stream);
+}
+int khan_ani_charge_f64(const double* xs, const double* ys, const double* zs, const double* qs,
+                        const int32_t* mos, const int32_t* macs, int32_t n_mols, double* e,
+                        khan_stream_t stream)
+{
+    return charge_impl<double>(xs, ys, zs, qs, mos, macs, n_mols, e, stream);
+}
+
+int khan_ani_charge_grad_f32(const float* xs, const float* ys, const float* zs, const float* qs,
+                             const int32_t* mos, const int32_t* macs, int32_t n_mols,
+                             const float* grads, float* q_grads, khan_stream_t stream)
+{
+    return charge_grad_impl<float>(xs, ys, zs, qs, mos, macs, n_mols, grads, q_grads, nullptr, nullptr,
+                                   nullptr, false, stream);
+}
+int khan_ani_charge_grad_f64(const double* xs, const double* ys, const double* zs, const double* qs,
+                             const int32_t* mos, const int32_t* macs, int32_t n_mols,
+                             const double* grads, double* q_grads, khan_stream_t stream)
+{
+    return charge_grad_impl<double>(xs, ys, zs, qs, mos, macs, n_mols, grads, q_grads, nullptr, nullptr,
+                                    nullptr, false, stream);
+}
+
+int khan_ani_charge_grad_xyz_f32(const float* xs, const float* ys, const float* zs, const float* qs,
+                                 const int32_t* mos, const int32_t* macs, int32_t n_mols,
+                                 const float* grads, float* q_grads, float* gx, float* gy, float* gz,
+                                 khan_stream_t stream)
+{
+    return charge_grad_impl<float>(xs, ys, zs, qs, mos, macs, n_mols, grads, q_grads, gx, gy, gz, true, stream);
+}
+int khan_ani_charge_grad_xyz_f64(const double* xs, const double* ys, const double* zs,
+                                 const double* qs, const int32_t* mos, const int32_t* macs,
+                                 int32_t n_mols, const double* grads, double* q_grads, double* gx,
+                                 double* gy, double* gz, khan_stream_t stream)
+{
+    return charge_grad_impl<double>(xs, ys, zs, qs, mos, macs, n_mols, grads, q_grads, gx, gy, gz, true, stream);
+}
+
+}  // extern "C"

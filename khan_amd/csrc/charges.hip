@@ -1,0 +1,130 @@
+// Damped-Coulomb charge energy and its gradients on gfx950.
+//
+// Reference: gpu_featurizer/ani_charges.cpp:58-71 (energy), 138-160 (dE/dq):
+//     E_m = sum_{i<j in m} K q_i q_j (1 - f_C(r_ij, R_Rc)) / r_ij,   K = 0.529176917f, R_Rc = 4.6f
+//     dL/dq_i = g_m * sum_{j != i} K q_j (1 - f_C(r_ij)) / r_ij
+// f_C(r) = 0.5 cos(pi r / Rc) + 0.5 for r <= Rc, else 0 (so pairs beyond Rc are plain K q q / r).
+// The coordinate gradient has no reference counterpart (the reference returns None for x, y, z,
+// khan/training/trainer_multi_tower.py:112-119); it is the closed form
+//     dL/dx_i = g_m K q_i sum_{j != i} q_j d/dr[(1 - f_C)/r] (x_i - x_j)/r.
+//
+// One wavefront per molecule, one lane per atom i (strided for molecules above 64 atoms); every lane
+// walks all partners j, whose loads are wave-uniform.  Each output element is written once by its
+// own lane: no atomics and no pre-zeroing.
+#include "khan_internal.h"
+#include "khan_params.h"
+
+namespace khan {
+
+namespace {
+
+template <typename T>
+__device__ __forceinline__ void pair_terms(T dx, T dy, T dz, T pi_rc, T rc, T& u, T& dudr_over_r)
+{
+    const T r = Real<T>::sqrt_(dx * dx + dy * dy + dz * dz);
+    T fc = T(0), dfc = T(0);
+    if (r <= rc) {
+        fc = cutoff_fn(r, pi_rc);
+        dfc = cutoff_dfn(r, pi_rc);
+    }
+    const T inv = T(1) / r;
+    u = (T(1) - fc) * inv;                            // (1 - f_C) / r
+    dudr_over_r = (-dfc * inv - u * inv) * inv;       // d/dr[(1-f_C)/r] / r
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void charge_energy_kernel(
+    const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
+    const T* __restrict__ Q, const int32_t* __restrict__ MOs, const int32_t* __restrict__ MACs,
+    int32_t n_mols, T* __restrict__ E)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t mol = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (mol >= n_mols) return;
+    const int n = MACs[mol], off = MOs[mol];
+    const T rc = static_cast<T>(kR_Rc_f), pi_rc = static_cast<T>(kPi / static_cast<double>(kR_Rc_f));
+    const T K = static_cast<T>(kChargeK_f);
+    T acc = T(0);
+    for (int i0 = 0; i0 < n; i0 += 64) {
+        const int i = i0 + lane;
+        const bool active = i < n;
+        const T xi = active ? X[off + i] : T(0), yi = active ? Y[off + i] : T(0),
+                zi = active ? Z[off + i] : T(0), qi = active ? Q[off + i] : T(0);
+        for (int j = i0 + 1; j < n; ++j) {
+            if (active && j > i) {
+                T u, du;
+                pair_terms(xi - X[off + j], yi - Y[off + j], zi - Z[off + j], pi_rc, rc, u, du);
+                acc += K * qi * Q[off + j] * u;
+            }
+        }
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) E[mol] = acc;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void charge_grad_kernel(
+    const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
+    const T* __restrict__ Q, const int32_t* __restrict__ MOs, const int32_t* __restrict__ MACs,
+    int32_t n_mols, const T* __restrict__ grads, T* __restrict__ q_grads, T* __restrict__ gX,
+    T* __restrict__ gY, T* __restrict__ gZ)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t mol = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (mol >= n_mols) return;
+    const int n = MACs[mol], off = MOs[mol];
+    const T rc = static_cast<T>(kR_Rc_f), pi_rc = static_cast<T>(kPi / static_cast<double>(kR_Rc_f));
+    const T gK = grads[mol] * static_cast<T>(kChargeK_f);
+    for (int i = lane; i < n; i += 64) {
+        const T xi = X[off + i], yi = Y[off + i], zi = Z[off + i], qi = Q[off + i];
+        T dq = T(0), fx = T(0), fy = T(0), fz = T(0);
+        for (int j = 0; j < n; ++j) {
+            if (j == i) continue;
+            const T dx = xi - X[off + j], dy = yi - Y[off + j], dz = zi - Z[off + j];
+            T u, du;
+            pair_terms(dx, dy, dz, pi_rc, rc, u, du);
+            const T qj = Q[off + j];
+            dq += qj * u;
+            const T w = qj * du;
+            fx += w * dx;
+            fy += w * dy;
+            fz += w * dz;
+        }
+        if (q_grads) q_grads[off + i] = gK * dq;
+        if (gX) {
+            gX[off + i] = gK * qi * fx;
+            gY[off + i] = gK * qi * fy;
+            gZ[off + i] = gK * qi * fz;
+        }
+    }
+}
+
+}  // namespace
+
+template <typename T>
+hipError_t launch_charge_energy(const T* X, const T* Y, const T* Z, const T* Q, const int32_t* MOs,
+                                const int32_t* MACs, int32_t n_mols, T* E, hipStream_t stream)
+{
+    if (n_mols <= 0) return hipSuccess;
+    const unsigned blocks = (static_cast<unsigned>(n_mols) + 3u) / 4u;
+    charge_energy_kernel<T><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, E);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_charge_grad(const T* X, const T* Y, const T* Z, const T* Q, const int32_t* MOs,
+                              const int32_t* MACs, int32_t n_mols, const T* grads, T* q_grads,
+                              T* gX, T* gY, T* gZ, hipStream_t stream)
+{
+    if (n_mols <= 0) return hipSuccess;
+    const unsigned blocks = (static_cast<unsigned>(n_mols) + 3u) / 4u;
+    charge_grad_kernel<T><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, q_grads, gX, gY, gZ);
+    return hipGetLastError();
+}
+
+template hipError_t launch_charge_energy<float>(const float*, const float*, const float*, const float*, const int32_t*, const int32_t*, int32_t, float*, hipStream_t);
+template hipError_t launch_charge_energy<double>(const double*, const double*, const double*, const double*, const int32_t*, const int32_t*, int32_t, double*, hipStream_t);
+template hipError_t launch_charge_grad<float>(const float*, const float*, const float*, const float*, const int32_t*, const int32_t*, int32_t, const float*, float*, float*, float*, float*, hipStream_t);
+template hipError_t launch_charge_grad<double>(const double*, const double*, const double*, const double*, const int32_t*, const int32_t*, int32_t, const double*, double*, double*, double*, double*, hipStream_t);
+
+}  // namespace khan

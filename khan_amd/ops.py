@@ -1,0 +1,192 @@
+"""Python mirror of the reference's custom ops, same names and argument orders as `ani_mod.<op>(...)`:
+
+    ani_sort(as)                                   gpu_featurizer/ani_sort.cpp:27-31
+    featurize(xs, ys, zs, as, mos, macs, sis, acs)                 ani_op.cpp:95-107
+    featurize_grad(..., acs, h_grads, c_grads, n_grads, o_grads)   ani_op.cpp:200-215
+    ani_charge(xs, ys, zs, qs, mos, macs)                          ani_charges.cpp:45-52
+    ani_charge_grad(xs, ys, zs, qs, mos, macs, grads)              ani_charges.cpp:123-131
+    mol_offsets(mol_idxs, n_mols)   the segment_sum + exclusive cumsum the trainer runs first
+                                    (khan/training/trainer_multi_tower.py:302-303)
+
+Tensors are torch CUDA tensors (PyTorch only owns the device memory and the stream); every op
+enqueues HIP kernels from libkhan_aev.so on the current stream.  Flat 1-D tensors in, flat 1-D tensors
+out, float32 or float64, int32 indices -- as in the reference.  There is no CPU implementation here.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+FEATURE_SIZE = 384
+
+_SUFFIX = {torch.float32: "f32", torch.float64: "f64"}
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev(t, dtype, name):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TypeError("%s must be a CUDA tensor" % name)
+    if t.dtype != dtype:
+        raise TypeError("%s must have dtype %s, got %s" % (name, dtype, t.dtype))
+    if t.dim() != 1:
+        raise ValueError("%s must be rank 1 (flat), got shape %s" % (name, tuple(t.shape)))
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous" % name)
+    return t
+
+
+def _p(t):
+    return ctypes.c_void_p(t.data_ptr() if t is not None and t.numel() > 0 else None)
+
+
+def _float_dtype(x):
+    if x.dtype not in _SUFFIX:
+        raise TypeError("coordinates must be float32 or float64, got %s" % x.dtype)
+    return x.dtype
+
+
+def _acs_host(acs):
+    """atom_counts lives in host memory in the reference (ani_op.cpp:333); a device tensor is copied."""
+    if isinstance(acs, torch.Tensor):
+        vals = [int(v) for v in acs.detach().cpu().tolist()]
+    else:
+        vals = [int(v) for v in acs]
+    if len(vals) != 4:
+        raise ValueError("acs must hold 4 atom counts")
+    return (ctypes.c_int32 * 4)(*vals), vals
+
+
+def mol_offsets(mol_idxs, n_mols):
+    """-> (mol_atom_counts, mol_offsets), both int32[n_mols]; mol_idxs sorted ascending."""
+    lib = _lib.load()
+    mol_idxs = _dev(mol_idxs, torch.int32, "mol_idxs")
+    macs = torch.empty(n_mols, dtype=torch.int32, device=mol_idxs.device)
+    mos = torch.empty(n_mols, dtype=torch.int32, device=mol_idxs.device)
+    _lib.check(lib.khan_mol_offsets(_p(mol_idxs), mol_idxs.numel(), n_mols, _p(macs), _p(mos), _stream()))
+    return macs, mos
+
+
+def ani_sort(atomic_numbers):
+    """-> (scatter_idxs, gather_idxs, atom_counts); atom_counts is an int32[4] DEVICE tensor."""
+    lib = _lib.load()
+    a = _dev(atomic_numbers, torch.int32, "atomic_numbers")
+    scatter = torch.empty_like(a)
+    gather = torch.empty_like(a)
+    counts = torch.empty(4, dtype=torch.int32, device=a.device)
+    _lib.check(lib.khan_ani_sort(_p(a), a.numel(), _p(scatter), _p(gather), _p(counts), _stream()))
+    return scatter, gather, counts
+
+
+def _check_common(xs, ys, zs, as_, mos, macs, sis):
+    dt = _float_dtype(xs)
+    _dev(xs, dt, "xs"); _dev(ys, dt, "ys"); _dev(zs, dt, "zs")
+    _dev(as_, torch.int32, "as"); _dev(mos, torch.int32, "mos"); _dev(macs, torch.int32, "macs")
+    _dev(sis, torch.int32, "sis")
+    n = xs.numel()
+    if not (ys.numel() == n and zs.numel() == n and as_.numel() == n and sis.numel() == n):
+        raise ValueError("xs, ys, zs, as, sis must have the same length")
+    if mos.numel() != macs.numel():
+        raise ValueError("mos and macs must have the same length")
+    return dt, n
+
+
+def featurize(xs, ys, zs, as_, mos, macs, sis, acs):
+    """-> (h_feat, c_feat, n_feat, o_feat), flat tensors of acs[t]*384 elements.
+
+    The four outputs are consecutive slices of one allocation, so
+    ``torch.cat([h, c, n, o]).view(-1, 384)[gather_idxs]`` needs no copy for the concatenation.
+    """
+    lib = _lib.load()
+    dt, n = _check_common(xs, ys, zs, as_, mos, macs, sis)
+    acs_c, acs_v = _acs_host(acs)
+    if sum(acs_v) != n:
+        raise ValueError("sum(acs)=%d does not match the number of atoms %d" % (sum(acs_v), n))
+    packed = torch.empty(n * FEATURE_SIZE, dtype=dt, device=xs.device)
+    outs, start = [], 0
+    for c in acs_v:
+        outs.append(packed[start * FEATURE_SIZE:(start + c) * FEATURE_SIZE])
+        start += c
+    fn = getattr(lib, "khan_featurize_" + _SUFFIX[dt])
+    _lib.check(fn(_p(xs), _p(ys), _p(zs), _p(as_), _p(mos), _p(macs), mos.numel(), _p(sis),
+                  _p(outs[0]), _p(outs[1]), _p(outs[2]), _p(outs[3]), acs_c, _stream()))
+    return tuple(outs)
+
+
+def featurize_grad(xs, ys, zs, as_, mos, macs, sis, acs, h_grads, c_grads, n_grads, o_grads):
+    """-> (x_grads, y_grads, z_grads), each [n_atoms] in original atom order."""
+    lib = _lib.load()
+    dt, n = _check_common(xs, ys, zs, as_, mos, macs, sis)
+    acs_c, acs_v = _acs_host(acs)
+    if sum(acs_v) != n:
+        raise ValueError("sum(acs)=%d does not match the number of atoms %d" % (sum(acs_v), n))
+    grads = []
+    for name, g, c in zip("hcno", (h_grads, c_grads, n_grads, o_grads), acs_v):
+        g = _dev(g.reshape(-1), dt, name + "_grads")
+        if g.numel() != c * FEATURE_SIZE:
+            raise ValueError("%s_grads has %d elements, expected %d" % (name, g.numel(), c * FEATURE_SIZE))
+        grads.append(g)
+    gx = torch.empty(n, dtype=dt, device=xs.device)
+    gy = torch.empty_like(gx)
+    gz = torch.empty_like(gx)
+    fn = getattr(lib, "khan_featurize_grad_" + _SUFFIX[dt])
+    _lib.check(fn(_p(xs), _p(ys), _p(zs), _p(as_), _p(mos), _p(macs), mos.numel(), _p(sis),
+                  _p(grads[0]), _p(grads[1]), _p(grads[2]), _p(grads[3]), _p(gx), _p(gy), _p(gz),
+                  acs_c, _stream()))
+    return gx, gy, gz
+
+
+def _check_charge(xs, ys, zs, qs, mos, macs):
+    dt = _float_dtype(xs)
+    for name, t in (("xs", xs), ("ys", ys), ("zs", zs), ("qs", qs)):
+        _dev(t, dt, name)
+    _dev(mos, torch.int32, "mos"); _dev(macs, torch.int32, "macs")
+    n = xs.numel()
+    if not (ys.numel() == n and zs.numel() == n and qs.numel() == n):
+        raise ValueError("xs, ys, zs, qs must have the same length")
+    if mos.numel() != macs.numel():
+        raise ValueError("mos and macs must have the same length")
+    return dt, n
+
+
+def ani_charge(xs, ys, zs, qs, mos, macs):
+    """-> charge_energies[n_mols]"""
+    lib = _lib.load()
+    dt, _ = _check_charge(xs, ys, zs, qs, mos, macs)
+    e = torch.empty(mos.numel(), dtype=dt, device=xs.device)
+    fn = getattr(lib, "khan_ani_charge_" + _SUFFIX[dt])
+    _lib.check(fn(_p(xs), _p(ys), _p(zs), _p(qs), _p(mos), _p(macs), mos.numel(), _p(e), _stream()))
+    return e
+
+
+def ani_charge_grad(xs, ys, zs, qs, mos, macs, grads):
+    """-> q_grads[n_atoms]"""
+    lib = _lib.load()
+    dt, n = _check_charge(xs, ys, zs, qs, mos, macs)
+    grads = _dev(grads, dt, "grads")
+    if grads.numel() != mos.numel():
+        raise ValueError("grads must have one element per molecule")
+    qg = torch.zeros(n, dtype=dt, device=xs.device)
+    fn = getattr(lib, "khan_ani_charge_grad_" + _SUFFIX[dt])
+    _lib.check(fn(_p(xs), _p(ys), _p(zs), _p(qs), _p(mos), _p(macs), mos.numel(), _p(grads), _p(qg), _stream()))
+    return qg
+
+
+def ani_charge_grad_xyz(xs, ys, zs, qs, mos, macs, grads):
+    """-> (q_grads, x_grads, y_grads, z_grads); the coordinate gradient is not offered by the reference."""
+    lib = _lib.load()
+    dt, n = _check_charge(xs, ys, zs, qs, mos, macs)
+    grads = _dev(grads, dt, "grads")
+    if grads.numel() != mos.numel():
+        raise ValueError("grads must have one element per molecule")
+    qg = torch.zeros(n, dtype=dt, device=xs.device)
+    gx = torch.zeros(n, dtype=dt, device=xs.device)
+    gy = torch.zeros_like(gx)
+    gz = torch.zeros_like(gx)
+    fn = getattr(lib, "khan_ani_charge_grad_xyz_" + _SUFFIX[dt])
+    _lib.check(fn(_p(xs), _p(ys), _p(zs), _p(qs), _p(mos), _p(macs), mos.numel(), _p(grads), _p(qg),
+                  _p(gx), _p(gy), _p(gz), _stream()))
+    return qg, gx, gy, gz
