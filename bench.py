@@ -1,0 +1,210 @@
+#!/usr/bin/env python3
+"""Benchmark of the ANI-1 featurization hot path on one MI355X.
+
+One "step" = one pass of the hot path over one synthetic batch that is already resident in HBM:
+    mol_offsets + ani_sort  ->  featurize (float32 forward)  ->  featurize_grad (float32 backward)
+on the 65,536-molecule organic batch (the configuration the headline metric is quoted on).
+Prints ONE JSON line: atoms/s for forward+gradient, with the roofline position of the dominant
+kernel and a CPU baseline (the reference's own CPU kernels compiled in place when available,
+else this repo's CPU port) timed on a bounded sample of the same batch.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload organic65536|organic1024|boxes4096]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+FP32_PEAK_TFLOPS = 157.3       # MI355X vector FP32, published
+FP64_PEAK_TFLOPS = 78.6
+
+WORKLOADS = {
+    "organic65536": ("organic", 65536),
+    "organic16384": ("organic", 16384),
+    "organic1024": ("organic", 1024),
+    "boxes4096": ("boxes", 4096),
+}
+
+
+def algorithmic_work(counts, n_atoms, n_mols, w):
+    """Contract figures: minimal flops / compulsory HBM bytes per pass (D, P_R, P_A, T = pair and
+    triple counts of the batch, w = bytes per float)."""
+    D, PR, PA, T = counts["D"], counts["P_R"], counts["P_A"], counts["T"]
+    return {
+        "flops_fwd": 9 * D + 100 * PR + 5 * PA + 150 * T,
+        "flops_bwd": 9 * D + 220 * PR + 8 * PA + 390 * T,
+        "bytes_fwd": n_atoms * (384 * w + 3 * w + 8) + 8 * n_mols,
+        "bytes_bwd": n_atoms * (384 * w + 3 * w + 8 + 3 * w) + 8 * n_mols,
+        "bytes_sort": n_atoms * (4 + 8) + 8 * n_mols + 4 * n_atoms,
+    }
+
+
+def cpu_baseline(batch, sample_mols_fwd, sample_mols_bwd):
+    """Forward+gradient float32 on the host, single thread, bounded sample (rank 0, N=1 only)."""
+    import numpy as np
+    from oracle import binding as ob
+    from khan_amd import datagen
+
+    have_ref = ob.ref_lib(fast=True) is not None
+    impl = "ref" if have_ref else "oracle"
+
+    def sub(n_mols):
+        b = datagen.make_batch(batch.kind, n_mols, seed=batch.seed)
+        sc, ga, ac = ob.ani_sort(b.A)
+        return b, sc, ac
+
+    b, sc, ac = sub(sample_mols_fwd)
+    t0 = time.perf_counter()
+    ob.featurize(b.X, b.Y, b.Z, b.A, b.MOs, b.MACs, sc, ac, dtype=np.float32, impl=impl, fast=True)
+    t_fwd = (time.perf_counter() - t0) / b.n_atoms
+    b2, sc2, ac2 = sub(sample_mols_bwd)
+    up = datagen.normal(b2.n_atoms * 384).reshape(-1, 384)
+    g = ob.scatter_rows(up, b2.A, sc2, ac2)
+    t0 = time.perf_counter()
+    ob.featurize_grad(b2.X, b2.Y, b2.Z, b2.A, b2.MOs, b2.MACs, sc2, ac2, g, dtype=np.float32, impl=impl, fast=True)
+    t_bwd = (time.perf_counter() - t0) / b2.n_atoms
+    return {
+        "value": 1.0 / (t_fwd + t_bwd),
+        "unit": "atoms/s",
+        "cores": 1,
+        "kind": "reference" if have_ref else "port",
+        "sample": "forward on the first %d molecules (%d atoms), gradient on the first %d molecules (%d atoms) "
+                  "of the same batch; per-atom times added; built -O3 -Ofast" % (
+                      sample_mols_fwd, b.n_atoms, sample_mols_bwd, b2.n_atoms),
+        "fwd_atoms_per_s": 1.0 / t_fwd,
+        "bwd_atoms_per_s": 1.0 / t_bwd,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="organic65536", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; the path shards by molecule with no exchange, "
+                 "but no multi-GPU launch is part of this run (got --gpus %d)" % args.gpus)
+
+    import numpy as np
+    import torch
+    from khan_amd import datagen, ops, _lib
+
+    _lib.load()   # fails loudly if the HIP library is missing
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    kind, n_mols = WORKLOADS[args.workload]
+    batch = datagen.make_batch(kind, n_mols)
+    N = batch.n_atoms
+    counts = batch.work_counts()
+    work = algorithmic_work(counts, N, n_mols, 4)
+
+    X, Y, Z = (torch.from_numpy(v).to(dev) for v in (batch.X, batch.Y, batch.Z))
+    A = torch.from_numpy(batch.A).to(dev)
+    mol_idxs = torch.from_numpy(batch.mol_idxs).to(dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1234)
+    upstream = torch.randn(N * 384, dtype=torch.float32, device=dev, generator=gen)   # dL/dAEV ~ N(0,1)
+    torch.cuda.synchronize()
+
+    ev = {k: [] for k in ("sort", "fwd", "bwd")}
+
+    def step(timed):
+        # events sit directly around each op, on the stream the kernels are launched on
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(6)] if timed else None
+        if timed:
+            marks[0].record()
+        macs, mos = ops.mol_offsets(mol_idxs, n_mols)
+        sc, ga, ac = ops.ani_sort(A)
+        if timed:
+            marks[1].record()
+        acs = ac.cpu()                       # atom_counts is a host-memory input of featurize
+        acs_l = acs.tolist()
+        grads, start = [], 0
+        for c in acs_l:
+            grads.append(upstream[start * 384:(start + c) * 384])
+            start += c
+        if timed:
+            marks[2].record()
+        feats = ops.featurize(X, Y, Z, A, mos, macs, sc, acs)
+        if timed:
+            marks[3].record()
+            marks[4].record()
+        gx, gy, gz = ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *grads)
+        if timed:
+            marks[5].record()
+        return marks, (feats, gx, gy, gz)
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    all_marks = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        m, out = step(True)
+        all_marks.append(m)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    for m in all_marks:
+        ev["sort"].append(m[0].elapsed_time(m[1]))
+        ev["fwd"].append(m[2].elapsed_time(m[3]))
+        ev["bwd"].append(m[4].elapsed_time(m[5]))
+    ms = {k: float(np.mean(v)) for k, v in ev.items()}      # event intervals on the launch stream
+    ms_per_step = elapsed / args.steps * 1e3
+
+    # dominant kernel = the longer of forward / backward; both bound by HBM when the arithmetic is minimal
+    dom = "bwd" if ms["bwd"] >= ms["fwd"] else "fwd"
+    dom_bytes = work["bytes_" + dom]
+    dom_flops = work["flops_" + dom]
+    achieved = dom_bytes / (ms[dom] * 1e-3) / 1e9
+    roofline = {
+        "kernel": "aev_bwd" if dom == "bwd" else "aev_fwd",
+        "bound": "hbm",
+        "achieved": achieved,
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": achieved / HBM_PEAK_GBS,
+        "traffic": None,
+        "launch_ms": ms[dom],
+        "algorithmic_bytes": dom_bytes,
+        "valu_frac_fp32": dom_flops / (ms[dom] * 1e-3) / 1e12 / FP32_PEAK_TFLOPS,
+        "fwd": {"ms": ms["fwd"], "hbm_frac": work["bytes_fwd"] / (ms["fwd"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                "valu_frac_fp32": work["flops_fwd"] / (ms["fwd"] * 1e-3) / 1e12 / FP32_PEAK_TFLOPS},
+        "bwd": {"ms": ms["bwd"], "hbm_frac": work["bytes_bwd"] / (ms["bwd"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                "valu_frac_fp32": work["flops_bwd"] / (ms["bwd"] * 1e-3) / 1e12 / FP32_PEAK_TFLOPS},
+        "sort_offsets_ms": ms["sort"],
+    }
+
+    result = {
+        "metric": "AEV fwd+grad atoms/sec, fp32, 1 MI355X",
+        "value": N / (ms_per_step * 1e-3),
+        "unit": "atoms/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "%s: ani_sort + AEV forward + AEV backward, %d molecules, %d atoms" % (
+            args.workload, n_mols, N), "n_mols": n_mols, "n_atoms": N, "work_counts": counts},
+        "molecules_per_s": n_mols / (ms_per_step * 1e-3),
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(batch, 1024 if kind == "organic" else 8, 256 if kind == "organic" else 2)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -92,13 +92,15 @@ def brute_force_aev(types, xyz):
 
 
 def brute_force_charge_energy(xyz, q):
-    """sum_{i<j} K q_i q_j (1 - f_C(r, R_Rc)) / r for one molecule, accumulated in long double."""
+    """sum_{i<j} K q_i q_j (1 - f_C(r, R_Rc)) / r for one molecule, accumulated in long double.
+    K and R_Rc are the float-rounded values the reference compiles in (parameters.h:10,72)."""
     xyz = np.asarray(xyz, dtype=np.float64)
+    k32, rc32 = float(np.float32(CHARGE_K)), float(np.float32(R_RC))
     e = np.longdouble(0)
     for i in range(len(q)):
         for j in range(i + 1, len(q)):
             r = float(np.linalg.norm(xyz[i] - xyz[j]))
-            e += np.longdouble(CHARGE_K * q[i] * q[j] * (1 - f_c(r, R_RC)) / r)
+            e += np.longdouble(k32 * q[i] * q[j] * (1 - f_c(r, rc32)) / r)
     return float(e)
 
 

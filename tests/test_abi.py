@@ -1,0 +1,115 @@
+"""Host-side checks that run without a GPU: the C-ABI library loads, exports every symbol that
+include/khan_aev.h declares, rejects bad arguments with status codes (never exits), and treats empty
+batches as successful no-ops.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from khan_amd import _lib, datagen
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "khan_aev.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(khan_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    lib = _lib.load()
+    names = declared_symbols()
+    assert len(names) >= 16
+    for name in names:
+        assert hasattr(lib, name), "libkhan_aev.so does not export " + name
+    assert set(names) == set(_lib.EXPORTED_SYMBOLS)
+
+
+def test_feature_size_and_parameters():
+    lib = _lib.load()
+    assert lib.khan_feature_size() == 384
+    r, t, a, s = ((ctypes.c_float * n)() for n in (16, 8, 4, 6))
+    lib.khan_get_parameters(r, t, a, s)
+    # gpu_featurizer/parameters.h:61-114
+    assert list(r)[:3] == [0.5, np.float32(0.75625), np.float32(1.0125)] and r[15] == np.float32(4.34375)
+    assert t[4] == np.float32(3.1415927) and list(a) == [np.float32(v) for v in (0.5, 1.15, 1.8, 2.45)]
+    assert list(s) == [16.0, np.float32(4.6), np.float32(3.1), 6.0, 8.0, np.float32(0.529176917)]
+
+
+def test_status_codes_without_touching_the_gpu():
+    lib = _lib.load()
+    assert lib.khan_status_string(0) == b"ok"
+    acs0 = (ctypes.c_int32 * 4)(0, 0, 0, 0)
+    acs = (ctypes.c_int32 * 4)(1, 0, 0, 0)
+    n = None
+    # empty batches: success, nothing launched (the reference trainer feeds them, trainer_multi_tower.py:795-817)
+    assert lib.khan_featurize_f32(n, n, n, n, n, n, 0, n, n, n, n, n, acs0, n) == 0
+    assert lib.khan_featurize_grad_f64(n, n, n, n, n, n, 0, n, n, n, n, n, n, n, n, acs0, n) == 0
+    assert lib.khan_ani_charge_f32(n, n, n, n, n, n, 0, n, n) == 0
+    assert lib.khan_mol_offsets(n, 0, 0, n, n, n) == 0
+    # invalid arguments: a status code, not a crash
+    assert lib.khan_featurize_f32(n, n, n, n, n, n, 1, n, n, n, n, n, acs, n) == 1
+    assert lib.khan_featurize_f32(n, n, n, n, n, n, -1, n, n, n, n, n, acs, n) == 1
+    assert lib.khan_featurize_f32(n, n, n, n, n, n, 1, n, n, n, n, n, None, n) == 1
+    assert lib.khan_featurize_grad_f32(n, n, n, n, n, n, 1, n, n, n, n, n, n, n, n, acs, n) == 1
+    assert lib.khan_ani_sort(n, 5, n, n, n, n) == 1
+    assert lib.khan_ani_sort(n, -1, n, n, n, n) == 1
+    assert lib.khan_ani_charge_grad_f64(n, n, n, n, n, n, 3, n, n, n) == 1
+    assert lib.khan_mol_offsets(n, 1 << 40, 1, n, n, n) == 3
+    assert b"invalid" in lib.khan_status_string(1)
+
+
+def test_ops_refuse_cpu_tensors():
+    torch = pytest.importorskip("torch")
+    from khan_amd import ops
+    with pytest.raises(TypeError):
+        ops.ani_sort(torch.zeros(4, dtype=torch.int32))
+
+
+def test_generator_is_seeded_prefix_stable_and_physical():
+    a = datagen.make_batch("organic", 200)
+    b = datagen.make_batch("organic", 50)
+    assert np.array_equal(a.X[:b.n_atoms], b.X) and np.array_equal(a.A[:b.n_atoms], b.A)
+    c = datagen.make_batch("organic", 50, first_mol=150)
+    assert np.array_equal(a.X[a.MOs[150]:], c.X)
+    assert a.MACs.min() >= 3 and a.MACs.max() <= 26
+    assert np.array_equal(a.MOs, np.concatenate([[0], np.cumsum(a.MACs)[:-1]]))
+    xyz = np.stack([a.X, a.Y, a.Z], axis=1).astype(np.float64)
+    valence = {0: 1, 1: 4, 2: 3, 3: 2}
+    for m in range(a.n_mols):
+        s = slice(a.MOs[m], a.MOs[m] + a.MACs[m])
+        d = np.linalg.norm(xyz[s, None] - xyz[None, s], axis=-1)
+        np.fill_diagonal(d, 10)
+        assert d.min() >= 0.8 - 1e-6
+        # hydrogens fill the valence: sum of valences is even and H count is consistent with a tree
+        heavy = a.A[s][a.A[s] > 0]
+        nh = int((a.A[s] == 0).sum())
+        assert nh == sum(valence[int(t)] for t in heavy) - 2 * (len(heavy) - 1)
+    frac = np.bincount(a.A[a.A > 0], minlength=4)[1:] / (a.A > 0).sum()
+    assert abs(frac[0] - 0.6) < 0.08 and abs(frac[1] - 0.2) < 0.06
+    w = b.work_counts()
+    assert w["D"] == int((b.MACs.astype(np.int64) * (b.MACs - 1)).sum()) and w["C"] * 2 == w["D"]
+    assert w["P_A"] <= w["P_R"] <= w["D"] and w["T"] > 0
+
+
+def test_box_generator_density_and_spacing():
+    b = datagen.make_batch("boxes", 3)
+    assert b.MACs.min() >= 64 and b.MACs.max() <= 256
+    xyz = np.stack([b.X, b.Y, b.Z], axis=1).astype(np.float64)
+    for m in range(3):
+        s = slice(b.MOs[m], b.MOs[m] + b.MACs[m])
+        side = (b.MACs[m] / 0.1) ** (1 / 3)
+        assert xyz[s].min() >= 0 and xyz[s].max() <= side + 1e-5
+        d = np.linalg.norm(xyz[s, None] - xyz[None, s], axis=-1)
+        np.fill_diagonal(d, 10)
+        assert d.min() >= 0.9 - 1e-6
+
+
+def test_normal_stream_is_position_keyed():
+    full = datagen.normal(5000, 0.3, datagen.TAG_CHARGES)
+    part = datagen.normal(1500, 0.3, datagen.TAG_CHARGES, first=2100)
+    assert np.array_equal(full[2100:3600], part)
+    assert abs(full.std() - 0.3) < 0.02 and abs(full.mean()) < 0.02

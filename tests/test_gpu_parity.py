@@ -1,0 +1,348 @@
+"""Parity of the HIP path (through the C ABI of libkhan_aev.so) with the CPU oracle, on a real MI355X.
+
+Tolerances (stated once, used everywhere below):
+  integers (sort, offsets)        bit-exact
+  float32 features                |gpu - ref| <= 1e-6 + 1e-5 |ref|, ref = float64 oracle
+                                  (and, against the float32 oracle, the same bound widened by the float32
+                                  oracle's own distance from the float64 one: the reference's float path
+                                  takes acos of a float, which alone moves some entries by > 1e-5 relative)
+  float64 features                |gpu - ref| <= 1e-15 + 1e-12 |ref|
+  gradients                       |gpu - ref| <= atol + rtol * max(|ref|, S), S = largest |component| of the
+                                  reference gradient in the same molecule (components are sums of terms of
+                                  both signs, so a tolerance relative to each component alone is not
+                                  meaningful); rtol = 1e-5, atol = 1e-6 in float32, rtol = 1e-12 in float64.
+                                  float32 gradients are judged against the float64 oracle: the reference's
+                                  own float functor is not finite everywhere (see test_oracle_featurize.py).
+  charges                         rtol as above relative to max(|ref|, largest |value| in the molecule).
+"""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+import helpers
+from khan_amd import datagen
+from oracle import binding as ob
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+F32_RTOL, F32_ATOL = 1e-5, 1e-6
+F64_RTOL, F64_ATOL = 1e-12, 1e-15
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    from khan_amd import ops as _ops
+    from khan_amd import _lib
+    _lib.load()      # fails loudly if the HIP library is missing
+    return _ops
+
+
+def dev(a, dtype=None):
+    a = np.ascontiguousarray(a if dtype is None else np.asarray(a).astype(dtype))
+    return torch.from_numpy(a).to("cuda:0")
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.detach().cpu().numpy()
+
+
+def mol_scale(ref, MOs, MACs):
+    """per-element scale S: largest |ref| inside the element's molecule (ref is [N] or [N,k])."""
+    ref = np.asarray(ref, dtype=np.float64)
+    flat = np.abs(ref.reshape(ref.shape[0], -1)).max(axis=1) if ref.shape[0] else np.zeros(0)
+    S = np.zeros(ref.shape[0])
+    for m in range(len(MOs)):
+        s = slice(MOs[m], MOs[m] + MACs[m])
+        if MACs[m] > 0:
+            S[s] = flat[s].max()
+    return S.reshape((-1,) + (1,) * (ref.ndim - 1))
+
+
+def assert_close(name, got, ref, rtol, atol, scale=None, slack=None):
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    assert got.shape == ref.shape, (name, got.shape, ref.shape)
+    assert np.all(np.isfinite(got)), name + ": non-finite output"
+    mag = np.abs(ref) if scale is None else np.maximum(np.abs(ref), scale)
+    bound = atol + rtol * mag
+    if slack is not None:
+        bound = bound + slack
+    err = np.abs(got - ref)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        ratio = np.where(bound > 0, err / bound, np.where(err == 0, 0.0, np.inf))   # bound 0: must be exact
+    worst = float(ratio.max()) if err.size else 0.0
+    say("   %-34s max|err| %.3e  worst err/bound %.3f" % (name, err.max() if err.size else 0.0, worst))
+    assert worst <= 1.0, "%s: err/bound %.3f" % (name, worst)
+
+
+class Case:
+    """A batch on the device plus oracle results, built lazily."""
+
+    def __init__(self, X, Y, Z, A, mol_idxs, n_mols):
+        self.X, self.Y, self.Z = (np.asarray(v, dtype=np.float32) for v in (X, Y, Z))
+        self.A = np.asarray(A, dtype=np.int32)
+        self.mol_idxs = np.asarray(mol_idxs, dtype=np.int32)
+        self.n_mols = n_mols
+        self.N = self.A.size
+        self.MACs, self.MOs = ob.mol_offsets(self.mol_idxs, n_mols)
+        self.sc, self.ga, self.ac = ob.ani_sort(self.A)
+
+    @classmethod
+    def from_batch(cls, b):
+        return cls(b.X, b.Y, b.Z, b.A, b.mol_idxs, b.n_mols)
+
+    def oracle_feat(self, dtype):
+        return ob.featurize(self.X, self.Y, self.Z, self.A, self.MOs, self.MACs, self.sc, self.ac, dtype=dtype)
+
+    def upstream(self, seed=11):
+        up = np.random.default_rng(seed).standard_normal((self.N, 384)).astype(np.float32).astype(np.float64)
+        return ob.scatter_rows(up, self.A, self.sc, self.ac)
+
+    def oracle_grad(self, upb):
+        return np.stack(ob.featurize_grad(self.X, self.Y, self.Z, self.A, self.MOs, self.MACs, self.sc, self.ac,
+                                          upb, dtype=np.float64), axis=1)
+
+
+def gpu_sort_offsets(ops, c):
+    macs, mos = ops.mol_offsets(dev(c.mol_idxs), c.n_mols)
+    sc, ga, ac = ops.ani_sort(dev(c.A))
+    return macs, mos, sc, ga, ac
+
+
+def check_forward_backward(ops, c, grad=True):
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+    assert np.array_equal(host(macs), c.MACs) and np.array_equal(host(mos), c.MOs)
+    assert np.array_equal(host(sc), c.sc) and np.array_equal(host(ga), c.ga) and np.array_equal(host(ac), c.ac)
+    acs = ac.cpu()
+    ref64 = np.concatenate(c.oracle_feat(np.float64))
+    ref32 = np.concatenate(c.oracle_feat(np.float32)).astype(np.float64)
+    upb = c.upstream() if grad else None
+    g64 = c.oracle_grad(upb) if grad else None
+    A = dev(c.A)
+    for tdt, ndt in ((torch.float32, np.float32), (torch.float64, np.float64)):
+        X, Y, Z = dev(c.X, ndt), dev(c.Y, ndt), dev(c.Z, ndt)
+        f = ops.featurize(X, Y, Z, A, mos, macs, sc, acs)
+        got = host(torch.cat(f))
+        if ndt == np.float32:
+            assert_close("features f32 vs f64 oracle", got, ref64, F32_RTOL, F32_ATOL)
+            assert_close("features f32 vs f32 oracle", got, ref32, F32_RTOL, F32_ATOL, slack=np.abs(ref32 - ref64))
+        else:
+            assert_close("features f64 vs f64 oracle", got, ref64, F64_RTOL, F64_ATOL)
+        if grad:
+            gb = [dev(x, ndt) for x in upb]
+            gx, gy, gz = ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *gb)
+            gg = host(torch.stack([gx, gy, gz], dim=1))
+            S = mol_scale(g64, c.MOs, c.MACs)
+            if ndt == np.float32:
+                assert_close("gradient f32 vs f64 oracle", gg, g64, F32_RTOL, F32_ATOL, scale=S)
+            else:
+                assert_close("gradient f64 vs f64 oracle", gg, g64, F64_RTOL, 0.0, scale=S)
+
+
+# ----------------------------------------------------------------------------- integers
+def test_sort_reference_kat(ops):
+    say("case: sort KAT, 11-atom fixture")
+    _, _, _, a, mi = helpers.fixture11()
+    sc, ga, ac = ops.ani_sort(dev(a))
+    assert host(ac).tolist() == helpers.FIXTURE11_ATOM_COUNTS
+    assert host(sc).tolist() == helpers.FIXTURE11_SCATTER
+    assert host(ga).tolist() == helpers.FIXTURE11_GATHER
+    macs, mos = ops.mol_offsets(dev(mi), 2)
+    assert host(macs).tolist() == [8, 3] and host(mos).tolist() == [0, 8]
+
+
+@pytest.mark.parametrize("n", [0, 1, 63, 64, 65, 255, 256, 257, 2047, 2048, 2049, 100003, 1 << 20])
+def test_sort_bit_exact_random(ops, n):
+    say("case: sort random n=%d" % n)
+    rng = np.random.default_rng(n)
+    a = rng.choice(4, size=n, p=[0.55, 0.3, 0.1, 0.05]).astype(np.int32)
+    sc, ga, ac = ops.ani_sort(dev(a))
+    osc, oga, oac = ob.ani_sort(a)
+    assert np.array_equal(host(ac), oac)
+    assert np.array_equal(host(sc), osc)
+    assert np.array_equal(host(ga), oga)
+
+
+def test_sort_single_type_and_out_of_range_types(ops):
+    say("case: sort single type / folded types")
+    a = np.full(5000, 1, dtype=np.int32)
+    sc, ga, ac = ops.ani_sort(dev(a))
+    assert host(ac).tolist() == [0, 5000, 0, 0] and np.array_equal(host(sc), np.arange(5000))
+    # types outside 0..3 are treated as O, like the reference featurizer's else-branch
+    a = np.array([0, 7, 3, -1, 1], dtype=np.int32)
+    sc, ga, ac = ops.ani_sort(dev(a))
+    osc, oga, oac = ob.ani_sort(np.array([0, 3, 3, 3, 1], dtype=np.int32))
+    assert np.array_equal(host(sc), osc) and np.array_equal(host(ga), oga) and np.array_equal(host(ac), oac)
+
+
+def test_mol_offsets_with_empty_molecules(ops):
+    say("case: mol_offsets with empty molecules")
+    rng = np.random.default_rng(2)
+    counts = rng.integers(0, 30, size=3000)
+    counts[[0, 5, 2999]] = 0
+    idx = np.repeat(np.arange(3000), counts).astype(np.int32)
+    macs, mos = ops.mol_offsets(dev(idx), 3000)
+    omacs, omos = ob.mol_offsets(idx, 3000)
+    assert np.array_equal(host(macs), omacs) and np.array_equal(host(mos), omos)
+    macs, mos = ops.mol_offsets(dev(np.zeros(0, np.int32)), 4)
+    assert host(macs).tolist() == [0] * 4 and host(mos).tolist() == [0] * 4
+
+
+# ----------------------------------------------------------------------------- golden vectors
+@pytest.mark.parametrize("prefix", ["fx11", "org8"])
+def test_golden_vectors(ops, golden_dir, prefix):
+    say("case: golden", prefix)
+    g = np.load(os.path.join(golden_dir, "aev_golden.npz"))
+    n_mols = int(g[prefix + "_macs"].size)
+    c = Case(g[prefix + "_X"], g[prefix + "_Y"], g[prefix + "_Z"], g[prefix + "_A"], g[prefix + "_mol_idxs"], n_mols)
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+    assert np.array_equal(host(sc), g[prefix + "_scatter"]) and np.array_equal(host(ga), g[prefix + "_gather"])
+    acs = ac.cpu()
+    A = dev(c.A)
+    up = g[prefix + "_upstream"]
+    for tdt, ndt, tag in ((torch.float32, np.float32, "f32"), (torch.float64, np.float64, "f64")):
+        X, Y, Z = dev(c.X, ndt), dev(c.Y, ndt), dev(c.Z, ndt)
+        f = ops.featurize(X, Y, Z, A, mos, macs, sc, acs)
+        rows = host(torch.cat(f).view(-1, 384)[ga.long()])
+        ref64 = g[prefix + "_feat_f64"]
+        if ndt == np.float32:
+            ref32 = g[prefix + "_feat_f32"].astype(np.float64)
+            assert_close("features f32 vs reference f64", rows, ref64, F32_RTOL, F32_ATOL)
+            assert_close("features f32 vs reference f32", rows, ref32, F32_RTOL, F32_ATOL, slack=np.abs(ref32 - ref64))
+        else:
+            assert_close("features f64 vs reference f64", rows, ref64, F64_RTOL, F64_ATOL)
+        gb = [dev(x, ndt) for x in ob.scatter_rows(up, c.A, c.sc, c.ac)]
+        gx, gy, gz = ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *gb)
+        gg = host(torch.stack([gx, gy, gz], dim=1))
+        gref = g[prefix + "_grad_f64"]
+        S = mol_scale(gref, c.MOs, c.MACs)
+        if ndt == np.float32:
+            assert_close("gradient f32 vs reference f64", gg, gref, F32_RTOL, F32_ATOL, scale=S)
+        else:
+            assert_close("gradient f64 vs reference f64", gg, gref, F64_RTOL, 0.0, scale=S)
+
+
+# ----------------------------------------------------------------------------- seeded batches
+def test_organic_batch(ops):
+    say("case: organic 1024 molecules (the reference-CPU-sized configuration)")
+    check_forward_backward(ops, Case.from_batch(datagen.make_batch("organic", 1024)))
+
+
+def test_dense_boxes(ops):
+    say("case: dense boxes, 6 boxes of 64-256 atoms")
+    check_forward_backward(ops, Case.from_batch(datagen.make_batch("boxes", 6)))
+
+
+def test_edge_shapes(ops):
+    say("case: ragged edge shapes")
+    rng = np.random.default_rng(9)
+    mols = []
+    # single atoms, a pair beyond every cutoff, a pair between the cutoffs, an empty molecule,
+    # one with 65 atoms and one with 300 atoms (more than a wavefront / more than four wavefronts)
+    mols.append((np.array([2]), np.zeros((1, 3))))
+    mols.append((np.array([0, 3]), np.array([[0, 0, 0], [0, 0, 5.0]])))
+    mols.append((np.array([1, 1]), np.array([[0, 0, 0], [0, 3.5, 0]])))
+    mols.append((np.zeros(0, dtype=int), np.zeros((0, 3))))
+    for n in (65, 300):
+        side = (n / 0.1) ** (1 / 3)
+        pts = []
+        while len(pts) < n:
+            p = rng.uniform(0, side, 3)
+            if all(np.linalg.norm(p - q) >= 0.9 for q in pts):
+                pts.append(p)
+        mols.append((rng.integers(0, 4, n), np.array(pts)))
+    mols.append((np.array([3]), np.ones((1, 3))))
+    A = np.concatenate([m[0] for m in mols]).astype(np.int32)
+    xyz = np.concatenate([m[1] for m in mols])
+    mi = np.concatenate([np.full(len(m[0]), k) for k, m in enumerate(mols)]).astype(np.int32)
+    check_forward_backward(ops, Case(xyz[:, 0], xyz[:, 1], xyz[:, 2], A, mi, len(mols)))
+
+
+def test_empty_batch(ops):
+    say("case: empty batch (0 atoms, 0 molecules)")
+    e32 = torch.empty(0, dtype=torch.float32, device="cuda:0")
+    ei = torch.empty(0, dtype=torch.int32, device="cuda:0")
+    sc, ga, ac = ops.ani_sort(ei)
+    assert host(ac).tolist() == [0, 0, 0, 0]
+    f = ops.featurize(e32, e32, e32, ei, ei, ei, sc, ac.cpu())
+    assert all(t.numel() == 0 for t in f)
+    g = ops.featurize_grad(e32, e32, e32, ei, ei, ei, sc, ac.cpu(), *f)
+    assert all(t.numel() == 0 for t in g)
+    assert ops.ani_charge(e32, e32, e32, e32, ei, ei).numel() == 0
+
+
+def test_out_of_range_type_goes_to_oxygen_bucket(ops):
+    say("case: atom type outside 0..3 is treated as O")
+    b = datagen.make_batch("organic", 4, first_mol=77)
+    A_bad = b.A.copy()
+    A_bad[b.A == 3] = 9
+    c = Case(b.X, b.Y, b.Z, b.A, b.mol_idxs, b.n_mols)
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+    X, Y, Z = dev(c.X), dev(c.Y), dev(c.Z)
+    good = host(torch.cat(ops.featurize(X, Y, Z, dev(b.A), mos, macs, sc, ac.cpu())))
+    bad = host(torch.cat(ops.featurize(X, Y, Z, dev(A_bad), mos, macs, sc, ac.cpu())))
+    assert np.array_equal(good, bad)
+
+
+# ----------------------------------------------------------------------------- charges
+@pytest.mark.parametrize("kind,n_mols", [("organic", 512), ("boxes", 4)])
+def test_charges(ops, kind, n_mols):
+    say("case: charges", kind, n_mols)
+    b = datagen.make_batch(kind, n_mols)
+    q = datagen.charges(b.n_atoms).astype(np.float64)
+    gm = np.random.default_rng(4).standard_normal(n_mols)
+    E64 = ob.ani_charge(b.X, b.Y, b.Z, q, b.MOs, b.MACs, dtype=np.float64)
+    dq64 = ob.ani_charge_grad(b.X, b.Y, b.Z, q, b.MOs, b.MACs, gm, dtype=np.float64)
+    dx64 = np.stack(ob.ani_charge_grad_xyz(b.X, b.Y, b.Z, q, b.MOs, b.MACs, gm, dtype=np.float64), axis=1)
+    # the energy is a sum of terms of both signs: scale = sum of |terms| per molecule = energy with |q|
+    Eabs = ob.ani_charge(b.X, b.Y, b.Z, np.abs(q), b.MOs, b.MACs, dtype=np.float64)
+    mos, macs = dev(b.MOs), dev(b.MACs)
+    for tdt, ndt, rtol in ((torch.float32, np.float32, F32_RTOL), (torch.float64, np.float64, F64_RTOL)):
+        X, Y, Z, Q, G = dev(b.X, ndt), dev(b.Y, ndt), dev(b.Z, ndt), dev(q, ndt), dev(gm, ndt)
+        E = host(ops.ani_charge(X, Y, Z, Q, mos, macs))
+        assert_close("charge energy %s" % ndt.__name__, E, E64, rtol, 0.0, scale=Eabs)
+        dq = host(ops.ani_charge_grad(X, Y, Z, Q, mos, macs, G))
+        assert_close("charge dE/dq %s" % ndt.__name__, dq, dq64, rtol, 0.0, scale=mol_scale(dq64, b.MOs, b.MACs))
+        qg, gx, gy, gz = ops.ani_charge_grad_xyz(X, Y, Z, Q, mos, macs, G)
+        assert np.array_equal(host(qg), dq)
+        dxyz = host(torch.stack([gx, gy, gz], dim=1))
+        assert_close("charge dE/dxyz %s" % ndt.__name__, dxyz, dx64, rtol, 0.0, scale=mol_scale(dx64, b.MOs, b.MACs))
+        # Euler: E is bilinear in q, so E = 1/2 sum_i q_i dE/dq_i (with unit upstream gradient)
+        ones = torch.ones(n_mols, dtype=tdt, device="cuda:0")
+        dq1 = host(ops.ani_charge_grad(X, Y, Z, Q, mos, macs, ones)).astype(np.float64)
+        euler = 0.5 * np.add.reduceat(np.asarray(q, ndt).astype(np.float64) * dq1, b.MOs)
+        assert_close("Euler identity %s" % ndt.__name__, euler, E.astype(np.float64), 10 * rtol, 0.0, scale=Eabs)
+
+
+def test_charge_reference_fixture_gradient_consistency(ops):
+    # the reference's only check of charges: dE/dq from the op agrees with a numeric derivative of the
+    # energy op (gpu_featurizer/test_kernel.py:403-459, delta 1e-3, tol 1e-11 in float64)
+    say("case: charges on the 11-atom fixture, numeric dE/dq")
+    x, y, z, a, mi = helpers.fixture11()
+    q = helpers.FIXTURE11_QS
+    X, Y, Z = dev(x), dev(y), dev(z)
+    mos, macs = dev(np.array([0, 8], np.int32)), dev(np.array([8, 3], np.int32))
+    ones = torch.ones(2, dtype=torch.float64, device="cuda:0")
+    dq = host(ops.ani_charge_grad(X, Y, Z, dev(q), mos, macs, ones))
+    delta = 1e-3
+    for i in range(11):
+        qp, qm = q.copy(), q.copy()
+        qp[i] += delta
+        qm[i] -= delta
+        ep = host(ops.ani_charge(X, Y, Z, dev(qp), mos, macs)).sum()
+        em = host(ops.ani_charge(X, Y, Z, dev(qm), mos, macs)).sum()
+        assert abs((ep - em) / (2 * delta) - dq[i]) < 1e-11
+    xyz = np.stack([x, y, z], axis=1)
+    for m, s in enumerate((slice(0, 8), slice(8, 11))):
+        e = host(ops.ani_charge(X, Y, Z, dev(q), mos, macs))[m]
+        assert e == pytest.approx(helpers.brute_force_charge_energy(xyz[s], q[s]), rel=1e-12)
