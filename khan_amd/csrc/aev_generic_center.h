@@ -1,0 +1,165 @@
+// Per-centre building blocks of the general-shape AEV kernels, shared by the general kernel and by
+// the small-molecule kernel (which falls back to them for centres that overflow its neighbour lists).
+#pragma once
+#include "khan_internal.h"
+#include "khan_params.h"
+
+namespace khan {
+
+template <typename T>
+struct LaneConsts {
+    T ct, st, ars;        // angular: cos/sin(theta_t), Rs_s of this lane's (t,s) slot
+    T rrs;                // radial: Rs of this lane's shell
+    int rtype;            // radial: partner type of this lane's slot
+    int ts, half;
+    T pi_rc_R, pi_rc_A, R_Rc, A_Rc, R_eta, A_eta;
+};
+
+template <typename T>
+__device__ __forceinline__ LaneConsts<T> lane_consts(int lane)
+{
+    LaneConsts<T> c;
+    c.ts = lane & 31;
+    c.half = lane >> 5;
+    const int t = c.ts >> 2, s = c.ts & 3;
+    c.ct = static_cast<T>(kCosTheta[t]);
+    c.st = static_cast<T>(kSinTheta[t]);
+    c.ars = static_cast<T>(kA_Rs_f[s]);
+    c.rrs = static_cast<T>(kR_Rs_f[lane & 15]);
+    c.rtype = lane >> 4;
+    c.R_Rc = static_cast<T>(kR_Rc_f);
+    c.A_Rc = static_cast<T>(kA_Rc_f);
+    c.R_eta = static_cast<T>(kR_eta_f);
+    c.A_eta = static_cast<T>(kA_eta_f);
+    c.pi_rc_R = static_cast<T>(kPi / static_cast<double>(kR_Rc_f));
+    c.pi_rc_A = static_cast<T>(kPi / static_cast<double>(kA_Rc_f));
+    return c;
+}
+
+// data of one scanned partner atom, held by the lane that scanned it
+template <typename T>
+struct Partner {
+    T dx, dy, dz, r;
+    int type;
+};
+
+template <typename T>
+__device__ __forceinline__ Partner<T> scan_partner(const T* X, const T* Y, const T* Z,
+                                                   const int32_t* A, int off, int j, int n, T xi,
+                                                   T yi, T zi)
+{
+    Partner<T> p;
+    p.dx = p.dy = p.dz = T(0);
+    p.r = T(1e30);
+    p.type = 0;
+    if (j < n) {
+        p.dx = xi - X[off + j];
+        p.dy = yi - Y[off + j];
+        p.dz = zi - Z[off + j];
+        p.r = Real<T>::sqrt_(p.dx * p.dx + p.dy * p.dy + p.dz * p.dz);
+        p.type = fold_type(A[off + j]);
+    }
+    return p;
+}
+
+template <typename T>
+__device__ __forceinline__ Partner<T> partner_from_lane(const Partner<T>& p, int src)
+{
+    Partner<T> q;
+    q.dx = wave_get(p.dx, src);
+    q.dy = wave_get(p.dy, src);
+    q.dz = wave_get(p.dz, src);
+    q.r = wave_get(p.r, src);
+    q.type = wave_get(p.type, src);
+    return q;
+}
+
+// Forward pass of ONE centre atom i of the molecule at [off, off+n), executed by one whole wavefront.
+// `ang` is kAngular elements of this wavefront's LDS; the finished 384-wide row is stored to `row`.
+template <typename T>
+__device__ __forceinline__ void fwd_center_generic(const LaneConsts<T>& L, int lane, const T* __restrict__ X,
+                                                   const T* __restrict__ Y, const T* __restrict__ Z,
+                                                   const int32_t* __restrict__ A, int off, int n, int i,
+                                                   T* ang, T* __restrict__ row)
+{
+        for (int q = lane; q < kAngular; q += 64) ang[q] = T(0);
+        wave_lds_fence();
+        const T xi = X[off + i], yi = Y[off + i], zi = Z[off + i];
+        T acc_rad = T(0);
+
+        for (int jc = 0; jc < n; jc += 64) {
+            const int j = jc + lane;
+            const Partner<T> pj = scan_partner(X, Y, Z, A, off, j, n, xi, yi, zi);
+            const bool valid = (j < n) && (j != i);
+            const bool inR = valid && (pj.r < L.R_Rc);
+            const bool inA = valid && (pj.r < L.A_Rc);
+            const T fcR = inR ? cutoff_fn(pj.r, L.pi_rc_R) : T(0);
+            const T fcA = inA ? cutoff_fn(pj.r, L.pi_rc_A) : T(0);
+
+            // radial: every partner inside R_Rc adds 16 shell values to the slots of its type
+            for (unsigned long long m = wave_ballot(inR); m; m &= m - 1) {
+                const int b = lowest_bit(m);
+                const T rb = wave_get(pj.r, b), fb = wave_get(fcR, b);
+                const int tb = wave_get(pj.type, b);
+                const T d = rb - L.rrs;
+                const T g = Real<T>::exp_(-L.R_eta * d * d) * fb;
+                acc_rad += (tb == L.rtype) ? g : T(0);
+            }
+
+            // angular: j from this chunk, k > j from this and later chunks
+            for (unsigned long long mj = wave_ballot(inA); mj; mj &= mj - 1) {
+                const int bj = lowest_bit(mj);
+                const Partner<T> J = partner_from_lane(pj, bj);
+                const T Jfc = wave_get(fcA, bj);
+                for (int kc = jc; kc < n; kc += 64) {
+                    Partner<T> pk;
+                    T fcK;
+                    bool kin;
+                    if (kc == jc) {
+                        pk = pj;
+                        fcK = fcA;
+                        kin = inA && (lane > bj);
+                    } else {
+                        const int k = kc + lane;
+                        pk = scan_partner(X, Y, Z, A, off, k, n, xi, yi, zi);
+                        kin = (k < n) && (k != i) && (pk.r < L.A_Rc);
+                        fcK = kin ? cutoff_fn(pk.r, L.pi_rc_A) : T(0);
+                    }
+                    unsigned long long mk = wave_ballot(kin);
+                    while (mk) {
+                        const int b0 = lowest_bit(mk);
+                        mk &= mk - 1;
+                        int b1 = -1;
+                        if (mk) {
+                            b1 = lowest_bit(mk);
+                            mk &= mk - 1;
+                        }
+                        const bool act = (L.half == 0) || (b1 >= 0);
+                        const int src = (L.half == 0 || b1 < 0) ? b0 : b1;
+                        const Partner<T> K = partner_from_lane(pk, src);
+                        const T Kfc = wave_get(fcK, src);
+
+                        const T inv = T(1) / (J.r * K.r);
+                        T c = (J.dx * K.dx + J.dy * K.dy + J.dz * K.dz) * inv;
+                        c = fmin(fmax(c, T(-1)), T(1));
+                        const T cx = J.dy * K.dz - J.dz * K.dy;
+                        const T cy = J.dz * K.dx - J.dx * K.dz;
+                        const T cz = J.dx * K.dy - J.dy * K.dx;
+                        const T s = Real<T>::sqrt_(cx * cx + cy * cy + cz * cz) * inv;
+                        const T base = T(1) + c * L.ct + s * L.st;
+                        const T b2 = base * base, b4 = b2 * b2, b8 = b4 * b4;
+                        const T dav = (J.r + K.r) * T(0.5) - L.ars;
+                        const T val = T(0.0078125) * b8 * Real<T>::exp_(-L.A_eta * dav * dav) * Jfc * Kfc;
+                        if (act) atomicAdd(&ang[pair_block(J.type, K.type) * kAngBlock + L.ts], val);
+                    }
+                }
+            }
+        }
+
+        wave_lds_fence();
+        row[lane] = acc_rad;
+        for (int q = lane; q < kAngular; q += 64) row[kRadial + q] = ang[q];
+        wave_lds_fence();
+}
+
+}  // namespace khan

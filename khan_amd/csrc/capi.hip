@@ -1,4 +1,5 @@
 // extern "C" surface of libkhan_aev.so: argument checks and dispatch to the kernel launchers.
+#include <cstdlib>
 #include <string>
 
 #include "../../include/khan_aev.h"
@@ -18,6 +19,37 @@ int hip_status(hipError_t e)
 
 inline hipStream_t as_stream(khan_stream_t s) { return static_cast<hipStream_t>(s); }
 
+// KHAN_AEV_FORCE_GENERIC=1 in the environment routes every molecule through the general-shape
+// kernels (read once; meant for A/B checks of the specialised kernels).
+bool force_generic()
+{
+    static const bool v = [] {
+        const char* e = getenv("KHAN_AEV_FORCE_GENERIC");
+        return e && e[0] == '1';
+    }();
+    return v;
+}
+
+int forward_dispatch(const float* xs, const float* ys, const float* zs, const int32_t* as,
+                     const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
+                     khan::Buckets<float> out, hipStream_t stream)
+{
+    if (force_generic())
+        return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, stream));
+    // molecules of up to 64 atoms: one wavefront each; the rest: general kernel
+    int st = hip_status(khan::launch_fwd_small_f32(xs, ys, zs, as, mos, macs, n_mols, sis, out, stream));
+    if (st != KHAN_OK) return st;
+    return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
+                                                      khan::kSmallMaxAtoms + 1, stream));
+}
+
+int forward_dispatch(const double* xs, const double* ys, const double* zs, const int32_t* as,
+                     const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
+                     khan::Buckets<double> out, hipStream_t stream)
+{
+    return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, stream));
+}
+
 template <typename T>
 int featurize_impl(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
                    const int32_t* macs, int32_t n_mols, const int32_t* sis, T* h, T* c, T* n, T* o,
@@ -32,7 +64,7 @@ int featurize_impl(const T* xs, const T* ys, const T* zs, const int32_t* as, con
     if ((acs_host[0] && !h) || (acs_host[1] && !c) || (acs_host[2] && !n) || (acs_host[3] && !o))
         return KHAN_ERR_INVALID_ARG;
     khan::Buckets<T> out{{h, c, n, o}};
-    return hip_status(khan::launch_fwd_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out, as_stream(stream)));
+    return forward_dispatch(xs, ys, zs, as, mos, macs, n_mols, sis, out, as_stream(stream));
 }
 
 template <typename T>

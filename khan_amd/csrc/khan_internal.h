@@ -15,7 +15,14 @@ struct Buckets {
 template <typename T>
 hipError_t launch_fwd_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
                               const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
-                              const int32_t* SIs, Buckets<T> out, hipStream_t stream);
+                              const int32_t* SIs, Buckets<T> out, int min_atoms, hipStream_t stream);
+
+// ---- AEV forward for molecules of up to 64 atoms, float32 (larger molecules are skipped) ----
+constexpr int kSmallMaxAtoms = 64;
+hipError_t launch_fwd_small_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
+                                const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                                const int32_t* SIs, Buckets<float> out, hipStream_t stream);
+
 template <typename T>
 hipError_t launch_bwd_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
                               const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
