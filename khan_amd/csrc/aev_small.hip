@@ -1,51 +1,53 @@
 // AEV forward for molecules of up to 64 atoms (float32): one wavefront per molecule.
 //
-// Layout of the work inside a wavefront
-//   * the molecule lives in registers, one atom per lane, lanes ordered by atom type (a 4-bin
-//     counting sort with ballots), so every neighbour list built in lane order is type-sorted and an
-//     unordered type pair (a<=b) owns a contiguous range of (j,k) pairs;
-//   * centres are taken six at a time.  For each centre the 64 lanes test all partners at once; the
-//     partners inside the radial cutoff go to a (r, f_C) list and the 64 lanes, as (type, shell)
-//     slots, walk their own type's part of that list: the radial 64 floats of the row are produced
-//     in registers and stored with one coalesced 256-byte store.  Partners inside the angular cutoff
-//     go to a per-centre list of unit vectors in LDS;
-//   * phase 1: the triples (centre; j<k) of the six centres are enumerated in (centre, type-pair)
-//     order, padded to even counts, and dealt one per lane.  A lane computes everything that depends
-//     on the triple alone -- the 8 angular factors (1+cos(theta-theta_t))^8 and the 4 radial factors
-//     2^-7 f_C f_C exp(-eta (rho-Rs_s)^2) -- 12 floats, written to LDS;
-//   * phase 2: lanes become (half, theta_t, Rs_s) slots.  The two halves take alternate records; a
-//     lane reads A_t and G_s of its record and does one FMA into a register accumulator.  When the
-//     (centre, type-pair) segment changes, the halves are added and the 32 values are stored straight
-//     to the row in HBM; empty segments are stored as zeros.  No atomics, no output pre-zeroing.
-//
-// A centre with more than 32 angular neighbours (not reachable with physical geometries: the angular
-// cutoff sphere of 3.1 A holds about 25 atoms at the densest packing seen) is redone by the
-// general-shape per-centre routine.  Semantics: gpu_featurizer/kernel_cpu.cpp:406-537.
+// How one wavefront spends its 64 lanes
+//   sort     one atom per lane, lanes reordered by atom type (4-bin counting sort with ballots).  Every
+//            neighbour list built in lane order is then type-sorted, so an unordered type pair (a<=b)
+//            owns a contiguous block of (j,k) pairs of a centre.
+//   scan     centres are taken six at a time.  A scan step tests 64 (centre, partner) pairs at once:
+//            4 centres x 16 partners for molecules of up to 16 atoms, 2 x 32 up to 32, 1 x 64 above.
+//            Partners inside the radial cutoff go to a (r, f_C) list, partners inside the angular
+//            cutoff to a per-centre list of unit vectors, both compacted with ballot + popcount.
+//   radial   lanes = (group of 16) x (shell): a group walks one centre's radial list type by type,
+//            four entries per trip, and stores 16 finished floats per (centre, type).
+//   phase 1  the triples (centre; j<k) of the six centres are enumerated in (centre, type-pair)
+//            order, each segment padded to an even length, and dealt one per lane.  A lane computes
+//            what depends on the triple alone: the 8 angular factors (1+cos(theta-theta_t))^8 and the
+//            4 radial factors 2^-7 f_C f_C exp(-eta (rho-Rs_s)^2).  12 floats go to LDS.
+//   phase 2  lanes = (half, theta_t, Rs_s).  The halves take alternate records; a lane reads A_t and
+//            G_s of its record and does one FMA into a register.  Segment boundaries are a bit mask
+//            held in scalar registers; at a boundary the halves are added and 32 floats are stored
+//            straight to the row in HBM.  Segments without triples are stored as zeros at the end.
+// No atomics and no pre-zeroed output.  A centre with more than 32 angular neighbours (the 3.1 A
+// sphere holds about 25 atoms at the densest packings tested) is redone by the general-shape
+// per-centre routine.  Semantics: gpu_featurizer/kernel_cpu.cpp:406-537.
 #include "aev_generic_center.h"
 
 namespace khan {
 
 namespace {
 
-constexpr int kB = 6;                          // centres per batch
-constexpr int kCapA = 32;                      // angular neighbours kept per centre
-constexpr int kSegLanes = kB * kNumPairBlocks; // 60 (centre, type-pair) segments per batch
+constexpr int kB = 6;          // centres per batch: 6 x 10 type pairs = 60 segment lanes
+constexpr int kCapA = 32;      // angular neighbours kept per centre
+constexpr int kBitWords = 96;  // 6 centres x (496 triples + padding) fit in 96 x 32 slot bits
 
 struct __align__(16) SegDesc {
     int start;       // first triple slot of the segment inside the batch (even)
-    int cnt;         // triples in the segment (the slot range is padded to an even length)
-    int packed;      // centre-in-batch | list offset of type a | offset of type b | n_a | a==b
+    int cnt;         // triples in the segment (its slot range is padded to an even length)
+    int packed;      // centre-in-batch | offset of type a | offset of type b | n_a | a==b | pair index
     float rcp_na;    // 1 / n_a
 };
 
 struct __align__(16) SmallLds {
-    float4 nbr[kB][kCapA];      // unit vector centre->partner (centre minus partner) and distance
+    float4 atom[64];            // x, y, z, type (sorted order)
+    float4 nbr[kB][kCapA];      // unit vector (centre minus partner)/r, and r
     float nbr_fc[kB][kCapA];    // f_C(r, A_Rc)
-    float2 rad[64];             // (r, f_C(r, R_Rc)) of the current centre's radial partners
+    float2 rad[64];             // (r, f_C(r, R_Rc)); group g of a scan step owns [g*W, (g+1)*W)
     float rec[64][12];          // phase-1 records: A_0..7, G_0..3
-    SegDesc seg[64];
-    int marker[64];
-    int nA[kB][4];              // angular partners per type, per centre
+    SegDesc seg[64];            // non-empty segments of the batch, in order
+    unsigned bits[kBitWords];   // bit per triple slot: a segment starts here
+    int nA[kB][4];              // angular partners per type, per centre of the batch
+    int nR[4][4];               // radial partners per type, per group of the scan step
 };
 
 __device__ __forceinline__ float lane_read(float v, int src_lane)
@@ -53,29 +55,29 @@ __device__ __forceinline__ float lane_read(float v, int src_lane)
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src_lane));
 }
 __device__ __forceinline__ int lane_read(int v, int src_lane) { return __builtin_amdgcn_readlane(v, src_lane); }
-
-__device__ __forceinline__ float lane_push(int dest_lane, float v)   // value lands in lane dest_lane
+__device__ __forceinline__ float lane_push(int dest_lane, float v)   // the value lands in lane dest_lane
 {
     return __int_as_float(__builtin_amdgcn_ds_permute(dest_lane << 2, __float_as_int(v)));
 }
 __device__ __forceinline__ int lane_push(int dest_lane, int v) { return __builtin_amdgcn_ds_permute(dest_lane << 2, v); }
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
-__device__ __forceinline__ int scan_add(int v, int lane)
+// Inclusive add-scan across the 64 lanes with data-parallel-primitive moves: four shifts inside each
+// row of 16 lanes, then lane 15 of rows 0,2 is carried into rows 1,3 and lane 31 into rows 2,3.
+// Lanes without a source take the identity 0.
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ int dpp_take(int v)
 {
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const int y = __shfl_up(v, d, 64);
-        if (lane >= d) v += y;
-    }
-    return v;
+    return __builtin_amdgcn_update_dpp(0, v, kCtrl, kRowMask, 0xf, false);
 }
-__device__ __forceinline__ int scan_max(int v, int lane)
+__device__ __forceinline__ int scan_add(int v)
 {
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const int y = __shfl_up(v, d, 64);
-        if (lane >= d) v = max(v, y);
-    }
+    v += dpp_take<0x111, 0xf>(v);   // row_shr:1
+    v += dpp_take<0x112, 0xf>(v);   // row_shr:2
+    v += dpp_take<0x114, 0xf>(v);   // row_shr:4
+    v += dpp_take<0x118, 0xf>(v);   // row_shr:8
+    v += dpp_take<0x142, 0xa>(v);   // row_bcast:15 into rows 1 and 3
+    v += dpp_take<0x143, 0xc>(v);   // row_bcast:31 into rows 2 and 3
     return v;
 }
 
@@ -84,10 +86,29 @@ __device__ __forceinline__ float pow8(float b)
     const float b2 = b * b, b4 = b2 * b2;
     return b4 * b4;
 }
-
 __device__ __forceinline__ int sel4(int a, int v0, int v1, int v2, int v3)
 {
     return a == 0 ? v0 : a == 1 ? v1 : a == 2 ? v2 : v3;
+}
+__device__ __forceinline__ int popc64(unsigned long long m) { return __popcll(m); }
+__device__ __forceinline__ unsigned long long low_bits(int w)   // w ones, 1 <= w <= 64
+{
+    return w >= 64 ? ~0ull : ((1ull << w) - 1ull);
+}
+
+// f_C(r, rc) = 0.5 cos(pi u) + 0.5 = cos^2(pi u / 2), u = r / rc in [0, 1).
+// With w = min(u, 1-u) and s = sin(pi w / 2) (odd minimax polynomial on [0, 0.5], |err| < 1.1e-7):
+// f_C = 1 - s^2 for u <= 0.5 and s^2 above, which keeps full relative accuracy where f_C -> 0.
+__device__ __forceinline__ float cutoff_poly(float u)
+{
+    const float w = fminf(u, 1.0f - u);
+    const float w2 = w * w;
+    float p = fmaf(w2, -0.00459228908981766f, 0.07967590297660462f);
+    p = fmaf(w2, p, -0.645962938168251f);
+    p = fmaf(w2, p, 1.5707963050854938f);
+    const float s = p * w;
+    const float q = s * s;
+    return (u <= 0.5f) ? 1.0f - q : q;
 }
 
 __global__ __launch_bounds__(256) void aev_fwd_small_kernel(
@@ -98,73 +119,86 @@ __global__ __launch_bounds__(256) void aev_fwd_small_kernel(
 {
     __shared__ SmallLds lds_all[4];
     const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave = uniform(threadIdx.x >> 6);
     const int mol = blockIdx.x * 4 + wave;
     if (mol >= n_mols) return;
-    const int n = __builtin_amdgcn_readfirstlane(MACs[mol]);
-    const int off = __builtin_amdgcn_readfirstlane(MOs[mol]);
+    const int n = uniform(MACs[mol]);
+    const int off = uniform(MOs[mol]);
     if (n <= 0 || n > 64) return;                 // larger molecules belong to the general kernel
     SmallLds& S = lds_all[wave];
     const LaneConsts<float> L = lane_consts<float>(lane);
-    const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    const unsigned long long lane_bit = 1ull << lane;
+    const unsigned long long lt_mask = lane_bit - 1ull;
 
-    // ---- one atom per lane, then lanes reordered by type
+    // ------------------------------------------------------------ load, sort lanes by type
     const bool have = lane < n;
     float x = 0.f, y = 0.f, z = 0.f;
     int type = 0, orig = lane;
-    float* rowp = nullptr;
+    unsigned long long rowbits = 0;
     if (have) {
         x = X[off + lane];
         y = Y[off + lane];
         z = Z[off + lane];
         type = fold_type(A[off + lane]);
-        rowp = out.p[type] + static_cast<size_t>(SIs[off + lane]) * kFeats;
+        rowbits = reinterpret_cast<unsigned long long>(out.p[type] + static_cast<size_t>(SIs[off + lane]) * kFeats);
     }
-    unsigned long long tmask[4];
     int tcount[4], tbase[4];
-#pragma unroll
-    for (int a = 0; a < 4; ++a) {
-        tmask[a] = wave_ballot(have && type == a);
-        tcount[a] = __popcll(tmask[a]);
-    }
-    tbase[0] = 0;
-    tbase[1] = tcount[0];
-    tbase[2] = tbase[1] + tcount[1];
-    tbase[3] = tbase[2] + tcount[2];
     int dest = lane;    // lanes without an atom keep their place, so the map is a permutation
-    if (have) {
-        const unsigned long long mine = type == 0 ? tmask[0] : type == 1 ? tmask[1] : type == 2 ? tmask[2] : tmask[3];
-        dest = sel4(type, tbase[0], tbase[1], tbase[2], tbase[3]) + __popcll(mine & lt_mask);
+    {
+        unsigned long long tmask[4];
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            tmask[a] = wave_ballot(have && type == a);
+            tcount[a] = popc64(tmask[a]);
+        }
+        tbase[0] = 0;
+        tbase[1] = tcount[0];
+        tbase[2] = tbase[1] + tcount[1];
+        tbase[3] = tbase[2] + tcount[2];
+        if (have) {
+            const unsigned long long mine = type == 0 ? tmask[0] : type == 1 ? tmask[1] : type == 2 ? tmask[2] : tmask[3];
+            dest = sel4(type, tbase[0], tbase[1], tbase[2], tbase[3]) + popc64(mine & lt_mask);
+        }
     }
     x = lane_push(dest, x);
     y = lane_push(dest, y);
     z = lane_push(dest, z);
     type = lane_push(dest, type);
     orig = lane_push(dest, orig);
-    {
-        const unsigned long long rp = reinterpret_cast<unsigned long long>(rowp);
-        const int lo = lane_push(dest, static_cast<int>(rp & 0xffffffffull));
-        const int hi = lane_push(dest, static_cast<int>(rp >> 32));
-        rowp = reinterpret_cast<float*>((static_cast<unsigned long long>(static_cast<unsigned>(hi)) << 32) |
-                                        static_cast<unsigned>(lo));
-    }
-    const int rp_lo = static_cast<int>(reinterpret_cast<unsigned long long>(rowp) & 0xffffffffull);
-    const int rp_hi = static_cast<int>(reinterpret_cast<unsigned long long>(rowp) >> 32);
-    // masks of the sorted lanes that hold each type
-    unsigned long long smask[4];
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-        smask[a] = (tcount[a] == 0) ? 0ull : ((tcount[a] >= 64 ? ~0ull : ((1ull << tcount[a]) - 1ull)) << tbase[a]);
-
-    auto row_of = [&](int sorted_lane) -> float* {
+    const int rp_lo = lane_push(dest, static_cast<int>(rowbits & 0xffffffffull));
+    const int rp_hi = lane_push(dest, static_cast<int>(rowbits >> 32));
+    S.atom[lane] = make_float4(x, y, z, __int_as_float(type));
+    auto row_of = [&](int sorted_lane) -> float* {     // sorted_lane is wave-uniform
         const unsigned lo = static_cast<unsigned>(lane_read(rp_lo, sorted_lane));
         const unsigned hi = static_cast<unsigned>(lane_read(rp_hi, sorted_lane));
         return reinterpret_cast<float*>((static_cast<unsigned long long>(hi) << 32) | lo);
     };
+    // sorted-order type ranges: partner index p has type a iff tbase[a] <= p < tbase[a] + tcount[a]
+    unsigned long long smask[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) smask[a] = (tcount[a] == 0) ? 0ull : (low_bits(tcount[a]) << tbase[a]);
 
-    // per-lane constants of the segment table: lane = centre-in-batch * 10 + type-pair index
+    // scan geometry: G centres x W partners per step
+    const int logW = n <= 16 ? 4 : n <= 32 ? 5 : 6;
+    const int W = 1 << logW, G = 64 >> logW;
+    const int grp = lane >> logW, jl = lane & (W - 1);
+    const unsigned long long sub_mask = low_bits(W) << ((grp * W) & 63);
+    const unsigned long long ltg_mask = lt_mask & sub_mask;
+    // count lanes: lane l < 16 counts partners of type (l & 3) for group (l >> 2)
+    const int cl_g = (lane >> 2) & 3, cl_a = lane & 3;
+    const bool cl_on = (lane < 16) && (cl_g < G);
+    const unsigned long long cl_sub = cl_on ? (low_bits(W) << ((cl_g * W) & 63)) : 0ull;
+    const unsigned long long cl_mask =
+        cl_on ? ((cl_a == 0 ? smask[0] : cl_a == 1 ? smask[1] : cl_a == 2 ? smask[2] : smask[3]) << ((cl_g * W) & 63)) : 0ull;
+    // radial lanes: 16-lane group rg, shell = lane & 15; the group serves centre group rg_g with
+    // entry slot rg_s out of rg_ns slots
+    const int rg = lane >> 4;
+    const int rg_ns = 4 / G;                                   // 1, 2 or 4
+    const int rg_g = G == 4 ? rg : G == 2 ? (rg >> 1) : 0;
+    const int rg_s = G == 4 ? 0 : G == 2 ? (rg & 1) : rg;
+
+    // segment-table lanes: lane = centre-in-batch * 10 + type-pair index (HH HC HN HO CC CN CO NN NO OO)
     const int seg_b = lane / kNumPairBlocks, seg_pt = lane - seg_b * kNumPairBlocks;
-    // type pair (a <= b) of pair index pt:  HH HC HN HO CC CN CO NN NO OO
     const int seg_a = seg_pt < 4 ? 0 : seg_pt < 7 ? 1 : seg_pt < 9 ? 2 : 3;
     const int seg_bt = seg_pt < 4 ? seg_pt : seg_pt < 7 ? seg_pt - 3 : seg_pt < 9 ? seg_pt - 5 : 3;
 
@@ -172,52 +206,83 @@ __global__ __launch_bounds__(256) void aev_fwd_small_kernel(
     const float kRadExp = -kR_eta_f * 1.44269504088896340736f;   // exp(-eta d^2) = exp2(kRadExp d^2)
     const float kAngExp = -kA_eta_f * 1.44269504088896340736f;
     const int ang_t = L.ts >> 2, ang_s = L.ts & 3;
+    wave_lds_fence();
 
     for (int c0 = 0; c0 < n; c0 += kB) {
         const int nb = min(kB, n - c0);
         unsigned overflow = 0;
 
-        // ------------------------------------------------ scan + radial part, centre by centre
-        for (int b = 0; b < nb; ++b) {
+        // ------------------------------------------------ scan steps: G centres x W partners
+        for (int b0 = 0; b0 < nb; b0 += G) {
+            const int b = b0 + grp;                      // centre-in-batch of this lane's group
             const int i = c0 + b;
-            const float dx = lane_read(x, i) - x, dy = lane_read(y, i) - y, dz = lane_read(z, i) - z;
+            const bool centre_ok = b < nb;
+            const float4 ai = S.atom[centre_ok ? i : 0];
+            const float4 aj = S.atom[jl];
+            const float dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
             const float r = sqrtf(dx * dx + dy * dy + dz * dz);
-            const bool valid = have && (lane != i);
+            const bool valid = centre_ok && (jl < n) && (jl != i);
             const bool inR = valid && (r < kR_Rc_f);
             const bool inA = valid && (r < kA_Rc_f);
             const unsigned long long mR = wave_ballot(inR), mA = wave_ballot(inA);
-            if (inR) S.rad[__popcll(mR & lt_mask)] = make_float2(r, 0.5f * cospif(r * inv_rc_R) + 0.5f);
-            const int cntA = __popcll(mA);
-            const bool fits = cntA <= kCapA;
-            if (!fits) overflow |= 1u << b;
+            const bool fits = popc64(mA & sub_mask) <= kCapA;
+            if (inR) S.rad[grp * W + popc64(mR & ltg_mask)] = make_float2(r, cutoff_poly(r * inv_rc_R));
             if (inA && fits) {
-                const int pos = __popcll(mA & lt_mask);
+                const int pos = popc64(mA & ltg_mask);
                 const float inv = __builtin_amdgcn_rcpf(r);
-                S.nbr[b][pos] = make_float4(dx * inv, dy * inv, dz * inv, r);
-                S.nbr_fc[b][pos] = 0.5f * cospif(r * inv_rc_A) + 0.5f;
+                S.nbr[centre_ok ? b : 0][pos] = make_float4(dx * inv, dy * inv, dz * inv, r);
+                S.nbr_fc[centre_ok ? b : 0][pos] = cutoff_poly(r * inv_rc_A);
             }
-            {
-                const int a0 = __popcll(mA & smask[0]), a1 = __popcll(mA & smask[1]),
-                          a2 = __popcll(mA & smask[2]), a3 = __popcll(mA & smask[3]);
-                if (lane < 4) S.nA[b][lane] = fits ? sel4(lane, a0, a1, a2, a3) : 0;
+            {   // bit b of `overflow`: centre b of the batch has too many angular partners
+                const unsigned long long ov = wave_ballot(!fits && jl == 0 && centre_ok);
+                for (int g = 0; g < G; ++g)
+                    if ((ov >> (g * W)) & 1ull) overflow |= 1u << (b0 + g);
             }
-            const int r0 = __popcll(mR & smask[0]), r1 = __popcll(mR & smask[1]),
-                      r2 = __popcll(mR & smask[2]), r3 = __popcll(mR & smask[3]);
+            int cntR = 0;
+            if (cl_on) {
+                const int cb = b0 + cl_g;
+                cntR = popc64(mR & cl_mask);
+                if (cb < nb) S.nA[cb][cl_a] = (popc64(mA & cl_sub) <= kCapA) ? popc64(mA & cl_mask) : 0;
+                S.nR[cl_g][cl_a] = cntR;
+            }
+            // largest radial count of each type over the groups of this step (lanes 0..15 hold them)
+            int mx = cntR;
+            mx = max(mx, __builtin_amdgcn_update_dpp(0, mx, 0x124, 0xf, 0xf, false));   // row_ror:4
+            mx = max(mx, __builtin_amdgcn_update_dpp(0, mx, 0x128, 0xf, 0xf, false));   // row_ror:8
+            const int mxR[4] = {lane_read(mx, 0), lane_read(mx, 1), lane_read(mx, 2), lane_read(mx, 3)};
             wave_lds_fence();
+
+            // ---- radial features of the G centres of this step
             {
-                // lane = (partner type, shell): walk this type's part of the radial list
-                const int my_n = sel4(L.rtype, r0, r1, r2, r3);
-                const int my_o = sel4(L.rtype, 0, r0, r0 + r1, r0 + r1 + r2);
-                const int max_n = max(max(r0, r1), max(r2, r3));
-                float acc_rad = 0.f;
-                for (int q = 0; q < max_n; ++q) {
-                    if (q < my_n) {
-                        const float2 e = S.rad[my_o + q];
-                        const float d = e.x - L.rrs;
-                        acc_rad += __builtin_amdgcn_exp2f(kRadExp * d * d) * e.y;
+                const int4 cn = *reinterpret_cast<const int4*>(S.nR[rg_g]);
+                const float2* list = &S.rad[rg_g * W];
+                const int cb = b0 + rg_g;
+                const int ci = min(c0 + cb, 63);
+                const unsigned rlo = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(ci << 2, rp_lo));
+                const unsigned rhi = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(ci << 2, rp_hi));
+                float* row = reinterpret_cast<float*>((static_cast<unsigned long long>(rhi) << 32) | rlo);
+                int obase = 0;
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    const int cnt_a = a == 0 ? cn.x : a == 1 ? cn.y : a == 2 ? cn.z : cn.w;
+                    float acc_r = 0.f;
+                    for (int q0 = 0; q0 < mxR[a]; q0 += 4 * rg_ns) {
+                        // four entries of this lane's slot per trip; slot s takes q = s, s+ns, s+2ns, ...
+                        float2 e[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) e[u] = list[min(obase + q0 + u * rg_ns + rg_s, W - 1)];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const float dd = e[u].x - L.rrs;
+                            const float v = __builtin_amdgcn_exp2f(kRadExp * dd * dd) * e[u].y;
+                            acc_r += (q0 + u * rg_ns + rg_s < cnt_a) ? v : 0.f;   // stale entries: select
+                        }
                     }
+                    if (rg_ns >= 2) acc_r += __shfl_xor(acc_r, 16, 64);
+                    if (rg_ns == 4) acc_r += __shfl_xor(acc_r, 32, 64);
+                    if (rg_s == 0 && cb < nb) row[a * kNumRRs + (lane & 15)] = acc_r;
+                    obase += cnt_a;
                 }
-                row_of(i)[lane] = acc_rad;
             }
             wave_lds_fence();
         }
@@ -233,49 +298,40 @@ __global__ __launch_bounds__(256) void aev_fwd_small_kernel(
             const int ob = sel4(seg_bt, 0, nn.x, nn.x + nn.y, nn.x + nn.y + nn.z);
             const bool same = seg_a == seg_bt;
             cnt = same ? (na * (na - 1)) / 2 : na * nbt;
-            packed = seg_b | (oa << 3) | (ob << 9) | (na << 15) | (same ? (1 << 21) : 0);
-            rcp_na = na > 0 ? 1.0f / static_cast<float>(na) : 0.f;
+            packed = seg_b | (oa << 3) | (ob << 9) | (na << 15) | (same ? (1 << 21) : 0) | (seg_pt << 22);
+            rcp_na = na > 0 ? __builtin_amdgcn_rcpf(static_cast<float>(na)) : 0.f;
         }
         const int padded = (cnt + 1) & ~1;
-        const int incl = scan_add(padded, lane);
+        const int incl = scan_add(padded);
         const int start = incl - padded;
         const int total = lane_read(incl, 63);            // triple slots in this batch (even)
-        {
+        const unsigned long long nonempty = wave_ballot(cnt > 0);
+        for (int w = lane; w < kBitWords; w += 64) S.bits[w] = 0u;
+        wave_lds_fence();
+        if (cnt > 0) {
             SegDesc d;
             d.start = start;
             d.cnt = cnt;
             d.packed = packed;
             d.rcp_na = rcp_na;
-            S.seg[lane] = d;
+            S.seg[popc64(nonempty & lt_mask)] = d;
+            atomicOr(&S.bits[start >> 5], 1u << (start & 31));
         }
         wave_lds_fence();
 
         // ------------------------------------------------ phases 1 and 2, 64 triple slots at a time
-        int cur = -1;          // segment whose sum is in `acc` (-1: none yet in this batch)
+        bool open = false;          // a segment's partial sums are in `acc`
         float acc = 0.f;
-        auto store_segment = [&](int sgi, float v) {
-            const int bb = sgi / kNumPairBlocks, pt = sgi - bb * kNumPairBlocks;
-            float* row = row_of(c0 + bb);
-            if (lane < 32) row[kRadial + pt * kAngBlock + lane] = v;
-        };
-        auto flush_until = [&](int next) {      // close `cur`, zero-fill the empty segments up to `next`
-            if (cur >= 0) store_segment(cur, acc + __shfl_xor(acc, 32, 64));
-            for (int s2 = cur + 1; s2 < next; ++s2) store_segment(s2, 0.f);
-        };
+        float* cur_row = nullptr;   // where the open segment's 32 floats go
+        int carry = 0;              // non-empty segments that start before this step
 
         for (int base = 0; base < total; base += 64) {
-            // which segment does each of the 64 slots belong to: segment starts are marked, then
-            // carried forward with a max-scan (segment ids grow with the slot index)
-            S.marker[lane] = 0;
-            wave_lds_fence();
-            if (cnt > 0) {
-                const int rel = start - base;
-                if (rel >= 0 && rel < 64) S.marker[rel] = lane + 1;
-                else if (rel < 0 && start + padded > base) S.marker[0] = lane + 1;
-            }
-            wave_lds_fence();
-            const int seg_of_lane = max(scan_max(S.marker[lane], lane) - 1, 0);
-            const SegDesc d = S.seg[seg_of_lane];
+            const unsigned w0 = static_cast<unsigned>(uniform(static_cast<int>(S.bits[base >> 5])));
+            const unsigned w1 = static_cast<unsigned>(uniform(static_cast<int>(S.bits[(base >> 5) + 1])));
+            const unsigned long long starts = (static_cast<unsigned long long>(w1) << 32) | w0;
+            const int ord = carry + popc64(starts & (lt_mask | lane_bit)) - 1;
+            carry += popc64(starts);
+            const SegDesc d = S.seg[max(ord, 0)];
             const int slot = base + lane;
             const int q = slot - d.start;
             const bool ok = (slot < total) && (q >= 0) && (q < d.cnt);
@@ -283,17 +339,17 @@ __global__ __launch_bounds__(256) void aev_fwd_small_kernel(
             // decode q -> (j,k) inside the centre's type-sorted list
             int bsel = d.packed & 7;
             const int oa = (d.packed >> 3) & 63, ob = (d.packed >> 9) & 63, na = (d.packed >> 15) & 63;
-            int kl, jl;
+            int kl, jl2;
             if ((d.packed >> 21) & 1) {                     // same type: pairs jl < kl, kl-major
                 kl = static_cast<int>((1.0f + __builtin_amdgcn_sqrtf(8.0f * static_cast<float>(q) + 1.0f)) * 0.5f);
                 if ((kl * (kl - 1)) / 2 > q) --kl;
                 if (((kl + 1) * kl) / 2 <= q) ++kl;
-                jl = q - (kl * (kl - 1)) / 2;
+                jl2 = q - (kl * (kl - 1)) / 2;
             } else {                                        // q = kl * n_a + jl
                 kl = static_cast<int>((static_cast<float>(q) + 0.5f) * d.rcp_na);
-                jl = q - kl * na;
+                jl2 = q - kl * na;
             }
-            int j = oa + jl, k = ob + kl;
+            int j = oa + jl2, k = ob + kl;
             if (!ok) {
                 j = 0;
                 k = 0;
@@ -330,22 +386,59 @@ __global__ __launch_bounds__(256) void aev_fwd_small_kernel(
             recp[2] = make_float4(Gf[0], Gf[1], Gf[2], Gf[3]);
             wave_lds_fence();
 
-            // phase 2: lane = (half, theta_t, Rs_s); the halves take alternate records
+            // phase 2: lane = (half, theta_t, Rs_s); the halves take alternate records.  Records past
+            // `total` in the last step are zeros, so whole groups of eight pairs can always be run.
             const int npairs = min(64, total - base) >> 1;
             const float* pa = &S.rec[L.half][ang_t];
             const float* pg = &S.rec[L.half][8 + ang_s];
-            for (int qq = 0; qq < npairs; ++qq) {
-                const int sg = lane_read(seg_of_lane, 2 * qq);
-                if (sg != cur) {
-                    flush_until(sg);
-                    cur = sg;
-                    acc = 0.f;
+            unsigned long long mm = starts;
+            for (int q0 = 0; q0 < npairs; q0 += 8) {
+                float av[8], gv[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    av[u] = pa[(q0 + u) * 24];
+                    gv[u] = pg[(q0 + u) * 24];
                 }
-                acc = fmaf(pa[qq * 24], pg[qq * 24], acc);
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    if (__builtin_expect(static_cast<int>(mm & 1ull), 0)) {
+                        // a segment starts at record pair q0+u: close the open one, open the new one
+                        if (open) {
+                            const float tot = acc + __shfl_xor(acc, 32, 64);
+                            if (lane < 32) cur_row[lane] = tot;
+                        }
+                        const int pk = lane_read(d.packed, 2 * (q0 + u));
+                        cur_row = row_of(c0 + (pk & 7)) + kRadial + ((pk >> 22) & 15) * kAngBlock;
+                        open = true;
+                        acc = 0.f;
+                    }
+                    mm >>= 2;
+                    acc = fmaf(av[u], gv[u], acc);
+                }
             }
             wave_lds_fence();
         }
-        flush_until(nb * kNumPairBlocks);
+        if (open) {
+            const float tot = acc + __shfl_xor(acc, 32, 64);
+            if (lane < 32) cur_row[lane] = tot;
+        }
+
+        // ------------------------------------------------ segments without triples are zeros
+        {
+            const unsigned long long empty = ~nonempty;
+            for (int b = 0; b < nb; ++b) {
+                const unsigned eb = static_cast<unsigned>(empty >> (b * kNumPairBlocks)) & 0x3ffu;
+                if (eb == 0u) continue;
+                float* row = row_of(c0 + b) + kRadial;
+#pragma unroll
+                for (int pp = 0; pp < 5; ++pp) {
+                    if (((eb >> (2 * pp)) & 3u) != 0u) {
+                        const int pt = 2 * pp + L.half;
+                        if ((eb >> pt) & 1u) row[pt * kAngBlock + L.ts] = 0.f;
+                    }
+                }
+            }
+        }
 
         // ------------------------------------------------ centres whose list overflowed
         if (overflow) {
@@ -357,6 +450,7 @@ __global__ __launch_bounds__(256) void aev_fwd_small_kernel(
                                               reinterpret_cast<float*>(S.rec), row_of(c0 + b));
                 }
             }
+            wave_lds_fence();
         }
     }
 }
