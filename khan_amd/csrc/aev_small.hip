@@ -62,6 +62,21 @@ __device__ __forceinline__ float lane_push(int dest_lane, float v)   // the valu
 __device__ __forceinline__ int lane_push(int dest_lane, int v) { return __builtin_amdgcn_ds_permute(dest_lane << 2, v); }
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
+// Row pointers are rebuilt from two 32-bit lane reads; storing through an explicit global-address-space
+// pointer keeps the stores on the global (not the flat) path.
+typedef float __attribute__((address_space(1))) global_float;
+__device__ __forceinline__ void store_global(float* p, float v)
+{
+    *((global_float*)(p)) = v;
+}
+// sum of the two half-waves, in every lane: swap the upper half of one copy with the lower half of
+// the other (one cross-lane VALU move, no LDS round trip), then add
+__device__ __forceinline__ float half_wave_sum(float v)
+{
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_int(v), __float_as_int(v), false, false);
+    return __int_as_float(r[0]) + __int_as_float(r[1]);
+}
+
 // Inclusive add-scan across the 64 lanes with data-parallel-primitive moves: four shifts inside each
 // row of 16 lanes, then lane 15 of rows 0,2 is carried into rows 1,3 and lane 31 into rows 2,3.
 // Lanes without a source take the identity 0.
@@ -280,7 +295,7 @@ __global__ __launch_bounds__(256) void aev_fwd_small_kernel(
                     }
                     if (rg_ns >= 2) acc_r += __shfl_xor(acc_r, 16, 64);
                     if (rg_ns == 4) acc_r += __shfl_xor(acc_r, 32, 64);
-                    if (rg_s == 0 && cb < nb) row[a * kNumRRs + (lane & 15)] = acc_r;
+                    if (rg_s == 0 && cb < nb) store_global(row + a * kNumRRs + (lane & 15), acc_r);
                     obase += cnt_a;
                 }
             }
@@ -392,20 +407,21 @@ __global__ __launch_bounds__(256) void aev_fwd_small_kernel(
             const float* pa = &S.rec[L.half][ang_t];
             const float* pg = &S.rec[L.half][8 + ang_s];
             unsigned long long mm = starts;
-            for (int q0 = 0; q0 < npairs; q0 += 8) {
-                float av[8], gv[8];
+            auto load8 = [&](int q0, float (&av)[8], float (&gv)[8]) {
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
                     av[u] = pa[(q0 + u) * 24];
                     gv[u] = pg[(q0 + u) * 24];
                 }
+            };
+            auto run8 = [&](int q0, const float (&av)[8], const float (&gv)[8]) {
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
                     if (__builtin_expect(static_cast<int>(mm & 1ull), 0)) {
                         // a segment starts at record pair q0+u: close the open one, open the new one
                         if (open) {
-                            const float tot = acc + __shfl_xor(acc, 32, 64);
-                            if (lane < 32) cur_row[lane] = tot;
+                            const float tot = half_wave_sum(acc);
+                            if (lane < 32) store_global(cur_row + lane, tot);
                         }
                         const int pk = lane_read(d.packed, 2 * (q0 + u));
                         cur_row = row_of(c0 + (pk & 7)) + kRadial + ((pk >> 22) & 15) * kAngBlock;
@@ -415,12 +431,24 @@ __global__ __launch_bounds__(256) void aev_fwd_small_kernel(
                     mm >>= 2;
                     acc = fmaf(av[u], gv[u], acc);
                 }
+            };
+            // eight record pairs per group, the next group's LDS reads in flight while one is summed
+            float a0[8], g0[8], a1[8], g1[8];
+            load8(0, a0, g0);
+            for (int q0 = 0; q0 < npairs; q0 += 16) {
+                const bool more1 = q0 + 8 < npairs;
+                if (more1) load8(q0 + 8, a1, g1);
+                run8(q0, a0, g0);
+                if (more1) {
+                    if (q0 + 16 < npairs) load8(q0 + 16, a0, g0);
+                    run8(q0 + 8, a1, g1);
+                }
             }
             wave_lds_fence();
         }
         if (open) {
-            const float tot = acc + __shfl_xor(acc, 32, 64);
-            if (lane < 32) cur_row[lane] = tot;
+            const float tot = half_wave_sum(acc);
+            if (lane < 32) store_global(cur_row + lane, tot);
         }
 
         // ------------------------------------------------ segments without triples are zeros
@@ -434,7 +462,7 @@ __global__ __launch_bounds__(256) void aev_fwd_small_kernel(
                 for (int pp = 0; pp < 5; ++pp) {
                     if (((eb >> (2 * pp)) & 3u) != 0u) {
                         const int pt = 2 * pp + L.half;
-                        if ((eb >> pt) & 1u) row[pt * kAngBlock + L.ts] = 0.f;
+                        if ((eb >> pt) & 1u) store_global(row + pt * kAngBlock + L.ts, 0.f);
                     }
                 }
             }
