@@ -162,4 +162,144 @@ __device__ __forceinline__ void fwd_center_generic(const LaneConsts<T>& L, int l
         wave_lds_fence();
 }
 
+// Backward pass of ONE centre atom i (general shape), executed by one whole wavefront: adds
+// dL/dxyz of every atom touched by centre i's row through `add(atom, fx, fy, fz)`, where `atom` is
+// the index inside the molecule.  `g_ang` is kAngular elements of this wavefront's LDS and `grow` the
+// centre's upstream 384-wide row.  Reference: kernel_cpu.cpp:217-366.
+template <typename T, typename AddForce>
+__device__ __forceinline__ void bwd_center_generic(const LaneConsts<T>& L, int lane, const T* __restrict__ X,
+                                                   const T* __restrict__ Y, const T* __restrict__ Z,
+                                                   const int32_t* __restrict__ A, int off, int n, int i,
+                                                   T* g_ang, const T* __restrict__ grow, AddForce add)
+{
+        const T g_rad = grow[lane];                       // upstream for slot (rtype, shell)
+        for (int q = lane; q < kAngular; q += 64) g_ang[q] = grow[kRadial + q];
+        wave_lds_fence();
+        const T xi = X[off + i], yi = Y[off + i], zi = Z[off + i];
+        T ix = T(0), iy = T(0), iz = T(0);   // gradient on i: per-half partials, summed at the end
+
+        for (int jc = 0; jc < n; jc += 64) {
+            const int j = jc + lane;
+            const Partner<T> pj = scan_partner(X, Y, Z, A, off, j, n, xi, yi, zi);
+            const bool valid = (j < n) && (j != i);
+            const bool inR = valid && (pj.r < L.R_Rc);
+            const bool inA = valid && (pj.r < L.A_Rc);
+            const T fcR = inR ? cutoff_fn(pj.r, L.pi_rc_R) : T(0);
+            const T dfcR = inR ? cutoff_dfn(pj.r, L.pi_rc_R) : T(0);
+            const T fcA = inA ? cutoff_fn(pj.r, L.pi_rc_A) : T(0);
+            const T dfcA = inA ? cutoff_dfn(pj.r, L.pi_rc_A) : T(0);
+
+            // radial: dE/dr_ij = sum_shells g * exp(-eta d^2) * (f_C' - 2 eta d f_C)
+            for (unsigned long long m = wave_ballot(inR); m; m &= m - 1) {
+                const int b = lowest_bit(m);
+                const Partner<T> J = partner_from_lane(pj, b);
+                const T fb = wave_get(fcR, b), dfb = wave_get(dfcR, b);
+                const T d = J.r - L.rrs;
+                T w = g_rad * Real<T>::exp_(-L.R_eta * d * d) * (dfb - T(2) * L.R_eta * d * fb);
+                w = (J.type == L.rtype) ? w : T(0);
+                const T G = wave_sum(w) / J.r;            // dE/dr divided by r: multiplies d = x_i - x_j
+                const T fx = G * J.dx, fy = G * J.dy, fz = G * J.dz;
+                if (L.half == 0) { ix += fx; iy += fy; iz += fz; }
+                if (lane == 0) {
+                    add(jc + b, -fx, -fy, -fz);
+                }
+            }
+
+            // angular
+            for (unsigned long long mj = wave_ballot(inA); mj; mj &= mj - 1) {
+                const int bj = lowest_bit(mj);
+                const Partner<T> J = partner_from_lane(pj, bj);
+                const T Jfc = wave_get(fcA, bj), Jdfc = wave_get(dfcA, bj);
+                const T Jinv = T(1) / J.r;
+                const T ujx = J.dx * Jinv, ujy = J.dy * Jinv, ujz = J.dz * Jinv;
+                T jx = T(0), jy = T(0), jz = T(0);          // force on j: per-half partials
+                for (int kc = jc; kc < n; kc += 64) {
+                    Partner<T> pk;
+                    T fcK, dfcK;
+                    bool kin;
+                    if (kc == jc) {
+                        pk = pj;
+                        fcK = fcA;
+                        dfcK = dfcA;
+                        kin = inA && (lane > bj);
+                    } else {
+                        const int k = kc + lane;
+                        pk = scan_partner(X, Y, Z, A, off, k, n, xi, yi, zi);
+                        kin = (k < n) && (k != i) && (pk.r < L.A_Rc);
+                        fcK = kin ? cutoff_fn(pk.r, L.pi_rc_A) : T(0);
+                        dfcK = kin ? cutoff_dfn(pk.r, L.pi_rc_A) : T(0);
+                    }
+                    unsigned long long mk = wave_ballot(kin);
+                    while (mk) {
+                        const int b0 = lowest_bit(mk);
+                        mk &= mk - 1;
+                        int b1 = -1;
+                        if (mk) {
+                            b1 = lowest_bit(mk);
+                            mk &= mk - 1;
+                        }
+                        const bool act = (L.half == 0) || (b1 >= 0);
+                        const int src = (L.half == 0 || b1 < 0) ? b0 : b1;
+                        const Partner<T> K = partner_from_lane(pk, src);
+                        const T Kfc = wave_get(fcK, src), Kdfc = wave_get(dfcK, src);
+                        const T Kinv = T(1) / K.r;
+                        const T ukx = K.dx * Kinv, uky = K.dy * Kinv, ukz = K.dz * Kinv;
+
+                        T c = ujx * ukx + ujy * uky + ujz * ukz;
+                        c = fmin(fmax(c, T(-1)), T(1));
+                        const T cx = ujy * ukz - ujz * uky;
+                        const T cy = ujz * ukx - ujx * ukz;
+                        const T cz = ujx * uky - ujy * ukx;
+                        // guard: exactly collinear triples have no finite derivative
+                        const T s = fmax(Real<T>::sqrt_(cx * cx + cy * cy + cz * cz), T(1e-30));
+                        const T base = T(1) + c * L.ct + s * L.st;
+                        const T b2 = base * base, b4 = b2 * b2;
+                        const T Am1 = b4 * b2 * base;                         // base^(zeta-1)
+                        const T At = Am1 * base;
+                        const T dAt = T(8) * Am1 * (L.ct - (c / s) * L.st);   // d/dc (1+cos(th-th_t))^8
+                        const T dav = (J.r + K.r) * T(0.5) - L.ars;
+                        const T Gs = Real<T>::exp_(-L.A_eta * dav * dav);
+                        const T g = g_ang[pair_block(J.type, K.type) * kAngBlock + L.ts];
+                        const T gAG = g * At * Gs;
+                        const T W0 = half_sum(gAG);
+                        const T Wc = half_sum(g * dAt * Gs);
+                        const T Wr = half_sum(gAG * (T(-2) * L.A_eta * dav));
+
+                        const T two_pow = T(0.0078125);
+                        const T P = two_pow * Jfc * Kfc;
+                        const T Fj = P * Wr * T(0.5) + two_pow * W0 * Jdfc * Kfc;   // dE/dr_ij
+                        const T Fk = P * Wr * T(0.5) + two_pow * W0 * Jfc * Kdfc;   // dE/dr_ik
+                        const T Fc = P * Wc;                                        // dE/dcos
+                        const T vjx = Fj * ujx + Fc * (ukx - c * ujx) * Jinv;
+                        const T vjy = Fj * ujy + Fc * (uky - c * ujy) * Jinv;
+                        const T vjz = Fj * ujz + Fc * (ukz - c * ujz) * Jinv;
+                        const T vkx = Fk * ukx + Fc * (ujx - c * ukx) * Kinv;
+                        const T vky = Fk * uky + Fc * (ujy - c * uky) * Kinv;
+                        const T vkz = Fk * ukz + Fc * (ujz - c * ukz) * Kinv;
+                        if (act) {
+                            ix += vjx + vkx; iy += vjy + vky; iz += vjz + vkz;
+                            jx += vjx; jy += vjy; jz += vjz;
+                            if (L.ts == 0) {
+                                add(kc + src, -vkx, -vky, -vkz);
+                            }
+                        }
+                    }
+                }
+                jx += __shfl_xor(jx, 32, 64);
+                jy += __shfl_xor(jy, 32, 64);
+                jz += __shfl_xor(jz, 32, 64);
+                if (lane == 0) {
+                    add(jc + bj, -jx, -jy, -jz);
+                }
+            }
+        }
+        ix += __shfl_xor(ix, 32, 64);
+        iy += __shfl_xor(iy, 32, 64);
+        iz += __shfl_xor(iz, 32, 64);
+        if (lane == 0) {
+            add(i, ix, iy, iz);
+        }
+        wave_lds_fence();
+}
+
 }  // namespace khan

@@ -21,22 +21,11 @@
 // No atomics and no pre-zeroed output.  A centre with more than 32 angular neighbours (the 3.1 A
 // sphere holds about 25 atoms at the densest packings tested) is redone by the general-shape
 // per-centre routine.  Semantics: gpu_featurizer/kernel_cpu.cpp:406-537.
-#include "aev_generic_center.h"
+#include "aev_small_common.h"
 
 namespace khan {
 
 namespace {
-
-constexpr int kB = 6;          // centres per batch: 6 x 10 type pairs = 60 segment lanes
-constexpr int kCapA = 32;      // angular neighbours kept per centre
-constexpr int kBitWords = 96;  // 6 centres x (496 triples + padding) fit in 96 x 32 slot bits
-
-struct __align__(16) SegDesc {
-    int start;       // first triple slot of the segment inside the batch (even)
-    int cnt;         // triples in the segment (its slot range is padded to an even length)
-    int packed;      // centre-in-batch | offset of type a | offset of type b | n_a | a==b | pair index
-    float rcp_na;    // 1 / n_a
-};
 
 struct __align__(16) SmallLds {
     float4 atom[64];            // x, y, z, type (sorted order)
@@ -49,82 +38,6 @@ struct __align__(16) SmallLds {
     int nA[kB][4];              // angular partners per type, per centre of the batch
     int nR[4][4];               // radial partners per type, per group of the scan step
 };
-
-__device__ __forceinline__ float lane_read(float v, int src_lane)
-{
-    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src_lane));
-}
-__device__ __forceinline__ int lane_read(int v, int src_lane) { return __builtin_amdgcn_readlane(v, src_lane); }
-__device__ __forceinline__ float lane_push(int dest_lane, float v)   // the value lands in lane dest_lane
-{
-    return __int_as_float(__builtin_amdgcn_ds_permute(dest_lane << 2, __float_as_int(v)));
-}
-__device__ __forceinline__ int lane_push(int dest_lane, int v) { return __builtin_amdgcn_ds_permute(dest_lane << 2, v); }
-__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
-
-// Row pointers are rebuilt from two 32-bit lane reads; storing through an explicit global-address-space
-// pointer keeps the stores on the global (not the flat) path.
-typedef float __attribute__((address_space(1))) global_float;
-__device__ __forceinline__ void store_global(float* p, float v)
-{
-    *((global_float*)(p)) = v;
-}
-// sum of the two half-waves, in every lane: swap the upper half of one copy with the lower half of
-// the other (one cross-lane VALU move, no LDS round trip), then add
-__device__ __forceinline__ float half_wave_sum(float v)
-{
-    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_int(v), __float_as_int(v), false, false);
-    return __int_as_float(r[0]) + __int_as_float(r[1]);
-}
-
-// Inclusive add-scan across the 64 lanes with data-parallel-primitive moves: four shifts inside each
-// row of 16 lanes, then lane 15 of rows 0,2 is carried into rows 1,3 and lane 31 into rows 2,3.
-// Lanes without a source take the identity 0.
-template <int kCtrl, int kRowMask>
-__device__ __forceinline__ int dpp_take(int v)
-{
-    return __builtin_amdgcn_update_dpp(0, v, kCtrl, kRowMask, 0xf, false);
-}
-__device__ __forceinline__ int scan_add(int v)
-{
-    v += dpp_take<0x111, 0xf>(v);   // row_shr:1
-    v += dpp_take<0x112, 0xf>(v);   // row_shr:2
-    v += dpp_take<0x114, 0xf>(v);   // row_shr:4
-    v += dpp_take<0x118, 0xf>(v);   // row_shr:8
-    v += dpp_take<0x142, 0xa>(v);   // row_bcast:15 into rows 1 and 3
-    v += dpp_take<0x143, 0xc>(v);   // row_bcast:31 into rows 2 and 3
-    return v;
-}
-
-__device__ __forceinline__ float pow8(float b)
-{
-    const float b2 = b * b, b4 = b2 * b2;
-    return b4 * b4;
-}
-__device__ __forceinline__ int sel4(int a, int v0, int v1, int v2, int v3)
-{
-    return a == 0 ? v0 : a == 1 ? v1 : a == 2 ? v2 : v3;
-}
-__device__ __forceinline__ int popc64(unsigned long long m) { return __popcll(m); }
-__device__ __forceinline__ unsigned long long low_bits(int w)   // w ones, 1 <= w <= 64
-{
-    return w >= 64 ? ~0ull : ((1ull << w) - 1ull);
-}
-
-// f_C(r, rc) = 0.5 cos(pi u) + 0.5 = cos^2(pi u / 2), u = r / rc in [0, 1).
-// With w = min(u, 1-u) and s = sin(pi w / 2) (odd minimax polynomial on [0, 0.5], |err| < 1.1e-7):
-// f_C = 1 - s^2 for u <= 0.5 and s^2 above, which keeps full relative accuracy where f_C -> 0.
-__device__ __forceinline__ float cutoff_poly(float u)
-{
-    const float w = fminf(u, 1.0f - u);
-    const float w2 = w * w;
-    float p = fmaf(w2, -0.00459228908981766f, 0.07967590297660462f);
-    p = fmaf(w2, p, -0.645962938168251f);
-    p = fmaf(w2, p, 1.5707963050854938f);
-    const float s = p * w;
-    const float q = s * s;
-    return (u <= 0.5f) ? 1.0f - q : q;
-}
 
 __global__ __launch_bounds__(256) void aev_fwd_small_kernel(
     const float* __restrict__ X, const float* __restrict__ Y, const float* __restrict__ Z,

@@ -50,6 +50,31 @@ int forward_dispatch(const double* xs, const double* ys, const double* zs, const
     return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, stream));
 }
 
+int backward_dispatch(const float* xs, const float* ys, const float* zs, const int32_t* as,
+                      const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
+                      khan::Buckets<const float> g, float* gx, float* gy, float* gz, int64_t n_atoms,
+                      hipStream_t stream)
+{
+    if (force_generic())
+        return hip_status(khan::launch_bwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                          n_atoms, 0, stream));
+    // general kernel first (it zero-fills and accumulates with atomics, molecules above 64 atoms
+    // only), then the small-molecule kernel, which stores every gradient of its molecules itself
+    int st = hip_status(khan::launch_bwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                        n_atoms, khan::kSmallMaxAtoms + 1, stream));
+    if (st != KHAN_OK) return st;
+    return hip_status(khan::launch_bwd_small_f32(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, stream));
+}
+
+int backward_dispatch(const double* xs, const double* ys, const double* zs, const int32_t* as,
+                      const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
+                      khan::Buckets<const double> g, double* gx, double* gy, double* gz, int64_t n_atoms,
+                      hipStream_t stream)
+{
+    return hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                       n_atoms, 0, stream));
+}
+
 template <typename T>
 int featurize_impl(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
                    const int32_t* macs, int32_t n_mols, const int32_t* sis, T* h, T* c, T* n, T* o,
@@ -83,8 +108,7 @@ int featurize_grad_impl(const T* xs, const T* ys, const T* zs, const int32_t* as
     if ((acs_host[0] && !gh) || (acs_host[1] && !gc) || (acs_host[2] && !gn) || (acs_host[3] && !go))
         return KHAN_ERR_INVALID_ARG;
     khan::Buckets<const T> g{{gh, gc, gn, go}};
-    return hip_status(khan::launch_bwd_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                  n_atoms, as_stream(stream)));
+    return backward_dispatch(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, n_atoms, as_stream(stream));
 }
 
 template <typename T>

@@ -27,7 +27,11 @@ template <typename T>
 hipError_t launch_bwd_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
                               const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
                               const int32_t* SIs, Buckets<const T> g, T* gX, T* gY, T* gZ,
-                              int64_t n_atoms, hipStream_t stream);
+                              int64_t n_atoms, int min_atoms, hipStream_t stream);
+hipError_t launch_bwd_small_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
+                                const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                                const int32_t* SIs, Buckets<const float> g, float* gX, float* gY,
+                                float* gZ, hipStream_t stream);
 
 // ---- integer path ----
 hipError_t launch_mol_offsets(const int32_t* mol_idxs, int64_t n_atoms, int32_t n_mols,
