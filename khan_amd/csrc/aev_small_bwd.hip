@@ -170,6 +170,7 @@ __global__ __launch_bounds__(256) void aev_bwd_small_kernel(
 
             // ---- radial pairs: this lane's (centre, partner) pair over its 16 shells
             const float* grow = row_of_lane(ci);
+            float cfx = 0.f, cfy = 0.f, cfz = 0.f;       // this pair's pull on the centre
             if (inR && fits) {      // an overflowing centre is redone as a whole by the general routine
                 const int tj = __float_as_int(aj.w);
                 const global_v4f_ptr gp = (global_v4f_ptr)(grow + tj * kNumRRs);
@@ -187,13 +188,21 @@ __global__ __launch_bounds__(256) void aev_bwd_small_kernel(
                     Gsum = fmaf(gr[q] * e, fmaf(m2eta_fc, d, dfc), Gsum);   // g e (f_C' - 2 eta d f_C)
                 }
                 const float sc = Gsum * inv;           // dE/dr / r, multiplies (x_i - x_j)
-                const float fx = sc * dx, fy = sc * dy, fz = sc * dz;
-                atomicAdd(&S.force[0][i], fx);
-                atomicAdd(&S.force[1][i], fy);
-                atomicAdd(&S.force[2][i], fz);
-                atomicAdd(&S.force[0][jl], -fx);
-                atomicAdd(&S.force[1][jl], -fy);
-                atomicAdd(&S.force[2][jl], -fz);
+                cfx = sc * dx;
+                cfy = sc * dy;
+                cfz = sc * dz;
+                atomicAdd(&S.force[0][jl], -cfx);
+                atomicAdd(&S.force[1][jl], -cfy);
+                atomicAdd(&S.force[2][jl], -cfz);
+            }
+            // the W lanes of a group share their centre: sum inside the group, one lane adds
+            cfx = group_sum_to_last_lane(cfx, logW);
+            cfy = group_sum_to_last_lane(cfy, logW);
+            cfz = group_sum_to_last_lane(cfz, logW);
+            if (jl == W - 1 && centre_ok) {
+                atomicAdd(&S.force[0][i], cfx);
+                atomicAdd(&S.force[1][i], cfy);
+                atomicAdd(&S.force[2][i], cfz);
             }
         }
         wave_lds_fence();
@@ -262,6 +271,7 @@ __global__ __launch_bounds__(256) void aev_bwd_small_kernel(
                 bsel = 0;
             }
             const float* grow = row_of_lane(c0 + bsel);
+            float cix = 0.f, ciy = 0.f, ciz = 0.f;       // this triple's pull on its centre
             if (ok) {
                 const global_v4f_ptr gp = (global_v4f_ptr)(grow + kRadial + pt * kAngBlock);
                 v4f g[8];
@@ -314,16 +324,31 @@ __global__ __launch_bounds__(256) void aev_bwd_small_kernel(
                 const float vkx = fmaf(Fk, vk.x, ik * (vj.x - c * vk.x));
                 const float vky = fmaf(Fk, vk.y, ik * (vj.y - c * vk.y));
                 const float vkz = fmaf(Fk, vk.z, ik * (vj.z - c * vk.z));
-                const int atom_i = c0 + bsel;
-                atomicAdd(&S.force[0][atom_i], vjx + vkx);
-                atomicAdd(&S.force[1][atom_i], vjy + vky);
-                atomicAdd(&S.force[2][atom_i], vjz + vkz);
+                cix = vjx + vkx;
+                ciy = vjy + vky;
+                ciz = vjz + vkz;
                 atomicAdd(&S.force[0][atom_j], -vjx);
                 atomicAdd(&S.force[1][atom_j], -vjy);
                 atomicAdd(&S.force[2][atom_j], -vjz);
                 atomicAdd(&S.force[0][atom_k], -vkx);
                 atomicAdd(&S.force[1][atom_k], -vky);
                 atomicAdd(&S.force[2][atom_k], -vkz);
+            }
+            // lanes of one centre are contiguous: one wave sum per centre present in this step
+            {
+                const int b_first = lane_read(bsel, 0);
+                const int b_last = lane_read(bsel, min(63, total - base - 1));
+                for (int bb = b_first; bb <= b_last; ++bb) {
+                    const bool mine = ok && (bsel == bb);
+                    const float sx = group_sum_to_last_lane(mine ? cix : 0.f, 6);
+                    const float sy = group_sum_to_last_lane(mine ? ciy : 0.f, 6);
+                    const float sz = group_sum_to_last_lane(mine ? ciz : 0.f, 6);
+                    if (lane == 63) {
+                        S.force[0][c0 + bb] += sx;
+                        S.force[1][c0 + bb] += sy;
+                        S.force[2][c0 + bb] += sz;
+                    }
+                }
             }
         }
         wave_lds_fence();

@@ -62,6 +62,24 @@ __device__ __forceinline__ int scan_add(int v)
     return v;
 }
 
+// Float add-scan with the same data-parallel-primitive moves.  After `rows` steps the last lane of
+// each group of 16 (rows = 4), 32 (rows = 5) or 64 (rows = 6) lanes holds that group's sum.
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ float dpp_take_f(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, kRowMask, 0xf, false));
+}
+__device__ __forceinline__ float group_sum_to_last_lane(float v, int log_group)
+{
+    v += dpp_take_f<0x111, 0xf>(v);
+    v += dpp_take_f<0x112, 0xf>(v);
+    v += dpp_take_f<0x114, 0xf>(v);
+    v += dpp_take_f<0x118, 0xf>(v);
+    if (log_group >= 5) v += dpp_take_f<0x142, 0xa>(v);
+    if (log_group >= 6) v += dpp_take_f<0x143, 0xc>(v);
+    return v;
+}
+
 __device__ __forceinline__ float pow8(float b)
 {
     const float b2 = b * b, b4 = b2 * b2;
