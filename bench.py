@@ -23,6 +23,13 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3       # MI355X vector FP32, published
 FP64_PEAK_TFLOPS = 78.6
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the same
+# counter reads for a plain 64 MiB copy); the summaries and commands are under profiles/.
+MEASURED_TRAFFIC = {
+    ("organic65536", "fwd"): 1208.4e6,
+    ("organic65536", "bwd"): 755.6e6,
+}
+
 WORKLOADS = {
     "organic65536": ("organic", 65536),
     "organic16384": ("organic", 16384),
@@ -172,7 +179,7 @@ def main():
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": achieved / HBM_PEAK_GBS,
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC.get((args.workload, dom)),
         "launch_ms": ms[dom],
         "algorithmic_bytes": dom_bytes,
         "valu_frac_fp32": dom_flops / (ms[dom] * 1e-3) / 1e12 / FP32_PEAK_TFLOPS,
