@@ -1,16 +1,22 @@
 // AEV backward (dL/dxyz) for molecules of up to 64 atoms, float32: one wavefront per molecule.
 //
-// Same skeleton as the small-molecule forward kernel (lanes sorted by type, six centres per batch,
-// scan steps of G centres x W partners, type-sorted neighbour lists in LDS, triples enumerated in
-// (centre, type-pair) order and dealt one per lane), but here a lane owns its triple completely:
-// it recomputes the geometry, reads the 32 upstream values g[type pair][theta_t][Rs_s] of its centre
-// straight from the upstream row (lanes of one segment read the same 128 bytes, served by the
-// vector L1), forms the three weighted sums
-//     W0 = sum g A_t G_s,   Wc = sum g dA_t/dcos G_s,   Wr = sum g A_t dG_s/drho
-// serially over the 32 slots -- no cross-lane reduction -- and adds the forces on i, j and k into
-// a per-molecule force array in LDS.  Radial pairs are handled the same way in the scan step, one
-// (centre, partner) pair per lane over its 16 shells.  When the molecule is finished each lane
-// stores the gradient of its own atom: no global atomics, no pre-zeroed output.
+// Lanes are sorted by atom type and centres are scanned six at a time exactly as in the forward
+// kernel, producing per-centre lists of angular partners (unit vector, distance, f_C, f_C').  Then
+//   radial   a lane owns one (centre, partner) pair: it reads the 16 upstream values of the partner's
+//            type from the centre's row, sums g e (f_C' - 2 eta d f_C) over the shells, and the pull
+//            goes to the partner (one group at a time, so targets are distinct) and, summed over the
+//            group with DPP moves, to the centre;
+//   angular  a lane owns one list entry (centre b, partner j) and walks the other partners of the
+//            same centre in round-robin order, k = j+1, j+2, ... (mod m): in every round all lanes of
+//            a centre hold distinct j AND distinct k, each unordered pair {j,k} is met exactly once,
+//            and all lanes finish together.  A lane computes its triple completely (32 upstream
+//            values read straight from the row, three weighted sums formed serially, no cross-lane
+//            reduction), keeps the force on j in registers and adds the force on k to a per-centre
+//            slot in LDS with a plain read-add-write: targets are distinct by construction, so no
+//            atomics are needed (float atomics on LDS cost ~190 cycles per wave instruction here);
+//   gather   per centre, the slot of every partner is added to its atom's force, and the centre gets
+//            minus the sum (each row's forces add up to zero by translation invariance).
+// Finally every lane stores the gradient of its own atom: no global atomics, no pre-zeroed output.
 // The derivative is the algebraically reduced form (no acos, no 1/(1+cos) factor); reference:
 // gpu_featurizer/kernel_cpu.cpp:217-366.
 #include "aev_small_common.h"
@@ -25,11 +31,10 @@ typedef const __attribute__((address_space(1))) v4f* global_v4f_ptr;
 struct __align__(16) BwdLds {
     float4 atom[64];                     // x, y, z, type (sorted order)
     float4 nbr[kB][kCapA];               // unit vector (centre minus partner)/r, and r
+    float4 facc[kB][kCapA];              // force on each partner from its centre's row (xyz, pad)
     float2 nbr_fc[kB][kCapA];            // f_C(r, A_Rc) and its derivative in r
     float force[3][64];                  // dL/dx, dL/dy, dL/dz per sorted atom
-    SegDesc seg[64];
-    unsigned bits[kBitWords];
-    int nA[kB][4];
+    int nM[8];                           // angular partners per centre of the batch
     unsigned char nbr_idx[kB][kCapA];    // sorted lane of the partner
     unsigned char inv[64];               // original atom index -> sorted lane
 };
@@ -105,34 +110,26 @@ __global__ __launch_bounds__(256) void aev_bwd_small_kernel(
         const unsigned hi = static_cast<unsigned>(lane_read(rp_hi, sorted_lane));
         return reinterpret_cast<const float*>((static_cast<unsigned long long>(hi) << 32) | lo);
     };
-    unsigned long long smask[4];
-#pragma unroll
-    for (int a = 0; a < 4; ++a) smask[a] = (tcount[a] == 0) ? 0ull : (low_bits(tcount[a]) << tbase[a]);
-
     const int logW = n <= 16 ? 4 : n <= 32 ? 5 : 6;
     const int W = 1 << logW, G = 64 >> logW;
     const int grp = lane >> logW, jl = lane & (W - 1);
     const unsigned long long sub_mask = low_bits(W) << ((grp * W) & 63);
     const unsigned long long ltg_mask = lt_mask & sub_mask;
-    const int cl_g = (lane >> 2) & 3, cl_a = lane & 3;
-    const bool cl_on = (lane < 16) && (cl_g < G);
-    const unsigned long long cl_sub = cl_on ? (low_bits(W) << ((cl_g * W) & 63)) : 0ull;
-    const unsigned long long cl_mask =
-        cl_on ? ((cl_a == 0 ? smask[0] : cl_a == 1 ? smask[1] : cl_a == 2 ? smask[2] : smask[3]) << ((cl_g * W) & 63)) : 0ull;
-
-    const int seg_b = lane / kNumPairBlocks, seg_pt = lane - seg_b * kNumPairBlocks;
-    const int seg_a = seg_pt < 4 ? 0 : seg_pt < 7 ? 1 : seg_pt < 9 ? 2 : 3;
-    const int seg_bt = seg_pt < 4 ? seg_pt : seg_pt < 7 ? seg_pt - 3 : seg_pt < 9 ? seg_pt - 5 : 3;
-
     const float inv_rc_R = 1.0f / kR_Rc_f, inv_rc_A = 1.0f / kA_Rc_f;
     const float kLog2e = 1.44269504088896340736f;
     const float kRadExp = -kR_eta_f * kLog2e;
     const float kAngExp = -kA_eta_f * kLog2e;
+    // type of a sorted lane from the type boundaries
+    const int tb1 = tbase[1], tb2 = tbase[2], tb3 = tbase[3];
+    auto type_of = [&](int sorted_lane) { return (sorted_lane >= tb1) + (sorted_lane >= tb2) + (sorted_lane >= tb3); };
     wave_lds_fence();
 
     for (int c0 = 0; c0 < n; c0 += kB) {
         const int nb = min(kB, n - c0);
         unsigned overflow = 0;
+        for (int q = lane; q < kB * kCapA; q += 64) (&S.facc[0][0])[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (lane < 8) S.nM[lane] = 0;
+        wave_lds_fence();
 
         // ------------------------------------------------ scan steps: G centres x W partners
         for (int b0 = 0; b0 < nb; b0 += G) {
@@ -140,6 +137,7 @@ __global__ __launch_bounds__(256) void aev_bwd_small_kernel(
             const int i = c0 + b;
             const bool centre_ok = b < nb;
             const int ci = centre_ok ? i : 0;
+            const int cb = centre_ok ? b : 0;
             const float4 ai = S.atom[ci];
             const float4 aj = S.atom[jl];
             const float dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
@@ -148,30 +146,29 @@ __global__ __launch_bounds__(256) void aev_bwd_small_kernel(
             const bool inR = valid && (r < kR_Rc_f);
             const bool inA = valid && (r < kA_Rc_f);
             const unsigned long long mA = wave_ballot(inA);
-            const bool fits = popc64(mA & sub_mask) <= kCapA;
+            const int cntA = popc64(mA & sub_mask);
+            const bool fits = cntA <= kCapA;
             const float inv = __builtin_amdgcn_rcpf(r);
             if (inA && fits) {
                 const int pos = popc64(mA & ltg_mask);
                 float fc, dfc;
                 cutoff_poly_grad(r * inv_rc_A, inv_rc_A, fc, dfc);
-                S.nbr[ci - c0][pos] = make_float4(dx * inv, dy * inv, dz * inv, r);
-                S.nbr_fc[ci - c0][pos] = make_float2(fc, dfc);
-                S.nbr_idx[ci - c0][pos] = static_cast<unsigned char>(jl);
+                S.nbr[cb][pos] = make_float4(dx * inv, dy * inv, dz * inv, r);
+                S.nbr_fc[cb][pos] = make_float2(fc, dfc);
+                S.nbr_idx[cb][pos] = static_cast<unsigned char>(jl);
             }
+            if (jl == 0 && centre_ok) S.nM[b] = fits ? cntA : 0;
             {
                 const unsigned long long ov = wave_ballot(!fits && jl == 0 && centre_ok);
                 for (int g = 0; g < G; ++g)
                     if ((ov >> (g * W)) & 1ull) overflow |= 1u << (b0 + g);
             }
-            if (cl_on) {
-                const int cb = b0 + cl_g;
-                if (cb < nb) S.nA[cb][cl_a] = (popc64(mA & cl_sub) <= kCapA) ? popc64(mA & cl_mask) : 0;
-            }
 
             // ---- radial pairs: this lane's (centre, partner) pair over its 16 shells
             const float* grow = row_of_lane(ci);
             float cfx = 0.f, cfy = 0.f, cfz = 0.f;       // this pair's pull on the centre
-            if (inR && fits) {      // an overflowing centre is redone as a whole by the general routine
+            const bool do_rad = inR && fits;              // an overflowing centre is redone as a whole
+            if (do_rad) {
                 const int tj = __float_as_int(aj.w);
                 const global_v4f_ptr gp = (global_v4f_ptr)(grow + tj * kNumRRs);
                 const v4f g0 = gp[0], g1 = gp[1], g2 = gp[2], g3 = gp[3];
@@ -191,167 +188,148 @@ __global__ __launch_bounds__(256) void aev_bwd_small_kernel(
                 cfx = sc * dx;
                 cfy = sc * dy;
                 cfz = sc * dz;
-                atomicAdd(&S.force[0][jl], -cfx);
-                atomicAdd(&S.force[1][jl], -cfy);
-                atomicAdd(&S.force[2][jl], -cfz);
             }
-            // the W lanes of a group share their centre: sum inside the group, one lane adds
+            // partner forces: one group per round, so the targets of a round are distinct atoms
+            for (int g = 0; g < G; ++g) {
+                if (do_rad && grp == g) {
+                    S.force[0][jl] -= cfx;
+                    S.force[1][jl] -= cfy;
+                    S.force[2][jl] -= cfz;
+                }
+            }
+            // the W lanes of a group share their centre: sum inside the group, its last lane adds
             cfx = group_sum_to_last_lane(cfx, logW);
             cfy = group_sum_to_last_lane(cfy, logW);
             cfz = group_sum_to_last_lane(cfz, logW);
             if (jl == W - 1 && centre_ok) {
-                atomicAdd(&S.force[0][i], cfx);
-                atomicAdd(&S.force[1][i], cfy);
-                atomicAdd(&S.force[2][i], cfz);
+                S.force[0][i] += cfx;
+                S.force[1][i] += cfy;
+                S.force[2][i] += cfz;
             }
         }
         wave_lds_fence();
 
-        // ------------------------------------------------ segment table of the batch
-        int cnt = 0, packed = 0;
-        float rcp_na = 0.f;
-        if (lane < nb * kNumPairBlocks) {
-            const int4 nn = *reinterpret_cast<const int4*>(S.nA[seg_b]);
-            const int na = sel4(seg_a, nn.x, nn.y, nn.z, nn.w);
-            const int nbt = sel4(seg_bt, nn.x, nn.y, nn.z, nn.w);
-            const int oa = sel4(seg_a, 0, nn.x, nn.x + nn.y, nn.x + nn.y + nn.z);
-            const int ob = sel4(seg_bt, 0, nn.x, nn.x + nn.y, nn.x + nn.y + nn.z);
-            const bool same = seg_a == seg_bt;
-            cnt = same ? (na * (na - 1)) / 2 : na * nbt;
-            packed = seg_b | (oa << 3) | (ob << 9) | (na << 15) | (same ? (1 << 21) : 0) | (seg_pt << 22);
-            rcp_na = na > 0 ? __builtin_amdgcn_rcpf(static_cast<float>(na)) : 0.f;
-        }
-        const int incl = scan_add(cnt);
-        const int start = incl - cnt;
-        const int total = lane_read(incl, 63);
-        const unsigned long long nonempty = wave_ballot(cnt > 0);
-        for (int w = lane; w < kBitWords; w += 64) S.bits[w] = 0u;
-        wave_lds_fence();
-        if (cnt > 0) {
-            SegDesc d;
-            d.start = start;
-            d.cnt = cnt;
-            d.packed = packed;
-            d.rcp_na = rcp_na;
-            S.seg[popc64(nonempty & lt_mask)] = d;
-            atomicOr(&S.bits[start >> 5], 1u << (start & 31));
-        }
-        wave_lds_fence();
+        // ------------------------------------------------ angular: lane = (centre, partner j), round robin over k
+        const int4 m03 = *reinterpret_cast<const int4*>(&S.nM[0]);
+        const int4 m47 = *reinterpret_cast<const int4*>(&S.nM[4]);
+        const int p1 = m03.x, p2 = p1 + m03.y, p3 = p2 + m03.z, p4 = p3 + m03.w, p5 = p4 + m47.x;
+        const int total = uniform(p5 + m47.y);
+        for (int pass0 = 0; pass0 < total; pass0 += 64) {
+            const int slot = pass0 + lane;
+            const bool live = slot < total;
+            const int b = (slot >= p1) + (slot >= p2) + (slot >= p3) + (slot >= p4) + (slot >= p5);
+            const int bs = live ? b : 0;
+            const int pb = bs == 0 ? 0 : bs == 1 ? p1 : bs == 2 ? p2 : bs == 3 ? p3 : bs == 4 ? p4 : p5;
+            const int m = bs == 0 ? m03.x : bs == 1 ? m03.y : bs == 2 ? m03.z : bs == 3 ? m03.w : bs == 4 ? m47.x : m47.y;
+            const int e = live ? slot - pb : 0;
+            // rounds: d = 1 .. (m-1)/2 for every lane; when m is even one more round for the lower half
+            const int full = (m - 1) >> 1;
+            const int rounds = live ? full + ((((m & 1) == 0) && (e < (m >> 1))) ? 1 : 0) : 0;
+            const int max_rounds = wave_max(rounds);
+            const float4 vj = S.nbr[bs][e];
+            const float2 fj = S.nbr_fc[bs][e];
+            const int tj = type_of(S.nbr_idx[bs][e]);
+            const float inv_rj = __builtin_amdgcn_rcpf(vj.w);
+            const float* grow = row_of_lane(c0 + bs);
+            float ajx = 0.f, ajy = 0.f, ajz = 0.f;           // force on j, kept in registers
 
-        // ------------------------------------------------ triples, one per lane
-        int carry = 0;
-        for (int base = 0; base < total; base += 64) {
-            const unsigned w0 = static_cast<unsigned>(uniform(static_cast<int>(S.bits[base >> 5])));
-            const unsigned w1 = static_cast<unsigned>(uniform(static_cast<int>(S.bits[(base >> 5) + 1])));
-            const unsigned long long starts = (static_cast<unsigned long long>(w1) << 32) | w0;
-            const int ord = carry + popc64(starts & (lt_mask | lane_bit)) - 1;
-            carry += popc64(starts);
-            const SegDesc d = S.seg[max(ord, 0)];
-            const int slot = base + lane;
-            const int q = slot - d.start;
-            const bool ok = (slot < total) && (q >= 0) && (q < d.cnt);
+            for (int d = 1; d <= max_rounds; ++d) {
+                const bool act = d <= rounds;
+                int k = e + d;
+                k -= (k >= m) ? m : 0;
+                k = act ? k : 0;
+                const float4 vk = S.nbr[bs][k];
+                const float2 fk = S.nbr_fc[bs][k];
+                const int tk = type_of(S.nbr_idx[bs][k]);
+                if (act) {
+                    const int pt = pair_block(tj, tk);
+                    const global_v4f_ptr gp = (global_v4f_ptr)(grow + kRadial + pt * kAngBlock);
+                    v4f g[8];
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) g[t] = gp[t];
 
-            int bsel = d.packed & 7;
-            const int oa = (d.packed >> 3) & 63, ob = (d.packed >> 9) & 63, na = (d.packed >> 15) & 63;
-            const int pt = (d.packed >> 22) & 15;
-            int kl, jl2;
-            if ((d.packed >> 21) & 1) {
-                kl = static_cast<int>((1.0f + __builtin_amdgcn_sqrtf(8.0f * static_cast<float>(q) + 1.0f)) * 0.5f);
-                if ((kl * (kl - 1)) / 2 > q) --kl;
-                if (((kl + 1) * kl) / 2 <= q) ++kl;
-                jl2 = q - (kl * (kl - 1)) / 2;
-            } else {
-                kl = static_cast<int>((static_cast<float>(q) + 0.5f) * d.rcp_na);
-                jl2 = q - kl * na;
-            }
-            int j = oa + jl2, k = ob + kl;
-            if (!ok) {
-                j = 0;
-                k = 0;
-                bsel = 0;
-            }
-            const float* grow = row_of_lane(c0 + bsel);
-            float cix = 0.f, ciy = 0.f, ciz = 0.f;       // this triple's pull on its centre
-            if (ok) {
-                const global_v4f_ptr gp = (global_v4f_ptr)(grow + kRadial + pt * kAngBlock);
-                v4f g[8];
+                    float c = vj.x * vk.x + vj.y * vk.y + vj.z * vk.z;
+                    c = fminf(fmaxf(c, -1.0f), 1.0f);
+                    const float cx = vj.y * vk.z - vj.z * vk.y;
+                    const float cy = vj.z * vk.x - vj.x * vk.z;
+                    const float cz = vj.x * vk.y - vj.y * vk.x;
+                    // exactly collinear triples have no finite derivative: keep the result finite
+                    const float s = fmaxf(__builtin_amdgcn_sqrtf(cx * cx + cy * cy + cz * cz), 1e-30f);
+                    const float c_over_s = c * __builtin_amdgcn_rcpf(s);
+                    const float rho = 0.5f * (vj.w + vk.w);
+                    float Gs[4], Hs[4];
 #pragma unroll
-                for (int t = 0; t < 8; ++t) g[t] = gp[t];
-                const float4 vj = S.nbr[bsel][j], vk = S.nbr[bsel][k];
-                const float2 fj = S.nbr_fc[bsel][j], fk = S.nbr_fc[bsel][k];
-                const int atom_j = S.nbr_idx[bsel][j], atom_k = S.nbr_idx[bsel][k];
-
-                float c = vj.x * vk.x + vj.y * vk.y + vj.z * vk.z;
-                c = fminf(fmaxf(c, -1.0f), 1.0f);
-                const float cx = vj.y * vk.z - vj.z * vk.y;
-                const float cy = vj.z * vk.x - vj.x * vk.z;
-                const float cz = vj.x * vk.y - vj.y * vk.x;
-                // exactly collinear triples have no finite derivative: keep the result finite
-                const float s = fmaxf(__builtin_amdgcn_sqrtf(cx * cx + cy * cy + cz * cz), 1e-30f);
-                const float c_over_s = c * __builtin_amdgcn_rcpf(s);
-                const float rho = 0.5f * (vj.w + vk.w);
-                float Gs[4], Hs[4];
-#pragma unroll
-                for (int sidx = 0; sidx < 4; ++sidx) {
-                    const float dd = rho - kA_Rs_f[sidx];
-                    Gs[sidx] = __builtin_amdgcn_exp2f(kAngExp * dd * dd);
-                    Hs[sidx] = Gs[sidx] * (-2.0f * kA_eta_f * dd);          // dG/drho
-                }
-                float W0 = 0.f, Wc = 0.f, Wr = 0.f;
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    const float ct = static_cast<float>(kCosTheta[t]), st = static_cast<float>(kSinTheta[t]);
-                    const float bs = fmaf(s, st, fmaf(c, ct, 1.0f));        // 1 + cos(theta - theta_t)
-                    const float b2 = bs * bs, b4 = b2 * b2;
-                    const float Am1 = b4 * b2 * bs;                          // ^7
-                    const float At = Am1 * bs;                               // ^8
-                    const float dAt = 8.0f * Am1 * fmaf(-c_over_s, st, ct);  // d/dcos
-                    const float ut = g[t].x * Gs[0] + g[t].y * Gs[1] + g[t].z * Gs[2] + g[t].w * Gs[3];
-                    const float vt = g[t].x * Hs[0] + g[t].y * Hs[1] + g[t].z * Hs[2] + g[t].w * Hs[3];
-                    W0 = fmaf(At, ut, W0);
-                    Wc = fmaf(dAt, ut, Wc);
-                    Wr = fmaf(At, vt, Wr);
-                }
-                const float two_pow = 0.0078125f;
-                const float P = two_pow * fj.x * fk.x;
-                const float Fj = fmaf(P * 0.5f, Wr, two_pow * W0 * fj.y * fk.x);    // dE/dr_ij
-                const float Fk = fmaf(P * 0.5f, Wr, two_pow * W0 * fj.x * fk.y);    // dE/dr_ik
-                const float Fc = P * Wc;                                            // dE/dcos
-                const float ij = Fc * __builtin_amdgcn_rcpf(vj.w), ik = Fc * __builtin_amdgcn_rcpf(vk.w);
-                const float vjx = fmaf(Fj, vj.x, ij * (vk.x - c * vj.x));
-                const float vjy = fmaf(Fj, vj.y, ij * (vk.y - c * vj.y));
-                const float vjz = fmaf(Fj, vj.z, ij * (vk.z - c * vj.z));
-                const float vkx = fmaf(Fk, vk.x, ik * (vj.x - c * vk.x));
-                const float vky = fmaf(Fk, vk.y, ik * (vj.y - c * vk.y));
-                const float vkz = fmaf(Fk, vk.z, ik * (vj.z - c * vk.z));
-                cix = vjx + vkx;
-                ciy = vjy + vky;
-                ciz = vjz + vkz;
-                atomicAdd(&S.force[0][atom_j], -vjx);
-                atomicAdd(&S.force[1][atom_j], -vjy);
-                atomicAdd(&S.force[2][atom_j], -vjz);
-                atomicAdd(&S.force[0][atom_k], -vkx);
-                atomicAdd(&S.force[1][atom_k], -vky);
-                atomicAdd(&S.force[2][atom_k], -vkz);
-            }
-            // lanes of one centre are contiguous: one wave sum per centre present in this step
-            {
-                const int b_first = lane_read(bsel, 0);
-                const int b_last = lane_read(bsel, min(63, total - base - 1));
-                for (int bb = b_first; bb <= b_last; ++bb) {
-                    const bool mine = ok && (bsel == bb);
-                    const float sx = group_sum_to_last_lane(mine ? cix : 0.f, 6);
-                    const float sy = group_sum_to_last_lane(mine ? ciy : 0.f, 6);
-                    const float sz = group_sum_to_last_lane(mine ? ciz : 0.f, 6);
-                    if (lane == 63) {
-                        S.force[0][c0 + bb] += sx;
-                        S.force[1][c0 + bb] += sy;
-                        S.force[2][c0 + bb] += sz;
+                    for (int sidx = 0; sidx < 4; ++sidx) {
+                        const float dd = rho - kA_Rs_f[sidx];
+                        Gs[sidx] = __builtin_amdgcn_exp2f(kAngExp * dd * dd);
+                        Hs[sidx] = Gs[sidx] * (-2.0f * kA_eta_f * dd);          // dG/drho
                     }
+                    float W0 = 0.f, Wc = 0.f, Wr = 0.f;
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) {
+                        const float ct = static_cast<float>(kCosTheta[t]), st = static_cast<float>(kSinTheta[t]);
+                        const float bs1 = fmaf(s, st, fmaf(c, ct, 1.0f));       // 1 + cos(theta - theta_t)
+                        const float b2 = bs1 * bs1, b4 = b2 * b2;
+                        const float Am1 = b4 * b2 * bs1;                         // ^7
+                        const float At = Am1 * bs1;                              // ^8
+                        const float dAt = 8.0f * Am1 * fmaf(-c_over_s, st, ct);  // d/dcos
+                        const float ut = g[t].x * Gs[0] + g[t].y * Gs[1] + g[t].z * Gs[2] + g[t].w * Gs[3];
+                        const float vt = g[t].x * Hs[0] + g[t].y * Hs[1] + g[t].z * Hs[2] + g[t].w * Hs[3];
+                        W0 = fmaf(At, ut, W0);
+                        Wc = fmaf(dAt, ut, Wc);
+                        Wr = fmaf(At, vt, Wr);
+                    }
+                    const float two_pow = 0.0078125f;
+                    const float P = two_pow * fj.x * fk.x;
+                    const float Fj = fmaf(P * 0.5f, Wr, two_pow * W0 * fj.y * fk.x);    // dE/dr_ij
+                    const float Fk = fmaf(P * 0.5f, Wr, two_pow * W0 * fj.x * fk.y);    // dE/dr_ik
+                    const float Fc = P * Wc;                                            // dE/dcos
+                    const float ij = Fc * inv_rj, ik = Fc * __builtin_amdgcn_rcpf(vk.w);
+                    ajx -= fmaf(Fj, vj.x, ij * (vk.x - c * vj.x));
+                    ajy -= fmaf(Fj, vj.y, ij * (vk.y - c * vj.y));
+                    ajz -= fmaf(Fj, vj.z, ij * (vk.z - c * vj.z));
+                    // force on k: in a round every lane of a centre holds a different k
+                    float4 fk_acc = S.facc[bs][k];
+                    fk_acc.x -= fmaf(Fk, vk.x, ik * (vj.x - c * vk.x));
+                    fk_acc.y -= fmaf(Fk, vk.y, ik * (vj.y - c * vk.y));
+                    fk_acc.z -= fmaf(Fk, vk.z, ik * (vj.z - c * vk.z));
+                    S.facc[bs][k] = fk_acc;
                 }
+                wave_lds_fence();
             }
+            if (live) {
+                float4 f = S.facc[bs][e];
+                f.x += ajx;
+                f.y += ajy;
+                f.z += ajz;
+                S.facc[bs][e] = f;
+            }
+            wave_lds_fence();
         }
-        wave_lds_fence();
+
+        // ------------------------------------------------ gather: partners get their slot, the centre minus the sum
+        for (int b = 0; b < nb; ++b) {
+            const int m = b == 0 ? m03.x : b == 1 ? m03.y : b == 2 ? m03.z : b == 3 ? m03.w : b == 4 ? m47.x : m47.y;
+            const int mu = uniform(m);
+            if (mu == 0) continue;
+            float4 f = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (lane < mu) {
+                f = S.facc[b][lane];
+                const int atom = S.nbr_idx[b][lane];
+                S.force[0][atom] += f.x;
+                S.force[1][atom] += f.y;
+                S.force[2][atom] += f.z;
+            }
+            const float sx = group_sum_to_last_lane(f.x, 6);
+            const float sy = group_sum_to_last_lane(f.y, 6);
+            const float sz = group_sum_to_last_lane(f.z, 6);
+            if (lane == 63) {
+                S.force[0][c0 + b] -= sx;
+                S.force[1][c0 + b] -= sy;
+                S.force[2][c0 + b] -= sz;
+            }
+            wave_lds_fence();
+        }
 
         // ------------------------------------------------ centres whose list overflowed
         if (overflow) {

@@ -62,6 +62,17 @@ __device__ __forceinline__ int scan_add(int v)
     return v;
 }
 
+__device__ __forceinline__ int wave_max(int v)       // all inputs >= 0; result is wave-uniform
+{
+    v = max(v, dpp_take<0x111, 0xf>(v));
+    v = max(v, dpp_take<0x112, 0xf>(v));
+    v = max(v, dpp_take<0x114, 0xf>(v));
+    v = max(v, dpp_take<0x118, 0xf>(v));
+    v = max(v, dpp_take<0x142, 0xa>(v));
+    v = max(v, dpp_take<0x143, 0xc>(v));
+    return __builtin_amdgcn_readlane(v, 63);
+}
+
 // Float add-scan with the same data-parallel-primitive moves.  After `rows` steps the last lane of
 // each group of 16 (rows = 4), 32 (rows = 5) or 64 (rows = 6) lanes holds that group's sum.
 template <int kCtrl, int kRowMask>
