@@ -95,6 +95,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="organic65536", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic-probe", choices=("fwd", "bwd"), default=None,
+                    help="counter-collection mode: launch that pass twice, then a plain 64 MiB device copy of "
+                         "known traffic (scales FETCH_SIZE / WRITE_SIZE), print nothing else and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; the path shards by molecule with no exchange, "
@@ -121,6 +124,26 @@ def main():
     gen.manual_seed(1234)
     upstream = torch.randn(N * 384, dtype=torch.float32, device=dev, generator=gen)   # dL/dAEV ~ N(0,1)
     torch.cuda.synchronize()
+
+    if args.traffic_probe:
+        macs, mos = ops.mol_offsets(mol_idxs, n_mols)
+        sc, ga, ac = ops.ani_sort(A)
+        acs = ac.cpu()
+        grads, start = [], 0
+        for c in acs.tolist():
+            grads.append(upstream[start * 384:(start + c) * 384])
+            start += c
+        for _ in range(2):
+            if args.traffic_probe == "fwd":
+                ops.featurize(X, Y, Z, A, mos, macs, sc, acs)
+            else:
+                ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *grads)
+        src = torch.empty(64 * 1024 * 1024 // 4, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        print("traffic probe: %s x2 on %s, then a 64 MiB device copy" % (args.traffic_probe, args.workload))
+        return
 
     ev = {k: [] for k in ("sort", "fwd", "bwd")}
 
