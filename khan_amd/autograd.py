@@ -1,0 +1,62 @@
+"""Gradient wiring of the featurization ops for torch.autograd, the counterpart of the
+`ops.RegisterGradient` blocks in khan/training/trainer_multi_tower.py:23-120:
+
+    Featurize   d/d(xs,ys,zs) through `featurize_grad`; no gradient for the index inputs
+                (trainer_multi_tower.py:23-51)
+    AniCharge   d/dqs through `ani_charge_grad` (trainer_multi_tower.py:88-120); here the
+                coordinates get a gradient too (`ani_charge_grad_xyz`), which the reference
+                leaves as None
+
+Both call the HIP library through `khan_amd.ops`; there is no other implementation behind them.
+"""
+import torch
+
+from . import ops
+
+
+class _Featurize(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, xs, ys, zs, as_, mos, macs, sis, acs):
+        acs_host = [int(v) for v in (acs.detach().cpu().tolist() if isinstance(acs, torch.Tensor) else acs)]
+        ctx.save_for_backward(xs, ys, zs, as_, mos, macs, sis)
+        ctx.acs_host = acs_host
+        return ops.featurize(xs.detach(), ys.detach(), zs.detach(), as_, mos, macs, sis, acs_host)
+
+    @staticmethod
+    def backward(ctx, grad_h, grad_c, grad_n, grad_o):
+        xs, ys, zs, as_, mos, macs, sis = ctx.saved_tensors
+        grads = []
+        for g, c in zip((grad_h, grad_c, grad_n, grad_o), ctx.acs_host):
+            if g is None:
+                g = torch.zeros(c * ops.FEATURE_SIZE, dtype=xs.dtype, device=xs.device)
+            grads.append(g.contiguous())
+        gx, gy, gz = ops.featurize_grad(xs.detach(), ys.detach(), zs.detach(), as_, mos, macs, sis,
+                                        ctx.acs_host, *grads)
+        return gx, gy, gz, None, None, None, None, None
+
+
+class _AniCharge(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, xs, ys, zs, qs, mos, macs):
+        ctx.save_for_backward(xs, ys, zs, qs, mos, macs)
+        return ops.ani_charge(xs.detach(), ys.detach(), zs.detach(), qs.detach(), mos, macs)
+
+    @staticmethod
+    def backward(ctx, grads):
+        xs, ys, zs, qs, mos, macs = ctx.saved_tensors
+        need_xyz = any(ctx.needs_input_grad[:3])
+        args = (xs.detach(), ys.detach(), zs.detach(), qs.detach(), mos, macs, grads.contiguous())
+        if need_xyz:
+            qg, gx, gy, gz = ops.ani_charge_grad_xyz(*args)
+            return gx, gy, gz, qg, None, None
+        return None, None, None, ops.ani_charge_grad(*args), None, None
+
+
+def featurize(xs, ys, zs, as_, mos, macs, sis, acs):
+    """Differentiable `featurize`: -> (h_feat, c_feat, n_feat, o_feat); gradients flow to xs, ys, zs."""
+    return _Featurize.apply(xs, ys, zs, as_, mos, macs, sis, acs)
+
+
+def ani_charge(xs, ys, zs, qs, mos, macs):
+    """Differentiable `ani_charge`: -> charge_energies[n_mols]; gradients flow to qs and to xs, ys, zs."""
+    return _AniCharge.apply(xs, ys, zs, qs, mos, macs)

@@ -346,3 +346,146 @@ def test_charge_reference_fixture_gradient_consistency(ops):
     for m, s in enumerate((slice(0, 8), slice(8, 11))):
         e = host(ops.ani_charge(X, Y, Z, dev(q), mos, macs))[m]
         assert e == pytest.approx(helpers.brute_force_charge_energy(xyz[s], q[s]), rel=1e-12)
+
+
+# ----------------------------------------------------------------------------- crowded centres
+def _packed_ball(rng, n, radius, min_dist):
+    pts = []
+    while len(pts) < n:
+        p = rng.uniform(-radius, radius, 3)
+        if np.linalg.norm(p) <= radius and all(np.linalg.norm(p - q) >= min_dist for q in pts):
+            pts.append(p)
+    return np.array(pts)
+
+
+def test_crowded_centres_take_the_fallback(ops):
+    # molecules of at most 64 atoms in which centres have more than 32 partners inside the 3.1 A angular
+    # cutoff: the one-wavefront-per-molecule kernels keep 32 per centre and must redo such a centre with
+    # the general per-centre routine.  Mixed with ordinary molecules in the same workgroup.
+    say("case: centres with more than 32 angular partners")
+    rng = np.random.default_rng(31)
+    mols = []
+    small = datagen.make_batch("organic", 3, first_mol=5)
+    for m in range(3):
+        s = slice(small.MOs[m], small.MOs[m] + small.MACs[m])
+        mols.append((small.A[s], np.stack([small.X[s], small.Y[s], small.Z[s]], axis=1)))
+    mols.insert(1, (rng.integers(0, 4, 60), _packed_ball(rng, 60, 2.3, 0.85)))       # every centre crowded
+    # a dumbbell: a crowded ball joined to a sparse tail, so only some centres overflow
+    ball = _packed_ball(rng, 40, 2.0, 0.85)
+    # (jittered: exactly collinear triples have no derivative, the oracle returns NaN for them)
+    tail = np.array([[2.5 + 1.1 * k, 0.2 * (-1) ** k, 0.0] for k in range(12)]) + rng.uniform(-0.05, 0.05, (12, 3))
+    mols.append((rng.integers(0, 4, 52), np.concatenate([ball, tail])))
+    mols.append((np.full(45, 1), _packed_ball(rng, 45, 2.1, 0.85)))                   # one type only
+    A = np.concatenate([m[0] for m in mols]).astype(np.int32)
+    xyz = np.concatenate([m[1] for m in mols])
+    mi = np.concatenate([np.full(len(m[0]), k) for k, m in enumerate(mols)]).astype(np.int32)
+    c = Case(xyz[:, 0], xyz[:, 1], xyz[:, 2], A, mi, len(mols))
+    # the premise of the test: some centre really has more than 32 angular partners
+    worst = 0
+    for m in range(len(mols)):
+        p = mols[m][1]
+        dm = np.linalg.norm(p[:, None] - p[None], axis=2)
+        worst = max(worst, int(((dm < 3.1) & (dm > 0)).sum(axis=1).max()))
+    assert worst > 32, worst
+    check_forward_backward(ops, c)
+
+
+# ----------------------------------------------------------------------------- full-size batch
+def test_full_size_batch_properties(ops):
+    # 65,536 molecules (the benchmark batch) in float32: properties that need no oracle at full size, plus
+    # the oracle on the first and last 256 molecules.
+    say("case: organic 65536, full-size properties")
+    M = 65536
+    b = datagen.make_batch("organic", M)
+    c = Case.from_batch(b)
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+    assert np.array_equal(host(sc), c.sc) and np.array_equal(host(ga), c.ga) and np.array_equal(host(ac), c.ac)
+    assert np.array_equal(host(macs), c.MACs) and np.array_equal(host(mos), c.MOs)
+    # ga is the inverse of the bucket placement: sorted-by-type rows gathered back give atom order
+    acs = ac.cpu()
+    X, Y, Z, A = dev(c.X), dev(c.Y), dev(c.Z), dev(c.A)
+    f = ops.featurize(X, Y, Z, A, mos, macs, sc, acs)
+    rows = torch.cat(f).view(-1, 384)[ga.long()]          # [N, 384] in atom order
+    assert bool(torch.isfinite(rows).all())
+    assert float(rows.min()) >= 0.0                        # every term of every feature is non-negative
+    up = torch.from_numpy(datagen.normal(c.N * 384)).to("cuda:0").view(-1, 384)
+    inv = torch.empty_like(ga.long())
+    inv[ga.long()] = torch.arange(c.N, device="cuda:0")
+    upb_all = up[inv]                                      # upstream rows in bucket order
+    gb, start = [], 0
+    for k in acs.tolist():
+        gb.append(upb_all[start:start + k].reshape(-1))
+        start += k
+    gx, gy, gz = ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *gb)
+    g = torch.stack([gx, gy, gz], dim=1)
+    assert bool(torch.isfinite(g).all())
+    # translation invariance: the gradient components of a molecule add up to zero
+    seg = torch.from_numpy(c.mol_idxs.astype(np.int64)).to("cuda:0")
+    net = torch.zeros(M, 3, device="cuda:0", dtype=torch.float64).index_add_(0, seg, g.double())
+    mag = torch.zeros(M, 3, device="cuda:0", dtype=torch.float64).index_add_(0, seg, g.double().abs())
+    rel = (net.abs() / (mag + 1e-30)).max().item()
+    say("   net force / sum |force| per molecule, worst %.3e" % rel)
+    assert rel < 2e-5
+    # batch independence: a molecule's rows do not depend on what else is in the batch -- bit for bit
+    for first, cnt in ((0, 256), (M - 256, 256), (30000, 64)):
+        sb = datagen.make_batch("organic", cnt, first_mol=first)
+        sc_ = Case.from_batch(sb)
+        a0 = int(c.MOs[first])
+        assert np.array_equal(sb.X, c.X[a0:a0 + sb.n_atoms])
+        m2, o2, s2, g2, c2 = gpu_sort_offsets(ops, sc_)
+        f2 = ops.featurize(dev(sb.X), dev(sb.Y), dev(sb.Z), dev(sb.A), o2, m2, s2, c2.cpu())
+        rows2 = torch.cat(f2).view(-1, 384)[g2.long()]
+        assert torch.equal(rows2, rows[a0:a0 + sb.n_atoms])
+        ref64 = ob.gather_rows(sc_.oracle_feat(np.float64), sc_.ga)
+        assert_close("rows of molecules %d.. vs f64 oracle" % first, host(rows2), ref64, F32_RTOL, F32_ATOL)
+        upb = ob.scatter_rows(host(up[a0:a0 + sb.n_atoms]).astype(np.float64), sb.A, sc_.sc, sc_.ac)
+        g64 = sc_.oracle_grad(upb)
+        assert_close("gradient of molecules %d.. vs f64 oracle" % first, host(g[a0:a0 + sb.n_atoms]), g64,
+                     F32_RTOL, F32_ATOL, scale=mol_scale(g64, sc_.MOs, sc_.MACs))
+
+
+# ----------------------------------------------------------------------------- autograd wiring
+def test_autograd_wiring(ops):
+    say("case: torch.autograd wiring of featurize and ani_charge")
+    from khan_amd import autograd as kag
+    b = datagen.make_batch("organic", 16, first_mol=100)
+    c = Case.from_batch(b)
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+    acs = ac.cpu()
+    A = dev(c.A)
+    X, Y, Z = (dev(v, np.float64).requires_grad_(True) for v in (c.X, c.Y, c.Z))
+    w = torch.from_numpy(np.random.default_rng(3).standard_normal(c.N * 384)).to("cuda:0")
+    feats = kag.featurize(X, Y, Z, A, mos, macs, sc, acs)
+    loss = (torch.cat(feats) * w).sum()
+    loss.backward()
+    wb, start = [], 0
+    for k in acs.tolist():
+        wb.append(w[start * 384:(start + k) * 384])
+        start += k
+    gx, gy, gz = ops.featurize_grad(X.detach(), Y.detach(), Z.detach(), A, mos, macs, sc, acs, *wb)
+    # (the float64 kernels add forces with atomics, so two runs differ in the last bits)
+    same = lambda a, b: torch.allclose(a, b, rtol=1e-11, atol=1e-11)
+    assert same(X.grad, gx) and same(Y.grad, gy) and same(Z.grad, gz)
+    # central difference of the loss along one random direction, float64
+    rng = np.random.default_rng(5)
+    d = [dev(rng.standard_normal(c.N)) for _ in range(3)]
+    h = 1e-5
+
+    def L(s):
+        f = ops.featurize(X.detach() + s * d[0], Y.detach() + s * d[1], Z.detach() + s * d[2], A, mos, macs, sc, acs)
+        return float((torch.cat(f) * w).sum())
+    num = (L(h) - L(-h)) / (2 * h)
+    ana = float((gx * d[0]).sum() + (gy * d[1]).sum() + (gz * d[2]).sum())
+    say("   directional derivative: numeric %.10e analytic %.10e" % (num, ana))
+    assert abs(num - ana) <= 1e-6 * max(1.0, abs(ana))
+
+    q = dev(datagen.charges(c.N).astype(np.float64)).requires_grad_(True)
+    X2, Y2, Z2 = (dev(v, np.float64).requires_grad_(True) for v in (c.X, c.Y, c.Z))
+    gm = dev(np.random.default_rng(6).standard_normal(c.n_mols))
+    (kag.ani_charge(X2, Y2, Z2, q, mos, macs) * gm).sum().backward()
+    qg, cx, cy, cz = ops.ani_charge_grad_xyz(X2.detach(), Y2.detach(), Z2.detach(), q.detach(), mos, macs, gm)
+    assert same(q.grad, qg) and same(X2.grad, cx) and same(Y2.grad, cy) and same(Z2.grad, cz)
+    # only the charges need a gradient: the reference's own wiring
+    q3 = q.detach().clone().requires_grad_(True)
+    (kag.ani_charge(X2.detach(), Y2.detach(), Z2.detach(), q3, mos, macs) * gm).sum().backward()
+    assert same(q3.grad, qg)
