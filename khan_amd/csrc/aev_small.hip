@@ -39,16 +39,16 @@ struct __align__(16) SmallLds {
     int nR[4][4];               // radial partners per type, per group of the scan step
 };
 
-__global__ __launch_bounds__(256) void aev_fwd_small_kernel(
+__global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) void aev_fwd_small_kernel(
     const float* __restrict__ X, const float* __restrict__ Y, const float* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
     Buckets<float> out)
 {
-    __shared__ SmallLds lds_all[4];
+    __shared__ SmallLds lds_all[kWavesPerBlock];
     const int lane = threadIdx.x & 63;
     const int wave = uniform(threadIdx.x >> 6);
-    const int mol = blockIdx.x * 4 + wave;
+    const int mol = blockIdx.x * kWavesPerBlock + wave;
     if (mol >= n_mols) return;
     const int n = uniform(MACs[mol]);
     const int off = uniform(MOs[mol]);
@@ -403,8 +403,8 @@ hipError_t launch_fwd_small_f32(const float* X, const float* Y, const float* Z, 
                                 const int32_t* SIs, Buckets<float> out, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
-    const unsigned blocks = (static_cast<unsigned>(n_mols) + 3u) / 4u;
-    aev_fwd_small_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, out);
+    const unsigned blocks = (static_cast<unsigned>(n_mols) + kWavesPerBlock - 1u) / kWavesPerBlock;
+    aev_fwd_small_kernel<<<dim3(blocks), dim3(64 * kWavesPerBlock), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, out);
     return hipGetLastError();
 }
 

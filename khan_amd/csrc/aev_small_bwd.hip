@@ -39,16 +39,16 @@ struct __align__(16) BwdLds {
     unsigned char inv[64];               // original atom index -> sorted lane
 };
 
-__global__ __launch_bounds__(256) void aev_bwd_small_kernel(
+__global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) void aev_bwd_small_kernel(
     const float* __restrict__ X, const float* __restrict__ Y, const float* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
     Buckets<const float> gin, float* __restrict__ gX, float* __restrict__ gY, float* __restrict__ gZ)
 {
-    __shared__ BwdLds lds_all[4];
+    __shared__ BwdLds lds_all[kWavesPerBlock];
     const int lane = threadIdx.x & 63;
     const int wave = uniform(threadIdx.x >> 6);
-    const int mol = blockIdx.x * 4 + wave;
+    const int mol = blockIdx.x * kWavesPerBlock + wave;
     if (mol >= n_mols) return;
     const int n = uniform(MACs[mol]);
     const int off = uniform(MOs[mol]);
@@ -367,8 +367,8 @@ hipError_t launch_bwd_small_f32(const float* X, const float* Y, const float* Z, 
                                 float* gZ, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
-    const unsigned blocks = (static_cast<unsigned>(n_mols) + 3u) / 4u;
-    aev_bwd_small_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ);
+    const unsigned blocks = (static_cast<unsigned>(n_mols) + kWavesPerBlock - 1u) / kWavesPerBlock;
+    aev_bwd_small_kernel<<<dim3(blocks), dim3(64 * kWavesPerBlock), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ);
     return hipGetLastError();
 }
 
