@@ -1,20 +1,25 @@
 // AEV backward (dL/dxyz) for molecules of up to 64 atoms, float32: one wavefront per molecule.
 //
-// Lanes are sorted by atom type and centres are scanned six at a time exactly as in the forward
-// kernel, producing per-centre lists of angular partners (unit vector, distance, f_C, f_C').  Then
+// Lanes are sorted by atom type as in the forward kernel.  A first sweep counts the angular partners
+// of every atom; centres are then taken in order of decreasing count, in batches of up to six whose
+// partner lists together fill at most the 64 lanes.  Per batch:
+//   stage    the 320 angular upstream values of each centre's row are fetched with full-line loads
+//            (issued before the scan, so their latency is covered) and laid out in LDS by type pair;
+//   scan     64 (centre, partner) pairs per step; angular partners (unit vector, distance, f_C, f_C')
+//            go to one pooled list, centre after centre;
 //   radial   a lane owns one (centre, partner) pair: it reads the 16 upstream values of the partner's
 //            type from the centre's row, sums g e (f_C' - 2 eta d f_C) over the shells, and the pull
 //            goes to the partner (one group at a time, so targets are distinct) and, summed over the
 //            group with DPP moves, to the centre;
-//   angular  a lane owns one list entry (centre b, partner j) and walks the other partners of the
-//            same centre in round-robin order, k = j+1, j+2, ... (mod m): in every round all lanes of
-//            a centre hold distinct j AND distinct k, each unordered pair {j,k} is met exactly once,
-//            and all lanes finish together.  A lane computes its triple completely (32 upstream
-//            values read straight from the row, three weighted sums formed serially, no cross-lane
-//            reduction), keeps the force on j in registers and adds the force on k to a per-centre
-//            slot in LDS with a plain read-add-write: targets are distinct by construction, so no
-//            atomics are needed (float atomics on LDS cost ~190 cycles per wave instruction here);
-//   gather   per centre, the slot of every partner is added to its atom's force, and the centre gets
+//   angular  lane = one list entry (centre b, partner j).  It walks the other partners of the same
+//            centre in round-robin order, k = j+1, j+2, ... (mod m): in every round all lanes of a
+//            centre hold distinct j AND distinct k, each unordered pair {j,k} is met exactly once.
+//            A lane computes its triple completely (32 upstream values from the staged block, three
+//            weighted sums formed serially, no cross-lane reduction), keeps the force on j in
+//            registers and adds the force on k to slot k of the pooled list with a plain
+//            read-add-write: targets are distinct by construction, so no atomics are needed (float
+//            atomics on LDS cost ~190 cycles per wave instruction here);
+//   gather   centre by centre, every partner's slot is added to its atom's force, and the centre gets
 //            minus the sum (each row's forces add up to zero by translation invariance).
 // Finally every lane stores the gradient of its own atom: no global atomics, no pre-zeroed output.
 // The derivative is the algebraically reduced form (no acos, no 1/(1+cos) factor); reference:
@@ -28,32 +33,38 @@ namespace {
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef const __attribute__((address_space(1))) v4f* global_v4f_ptr;
 
+constexpr int kBlockStride = 36;   // floats between staged 32-float blocks: rotates the LDS banks
+
 struct __align__(16) BwdLds {
-    float4 atom[64];                     // x, y, z, type (sorted order)
-    float4 nbr[kB][kCapA];               // unit vector (centre minus partner)/r, and r
-    float4 facc[kB][kCapA];              // force on each partner from its centre's row (xyz, pad)
-    float2 nbr_fc[kB][kCapA];            // f_C(r, A_Rc) and its derivative in r
-    float force[3][64];                  // dL/dx, dL/dy, dL/dz per sorted atom
-    int nM[8];                           // angular partners per centre of the batch
-    unsigned char nbr_idx[kB][kCapA];    // sorted lane of the partner
-    unsigned char inv[64];               // original atom index -> sorted lane
+    float4 atom[64];                              // x, y, z, type (sorted order)
+    float4 nbr[64];                               // pooled lists: unit vector (centre minus partner)/r, and r
+    float4 facc[64];                              // force on each list entry from its centre's row
+    float2 nbr_fc[64];                            // f_C(r, A_Rc) and its derivative in r
+    float gst[kB * kNumPairBlocks * kBlockStride];   // staged upstream blocks [centre][type pair][32]
+    float force[3][64];                           // dL/dx, dL/dy, dL/dz per sorted atom
+    int nM[8];                                    // angular partners per centre of the batch
+    unsigned char nbr_idx[64];                    // sorted lane of the partner
+    unsigned char inv[64];                        // original atom index -> sorted lane
 };
 
-__global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) void aev_bwd_small_kernel(
+__device__ __forceinline__ int sel6(int b, int v0, int v1, int v2, int v3, int v4, int v5)
+{
+    return b == 0 ? v0 : b == 1 ? v1 : b == 2 ? v2 : b == 3 ? v3 : b == 4 ? v4 : v5;
+}
+
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void aev_bwd_small_kernel(
     const float* __restrict__ X, const float* __restrict__ Y, const float* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
     Buckets<const float> gin, float* __restrict__ gX, float* __restrict__ gY, float* __restrict__ gZ)
 {
-    __shared__ BwdLds lds_all[kWavesPerBlock];
-    const int lane = threadIdx.x & 63;
-    const int wave = uniform(threadIdx.x >> 6);
-    const int mol = blockIdx.x * kWavesPerBlock + wave;
+    __shared__ BwdLds S;
+    const int lane = threadIdx.x;
+    const int mol = blockIdx.x;
     if (mol >= n_mols) return;
     const int n = uniform(MACs[mol]);
     const int off = uniform(MOs[mol]);
     if (n <= 0 || n > 64) return;                 // larger molecules belong to the general kernel
-    BwdLds& S = lds_all[wave];
     const LaneConsts<float> L = lane_consts<float>(lane);
     const unsigned long long lane_bit = 1ull << lane;
     const unsigned long long lt_mask = lane_bit - 1ull;
@@ -123,23 +134,87 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
     const int tb1 = tbase[1], tb2 = tbase[2], tb3 = tbase[3];
     auto type_of = [&](int sorted_lane) { return (sorted_lane >= tb1) + (sorted_lane >= tb2) + (sorted_lane >= tb3); };
     wave_lds_fence();
+    const float4 aj = S.atom[jl];      // the partner this lane tests in every scan step
 
-    for (int c0 = 0; c0 < n; c0 += kB) {
-        const int nb = min(kB, n - c0);
+    // ------------------------------------------------------------ order of the centres
+    // Angular partner count of every atom, then centres in order of decreasing count: a batch of
+    // centres shares the lanes of the round-robin walk and runs as long as its busiest centre, so
+    // centres with similar counts go together and a batch is cut where its lists fill the 64 lanes.
+    int cord, m_at;     // lane p: sorted lane of the centre at position p, and its partner count
+    {
+        int m_mine = 0;
+        for (int s0 = 0; s0 < n; s0 += G) {
+            const int i = s0 + grp;
+            const float4 ai = S.atom[min(i, 63)];
+            const float dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
+            const float r = sqrtf(dx * dx + dy * dy + dz * dz);
+            const bool inA = (i < n) && (jl < n) && (jl != i) && (r < kA_Rc_f);
+            const int cnt = popc64(wave_ballot(inA) & sub_mask);          // in every lane of the group
+            const int got = __builtin_amdgcn_ds_bpermute((((lane - s0) << logW) & 63) << 2, cnt);
+            if (lane >= s0 && lane < s0 + G) m_mine = got;
+        }
+        const int key = have ? ((m_mine << 6) | (63 - lane)) : -1;
+        int rank = 0;
+        for (int l = 0; l < n; ++l) rank += (lane_read(key, l) > key) ? 1 : 0;
+        if (!have) rank = lane;
+        cord = lane_push(rank, lane);
+        m_at = lane_push(rank, m_mine);
+    }
+
+    for (int c0 = 0, nb = 0; c0 < n; c0 += nb) {
+        // centres of this batch: up to kB, lists fitting the 64 lanes; pf[b] = first list slot of centre b
+        int pf[kB + 1];
+        {
+            bool open = true;
+            int tot = 0;
+            nb = 0;
+            pf[0] = 0;
+#pragma unroll
+            for (int k = 0; k < kB; ++k) {
+                int m = 0;
+                if (open && c0 + k < n) {
+                    m = lane_read(m_at, min(c0 + k, 63));
+                    if (k > 0 && tot + m > 64) {
+                        open = false;
+                        m = 0;
+                    } else {
+                        ++nb;
+                    }
+                } else {
+                    open = false;
+                }
+                tot += m;
+                pf[k + 1] = tot;
+            }
+        }
+        const int total = pf[kB];
         unsigned overflow = 0;
-        for (int q = lane; q < kB * kCapA; q += 64) (&S.facc[0][0])[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+
+        // ---- fetch the angular upstream blocks of the batch's rows (80 x 16 bytes per row)
+        v4f st0[kB], st1[kB];
+#pragma unroll
+        for (int b = 0; b < kB; ++b) {
+            st0[b] = v4f{0.f, 0.f, 0.f, 0.f};
+            st1[b] = v4f{0.f, 0.f, 0.f, 0.f};
+            if (b < nb) {
+                const global_v4f_ptr rowp = (global_v4f_ptr)(row_of(lane_read(cord, min(c0 + b, 63))) + kRadial);
+                st0[b] = rowp[lane];
+                if (lane < 16) st1[b] = rowp[64 + lane];
+            }
+        }
+        S.facc[lane] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (lane < 8) S.nM[lane] = 0;
         wave_lds_fence();
 
         // ------------------------------------------------ scan steps: G centres x W partners
         for (int b0 = 0; b0 < nb; b0 += G) {
             const int b = b0 + grp;
-            const int i = c0 + b;
             const bool centre_ok = b < nb;
-            const int ci = centre_ok ? i : 0;
             const int cb = centre_ok ? b : 0;
-            const float4 ai = S.atom[ci];
-            const float4 aj = S.atom[jl];
+            const int i = __builtin_amdgcn_ds_bpermute(min(c0 + cb, 63) << 2, cord);
+            const int base = sel6(cb, pf[0], pf[1], pf[2], pf[3], pf[4], pf[5]);
+            const int room = sel6(cb, pf[1], pf[2], pf[3], pf[4], pf[5], pf[6]) - base;
+            const float4 ai = S.atom[i];
             const float dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
             const float r = sqrtf(dx * dx + dy * dy + dz * dz);
             const bool valid = centre_ok && (jl < n) && (jl != i);
@@ -147,15 +222,15 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
             const bool inA = valid && (r < kA_Rc_f);
             const unsigned long long mA = wave_ballot(inA);
             const int cntA = popc64(mA & sub_mask);
-            const bool fits = cntA <= kCapA;
+            const bool fits = cntA == room;       // the list has the length the first sweep counted
             const float inv = __builtin_amdgcn_rcpf(r);
             if (inA && fits) {
-                const int pos = popc64(mA & ltg_mask);
+                const int pos = base + popc64(mA & ltg_mask);
                 float fc, dfc;
                 cutoff_poly_grad(r * inv_rc_A, inv_rc_A, fc, dfc);
-                S.nbr[cb][pos] = make_float4(dx * inv, dy * inv, dz * inv, r);
-                S.nbr_fc[cb][pos] = make_float2(fc, dfc);
-                S.nbr_idx[cb][pos] = static_cast<unsigned char>(jl);
+                S.nbr[pos] = make_float4(dx * inv, dy * inv, dz * inv, r);
+                S.nbr_fc[pos] = make_float2(fc, dfc);
+                S.nbr_idx[pos] = static_cast<unsigned char>(jl);
             }
             if (jl == 0 && centre_ok) S.nM[b] = fits ? cntA : 0;
             {
@@ -165,9 +240,9 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
             }
 
             // ---- radial pairs: this lane's (centre, partner) pair over its 16 shells
-            const float* grow = row_of_lane(ci);
+            const float* grow = row_of_lane(i);
             float cfx = 0.f, cfy = 0.f, cfz = 0.f;       // this pair's pull on the centre
-            const bool do_rad = inR && fits;              // an overflowing centre is redone as a whole
+            const bool do_rad = inR && fits;              // a centre that does not fit is redone as a whole
             if (do_rad) {
                 const int tj = __float_as_int(aj.w);
                 const global_v4f_ptr gp = (global_v4f_ptr)(grow + tj * kNumRRs);
@@ -207,43 +282,50 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
                 S.force[2][i] += cfz;
             }
         }
+
+        // ---- the fetched upstream blocks go to LDS: chunk c of a row = block c/8, part c%8
+#pragma unroll
+        for (int b = 0; b < kB; ++b) {
+            if (b < nb) {
+                float* blk = &S.gst[b * kNumPairBlocks * kBlockStride];
+                *reinterpret_cast<v4f*>(blk + (lane >> 3) * kBlockStride + (lane & 7) * 4) = st0[b];
+                if (lane < 16) *reinterpret_cast<v4f*>(blk + (8 + (lane >> 3)) * kBlockStride + (lane & 7) * 4) = st1[b];
+            }
+        }
         wave_lds_fence();
 
-        // ------------------------------------------------ angular: lane = (centre, partner j), round robin over k
-        const int4 m03 = *reinterpret_cast<const int4*>(&S.nM[0]);
-        const int4 m47 = *reinterpret_cast<const int4*>(&S.nM[4]);
-        const int p1 = m03.x, p2 = p1 + m03.y, p3 = p2 + m03.z, p4 = p3 + m03.w, p5 = p4 + m47.x;
-        const int total = uniform(p5 + m47.y);
-        for (int pass0 = 0; pass0 < total; pass0 += 64) {
-            const int slot = pass0 + lane;
-            const bool live = slot < total;
-            const int b = (slot >= p1) + (slot >= p2) + (slot >= p3) + (slot >= p4) + (slot >= p5);
-            const int bs = live ? b : 0;
-            const int pb = bs == 0 ? 0 : bs == 1 ? p1 : bs == 2 ? p2 : bs == 3 ? p3 : bs == 4 ? p4 : p5;
-            const int m = bs == 0 ? m03.x : bs == 1 ? m03.y : bs == 2 ? m03.z : bs == 3 ? m03.w : bs == 4 ? m47.x : m47.y;
-            const int e = live ? slot - pb : 0;
+        // ------------------------------------------------ angular: lane = list entry (centre, partner j)
+        {
+            const int4 m03 = *reinterpret_cast<const int4*>(&S.nM[0]);
+            const int4 m47 = *reinterpret_cast<const int4*>(&S.nM[4]);
+            const int b = (lane >= pf[1]) + (lane >= pf[2]) + (lane >= pf[3]) + (lane >= pf[4]) + (lane >= pf[5]);
+            const int bs = lane < total ? b : 0;
+            const int pb = sel6(bs, pf[0], pf[1], pf[2], pf[3], pf[4], pf[5]);
+            const int m = sel6(bs, m03.x, m03.y, m03.z, m03.w, m47.x, m47.y);   // 0 for a centre that did not fit
+            const bool live = (lane < total) && (m > 0);
+            const int e = live ? lane - pb : 0;
             // rounds: d = 1 .. (m-1)/2 for every lane; when m is even one more round for the lower half
             const int full = (m - 1) >> 1;
             const int rounds = live ? full + ((((m & 1) == 0) && (e < (m >> 1))) ? 1 : 0) : 0;
             const int max_rounds = wave_max(rounds);
-            const float4 vj = S.nbr[bs][e];
-            const float2 fj = S.nbr_fc[bs][e];
-            const int tj = type_of(S.nbr_idx[bs][e]);
+            const int self = live ? lane : 0;
+            const float4 vj = S.nbr[self];
+            const float2 fj = S.nbr_fc[self];
+            const int tj = type_of(S.nbr_idx[self]);
             const float inv_rj = __builtin_amdgcn_rcpf(vj.w);
-            const float* grow = row_of_lane(c0 + bs);
+            const float* gbase = &S.gst[bs * kNumPairBlocks * kBlockStride];
             float ajx = 0.f, ajy = 0.f, ajz = 0.f;           // force on j, kept in registers
 
             for (int d = 1; d <= max_rounds; ++d) {
                 const bool act = d <= rounds;
                 int k = e + d;
                 k -= (k >= m) ? m : 0;
-                k = act ? k : 0;
-                const float4 vk = S.nbr[bs][k];
-                const float2 fk = S.nbr_fc[bs][k];
-                const int tk = type_of(S.nbr_idx[bs][k]);
+                const int ks = act ? pb + k : 0;
+                const float4 vk = S.nbr[ks];
+                const float2 fk = S.nbr_fc[ks];
+                const int tk = type_of(S.nbr_idx[ks]);
                 if (act) {
-                    const int pt = pair_block(tj, tk);
-                    const global_v4f_ptr gp = (global_v4f_ptr)(grow + kRadial + pt * kAngBlock);
+                    const v4f* gp = reinterpret_cast<const v4f*>(gbase + pair_block(tj, tk) * kBlockStride);
                     v4f g[8];
 #pragma unroll
                     for (int t = 0; t < 8; ++t) g[t] = gp[t];
@@ -253,18 +335,21 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
                     const float cx = vj.y * vk.z - vj.z * vk.y;
                     const float cy = vj.z * vk.x - vj.x * vk.z;
                     const float cz = vj.x * vk.y - vj.y * vk.x;
-                    // exactly collinear triples have no finite derivative: keep the result finite
-                    const float s = fmaxf(__builtin_amdgcn_sqrtf(cx * cx + cy * cy + cz * cz), 1e-30f);
-                    const float c_over_s = c * __builtin_amdgcn_rcpf(s);
+                    // cot(theta) = c/s has no limit for collinear triples (the angle has a cusp there, the
+                    // reference returns NaN): c s / (s^2 + 1e-12) equals c/s to 1e-7 relative from 0.2 degrees
+                    // off the line and goes to zero on it
+                    const float s2 = cx * cx + cy * cy + cz * cz;
+                    const float s = __builtin_amdgcn_sqrtf(s2);
+                    const float c_over_s = c * s * __builtin_amdgcn_rcpf(s2 + 1e-12f);
                     const float rho = 0.5f * (vj.w + vk.w);
-                    float Gs[4], Hs[4];
+                    float Gs[4], dds[4];
 #pragma unroll
                     for (int sidx = 0; sidx < 4; ++sidx) {
-                        const float dd = rho - kA_Rs_f[sidx];
-                        Gs[sidx] = __builtin_amdgcn_exp2f(kAngExp * dd * dd);
-                        Hs[sidx] = Gs[sidx] * (-2.0f * kA_eta_f * dd);          // dG/drho
+                        dds[sidx] = rho - kA_Rs_f[sidx];
+                        Gs[sidx] = __builtin_amdgcn_exp2f(kAngExp * dds[sidx] * dds[sidx]);
                     }
-                    float W0 = 0.f, Wc = 0.f, Wr = 0.f;
+                    // X_s = sum_t g_ts A_t and Y_s = sum_t g_ts dA_t/dcos (without its factor 8)
+                    float Xs[4] = {0.f, 0.f, 0.f, 0.f}, Ys[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int t = 0; t < 8; ++t) {
                         const float ct = static_cast<float>(kCosTheta[t]), st = static_cast<float>(kSinTheta[t]);
@@ -272,72 +357,76 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
                         const float b2 = bs1 * bs1, b4 = b2 * b2;
                         const float Am1 = b4 * b2 * bs1;                         // ^7
                         const float At = Am1 * bs1;                              // ^8
-                        const float dAt = 8.0f * Am1 * fmaf(-c_over_s, st, ct);  // d/dcos
-                        const float ut = g[t].x * Gs[0] + g[t].y * Gs[1] + g[t].z * Gs[2] + g[t].w * Gs[3];
-                        const float vt = g[t].x * Hs[0] + g[t].y * Hs[1] + g[t].z * Hs[2] + g[t].w * Hs[3];
-                        W0 = fmaf(At, ut, W0);
-                        Wc = fmaf(dAt, ut, Wc);
-                        Wr = fmaf(At, vt, Wr);
+                        const float dAt = Am1 * fmaf(-c_over_s, st, ct);         // (d/dcos) / 8
+                        Xs[0] = fmaf(g[t].x, At, Xs[0]);
+                        Xs[1] = fmaf(g[t].y, At, Xs[1]);
+                        Xs[2] = fmaf(g[t].z, At, Xs[2]);
+                        Xs[3] = fmaf(g[t].w, At, Xs[3]);
+                        Ys[0] = fmaf(g[t].x, dAt, Ys[0]);
+                        Ys[1] = fmaf(g[t].y, dAt, Ys[1]);
+                        Ys[2] = fmaf(g[t].z, dAt, Ys[2]);
+                        Ys[3] = fmaf(g[t].w, dAt, Ys[3]);
                     }
+                    // W0 = sum G_s X_s, Wc = 8 sum G_s Y_s, Wr = sum (dG_s/drho) X_s with dG/drho = -2 eta dd G
+                    const float gx0 = Gs[0] * Xs[0], gx1 = Gs[1] * Xs[1], gx2 = Gs[2] * Xs[2], gx3 = Gs[3] * Xs[3];
+                    const float W0 = (gx0 + gx1) + (gx2 + gx3);
+                    const float Wc = 8.0f * fmaf(Gs[0], Ys[0], fmaf(Gs[1], Ys[1], fmaf(Gs[2], Ys[2], Gs[3] * Ys[3])));
+                    const float Wr = (-2.0f * kA_eta_f) * fmaf(dds[0], gx0, fmaf(dds[1], gx1, fmaf(dds[2], gx2, dds[3] * gx3)));
                     const float two_pow = 0.0078125f;
                     const float P = two_pow * fj.x * fk.x;
                     const float Fj = fmaf(P * 0.5f, Wr, two_pow * W0 * fj.y * fk.x);    // dE/dr_ij
                     const float Fk = fmaf(P * 0.5f, Wr, two_pow * W0 * fj.x * fk.y);    // dE/dr_ik
                     const float Fc = P * Wc;                                            // dE/dcos
                     const float ij = Fc * inv_rj, ik = Fc * __builtin_amdgcn_rcpf(vk.w);
-                    ajx -= fmaf(Fj, vj.x, ij * (vk.x - c * vj.x));
-                    ajy -= fmaf(Fj, vj.y, ij * (vk.y - c * vj.y));
-                    ajz -= fmaf(Fj, vj.z, ij * (vk.z - c * vj.z));
+                    // force on j = -[Fj u_j + ij (u_k - c u_j)]; the bracket's second part is formed first, it
+                    // is small near the line where ij is large
+                    ajx = fmaf(-Fj, vj.x, fmaf(-ij, fmaf(-c, vj.x, vk.x), ajx));
+                    ajy = fmaf(-Fj, vj.y, fmaf(-ij, fmaf(-c, vj.y, vk.y), ajy));
+                    ajz = fmaf(-Fj, vj.z, fmaf(-ij, fmaf(-c, vj.z, vk.z), ajz));
                     // force on k: in a round every lane of a centre holds a different k
-                    float4 fk_acc = S.facc[bs][k];
-                    fk_acc.x -= fmaf(Fk, vk.x, ik * (vj.x - c * vk.x));
-                    fk_acc.y -= fmaf(Fk, vk.y, ik * (vj.y - c * vk.y));
-                    fk_acc.z -= fmaf(Fk, vk.z, ik * (vj.z - c * vk.z));
-                    S.facc[bs][k] = fk_acc;
+                    float4 fk_acc = S.facc[ks];
+                    fk_acc.x = fmaf(-Fk, vk.x, fmaf(-ik, fmaf(-c, vk.x, vj.x), fk_acc.x));
+                    fk_acc.y = fmaf(-Fk, vk.y, fmaf(-ik, fmaf(-c, vk.y, vj.y), fk_acc.y));
+                    fk_acc.z = fmaf(-Fk, vk.z, fmaf(-ik, fmaf(-c, vk.z, vj.z), fk_acc.z));
+                    S.facc[ks] = fk_acc;
                 }
                 wave_lds_fence();
             }
-            if (live) {
-                float4 f = S.facc[bs][e];
-                f.x += ajx;
-                f.y += ajy;
-                f.z += ajz;
-                S.facc[bs][e] = f;
+
+            // -------------------------------------------- gather: partners get their slot, the centre minus the sum
+            float4 f = S.facc[self];
+            f.x = live ? f.x + ajx : 0.f;
+            f.y = live ? f.y + ajy : 0.f;
+            f.z = live ? f.z + ajz : 0.f;
+            const int atom = S.nbr_idx[self];
+            for (int bb = 0; bb < nb; ++bb) {
+                if (uniform(pf[bb + 1] - pf[bb]) == 0) continue;
+                const bool mine = live && (bs == bb);
+                if (mine) {
+                    S.force[0][atom] += f.x;
+                    S.force[1][atom] += f.y;
+                    S.force[2][atom] += f.z;
+                }
+                const float sx = group_sum_to_last_lane(mine ? f.x : 0.f, 6);
+                const float sy = group_sum_to_last_lane(mine ? f.y : 0.f, 6);
+                const float sz = group_sum_to_last_lane(mine ? f.z : 0.f, 6);
+                if (lane == 63) {
+                    const int i_b = lane_read(cord, min(c0 + bb, 63));
+                    S.force[0][i_b] -= sx;
+                    S.force[1][i_b] -= sy;
+                    S.force[2][i_b] -= sz;
+                }
+                wave_lds_fence();
             }
-            wave_lds_fence();
         }
 
-        // ------------------------------------------------ gather: partners get their slot, the centre minus the sum
-        for (int b = 0; b < nb; ++b) {
-            const int m = b == 0 ? m03.x : b == 1 ? m03.y : b == 2 ? m03.z : b == 3 ? m03.w : b == 4 ? m47.x : m47.y;
-            const int mu = uniform(m);
-            if (mu == 0) continue;
-            float4 f = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (lane < mu) {
-                f = S.facc[b][lane];
-                const int atom = S.nbr_idx[b][lane];
-                S.force[0][atom] += f.x;
-                S.force[1][atom] += f.y;
-                S.force[2][atom] += f.z;
-            }
-            const float sx = group_sum_to_last_lane(f.x, 6);
-            const float sy = group_sum_to_last_lane(f.y, 6);
-            const float sz = group_sum_to_last_lane(f.z, 6);
-            if (lane == 63) {
-                S.force[0][c0 + b] -= sx;
-                S.force[1][c0 + b] -= sy;
-                S.force[2][c0 + b] -= sz;
-            }
-            wave_lds_fence();
-        }
-
-        // ------------------------------------------------ centres whose list overflowed
+        // ------------------------------------------------ centres whose list did not match the first sweep
         if (overflow) {
             for (int b = 0; b < nb; ++b) {
                 if (overflow & (1u << b)) {
-                    const int i_orig = lane_read(orig, c0 + b);
-                    bwd_center_generic<float>(L, lane, X, Y, Z, A, off, n, i_orig,
-                                              reinterpret_cast<float*>(S.nbr), row_of(c0 + b),
+                    const int i_b = lane_read(cord, min(c0 + b, 63));
+                    const int i_orig = lane_read(orig, i_b);
+                    bwd_center_generic<float>(L, lane, X, Y, Z, A, off, n, i_orig, S.gst, row_of(i_b),
                                               [&](int atom, float fx, float fy, float fz) {
                                                   const int sl = S.inv[atom];
                                                   atomicAdd(&S.force[0][sl], fx);
@@ -367,8 +456,7 @@ hipError_t launch_bwd_small_f32(const float* X, const float* Y, const float* Z, 
                                 float* gZ, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
-    const unsigned blocks = (static_cast<unsigned>(n_mols) + kWavesPerBlock - 1u) / kWavesPerBlock;
-    aev_bwd_small_kernel<<<dim3(blocks), dim3(64 * kWavesPerBlock), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ);
+    aev_bwd_small_kernel<<<dim3(static_cast<unsigned>(n_mols)), dim3(64), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ);
     return hipGetLastError();
 }
 
