@@ -217,7 +217,17 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
 
         // ------------------------------------------------ segment table of the batch
         int cnt = 0, packed = 0;
-        float rcp_na = 0.f;
+        unsigned seg_row_lo = 0, seg_row_hi = 0;          // where the segment's 32 floats go
+        {
+            // row of the segment's centre (every lane takes part in the lane exchange)
+            const int cl = min(c0 + min(seg_b, kB - 1), 63);
+            const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(cl << 2, rp_lo));
+            const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(cl << 2, rp_hi));
+            const unsigned long long rowp = ((static_cast<unsigned long long>(hi) << 32) | lo) +
+                                            static_cast<unsigned long long>((kRadial + seg_pt * kAngBlock) * sizeof(float));
+            seg_row_lo = static_cast<unsigned>(rowp);
+            seg_row_hi = static_cast<unsigned>(rowp >> 32);
+        }
         if (lane < nb * kNumPairBlocks) {
             const int4 nn = *reinterpret_cast<const int4*>(S.nA[seg_b]);
             const int na = sel4(seg_a, nn.x, nn.y, nn.z, nn.w);
@@ -227,7 +237,6 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
             const bool same = seg_a == seg_bt;
             cnt = same ? (na * (na - 1)) / 2 : na * nbt;
             packed = seg_b | (oa << 3) | (ob << 9) | (na << 15) | (same ? (1 << 21) : 0) | (seg_pt << 22);
-            rcp_na = na > 0 ? __builtin_amdgcn_rcpf(static_cast<float>(na)) : 0.f;
         }
         const int padded = (cnt + 1) & ~1;
         const int incl = scan_add(padded);
@@ -238,20 +247,25 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
         wave_lds_fence();
         if (cnt > 0) {
             SegDesc d;
-            d.start = start;
-            d.cnt = cnt;
+            d.start_cnt = start | (cnt << 12);
             d.packed = packed;
-            d.rcp_na = rcp_na;
+            d.row_lo = seg_row_lo;
+            d.row_hi = seg_row_hi;
             S.seg[popc64(nonempty & lt_mask)] = d;
             atomicOr(&S.bits[start >> 5], 1u << (start & 31));
         }
         wave_lds_fence();
 
         // ------------------------------------------------ phases 1 and 2, 64 triple slots at a time
-        bool open = false;          // a segment's partial sums are in `acc`
-        float acc = 0.f;
-        float* cur_row = nullptr;   // where the open segment's 32 floats go
+        float acc = 0.f;            // partial sums of the open segment
+        unsigned cur_lo = 0, cur_hi = 0;   // where the open segment's 32 floats go (wave-uniform)
         int carry = 0;              // non-empty segments that start before this step
+        // closes the open segment: the halves are added and 32 floats go straight to the row
+        auto flush = [&]() {
+            const float tot = half_wave_sum(acc);
+            float* dst = reinterpret_cast<float*>((static_cast<unsigned long long>(cur_hi) << 32) | cur_lo);
+            if (lane < 32) store_global(dst + lane, tot);
+        };
 
         for (int base = 0; base < total; base += 64) {
             const unsigned w0 = static_cast<unsigned>(uniform(static_cast<int>(S.bits[base >> 5])));
@@ -261,8 +275,8 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
             carry += popc64(starts);
             const SegDesc d = S.seg[max(ord, 0)];
             const int slot = base + lane;
-            const int q = slot - d.start;
-            const bool ok = (slot < total) && (q >= 0) && (q < d.cnt);
+            const int q = slot - (d.start_cnt & 0xfff);
+            const bool ok = (slot < total) && (q >= 0) && (q < (d.start_cnt >> 12));
 
             // decode q -> (j,k) inside the centre's type-sorted list
             int bsel = d.packed & 7;
@@ -274,7 +288,7 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
                 if (((kl + 1) * kl) / 2 <= q) ++kl;
                 jl2 = q - (kl * (kl - 1)) / 2;
             } else {                                        // q = kl * n_a + jl
-                kl = static_cast<int>((static_cast<float>(q) + 0.5f) * d.rcp_na);
+                kl = static_cast<int>((static_cast<float>(q) + 0.5f) * __builtin_amdgcn_rcpf(static_cast<float>(na)));
                 jl2 = q - kl * na;
             }
             int j = oa + jl2, k = ob + kl;
@@ -320,6 +334,11 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
             const float* pa = &S.rec[L.half][ang_t];
             const float* pg = &S.rec[L.half][8 + ang_s];
             unsigned long long mm = starts;
+            if (base == 0) {            // the batch's first segment opens here; nothing to close
+                cur_lo = static_cast<unsigned>(lane_read(static_cast<int>(d.row_lo), 0));
+                cur_hi = static_cast<unsigned>(lane_read(static_cast<int>(d.row_hi), 0));
+                mm &= ~1ull;
+            }
             auto load8 = [&](int q0, float (&av)[8], float (&gv)[8]) {
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
@@ -328,20 +347,19 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
                 }
             };
             auto run8 = [&](int q0, const float (&av)[8], const float (&gv)[8]) {
+                const unsigned m16 = static_cast<unsigned>(mm) & 0xffffu;     // this group's 16 slots
+                mm >>= 16;
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
-                    if (__builtin_expect(static_cast<int>(mm & 1ull), 0)) {
+                    if (__builtin_expect((m16 >> (2 * u)) & 1u, 0)) {
                         // a segment starts at record pair q0+u: close the open one, open the new one
-                        if (open) {
-                            const float tot = half_wave_sum(acc);
-                            if (lane < 32) store_global(cur_row + lane, tot);
-                        }
-                        const int pk = lane_read(d.packed, 2 * (q0 + u));
-                        cur_row = row_of(c0 + (pk & 7)) + kRadial + ((pk >> 22) & 15) * kAngBlock;
-                        open = true;
+                        flush();
+                        int first = 2 * (q0 + u);
+                        asm volatile("" : "+s"(first));      // keeps the lane reads inside this branch
+                        cur_lo = static_cast<unsigned>(lane_read(static_cast<int>(d.row_lo), first));
+                        cur_hi = static_cast<unsigned>(lane_read(static_cast<int>(d.row_hi), first));
                         acc = 0.f;
                     }
-                    mm >>= 2;
                     acc = fmaf(av[u], gv[u], acc);
                 }
             };
@@ -359,10 +377,7 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
             }
             wave_lds_fence();
         }
-        if (open) {
-            const float tot = half_wave_sum(acc);
-            if (lane < 32) store_global(cur_row + lane, tot);
-        }
+        if (total > 0) flush();
 
         // ------------------------------------------------ segments without triples are zeros
         {

@@ -12,10 +12,10 @@ constexpr int kCapA = 32;      // angular neighbours kept per centre
 constexpr int kBitWords = 96;  // 6 centres x (496 triples + padding) fit in 96 x 32 slot bits
 
 struct __align__(16) SegDesc {
-    int start;       // first triple slot of the segment inside the batch (even)
-    int cnt;         // triples in the segment (its slot range is padded to an even length)
-    int packed;      // centre-in-batch | offset of type a | offset of type b | n_a | a==b | pair index
-    float rcp_na;    // 1 / n_a
+    int start_cnt;       // first triple slot of the segment inside the batch (even, low 12 bits) | triples << 12
+    int packed;          // centre-in-batch | offset of type a | offset of type b | n_a | a==b | pair index
+    unsigned row_lo;     // address of the segment's 32 output floats
+    unsigned row_hi;
 };
 
 
