@@ -22,35 +22,27 @@ namespace khan {
 
 namespace {
 
-template <typename T>
-__global__ __launch_bounds__(256) void zero3_kernel(T* a, T* b, T* c, int64_t n)
-{
-    const int64_t g = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-    if (g < n) {
-        a[g] = T(0);
-        b[g] = T(0);
-        c[g] = T(0);
-    }
-}
-
 // ------------------------------------------------------------------------------------ forward
 template <typename T>
 __global__ __launch_bounds__(256) void aev_fwd_generic_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
-    const int32_t* __restrict__ MACs, const int32_t* __restrict__ SIs, Buckets<T> out, int min_atoms)
+    const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs, Buckets<T> out,
+    int min_atoms)
 {
     __shared__ T ang_rows[4][kAngular];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int mol = blockIdx.x;
-    const int n = MACs[mol], off = MOs[mol];
-    if (n < min_atoms) return;        // smaller molecules are handled by the small-molecule kernel
     const LaneConsts<T> L = lane_consts<T>(lane);
     T* ang = ang_rows[wave];
-
-    for (int i = wave; i < n; i += 4) {
-        T* row = out.p[fold_type(A[off + i])] + static_cast<size_t>(SIs[off + i]) * kFeats;
-        fwd_center_generic<T>(L, lane, X, Y, Z, A, off, n, i, ang, row);
+    // a workgroup walks molecules with the grid's stride, so that a launch in which most molecules
+    // belong to the small-molecule kernel costs a few loads per molecule, not a workgroup each
+    for (int mol = blockIdx.x; mol < n_mols; mol += gridDim.x) {
+        const int n = MACs[mol], off = MOs[mol];
+        if (n < min_atoms) continue;
+        for (int i = wave; i < n; i += 4) {
+            T* row = out.p[fold_type(A[off + i])] + static_cast<size_t>(SIs[off + i]) * kFeats;
+            fwd_center_generic<T>(L, lane, X, Y, Z, A, off, n, i, ang, row);
+        }
     }
 }
 
@@ -59,29 +51,45 @@ template <typename T>
 __global__ __launch_bounds__(256) void aev_bwd_generic_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
-    const int32_t* __restrict__ MACs, const int32_t* __restrict__ SIs, Buckets<const T> gin,
-    T* __restrict__ gX, T* __restrict__ gY, T* __restrict__ gZ, int min_atoms)
+    const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
+    Buckets<const T> gin, T* __restrict__ gX, T* __restrict__ gY, T* __restrict__ gZ, int min_atoms)
 {
     __shared__ T g_rows[4][kAngular];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int mol = blockIdx.x;
-    const int n = MACs[mol], off = MOs[mol];
-    if (n < min_atoms) return;        // smaller molecules are handled by the small-molecule kernel
     const LaneConsts<T> L = lane_consts<T>(lane);
     T* g_ang = g_rows[wave];
-
-    for (int i = wave; i < n; i += 4) {
-        const T* grow = gin.p[fold_type(A[off + i])] + static_cast<size_t>(SIs[off + i]) * kFeats;
-        bwd_center_generic<T>(L, lane, X, Y, Z, A, off, n, i, g_ang, grow,
-                              [&](int atom, T fx, T fy, T fz) {
-                                  atomicAdd(&gX[off + atom], fx);
-                                  atomicAdd(&gY[off + atom], fy);
-                                  atomicAdd(&gZ[off + atom], fz);
-                              });
+    for (int mol = blockIdx.x; mol < n_mols; mol += gridDim.x) {
+        const int n = MACs[mol], off = MOs[mol];
+        if (n < min_atoms) continue;        // smaller molecules are handled by the small-molecule kernel
+        // every contribution to this molecule's atoms comes from this workgroup: zero them here, then
+        // accumulate with atomics (no separate fill pass, nothing to pre-zero for the caller)
+        for (int a = threadIdx.x; a < n; a += 256) {
+            gX[off + a] = T(0);
+            gY[off + a] = T(0);
+            gZ[off + a] = T(0);
+        }
+        __syncthreads();
+        for (int i = wave; i < n; i += 4) {
+            const T* grow = gin.p[fold_type(A[off + i])] + static_cast<size_t>(SIs[off + i]) * kFeats;
+            bwd_center_generic<T>(L, lane, X, Y, Z, A, off, n, i, g_ang, grow,
+                                  [&](int atom, T fx, T fy, T fz) {
+                                      atomicAdd(&gX[off + atom], fx);
+                                      atomicAdd(&gY[off + atom], fy);
+                                      atomicAdd(&gZ[off + atom], fz);
+                                  });
+        }
     }
 }
 
 }  // namespace
+
+// Workgroups walk the molecules with the grid's stride.  When only the few molecules above
+// `min_atoms` are wanted, a small grid keeps the cost of skipping the others low.
+static unsigned generic_grid(int32_t n_mols, int min_atoms)
+{
+    const int32_t cap = min_atoms > 1 ? 2048 : (1 << 20);
+    return static_cast<unsigned>(n_mols < cap ? n_mols : cap);
+}
 
 template <typename T>
 hipError_t launch_fwd_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
@@ -89,7 +97,7 @@ hipError_t launch_fwd_generic(const T* X, const T* Y, const T* Z, const int32_t*
                               const int32_t* SIs, Buckets<T> out, int min_atoms, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
-    aev_fwd_generic_kernel<T><<<dim3(n_mols), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, SIs, out, min_atoms);
+    aev_fwd_generic_kernel<T><<<dim3(generic_grid(n_mols, min_atoms)), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, out, min_atoms);
     return hipGetLastError();
 }
 
@@ -99,16 +107,11 @@ hipError_t launch_bwd_generic(const T* X, const T* Y, const T* Z, const int32_t*
                               const int32_t* SIs, Buckets<const T> g, T* gX, T* gY, T* gZ,
                               int64_t n_atoms, int min_atoms, hipStream_t stream)
 {
-    // outputs are accumulated with atomics, so they start from zero (functor_op_cpu.cpp:70-72);
-    // a fill kernel rather than a memset node keeps the sequence safe to capture in a HIP graph
-    if (n_atoms > 0) {
-        const int64_t blocks = (n_atoms + 255) / 256;
-        zero3_kernel<T><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(gX, gY, gZ, n_atoms);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return e;
-    }
+    // the kernel zeroes each molecule's outputs itself before accumulating (the reference zero-fills
+    // first, functor_op_cpu.cpp:70-72); no memset node, so the launch is safe to capture in a HIP graph
+    (void)n_atoms;
     if (n_mols <= 0) return hipSuccess;
-    aev_bwd_generic_kernel<T><<<dim3(n_mols), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, SIs, g, gX, gY, gZ, min_atoms);
+    aev_bwd_generic_kernel<T><<<dim3(generic_grid(n_mols, min_atoms)), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ, min_atoms);
     return hipGetLastError();
 }
 
