@@ -93,6 +93,27 @@ int khan_featurize_grad_f64(const double *xs, const double *ys, const double *zs
                             double *y_grads, double *z_grads, const int32_t *acs_host,
                             khan_stream_t stream);
 
+/* FeaturizeGradInverse (op: gpu_featurizer/ani_op.cpp:309-343; functor: functor_op.h:50-69,
+ * functor_op_cpu.cpp:86-121; kernel: kernel_cpu.cpp:37-179 -- CPU-only in the reference; it is the
+ * gradient of FeaturizeGrad with respect to its upstream gradients, trainer_multi_tower.py:64-91).
+ * in : the Featurize inputs, then x_grads, y_grads, z_grads [sum(acs_host)]: one vector per atom
+ * out: h..o laid out like the Featurize outputs: row_i[f] = sum_a dAEV_i[f]/dxyz_a . (x,y,z)_grads[a].
+ * The reference routine reads the incoming vectors by the centre's atomic number instead of by atom
+ * (kernel_cpu.cpp:111, 118, 155, 162, 169), which makes its result zero for every input; this entry
+ * point computes the contraction that the gradient wiring means, indexed by atom. */
+int khan_featurize_grad_inverse_f32(const float *xs, const float *ys, const float *zs,
+                                    const int32_t *as, const int32_t *mos, const int32_t *macs,
+                                    int32_t n_mols, const int32_t *sis, const float *x_grads,
+                                    const float *y_grads, const float *z_grads, float *h_grads,
+                                    float *c_grads, float *n_grads, float *o_grads,
+                                    const int32_t *acs_host, khan_stream_t stream);
+int khan_featurize_grad_inverse_f64(const double *xs, const double *ys, const double *zs,
+                                    const int32_t *as, const int32_t *mos, const int32_t *macs,
+                                    int32_t n_mols, const int32_t *sis, const double *x_grads,
+                                    const double *y_grads, const double *z_grads, double *h_grads,
+                                    double *c_grads, double *n_grads, double *o_grads,
+                                    const int32_t *acs_host, khan_stream_t stream);
+
 /* AniCharge (gpu_featurizer/ani_charges.cpp:45-52 registration, 58-71 charge_energy, 81-119 Compute;
  * CUDA twin ani_charges_gpu.cu:70-128).
  * in : xs, ys, zs, qs [n_atoms]; mos, macs [n_mols]      out: charge_energies[n_mols] */

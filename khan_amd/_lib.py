@@ -38,6 +38,8 @@ _SIGNATURES = {
     "khan_featurize_f64": (ctypes.c_int, _featurize_sig()),
     "khan_featurize_grad_f32": (ctypes.c_int, _featurize_grad_sig()),
     "khan_featurize_grad_f64": (ctypes.c_int, _featurize_grad_sig()),
+    "khan_featurize_grad_inverse_f32": (ctypes.c_int, _featurize_grad_sig()),
+    "khan_featurize_grad_inverse_f64": (ctypes.c_int, _featurize_grad_sig()),
     "khan_ani_charge_f32": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32, _ptr, _ptr]),
     "khan_ani_charge_f64": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32, _ptr, _ptr]),
     "khan_ani_charge_grad_f32": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32, _ptr, _ptr, _ptr]),

@@ -1,9 +1,13 @@
 """Gradient wiring of the featurization ops for torch.autograd, the counterpart of the
 `ops.RegisterGradient` blocks in khan/training/trainer_multi_tower.py:23-120:
 
-    Featurize   d/d(xs,ys,zs) through `featurize_grad`; no gradient for the index inputs
-                (trainer_multi_tower.py:23-51)
-    AniCharge   d/dqs through `ani_charge_grad` (trainer_multi_tower.py:88-120); here the
+    Featurize      d/d(xs,ys,zs) through `featurize_grad`; no gradient for the index inputs
+                   (trainer_multi_tower.py:23-51)
+    FeaturizeGrad  d/d(upstream gradients) through `featurize_grad_inverse`, so that a loss on forces
+                   can be differentiated with respect to the network parameters; like the reference
+                   it offers no second derivative with respect to the coordinates
+                   (trainer_multi_tower.py:64-91)
+    AniCharge      d/dqs through `ani_charge_grad` (trainer_multi_tower.py:88-120); here the
                 coordinates get a gradient too (`ani_charge_grad_xyz`), which the reference
                 leaves as None
 
@@ -12,6 +16,23 @@ Both call the HIP library through `khan_amd.ops`; there is no other implementati
 import torch
 
 from . import ops
+
+
+class _FeaturizeGrad(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, xs, ys, zs, as_, mos, macs, sis, acs_host, grad_h, grad_c, grad_n, grad_o):
+        ctx.save_for_backward(xs, ys, zs, as_, mos, macs, sis)
+        ctx.acs_host = acs_host
+        return ops.featurize_grad(xs, ys, zs, as_, mos, macs, sis, acs_host,
+                                  grad_h.contiguous(), grad_c.contiguous(), grad_n.contiguous(), grad_o.contiguous())
+
+    @staticmethod
+    def backward(ctx, dx, dy, dz):
+        xs, ys, zs, as_, mos, macs, sis = ctx.saved_tensors
+        zero = lambda: torch.zeros_like(xs)
+        dx, dy, dz = (zero() if d is None else d.contiguous() for d in (dx, dy, dz))
+        dh, dc, dn, do = ops.featurize_grad_inverse(xs, ys, zs, as_, mos, macs, sis, ctx.acs_host, dx, dy, dz)
+        return (None,) * 8 + (dh, dc, dn, do)
 
 
 class _Featurize(torch.autograd.Function):
@@ -29,9 +50,9 @@ class _Featurize(torch.autograd.Function):
         for g, c in zip((grad_h, grad_c, grad_n, grad_o), ctx.acs_host):
             if g is None:
                 g = torch.zeros(c * ops.FEATURE_SIZE, dtype=xs.dtype, device=xs.device)
-            grads.append(g.contiguous())
-        gx, gy, gz = ops.featurize_grad(xs.detach(), ys.detach(), zs.detach(), as_, mos, macs, sis,
-                                        ctx.acs_host, *grads)
+            grads.append(g)
+        gx, gy, gz = _FeaturizeGrad.apply(xs.detach(), ys.detach(), zs.detach(), as_, mos, macs, sis,
+                                          ctx.acs_host, *grads)
         return gx, gy, gz, None, None, None, None, None
 
 

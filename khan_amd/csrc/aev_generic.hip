@@ -46,6 +46,29 @@ __global__ __launch_bounds__(256) void aev_fwd_generic_kernel(
     }
 }
 
+// ------------------------------------------------------------------- Jacobian-vector product
+template <typename T>
+__global__ __launch_bounds__(256) void aev_jvp_generic_kernel(
+    const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
+    const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
+    const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
+    const T* __restrict__ VX, const T* __restrict__ VY, const T* __restrict__ VZ, Buckets<T> out,
+    int min_atoms)
+{
+    __shared__ T ang_rows[4][kAngular];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const LaneConsts<T> L = lane_consts<T>(lane);
+    T* ang = ang_rows[wave];
+    for (int mol = blockIdx.x; mol < n_mols; mol += gridDim.x) {
+        const int n = MACs[mol], off = MOs[mol];
+        if (n < min_atoms) continue;
+        for (int i = wave; i < n; i += 4) {
+            T* row = out.p[fold_type(A[off + i])] + static_cast<size_t>(SIs[off + i]) * kFeats;
+            jvp_center_generic<T>(L, lane, X, Y, Z, A, VX, VY, VZ, off, n, i, ang, row);
+        }
+    }
+}
+
 // ----------------------------------------------------------------------------------- backward
 template <typename T>
 __global__ __launch_bounds__(256) void aev_bwd_generic_kernel(
@@ -102,6 +125,17 @@ hipError_t launch_fwd_generic(const T* X, const T* Y, const T* Z, const int32_t*
 }
 
 template <typename T>
+hipError_t launch_jvp_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
+                              const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                              const int32_t* SIs, const T* VX, const T* VY, const T* VZ, Buckets<T> out,
+                              int min_atoms, hipStream_t stream)
+{
+    if (n_mols <= 0) return hipSuccess;
+    aev_jvp_generic_kernel<T><<<dim3(generic_grid(n_mols, min_atoms)), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, VX, VY, VZ, out, min_atoms);
+    return hipGetLastError();
+}
+
+template <typename T>
 hipError_t launch_bwd_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
                               const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
                               const int32_t* SIs, Buckets<const T> g, T* gX, T* gY, T* gZ,
@@ -117,6 +151,8 @@ hipError_t launch_bwd_generic(const T* X, const T* Y, const T* Z, const int32_t*
 
 template hipError_t launch_fwd_generic<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<float>, int, hipStream_t);
 template hipError_t launch_fwd_generic<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<double>, int, hipStream_t);
+template hipError_t launch_jvp_generic<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const float*, const float*, const float*, Buckets<float>, int, hipStream_t);
+template hipError_t launch_jvp_generic<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const double*, const double*, const double*, Buckets<double>, int, hipStream_t);
 template hipError_t launch_bwd_generic<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const float>, float*, float*, float*, int64_t, int, hipStream_t);
 template hipError_t launch_bwd_generic<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const double>, double*, double*, double*, int64_t, int, hipStream_t);
 

@@ -302,4 +302,148 @@ __device__ __forceinline__ void bwd_center_generic(const LaneConsts<T>& L, int l
         wave_lds_fence();
 }
 
+// Jacobian-vector product of ONE centre atom i (general shape), executed by one whole wavefront:
+// row[f] = sum_a dAEV_i[f]/dx_a . v_a with v_a = (VX[a], VY[a], VZ[a]), a = i and its partners.
+// Lanes hold the output slots as in the forward routine; every term of the forward sum is replaced
+// by its derivative along v:  d r_ij = u_ij.(v_i - v_j),  d cos = ((u_k - c u_j).w_j)/r_j +
+// ((u_j - c u_k).w_k)/r_k.  `ang` is kAngular elements of this wavefront's LDS.
+// Contraction of the reference's featurize_grad_inverse (kernel_cpu.cpp:37-179), with the incoming
+// vectors read by atom index.
+template <typename T>
+__device__ __forceinline__ void jvp_center_generic(const LaneConsts<T>& L, int lane, const T* __restrict__ X,
+                                                   const T* __restrict__ Y, const T* __restrict__ Z,
+                                                   const int32_t* __restrict__ A,
+                                                   const T* __restrict__ VX, const T* __restrict__ VY,
+                                                   const T* __restrict__ VZ, int off, int n, int i,
+                                                   T* ang, T* __restrict__ row)
+{
+        for (int q = lane; q < kAngular; q += 64) ang[q] = T(0);
+        wave_lds_fence();
+        const T xi = X[off + i], yi = Y[off + i], zi = Z[off + i];
+        const T vxi = VX[off + i], vyi = VY[off + i], vzi = VZ[off + i];
+        T acc_rad = T(0);
+
+        // a scanned partner plus what the derivative needs: relative vector w = v_i - v_j, d r = u.w
+        struct Extra {
+            T wx, wy, wz, rd;
+        };
+        auto scan_extra = [&](const Partner<T>& p, int j) {
+            Extra e;
+            e.wx = e.wy = e.wz = e.rd = T(0);
+            if (j < n) {
+                e.wx = vxi - VX[off + j];
+                e.wy = vyi - VY[off + j];
+                e.wz = vzi - VZ[off + j];
+                e.rd = (p.dx * e.wx + p.dy * e.wy + p.dz * e.wz) / p.r;
+            }
+            return e;
+        };
+        auto extra_from_lane = [&](const Extra& e, int src) {
+            Extra q;
+            q.wx = wave_get(e.wx, src);
+            q.wy = wave_get(e.wy, src);
+            q.wz = wave_get(e.wz, src);
+            q.rd = wave_get(e.rd, src);
+            return q;
+        };
+
+        for (int jc = 0; jc < n; jc += 64) {
+            const int j = jc + lane;
+            const Partner<T> pj = scan_partner(X, Y, Z, A, off, j, n, xi, yi, zi);
+            const Extra ej = scan_extra(pj, j);
+            const bool valid = (j < n) && (j != i);
+            const bool inR = valid && (pj.r < L.R_Rc);
+            const bool inA = valid && (pj.r < L.A_Rc);
+            const T fcR = inR ? cutoff_fn(pj.r, L.pi_rc_R) : T(0);
+            const T dfcR = inR ? cutoff_dfn(pj.r, L.pi_rc_R) : T(0);
+            const T fcA = inA ? cutoff_fn(pj.r, L.pi_rc_A) : T(0);
+            const T dfcA = inA ? cutoff_dfn(pj.r, L.pi_rc_A) : T(0);
+
+            // radial: d/dr [exp(-eta d^2) f_C] * d r
+            for (unsigned long long m = wave_ballot(inR); m; m &= m - 1) {
+                const int b = lowest_bit(m);
+                const T rb = wave_get(pj.r, b), fb = wave_get(fcR, b), dfb = wave_get(dfcR, b);
+                const T rdb = wave_get(ej.rd, b);
+                const int tb = wave_get(pj.type, b);
+                const T d = rb - L.rrs;
+                const T g = Real<T>::exp_(-L.R_eta * d * d) * (dfb - T(2) * L.R_eta * d * fb) * rdb;
+                acc_rad += (tb == L.rtype) ? g : T(0);
+            }
+
+            // angular: j from this chunk, k > j from this and later chunks
+            for (unsigned long long mj = wave_ballot(inA); mj; mj &= mj - 1) {
+                const int bj = lowest_bit(mj);
+                const Partner<T> J = partner_from_lane(pj, bj);
+                const Extra Je = extra_from_lane(ej, bj);
+                const T Jfc = wave_get(fcA, bj), Jdfc = wave_get(dfcA, bj);
+                const T Jinv = T(1) / J.r;
+                const T ujx = J.dx * Jinv, ujy = J.dy * Jinv, ujz = J.dz * Jinv;
+                for (int kc = jc; kc < n; kc += 64) {
+                    Partner<T> pk;
+                    Extra ek;
+                    T fcK, dfcK;
+                    bool kin;
+                    if (kc == jc) {
+                        pk = pj;
+                        ek = ej;
+                        fcK = fcA;
+                        dfcK = dfcA;
+                        kin = inA && (lane > bj);
+                    } else {
+                        const int k = kc + lane;
+                        pk = scan_partner(X, Y, Z, A, off, k, n, xi, yi, zi);
+                        ek = scan_extra(pk, k);
+                        kin = (k < n) && (k != i) && (pk.r < L.A_Rc);
+                        fcK = kin ? cutoff_fn(pk.r, L.pi_rc_A) : T(0);
+                        dfcK = kin ? cutoff_dfn(pk.r, L.pi_rc_A) : T(0);
+                    }
+                    unsigned long long mk = wave_ballot(kin);
+                    while (mk) {
+                        const int b0 = lowest_bit(mk);
+                        mk &= mk - 1;
+                        int b1 = -1;
+                        if (mk) {
+                            b1 = lowest_bit(mk);
+                            mk &= mk - 1;
+                        }
+                        const bool act = (L.half == 0) || (b1 >= 0);
+                        const int src = (L.half == 0 || b1 < 0) ? b0 : b1;
+                        const Partner<T> K = partner_from_lane(pk, src);
+                        const Extra Ke = extra_from_lane(ek, src);
+                        const T Kfc = wave_get(fcK, src), Kdfc = wave_get(dfcK, src);
+                        const T Kinv = T(1) / K.r;
+                        const T ukx = K.dx * Kinv, uky = K.dy * Kinv, ukz = K.dz * Kinv;
+
+                        T c = ujx * ukx + ujy * uky + ujz * ukz;
+                        c = fmin(fmax(c, T(-1)), T(1));
+                        const T cx = ujy * ukz - ujz * uky;
+                        const T cy = ujz * ukx - ujx * ukz;
+                        const T cz = ujx * uky - ujy * ukx;
+                        const T s = Real<T>::sqrt_(cx * cx + cy * cy + cz * cz);
+                        const T dc = ((ukx - c * ujx) * Je.wx + (uky - c * ujy) * Je.wy + (ukz - c * ujz) * Je.wz) * Jinv +
+                                     ((ujx - c * ukx) * Ke.wx + (ujy - c * uky) * Ke.wy + (ujz - c * ukz) * Ke.wz) * Kinv;
+                        const T base = T(1) + c * L.ct + s * L.st;
+                        const T b2 = base * base, b4 = b2 * b2;
+                        const T Am1 = b4 * b2 * base;
+                        const T At = Am1 * base;
+                        const T dAt = T(8) * Am1 * (L.ct - cot_reg(c, s) * L.st) * dc;
+                        const T dav = (J.r + K.r) * T(0.5) - L.ars;
+                        const T Gs = Real<T>::exp_(-L.A_eta * dav * dav);
+                        const T dGs = Gs * (T(-2) * L.A_eta * dav) * T(0.5) * (Je.rd + Ke.rd);
+                        const T two_pow = T(0.0078125);
+                        const T P = two_pow * Jfc * Kfc;
+                        const T dP = two_pow * (Jdfc * Je.rd * Kfc + Jfc * Kdfc * Ke.rd);
+                        const T val = dAt * Gs * P + At * (dGs * P + Gs * dP);
+                        if (act) atomicAdd(&ang[pair_block(J.type, K.type) * kAngBlock + L.ts], val);
+                    }
+                }
+            }
+        }
+
+        wave_lds_fence();
+        row[lane] = acc_rad;
+        for (int q = lane; q < kAngular; q += 64) row[kRadial + q] = ang[q];
+        wave_lds_fence();
+}
+
 }  // namespace khan

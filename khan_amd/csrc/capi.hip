@@ -112,6 +112,26 @@ int featurize_grad_impl(const T* xs, const T* ys, const T* zs, const int32_t* as
 }
 
 template <typename T>
+int featurize_grad_inverse_impl(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
+                                const int32_t* macs, int32_t n_mols, const int32_t* sis, const T* vx,
+                                const T* vy, const T* vz, T* h, T* c, T* n, T* o,
+                                const int32_t* acs_host, khan_stream_t stream)
+{
+    if (n_mols < 0 || !acs_host) return KHAN_ERR_INVALID_ARG;
+    if (n_mols == 0) return KHAN_OK;
+    if (acs_host[0] < 0 || acs_host[1] < 0 || acs_host[2] < 0 || acs_host[3] < 0) return KHAN_ERR_INVALID_ARG;
+    const int64_t n_atoms = static_cast<int64_t>(acs_host[0]) + acs_host[1] + acs_host[2] + acs_host[3];
+    if (n_atoms == 0) return KHAN_OK;
+    if (!xs || !ys || !zs || !as || !mos || !macs || !sis || !vx || !vy || !vz) return KHAN_ERR_INVALID_ARG;
+    if ((acs_host[0] && !h) || (acs_host[1] && !c) || (acs_host[2] && !n) || (acs_host[3] && !o))
+        return KHAN_ERR_INVALID_ARG;
+    khan::Buckets<T> out{{h, c, n, o}};
+    // every molecule size and both precisions run on the general-shape kernel
+    return hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, 0,
+                                                  as_stream(stream)));
+}
+
+template <typename T>
 int charge_impl(const T* xs, const T* ys, const T* zs, const T* qs, const int32_t* mos,
                 const int32_t* macs, int32_t n_mols, T* e, khan_stream_t stream)
 {
@@ -225,6 +245,25 @@ int khan_featurize_grad_f64(const double* xs, const double* ys, const double* zs
 {
     return featurize_grad_impl<double>(xs, ys, zs, as, mos, macs, n_mols, sis, gh, gc, gn, go, gx, gy, gz,
                                        acs_host, stream);
+}
+
+int khan_featurize_grad_inverse_f32(const float* xs, const float* ys, const float* zs, const int32_t* as,
+                                    const int32_t* mos, const int32_t* macs, int32_t n_mols,
+                                    const int32_t* sis, const float* x_grads, const float* y_grads,
+                                    const float* z_grads, float* h, float* c, float* n, float* o,
+                                    const int32_t* acs_host, khan_stream_t stream)
+{
+    return featurize_grad_inverse_impl<float>(xs, ys, zs, as, mos, macs, n_mols, sis, x_grads, y_grads, z_grads,
+                                              h, c, n, o, acs_host, stream);
+}
+int khan_featurize_grad_inverse_f64(const double* xs, const double* ys, const double* zs, const int32_t* as,
+                                    const int32_t* mos, const int32_t* macs, int32_t n_mols,
+                                    const int32_t* sis, const double* x_grads, const double* y_grads,
+                                    const double* z_grads, double* h, double* c, double* n, double* o,
+                                    const int32_t* acs_host, khan_stream_t stream)
+{
+    return featurize_grad_inverse_impl<double>(xs, ys, zs, as, mos, macs, n_mols, sis, x_grads, y_grads, z_grads,
+                                               h, c, n, o, acs_host, stream);
 }
 
 int khan_ani_charge_f32(const float* xs, const float* ys, const float* zs, const float* qs,

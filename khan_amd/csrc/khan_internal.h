@@ -17,6 +17,13 @@ hipError_t launch_fwd_generic(const T* X, const T* Y, const T* Z, const int32_t*
                               const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
                               const int32_t* SIs, Buckets<T> out, int min_atoms, hipStream_t stream);
 
+// Jacobian applied to per-atom vectors (VX, VY, VZ): one 384-wide row per atom, laid out like the forward's
+template <typename T>
+hipError_t launch_jvp_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
+                              const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                              const int32_t* SIs, const T* VX, const T* VY, const T* VZ, Buckets<T> out,
+                              int min_atoms, hipStream_t stream);
+
 // ---- AEV forward for molecules of up to 64 atoms, float32 (larger molecules are skipped) ----
 constexpr int kSmallMaxAtoms = 64;
 hipError_t launch_fwd_small_f32(const float* X, const float* Y, const float* Z, const int32_t* A,

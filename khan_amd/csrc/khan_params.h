@@ -60,13 +60,23 @@ template <> struct Real<float> {
     __device__ static __forceinline__ float sqrt_(float x) { return sqrtf(x); }
     __device__ static __forceinline__ float cos_(float x) { return cosf(x); }
     __device__ static __forceinline__ float sin_(float x) { return sinf(x); }
+    static constexpr float kCotEps = 1e-12f;
 };
 template <> struct Real<double> {
     __device__ static __forceinline__ double exp_(double x) { return exp(x); }
     __device__ static __forceinline__ double sqrt_(double x) { return sqrt(x); }
     __device__ static __forceinline__ double cos_(double x) { return cos(x); }
     __device__ static __forceinline__ double sin_(double x) { return sin(x); }
+    static constexpr double kCotEps = 1e-24;
 };
+
+// cot(theta) = c/s from c = cos(theta) and s = sin(theta) >= 0, regularised on the line theta = 0, pi where
+// the angle has a cusp: c s / (s^2 + eps) differs from c/s by eps/s^2 relative and goes to zero with s.
+template <typename T>
+__device__ __forceinline__ T cot_reg(T c, T s)
+{
+    return c * s / (s * s + Real<T>::kCotEps);
+}
 
 // f_C(r, rc) = 0.5 cos(pi r / rc) + 0.5 for r <= rc (kernel_cpu.cpp:29-35); callers only evaluate it
 // inside the strict cutoff, so the r > rc branch is not needed here.

@@ -3,6 +3,7 @@
     ani_sort(as)                                   gpu_featurizer/ani_sort.cpp:27-31
     featurize(xs, ys, zs, as, mos, macs, sis, acs)                 ani_op.cpp:95-107
     featurize_grad(..., acs, h_grads, c_grads, n_grads, o_grads)   ani_op.cpp:200-215
+    featurize_grad_inverse(..., acs, x_grads, y_grads, z_grads)    ani_op.cpp:309-324
     ani_charge(xs, ys, zs, qs, mos, macs)                          ani_charges.cpp:45-52
     ani_charge_grad(xs, ys, zs, qs, mos, macs, grads)              ani_charges.cpp:123-131
     mol_offsets(mol_idxs, n_mols)   the segment_sum + exclusive cumsum the trainer runs first
@@ -137,6 +138,34 @@ def featurize_grad(xs, ys, zs, as_, mos, macs, sis, acs, h_grads, c_grads, n_gra
                   _p(grads[0]), _p(grads[1]), _p(grads[2]), _p(grads[3]), _p(gx), _p(gy), _p(gz),
                   acs_c, _stream()))
     return gx, gy, gz
+
+
+def featurize_grad_inverse(xs, ys, zs, as_, mos, macs, sis, acs, x_grads, y_grads, z_grads):
+    """-> (h_grads, c_grads, n_grads, o_grads) laid out like `featurize`'s outputs: the Jacobian of the
+    features applied to one vector per atom, row_i[f] = sum_a dAEV_i[f]/dxyz_a . (x,y,z)_grads[a].
+    It is the gradient of `featurize_grad` with respect to its upstream gradients
+    (khan/training/trainer_multi_tower.py:64-91)."""
+    lib = _lib.load()
+    dt, n = _check_common(xs, ys, zs, as_, mos, macs, sis)
+    acs_c, acs_v = _acs_host(acs)
+    if sum(acs_v) != n:
+        raise ValueError("sum(acs)=%d does not match the number of atoms %d" % (sum(acs_v), n))
+    vs = []
+    for name, v in zip("xyz", (x_grads, y_grads, z_grads)):
+        v = _dev(v, dt, name + "_grads")
+        if v.numel() != n:
+            raise ValueError("%s_grads has %d elements, expected %d" % (name, v.numel(), n))
+        vs.append(v)
+    packed = torch.empty(n * FEATURE_SIZE, dtype=dt, device=xs.device)
+    outs, start = [], 0
+    for c in acs_v:
+        outs.append(packed[start * FEATURE_SIZE:(start + c) * FEATURE_SIZE])
+        start += c
+    fn = getattr(lib, "khan_featurize_grad_inverse_" + _SUFFIX[dt])
+    _lib.check(fn(_p(xs), _p(ys), _p(zs), _p(as_), _p(mos), _p(macs), mos.numel(), _p(sis),
+                  _p(vs[0]), _p(vs[1]), _p(vs[2]), _p(outs[0]), _p(outs[1]), _p(outs[2]), _p(outs[3]),
+                  acs_c, _stream()))
+    return tuple(outs)
 
 
 def _check_charge(xs, ys, zs, qs, mos, macs):

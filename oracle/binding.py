@@ -137,6 +137,29 @@ def featurize_grad(X, Y, Z, A, MOs, MACs, SIs, acs, grads, dtype=np.float64, imp
     return gx, gy, gz
 
 
+def featurize_grad_inverse(X, Y, Z, A, MOs, MACs, SIs, acs, vX, vY, vZ, dtype=np.float64, impl="oracle", fast=False):
+    """Jacobian applied to per-atom vectors v -> [h, c, n, o] flat buckets.  impl="ref" runs the
+    reference's own routine (which reads v by atom type, not by atom)."""
+    X, Y, Z = _c(X, dtype), _c(Y, dtype), _c(Z, dtype)
+    vX, vY, vZ = _c(vX, dtype), _c(vY, dtype), _c(vZ, dtype)
+    A, MOs, MACs, SIs = _c(A, np.int32), _c(MOs, np.int32), _c(MACs, np.int32), _c(SIs, np.int32)
+    acs = _c(acs, np.int32)
+    outs = [np.zeros(int(c) * FEATS, dtype=dtype) for c in acs]
+    sfx = _suffix(dtype)
+    if impl == "ref":
+        lib = ref_lib(fast)
+        if lib is None:
+            raise RuntimeError("oracle/_ref not built")
+        fn = getattr(lib, "ref_featurize_grad_inverse_" + sfx)
+        fn(_p(X), _p(Y), _p(Z), _p(A), _p(MOs), _p(MACs), _i32(MOs.size), _p(SIs), _p(vX), _p(vY), _p(vZ),
+           _p(outs[0]), _p(outs[1]), _p(outs[2]), _p(outs[3]), _p(acs))
+    else:
+        fn = getattr(oracle_lib(fast), "khan_oracle_featurize_grad_inverse_" + sfx)
+        fn(_p(X), _p(Y), _p(Z), _p(A), _p(MOs), _p(MACs), _i32(MOs.size), _p(SIs), _p(vX), _p(vY), _p(vZ),
+           _p(outs[0]), _p(outs[1]), _p(outs[2]), _p(outs[3]), _p(acs))
+    return outs
+
+
 def ani_charge(X, Y, Z, Q, MOs, MACs, dtype=np.float64):
     X, Y, Z, Q = _c(X, dtype), _c(Y, dtype), _c(Z, dtype), _c(Q, dtype)
     MOs, MACs = _c(MOs, np.int32), _c(MACs, np.int32)

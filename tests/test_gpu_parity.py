@@ -489,3 +489,75 @@ def test_autograd_wiring(ops):
     q3 = q.detach().clone().requires_grad_(True)
     (kag.ani_charge(X2.detach(), Y2.detach(), Z2.detach(), q3, mos, macs) * gm).sum().backward()
     assert same(q3.grad, qg)
+
+
+# ----------------------------------------------------------------------------- grad-inverse (Jacobian . v)
+def _check_grad_inverse(ops, c, seed=23):
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+    acs = ac.cpu()
+    v = np.random.default_rng(seed).standard_normal((c.N, 3)).astype(np.float32).astype(np.float64)
+    ref = ob.gather_rows(ob.featurize_grad_inverse(c.X, c.Y, c.Z, c.A, c.MOs, c.MACs, c.sc, c.ac,
+                                                    v[:, 0], v[:, 1], v[:, 2]), c.ga)
+    S = mol_scale(ref, c.MOs, c.MACs)
+    A = dev(c.A)
+    for ndt, rtol, atol in ((np.float32, F32_RTOL, F32_ATOL), (np.float64, F64_RTOL, 0.0)):
+        X, Y, Z = dev(c.X, ndt), dev(c.Y, ndt), dev(c.Z, ndt)
+        out = ops.featurize_grad_inverse(X, Y, Z, A, mos, macs, sc, acs, dev(v[:, 0], ndt), dev(v[:, 1], ndt), dev(v[:, 2], ndt))
+        rows = host(torch.cat(out).view(-1, 384)[ga.long()])
+        assert_close("grad-inverse %s vs f64 oracle" % ndt.__name__, rows, ref, rtol, atol, scale=S)
+    return X, Y, Z, A, mos, macs, sc, acs
+
+
+def test_grad_inverse_organic_and_boxes(ops):
+    say("case: featurize_grad_inverse, organic 256 molecules / 2 boxes / fixture")
+    _check_grad_inverse(ops, Case.from_batch(datagen.make_batch("organic", 256)))
+    _check_grad_inverse(ops, Case.from_batch(datagen.make_batch("boxes", 2)))
+    x, y, z, a, mi = helpers.fixture11()
+    _check_grad_inverse(ops, Case(x, y, z, a, mi, 2))
+
+
+def test_grad_inverse_adjoint_identity_and_uniform_vector(ops):
+    # on the device, in float64: <u, J v> = <J^T u, v> with J^T u from featurize_grad, and J applied to a
+    # uniform vector (the reference's only test input, test_kernel.py:363-400) is zero
+    say("case: featurize_grad_inverse adjoint identity, 512 molecules")
+    c = Case.from_batch(datagen.make_batch("organic", 512, first_mol=2000))
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+    acs = ac.cpu()
+    X, Y, Z, A = dev(c.X, np.float64), dev(c.Y, np.float64), dev(c.Z, np.float64), dev(c.A)
+    gen = torch.Generator(device="cuda:0")
+    gen.manual_seed(5)
+    v = [torch.randn(c.N, dtype=torch.float64, device="cuda:0", generator=gen) for _ in range(3)]
+    u = torch.randn(c.N * 384, dtype=torch.float64, device="cuda:0", generator=gen)
+    ub, start = [], 0
+    for k in acs.tolist():
+        ub.append(u[start * 384:(start + k) * 384])
+        start += k
+    Jv = torch.cat(ops.featurize_grad_inverse(X, Y, Z, A, mos, macs, sc, acs, *v))
+    JTu = ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *ub)
+    lhs = float((u * Jv).sum())
+    rhs = float(sum((a * b).sum() for a, b in zip(JTu, v)))
+    say("   <u,Jv> = %.12e   <J^T u,v> = %.12e" % (lhs, rhs))
+    assert abs(lhs - rhs) <= 1e-10 * max(abs(lhs), abs(rhs))
+    one, zero = torch.ones(c.N, dtype=torch.float64, device="cuda:0"), torch.zeros(c.N, dtype=torch.float64, device="cuda:0")
+    J1 = torch.cat(ops.featurize_grad_inverse(X, Y, Z, A, mos, macs, sc, acs, one, zero, zero))
+    assert float(J1.abs().max()) < 1e-11
+
+
+def test_autograd_second_order_wiring(ops):
+    # gradient of a function of the coordinate gradient with respect to the upstream weights goes
+    # through featurize_grad_inverse (trainer_multi_tower.py:64-91)
+    say("case: torch.autograd double backward through featurize")
+    from khan_amd import autograd as kag
+    c = Case.from_batch(datagen.make_batch("organic", 8, first_mol=300))
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+    acs = ac.cpu()
+    A = dev(c.A)
+    X, Y, Z = (dev(t, np.float64).requires_grad_(True) for t in (c.X, c.Y, c.Z))
+    w = torch.from_numpy(np.random.default_rng(3).standard_normal(c.N * 384)).to("cuda:0").requires_grad_(True)
+    energy = (torch.cat(kag.featurize(X, Y, Z, A, mos, macs, sc, acs)) * w).sum()
+    fx, fy, fz = torch.autograd.grad(energy, (X, Y, Z), create_graph=True)
+    a = [dev(np.random.default_rng(k).standard_normal(c.N)) for k in (7, 8, 9)]
+    force_loss = (fx * a[0]).sum() + (fy * a[1]).sum() + (fz * a[2]).sum()
+    (dw,) = torch.autograd.grad(force_loss, (w,))
+    want = torch.cat(ops.featurize_grad_inverse(X.detach(), Y.detach(), Z.detach(), A, mos, macs, sc, acs, *a))
+    assert torch.allclose(dw, want, rtol=1e-11, atol=1e-11)

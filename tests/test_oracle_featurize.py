@@ -201,3 +201,71 @@ def test_backward_matches_compiled_reference_f64():
     mine = np.stack(ob.featurize_grad(b.X, b.Y, b.Z, b.A, b.MOs, b.MACs, sc, ac, g, dtype=np.float64), axis=1)
     ref = np.stack(ob.featurize_grad(b.X, b.Y, b.Z, b.A, b.MOs, b.MACs, sc, ac, g, dtype=np.float64, impl="ref"), axis=1)
     assert np.abs(mine - ref).max() <= 1e-11 * np.abs(ref).max()
+
+
+# ----------------------------------------------------------------------------- grad-inverse (Jacobian . v)
+def _jvp_case(n_mols=12, first_mol=40):
+    b = datagen.make_batch("organic", n_mols, first_mol=first_mol)
+    sc, ga, ac = ob.ani_sort(b.A)
+    rng = np.random.default_rng(17)
+    v = rng.standard_normal((b.n_atoms, 3))
+    return b, sc, ga, ac, v
+
+
+def test_grad_inverse_is_the_adjoint_of_the_gradient():
+    # <u, J v> = <J^T u, v>: J^T u is featurize_grad (pinned against the compiled reference above), so
+    # this identity pins J v for arbitrary v; a wrong index, sign or dropped term breaks it
+    b, sc, ga, ac, v = _jvp_case()
+    rng = np.random.default_rng(3)
+    u_rows = rng.standard_normal((b.n_atoms, 384))
+    u = ob.scatter_rows(u_rows, b.A, sc, ac)
+    Jv = ob.featurize_grad_inverse(b.X, b.Y, b.Z, b.A, b.MOs, b.MACs, sc, ac, v[:, 0], v[:, 1], v[:, 2])
+    JTu = ob.featurize_grad(b.X, b.Y, b.Z, b.A, b.MOs, b.MACs, sc, ac, u)
+    lhs = sum(float(np.dot(a.reshape(-1), c.reshape(-1))) for a, c in zip(u, Jv))
+    rhs = float(np.dot(JTu[0], v[:, 0]) + np.dot(JTu[1], v[:, 1]) + np.dot(JTu[2], v[:, 2]))
+    assert abs(lhs - rhs) <= 1e-11 * max(abs(lhs), abs(rhs), 1.0)
+    # one molecule at a time as well, so that errors cannot cancel between molecules
+    Jv_rows = ob.gather_rows(Jv, ga)
+    for m in range(b.n_mols):
+        s = slice(b.MOs[m], b.MOs[m] + b.MACs[m])
+        lhs = float((u_rows[s] * Jv_rows[s]).sum())
+        rhs = float(sum(np.dot(JTu[k][s], v[s, k]) for k in range(3)))
+        assert abs(lhs - rhs) <= 1e-11 * max(abs(lhs), abs(rhs), 1.0)
+
+
+def test_grad_inverse_matches_central_differences_of_the_forward():
+    b, sc, ga, ac, v = _jvp_case(n_mols=6)
+    h = 1e-6
+    X, Y, Z = (np.asarray(t, dtype=np.float64) for t in (b.X, b.Y, b.Z))
+    fp = ob.featurize(X + h * v[:, 0], Y + h * v[:, 1], Z + h * v[:, 2], b.A, b.MOs, b.MACs, sc, ac, dtype=np.float64)
+    fm = ob.featurize(X - h * v[:, 0], Y - h * v[:, 1], Z - h * v[:, 2], b.A, b.MOs, b.MACs, sc, ac, dtype=np.float64)
+    num = [(p - m) / (2 * h) for p, m in zip(fp, fm)]
+    Jv = ob.featurize_grad_inverse(X, Y, Z, b.A, b.MOs, b.MACs, sc, ac, v[:, 0], v[:, 1], v[:, 2])
+    for a, n_ in zip(Jv, num):
+        if a.size:
+            assert np.max(np.abs(a - n_)) <= 2e-8 * max(1.0, float(np.max(np.abs(n_))))
+
+
+def test_grad_inverse_uniform_vector_gives_zero_like_the_reference_test():
+    # the reference's only check feeds dL/dx = 1, dL/dy = dL/dz = 0 for every atom (test_kernel.py:
+    # 363-400): features are translation invariant, so the result is zero up to rounding
+    b, sc, ga, ac, v = _jvp_case()
+    one, zero = np.ones(b.n_atoms), np.zeros(b.n_atoms)
+    Jv = ob.featurize_grad_inverse(b.X, b.Y, b.Z, b.A, b.MOs, b.MACs, sc, ac, one, zero, zero)
+    assert max(float(np.max(np.abs(a))) for a in Jv if a.size) < 1e-12
+    if ob.have_ref():
+        ref = ob.featurize_grad_inverse(b.X, b.Y, b.Z, b.A, b.MOs, b.MACs, sc, ac, one, zero, zero, impl="ref")
+        assert max(float(np.max(np.abs(a))) for a in ref if a.size) < 1e-9
+        # and the reference returns (numerically) zero for ANY input, because it reads the vectors
+        # by atomic number of the centre for all three atoms of a term (kernel_cpu.cpp:111-169)
+        ref2 = ob.featurize_grad_inverse(b.X, b.Y, b.Z, b.A, b.MOs, b.MACs, sc, ac, v[:, 0], v[:, 1], v[:, 2], impl="ref")
+        assert max(float(np.max(np.abs(a))) for a in ref2 if a.size) < 1e-9
+
+
+def test_grad_inverse_float32_oracle_close_to_float64():
+    b, sc, ga, ac, v = _jvp_case()
+    a64 = ob.featurize_grad_inverse(b.X, b.Y, b.Z, b.A, b.MOs, b.MACs, sc, ac, v[:, 0], v[:, 1], v[:, 2])
+    a32 = ob.featurize_grad_inverse(b.X, b.Y, b.Z, b.A, b.MOs, b.MACs, sc, ac, v[:, 0], v[:, 1], v[:, 2], dtype=np.float32)
+    for p, q in zip(a32, a64):
+        if p.size:
+            assert np.max(np.abs(p - q)) <= 2e-5 * max(1.0, float(np.max(np.abs(q))))
