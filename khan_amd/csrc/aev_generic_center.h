@@ -74,6 +74,21 @@ __device__ __forceinline__ Partner<T> partner_from_lane(const Partner<T>& p, int
     return q;
 }
 
+// Adds `val` to slot (blk, ts) of a centre's angular row in LDS.  The two half-waves hold two different
+// triples; their 32 slots collide only when both triples fall into the same type-pair block, in which case
+// the lower half adds both values.  A plain read-add-write then touches distinct addresses across the wave
+// (float atomics on LDS cost two orders of magnitude more per wave instruction on this part).
+template <typename T>
+__device__ __forceinline__ void ang_accumulate(T* ang, int blk, int ts, int half, bool act, T val)
+{
+    const T v = act ? val : T(0);
+    const int mine = act ? blk : -1;
+    const int other = __shfl_xor(mine, 32, 64);
+    const T other_v = __shfl_xor(v, 32, 64);
+    const bool same = mine == other;
+    if (act && (!same || half == 0)) ang[blk * kAngBlock + ts] += same ? v + other_v : v;
+}
+
 // Forward pass of ONE centre atom i of the molecule at [off, off+n), executed by one whole wavefront.
 // `ang` is kAngular elements of this wavefront's LDS; the finished 384-wide row is stored to `row`.
 template <typename T>
@@ -150,7 +165,7 @@ __device__ __forceinline__ void fwd_center_generic(const LaneConsts<T>& L, int l
                         const T b2 = base * base, b4 = b2 * b2, b8 = b4 * b4;
                         const T dav = (J.r + K.r) * T(0.5) - L.ars;
                         const T val = T(0.0078125) * b8 * Real<T>::exp_(-L.A_eta * dav * dav) * Jfc * Kfc;
-                        if (act) atomicAdd(&ang[pair_block(J.type, K.type) * kAngBlock + L.ts], val);
+                        ang_accumulate(ang, pair_block(J.type, K.type), L.ts, L.half, act, val);
                     }
                 }
             }
@@ -434,7 +449,7 @@ __device__ __forceinline__ void jvp_center_generic(const LaneConsts<T>& L, int l
                         const T P = two_pow * Jfc * Kfc;
                         const T dP = two_pow * (Jdfc * Je.rd * Kfc + Jfc * Kdfc * Ke.rd);
                         const T val = dAt * Gs * P + At * (dGs * P + Gs * dP);
-                        if (act) atomicAdd(&ang[pair_block(J.type, K.type) * kAngBlock + L.ts], val);
+                        ang_accumulate(ang, pair_block(J.type, K.type), L.ts, L.half, act, val);
                     }
                 }
             }
