@@ -36,11 +36,13 @@ int forward_dispatch(const float* xs, const float* ys, const float* zs, const in
 {
     if (force_generic())
         return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, stream));
-    // molecules of up to 64 atoms: one wavefront each; the rest: general kernel
+    // molecules of up to 64 atoms: one wavefront each; up to 256: one workgroup each; the rest: general kernel
     int st = hip_status(khan::launch_fwd_small_f32(xs, ys, zs, as, mos, macs, n_mols, sis, out, stream));
     if (st != KHAN_OK) return st;
+    st = hip_status(khan::launch_fwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, out, stream));
+    if (st != KHAN_OK) return st;
     return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
-                                                      khan::kSmallMaxAtoms + 1, stream));
+                                                      khan::kMediumMaxAtoms + 1, stream));
 }
 
 int forward_dispatch(const double* xs, const double* ys, const double* zs, const int32_t* as,

@@ -376,6 +376,10 @@ def test_crowded_centres_take_the_fallback(ops):
     tail = np.array([[2.5 + 1.1 * k, 0.2 * (-1) ** k, 0.0] for k in range(12)]) + rng.uniform(-0.05, 0.05, (12, 3))
     mols.append((rng.integers(0, 4, 52), np.concatenate([ball, tail])))
     mols.append((np.full(45, 1), _packed_ball(rng, 45, 2.1, 0.85)))                   # one type only
+    # the same for the one-workgroup-per-molecule kernels (65..256 atoms): more than 32 angular and more
+    # than 64 radial partners around the inner atoms
+    mols.append((rng.integers(0, 4, 110), _packed_ball(rng, 110, 3.0, 0.85)))
+    mols.append((rng.integers(0, 4, 200), _packed_ball(rng, 200, 3.9, 0.85)))
     A = np.concatenate([m[0] for m in mols]).astype(np.int32)
     xyz = np.concatenate([m[1] for m in mols])
     mi = np.concatenate([np.full(len(m[0]), k) for k, m in enumerate(mols)]).astype(np.int32)
