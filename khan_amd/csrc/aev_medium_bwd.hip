@@ -1,0 +1,266 @@
+// AEV backward (dL/dxyz) for molecules of 65 to 256 atoms, float32: one workgroup of four wavefronts
+// per molecule.
+//
+// The workgroup sorts the atoms by type into LDS once and zeroes the molecule's outputs.  Wavefronts
+// then draw centres from a shared counter.  A wavefront collects centres into a batch while their
+// angular partner lists fit the 64 entries of its pool (at most six), and for each centre it takes in:
+//   scan + radial   the centre is tested against the sorted atoms 64 at a time; a lane owns one
+//                   (centre, partner) pair, sums g e (f_C' - 2 eta d f_C) over the 16 shells, and adds
+//                   the pull to the partner and (summed over the wave) to the centre;
+// then for the batch:
+//   stage           the 320 angular upstream values of each centre's row go to LDS by type pair;
+//   angular         the round-robin walk shared with the small-molecule kernel: lane = list entry,
+//                   partner forces by conflict-free read-add-write in LDS;
+//   gather          every list entry adds its total to its atom, every centre gets minus its list's sum.
+// Forces go to the output arrays with global atomics (a molecule's atoms are shared by four wavefronts).
+// A centre with more than 64 angular partners is handled by the general per-centre routine.
+// Reference: gpu_featurizer/kernel_cpu.cpp:217-366.
+#include "aev_bwd_batch.h"
+
+namespace khan {
+
+namespace {
+
+constexpr int kMedMin = kSmallMaxAtoms + 1;   // smaller molecules run one wavefront each
+constexpr int kChunks = kMediumMaxAtoms / 64;
+
+struct __align__(16) MedBwdShared {
+    float4 atom[kMediumMaxAtoms];          // x, y, z, type (sorted order)
+    unsigned row_lo[kMediumMaxAtoms];      // address of the atom's upstream row
+    unsigned row_hi[kMediumMaxAtoms];
+    unsigned short orig[kMediumMaxAtoms];  // sorted position -> index inside the molecule
+    int wcount[4][4];                      // atoms of each type held by each wavefront before the sort
+    int next;                              // next centre (sorted position) to hand out
+};
+
+__global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
+    const float* __restrict__ X, const float* __restrict__ Y, const float* __restrict__ Z,
+    const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
+    const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
+    Buckets<const float> gin, float* __restrict__ gX, float* __restrict__ gY, float* __restrict__ gZ)
+{
+    __shared__ MedBwdShared M;
+    __shared__ BwdPool pools[4];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = uniform(tid >> 6);
+    BwdPool& P = pools[wave];
+    const LaneConsts<float> L = lane_consts<float>(lane);
+    const unsigned long long lt_mask = (1ull << lane) - 1ull;
+    const float inv_rc_A = 1.0f / kA_Rc_f;
+
+    for (int mol = blockIdx.x; mol < n_mols; mol += gridDim.x) {
+        const int n = uniform(MACs[mol]);
+        const int off = uniform(MOs[mol]);
+        if (n < kMedMin || n > kMediumMaxAtoms) continue;
+
+        // ------------------------------------------------------------ load, sort by type into LDS, zero outputs
+        const bool have = tid < n;
+        float x = 0.f, y = 0.f, z = 0.f;
+        int type = 0;
+        unsigned long long rowbits = 0;
+        if (have) {
+            x = X[off + tid];
+            y = Y[off + tid];
+            z = Z[off + tid];
+            type = fold_type(A[off + tid]);
+            rowbits = reinterpret_cast<unsigned long long>(gin.p[type] + static_cast<size_t>(SIs[off + tid]) * kFeats);
+            gX[off + tid] = 0.f;
+            gY[off + tid] = 0.f;
+            gZ[off + tid] = 0.f;
+        }
+        unsigned long long tmask[4];
+#pragma unroll
+        for (int a = 0; a < 4; ++a) tmask[a] = wave_ballot(have && type == a);
+        if (lane < 4) M.wcount[wave][lane] = popc64(lane == 0 ? tmask[0] : lane == 1 ? tmask[1] : lane == 2 ? tmask[2] : tmask[3]);
+        if (tid == 0) M.next = 0;
+        __syncthreads();
+        int tbase[4];
+        {
+            int run = 0;
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                tbase[a] = run;
+                run += M.wcount[0][a] + M.wcount[1][a] + M.wcount[2][a] + M.wcount[3][a];
+            }
+        }
+        if (have) {
+            int before = 0;                     // atoms of my type held by earlier wavefronts
+            for (int w = 0; w < wave; ++w) before += M.wcount[w][type];
+            const unsigned long long mine = type == 0 ? tmask[0] : type == 1 ? tmask[1] : type == 2 ? tmask[2] : tmask[3];
+            const int dest = sel4(type, tbase[0], tbase[1], tbase[2], tbase[3]) + before + popc64(mine & lt_mask);
+            M.atom[dest] = make_float4(x, y, z, __int_as_float(type));
+            M.row_lo[dest] = static_cast<unsigned>(rowbits & 0xffffffffull);
+            M.row_hi[dest] = static_cast<unsigned>(rowbits >> 32);
+            M.orig[dest] = static_cast<unsigned short>(tid);
+        }
+        __syncthreads();       // sorted arrays complete; the zeroed outputs are visible before any atomic add
+        const int tb1 = tbase[1], tb2 = tbase[2], tb3 = tbase[3];
+        auto type_of = [&](int sorted_idx) { return (sorted_idx >= tb1) + (sorted_idx >= tb2) + (sorted_idx >= tb3); };
+        auto row_of = [&](int sorted_idx) -> const float* {            // wave-uniform index
+            const unsigned lo = static_cast<unsigned>(uniform(static_cast<int>(M.row_lo[sorted_idx])));
+            const unsigned hi = static_cast<unsigned>(uniform(static_cast<int>(M.row_hi[sorted_idx])));
+            return reinterpret_cast<const float*>((static_cast<unsigned long long>(hi) << 32) | lo);
+        };
+        auto add_force = [&](int sorted_idx, float fx, float fy, float fz) {   // per-lane target
+            const int g = off + M.orig[sorted_idx];
+            atomicAdd(&gX[g], fx);
+            atomicAdd(&gY[g], fy);
+            atomicAdd(&gZ[g], fz);
+        };
+
+        int pending = -1;          // a centre that was drawn but did not fit the previous batch
+        for (;;) {
+            // ------------------------------------------------ collect a batch of centres
+            int nb = 0, used = 0;
+            int pfv = 0, cv = 0;   // lane k: first pool slot and sorted position of centre k of the batch
+            P.facc[lane] = make_float4(0.f, 0.f, 0.f, 0.f);
+            while (nb < kB) {
+                int c = pending;
+                pending = -1;
+                if (c < 0) {
+                    int drawn = 0;
+                    if (lane == 0) drawn = atomicAdd(&M.next, 1);
+                    c = uniform(drawn);
+                }
+                if (c >= n) break;
+                const float4 ai = M.atom[c];
+                // first pass over the partners: who is inside the cutoffs
+                float dx[kChunks], dy[kChunks], dz[kChunks], r[kChunks];
+                unsigned long long mA[kChunks], mR[kChunks];
+                int m_c = 0;
+#pragma unroll
+                for (int ch = 0; ch < kChunks; ++ch) {
+                    mA[ch] = 0ull;
+                    mR[ch] = 0ull;
+                    dx[ch] = dy[ch] = dz[ch] = 0.f;
+                    r[ch] = 1.f;
+                    if (ch * 64 < n) {
+                        const int j = ch * 64 + lane;
+                        const float4 aj = M.atom[j];
+                        dx[ch] = ai.x - aj.x;
+                        dy[ch] = ai.y - aj.y;
+                        dz[ch] = ai.z - aj.z;
+                        r[ch] = sqrtf(dx[ch] * dx[ch] + dy[ch] * dy[ch] + dz[ch] * dz[ch]);
+                        const bool valid = (j < n) && (j != c);
+                        mR[ch] = wave_ballot(valid && (r[ch] < kR_Rc_f));
+                        mA[ch] = wave_ballot(valid && (r[ch] < kA_Rc_f));
+                        m_c += popc64(mA[ch]);
+                    }
+                }
+                if (m_c > 64) {
+                    // more partners than a pool holds: the general per-centre routine does this centre alone
+                    const int i_orig = uniform(static_cast<int>(M.orig[c]));
+                    wave_lds_fence();
+                    bwd_center_generic<float>(L, lane, X, Y, Z, A, off, n, i_orig, P.gst, row_of(c),
+                                              [&](int atom, float fx, float fy, float fz) {
+                                                  atomicAdd(&gX[off + atom], fx);
+                                                  atomicAdd(&gY[off + atom], fy);
+                                                  atomicAdd(&gZ[off + atom], fz);
+                                              });
+                    continue;
+                }
+                if (nb > 0 && used + m_c > 64) {       // full: this centre opens the next batch
+                    pending = c;
+                    break;
+                }
+                // second pass: list entries, radial pulls
+                const float* grow = row_of(c);
+                float cfx = 0.f, cfy = 0.f, cfz = 0.f;          // pull on the centre, this lane's pairs
+                int pos = used;
+#pragma unroll
+                for (int ch = 0; ch < kChunks; ++ch) {
+                    if (ch * 64 < n) {
+                        const int j = ch * 64 + lane;
+                        const float inv = __builtin_amdgcn_rcpf(r[ch]);
+                        if ((mA[ch] >> lane) & 1ull) {
+                            const int p = pos + popc64(mA[ch] & lt_mask);
+                            float fc, dfc;
+                            cutoff_poly_grad(r[ch] * inv_rc_A, inv_rc_A, fc, dfc);
+                            P.nbr[p] = make_float4(dx[ch] * inv, dy[ch] * inv, dz[ch] * inv, r[ch]);
+                            P.nbr_fc[p] = make_float2(fc, dfc);
+                            P.nbr_idx[p] = static_cast<unsigned char>(j);
+                        }
+                        pos += popc64(mA[ch]);
+                        if ((mR[ch] >> lane) & 1ull) {
+                            const float sc = bwd_radial_pair(grow, type_of(j), r[ch], inv);
+                            const float fx = sc * dx[ch], fy = sc * dy[ch], fz = sc * dz[ch];
+                            cfx += fx;
+                            cfy += fy;
+                            cfz += fz;
+                            add_force(j, -fx, -fy, -fz);
+                        }
+                    }
+                }
+                cfx = group_sum_to_last_lane(cfx, 6);
+                cfy = group_sum_to_last_lane(cfy, 6);
+                cfz = group_sum_to_last_lane(cfz, 6);
+                if (lane == 63) add_force(c, cfx, cfy, cfz);
+                if (lane == nb) {
+                    pfv = used;
+                    cv = c;
+                }
+                used += m_c;
+                ++nb;
+            }
+            if (nb == 0) break;
+            if (lane >= nb) pfv = used;              // lanes nb.. hold the end of the pool
+
+            // ---- the angular upstream blocks of the batch's rows go to LDS (80 x 16 bytes per row)
+            {
+                v4f st0[kB], st1[kB];
+#pragma unroll
+                for (int b = 0; b < kB; ++b) {
+                    st0[b] = v4f{0.f, 0.f, 0.f, 0.f};
+                    st1[b] = v4f{0.f, 0.f, 0.f, 0.f};
+                    if (b < nb) {
+                        const global_v4f_ptr rowp = (global_v4f_ptr)(row_of(lane_read(cv, b)) + kRadial);
+                        st0[b] = rowp[lane];
+                        if (lane < 16) st1[b] = rowp[64 + lane];
+                    }
+                }
+                bwd_stage_blocks(P, lane, nb, st0, st1);
+            }
+            wave_lds_fence();
+
+            // ------------------------------------------------ angular: lane = list entry (centre, partner j)
+            const int pf1 = lane_read(pfv, 1), pf2 = lane_read(pfv, 2), pf3 = lane_read(pfv, 3),
+                      pf4 = lane_read(pfv, 4), pf5 = lane_read(pfv, 5), pf6 = lane_read(pfv, 6);
+            const int total = used;
+            const int b = (lane >= pf1) + (lane >= pf2) + (lane >= pf3) + (lane >= pf4) + (lane >= pf5);
+            const bool live = lane < total;
+            const int bs = live ? b : 0;
+            const int pb = sel6(bs, 0, pf1, pf2, pf3, pf4, pf5);
+            const int m = sel6(bs, pf1, pf2, pf3, pf4, pf5, pf6) - pb;
+            const float4 f = bwd_angular_rounds(P, lane, live, bs, pb, m, type_of);
+
+            // ------------------------------------------------ gather
+            if (live) add_force(P.nbr_idx[lane], f.x, f.y, f.z);
+            for (int bb = 0; bb < nb; ++bb) {
+                const bool mine = live && (bs == bb);
+                const float sx = group_sum_to_last_lane(mine ? f.x : 0.f, 6);
+                const float sy = group_sum_to_last_lane(mine ? f.y : 0.f, 6);
+                const float sz = group_sum_to_last_lane(mine ? f.z : 0.f, 6);
+                if (lane == 63) add_force(lane_read(cv, bb), -sx, -sy, -sz);
+            }
+            wave_lds_fence();
+        }
+        __syncthreads();      // the next molecule reuses the sorted arrays
+    }
+}
+
+}  // namespace
+
+hipError_t launch_bwd_medium_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
+                                 const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                                 const int32_t* SIs, Buckets<const float> g, float* gX, float* gY,
+                                 float* gZ, hipStream_t stream)
+{
+    if (n_mols <= 0) return hipSuccess;
+    // workgroups walk the molecules with the grid's stride and skip those of other sizes
+    const unsigned blocks = static_cast<unsigned>(n_mols < 4096 ? n_mols : 4096);
+    aev_bwd_medium_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ);
+    return hipGetLastError();
+}
+
+}  // namespace khan

@@ -24,33 +24,19 @@
 // Finally every lane stores the gradient of its own atom: no global atomics, no pre-zeroed output.
 // The derivative is the algebraically reduced form (no acos, no 1/(1+cos) factor); reference:
 // gpu_featurizer/kernel_cpu.cpp:217-366.
-#include "aev_small_common.h"
+#include "aev_bwd_batch.h"
 
 namespace khan {
 
 namespace {
 
-typedef float v4f __attribute__((ext_vector_type(4)));
-typedef const __attribute__((address_space(1))) v4f* global_v4f_ptr;
-
-constexpr int kBlockStride = 36;   // floats between staged 32-float blocks: rotates the LDS banks
-
 struct __align__(16) BwdLds {
-    float4 atom[64];                              // x, y, z, type (sorted order)
-    float4 nbr[64];                               // pooled lists: unit vector (centre minus partner)/r, and r
-    float4 facc[64];                              // force on each list entry from its centre's row
-    float2 nbr_fc[64];                            // f_C(r, A_Rc) and its derivative in r
-    float gst[kB * kNumPairBlocks * kBlockStride];   // staged upstream blocks [centre][type pair][32]
-    float force[3][64];                           // dL/dx, dL/dy, dL/dz per sorted atom
-    int nM[8];                                    // angular partners per centre of the batch
-    unsigned char nbr_idx[64];                    // sorted lane of the partner
-    unsigned char inv[64];                        // original atom index -> sorted lane
+    float4 atom[64];                     // x, y, z, type (sorted order)
+    BwdPool pool;                        // partner lists and staged upstream values of the batch
+    float force[3][64];                  // dL/dx, dL/dy, dL/dz per sorted atom
+    int nM[8];                           // angular partners per centre of the batch
+    unsigned char inv[64];               // original atom index -> sorted lane
 };
-
-__device__ __forceinline__ int sel6(int b, int v0, int v1, int v2, int v3, int v4, int v5)
-{
-    return b == 0 ? v0 : b == 1 ? v1 : b == 2 ? v2 : b == 3 ? v3 : b == 4 ? v4 : v5;
-}
 
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void aev_bwd_small_kernel(
     const float* __restrict__ X, const float* __restrict__ Y, const float* __restrict__ Z,
@@ -126,10 +112,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
     const int grp = lane >> logW, jl = lane & (W - 1);
     const unsigned long long sub_mask = low_bits(W) << ((grp * W) & 63);
     const unsigned long long ltg_mask = lt_mask & sub_mask;
-    const float inv_rc_R = 1.0f / kR_Rc_f, inv_rc_A = 1.0f / kA_Rc_f;
-    const float kLog2e = 1.44269504088896340736f;
-    const float kRadExp = -kR_eta_f * kLog2e;
-    const float kAngExp = -kA_eta_f * kLog2e;
+    const float inv_rc_A = 1.0f / kA_Rc_f;
     // type of a sorted lane from the type boundaries
     const int tb1 = tbase[1], tb2 = tbase[2], tb3 = tbase[3];
     auto type_of = [&](int sorted_lane) { return (sorted_lane >= tb1) + (sorted_lane >= tb2) + (sorted_lane >= tb3); };
@@ -202,7 +185,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
                 if (lane < 16) st1[b] = rowp[64 + lane];
             }
         }
-        S.facc[lane] = make_float4(0.f, 0.f, 0.f, 0.f);
+        S.pool.facc[lane] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (lane < 8) S.nM[lane] = 0;
         wave_lds_fence();
 
@@ -228,9 +211,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
                 const int pos = base + popc64(mA & ltg_mask);
                 float fc, dfc;
                 cutoff_poly_grad(r * inv_rc_A, inv_rc_A, fc, dfc);
-                S.nbr[pos] = make_float4(dx * inv, dy * inv, dz * inv, r);
-                S.nbr_fc[pos] = make_float2(fc, dfc);
-                S.nbr_idx[pos] = static_cast<unsigned char>(jl);
+                S.pool.nbr[pos] = make_float4(dx * inv, dy * inv, dz * inv, r);
+                S.pool.nbr_fc[pos] = make_float2(fc, dfc);
+                S.pool.nbr_idx[pos] = static_cast<unsigned char>(jl);
             }
             if (jl == 0 && centre_ok) S.nM[b] = fits ? cntA : 0;
             {
@@ -244,22 +227,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
             float cfx = 0.f, cfy = 0.f, cfz = 0.f;       // this pair's pull on the centre
             const bool do_rad = inR && fits;              // a centre that does not fit is redone as a whole
             if (do_rad) {
-                const int tj = __float_as_int(aj.w);
-                const global_v4f_ptr gp = (global_v4f_ptr)(grow + tj * kNumRRs);
-                const v4f g0 = gp[0], g1 = gp[1], g2 = gp[2], g3 = gp[3];
-                const float gr[16] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w,
-                                      g2.x, g2.y, g2.z, g2.w, g3.x, g3.y, g3.z, g3.w};
-                float fc, dfc;
-                cutoff_poly_grad(r * inv_rc_R, inv_rc_R, fc, dfc);
-                const float m2eta_fc = -2.0f * kR_eta_f * fc;
-                float Gsum = 0.f;
-#pragma unroll
-                for (int q = 0; q < kNumRRs; ++q) {
-                    const float d = r - kR_Rs_f[q];
-                    const float e = __builtin_amdgcn_exp2f(kRadExp * d * d);
-                    Gsum = fmaf(gr[q] * e, fmaf(m2eta_fc, d, dfc), Gsum);   // g e (f_C' - 2 eta d f_C)
-                }
-                const float sc = Gsum * inv;           // dE/dr / r, multiplies (x_i - x_j)
+                const float sc = bwd_radial_pair(grow, __float_as_int(aj.w), r, inv);   // dE/dr / r, multiplies (x_i - x_j)
                 cfx = sc * dx;
                 cfy = sc * dy;
                 cfz = sc * dz;
@@ -283,15 +251,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
             }
         }
 
-        // ---- the fetched upstream blocks go to LDS: chunk c of a row = block c/8, part c%8
-#pragma unroll
-        for (int b = 0; b < kB; ++b) {
-            if (b < nb) {
-                float* blk = &S.gst[b * kNumPairBlocks * kBlockStride];
-                *reinterpret_cast<v4f*>(blk + (lane >> 3) * kBlockStride + (lane & 7) * 4) = st0[b];
-                if (lane < 16) *reinterpret_cast<v4f*>(blk + (8 + (lane >> 3)) * kBlockStride + (lane & 7) * 4) = st1[b];
-            }
-        }
+        // ---- the fetched upstream blocks go to LDS
+        bwd_stage_blocks(S.pool, lane, nb, st0, st1);
         wave_lds_fence();
 
         // ------------------------------------------------ angular: lane = list entry (centre, partner j)
@@ -303,102 +264,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
             const int pb = sel6(bs, pf[0], pf[1], pf[2], pf[3], pf[4], pf[5]);
             const int m = sel6(bs, m03.x, m03.y, m03.z, m03.w, m47.x, m47.y);   // 0 for a centre that did not fit
             const bool live = (lane < total) && (m > 0);
-            const int e = live ? lane - pb : 0;
-            // rounds: d = 1 .. (m-1)/2 for every lane; when m is even one more round for the lower half
-            const int full = (m - 1) >> 1;
-            const int rounds = live ? full + ((((m & 1) == 0) && (e < (m >> 1))) ? 1 : 0) : 0;
-            const int max_rounds = wave_max(rounds);
+            const float4 f = bwd_angular_rounds(S.pool, lane, live, bs, pb, m, type_of);
             const int self = live ? lane : 0;
-            const float4 vj = S.nbr[self];
-            const float2 fj = S.nbr_fc[self];
-            const int tj = type_of(S.nbr_idx[self]);
-            const float inv_rj = __builtin_amdgcn_rcpf(vj.w);
-            const float* gbase = &S.gst[bs * kNumPairBlocks * kBlockStride];
-            float ajx = 0.f, ajy = 0.f, ajz = 0.f;           // force on j, kept in registers
-
-            for (int d = 1; d <= max_rounds; ++d) {
-                const bool act = d <= rounds;
-                int k = e + d;
-                k -= (k >= m) ? m : 0;
-                const int ks = act ? pb + k : 0;
-                const float4 vk = S.nbr[ks];
-                const float2 fk = S.nbr_fc[ks];
-                const int tk = type_of(S.nbr_idx[ks]);
-                if (act) {
-                    const v4f* gp = reinterpret_cast<const v4f*>(gbase + pair_block(tj, tk) * kBlockStride);
-                    v4f g[8];
-#pragma unroll
-                    for (int t = 0; t < 8; ++t) g[t] = gp[t];
-
-                    float c = vj.x * vk.x + vj.y * vk.y + vj.z * vk.z;
-                    c = fminf(fmaxf(c, -1.0f), 1.0f);
-                    const float cx = vj.y * vk.z - vj.z * vk.y;
-                    const float cy = vj.z * vk.x - vj.x * vk.z;
-                    const float cz = vj.x * vk.y - vj.y * vk.x;
-                    // cot(theta) = c/s has no limit for collinear triples (the angle has a cusp there, the
-                    // reference returns NaN): c s / (s^2 + 1e-12) equals c/s to 1e-7 relative from 0.2 degrees
-                    // off the line and goes to zero on it
-                    const float s2 = cx * cx + cy * cy + cz * cz;
-                    const float s = __builtin_amdgcn_sqrtf(s2);
-                    const float c_over_s = c * s * __builtin_amdgcn_rcpf(s2 + 1e-12f);
-                    const float rho = 0.5f * (vj.w + vk.w);
-                    float Gs[4], dds[4];
-#pragma unroll
-                    for (int sidx = 0; sidx < 4; ++sidx) {
-                        dds[sidx] = rho - kA_Rs_f[sidx];
-                        Gs[sidx] = __builtin_amdgcn_exp2f(kAngExp * dds[sidx] * dds[sidx]);
-                    }
-                    // X_s = sum_t g_ts A_t and Y_s = sum_t g_ts dA_t/dcos (without its factor 8)
-                    float Xs[4] = {0.f, 0.f, 0.f, 0.f}, Ys[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int t = 0; t < 8; ++t) {
-                        const float ct = static_cast<float>(kCosTheta[t]), st = static_cast<float>(kSinTheta[t]);
-                        const float bs1 = fmaf(s, st, fmaf(c, ct, 1.0f));       // 1 + cos(theta - theta_t)
-                        const float b2 = bs1 * bs1, b4 = b2 * b2;
-                        const float Am1 = b4 * b2 * bs1;                         // ^7
-                        const float At = Am1 * bs1;                              // ^8
-                        const float dAt = Am1 * fmaf(-c_over_s, st, ct);         // (d/dcos) / 8
-                        Xs[0] = fmaf(g[t].x, At, Xs[0]);
-                        Xs[1] = fmaf(g[t].y, At, Xs[1]);
-                        Xs[2] = fmaf(g[t].z, At, Xs[2]);
-                        Xs[3] = fmaf(g[t].w, At, Xs[3]);
-                        Ys[0] = fmaf(g[t].x, dAt, Ys[0]);
-                        Ys[1] = fmaf(g[t].y, dAt, Ys[1]);
-                        Ys[2] = fmaf(g[t].z, dAt, Ys[2]);
-                        Ys[3] = fmaf(g[t].w, dAt, Ys[3]);
-                    }
-                    // W0 = sum G_s X_s, Wc = 8 sum G_s Y_s, Wr = sum (dG_s/drho) X_s with dG/drho = -2 eta dd G
-                    const float gx0 = Gs[0] * Xs[0], gx1 = Gs[1] * Xs[1], gx2 = Gs[2] * Xs[2], gx3 = Gs[3] * Xs[3];
-                    const float W0 = (gx0 + gx1) + (gx2 + gx3);
-                    const float Wc = 8.0f * fmaf(Gs[0], Ys[0], fmaf(Gs[1], Ys[1], fmaf(Gs[2], Ys[2], Gs[3] * Ys[3])));
-                    const float Wr = (-2.0f * kA_eta_f) * fmaf(dds[0], gx0, fmaf(dds[1], gx1, fmaf(dds[2], gx2, dds[3] * gx3)));
-                    const float two_pow = 0.0078125f;
-                    const float P = two_pow * fj.x * fk.x;
-                    const float Fj = fmaf(P * 0.5f, Wr, two_pow * W0 * fj.y * fk.x);    // dE/dr_ij
-                    const float Fk = fmaf(P * 0.5f, Wr, two_pow * W0 * fj.x * fk.y);    // dE/dr_ik
-                    const float Fc = P * Wc;                                            // dE/dcos
-                    const float ij = Fc * inv_rj, ik = Fc * __builtin_amdgcn_rcpf(vk.w);
-                    // force on j = -[Fj u_j + ij (u_k - c u_j)]; the bracket's second part is formed first, it
-                    // is small near the line where ij is large
-                    ajx = fmaf(-Fj, vj.x, fmaf(-ij, fmaf(-c, vj.x, vk.x), ajx));
-                    ajy = fmaf(-Fj, vj.y, fmaf(-ij, fmaf(-c, vj.y, vk.y), ajy));
-                    ajz = fmaf(-Fj, vj.z, fmaf(-ij, fmaf(-c, vj.z, vk.z), ajz));
-                    // force on k: in a round every lane of a centre holds a different k
-                    float4 fk_acc = S.facc[ks];
-                    fk_acc.x = fmaf(-Fk, vk.x, fmaf(-ik, fmaf(-c, vk.x, vj.x), fk_acc.x));
-                    fk_acc.y = fmaf(-Fk, vk.y, fmaf(-ik, fmaf(-c, vk.y, vj.y), fk_acc.y));
-                    fk_acc.z = fmaf(-Fk, vk.z, fmaf(-ik, fmaf(-c, vk.z, vj.z), fk_acc.z));
-                    S.facc[ks] = fk_acc;
-                }
-                wave_lds_fence();
-            }
-
             // -------------------------------------------- gather: partners get their slot, the centre minus the sum
-            float4 f = S.facc[self];
-            f.x = live ? f.x + ajx : 0.f;
-            f.y = live ? f.y + ajy : 0.f;
-            f.z = live ? f.z + ajz : 0.f;
-            const int atom = S.nbr_idx[self];
+            const int atom = S.pool.nbr_idx[self];
             for (int bb = 0; bb < nb; ++bb) {
                 if (uniform(pf[bb + 1] - pf[bb]) == 0) continue;
                 const bool mine = live && (bs == bb);
@@ -426,7 +295,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
                 if (overflow & (1u << b)) {
                     const int i_b = lane_read(cord, min(c0 + b, 63));
                     const int i_orig = lane_read(orig, i_b);
-                    bwd_center_generic<float>(L, lane, X, Y, Z, A, off, n, i_orig, S.gst, row_of(i_b),
+                    bwd_center_generic<float>(L, lane, X, Y, Z, A, off, n, i_orig, S.pool.gst, row_of(i_b),
                                               [&](int atom, float fx, float fy, float fz) {
                                                   const int sl = S.inv[atom];
                                                   atomicAdd(&S.force[0][sl], fx);

@@ -60,10 +60,12 @@ int backward_dispatch(const float* xs, const float* ys, const float* zs, const i
     if (force_generic())
         return hip_status(khan::launch_bwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
                                                           n_atoms, 0, stream));
-    // general kernel first (it zero-fills and accumulates with atomics, molecules above 64 atoms
-    // only), then the small-molecule kernel, which stores every gradient of its molecules itself
+    // by molecule size: above 256 atoms the general kernel, 65..256 one workgroup per molecule, up to 64
+    // one wavefront per molecule; each kernel defines every gradient of its own molecules
     int st = hip_status(khan::launch_bwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                        n_atoms, khan::kSmallMaxAtoms + 1, stream));
+                                                        n_atoms, khan::kMediumMaxAtoms + 1, stream));
+    if (st != KHAN_OK) return st;
+    st = hip_status(khan::launch_bwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, stream));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_bwd_small_f32(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, stream));
 }

@@ -36,6 +36,11 @@ hipError_t launch_fwd_medium_f32(const float* X, const float* Y, const float* Z,
                                  const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
                                  const int32_t* SIs, Buckets<float> out, hipStream_t stream);
 
+hipError_t launch_bwd_medium_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
+                                 const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                                 const int32_t* SIs, Buckets<const float> g, float* gX, float* gY,
+                                 float* gZ, hipStream_t stream);
+
 template <typename T>
 hipError_t launch_bwd_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
                               const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
