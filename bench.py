@@ -8,7 +8,7 @@ Prints ONE JSON line: atoms/s for forward+gradient, with the roofline position o
 kernel and a CPU baseline (the reference's own CPU kernels compiled in place when available,
 else this repo's CPU port) timed on a bounded sample of the same batch.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload organic65536|organic1024|boxes4096]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload organic65536|organic16384_f64|boxes4096|...]
 """
 import argparse
 import json
@@ -30,11 +30,13 @@ MEASURED_TRAFFIC = {
     ("organic65536", "bwd"): 1240.5e6,
 }
 
+# name: (generator, molecules, float width in bytes, charges kernels in the step)
 WORKLOADS = {
-    "organic65536": ("organic", 65536),
-    "organic16384": ("organic", 16384),
-    "organic1024": ("organic", 1024),
-    "boxes4096": ("boxes", 4096),
+    "organic65536": ("organic", 65536, 4, False),        # the configuration the metric is quoted on
+    "organic16384": ("organic", 16384, 4, False),
+    "organic1024": ("organic", 1024, 4, False),
+    "organic16384_f64": ("organic", 16384, 8, True),     # double precision forward + backward + ani_charge
+    "boxes4096": ("boxes", 4096, 4, False),              # dense boxes of 64..256 atoms
 }
 
 
@@ -51,9 +53,10 @@ def algorithmic_work(counts, n_atoms, n_mols, w):
     }
 
 
-def cpu_baseline(batch, sample_mols_fwd, sample_mols_bwd):
-    """Forward+gradient float32 on the host, single thread, bounded sample (rank 0, N=1 only)."""
+def cpu_baseline(batch, sample_mols_fwd, sample_mols_bwd, w=4):
+    """Forward+gradient on the host, single thread, bounded sample (rank 0, N=1 only)."""
     import numpy as np
+    dtype = np.float32 if w == 4 else np.float64
     from oracle import binding as ob
     from khan_amd import datagen
 
@@ -67,13 +70,13 @@ def cpu_baseline(batch, sample_mols_fwd, sample_mols_bwd):
 
     b, sc, ac = sub(sample_mols_fwd)
     t0 = time.perf_counter()
-    ob.featurize(b.X, b.Y, b.Z, b.A, b.MOs, b.MACs, sc, ac, dtype=np.float32, impl=impl, fast=True)
+    ob.featurize(b.X, b.Y, b.Z, b.A, b.MOs, b.MACs, sc, ac, dtype=dtype, impl=impl, fast=True)
     t_fwd = (time.perf_counter() - t0) / b.n_atoms
     b2, sc2, ac2 = sub(sample_mols_bwd)
     up = datagen.normal(b2.n_atoms * 384).reshape(-1, 384)
     g = ob.scatter_rows(up, b2.A, sc2, ac2)
     t0 = time.perf_counter()
-    ob.featurize_grad(b2.X, b2.Y, b2.Z, b2.A, b2.MOs, b2.MACs, sc2, ac2, g, dtype=np.float32, impl=impl, fast=True)
+    ob.featurize_grad(b2.X, b2.Y, b2.Z, b2.A, b2.MOs, b2.MACs, sc2, ac2, g, dtype=dtype, impl=impl, fast=True)
     t_bwd = (time.perf_counter() - t0) / b2.n_atoms
     return {
         "value": 1.0 / (t_fwd + t_bwd),
@@ -111,18 +114,21 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
-    kind, n_mols = WORKLOADS[args.workload]
+    kind, n_mols, w, with_charges = WORKLOADS[args.workload]
+    tdt = torch.float32 if w == 4 else torch.float64
     batch = datagen.make_batch(kind, n_mols)
     N = batch.n_atoms
     counts = batch.work_counts()
-    work = algorithmic_work(counts, N, n_mols, 4)
+    work = algorithmic_work(counts, N, n_mols, w)
 
-    X, Y, Z = (torch.from_numpy(v).to(dev) for v in (batch.X, batch.Y, batch.Z))
+    X, Y, Z = (torch.from_numpy(v).to(dev).to(tdt) for v in (batch.X, batch.Y, batch.Z))
     A = torch.from_numpy(batch.A).to(dev)
     mol_idxs = torch.from_numpy(batch.mol_idxs).to(dev)
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
-    upstream = torch.randn(N * 384, dtype=torch.float32, device=dev, generator=gen)   # dL/dAEV ~ N(0,1)
+    upstream = torch.randn(N * 384, dtype=tdt, device=dev, generator=gen)   # dL/dAEV ~ N(0,1)
+    Q = torch.from_numpy(datagen.charges(N)).to(dev).to(tdt) if with_charges else None
+    ones_m = torch.ones(n_mols, dtype=tdt, device=dev) if with_charges else None
     torch.cuda.synchronize()
 
     if args.traffic_probe:
@@ -171,6 +177,9 @@ def main():
         gx, gy, gz = ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *grads)
         if timed:
             marks[5].record()
+        if with_charges:     # energy, then its gradient with respect to charges and coordinates
+            e = ops.ani_charge(X, Y, Z, Q, mos, macs)
+            qg = ops.ani_charge_grad_xyz(X, Y, Z, Q, mos, macs, ones_m)
         return marks, (feats, gx, gy, gz)
 
     for _ in range(args.warmup):
@@ -195,6 +204,7 @@ def main():
     dom_bytes = work["bytes_" + dom]
     dom_flops = work["flops_" + dom]
     achieved = dom_bytes / (ms[dom] * 1e-3) / 1e9
+    valu_peak = FP32_PEAK_TFLOPS if w == 4 else FP64_PEAK_TFLOPS
     roofline = {
         "kernel": "aev_bwd" if dom == "bwd" else "aev_fwd",
         "bound": "hbm",
@@ -205,16 +215,17 @@ def main():
         "traffic": MEASURED_TRAFFIC.get((args.workload, dom)),
         "launch_ms": ms[dom],
         "algorithmic_bytes": dom_bytes,
-        "valu_frac_fp32": dom_flops / (ms[dom] * 1e-3) / 1e12 / FP32_PEAK_TFLOPS,
+        "valu_frac": dom_flops / (ms[dom] * 1e-3) / 1e12 / valu_peak,
+        "valu_peak_tflops": valu_peak,
         "fwd": {"ms": ms["fwd"], "hbm_frac": work["bytes_fwd"] / (ms["fwd"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                "valu_frac_fp32": work["flops_fwd"] / (ms["fwd"] * 1e-3) / 1e12 / FP32_PEAK_TFLOPS},
+                "valu_frac": work["flops_fwd"] / (ms["fwd"] * 1e-3) / 1e12 / valu_peak},
         "bwd": {"ms": ms["bwd"], "hbm_frac": work["bytes_bwd"] / (ms["bwd"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                "valu_frac_fp32": work["flops_bwd"] / (ms["bwd"] * 1e-3) / 1e12 / FP32_PEAK_TFLOPS},
+                "valu_frac": work["flops_bwd"] / (ms["bwd"] * 1e-3) / 1e12 / valu_peak},
         "sort_offsets_ms": ms["sort"],
     }
 
     result = {
-        "metric": "AEV fwd+grad atoms/sec, fp32, 1 MI355X",
+        "metric": "AEV fwd+grad atoms/sec, fp%d, 1 MI355X" % (8 * w),
         "value": N / (ms_per_step * 1e-3),
         "unit": "atoms/s",
         "n_gpus": 1,
@@ -224,15 +235,15 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "f32" if w == 4 else "f64",
         "data": "synthetic",
-        "config": {"workload": "%s: ani_sort + AEV forward + AEV backward, %d molecules, %d atoms" % (
-            args.workload, n_mols, N), "n_mols": n_mols, "n_atoms": N, "work_counts": counts},
+        "config": {"workload": "%s: ani_sort + AEV forward + AEV backward%s, %d molecules, %d atoms" % (
+            args.workload, " + ani_charge energy and gradients" if with_charges else "", n_mols, N), "n_mols": n_mols, "n_atoms": N, "work_counts": counts},
         "molecules_per_s": n_mols / (ms_per_step * 1e-3),
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(batch, 1024 if kind == "organic" else 8, 256 if kind == "organic" else 2)
+        result["cpu_baseline"] = cpu_baseline(batch, 1024 if kind == "organic" else 8, 256 if kind == "organic" else 2, w)
     print(json.dumps(result))
 
 
