@@ -565,3 +565,132 @@ def test_autograd_second_order_wiring(ops):
     (dw,) = torch.autograd.grad(force_loss, (w,))
     want = torch.cat(ops.featurize_grad_inverse(X.detach(), Y.detach(), Z.detach(), A, mos, macs, sc, acs, *a))
     assert torch.allclose(dw, want, rtol=1e-11, atol=1e-11)
+
+
+# ----------------------------------------------------------------------------- the other full-size configurations
+def _property_checks(ops, c, ndt, grad_rtol):
+    """forward + backward of a whole batch on the device; returns rows (atom order) and gradients."""
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+    assert np.array_equal(host(sc), c.sc) and np.array_equal(host(ga), c.ga) and np.array_equal(host(ac), c.ac)
+    acs = ac.cpu()
+    tdt = torch.float32 if ndt == np.float32 else torch.float64
+    X, Y, Z, A = dev(c.X, ndt), dev(c.Y, ndt), dev(c.Z, ndt), dev(c.A)
+    f = ops.featurize(X, Y, Z, A, mos, macs, sc, acs)
+    rows = torch.cat(f).view(-1, 384)[ga.long()]
+    assert bool(torch.isfinite(rows).all()) and float(rows.min()) >= 0.0
+    gen = torch.Generator(device="cuda:0")
+    gen.manual_seed(77)
+    up = torch.randn(c.N, 384, dtype=tdt, device="cuda:0", generator=gen)
+    inv = torch.empty_like(ga.long())
+    inv[ga.long()] = torch.arange(c.N, device="cuda:0")
+    upb_all = up[inv]
+    gb, start = [], 0
+    for k in acs.tolist():
+        gb.append(upb_all[start:start + k].reshape(-1))
+        start += k
+    gx, gy, gz = ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *gb)
+    g = torch.stack([gx, gy, gz], dim=1)
+    assert bool(torch.isfinite(g).all())
+    seg = torch.from_numpy(c.mol_idxs.astype(np.int64)).to("cuda:0")
+    net = torch.zeros(c.n_mols, 3, device="cuda:0", dtype=torch.float64).index_add_(0, seg, g.double())
+    mag = torch.zeros(c.n_mols, 3, device="cuda:0", dtype=torch.float64).index_add_(0, seg, g.double().abs())
+    rel = (net.abs() / (mag + 1e-30)).max().item()
+    say("   net force / sum |force| per molecule, worst %.3e" % rel)
+    assert rel < grad_rtol
+    # radial symmetry: sum over centres of type a of their [partner type b] block = the same with a, b swapped
+    # (every unordered pair is counted once from each side), per molecule-independent global sums
+    types = torch.from_numpy(np.minimum(c.A, 3).astype(np.int64)).to("cuda:0")
+    rad = rows[:, :64].double().view(-1, 4, 16)
+    S = torch.zeros(4, 4, 16, dtype=torch.float64, device="cuda:0").index_add_(0, types, rad)
+    sym = float((S - S.transpose(0, 1)).abs().max() / S.abs().max())
+    say("   radial block symmetry, relative %.3e" % sym)
+    assert sym < (1e-5 if ndt == np.float32 else 1e-12)
+    return rows, g, up
+
+
+def test_full_size_double_precision_configuration(ops):
+    # 16,384 molecules in float64 with the charge kernels: properties at full size, the oracle on both ends
+    say("case: organic 16384 float64 + charges, full size")
+    M = 16384
+    b = datagen.make_batch("organic", M)
+    c = Case.from_batch(b)
+    rows, g, up = _property_checks(ops, c, np.float64, 1e-11)
+    for first, cnt in ((0, 128), (M - 128, 128)):
+        sb = datagen.make_batch("organic", cnt, first_mol=first)
+        sc_ = Case.from_batch(sb)
+        a0 = int(c.MOs[first])
+        ref64 = ob.gather_rows(sc_.oracle_feat(np.float64), sc_.ga)
+        assert_close("rows of molecules %d.. f64" % first, host(rows[a0:a0 + sb.n_atoms]), ref64, F64_RTOL, F64_ATOL)
+        upb = ob.scatter_rows(host(up[a0:a0 + sb.n_atoms]), sb.A, sc_.sc, sc_.ac)
+        g64 = sc_.oracle_grad(upb)
+        assert_close("gradient of molecules %d.. f64" % first, host(g[a0:a0 + sb.n_atoms]), g64, F64_RTOL, 0.0,
+                     scale=mol_scale(g64, sc_.MOs, sc_.MACs))
+    # charges at full size: Euler identity and zero net force per molecule, oracle on the first 256 molecules
+    q = datagen.charges(b.n_atoms).astype(np.float64)
+    X, Y, Z, Q = dev(b.X, np.float64), dev(b.Y, np.float64), dev(b.Z, np.float64), dev(q)
+    mos, macs = dev(b.MOs), dev(b.MACs)
+    ones = torch.ones(M, dtype=torch.float64, device="cuda:0")
+    E = ops.ani_charge(X, Y, Z, Q, mos, macs)
+    qg, cx, cy, cz = ops.ani_charge_grad_xyz(X, Y, Z, Q, mos, macs, ones)
+    seg = torch.from_numpy(b.mol_idxs.astype(np.int64)).to("cuda:0")
+    euler = 0.5 * torch.zeros(M, dtype=torch.float64, device="cuda:0").index_add_(0, seg, Q * qg)
+    Eabs = ops.ani_charge(X, Y, Z, Q.abs(), mos, macs)
+    assert float(((euler - E).abs() / (Eabs + 1e-300)).max()) < 1e-11
+    net = torch.zeros(M, 3, dtype=torch.float64, device="cuda:0").index_add_(0, seg, torch.stack([cx, cy, cz], 1))
+    mag = torch.zeros(M, 3, dtype=torch.float64, device="cuda:0").index_add_(0, seg, torch.stack([cx, cy, cz], 1).abs())
+    assert float((net.abs() / (mag + 1e-300)).max()) < 1e-10
+    n256 = int(b.MOs[256])
+    E64 = ob.ani_charge(b.X[:n256], b.Y[:n256], b.Z[:n256], q[:n256], b.MOs[:256], b.MACs[:256], dtype=np.float64)
+    Ea = host(Eabs)[:256]
+    assert_close("charge energy, first 256 molecules", host(E)[:256], E64, F64_RTOL, 0.0, scale=Ea)
+
+
+def test_full_size_dense_boxes_configuration(ops):
+    # 4,096 boxes of 64..256 atoms in float32: properties at full size, the oracle on the first and last boxes
+    say("case: boxes 4096 float32, full size")
+    M = 4096
+    b = datagen.make_batch("boxes", M)
+    c = Case.from_batch(b)
+    rows, g, up = _property_checks(ops, c, np.float32, 2e-5)
+    for first, cnt in ((0, 3), (M - 3, 3)):
+        sb = datagen.make_batch("boxes", cnt, first_mol=first)
+        sc_ = Case.from_batch(sb)
+        a0 = int(c.MOs[first])
+        assert np.array_equal(sb.X, c.X[a0:a0 + sb.n_atoms])
+        ref64 = ob.gather_rows(sc_.oracle_feat(np.float64), sc_.ga)
+        assert_close("rows of boxes %d.. vs f64 oracle" % first, host(rows[a0:a0 + sb.n_atoms]), ref64, F32_RTOL, F32_ATOL)
+        upb = ob.scatter_rows(host(up[a0:a0 + sb.n_atoms]).astype(np.float64), sb.A, sc_.sc, sc_.ac)
+        g64 = sc_.oracle_grad(upb)
+        assert_close("gradient of boxes %d.. vs f64 oracle" % first, host(g[a0:a0 + sb.n_atoms]), g64,
+                     F32_RTOL, F32_ATOL, scale=mol_scale(g64, sc_.MOs, sc_.MACs))
+
+
+def test_gradient_against_central_differences_on_64_molecules(ops):
+    # the backward pass against a central difference of the float64 forward pass, h = 1e-4 A, on 64 molecules:
+    # directional derivatives along 8 random directions
+    say("case: central differences of the float64 forward, 64 molecules")
+    c = Case.from_batch(datagen.make_batch("organic", 64, first_mol=500))
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+    acs = ac.cpu()
+    A = dev(c.A)
+    X, Y, Z = dev(c.X, np.float64), dev(c.Y, np.float64), dev(c.Z, np.float64)
+    rng = np.random.default_rng(8)
+    w = dev(rng.standard_normal(c.N * 384))
+    wb, start = [], 0
+    for k in acs.tolist():
+        wb.append(w[start * 384:(start + k) * 384])
+        start += k
+    g64 = ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *wb)
+    g32 = ops.featurize_grad(X.float(), Y.float(), Z.float(), A, mos, macs, sc, acs, *[t.float() for t in wb])
+    h = 1e-4
+    for trial in range(8):
+        d = [dev(rng.standard_normal(c.N)) for _ in range(3)]
+        Lp = float((torch.cat(ops.featurize(X + h * d[0], Y + h * d[1], Z + h * d[2], A, mos, macs, sc, acs)) * w).sum())
+        Lm = float((torch.cat(ops.featurize(X - h * d[0], Y - h * d[1], Z - h * d[2], A, mos, macs, sc, acs)) * w).sum())
+        num = (Lp - Lm) / (2 * h)
+        ana64 = float(sum((a * b_).sum() for a, b_ in zip(g64, d)))
+        ana32 = float(sum((a.double() * b_).sum() for a, b_ in zip(g32, d)))
+        scale = float(sum((a.abs() * b_.abs()).sum() for a, b_ in zip(g64, d)))
+        say("   direction %d: numeric %.9e  f64 %.9e  f32 %.9e" % (trial, num, ana64, ana32))
+        assert abs(num - ana64) <= 1e-6 * scale      # truncation of the difference quotient, O(h^2)
+        assert abs(ana32 - ana64) <= 1e-5 * scale
