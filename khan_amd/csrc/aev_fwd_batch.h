@@ -7,33 +7,33 @@
 namespace khan {
 
 // LDS working set of one wavefront
+template <typename T>
 struct __align__(16) FwdWaveLds {
-    float4 atom[64];            // x, y, z, type (sorted order)
-    float4 nbr[kB][kCapA];      // unit vector (centre minus partner)/r, and r
-    float nbr_fc[kB][kCapA];    // f_C(r, A_Rc)
-    float2 rad[64];             // (r, f_C(r, R_Rc)); group g of a scan step owns [g*W, (g+1)*W)
-    float rec[64][12];          // phase-1 records: A_0..7, G_0..3
-    SegDesc seg[64];            // non-empty segments of the batch, in order
-    unsigned bits[kBitWords];   // bit per triple slot: a segment starts here
-    int nA[kB][4];              // angular partners per type, per centre of the batch
-    int nR[4][4];               // radial partners per type, per group of the scan step
+    typename Fast<T>::vec4 atom[64];          // x, y, z, type (sorted order)
+    typename Fast<T>::vec4 nbr[kB][kCapA];    // unit vector (centre minus partner)/r, and r
+    T nbr_fc[kB][kCapA];                      // f_C(r, A_Rc)
+    typename Fast<T>::vec2 rad[64];           // (r, f_C(r, R_Rc)); group g of a scan step owns [g*W, (g+1)*W)
+    T rec[64][12];                            // phase-1 records: A_0..7, G_0..3
+    SegDesc seg[64];                          // non-empty segments of the batch, in order
+    unsigned bits[kBitWords];                 // bit per triple slot: a segment starts here
+    int nA[kB][4];                            // angular partners per type, per centre of the batch
+    int nR[4][4];                             // radial partners per type, per group of the scan step
 };
-
 
 // Segment table, phases 1 and 2 and the zero fill of empty blocks for centres 0..nb-1 of a batch.
 // `row_of_centre(b)` returns the address of centre b's 384-float output row; it is called by all
 // lanes together, with a per-lane b for the segment table and a wave-uniform b for the zero fill.
-template <typename RowOfCentre>
-__device__ __forceinline__ void fwd_angular_batch(FwdWaveLds& S, const LaneConsts<float>& L, int lane, int nb,
+template <typename T, typename RowOfCentre>
+__device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T>& S, const LaneConsts<T>& L, int lane, int nb,
                                                   RowOfCentre row_of_centre)
 {
+    typedef typename Fast<T>::vec4 vec4;
     const unsigned long long lane_bit = 1ull << lane;
     const unsigned long long lt_mask = lane_bit - 1ull;
     // segment-table lanes: lane = centre-in-batch * 10 + type-pair index (HH HC HN HO CC CN CO NN NO OO)
     const int seg_b = lane / kNumPairBlocks, seg_pt = lane - seg_b * kNumPairBlocks;
     const int seg_a = seg_pt < 4 ? 0 : seg_pt < 7 ? 1 : seg_pt < 9 ? 2 : 3;
     const int seg_bt = seg_pt < 4 ? seg_pt : seg_pt < 7 ? seg_pt - 3 : seg_pt < 9 ? seg_pt - 5 : 3;
-    const float kAngExp = -kA_eta_f * 1.44269504088896340736f;   // exp(-eta d^2) = exp2(kAngExp d^2)
     const int ang_t = L.ts >> 2, ang_s = L.ts & 3;
 
     // ------------------------------------------------ segment table of the batch
@@ -42,7 +42,7 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds& S, const LaneConst
     {
         // row of the segment's centre (every lane takes part: the lookup may be a lane exchange)
         const unsigned long long rowp = row_of_centre(min(seg_b, kB - 1)) +
-                                        static_cast<unsigned long long>((kRadial + seg_pt * kAngBlock) * sizeof(float));
+                                        static_cast<unsigned long long>((kRadial + seg_pt * kAngBlock) * sizeof(T));
         seg_row_lo = static_cast<unsigned>(rowp);
         seg_row_hi = static_cast<unsigned>(rowp >> 32);
     }
@@ -75,13 +75,13 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds& S, const LaneConst
     wave_lds_fence();
 
     // ------------------------------------------------ phases 1 and 2, 64 triple slots at a time
-    float acc = 0.f;            // partial sums of the open segment
+    T acc = T(0);               // partial sums of the open segment
     unsigned cur_lo = 0, cur_hi = 0;   // where the open segment's 32 floats go (wave-uniform)
     int carry = 0;              // non-empty segments that start before this step
     // closes the open segment: the halves are added and 32 floats go straight to the row
     auto flush = [&]() {
-        const float tot = half_wave_sum(acc);
-        float* dst = reinterpret_cast<float*>((static_cast<unsigned long long>(cur_hi) << 32) | cur_lo);
+        const T tot = half_wave_sum(acc);
+        T* dst = reinterpret_cast<T*>((static_cast<unsigned long long>(cur_hi) << 32) | cur_lo);
         if (lane < 32) store_global(dst + lane, tot);
     };
 
@@ -115,56 +115,56 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds& S, const LaneConst
             k = 0;
             bsel = 0;
         }
-        const float4 vj = S.nbr[bsel][j], vk = S.nbr[bsel][k];
-        const float fj = S.nbr_fc[bsel][j], fk = S.nbr_fc[bsel][k];
+        const vec4 vj = S.nbr[bsel][j], vk = S.nbr[bsel][k];
+        const T fj = S.nbr_fc[bsel][j], fk = S.nbr_fc[bsel][k];
 
-        float c = vj.x * vk.x + vj.y * vk.y + vj.z * vk.z;
-        c = fminf(fmaxf(c, -1.0f), 1.0f);
-        const float cx = vj.y * vk.z - vj.z * vk.y;
-        const float cy = vj.z * vk.x - vj.x * vk.z;
-        const float cz = vj.x * vk.y - vj.y * vk.x;
-        const float s = __builtin_amdgcn_sqrtf(cx * cx + cy * cy + cz * cz);
-        float Af[8];
+        T c = vj.x * vk.x + vj.y * vk.y + vj.z * vk.z;
+        c = fmin(fmax(c, T(-1)), T(1));
+        const T cx = vj.y * vk.z - vj.z * vk.y;
+        const T cy = vj.z * vk.x - vj.x * vk.z;
+        const T cz = vj.x * vk.y - vj.y * vk.x;
+        const T s = Fast<T>::sqrt_(cx * cx + cy * cy + cz * cz);
+        T Af[8];
 #pragma unroll
         for (int t = 0; t < 8; ++t)
-            Af[t] = pow8(fmaf(s, static_cast<float>(kSinTheta[t]), fmaf(c, static_cast<float>(kCosTheta[t]), 1.0f)));
-        const float rho = 0.5f * (vj.w + vk.w);
-        const float P = 0.0078125f * fj * fk;
-        float Gf[4];
+            Af[t] = pow8(fma(s, static_cast<T>(kSinTheta[t]), fma(c, static_cast<T>(kCosTheta[t]), T(1))));
+        const T rho = T(0.5) * (vj.w + vk.w);
+        const T P = T(0.0078125) * fj * fk;
+        T Gf[4];
 #pragma unroll
         for (int sidx = 0; sidx < 4; ++sidx) {
-            const float dd = rho - kA_Rs_f[sidx];
+            const T dd = rho - static_cast<T>(kA_Rs_f[sidx]);
             // padding slots read whatever sits in the list: select, do not multiply, so that a
             // stray NaN cannot reach the sums
-            Gf[sidx] = ok ? __builtin_amdgcn_exp2f(kAngExp * dd * dd) * P : 0.f;
+            Gf[sidx] = ok ? Fast<T>::gauss(static_cast<T>(kA_eta_f), dd) * P : T(0);
         }
 #pragma unroll
-        for (int t = 0; t < 8; ++t) Af[t] = ok ? Af[t] : 0.f;
-        float4* recp = reinterpret_cast<float4*>(S.rec[lane]);
-        recp[0] = make_float4(Af[0], Af[1], Af[2], Af[3]);
-        recp[1] = make_float4(Af[4], Af[5], Af[6], Af[7]);
-        recp[2] = make_float4(Gf[0], Gf[1], Gf[2], Gf[3]);
+        for (int t = 0; t < 8; ++t) Af[t] = ok ? Af[t] : T(0);
+        vec4* recp = reinterpret_cast<vec4*>(S.rec[lane]);
+        recp[0] = Fast<T>::make4(Af[0], Af[1], Af[2], Af[3]);
+        recp[1] = Fast<T>::make4(Af[4], Af[5], Af[6], Af[7]);
+        recp[2] = Fast<T>::make4(Gf[0], Gf[1], Gf[2], Gf[3]);
         wave_lds_fence();
 
         // phase 2: lane = (half, theta_t, Rs_s); the halves take alternate records.  Records past
         // `total` in the last step are zeros, so whole groups of eight pairs can always be run.
         const int npairs = min(64, total - base) >> 1;
-        const float* pa = &S.rec[L.half][ang_t];
-        const float* pg = &S.rec[L.half][8 + ang_s];
+        const T* pa = &S.rec[L.half][ang_t];
+        const T* pg = &S.rec[L.half][8 + ang_s];
         unsigned long long mm = starts;
         if (base == 0) {            // the batch's first segment opens here; nothing to close
             cur_lo = static_cast<unsigned>(lane_read(static_cast<int>(d.row_lo), 0));
             cur_hi = static_cast<unsigned>(lane_read(static_cast<int>(d.row_hi), 0));
             mm &= ~1ull;
         }
-        auto load8 = [&](int q0, float (&av)[8], float (&gv)[8]) {
+        auto load8 = [&](int q0, T (&av)[8], T (&gv)[8]) {
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
                 av[u] = pa[(q0 + u) * 24];
                 gv[u] = pg[(q0 + u) * 24];
             }
         };
-        auto run8 = [&](int q0, const float (&av)[8], const float (&gv)[8]) {
+        auto run8 = [&](int q0, const T (&av)[8], const T (&gv)[8]) {
             const unsigned m16 = static_cast<unsigned>(mm) & 0xffffu;     // this group's 16 slots
             mm >>= 16;
 #pragma unroll
@@ -176,13 +176,13 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds& S, const LaneConst
                     asm volatile("" : "+s"(first));      // keeps the lane reads inside this branch
                     cur_lo = static_cast<unsigned>(lane_read(static_cast<int>(d.row_lo), first));
                     cur_hi = static_cast<unsigned>(lane_read(static_cast<int>(d.row_hi), first));
-                    acc = 0.f;
+                    acc = T(0);
                 }
-                acc = fmaf(av[u], gv[u], acc);
+                acc = fma(av[u], gv[u], acc);
             }
         };
         // eight record pairs per group, the next group's LDS reads in flight while one is summed
-        float a0[8], g0[8], a1[8], g1[8];
+        T a0[8], g0[8], a1[8], g1[8];
         load8(0, a0, g0);
         for (int q0 = 0; q0 < npairs; q0 += 16) {
             const bool more1 = q0 + 8 < npairs;
@@ -204,13 +204,13 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds& S, const LaneConst
             const unsigned eb = static_cast<unsigned>(empty >> (b * kNumPairBlocks)) & 0x3ffu;
             if (eb == 0u) continue;
             const unsigned long long rb = row_of_centre(b);
-            float* row = reinterpret_cast<float*>((static_cast<unsigned long long>(static_cast<unsigned>(uniform(static_cast<int>(rb >> 32)))) << 32) |
+            T* row = reinterpret_cast<T*>((static_cast<unsigned long long>(static_cast<unsigned>(uniform(static_cast<int>(rb >> 32)))) << 32) |
                                                   static_cast<unsigned>(uniform(static_cast<int>(rb & 0xffffffffull)))) + kRadial;
 #pragma unroll
             for (int pp = 0; pp < 5; ++pp) {
                 if (((eb >> (2 * pp)) & 3u) != 0u) {
                     const int pt = 2 * pp + L.half;
-                    if ((eb >> pt) & 1u) store_global(row + pt * kAngBlock + L.ts, 0.f);
+                    if ((eb >> pt) & 1u) store_global(row + pt * kAngBlock + L.ts, T(0));
                 }
             }
         }

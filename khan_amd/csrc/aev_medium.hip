@@ -37,11 +37,11 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
     Buckets<float> out)
 {
     __shared__ MedShared M;
-    __shared__ FwdWaveLds lds_wave[4];
+    __shared__ FwdWaveLds<float> lds_wave[4];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = uniform(tid >> 6);
-    FwdWaveLds& S = lds_wave[wave];
+    FwdWaveLds<float>& S = lds_wave[wave];
     const LaneConsts<float> L = lane_consts<float>(lane);
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
     const float inv_rc_R = 1.0f / kR_Rc_f, inv_rc_A = 1.0f / kA_Rc_f;
@@ -172,7 +172,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
             }
 
             // ------------------------------------------------ segment table, phases 1 and 2, zero fill
-            fwd_angular_batch(S, L, lane, nb, [&](int b) -> unsigned long long {
+            fwd_angular_batch<float>(S, L, lane, nb, [&](int b) -> unsigned long long {
                 const int idx = min(c0 + b, kMediumMaxAtoms - 1);
                 return (static_cast<unsigned long long>(M.row_hi[idx]) << 32) | M.row_lo[idx];
             });

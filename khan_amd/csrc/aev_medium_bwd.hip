@@ -40,14 +40,13 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
     Buckets<const float> gin, float* __restrict__ gX, float* __restrict__ gY, float* __restrict__ gZ)
 {
     __shared__ MedBwdShared M;
-    __shared__ BwdPool pools[4];
+    __shared__ BwdPool<float> pools[4];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = uniform(tid >> 6);
-    BwdPool& P = pools[wave];
+    BwdPool<float>& P = pools[wave];
     const LaneConsts<float> L = lane_consts<float>(lane);
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
-    const float inv_rc_A = 1.0f / kA_Rc_f;
 
     for (int mol = blockIdx.x; mol < n_mols; mol += gridDim.x) {
         const int n = uniform(MACs[mol]);
@@ -176,14 +175,14 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                         if ((mA[ch] >> lane) & 1ull) {
                             const int p = pos + popc64(mA[ch] & lt_mask);
                             float fc, dfc;
-                            cutoff_poly_grad(r[ch] * inv_rc_A, inv_rc_A, fc, dfc);
+                            Fast<float>::cutoff_grad(r[ch], kA_Rc_f, fc, dfc);
                             P.nbr[p] = make_float4(dx[ch] * inv, dy[ch] * inv, dz[ch] * inv, r[ch]);
                             P.nbr_fc[p] = make_float2(fc, dfc);
                             P.nbr_idx[p] = static_cast<unsigned char>(j);
                         }
                         pos += popc64(mA[ch]);
                         if ((mR[ch] >> lane) & 1ull) {
-                            const float sc = bwd_radial_pair(grow, type_of(j), r[ch], inv);
+                            const float sc = bwd_radial_pair<float>(grow, type_of(j), r[ch], inv);
                             const float fx = sc * dx[ch], fy = sc * dy[ch], fz = sc * dz[ch];
                             cfx += fx;
                             cfy += fy;
@@ -208,18 +207,9 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
 
             // ---- the angular upstream blocks of the batch's rows go to LDS (80 x 16 bytes per row)
             {
-                v4f st0[kB], st1[kB];
-#pragma unroll
-                for (int b = 0; b < kB; ++b) {
-                    st0[b] = v4f{0.f, 0.f, 0.f, 0.f};
-                    st1[b] = v4f{0.f, 0.f, 0.f, 0.f};
-                    if (b < nb) {
-                        const global_v4f_ptr rowp = (global_v4f_ptr)(row_of(lane_read(cv, b)) + kRadial);
-                        st0[b] = rowp[lane];
-                        if (lane < 16) st1[b] = rowp[64 + lane];
-                    }
-                }
-                bwd_stage_blocks(P, lane, nb, st0, st1);
+                RowStage<float> stage;
+                stage.fetch(lane, nb, [&](int b) { return row_of(lane_read(cv, b)); });
+                stage.store(P, lane, nb);
             }
             wave_lds_fence();
 
@@ -232,7 +222,7 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
             const int bs = live ? b : 0;
             const int pb = sel6(bs, 0, pf1, pf2, pf3, pf4, pf5);
             const int m = sel6(bs, pf1, pf2, pf3, pf4, pf5, pf6) - pb;
-            const float4 f = bwd_angular_rounds(P, lane, live, bs, pb, m, type_of);
+            const float4 f = bwd_angular_rounds<float>(P, lane, live, bs, pb, m, type_of);
 
             // ------------------------------------------------ gather
             if (live) add_force(P.nbr_idx[lane], f.x, f.y, f.z);

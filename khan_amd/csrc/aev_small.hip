@@ -1,4 +1,4 @@
-// AEV forward for molecules of up to 64 atoms (float32): one wavefront per molecule.
+// AEV forward for molecules of up to 64 atoms (float32 and float64): one wavefront per molecule.
 //
 // How one wavefront spends its 64 lanes
 //   sort     one atom per lane, lanes reordered by atom type (4-bin counting sort with ballots).  Every
@@ -27,13 +27,18 @@ namespace khan {
 
 namespace {
 
-__global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) void aev_fwd_small_kernel(
-    const float* __restrict__ X, const float* __restrict__ Y, const float* __restrict__ Z,
+// float: 4 wavefronts per SIMD (LDS 9.8 KB, <= 128 VGPRs); double: 2 (LDS 19.6 KB)
+template <typename T>
+__global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 4 : 2, sizeof(T) == 4 ? 4 : 2)))
+void aev_fwd_small_kernel(
+    const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
-    Buckets<float> out)
+    Buckets<T> out)
 {
-    __shared__ FwdWaveLds lds_all[kWavesPerBlock];
+    typedef typename Fast<T>::vec4 vec4;
+    typedef typename Fast<T>::vec2 vec2;
+    __shared__ FwdWaveLds<T> lds_all[kWavesPerBlock];
     const int lane = threadIdx.x & 63;
     const int wave = uniform(threadIdx.x >> 6);
     const int mol = blockIdx.x * kWavesPerBlock + wave;
@@ -41,14 +46,14 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
     const int n = uniform(MACs[mol]);
     const int off = uniform(MOs[mol]);
     if (n <= 0 || n > 64) return;                 // larger molecules belong to the general kernel
-    FwdWaveLds& S = lds_all[wave];
-    const LaneConsts<float> L = lane_consts<float>(lane);
+    FwdWaveLds<T>& S = lds_all[wave];
+    const LaneConsts<T> L = lane_consts<T>(lane);
     const unsigned long long lane_bit = 1ull << lane;
     const unsigned long long lt_mask = lane_bit - 1ull;
 
     // ------------------------------------------------------------ load, sort lanes by type
     const bool have = lane < n;
-    float x = 0.f, y = 0.f, z = 0.f;
+    T x = T(0), y = T(0), z = T(0);
     int type = 0, orig = lane;
     unsigned long long rowbits = 0;
     if (have) {
@@ -83,11 +88,11 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
     orig = lane_push(dest, orig);
     const int rp_lo = lane_push(dest, static_cast<int>(rowbits & 0xffffffffull));
     const int rp_hi = lane_push(dest, static_cast<int>(rowbits >> 32));
-    S.atom[lane] = make_float4(x, y, z, __int_as_float(type));
-    auto row_of = [&](int sorted_lane) -> float* {     // sorted_lane is wave-uniform
+    S.atom[lane] = Fast<T>::make4(x, y, z, static_cast<T>(type));
+    auto row_of = [&](int sorted_lane) -> T* {     // sorted_lane is wave-uniform
         const unsigned lo = static_cast<unsigned>(lane_read(rp_lo, sorted_lane));
         const unsigned hi = static_cast<unsigned>(lane_read(rp_hi, sorted_lane));
-        return reinterpret_cast<float*>((static_cast<unsigned long long>(hi) << 32) | lo);
+        return reinterpret_cast<T*>((static_cast<unsigned long long>(hi) << 32) | lo);
     };
     // sorted-order type ranges: partner index p has type a iff tbase[a] <= p < tbase[a] + tcount[a]
     unsigned long long smask[4];
@@ -113,8 +118,6 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
     const int rg_g = G == 4 ? rg : G == 2 ? (rg >> 1) : 0;
     const int rg_s = G == 4 ? 0 : G == 2 ? (rg & 1) : rg;
 
-    const float inv_rc_R = 1.0f / kR_Rc_f, inv_rc_A = 1.0f / kA_Rc_f;
-    const float kRadExp = -kR_eta_f * 1.44269504088896340736f;   // exp(-eta d^2) = exp2(kRadExp d^2)
     wave_lds_fence();
 
     for (int c0 = 0; c0 < n; c0 += kB) {
@@ -126,21 +129,21 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
             const int b = b0 + grp;                      // centre-in-batch of this lane's group
             const int i = c0 + b;
             const bool centre_ok = b < nb;
-            const float4 ai = S.atom[centre_ok ? i : 0];
-            const float4 aj = S.atom[jl];
-            const float dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
-            const float r = sqrtf(dx * dx + dy * dy + dz * dz);
+            const vec4 ai = S.atom[centre_ok ? i : 0];
+            const vec4 aj = S.atom[jl];
+            const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
+            const T r = sqrt(dx * dx + dy * dy + dz * dz);
             const bool valid = centre_ok && (jl < n) && (jl != i);
             const bool inR = valid && (r < kR_Rc_f);
             const bool inA = valid && (r < kA_Rc_f);
             const unsigned long long mR = wave_ballot(inR), mA = wave_ballot(inA);
             const bool fits = popc64(mA & sub_mask) <= kCapA;
-            if (inR) S.rad[grp * W + popc64(mR & ltg_mask)] = make_float2(r, cutoff_poly(r * inv_rc_R));
+            if (inR) S.rad[grp * W + popc64(mR & ltg_mask)] = Fast<T>::make2(r, Fast<T>::cutoff(r, static_cast<T>(kR_Rc_f)));
             if (inA && fits) {
                 const int pos = popc64(mA & ltg_mask);
-                const float inv = __builtin_amdgcn_rcpf(r);
-                S.nbr[centre_ok ? b : 0][pos] = make_float4(dx * inv, dy * inv, dz * inv, r);
-                S.nbr_fc[centre_ok ? b : 0][pos] = cutoff_poly(r * inv_rc_A);
+                const T inv = Fast<T>::rcp(r);
+                S.nbr[centre_ok ? b : 0][pos] = Fast<T>::make4(dx * inv, dy * inv, dz * inv, r);
+                S.nbr_fc[centre_ok ? b : 0][pos] = Fast<T>::cutoff(r, static_cast<T>(kA_Rc_f));
             }
             {   // bit b of `overflow`: centre b of the batch has too many angular partners
                 const unsigned long long ov = wave_ballot(!fits && jl == 0 && centre_ok);
@@ -164,27 +167,27 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
             // ---- radial features of the G centres of this step
             {
                 const int4 cn = *reinterpret_cast<const int4*>(S.nR[rg_g]);
-                const float2* list = &S.rad[rg_g * W];
+                const vec2* list = &S.rad[rg_g * W];
                 const int cb = b0 + rg_g;
                 const int ci = min(c0 + cb, 63);
                 const unsigned rlo = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(ci << 2, rp_lo));
                 const unsigned rhi = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(ci << 2, rp_hi));
-                float* row = reinterpret_cast<float*>((static_cast<unsigned long long>(rhi) << 32) | rlo);
+                T* row = reinterpret_cast<T*>((static_cast<unsigned long long>(rhi) << 32) | rlo);
                 int obase = 0;
 #pragma unroll
                 for (int a = 0; a < 4; ++a) {
                     const int cnt_a = a == 0 ? cn.x : a == 1 ? cn.y : a == 2 ? cn.z : cn.w;
-                    float acc_r = 0.f;
+                    T acc_r = T(0);
                     for (int q0 = 0; q0 < mxR[a]; q0 += 4 * rg_ns) {
                         // four entries of this lane's slot per trip; slot s takes q = s, s+ns, s+2ns, ...
-                        float2 e[4];
+                        vec2 e[4];
 #pragma unroll
                         for (int u = 0; u < 4; ++u) e[u] = list[min(obase + q0 + u * rg_ns + rg_s, W - 1)];
 #pragma unroll
                         for (int u = 0; u < 4; ++u) {
-                            const float dd = e[u].x - L.rrs;
-                            const float v = __builtin_amdgcn_exp2f(kRadExp * dd * dd) * e[u].y;
-                            acc_r += (q0 + u * rg_ns + rg_s < cnt_a) ? v : 0.f;   // stale entries: select
+                            const T dd = e[u].x - L.rrs;
+                            const T v = Fast<T>::gauss(static_cast<T>(kR_eta_f), dd) * e[u].y;
+                            acc_r += (q0 + u * rg_ns + rg_s < cnt_a) ? v : T(0);   // stale entries: select
                         }
                     }
                     if (rg_ns >= 2) acc_r += __shfl_xor(acc_r, 16, 64);
@@ -197,7 +200,7 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
         }
 
         // ------------------------------------------------ segment table, phases 1 and 2, zero fill
-        fwd_angular_batch(S, L, lane, nb, [&](int b) -> unsigned long long {
+        fwd_angular_batch<T>(S, L, lane, nb, [&](int b) -> unsigned long long {
             const int cl = min(c0 + b, 63);
             const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(cl << 2, rp_lo));
             const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(cl << 2, rp_hi));
@@ -210,8 +213,8 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
             for (int b = 0; b < nb; ++b) {
                 if (overflow & (1u << b)) {
                     const int i_orig = lane_read(orig, c0 + b);
-                    fwd_center_generic<float>(L, lane, X, Y, Z, A, off, n, i_orig,
-                                              reinterpret_cast<float*>(S.rec), row_of(c0 + b));
+                    fwd_center_generic<T>(L, lane, X, Y, Z, A, off, n, i_orig,
+                                          reinterpret_cast<T*>(S.rec), row_of(c0 + b));
                 }
             }
             wave_lds_fence();
@@ -221,14 +224,18 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_pe
 
 }  // namespace
 
-hipError_t launch_fwd_small_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
-                                const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
-                                const int32_t* SIs, Buckets<float> out, hipStream_t stream)
+template <typename T>
+hipError_t launch_fwd_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
+                            const int32_t* MACs, int32_t n_mols, const int32_t* SIs, Buckets<T> out,
+                            hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
     const unsigned blocks = (static_cast<unsigned>(n_mols) + kWavesPerBlock - 1u) / kWavesPerBlock;
-    aev_fwd_small_kernel<<<dim3(blocks), dim3(64 * kWavesPerBlock), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, out);
+    aev_fwd_small_kernel<T><<<dim3(blocks), dim3(64 * kWavesPerBlock), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, out);
     return hipGetLastError();
 }
+
+template hipError_t launch_fwd_small<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<float>, hipStream_t);
+template hipError_t launch_fwd_small<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<double>, hipStream_t);
 
 }  // namespace khan

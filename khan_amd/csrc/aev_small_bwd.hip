@@ -1,4 +1,4 @@
-// AEV backward (dL/dxyz) for molecules of up to 64 atoms, float32: one wavefront per molecule.
+// AEV backward (dL/dxyz) for molecules of up to 64 atoms, float32 and float64: one wavefront per molecule.
 //
 // Lanes are sorted by atom type as in the forward kernel.  A first sweep counts the angular partners
 // of every atom; centres are then taken in order of decreasing count, in batches of up to six whose
@@ -30,34 +30,39 @@ namespace khan {
 
 namespace {
 
+template <typename T>
 struct __align__(16) BwdLds {
-    float4 atom[64];                     // x, y, z, type (sorted order)
-    BwdPool pool;                        // partner lists and staged upstream values of the batch
-    float force[3][64];                  // dL/dx, dL/dy, dL/dz per sorted atom
+    typename Fast<T>::vec4 atom[64];     // x, y, z, type (sorted order)
+    BwdPool<T> pool;                     // partner lists and staged upstream values of the batch
+    T force[3][64];                      // dL/dx, dL/dy, dL/dz per sorted atom
     int nM[8];                           // angular partners per centre of the batch
     unsigned char inv[64];               // original atom index -> sorted lane
 };
 
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void aev_bwd_small_kernel(
-    const float* __restrict__ X, const float* __restrict__ Y, const float* __restrict__ Z,
+// float: 3 wavefronts per SIMD (LDS 13.2 KB); double: 1 (LDS 26 KB, twice the registers)
+template <typename T>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 3 : 1, sizeof(T) == 4 ? 3 : 2)))
+void aev_bwd_small_kernel(
+    const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
-    Buckets<const float> gin, float* __restrict__ gX, float* __restrict__ gY, float* __restrict__ gZ)
+    Buckets<const T> gin, T* __restrict__ gX, T* __restrict__ gY, T* __restrict__ gZ)
 {
-    __shared__ BwdLds S;
+    typedef typename Fast<T>::vec4 vec4;
+    __shared__ BwdLds<T> S;
     const int lane = threadIdx.x;
     const int mol = blockIdx.x;
     if (mol >= n_mols) return;
     const int n = uniform(MACs[mol]);
     const int off = uniform(MOs[mol]);
     if (n <= 0 || n > 64) return;                 // larger molecules belong to the general kernel
-    const LaneConsts<float> L = lane_consts<float>(lane);
+    const LaneConsts<T> L = lane_consts<T>(lane);
     const unsigned long long lane_bit = 1ull << lane;
     const unsigned long long lt_mask = lane_bit - 1ull;
 
     // ------------------------------------------------------------ load, sort lanes by type
     const bool have = lane < n;
-    float x = 0.f, y = 0.f, z = 0.f;
+    T x = T(0), y = T(0), z = T(0);
     int type = 0, orig = lane;
     unsigned long long rowbits = 0;
     if (have) {
@@ -93,31 +98,30 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
     orig = lane_push(dest, orig);
     const int rp_lo = lane_push(dest, static_cast<int>(rowbits & 0xffffffffull));
     const int rp_hi = lane_push(dest, static_cast<int>(rowbits >> 32));
-    S.atom[lane] = make_float4(x, y, z, __int_as_float(type));
-    S.force[0][lane] = 0.f;
-    S.force[1][lane] = 0.f;
-    S.force[2][lane] = 0.f;
-    auto row_of_lane = [&](int sorted_lane) -> const float* {     // per-lane source index
+    S.atom[lane] = Fast<T>::make4(x, y, z, static_cast<T>(type));
+    S.force[0][lane] = T(0);
+    S.force[1][lane] = T(0);
+    S.force[2][lane] = T(0);
+    auto row_of_lane = [&](int sorted_lane) -> const T* {     // per-lane source index
         const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(sorted_lane << 2, rp_lo));
         const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(sorted_lane << 2, rp_hi));
-        return reinterpret_cast<const float*>((static_cast<unsigned long long>(hi) << 32) | lo);
+        return reinterpret_cast<const T*>((static_cast<unsigned long long>(hi) << 32) | lo);
     };
-    auto row_of = [&](int sorted_lane) -> const float* {          // wave-uniform source index
+    auto row_of = [&](int sorted_lane) -> const T* {          // wave-uniform source index
         const unsigned lo = static_cast<unsigned>(lane_read(rp_lo, sorted_lane));
         const unsigned hi = static_cast<unsigned>(lane_read(rp_hi, sorted_lane));
-        return reinterpret_cast<const float*>((static_cast<unsigned long long>(hi) << 32) | lo);
+        return reinterpret_cast<const T*>((static_cast<unsigned long long>(hi) << 32) | lo);
     };
     const int logW = n <= 16 ? 4 : n <= 32 ? 5 : 6;
     const int W = 1 << logW, G = 64 >> logW;
     const int grp = lane >> logW, jl = lane & (W - 1);
     const unsigned long long sub_mask = low_bits(W) << ((grp * W) & 63);
     const unsigned long long ltg_mask = lt_mask & sub_mask;
-    const float inv_rc_A = 1.0f / kA_Rc_f;
     // type of a sorted lane from the type boundaries
     const int tb1 = tbase[1], tb2 = tbase[2], tb3 = tbase[3];
     auto type_of = [&](int sorted_lane) { return (sorted_lane >= tb1) + (sorted_lane >= tb2) + (sorted_lane >= tb3); };
     wave_lds_fence();
-    const float4 aj = S.atom[jl];      // the partner this lane tests in every scan step
+    const vec4 aj = S.atom[jl];      // the partner this lane tests in every scan step
 
     // ------------------------------------------------------------ order of the centres
     // Angular partner count of every atom, then centres in order of decreasing count: a batch of
@@ -128,9 +132,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
         int m_mine = 0;
         for (int s0 = 0; s0 < n; s0 += G) {
             const int i = s0 + grp;
-            const float4 ai = S.atom[min(i, 63)];
-            const float dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
-            const float r = sqrtf(dx * dx + dy * dy + dz * dz);
+            const vec4 ai = S.atom[min(i, 63)];
+            const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
+            const T r = sqrt(dx * dx + dy * dy + dz * dz);
             const bool inA = (i < n) && (jl < n) && (jl != i) && (r < kA_Rc_f);
             const int cnt = popc64(wave_ballot(inA) & sub_mask);          // in every lane of the group
             const int got = __builtin_amdgcn_ds_bpermute((((lane - s0) << logW) & 63) << 2, cnt);
@@ -174,18 +178,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
         unsigned overflow = 0;
 
         // ---- fetch the angular upstream blocks of the batch's rows (80 x 16 bytes per row)
-        v4f st0[kB], st1[kB];
-#pragma unroll
-        for (int b = 0; b < kB; ++b) {
-            st0[b] = v4f{0.f, 0.f, 0.f, 0.f};
-            st1[b] = v4f{0.f, 0.f, 0.f, 0.f};
-            if (b < nb) {
-                const global_v4f_ptr rowp = (global_v4f_ptr)(row_of(lane_read(cord, min(c0 + b, 63))) + kRadial);
-                st0[b] = rowp[lane];
-                if (lane < 16) st1[b] = rowp[64 + lane];
-            }
-        }
-        S.pool.facc[lane] = make_float4(0.f, 0.f, 0.f, 0.f);
+        RowStage<T> stage;
+        stage.fetch(lane, nb, [&](int b) { return row_of(lane_read(cord, min(c0 + b, 63))); });
+        S.pool.facc[lane] = Fast<T>::make4(T(0), T(0), T(0), T(0));
         if (lane < 8) S.nM[lane] = 0;
         wave_lds_fence();
 
@@ -197,22 +192,22 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
             const int i = __builtin_amdgcn_ds_bpermute(min(c0 + cb, 63) << 2, cord);
             const int base = sel6(cb, pf[0], pf[1], pf[2], pf[3], pf[4], pf[5]);
             const int room = sel6(cb, pf[1], pf[2], pf[3], pf[4], pf[5], pf[6]) - base;
-            const float4 ai = S.atom[i];
-            const float dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
-            const float r = sqrtf(dx * dx + dy * dy + dz * dz);
+            const vec4 ai = S.atom[i];
+            const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
+            const T r = sqrt(dx * dx + dy * dy + dz * dz);
             const bool valid = centre_ok && (jl < n) && (jl != i);
             const bool inR = valid && (r < kR_Rc_f);
             const bool inA = valid && (r < kA_Rc_f);
             const unsigned long long mA = wave_ballot(inA);
             const int cntA = popc64(mA & sub_mask);
             const bool fits = cntA == room;       // the list has the length the first sweep counted
-            const float inv = __builtin_amdgcn_rcpf(r);
+            const T inv = Fast<T>::rcp(r);
             if (inA && fits) {
                 const int pos = base + popc64(mA & ltg_mask);
-                float fc, dfc;
-                cutoff_poly_grad(r * inv_rc_A, inv_rc_A, fc, dfc);
-                S.pool.nbr[pos] = make_float4(dx * inv, dy * inv, dz * inv, r);
-                S.pool.nbr_fc[pos] = make_float2(fc, dfc);
+                T fc, dfc;
+                Fast<T>::cutoff_grad(r, static_cast<T>(kA_Rc_f), fc, dfc);
+                S.pool.nbr[pos] = Fast<T>::make4(dx * inv, dy * inv, dz * inv, r);
+                S.pool.nbr_fc[pos] = Fast<T>::make2(fc, dfc);
                 S.pool.nbr_idx[pos] = static_cast<unsigned char>(jl);
             }
             if (jl == 0 && centre_ok) S.nM[b] = fits ? cntA : 0;
@@ -223,11 +218,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
             }
 
             // ---- radial pairs: this lane's (centre, partner) pair over its 16 shells
-            const float* grow = row_of_lane(i);
-            float cfx = 0.f, cfy = 0.f, cfz = 0.f;       // this pair's pull on the centre
+            const T* grow = row_of_lane(i);
+            T cfx = T(0), cfy = T(0), cfz = T(0);       // this pair's pull on the centre
             const bool do_rad = inR && fits;              // a centre that does not fit is redone as a whole
             if (do_rad) {
-                const float sc = bwd_radial_pair(grow, __float_as_int(aj.w), r, inv);   // dE/dr / r, multiplies (x_i - x_j)
+                const T sc = bwd_radial_pair<T>(grow, static_cast<int>(aj.w), r, inv);   // dE/dr / r, multiplies (x_i - x_j)
                 cfx = sc * dx;
                 cfy = sc * dy;
                 cfz = sc * dz;
@@ -252,7 +247,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
         }
 
         // ---- the fetched upstream blocks go to LDS
-        bwd_stage_blocks(S.pool, lane, nb, st0, st1);
+        stage.store(S.pool, lane, nb);
         wave_lds_fence();
 
         // ------------------------------------------------ angular: lane = list entry (centre, partner j)
@@ -264,7 +259,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
             const int pb = sel6(bs, pf[0], pf[1], pf[2], pf[3], pf[4], pf[5]);
             const int m = sel6(bs, m03.x, m03.y, m03.z, m03.w, m47.x, m47.y);   // 0 for a centre that did not fit
             const bool live = (lane < total) && (m > 0);
-            const float4 f = bwd_angular_rounds(S.pool, lane, live, bs, pb, m, type_of);
+            const vec4 f = bwd_angular_rounds<T>(S.pool, lane, live, bs, pb, m, type_of);
             const int self = live ? lane : 0;
             // -------------------------------------------- gather: partners get their slot, the centre minus the sum
             const int atom = S.pool.nbr_idx[self];
@@ -276,9 +271,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
                     S.force[1][atom] += f.y;
                     S.force[2][atom] += f.z;
                 }
-                const float sx = group_sum_to_last_lane(mine ? f.x : 0.f, 6);
-                const float sy = group_sum_to_last_lane(mine ? f.y : 0.f, 6);
-                const float sz = group_sum_to_last_lane(mine ? f.z : 0.f, 6);
+                const T sx = group_sum_to_last_lane(mine ? f.x : T(0), 6);
+                const T sy = group_sum_to_last_lane(mine ? f.y : T(0), 6);
+                const T sz = group_sum_to_last_lane(mine ? f.z : T(0), 6);
                 if (lane == 63) {
                     const int i_b = lane_read(cord, min(c0 + bb, 63));
                     S.force[0][i_b] -= sx;
@@ -295,8 +290,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
                 if (overflow & (1u << b)) {
                     const int i_b = lane_read(cord, min(c0 + b, 63));
                     const int i_orig = lane_read(orig, i_b);
-                    bwd_center_generic<float>(L, lane, X, Y, Z, A, off, n, i_orig, S.pool.gst, row_of(i_b),
-                                              [&](int atom, float fx, float fy, float fz) {
+                    bwd_center_generic<T>(L, lane, X, Y, Z, A, off, n, i_orig, S.pool.gst, row_of(i_b),
+                                              [&](int atom, T fx, T fy, T fz) {
                                                   const int sl = S.inv[atom];
                                                   atomicAdd(&S.force[0][sl], fx);
                                                   atomicAdd(&S.force[1][sl], fy);
@@ -319,14 +314,17 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
 
 }  // namespace
 
-hipError_t launch_bwd_small_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
-                                const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
-                                const int32_t* SIs, Buckets<const float> g, float* gX, float* gY,
-                                float* gZ, hipStream_t stream)
+template <typename T>
+hipError_t launch_bwd_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
+                            const int32_t* MACs, int32_t n_mols, const int32_t* SIs, Buckets<const T> g,
+                            T* gX, T* gY, T* gZ, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
-    aev_bwd_small_kernel<<<dim3(static_cast<unsigned>(n_mols)), dim3(64), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ);
+    aev_bwd_small_kernel<T><<<dim3(static_cast<unsigned>(n_mols)), dim3(64), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ);
     return hipGetLastError();
 }
+
+template hipError_t launch_bwd_small<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const float>, float*, float*, float*, hipStream_t);
+template hipError_t launch_bwd_small<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const double>, double*, double*, double*, hipStream_t);
 
 }  // namespace khan

@@ -30,6 +30,21 @@ __device__ __forceinline__ float lane_push(int dest_lane, float v)   // the valu
 }
 __device__ __forceinline__ int lane_push(int dest_lane, int v) { return __builtin_amdgcn_ds_permute(dest_lane << 2, v); }
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+// 64-bit values travel as two 32-bit halves
+__device__ __forceinline__ double lane_read(double v, int src_lane)
+{
+    const long long b = __double_as_longlong(v);
+    const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(b), src_lane));
+    const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(b >> 32), src_lane));
+    return __longlong_as_double(static_cast<long long>((static_cast<unsigned long long>(hi) << 32) | lo));
+}
+__device__ __forceinline__ double lane_push(int dest_lane, double v)
+{
+    const long long b = __double_as_longlong(v);
+    const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_ds_permute(dest_lane << 2, static_cast<int>(b)));
+    const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_ds_permute(dest_lane << 2, static_cast<int>(b >> 32)));
+    return __longlong_as_double(static_cast<long long>((static_cast<unsigned long long>(hi) << 32) | lo));
+}
 
 // Row pointers are rebuilt from two 32-bit lane reads; storing through an explicit global-address-space
 // pointer keeps the stores on the global (not the flat) path.
@@ -38,12 +53,28 @@ __device__ __forceinline__ void store_global(float* p, float v)
 {
     *((global_float*)(p)) = v;
 }
+typedef double __attribute__((address_space(1))) global_double;
+__device__ __forceinline__ void store_global(double* p, double v)
+{
+    *((global_double*)(p)) = v;
+}
 // sum of the two half-waves, in every lane: swap the upper half of one copy with the lower half of
 // the other (one cross-lane VALU move, no LDS round trip), then add
 __device__ __forceinline__ float half_wave_sum(float v)
 {
     const auto r = __builtin_amdgcn_permlane32_swap(__float_as_int(v), __float_as_int(v), false, false);
     return __int_as_float(r[0]) + __int_as_float(r[1]);
+}
+
+__device__ __forceinline__ double half_wave_sum(double v)
+{
+    const long long b = __double_as_longlong(v);
+    const int lo = static_cast<int>(b), hi = static_cast<int>(b >> 32);
+    const auto rl = __builtin_amdgcn_permlane32_swap(lo, lo, false, false);
+    const auto rh = __builtin_amdgcn_permlane32_swap(hi, hi, false, false);
+    const double a0 = __longlong_as_double(static_cast<long long>((static_cast<unsigned long long>(static_cast<unsigned>(rh[0])) << 32) | static_cast<unsigned>(rl[0])));
+    const double a1 = __longlong_as_double(static_cast<long long>((static_cast<unsigned long long>(static_cast<unsigned>(rh[1])) << 32) | static_cast<unsigned>(rl[1])));
+    return a0 + a1;
 }
 
 // Inclusive add-scan across the 64 lanes with data-parallel-primitive moves: four shifts inside each
@@ -83,6 +114,24 @@ __device__ __forceinline__ float dpp_take_f(float v)
 {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, kRowMask, 0xf, false));
 }
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ double dpp_take_f(double v)
+{
+    const long long b = __double_as_longlong(v);
+    const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(b), kCtrl, kRowMask, 0xf, false));
+    const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(b >> 32), kCtrl, kRowMask, 0xf, false));
+    return __longlong_as_double(static_cast<long long>((static_cast<unsigned long long>(hi) << 32) | lo));
+}
+__device__ __forceinline__ double group_sum_to_last_lane(double v, int log_group)
+{
+    v += dpp_take_f<0x111, 0xf>(v);
+    v += dpp_take_f<0x112, 0xf>(v);
+    v += dpp_take_f<0x114, 0xf>(v);
+    v += dpp_take_f<0x118, 0xf>(v);
+    if (log_group >= 5) v += dpp_take_f<0x142, 0xa>(v);
+    if (log_group >= 6) v += dpp_take_f<0x143, 0xc>(v);
+    return v;
+}
 __device__ __forceinline__ float group_sum_to_last_lane(float v, int log_group)
 {
     v += dpp_take_f<0x111, 0xf>(v);
@@ -94,9 +143,10 @@ __device__ __forceinline__ float group_sum_to_last_lane(float v, int log_group)
     return v;
 }
 
-__device__ __forceinline__ float pow8(float b)
+template <typename T>
+__device__ __forceinline__ T pow8(T b)
 {
-    const float b2 = b * b, b4 = b2 * b2;
+    const T b2 = b * b, b4 = b2 * b2;
     return b4 * b4;
 }
 __device__ __forceinline__ int sel4(int a, int v0, int v1, int v2, int v3)
@@ -143,5 +193,41 @@ __device__ __forceinline__ void cutoff_poly_grad(float u, float inv_rc, float& f
     fc = (u <= 0.5f) ? cs * cs : sn * sn;
     dfc_dr = -3.14159265358979323846f * inv_rc * sn * cs;
 }
+
+// Arithmetic of the one-wavefront kernels per precision.  float: hardware approximations (v_exp_f32,
+// v_rcp_f32, v_sqrt_f32, minimax cutoff), good to a few 1e-7 relative; double: correctly rounded library
+// routines, as the 1e-12 tolerance of the double-precision path needs.
+template <typename T> struct Fast;
+template <> struct Fast<float> {
+    typedef float4 vec4;
+    typedef float2 vec2;
+    static __device__ __forceinline__ float4 make4(float a, float b, float c, float d) { return make_float4(a, b, c, d); }
+    static __device__ __forceinline__ float2 make2(float a, float b) { return make_float2(a, b); }
+    static __device__ __forceinline__ float sqrt_(float x) { return __builtin_amdgcn_sqrtf(x); }
+    static __device__ __forceinline__ float rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+    // exp(-eta d^2)
+    static __device__ __forceinline__ float gauss(float eta, float d) { return __builtin_amdgcn_exp2f((-eta * 1.44269504088896340736f) * d * d); }
+    static __device__ __forceinline__ float cutoff(float r, float rc) { return cutoff_poly(r * (1.0f / rc)); }
+    static __device__ __forceinline__ void cutoff_grad(float r, float rc, float& fc, float& dfc)
+    {
+        cutoff_poly_grad(r * (1.0f / rc), 1.0f / rc, fc, dfc);
+    }
+};
+template <> struct Fast<double> {
+    typedef double4 vec4;
+    typedef double2 vec2;
+    static __device__ __forceinline__ double4 make4(double a, double b, double c, double d) { return make_double4(a, b, c, d); }
+    static __device__ __forceinline__ double2 make2(double a, double b) { return make_double2(a, b); }
+    static __device__ __forceinline__ double sqrt_(double x) { return sqrt(x); }
+    static __device__ __forceinline__ double rcp(double x) { return 1.0 / x; }
+    static __device__ __forceinline__ double gauss(double eta, double d) { return exp(-eta * d * d); }
+    static __device__ __forceinline__ double cutoff(double r, double rc) { return 0.5 * cos(kPi / rc * r) + 0.5; }
+    static __device__ __forceinline__ void cutoff_grad(double r, double rc, double& fc, double& dfc)
+    {
+        const double w = kPi / rc;
+        fc = 0.5 * cos(w * r) + 0.5;
+        dfc = -0.5 * w * sin(w * r);
+    }
+};
 
 }  // namespace khan

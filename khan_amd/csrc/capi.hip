@@ -37,7 +37,7 @@ int forward_dispatch(const float* xs, const float* ys, const float* zs, const in
     if (force_generic())
         return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, stream));
     // molecules of up to 64 atoms: one wavefront each; up to 256: one workgroup each; the rest: general kernel
-    int st = hip_status(khan::launch_fwd_small_f32(xs, ys, zs, as, mos, macs, n_mols, sis, out, stream));
+    int st = hip_status(khan::launch_fwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, stream));
     if (st != KHAN_OK) return st;
     st = hip_status(khan::launch_fwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, out, stream));
     if (st != KHAN_OK) return st;
@@ -49,7 +49,12 @@ int forward_dispatch(const double* xs, const double* ys, const double* zs, const
                      const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
                      khan::Buckets<double> out, hipStream_t stream)
 {
-    return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, stream));
+    if (force_generic())
+        return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, stream));
+    int st = hip_status(khan::launch_fwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, stream));
+    if (st != KHAN_OK) return st;
+    return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
+                                                       khan::kSmallMaxAtoms + 1, stream));
 }
 
 int backward_dispatch(const float* xs, const float* ys, const float* zs, const int32_t* as,
@@ -67,7 +72,7 @@ int backward_dispatch(const float* xs, const float* ys, const float* zs, const i
     if (st != KHAN_OK) return st;
     st = hip_status(khan::launch_bwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, stream));
     if (st != KHAN_OK) return st;
-    return hip_status(khan::launch_bwd_small_f32(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, stream));
+    return hip_status(khan::launch_bwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, stream));
 }
 
 int backward_dispatch(const double* xs, const double* ys, const double* zs, const int32_t* as,
@@ -75,8 +80,13 @@ int backward_dispatch(const double* xs, const double* ys, const double* zs, cons
                       khan::Buckets<const double> g, double* gx, double* gy, double* gz, int64_t n_atoms,
                       hipStream_t stream)
 {
-    return hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                       n_atoms, 0, stream));
+    if (force_generic())
+        return hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                           n_atoms, 0, stream));
+    int st = hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                         n_atoms, khan::kSmallMaxAtoms + 1, stream));
+    if (st != KHAN_OK) return st;
+    return hip_status(khan::launch_bwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, stream));
 }
 
 template <typename T>

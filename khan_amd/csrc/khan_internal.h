@@ -24,11 +24,12 @@ hipError_t launch_jvp_generic(const T* X, const T* Y, const T* Z, const int32_t*
                               const int32_t* SIs, const T* VX, const T* VY, const T* VZ, Buckets<T> out,
                               int min_atoms, hipStream_t stream);
 
-// ---- AEV forward for molecules of up to 64 atoms, float32 (larger molecules are skipped) ----
+// ---- AEV forward for molecules of up to 64 atoms (larger molecules are skipped) ----
 constexpr int kSmallMaxAtoms = 64;
-hipError_t launch_fwd_small_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
-                                const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
-                                const int32_t* SIs, Buckets<float> out, hipStream_t stream);
+template <typename T>
+hipError_t launch_fwd_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
+                            const int32_t* MACs, int32_t n_mols, const int32_t* SIs, Buckets<T> out,
+                            hipStream_t stream);
 
 // ---- AEV forward for molecules of 65 to 256 atoms, float32 (other sizes are skipped) ----
 constexpr int kMediumMaxAtoms = 256;
@@ -46,10 +47,10 @@ hipError_t launch_bwd_generic(const T* X, const T* Y, const T* Z, const int32_t*
                               const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
                               const int32_t* SIs, Buckets<const T> g, T* gX, T* gY, T* gZ,
                               int64_t n_atoms, int min_atoms, hipStream_t stream);
-hipError_t launch_bwd_small_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
-                                const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
-                                const int32_t* SIs, Buckets<const float> g, float* gX, float* gY,
-                                float* gZ, hipStream_t stream);
+template <typename T>
+hipError_t launch_bwd_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
+                            const int32_t* MACs, int32_t n_mols, const int32_t* SIs, Buckets<const T> g,
+                            T* gX, T* gY, T* gZ, hipStream_t stream);
 
 // ---- integer path ----
 hipError_t launch_mol_offsets(const int32_t* mol_idxs, int64_t n_atoms, int32_t n_mols,
