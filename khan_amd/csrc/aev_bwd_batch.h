@@ -75,7 +75,7 @@ template <typename T> struct RowStage {
                 const global_v4f_ptr rowp = (global_v4f_ptr)(row_of(b) + kRadial);
 #pragma unroll
                 for (int r = 0; r < kPieceRegs; ++r)
-                    if (r * 64 + lane < kRowPieces) st[b][r] = rowp[r * 64 + lane];
+                    if ((r + 1) * 64 <= kRowPieces || r * 64 + lane < kRowPieces) st[b][r] = rowp[r * 64 + lane];
             }
         }
     }
@@ -89,7 +89,7 @@ template <typename T> struct RowStage {
                 for (int r = 0; r < kPieceRegs; ++r) {
                     const int piece = r * 64 + lane;
                     const int elem = piece * kPerPiece;
-                    if (piece < kRowPieces)
+                    if ((r + 1) * 64 <= kRowPieces || piece < kRowPieces)
                         *reinterpret_cast<v4f*>(&pool.gst[b * kNumPairBlocks * kBlockStride + (elem >> 5) * kBlockStride + (elem & 31)]) = st[b][r];
                 }
             }
