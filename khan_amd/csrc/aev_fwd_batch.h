@@ -53,7 +53,7 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T>& S, const LaneCo
         const int oa = sel4(seg_a, 0, nn.x, nn.x + nn.y, nn.x + nn.y + nn.z);
         const int ob = sel4(seg_bt, 0, nn.x, nn.x + nn.y, nn.x + nn.y + nn.z);
         const bool same = seg_a == seg_bt;
-        cnt = same ? (na * (na - 1)) / 2 : na * nbt;
+        cnt = same ? (__mul24(na, na - 1) >> 1) : __mul24(na, nbt);
         packed = seg_b | (oa << 3) | (ob << 9) | (na << 15) | (same ? (1 << 21) : 0) | (seg_pt << 22);
     }
     const int padded = (cnt + 1) & ~1;
@@ -99,16 +99,17 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T>& S, const LaneCo
         // decode q -> (j,k) inside the centre's type-sorted list
         int bsel = d.packed & 7;
         const int oa = (d.packed >> 3) & 63, ob = (d.packed >> 9) & 63, na = (d.packed >> 15) & 63;
-        int kl, jl2;
-        if ((d.packed >> 21) & 1) {                     // same type: pairs jl < kl, kl-major
-            kl = static_cast<int>((1.0f + __builtin_amdgcn_sqrtf(8.0f * static_cast<float>(q) + 1.0f)) * 0.5f);
-            if ((kl * (kl - 1)) / 2 > q) --kl;
-            if (((kl + 1) * kl) / 2 <= q) ++kl;
-            jl2 = q - (kl * (kl - 1)) / 2;
-        } else {                                        // q = kl * n_a + jl
-            kl = static_cast<int>((static_cast<float>(q) + 0.5f) * __builtin_amdgcn_rcpf(static_cast<float>(na)));
-            jl2 = q - kl * na;
-        }
+        // both numberings are decoded and one is selected (no divergent branch).  Same type: pairs jl < kl,
+        // kl-major, q = kl (kl - 1) / 2 + jl; kl = floor((1 + sqrt(8 q + 1)) / 2) is computed with 1.5 under
+        // the root, which keeps the (approximate) hardware square root on the right side of every row
+        // start for q up to several thousand.  Different types: q = kl * n_a + jl.
+        const float qf = static_cast<float>(q);
+        const unsigned kt = static_cast<unsigned>((1.0f + __builtin_amdgcn_sqrtf(fmaf(8.0f, qf, 1.5f))) * 0.5f);
+        const unsigned jt = static_cast<unsigned>(q) - (__umul24(kt, kt - 1u) >> 1);
+        const unsigned kr = static_cast<unsigned>((qf + 0.5f) * __builtin_amdgcn_rcpf(static_cast<float>(na)));
+        const unsigned jr = static_cast<unsigned>(q) - __umul24(kr, static_cast<unsigned>(na));
+        const bool tri = (d.packed >> 21) & 1;
+        const int kl = static_cast<int>(tri ? kt : kr), jl2 = static_cast<int>(tri ? jt : jr);
         int j = oa + jl2, k = ob + kl;
         if (!ok) {
             j = 0;
