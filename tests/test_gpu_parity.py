@@ -694,3 +694,55 @@ def test_gradient_against_central_differences_on_64_molecules(ops):
         say("   direction %d: numeric %.9e  f64 %.9e  f32 %.9e" % (trial, num, ana64, ana32))
         assert abs(num - ana64) <= 1e-6 * scale      # truncation of the difference quotient, O(h^2)
         assert abs(ana32 - ana64) <= 1e-5 * scale
+
+
+# ----------------------------------------------------------------------------- HIP graph capture
+def test_forward_backward_replay_from_a_hip_graph(ops):
+    # featurize + featurize_grad launch only kernels on the caller's stream (no allocation, no memset node,
+    # no host synchronisation), so they can be captured once and replayed; every replay is checked against
+    # the eager result, with eager work and synchronisations in between
+    say("case: HIP graph capture and replay of forward + backward")
+    b = datagen.make_batch("organic", 512, first_mol=900)
+    big = datagen.make_batch("boxes", 2)               # brings the medium-molecule kernels into the graph
+    X = np.concatenate([b.X, big.X]); Y = np.concatenate([b.Y, big.Y]); Z = np.concatenate([b.Z, big.Z])
+    A = np.concatenate([b.A, big.A])
+    mi = np.concatenate([b.mol_idxs, big.mol_idxs + b.n_mols]).astype(np.int32)
+    c = Case(X, Y, Z, A, mi, b.n_mols + big.n_mols)
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+    acs = ac.cpu().tolist()
+    Xd, Yd, Zd, Ad = dev(c.X), dev(c.Y), dev(c.Z), dev(c.A)
+    gen = torch.Generator(device="cuda:0")
+    gen.manual_seed(3)
+    up = torch.randn(c.N * 384, device="cuda:0", generator=gen)
+    gb, start = [], 0
+    for k in acs:
+        gb.append(up[start * 384:(start + k) * 384])
+        start += k
+    feats = torch.cat(ops.featurize(Xd, Yd, Zd, Ad, mos, macs, sc, acs)).clone()
+    grads = torch.stack(ops.featurize_grad(Xd, Yd, Zd, Ad, mos, macs, sc, acs, *gb)).clone()
+    torch.cuda.synchronize()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                      # warm-up on the capture stream
+        ops.featurize(Xd, Yd, Zd, Ad, mos, macs, sc, acs)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        f_out = ops.featurize(Xd, Yd, Zd, Ad, mos, macs, sc, acs)
+        g_out = ops.featurize_grad(Xd, Yd, Zd, Ad, mos, macs, sc, acs, *gb)
+    f_cat = lambda: torch.cat(f_out)
+    for replay in range(4):
+        for t in f_out:
+            t.fill_(-1.0)                              # eager work between replays
+        for t in g_out:
+            t.fill_(-1.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(f_cat(), feats), "replay %d: features differ" % replay
+        got = torch.stack(list(g_out))
+        # molecules above 64 atoms add forces with atomics: the last bits depend on the order
+        assert torch.allclose(got, grads, rtol=1e-5, atol=1e-5), "replay %d: gradients differ" % replay
+        small = torch.from_numpy(c.mol_idxs < b.n_mols).to("cuda:0")
+        assert torch.equal(got[:, small], grads[:, small])
