@@ -7,7 +7,18 @@
 namespace khan {
 
 // LDS working set of one wavefront
-template <typename T>
+// what the Jacobian-vector variant keeps on top of the forward working set
+template <typename T, bool kJvp> struct FwdJvpLds {};
+template <typename T> struct __align__(16) FwdJvpLds<T, true> {
+    typename Fast<T>::vec4 vel[64];               // the incoming vector of every atom (sorted order)
+    typename Fast<T>::vec4 nbr_p[kB][kCapA];      // (v_centre - v_partner)/r, and its component along the unit vector
+    typename Fast<T>::vec2 nbr_d[kB][kCapA];      // f_C'(r) dr, and dr = change of the distance along the vectors
+    typename Fast<T>::vec2 rad_ab[64];            // radial entries: f_C' dr, and -2 eta f_C dr
+    T rec2[64][12];                               // phase-1 records: dA_0..7, H_0..3
+};
+
+// LDS working set of one wavefront
+template <typename T, bool kJvp = false>
 struct __align__(16) FwdWaveLds {
     typename Fast<T>::vec4 atom[64];          // x, y, z, type (sorted order)
     typename Fast<T>::vec4 nbr[kB][kCapA];    // unit vector (centre minus partner)/r, and r
@@ -18,16 +29,20 @@ struct __align__(16) FwdWaveLds {
     unsigned bits[kBitWords];                 // bit per triple slot: a segment starts here
     int nA[kB][4];                            // angular partners per type, per centre of the batch
     int nR[4][4];                             // radial partners per type, per group of the scan step
+    FwdJvpLds<T, kJvp> jvp;
 };
 
 // Segment table, phases 1 and 2 and the zero fill of empty blocks for centres 0..nb-1 of a batch.
 // `row_of_centre(b)` returns the address of centre b's 384-float output row; it is called by all
 // lanes together, with a per-lane b for the segment table and a wave-uniform b for the zero fill.
-template <typename T, typename RowOfCentre>
-__device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T>& S, const LaneConsts<T>& L, int lane, int nb,
+// With kJvp the same sums are formed for the derivative of every term along the atoms' incoming vectors:
+// d(A_t G_s P) = dA_t (G_s P) + A_t (dG_s P + G_s dP), two products per record instead of one.
+template <typename T, bool kJvp, typename RowOfCentre>
+__device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const LaneConsts<T>& L, int lane, int nb,
                                                   RowOfCentre row_of_centre)
 {
     typedef typename Fast<T>::vec4 vec4;
+    typedef typename Fast<T>::vec2 vec2;
     const unsigned long long lane_bit = 1ull << lane;
     const unsigned long long lt_mask = lane_bit - 1ull;
     // segment-table lanes: lane = centre-in-batch * 10 + type-pair index (HH HC HN HO CC CN CO NN NO OO)
@@ -125,19 +140,46 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T>& S, const LaneCo
         const T cy = vj.z * vk.x - vj.x * vk.z;
         const T cz = vj.x * vk.y - vj.y * vk.x;
         const T s = Fast<T>::sqrt_(cx * cx + cy * cy + cz * cz);
-        T Af[8];
+        T Af[8], dAf[8];
+        T dc = T(0), cot = T(0);
+        if constexpr (kJvp) {
+            // d cos = u_k.p_j + u_j.p_k - c (alpha_j + alpha_k), p = (v_i - v_partner)/r, alpha = u.p
+            const vec4 pj = S.jvp.nbr_p[bsel][j], pk = S.jvp.nbr_p[bsel][k];
+            dc = (vk.x * pj.x + vk.y * pj.y + vk.z * pj.z) + (vj.x * pk.x + vj.y * pk.y + vj.z * pk.z) - c * (pj.w + pk.w);
+            cot = c * s * Fast<T>::rcp(s * s + Real<T>::kCotEps);     // c/s, zero on the line (cusp of the angle)
+        }
 #pragma unroll
-        for (int t = 0; t < 8; ++t)
-            Af[t] = pow8(fma(s, static_cast<T>(kSinTheta[t]), fma(c, static_cast<T>(kCosTheta[t]), T(1))));
+        for (int t = 0; t < 8; ++t) {
+            const T ct = static_cast<T>(kCosTheta[t]), st = static_cast<T>(kSinTheta[t]);
+            const T base = fma(s, st, fma(c, ct, T(1)));
+            if constexpr (kJvp) {
+                const T b2 = base * base, b4 = b2 * b2;
+                const T Am1 = b4 * b2 * base;
+                Af[t] = Am1 * base;
+                dAf[t] = T(8) * Am1 * fma(-cot, st, ct) * dc;
+            } else {
+                Af[t] = pow8(base);
+                dAf[t] = T(0);
+            }
+        }
         const T rho = T(0.5) * (vj.w + vk.w);
         const T P = T(0.0078125) * fj * fk;
-        T Gf[4];
+        T Gf[4], Hf[4];
+        T dP = T(0), drho = T(0);
+        if constexpr (kJvp) {
+            const vec2 dj = S.jvp.nbr_d[bsel][j], dk = S.jvp.nbr_d[bsel][k];
+            dP = T(0.0078125) * (dj.x * fk + fj * dk.x);
+            drho = T(0.5) * (dj.y + dk.y);
+        }
 #pragma unroll
         for (int sidx = 0; sidx < 4; ++sidx) {
             const T dd = rho - static_cast<T>(kA_Rs_f[sidx]);
+            const T g = Fast<T>::gauss(static_cast<T>(kA_eta_f), dd);
             // padding slots read whatever sits in the list: select, do not multiply, so that a
             // stray NaN cannot reach the sums
-            Gf[sidx] = ok ? Fast<T>::gauss(static_cast<T>(kA_eta_f), dd) * P : T(0);
+            Gf[sidx] = ok ? g * P : T(0);
+            if constexpr (kJvp) Hf[sidx] = ok ? g * fma(T(-2) * static_cast<T>(kA_eta_f) * dd * drho, P, dP) : T(0);
+            else Hf[sidx] = T(0);
         }
 #pragma unroll
         for (int t = 0; t < 8; ++t) Af[t] = ok ? Af[t] : T(0);
@@ -145,6 +187,14 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T>& S, const LaneCo
         recp[0] = Fast<T>::make4(Af[0], Af[1], Af[2], Af[3]);
         recp[1] = Fast<T>::make4(Af[4], Af[5], Af[6], Af[7]);
         recp[2] = Fast<T>::make4(Gf[0], Gf[1], Gf[2], Gf[3]);
+        if constexpr (kJvp) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) dAf[t] = ok ? dAf[t] : T(0);
+            vec4* rec2p = reinterpret_cast<vec4*>(S.jvp.rec2[lane]);
+            rec2p[0] = Fast<T>::make4(dAf[0], dAf[1], dAf[2], dAf[3]);
+            rec2p[1] = Fast<T>::make4(dAf[4], dAf[5], dAf[6], dAf[7]);
+            rec2p[2] = Fast<T>::make4(Hf[0], Hf[1], Hf[2], Hf[3]);
+        }
         wave_lds_fence();
 
         // phase 2: lane = (half, theta_t, Rs_s); the halves take alternate records.  Records past
@@ -152,20 +202,33 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T>& S, const LaneCo
         const int npairs = min(64, total - base) >> 1;
         const T* pa = &S.rec[L.half][ang_t];
         const T* pg = &S.rec[L.half][8 + ang_s];
+        const T* pda = pa;
+        const T* ph = pg;
+        if constexpr (kJvp) {
+            pda = &S.jvp.rec2[L.half][ang_t];
+            ph = &S.jvp.rec2[L.half][8 + ang_s];
+        }
         unsigned long long mm = starts;
         if (base == 0) {            // the batch's first segment opens here; nothing to close
             cur_lo = static_cast<unsigned>(lane_read(static_cast<int>(d.row_lo), 0));
             cur_hi = static_cast<unsigned>(lane_read(static_cast<int>(d.row_hi), 0));
             mm &= ~1ull;
         }
-        auto load8 = [&](int q0, T (&av)[8], T (&gv)[8]) {
+        struct Group {
+            T a[8], g[8], da[kJvp ? 8 : 1], h[kJvp ? 8 : 1];
+        };
+        auto load8 = [&](int q0, Group& v) {
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
-                av[u] = pa[(q0 + u) * 24];
-                gv[u] = pg[(q0 + u) * 24];
+                v.a[u] = pa[(q0 + u) * 24];
+                v.g[u] = pg[(q0 + u) * 24];
+                if constexpr (kJvp) {
+                    v.da[u] = pda[(q0 + u) * 24];
+                    v.h[u] = ph[(q0 + u) * 24];
+                }
             }
         };
-        auto run8 = [&](int q0, const T (&av)[8], const T (&gv)[8]) {
+        auto run8 = [&](int q0, const Group& v) {
             const unsigned m16 = static_cast<unsigned>(mm) & 0xffffu;     // this group's 16 slots
             mm >>= 16;
 #pragma unroll
@@ -179,19 +242,20 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T>& S, const LaneCo
                     cur_hi = static_cast<unsigned>(lane_read(static_cast<int>(d.row_hi), first));
                     acc = T(0);
                 }
-                acc = fma(av[u], gv[u], acc);
+                if constexpr (kJvp) acc = fma(v.da[u], v.g[u], fma(v.a[u], v.h[u], acc));
+                else acc = fma(v.a[u], v.g[u], acc);
             }
         };
         // eight record pairs per group, the next group's LDS reads in flight while one is summed
-        T a0[8], g0[8], a1[8], g1[8];
-        load8(0, a0, g0);
+        Group v0, v1;
+        load8(0, v0);
         for (int q0 = 0; q0 < npairs; q0 += 16) {
             const bool more1 = q0 + 8 < npairs;
-            if (more1) load8(q0 + 8, a1, g1);
-            run8(q0, a0, g0);
+            if (more1) load8(q0 + 8, v1);
+            run8(q0, v0);
             if (more1) {
-                if (q0 + 16 < npairs) load8(q0 + 16, a0, g0);
-                run8(q0 + 8, a1, g1);
+                if (q0 + 16 < npairs) load8(q0 + 16, v0);
+                run8(q0 + 8, v1);
             }
         }
         wave_lds_fence();

@@ -110,7 +110,7 @@ __global__ __launch_bounds__(256) void aev_bwd_generic_kernel(
 // `min_atoms` are wanted, a small grid keeps the cost of skipping the others low.
 static unsigned generic_grid(int32_t n_mols, int min_atoms)
 {
-    const int32_t cap = min_atoms > 1 ? 2048 : (1 << 20);
+    const int32_t cap = min_atoms > 1 ? 16384 : (1 << 20);
     return static_cast<unsigned>(n_mols < cap ? n_mols : cap);
 }
 

@@ -28,17 +28,21 @@ namespace khan {
 namespace {
 
 // float: 4 wavefronts per SIMD (LDS 9.8 KB, <= 128 VGPRs); double: 2 (LDS 19.6 KB)
-template <typename T>
-__global__ __launch_bounds__(64 * kWavesPerBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 4 : 2, sizeof(T) == 4 ? 4 : 2)))
+// With kJvp the kernel computes the Jacobian-vector product instead (featurize_grad_inverse): every term of
+// the forward sums is replaced by its derivative along the per-atom vectors (VX, VY, VZ).
+// float: 4 wavefronts per SIMD (LDS 9.8 KB, <= 128 VGPRs); double or kJvp: 2 (LDS 19 KB); both: 1.
+template <typename T, bool kJvp>
+__global__ __launch_bounds__(64 * kWavesPerBlock)
+__attribute__((amdgpu_waves_per_eu((sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1), (sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1))))
 void aev_fwd_small_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
-    Buckets<T> out)
+    const T* __restrict__ VX, const T* __restrict__ VY, const T* __restrict__ VZ, Buckets<T> out)
 {
     typedef typename Fast<T>::vec4 vec4;
     typedef typename Fast<T>::vec2 vec2;
-    __shared__ FwdWaveLds<T> lds_all[kWavesPerBlock];
+    __shared__ FwdWaveLds<T, kJvp> lds_all[kWavesPerBlock];
     const int lane = threadIdx.x & 63;
     const int wave = uniform(threadIdx.x >> 6);
     const int mol = blockIdx.x * kWavesPerBlock + wave;
@@ -46,7 +50,7 @@ void aev_fwd_small_kernel(
     const int n = uniform(MACs[mol]);
     const int off = uniform(MOs[mol]);
     if (n <= 0 || n > 64) return;                 // larger molecules belong to the general kernel
-    FwdWaveLds<T>& S = lds_all[wave];
+    FwdWaveLds<T, kJvp>& S = lds_all[wave];
     const LaneConsts<T> L = lane_consts<T>(lane);
     const unsigned long long lane_bit = 1ull << lane;
     const unsigned long long lt_mask = lane_bit - 1ull;
@@ -62,6 +66,14 @@ void aev_fwd_small_kernel(
         z = Z[off + lane];
         type = fold_type(A[off + lane]);
         rowbits = reinterpret_cast<unsigned long long>(out.p[type] + static_cast<size_t>(SIs[off + lane]) * kFeats);
+    }
+    T vx = T(0), vy = T(0), vz = T(0);
+    if constexpr (kJvp) {
+        if (have) {
+            vx = VX[off + lane];
+            vy = VY[off + lane];
+            vz = VZ[off + lane];
+        }
     }
     int tcount[4], tbase[4];
     int dest = lane;    // lanes without an atom keep their place, so the map is a permutation
@@ -89,6 +101,12 @@ void aev_fwd_small_kernel(
     const int rp_lo = lane_push(dest, static_cast<int>(rowbits & 0xffffffffull));
     const int rp_hi = lane_push(dest, static_cast<int>(rowbits >> 32));
     S.atom[lane] = Fast<T>::make4(x, y, z, static_cast<T>(type));
+    if constexpr (kJvp) {
+        vx = lane_push(dest, vx);
+        vy = lane_push(dest, vy);
+        vz = lane_push(dest, vz);
+        S.jvp.vel[lane] = Fast<T>::make4(vx, vy, vz, T(0));
+    }
     auto row_of = [&](int sorted_lane) -> T* {     // sorted_lane is wave-uniform
         const unsigned lo = static_cast<unsigned>(lane_read(rp_lo, sorted_lane));
         const unsigned hi = static_cast<unsigned>(lane_read(rp_hi, sorted_lane));
@@ -138,12 +156,39 @@ void aev_fwd_small_kernel(
             const bool inA = valid && (r < kA_Rc_f);
             const unsigned long long mR = wave_ballot(inR), mA = wave_ballot(inA);
             const bool fits = popc64(mA & sub_mask) <= kCapA;
-            if (inR) S.rad[grp * W + popc64(mR & ltg_mask)] = Fast<T>::make2(r, Fast<T>::cutoff(r, static_cast<T>(kR_Rc_f)));
+            T wx = T(0), wy = T(0), wz = T(0), rd = T(0);        // v_centre - v_partner, and d r along it
+            const T inv = Fast<T>::rcp(r);
+            if constexpr (kJvp) {
+                const vec4 vi = S.jvp.vel[centre_ok ? i : 0], vjv = S.jvp.vel[jl];
+                wx = vi.x - vjv.x;
+                wy = vi.y - vjv.y;
+                wz = vi.z - vjv.z;
+                rd = (dx * wx + dy * wy + dz * wz) * inv;
+            }
+            if (inR) {
+                const int pos = grp * W + popc64(mR & ltg_mask);
+                if constexpr (kJvp) {
+                    T fc, dfc;
+                    Fast<T>::cutoff_grad(r, static_cast<T>(kR_Rc_f), fc, dfc);
+                    S.rad[pos] = Fast<T>::make2(r, fc);
+                    S.jvp.rad_ab[pos] = Fast<T>::make2(dfc * rd, T(-2) * static_cast<T>(kR_eta_f) * fc * rd);
+                } else {
+                    S.rad[pos] = Fast<T>::make2(r, Fast<T>::cutoff(r, static_cast<T>(kR_Rc_f)));
+                }
+            }
             if (inA && fits) {
                 const int pos = popc64(mA & ltg_mask);
-                const T inv = Fast<T>::rcp(r);
-                S.nbr[centre_ok ? b : 0][pos] = Fast<T>::make4(dx * inv, dy * inv, dz * inv, r);
-                S.nbr_fc[centre_ok ? b : 0][pos] = Fast<T>::cutoff(r, static_cast<T>(kA_Rc_f));
+                const int cb = centre_ok ? b : 0;
+                S.nbr[cb][pos] = Fast<T>::make4(dx * inv, dy * inv, dz * inv, r);
+                if constexpr (kJvp) {
+                    T fc, dfc;
+                    Fast<T>::cutoff_grad(r, static_cast<T>(kA_Rc_f), fc, dfc);
+                    S.nbr_fc[cb][pos] = fc;
+                    S.jvp.nbr_p[cb][pos] = Fast<T>::make4(wx * inv, wy * inv, wz * inv, rd * inv);
+                    S.jvp.nbr_d[cb][pos] = Fast<T>::make2(dfc * rd, rd);
+                } else {
+                    S.nbr_fc[cb][pos] = Fast<T>::cutoff(r, static_cast<T>(kA_Rc_f));
+                }
             }
             {   // bit b of `overflow`: centre b of the batch has too many angular partners
                 const unsigned long long ov = wave_ballot(!fits && jl == 0 && centre_ok);
@@ -180,13 +225,20 @@ void aev_fwd_small_kernel(
                     T acc_r = T(0);
                     for (int q0 = 0; q0 < mxR[a]; q0 += 4 * rg_ns) {
                         // four entries of this lane's slot per trip; slot s takes q = s, s+ns, s+2ns, ...
-                        vec2 e[4];
+                        vec2 e[4], ab[4];
 #pragma unroll
-                        for (int u = 0; u < 4; ++u) e[u] = list[min(obase + q0 + u * rg_ns + rg_s, W - 1)];
+                        for (int u = 0; u < 4; ++u) {
+                            const int at = min(obase + q0 + u * rg_ns + rg_s, W - 1);
+                            e[u] = list[at];
+                            if constexpr (kJvp) ab[u] = S.jvp.rad_ab[rg_g * W + at];
+                        }
 #pragma unroll
                         for (int u = 0; u < 4; ++u) {
                             const T dd = e[u].x - L.rrs;
-                            const T v = Fast<T>::gauss(static_cast<T>(kR_eta_f), dd) * e[u].y;
+                            // forward: exp(-eta d^2) f_C; derivative: exp(-eta d^2) (f_C' - 2 eta d f_C) dr
+                            T v = Fast<T>::gauss(static_cast<T>(kR_eta_f), dd);
+                            if constexpr (kJvp) v *= fma(ab[u].y, dd, ab[u].x);
+                            else v *= e[u].y;
                             acc_r += (q0 + u * rg_ns + rg_s < cnt_a) ? v : T(0);   // stale entries: select
                         }
                     }
@@ -200,7 +252,7 @@ void aev_fwd_small_kernel(
         }
 
         // ------------------------------------------------ segment table, phases 1 and 2, zero fill
-        fwd_angular_batch<T>(S, L, lane, nb, [&](int b) -> unsigned long long {
+        fwd_angular_batch<T, kJvp>(S, L, lane, nb, [&](int b) -> unsigned long long {
             const int cl = min(c0 + b, 63);
             const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(cl << 2, rp_lo));
             const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(cl << 2, rp_hi));
@@ -213,8 +265,12 @@ void aev_fwd_small_kernel(
             for (int b = 0; b < nb; ++b) {
                 if (overflow & (1u << b)) {
                     const int i_orig = lane_read(orig, c0 + b);
-                    fwd_center_generic<T>(L, lane, X, Y, Z, A, off, n, i_orig,
-                                          reinterpret_cast<T*>(S.rec), row_of(c0 + b));
+                    if constexpr (kJvp)
+                        jvp_center_generic<T>(L, lane, X, Y, Z, A, VX, VY, VZ, off, n, i_orig,
+                                              reinterpret_cast<T*>(S.rec), row_of(c0 + b));
+                    else
+                        fwd_center_generic<T>(L, lane, X, Y, Z, A, off, n, i_orig,
+                                              reinterpret_cast<T*>(S.rec), row_of(c0 + b));
                 }
             }
             wave_lds_fence();
@@ -231,11 +287,26 @@ hipError_t launch_fwd_small(const T* X, const T* Y, const T* Z, const int32_t* A
 {
     if (n_mols <= 0) return hipSuccess;
     const unsigned blocks = (static_cast<unsigned>(n_mols) + kWavesPerBlock - 1u) / kWavesPerBlock;
-    aev_fwd_small_kernel<T><<<dim3(blocks), dim3(64 * kWavesPerBlock), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, out);
+    aev_fwd_small_kernel<T, false><<<dim3(blocks), dim3(64 * kWavesPerBlock), 0, stream>>>(
+        X, Y, Z, A, MOs, MACs, n_mols, SIs, nullptr, nullptr, nullptr, out);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_jvp_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
+                            const int32_t* MACs, int32_t n_mols, const int32_t* SIs, const T* VX,
+                            const T* VY, const T* VZ, Buckets<T> out, hipStream_t stream)
+{
+    if (n_mols <= 0) return hipSuccess;
+    const unsigned blocks = (static_cast<unsigned>(n_mols) + kWavesPerBlock - 1u) / kWavesPerBlock;
+    aev_fwd_small_kernel<T, true><<<dim3(blocks), dim3(64 * kWavesPerBlock), 0, stream>>>(
+        X, Y, Z, A, MOs, MACs, n_mols, SIs, VX, VY, VZ, out);
     return hipGetLastError();
 }
 
 template hipError_t launch_fwd_small<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<float>, hipStream_t);
 template hipError_t launch_fwd_small<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<double>, hipStream_t);
+template hipError_t launch_jvp_small<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const float*, const float*, const float*, Buckets<float>, hipStream_t);
+template hipError_t launch_jvp_small<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const double*, const double*, const double*, Buckets<double>, hipStream_t);
 
 }  // namespace khan

@@ -140,9 +140,15 @@ int featurize_grad_inverse_impl(const T* xs, const T* ys, const T* zs, const int
     if ((acs_host[0] && !h) || (acs_host[1] && !c) || (acs_host[2] && !n) || (acs_host[3] && !o))
         return KHAN_ERR_INVALID_ARG;
     khan::Buckets<T> out{{h, c, n, o}};
-    // every molecule size and both precisions run on the general-shape kernel
-    return hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, 0,
+    if (force_generic())
+        return hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, 0,
+                                                      as_stream(stream)));
+    // molecules of up to 64 atoms: one wavefront each; the rest: general-shape kernel
+    int st = hip_status(khan::launch_jvp_small<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
                                                   as_stream(stream)));
+    if (st != KHAN_OK) return st;
+    return hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
+                                                  khan::kSmallMaxAtoms + 1, as_stream(stream)));
 }
 
 template <typename T>

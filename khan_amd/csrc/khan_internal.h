@@ -31,6 +31,11 @@ hipError_t launch_fwd_small(const T* X, const T* Y, const T* Z, const int32_t* A
                             const int32_t* MACs, int32_t n_mols, const int32_t* SIs, Buckets<T> out,
                             hipStream_t stream);
 
+template <typename T>
+hipError_t launch_jvp_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
+                            const int32_t* MACs, int32_t n_mols, const int32_t* SIs, const T* VX,
+                            const T* VY, const T* VZ, Buckets<T> out, hipStream_t stream);
+
 // ---- AEV forward for molecules of 65 to 256 atoms, float32 (other sizes are skipped) ----
 constexpr int kMediumMaxAtoms = 256;
 hipError_t launch_fwd_medium_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
