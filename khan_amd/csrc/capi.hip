@@ -30,6 +30,14 @@ bool force_generic()
     return v;
 }
 
+template <typename T>
+bool aligned16(const khan::Buckets<const T>& g)
+{
+    for (int t = 0; t < 4; ++t)
+        if (reinterpret_cast<uintptr_t>(g.p[t]) & 15u) return false;
+    return true;
+}
+
 int forward_dispatch(const float* xs, const float* ys, const float* zs, const int32_t* as,
                      const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
                      khan::Buckets<float> out, hipStream_t stream)
@@ -62,7 +70,9 @@ int backward_dispatch(const float* xs, const float* ys, const float* zs, const i
                       khan::Buckets<const float> g, float* gx, float* gy, float* gz, int64_t n_atoms,
                       hipStream_t stream)
 {
-    if (force_generic())
+    // the specialised kernels fetch upstream rows in 16-byte pieces; buckets that are not 16-byte aligned
+    // (rows are 1,536 bytes, so the bucket's base decides) go through the general kernel, which does not care
+    if (force_generic() || !aligned16(g))
         return hip_status(khan::launch_bwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
                                                           n_atoms, 0, stream));
     // by molecule size: above 256 atoms the general kernel, 65..256 one workgroup per molecule, up to 64
@@ -80,7 +90,7 @@ int backward_dispatch(const double* xs, const double* ys, const double* zs, cons
                       khan::Buckets<const double> g, double* gx, double* gy, double* gz, int64_t n_atoms,
                       hipStream_t stream)
 {
-    if (force_generic())
+    if (force_generic() || !aligned16(g))
         return hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
                                                            n_atoms, 0, stream));
     int st = hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,

@@ -746,3 +746,30 @@ def test_forward_backward_replay_from_a_hip_graph(ops):
         assert torch.allclose(got, grads, rtol=1e-5, atol=1e-5), "replay %d: gradients differ" % replay
         small = torch.from_numpy(c.mol_idxs < b.n_mols).to("cuda:0")
         assert torch.equal(got[:, small], grads[:, small])
+
+
+def test_upstream_buckets_without_16_byte_alignment(ops):
+    # the fast backward kernels read upstream rows in 16-byte pieces; buckets at an odd float offset must
+    # still give the same gradients (they are routed to the general kernel)
+    say("case: upstream gradient buckets at a 4-byte-aligned address")
+    c = Case.from_batch(datagen.make_batch("organic", 64, first_mol=1200))
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+    acs = ac.cpu().tolist()
+    X, Y, Z, A = dev(c.X), dev(c.Y), dev(c.Z), dev(c.A)
+    gen = torch.Generator(device="cuda:0")
+    gen.manual_seed(9)
+    up = torch.randn(c.N * 384, device="cuda:0", generator=gen)
+    aligned, shifted, start = [], [], 0
+    store = torch.empty(c.N * 384 + 8, device="cuda:0")
+    for k in acs:
+        seg = up[start * 384:(start + k) * 384]
+        aligned.append(seg)
+        off = start * 384 + 1                       # one float off a 16-byte boundary
+        store[off:off + k * 384] = seg
+        shifted.append(store[off:off + k * 384])
+        start += k
+    assert any(t.data_ptr() % 16 != 0 for t in shifted if t.numel())
+    ga_ = torch.stack(ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *aligned))
+    gs_ = torch.stack(ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *shifted))
+    scale = float(ga_.abs().max())
+    assert float((ga_ - gs_).abs().max()) <= 2e-5 * scale
