@@ -34,16 +34,14 @@ __global__ __launch_bounds__(256) void aev_fwd_generic_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const LaneConsts<T> L = lane_consts<T>(lane);
     T* ang = ang_rows[wave];
-    // a workgroup walks molecules with the grid's stride, so that a launch in which most molecules
-    // belong to the small-molecule kernel costs a few loads per molecule, not a workgroup each
-    for (int mol = blockIdx.x; mol < n_mols; mol += gridDim.x) {
+    __shared__ unsigned long long want[4];
+    for_each_molecule_in_range(MACs, n_mols, min_atoms, 0x7fffffff, want, [&](int mol) {
         const int n = MACs[mol], off = MOs[mol];
-        if (n < min_atoms) continue;
         for (int i = wave; i < n; i += 4) {
             T* row = out.p[fold_type(A[off + i])] + static_cast<size_t>(SIs[off + i]) * kFeats;
             fwd_center_generic<T>(L, lane, X, Y, Z, A, off, n, i, ang, row);
         }
-    }
+    });
 }
 
 // ------------------------------------------------------------------- Jacobian-vector product
@@ -59,14 +57,14 @@ __global__ __launch_bounds__(256) void aev_jvp_generic_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const LaneConsts<T> L = lane_consts<T>(lane);
     T* ang = ang_rows[wave];
-    for (int mol = blockIdx.x; mol < n_mols; mol += gridDim.x) {
+    __shared__ unsigned long long want[4];
+    for_each_molecule_in_range(MACs, n_mols, min_atoms, 0x7fffffff, want, [&](int mol) {
         const int n = MACs[mol], off = MOs[mol];
-        if (n < min_atoms) continue;
         for (int i = wave; i < n; i += 4) {
             T* row = out.p[fold_type(A[off + i])] + static_cast<size_t>(SIs[off + i]) * kFeats;
             jvp_center_generic<T>(L, lane, X, Y, Z, A, VX, VY, VZ, off, n, i, ang, row);
         }
-    }
+    });
 }
 
 // ----------------------------------------------------------------------------------- backward
@@ -81,9 +79,9 @@ __global__ __launch_bounds__(256) void aev_bwd_generic_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const LaneConsts<T> L = lane_consts<T>(lane);
     T* g_ang = g_rows[wave];
-    for (int mol = blockIdx.x; mol < n_mols; mol += gridDim.x) {
+    __shared__ unsigned long long want[4];
+    for_each_molecule_in_range(MACs, n_mols, min_atoms, 0x7fffffff, want, [&](int mol) {
         const int n = MACs[mol], off = MOs[mol];
-        if (n < min_atoms) continue;        // smaller molecules are handled by the small-molecule kernel
         // every contribution to this molecule's atoms comes from this workgroup: zero them here, then
         // accumulate with atomics (no separate fill pass, nothing to pre-zero for the caller)
         for (int a = threadIdx.x; a < n; a += 256) {
@@ -101,7 +99,7 @@ __global__ __launch_bounds__(256) void aev_bwd_generic_kernel(
                                       atomicAdd(&gZ[off + atom], fz);
                                   });
         }
-    }
+    });
 }
 
 }  // namespace
@@ -110,7 +108,7 @@ __global__ __launch_bounds__(256) void aev_bwd_generic_kernel(
 // `min_atoms` are wanted, a small grid keeps the cost of skipping the others low.
 static unsigned generic_grid(int32_t n_mols, int min_atoms)
 {
-    const int32_t cap = min_atoms > 1 ? 16384 : (1 << 20);
+    const int32_t cap = min_atoms > 1 ? 4096 : (1 << 20);
     return static_cast<unsigned>(n_mols < cap ? n_mols : cap);
 }
 

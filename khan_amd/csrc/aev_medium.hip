@@ -48,10 +48,10 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
     const float kRadExp = -kR_eta_f * 1.44269504088896340736f;   // exp(-eta d^2) = exp2(kRadExp d^2)
     const int rslot = lane >> 4;                                 // radial walk: entry slot of this 16-lane group
 
-    for (int mol = blockIdx.x; mol < n_mols; mol += gridDim.x) {
+    __shared__ unsigned long long want[4];
+    for_each_molecule_in_range(MACs, n_mols, kMedMin, kMediumMaxAtoms, want, [&](int mol) {
         const int n = uniform(MACs[mol]);
         const int off = uniform(MOs[mol]);
-        if (n < kMedMin || n > kMediumMaxAtoms) continue;
 
         // ------------------------------------------------------------ load, sort by type into LDS
         const bool have = tid < n;
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
             }
         }
         __syncthreads();      // the next molecule reuses the sorted arrays
-    }
+    });
 }
 
 }  // namespace

@@ -48,10 +48,10 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
     const LaneConsts<float> L = lane_consts<float>(lane);
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
 
-    for (int mol = blockIdx.x; mol < n_mols; mol += gridDim.x) {
+    __shared__ unsigned long long want[4];
+    for_each_molecule_in_range(MACs, n_mols, kMedMin, kMediumMaxAtoms, want, [&](int mol) {
         const int n = uniform(MACs[mol]);
         const int off = uniform(MOs[mol]);
-        if (n < kMedMin || n > kMediumMaxAtoms) continue;
 
         // ------------------------------------------------------------ load, sort by type into LDS, zero outputs
         const bool have = tid < n;
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
             wave_lds_fence();
         }
         __syncthreads();      // the next molecule reuses the sorted arrays
-    }
+    });
 }
 
 }  // namespace

@@ -97,4 +97,39 @@ __device__ __forceinline__ void wave_lds_fence()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Calls body(mol) for every molecule whose atom count lies in [lo, hi].  The workgroup walks the molecules
+// with the grid's stride; each thread looks at one molecule's count, the wavefronts publish ballots, and
+// all threads then visit the selected molecules together (body may use __syncthreads).  A launch in
+// which (nearly) every molecule belongs to another kernel therefore costs one load per thread, not a
+// dependent load per molecule.  `want` is shared memory, one word per wavefront of the workgroup.
+template <typename Body>
+__device__ __forceinline__ void for_each_molecule_in_range(const int32_t* __restrict__ MACs, int32_t n_mols,
+                                                           int lo, int hi, unsigned long long* want, Body body)
+{
+    const int tid = threadIdx.x, nthreads = blockDim.x, nwaves = nthreads >> 6;
+    for (long long base = blockIdx.x; base < n_mols; base += static_cast<long long>(gridDim.x) * nthreads) {
+        const long long m = base + static_cast<long long>(tid) * gridDim.x;
+        bool wanted = false;
+        if (m < n_mols) {
+            const int n = MACs[m];
+            wanted = n >= lo && n <= hi;
+        }
+        const unsigned long long mask = __ballot(wanted);
+        __syncthreads();                      // everyone is done reading the previous round's words
+        if ((tid & 63) == 0) want[tid >> 6] = mask;
+        __syncthreads();
+        for (int w = 0; w < nwaves; ++w) {
+            const unsigned long long word = want[w];
+            unsigned lo32 = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(word)));
+            unsigned hi32 = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(word >> 32)));
+            unsigned long long mm = (static_cast<unsigned long long>(hi32) << 32) | lo32;
+            while (mm) {
+                const int b = __ffsll(static_cast<long long>(mm)) - 1;
+                mm &= mm - 1;
+                body(static_cast<int>(base + static_cast<long long>(w * 64 + b) * gridDim.x));
+            }
+        }
+    }
+}
+
 }  // namespace khan
