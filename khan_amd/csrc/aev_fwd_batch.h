@@ -11,8 +11,8 @@ namespace khan {
 template <typename T, bool kJvp> struct FwdJvpLds {};
 template <typename T> struct __align__(16) FwdJvpLds<T, true> {
     typename Fast<T>::vec4 vel[64];               // the incoming vector of every atom (sorted order)
-    typename Fast<T>::vec4 nbr_p[kB][kCapA];      // (v_centre - v_partner)/r, and its component along the unit vector
-    typename Fast<T>::vec2 nbr_d[kB][kCapA];      // f_C'(r) dr, and dr = change of the distance along the vectors
+    typename Fast<T>::vec4 nbr_p[kFB][kCapA];      // (v_centre - v_partner)/r, and its component along the unit vector
+    typename Fast<T>::vec2 nbr_d[kFB][kCapA];      // f_C'(r) dr, and dr = change of the distance along the vectors
     typename Fast<T>::vec2 rad_ab[64];            // radial entries: f_C' dr, and -2 eta f_C dr
     T rec2[64][12];                               // phase-1 records: dA_0..7, H_0..3
 };
@@ -21,13 +21,13 @@ template <typename T> struct __align__(16) FwdJvpLds<T, true> {
 template <typename T, bool kJvp = false>
 struct __align__(16) FwdWaveLds {
     typename Fast<T>::vec4 atom[64];          // x, y, z, type (sorted order)
-    typename Fast<T>::vec4 nbr[kB][kCapA];    // unit vector (centre minus partner)/r, and r
-    T nbr_fc[kB][kCapA];                      // f_C(r, A_Rc)
+    typename Fast<T>::vec4 nbr[kFB][kCapA];    // unit vector (centre minus partner)/r, and r
+    T nbr_fc[kFB][kCapA];                      // f_C(r, A_Rc)
     typename Fast<T>::vec2 rad[64];           // (r, f_C(r, R_Rc)); group g of a scan step owns [g*W, (g+1)*W)
     T rec[64][12];                            // phase-1 records: A_0..7, G_0..3
     SegDesc seg[64];                          // non-empty segments of the batch, in order
     unsigned bits[kBitWords];                 // bit per triple slot: a segment starts here
-    int nA[kB][4];                            // angular partners per type, per centre of the batch
+    int nA[kFB][4];                            // angular partners per type, per centre of the batch
     int nR[4][4];                             // radial partners per type, per group of the scan step
     FwdJvpLds<T, kJvp> jvp;
 };
@@ -56,7 +56,7 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
     unsigned seg_row_lo = 0, seg_row_hi = 0;          // where the segment's 32 floats go
     {
         // row of the segment's centre (every lane takes part: the lookup may be a lane exchange)
-        const unsigned long long rowp = row_of_centre(min(seg_b, kB - 1)) +
+        const unsigned long long rowp = row_of_centre(min(seg_b, kFB - 1)) +
                                         static_cast<unsigned long long>((kRadial + seg_pt * kAngBlock) * sizeof(T));
         seg_row_lo = static_cast<unsigned>(rowp);
         seg_row_hi = static_cast<unsigned>(rowp >> 32);

@@ -98,8 +98,8 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
         };
 
         // ------------------------------------------------------------ batches of six centres per wavefront
-        for (int c0 = wave * kB; c0 < n; c0 += 4 * kB) {
-            const int nb = min(kB, n - c0);
+        for (int c0 = wave * kFB; c0 < n; c0 += 4 * kFB) {
+            const int nb = min(kFB, n - c0);
             unsigned overflow = 0;
 
             for (int b = 0; b < nb; ++b) {

@@ -138,8 +138,8 @@ void aev_fwd_small_kernel(
 
     wave_lds_fence();
 
-    for (int c0 = 0; c0 < n; c0 += kB) {
-        const int nb = min(kB, n - c0);
+    for (int c0 = 0; c0 < n; c0 += kFB) {
+        const int nb = min(kFB, n - c0);
         unsigned overflow = 0;
 
         // ------------------------------------------------ scan steps: G centres x W partners

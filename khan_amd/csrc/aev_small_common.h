@@ -7,6 +7,7 @@ namespace khan {
 // One wavefront per workgroup: molecules differ a lot in cost, and a workgroup's LDS is only released when
 // its slowest wavefront ends, so wider workgroups leave wave slots idle.
 constexpr int kWavesPerBlock = 1;
+constexpr int kFB = 6;         // centres per batch of the forward kernels
 constexpr int kB = 6;          // centres per batch: 6 x 10 type pairs = 60 segment lanes
 constexpr int kCapA = 32;      // angular neighbours kept per centre
 constexpr int kBitWords = 96;  // 6 centres x (496 triples + padding) fit in 96 x 32 slot bits
