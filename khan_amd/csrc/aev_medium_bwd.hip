@@ -4,9 +4,9 @@
 // The workgroup sorts the atoms by type into LDS once and zeroes the molecule's outputs.  Wavefronts
 // then draw centres from a shared counter.  A wavefront collects centres into a batch while their
 // angular partner lists fit the 64 entries of its pool (at most six), and for each centre it takes in:
-//   scan + radial   the centre is tested against the sorted atoms 64 at a time; a lane owns one
-//                   (centre, partner) pair, sums g e (f_C' - 2 eta d f_C) over the 16 shells, and adds
-//                   the pull to the partner and (summed over the wave) to the centre;
+//   scan + radial   the centre is tested against the sorted atoms 64 at a time; pairs inside the radial
+//                   cutoff are queued, and whenever 64 are waiting a lane takes one pair, sums
+//                   g e (f_C' - 2 eta d f_C) over the 16 shells, and adds the pull to partner and centre;
 // then for the batch:
 //   stage           the 320 angular upstream values of each centre's row go to LDS by type pair;
 //   angular         the round-robin walk shared with the small-molecule kernel: lane = list entry,
@@ -108,6 +108,65 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
             atomicAdd(&gZ[g], fz);
         };
 
+        // Radial pairs are queued and worked off 64 at a time: only about an eighth of the (centre, partner)
+        // pairs of a large molecule lie inside the radial cutoff, so evaluating them where they are found
+        // would leave most lanes idle.  The queue lives in the pool's staging area, which is free while a
+        // batch is being collected; it is emptied before the batch's upstream rows are staged.
+        float4* const q_d = reinterpret_cast<float4*>(P.gst);                      // 128 x (dx, dy, dz, r)
+        unsigned short* const q_j = reinterpret_cast<unsigned short*>(q_d + 128);  // partner (sorted position)
+        unsigned short* const q_c = q_j + 128;                                     // centre (sorted position)
+        int qn = 0;
+        auto radial_work_off = [&](int count) {      // entries 0..count-1, count <= 64
+            float fx = 0.f, fy = 0.f, fz = 0.f;
+            int c = -1;
+            if (lane < count) {
+                const float4 e = q_d[lane];
+                const int j = q_j[lane];
+                c = q_c[lane];
+                const float* grow = reinterpret_cast<const float*>((static_cast<unsigned long long>(M.row_hi[c]) << 32) | M.row_lo[c]);
+                const float inv = __builtin_amdgcn_rcpf(e.w);
+                const float sc = bwd_radial_pair<float>(grow, type_of(j), e.w, inv);
+                fx = sc * e.x;
+                fy = sc * e.y;
+                fz = sc * e.z;
+                add_force(j, -fx, -fy, -fz);
+            }
+            // the pairs of one centre are summed in the wave (a handful of centres per 64 pairs) and added once
+            unsigned long long todo = wave_ballot(lane < count);
+            while (todo) {
+                const int c0 = lane_read(c, lowest_bit(todo));
+                const bool mine = c == c0;
+                todo &= ~wave_ballot(mine);
+                const float sx = group_sum_to_last_lane(mine ? fx : 0.f, 6);
+                const float sy = group_sum_to_last_lane(mine ? fy : 0.f, 6);
+                const float sz = group_sum_to_last_lane(mine ? fz : 0.f, 6);
+                if (lane == 63) add_force(c0, sx, sy, sz);
+            }
+        };
+        auto radial_drain = [&]() {
+            wave_lds_fence();
+            while (qn > 0) {
+                const int take = min(qn, 64);
+                radial_work_off(take);
+                const int rest = qn - take;
+                float4 e = make_float4(0.f, 0.f, 0.f, 1.f);
+                unsigned short ej = 0, ec = 0;
+                if (lane < rest) {
+                    e = q_d[64 + lane];
+                    ej = q_j[64 + lane];
+                    ec = q_c[64 + lane];
+                }
+                wave_lds_fence();
+                if (lane < rest) {
+                    q_d[lane] = e;
+                    q_j[lane] = ej;
+                    q_c[lane] = ec;
+                }
+                wave_lds_fence();
+                qn = rest;
+            }
+        };
+
         int pending = -1;          // a centre that was drawn but did not fit the previous batch
         for (;;) {
             // ------------------------------------------------ collect a batch of centres
@@ -150,7 +209,7 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                 if (m_c > 64) {
                     // more partners than a pool holds: the general per-centre routine does this centre alone
                     const int i_orig = uniform(static_cast<int>(M.orig[c]));
-                    wave_lds_fence();
+                    radial_drain();                    // the routine uses the staging area as scratch
                     bwd_center_generic<float>(L, lane, X, Y, Z, A, off, n, i_orig, P.gst, row_of(c),
                                               [&](int atom, float fx, float fy, float fz) {
                                                   atomicAdd(&gX[off + atom], fx);
@@ -163,17 +222,15 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                     pending = c;
                     break;
                 }
-                // second pass: list entries, radial pulls
-                const float* grow = row_of(c);
-                float cfx = 0.f, cfy = 0.f, cfz = 0.f;          // pull on the centre, this lane's pairs
+                // second pass: list entries; radial pairs join the queue
                 int pos = used;
 #pragma unroll
                 for (int ch = 0; ch < kChunks; ++ch) {
                     if (ch * 64 < n) {
                         const int j = ch * 64 + lane;
-                        const float inv = __builtin_amdgcn_rcpf(r[ch]);
                         if ((mA[ch] >> lane) & 1ull) {
                             const int p = pos + popc64(mA[ch] & lt_mask);
+                            const float inv = __builtin_amdgcn_rcpf(r[ch]);
                             float fc, dfc;
                             Fast<float>::cutoff_grad(r[ch], kA_Rc_f, fc, dfc);
                             P.nbr[p] = make_float4(dx[ch] * inv, dy[ch] * inv, dz[ch] * inv, r[ch]);
@@ -182,19 +239,34 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                         }
                         pos += popc64(mA[ch]);
                         if ((mR[ch] >> lane) & 1ull) {
-                            const float sc = bwd_radial_pair<float>(grow, type_of(j), r[ch], inv);
-                            const float fx = sc * dx[ch], fy = sc * dy[ch], fz = sc * dz[ch];
-                            cfx += fx;
-                            cfy += fy;
-                            cfz += fz;
-                            add_force(j, -fx, -fy, -fz);
+                            const int p = qn + popc64(mR[ch] & lt_mask);
+                            q_d[p] = make_float4(dx[ch], dy[ch], dz[ch], r[ch]);
+                            q_j[p] = static_cast<unsigned short>(j);
+                            q_c[p] = static_cast<unsigned short>(c);
+                        }
+                        qn += popc64(mR[ch]);
+                        if (qn >= 64) {                  // a full wave of pairs: work it off, keep the rest
+                            wave_lds_fence();
+                            radial_work_off(64);
+                            const int rest = qn - 64;
+                            float4 e = make_float4(0.f, 0.f, 0.f, 1.f);
+                            unsigned short ej = 0, ec = 0;
+                            if (lane < rest) {
+                                e = q_d[64 + lane];
+                                ej = q_j[64 + lane];
+                                ec = q_c[64 + lane];
+                            }
+                            wave_lds_fence();
+                            if (lane < rest) {
+                                q_d[lane] = e;
+                                q_j[lane] = ej;
+                                q_c[lane] = ec;
+                            }
+                            wave_lds_fence();
+                            qn = rest;
                         }
                     }
                 }
-                cfx = group_sum_to_last_lane(cfx, 6);
-                cfy = group_sum_to_last_lane(cfy, 6);
-                cfz = group_sum_to_last_lane(cfz, 6);
-                if (lane == 63) add_force(c, cfx, cfy, cfz);
                 if (lane == nb) {
                     pfv = used;
                     cv = c;
@@ -202,6 +274,7 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                 used += m_c;
                 ++nb;
             }
+            radial_drain();                          // frees the staging area
             if (nb == 0) break;
             if (lane >= nb) pfv = used;              // lanes nb.. hold the end of the pool
 
