@@ -11,6 +11,8 @@
  *   khan_oracle_featurize_* gpu_featurizer/kernel_cpu.cpp:406-537 + functor_op_cpu.cpp:31-38
  *   khan_oracle_featurize_grad_*  gpu_featurizer/kernel_cpu.cpp:217-366 + functor_op_cpu.cpp:68-78
  *                                 (reduced-form derivative, see aev_real.inc)
+ *   khan_oracle_featurize_grad_inverse_*  the contraction meant by gpu_featurizer/kernel_cpu.cpp:37-179
+ *                                 (indexed by atom; the reference indexes by atomic number, see aev_real.inc)
  *   khan_oracle_ani_sort    gpu_featurizer/ani_sort.cpp:71-115
  *   khan_oracle_mol_offsets khan/training/trainer_multi_tower.py:302-303 (segment_sum + exclusive cumsum)
  *   khan_oracle_ani_charge* gpu_featurizer/ani_charges.cpp:58-71, 138-160
@@ -21,6 +23,8 @@
  *   featurize f32/f64 bit-compared with the compiled reference (oracle/_ref) where that is built;
  *                     committed golden vectors written from it; brute-force closed form
  *   featurize_grad    f64 compared with the compiled reference; central differences; invariants
+ *   featurize_grad_inverse  adjoint identity <u, Jv> = <J^T u, v> against featurize_grad, central
+ *                     differences of the forward, the reference's zero result for a uniform vector
  *   ani_charge, ani_charge_grad   closed form / brute force in long double, Euler identity, FD in q.
  *                     The reference holds no value KAT for charges (test_charges.py has no asserts).
  *   ani_charge_grad_xyz  no reference counterpart: pinned by finite differences only.
