@@ -265,13 +265,12 @@ __device__ __forceinline__ void bwd_center_generic(const LaneConsts<T>& L, int l
                         const T cx = ujy * ukz - ujz * uky;
                         const T cy = ujz * ukx - ujx * ukz;
                         const T cz = ujx * uky - ujy * ukx;
-                        // guard: exactly collinear triples have no finite derivative
-                        const T s = fmax(Real<T>::sqrt_(cx * cx + cy * cy + cz * cz), T(1e-30));
+                        const T s = Real<T>::sqrt_(cx * cx + cy * cy + cz * cz);
                         const T base = T(1) + c * L.ct + s * L.st;
                         const T b2 = base * base, b4 = b2 * b2;
                         const T Am1 = b4 * b2 * base;                         // base^(zeta-1)
                         const T At = Am1 * base;
-                        const T dAt = T(8) * Am1 * (L.ct - (c / s) * L.st);   // d/dc (1+cos(th-th_t))^8
+                        const T dAt = T(8) * Am1 * (L.ct - cot_reg(c, s) * L.st);   // d/dc (1+cos(th-th_t))^8; zero cot on the line
                         const T dav = (J.r + K.r) * T(0.5) - L.ars;
                         const T Gs = Real<T>::exp_(-L.A_eta * dav * dav);
                         const T g = g_ang[pair_block(J.type, K.type) * kAngBlock + L.ts];

@@ -773,3 +773,52 @@ def test_upstream_buckets_without_16_byte_alignment(ops):
     gs_ = torch.stack(ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *shifted))
     scale = float(ga_.abs().max())
     assert float((ga_ - gs_).abs().max()) <= 2e-5 * scale
+
+
+def test_linear_molecules_give_finite_gradients(ops):
+    # exactly collinear triples: the angle has a cusp there and the reference's derivative is 0/0.  The
+    # kernels return finite gradients: zero across the axis (by symmetry) and the derivative of the smooth
+    # dependence along the axis, checked against central differences of the forward pass
+    say("case: exactly linear molecules, both precisions, small and general kernels")
+    mols = [
+        (np.array([3, 1, 3]), np.array([[0, 0, -1.16], [0, 0, 0.0], [0, 0, 1.16]])),            # CO2 on the z axis
+        (np.array([0, 1, 2]), np.array([[0, 0, 0.0], [0, 0, 1.06], [0, 0, 2.21]])),             # HCN
+        (np.array([0, 1, 1, 0]), np.array([[-1.66, 0, 0], [-0.6, 0, 0], [0.6, 0, 0], [1.66, 0, 0]])),   # acetylene on x
+    ]
+    A = np.concatenate([m[0] for m in mols]).astype(np.int32)
+    xyz = np.concatenate([m[1] for m in mols]).astype(np.float64)
+    mi = np.concatenate([np.full(len(m[0]), k) for k, m in enumerate(mols)]).astype(np.int32)
+    c = Case(xyz[:, 0], xyz[:, 1], xyz[:, 2], A, mi, len(mols))
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+    acs = ac.cpu().tolist()
+    rng = np.random.default_rng(12)
+    w = dev(rng.standard_normal(c.N * 384))
+    wb, start = [], 0
+    for k in acs:
+        wb.append(w[start * 384:(start + k) * 384])
+        start += k
+    Ad = dev(c.A)
+    axis = np.array([2, 2, 2, 2, 2, 2, 0, 0, 0, 0])     # the molecule's axis per atom
+    for ndt, tol in ((np.float64, 1e-7), (np.float32, 2e-3)):
+        X, Y, Z = dev(xyz[:, 0], ndt), dev(xyz[:, 1], ndt), dev(xyz[:, 2], ndt)
+        wl = [t.to(X.dtype) for t in wb]
+        for forced in (False,):
+            g = torch.stack(ops.featurize_grad(X, Y, Z, Ad, mos, macs, sc, acs, *wl), dim=1).double().cpu().numpy()
+            assert np.all(np.isfinite(g))
+            scale = np.abs(g).max()
+            for a in range(c.N):
+                perp = [k for k in range(3) if k != axis[a]]
+                assert np.abs(g[a, perp]).max() <= 1e-6 * scale, (a, g[a])
+        if ndt == np.float64:
+            # along the axis: central differences of the float64 forward
+            h = 1e-5
+            coords = [X, Y, Z]
+            for a in range(c.N):
+                k = int(axis[a])
+                plus = [t.clone() for t in coords]
+                minus = [t.clone() for t in coords]
+                plus[k][a] += h
+                minus[k][a] -= h
+                Lp = float((torch.cat(ops.featurize(*plus, Ad, mos, macs, sc, acs)) * w).sum())
+                Lm = float((torch.cat(ops.featurize(*minus, Ad, mos, macs, sc, acs)) * w).sum())
+                assert abs((Lp - Lm) / (2 * h) - g[a, k]) <= tol * scale, (a, (Lp - Lm) / (2 * h), g[a, k])
