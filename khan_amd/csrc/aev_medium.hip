@@ -19,7 +19,7 @@ namespace khan {
 
 namespace {
 
-constexpr int kMedMin = kSmallMaxAtoms + 1;   // smaller molecules run one wavefront each
+constexpr int kMedMin = kSmallPreferredMax + 1;   // smaller molecules run one wavefront each
 constexpr int kRadCap = 64;                   // radial partners kept per centre
 
 struct __align__(16) MedShared {

@@ -21,7 +21,7 @@ namespace khan {
 
 namespace {
 
-constexpr int kMedMin = kSmallMaxAtoms + 1;   // smaller molecules run one wavefront each
+constexpr int kMedMin = kSmallPreferredMax + 1;   // smaller molecules run one wavefront each
 constexpr int kChunks = kMediumMaxAtoms / 64;
 
 struct __align__(16) MedBwdShared {

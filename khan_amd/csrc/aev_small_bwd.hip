@@ -46,7 +46,7 @@ void aev_bwd_small_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
-    Buckets<const T> gin, T* __restrict__ gX, T* __restrict__ gY, T* __restrict__ gZ)
+    Buckets<const T> gin, T* __restrict__ gX, T* __restrict__ gY, T* __restrict__ gZ, int max_atoms)
 {
     typedef typename Fast<T>::vec4 vec4;
     __shared__ BwdLds<T> S;
@@ -55,7 +55,7 @@ void aev_bwd_small_kernel(
     if (mol >= n_mols) return;
     const int n = uniform(MACs[mol]);
     const int off = uniform(MOs[mol]);
-    if (n <= 0 || n > 64) return;                 // larger molecules belong to the general kernel
+    if (n <= 0 || n > max_atoms) return;          // larger molecules belong to other kernels (max_atoms <= 64)
     const LaneConsts<T> L = lane_consts<T>(lane);
     const unsigned long long lane_bit = 1ull << lane;
     const unsigned long long lt_mask = lane_bit - 1ull;
@@ -317,14 +317,14 @@ void aev_bwd_small_kernel(
 template <typename T>
 hipError_t launch_bwd_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
                             const int32_t* MACs, int32_t n_mols, const int32_t* SIs, Buckets<const T> g,
-                            T* gX, T* gY, T* gZ, hipStream_t stream)
+                            T* gX, T* gY, T* gZ, int max_atoms, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
-    aev_bwd_small_kernel<T><<<dim3(static_cast<unsigned>(n_mols)), dim3(64), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ);
+    aev_bwd_small_kernel<T><<<dim3(static_cast<unsigned>(n_mols)), dim3(64), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ, max_atoms < 64 ? max_atoms : 64);
     return hipGetLastError();
 }
 
-template hipError_t launch_bwd_small<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const float>, float*, float*, float*, hipStream_t);
-template hipError_t launch_bwd_small<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const double>, double*, double*, double*, hipStream_t);
+template hipError_t launch_bwd_small<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const float>, float*, float*, float*, int, hipStream_t);
+template hipError_t launch_bwd_small<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const double>, double*, double*, double*, int, hipStream_t);
 
 }  // namespace khan

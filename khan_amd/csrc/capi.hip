@@ -44,8 +44,8 @@ int forward_dispatch(const float* xs, const float* ys, const float* zs, const in
 {
     if (force_generic())
         return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, stream));
-    // molecules of up to 64 atoms: one wavefront each; up to 256: one workgroup each; the rest: general kernel
-    int st = hip_status(khan::launch_fwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, stream));
+    // molecules of up to 32 atoms: one wavefront each; up to 256: one workgroup each; the rest: general kernel
+    int st = hip_status(khan::launch_fwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallPreferredMax, stream));
     if (st != KHAN_OK) return st;
     st = hip_status(khan::launch_fwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, out, stream));
     if (st != KHAN_OK) return st;
@@ -59,7 +59,7 @@ int forward_dispatch(const double* xs, const double* ys, const double* zs, const
 {
     if (force_generic())
         return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, stream));
-    int st = hip_status(khan::launch_fwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, stream));
+    int st = hip_status(khan::launch_fwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallMaxAtoms, stream));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
                                                        khan::kSmallMaxAtoms + 1, stream));
@@ -75,14 +75,14 @@ int backward_dispatch(const float* xs, const float* ys, const float* zs, const i
     if (force_generic() || !aligned16(g))
         return hip_status(khan::launch_bwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
                                                           n_atoms, 0, stream));
-    // by molecule size: above 256 atoms the general kernel, 65..256 one workgroup per molecule, up to 64
+    // by molecule size: above 256 atoms the general kernel, 33..256 one workgroup per molecule, up to 32
     // one wavefront per molecule; each kernel defines every gradient of its own molecules
     int st = hip_status(khan::launch_bwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
                                                         n_atoms, khan::kMediumMaxAtoms + 1, stream));
     if (st != KHAN_OK) return st;
     st = hip_status(khan::launch_bwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, stream));
     if (st != KHAN_OK) return st;
-    return hip_status(khan::launch_bwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, stream));
+    return hip_status(khan::launch_bwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, khan::kSmallPreferredMax, stream));
 }
 
 int backward_dispatch(const double* xs, const double* ys, const double* zs, const int32_t* as,
@@ -96,7 +96,7 @@ int backward_dispatch(const double* xs, const double* ys, const double* zs, cons
     int st = hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
                                                          n_atoms, khan::kSmallMaxAtoms + 1, stream));
     if (st != KHAN_OK) return st;
-    return hip_status(khan::launch_bwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, stream));
+    return hip_status(khan::launch_bwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, khan::kSmallMaxAtoms, stream));
 }
 
 template <typename T>

@@ -25,11 +25,14 @@ hipError_t launch_jvp_generic(const T* X, const T* Y, const T* Z, const int32_t*
                               int min_atoms, hipStream_t stream);
 
 // ---- AEV forward for molecules of up to 64 atoms (larger molecules are skipped) ----
-constexpr int kSmallMaxAtoms = 64;
+constexpr int kSmallMaxAtoms = 64;      // what one wavefront can hold
+// where a medium-molecule kernel exists, molecules above this size go to it: one wavefront working through a
+// dense 64-atom molecule alone takes as long as the rest of a batch
+constexpr int kSmallPreferredMax = 32;
 template <typename T>
 hipError_t launch_fwd_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
                             const int32_t* MACs, int32_t n_mols, const int32_t* SIs, Buckets<T> out,
-                            hipStream_t stream);
+                            int max_atoms, hipStream_t stream);
 
 template <typename T>
 hipError_t launch_jvp_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
@@ -55,7 +58,7 @@ hipError_t launch_bwd_generic(const T* X, const T* Y, const T* Z, const int32_t*
 template <typename T>
 hipError_t launch_bwd_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
                             const int32_t* MACs, int32_t n_mols, const int32_t* SIs, Buckets<const T> g,
-                            T* gX, T* gY, T* gZ, hipStream_t stream);
+                            T* gX, T* gY, T* gZ, int max_atoms, hipStream_t stream);
 
 // ---- integer path ----
 hipError_t launch_mol_offsets(const int32_t* mol_idxs, int64_t n_atoms, int32_t n_mols,
