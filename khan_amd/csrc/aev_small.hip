@@ -38,15 +38,17 @@ void aev_fwd_small_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
-    const T* __restrict__ VX, const T* __restrict__ VY, const T* __restrict__ VZ, Buckets<T> out, int max_atoms)
+    const T* __restrict__ VX, const T* __restrict__ VY, const T* __restrict__ VZ, Buckets<T> out, int max_atoms,
+    const int32_t* __restrict__ order)
 {
     typedef typename Fast<T>::vec4 vec4;
     typedef typename Fast<T>::vec2 vec2;
     __shared__ FwdWaveLds<T, kJvp> lds_all[kWavesPerBlock];
     const int lane = threadIdx.x & 63;
     const int wave = uniform(threadIdx.x >> 6);
-    const int mol = blockIdx.x * kWavesPerBlock + wave;
-    if (mol >= n_mols) return;
+    const int slot = blockIdx.x * kWavesPerBlock + wave;
+    if (slot >= n_mols) return;
+    const int mol = order ? uniform(order[slot]) : slot;      // largest molecules first when an order is given
     const int n = uniform(MACs[mol]);
     const int off = uniform(MOs[mol]);
     if (n <= 0 || n > max_atoms) return;          // larger molecules belong to other kernels (max_atoms <= 64)
@@ -283,30 +285,30 @@ void aev_fwd_small_kernel(
 template <typename T>
 hipError_t launch_fwd_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
                             const int32_t* MACs, int32_t n_mols, const int32_t* SIs, Buckets<T> out,
-                            int max_atoms, hipStream_t stream)
+                            int max_atoms, const int32_t* order, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
     const unsigned blocks = (static_cast<unsigned>(n_mols) + kWavesPerBlock - 1u) / kWavesPerBlock;
     aev_fwd_small_kernel<T, false><<<dim3(blocks), dim3(64 * kWavesPerBlock), 0, stream>>>(
-        X, Y, Z, A, MOs, MACs, n_mols, SIs, nullptr, nullptr, nullptr, out, max_atoms < 64 ? max_atoms : 64);
+        X, Y, Z, A, MOs, MACs, n_mols, SIs, nullptr, nullptr, nullptr, out, max_atoms < 64 ? max_atoms : 64, order);
     return hipGetLastError();
 }
 
 template <typename T>
 hipError_t launch_jvp_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
                             const int32_t* MACs, int32_t n_mols, const int32_t* SIs, const T* VX,
-                            const T* VY, const T* VZ, Buckets<T> out, hipStream_t stream)
+                            const T* VY, const T* VZ, Buckets<T> out, const int32_t* order, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
     const unsigned blocks = (static_cast<unsigned>(n_mols) + kWavesPerBlock - 1u) / kWavesPerBlock;
     aev_fwd_small_kernel<T, true><<<dim3(blocks), dim3(64 * kWavesPerBlock), 0, stream>>>(
-        X, Y, Z, A, MOs, MACs, n_mols, SIs, VX, VY, VZ, out, kSmallMaxAtoms);
+        X, Y, Z, A, MOs, MACs, n_mols, SIs, VX, VY, VZ, out, kSmallMaxAtoms, order);
     return hipGetLastError();
 }
 
-template hipError_t launch_fwd_small<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<float>, int, hipStream_t);
-template hipError_t launch_fwd_small<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<double>, int, hipStream_t);
-template hipError_t launch_jvp_small<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const float*, const float*, const float*, Buckets<float>, hipStream_t);
-template hipError_t launch_jvp_small<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const double*, const double*, const double*, Buckets<double>, hipStream_t);
+template hipError_t launch_fwd_small<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<float>, int, const int32_t*, hipStream_t);
+template hipError_t launch_fwd_small<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<double>, int, const int32_t*, hipStream_t);
+template hipError_t launch_jvp_small<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const float*, const float*, const float*, Buckets<float>, const int32_t*, hipStream_t);
+template hipError_t launch_jvp_small<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const double*, const double*, const double*, Buckets<double>, const int32_t*, hipStream_t);
 
 }  // namespace khan

@@ -46,13 +46,14 @@ void aev_bwd_small_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
-    Buckets<const T> gin, T* __restrict__ gX, T* __restrict__ gY, T* __restrict__ gZ, int max_atoms)
+    Buckets<const T> gin, T* __restrict__ gX, T* __restrict__ gY, T* __restrict__ gZ, int max_atoms,
+    const int32_t* __restrict__ order)
 {
     typedef typename Fast<T>::vec4 vec4;
     __shared__ BwdLds<T> S;
     const int lane = threadIdx.x;
-    const int mol = blockIdx.x;
-    if (mol >= n_mols) return;
+    if (static_cast<int>(blockIdx.x) >= n_mols) return;
+    const int mol = order ? uniform(order[blockIdx.x]) : static_cast<int>(blockIdx.x);   // largest first when ordered
     const int n = uniform(MACs[mol]);
     const int off = uniform(MOs[mol]);
     if (n <= 0 || n > max_atoms) return;          // larger molecules belong to other kernels (max_atoms <= 64)
@@ -317,14 +318,14 @@ void aev_bwd_small_kernel(
 template <typename T>
 hipError_t launch_bwd_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
                             const int32_t* MACs, int32_t n_mols, const int32_t* SIs, Buckets<const T> g,
-                            T* gX, T* gY, T* gZ, int max_atoms, hipStream_t stream)
+                            T* gX, T* gY, T* gZ, int max_atoms, const int32_t* order, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
-    aev_bwd_small_kernel<T><<<dim3(static_cast<unsigned>(n_mols)), dim3(64), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ, max_atoms < 64 ? max_atoms : 64);
+    aev_bwd_small_kernel<T><<<dim3(static_cast<unsigned>(n_mols)), dim3(64), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ, max_atoms < 64 ? max_atoms : 64, order);
     return hipGetLastError();
 }
 
-template hipError_t launch_bwd_small<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const float>, float*, float*, float*, int, hipStream_t);
-template hipError_t launch_bwd_small<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const double>, double*, double*, double*, int, hipStream_t);
+template hipError_t launch_bwd_small<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const float>, float*, float*, float*, int, const int32_t*, hipStream_t);
+template hipError_t launch_bwd_small<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const double>, double*, double*, double*, int, const int32_t*, hipStream_t);
 
 }  // namespace khan

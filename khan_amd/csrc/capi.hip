@@ -38,6 +38,43 @@ bool aligned16(const khan::Buckets<const T>& g)
     return true;
 }
 
+// Stream-ordered scratch holding the molecule indices by decreasing size for the one-wavefront kernels.
+// No order (the kernels then take molecules as they come) while the stream is being captured into a graph,
+// for very large or tiny batches, or when the allocation fails.
+class SizeOrder {
+public:
+    SizeOrder(const int32_t* macs, int32_t n_mols, hipStream_t stream) : stream_(stream)
+    {
+        if (n_mols < 2048 || n_mols > (1 << 20)) return;
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return;
+        }
+        if (hipMallocAsync(reinterpret_cast<void**>(&order_), sizeof(int32_t) * static_cast<size_t>(n_mols), stream) != hipSuccess) {
+            (void)hipGetLastError();
+            order_ = nullptr;
+            return;
+        }
+        if (khan::launch_size_order(macs, n_mols, order_, stream) != hipSuccess) {
+            (void)hipGetLastError();
+            (void)hipFreeAsync(order_, stream);
+            order_ = nullptr;
+        }
+    }
+    ~SizeOrder()
+    {
+        if (order_) (void)hipFreeAsync(order_, stream_);
+    }
+    SizeOrder(const SizeOrder&) = delete;
+    SizeOrder& operator=(const SizeOrder&) = delete;
+    const int32_t* get() const { return order_; }
+
+private:
+    int32_t* order_ = nullptr;
+    hipStream_t stream_;
+};
+
 int forward_dispatch(const float* xs, const float* ys, const float* zs, const int32_t* as,
                      const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
                      khan::Buckets<float> out, hipStream_t stream)
@@ -45,7 +82,9 @@ int forward_dispatch(const float* xs, const float* ys, const float* zs, const in
     if (force_generic())
         return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, stream));
     // molecules of up to 32 atoms: one wavefront each; up to 256: one workgroup each; the rest: general kernel
-    int st = hip_status(khan::launch_fwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallPreferredMax, stream));
+    SizeOrder order(macs, n_mols, stream);
+    int st = hip_status(khan::launch_fwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallPreferredMax,
+                                                      order.get(), stream));
     if (st != KHAN_OK) return st;
     st = hip_status(khan::launch_fwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, out, stream));
     if (st != KHAN_OK) return st;
@@ -59,7 +98,9 @@ int forward_dispatch(const double* xs, const double* ys, const double* zs, const
 {
     if (force_generic())
         return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, stream));
-    int st = hip_status(khan::launch_fwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallMaxAtoms, stream));
+    SizeOrder order(macs, n_mols, stream);
+    int st = hip_status(khan::launch_fwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallMaxAtoms,
+                                                       order.get(), stream));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
                                                        khan::kSmallMaxAtoms + 1, stream));
@@ -82,7 +123,9 @@ int backward_dispatch(const float* xs, const float* ys, const float* zs, const i
     if (st != KHAN_OK) return st;
     st = hip_status(khan::launch_bwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, stream));
     if (st != KHAN_OK) return st;
-    return hip_status(khan::launch_bwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, khan::kSmallPreferredMax, stream));
+    SizeOrder order(macs, n_mols, stream);
+    return hip_status(khan::launch_bwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                    khan::kSmallPreferredMax, order.get(), stream));
 }
 
 int backward_dispatch(const double* xs, const double* ys, const double* zs, const int32_t* as,
@@ -96,7 +139,9 @@ int backward_dispatch(const double* xs, const double* ys, const double* zs, cons
     int st = hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
                                                          n_atoms, khan::kSmallMaxAtoms + 1, stream));
     if (st != KHAN_OK) return st;
-    return hip_status(khan::launch_bwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, khan::kSmallMaxAtoms, stream));
+    SizeOrder order(macs, n_mols, stream);
+    return hip_status(khan::launch_bwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                     khan::kSmallMaxAtoms, order.get(), stream));
 }
 
 template <typename T>
@@ -154,7 +199,8 @@ int featurize_grad_inverse_impl(const T* xs, const T* ys, const T* zs, const int
         return hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, 0,
                                                       as_stream(stream)));
     // molecules of up to 64 atoms: one wavefront each; the rest: general-shape kernel
-    int st = hip_status(khan::launch_jvp_small<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
+    SizeOrder order(macs, n_mols, as_stream(stream));
+    int st = hip_status(khan::launch_jvp_small<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, order.get(),
                                                   as_stream(stream)));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,

@@ -32,12 +32,12 @@ constexpr int kSmallPreferredMax = 32;
 template <typename T>
 hipError_t launch_fwd_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
                             const int32_t* MACs, int32_t n_mols, const int32_t* SIs, Buckets<T> out,
-                            int max_atoms, hipStream_t stream);
+                            int max_atoms, const int32_t* order, hipStream_t stream);
 
 template <typename T>
 hipError_t launch_jvp_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
                             const int32_t* MACs, int32_t n_mols, const int32_t* SIs, const T* VX,
-                            const T* VY, const T* VZ, Buckets<T> out, hipStream_t stream);
+                            const T* VY, const T* VZ, Buckets<T> out, const int32_t* order, hipStream_t stream);
 
 // ---- AEV forward for molecules of 65 to 256 atoms, float32 (other sizes are skipped) ----
 constexpr int kMediumMaxAtoms = 256;
@@ -58,13 +58,16 @@ hipError_t launch_bwd_generic(const T* X, const T* Y, const T* Z, const int32_t*
 template <typename T>
 hipError_t launch_bwd_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
                             const int32_t* MACs, int32_t n_mols, const int32_t* SIs, Buckets<const T> g,
-                            T* gX, T* gY, T* gZ, int max_atoms, hipStream_t stream);
+                            T* gX, T* gY, T* gZ, int max_atoms, const int32_t* order, hipStream_t stream);
 
 // ---- integer path ----
 hipError_t launch_mol_offsets(const int32_t* mol_idxs, int64_t n_atoms, int32_t n_mols,
                               int32_t* MACs, int32_t* MOs, hipStream_t stream);
 hipError_t launch_ani_sort(const int32_t* A, int64_t n_atoms, int32_t* scatter, int32_t* gather,
                            int32_t* counts4, hipStream_t stream);
+
+// molecule indices by decreasing atom count (one workgroup; meant for up to about a million molecules)
+hipError_t launch_size_order(const int32_t* MACs, int32_t n_mols, int32_t* order, hipStream_t stream);
 
 // ---- charges ----
 template <typename T>

@@ -228,4 +228,48 @@ hipError_t launch_ani_sort(const int32_t* A, int64_t n_atoms, int32_t* scatter, 
     return (e != hipSuccess) ? e : e2;
 }
 
+// ---- molecules in order of decreasing atom count ----
+// One workgroup sorts the molecule indices by min(atom count, 65), largest first (counting sort with LDS
+// integer atomics; the order inside a size class is whatever the atomics give, which no result depends on).
+// The one-wavefront kernels take molecule order[b] in workgroup b: the dispatcher hands out workgroups in
+// index order, so the expensive molecules start first and the launch does not end on a few long waves.
+namespace {
+constexpr int kSizeBins = 66;
+constexpr int kOrderThreads = 1024;
+
+__global__ __launch_bounds__(kOrderThreads) void size_order_kernel(const int32_t* __restrict__ MACs, int32_t n_mols,
+                                                                    int32_t* __restrict__ order)
+{
+    __shared__ int hist[kSizeBins];
+    __shared__ int cursor[kSizeBins];
+    const int tid = threadIdx.x;
+    if (tid < kSizeBins) hist[tid] = 0;
+    __syncthreads();
+    for (int m = tid; m < n_mols; m += kOrderThreads) {
+        const int n = MACs[m];
+        atomicAdd(&hist[65 - min(max(n, 0), 65)], 1);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0;
+        for (int b = 0; b < kSizeBins; ++b) {
+            cursor[b] = run;
+            run += hist[b];
+        }
+    }
+    __syncthreads();
+    for (int m = tid; m < n_mols; m += kOrderThreads) {
+        const int n = MACs[m];
+        order[atomicAdd(&cursor[65 - min(max(n, 0), 65)], 1)] = m;
+    }
+}
+}  // namespace
+
+hipError_t launch_size_order(const int32_t* MACs, int32_t n_mols, int32_t* order, hipStream_t stream)
+{
+    if (n_mols <= 0) return hipSuccess;
+    size_order_kernel<<<dim3(1), dim3(kOrderThreads), 0, stream>>>(MACs, n_mols, order);
+    return hipGetLastError();
+}
+
 }  // namespace khan
