@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256) void aev_fwd_generic_kernel(
     const LaneConsts<T> L = lane_consts<T>(lane);
     T* ang = ang_rows[wave];
     __shared__ unsigned long long want[4];
-    for_each_molecule_in_range(MACs, n_mols, min_atoms, 0x7fffffff, want, [&](int mol) {
+    for_each_molecule_in_range(MACs, n_mols, min_atoms, 0x7fffffff, want, nullptr, [&](int mol) {
         const int n = MACs[mol], off = MOs[mol];
         for (int i = wave; i < n; i += 4) {
             T* row = out.p[fold_type(A[off + i])] + static_cast<size_t>(SIs[off + i]) * kFeats;
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256) void aev_jvp_generic_kernel(
     const LaneConsts<T> L = lane_consts<T>(lane);
     T* ang = ang_rows[wave];
     __shared__ unsigned long long want[4];
-    for_each_molecule_in_range(MACs, n_mols, min_atoms, 0x7fffffff, want, [&](int mol) {
+    for_each_molecule_in_range(MACs, n_mols, min_atoms, 0x7fffffff, want, nullptr, [&](int mol) {
         const int n = MACs[mol], off = MOs[mol];
         for (int i = wave; i < n; i += 4) {
             T* row = out.p[fold_type(A[off + i])] + static_cast<size_t>(SIs[off + i]) * kFeats;
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void aev_bwd_generic_kernel(
     const LaneConsts<T> L = lane_consts<T>(lane);
     T* g_ang = g_rows[wave];
     __shared__ unsigned long long want[4];
-    for_each_molecule_in_range(MACs, n_mols, min_atoms, 0x7fffffff, want, [&](int mol) {
+    for_each_molecule_in_range(MACs, n_mols, min_atoms, 0x7fffffff, want, nullptr, [&](int mol) {
         const int n = MACs[mol], off = MOs[mol];
         // every contribution to this molecule's atoms comes from this workgroup: zero them here, then
         // accumulate with atomics (no separate fill pass, nothing to pre-zero for the caller)

@@ -34,7 +34,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
     const float* __restrict__ X, const float* __restrict__ Y, const float* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
-    Buckets<float> out)
+    Buckets<float> out, const int32_t* __restrict__ order)
 {
     __shared__ MedShared M;
     __shared__ FwdWaveLds<float> lds_wave[4];
@@ -49,7 +49,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
     const int rslot = lane >> 4;                                 // radial walk: entry slot of this 16-lane group
 
     __shared__ unsigned long long want[4];
-    for_each_molecule_in_range(MACs, n_mols, kMedMin, kMediumMaxAtoms, want, [&](int mol) {
+    for_each_molecule_in_range(MACs, n_mols, kMedMin, kMediumMaxAtoms, want, order, [&](int mol) {
         const int n = uniform(MACs[mol]);
         const int off = uniform(MOs[mol]);
 
@@ -198,12 +198,12 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
 
 hipError_t launch_fwd_medium_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
                                  const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
-                                 const int32_t* SIs, Buckets<float> out, hipStream_t stream)
+                                 const int32_t* SIs, Buckets<float> out, const int32_t* order, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
     // workgroups walk the molecules with the grid's stride and skip those of other sizes
     const unsigned blocks = static_cast<unsigned>(n_mols < 4096 ? n_mols : 4096);
-    aev_fwd_medium_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, out);
+    aev_fwd_medium_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, out, order);
     return hipGetLastError();
 }
 

@@ -45,7 +45,7 @@ class SizeOrder {
 public:
     SizeOrder(const int32_t* macs, int32_t n_mols, hipStream_t stream) : stream_(stream)
     {
-        if (n_mols < 2048 || n_mols > (1 << 20)) return;
+        if (n_mols < 512 || n_mols > (1 << 20)) return;
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
             (void)hipGetLastError();
@@ -86,7 +86,7 @@ int forward_dispatch(const float* xs, const float* ys, const float* zs, const in
     int st = hip_status(khan::launch_fwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallPreferredMax,
                                                       order.get(), stream));
     if (st != KHAN_OK) return st;
-    st = hip_status(khan::launch_fwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, out, stream));
+    st = hip_status(khan::launch_fwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, out, order.get(), stream));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
                                                       khan::kMediumMaxAtoms + 1, stream));
@@ -121,9 +121,10 @@ int backward_dispatch(const float* xs, const float* ys, const float* zs, const i
     int st = hip_status(khan::launch_bwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
                                                         n_atoms, khan::kMediumMaxAtoms + 1, stream));
     if (st != KHAN_OK) return st;
-    st = hip_status(khan::launch_bwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, stream));
-    if (st != KHAN_OK) return st;
     SizeOrder order(macs, n_mols, stream);
+    // (the workgroup-per-molecule backward kernel measures slower when it is given the size order)
+    st = hip_status(khan::launch_bwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, nullptr, stream));
+    if (st != KHAN_OK) return st;
     return hip_status(khan::launch_bwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
                                                     khan::kSmallPreferredMax, order.get(), stream));
 }

@@ -43,12 +43,12 @@ hipError_t launch_jvp_small(const T* X, const T* Y, const T* Z, const int32_t* A
 constexpr int kMediumMaxAtoms = 256;
 hipError_t launch_fwd_medium_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
                                  const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
-                                 const int32_t* SIs, Buckets<float> out, hipStream_t stream);
+                                 const int32_t* SIs, Buckets<float> out, const int32_t* order, hipStream_t stream);
 
 hipError_t launch_bwd_medium_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
                                  const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
                                  const int32_t* SIs, Buckets<const float> g, float* gX, float* gY,
-                                 float* gZ, hipStream_t stream);
+                                 float* gZ, const int32_t* order, hipStream_t stream);
 
 template <typename T>
 hipError_t launch_bwd_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
@@ -107,17 +107,21 @@ __device__ __forceinline__ void wave_lds_fence()
 // with the grid's stride; each thread looks at one molecule's count, the wavefronts publish ballots, and
 // all threads then visit the selected molecules together (body may use __syncthreads).  A launch in
 // which (nearly) every molecule belongs to another kernel therefore costs one load per thread, not a
-// dependent load per molecule.  `want` is shared memory, one word per wavefront of the workgroup.
+// dependent load per molecule.  `want` is shared memory, one word per wavefront of the workgroup.  With
+// `order` (molecule indices by decreasing size) the molecules are visited in that order.
 template <typename Body>
 __device__ __forceinline__ void for_each_molecule_in_range(const int32_t* __restrict__ MACs, int32_t n_mols,
-                                                           int lo, int hi, unsigned long long* want, Body body)
+                                                           int lo, int hi, unsigned long long* want,
+                                                           const int32_t* __restrict__ order, Body body)
 {
     const int tid = threadIdx.x, nthreads = blockDim.x, nwaves = nthreads >> 6;
     for (long long base = blockIdx.x; base < n_mols; base += static_cast<long long>(gridDim.x) * nthreads) {
         const long long m = base + static_cast<long long>(tid) * gridDim.x;
         bool wanted = false;
+        int mol = 0;                          // position m of the size order, when one is given
         if (m < n_mols) {
-            const int n = MACs[m];
+            mol = order ? order[m] : static_cast<int>(m);
+            const int n = MACs[mol];
             wanted = n >= lo && n <= hi;
         }
         const unsigned long long mask = __ballot(wanted);
@@ -132,7 +136,8 @@ __device__ __forceinline__ void for_each_molecule_in_range(const int32_t* __rest
             while (mm) {
                 const int b = __ffsll(static_cast<long long>(mm)) - 1;
                 mm &= mm - 1;
-                body(static_cast<int>(base + static_cast<long long>(w * 64 + b) * gridDim.x));
+                const long long pos = base + static_cast<long long>(w * 64 + b) * gridDim.x;
+                body(order ? __builtin_amdgcn_readfirstlane(order[pos]) : static_cast<int>(pos));
             }
         }
     }

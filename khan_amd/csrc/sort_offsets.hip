@@ -229,12 +229,13 @@ hipError_t launch_ani_sort(const int32_t* A, int64_t n_atoms, int32_t* scatter, 
 }
 
 // ---- molecules in order of decreasing atom count ----
-// One workgroup sorts the molecule indices by min(atom count, 65), largest first (counting sort with LDS
+// One workgroup sorts the molecule indices by min(atom count, 257), largest first (counting sort with LDS
 // integer atomics; the order inside a size class is whatever the atomics give, which no result depends on).
-// The one-wavefront kernels take molecule order[b] in workgroup b: the dispatcher hands out workgroups in
+// The one-wavefront kernels take molecule order[b] in workgroup b (the workgroup-per-molecule kernels walk the
+// same order with the grid's stride): the dispatcher hands out workgroups in
 // index order, so the expensive molecules start first and the launch does not end on a few long waves.
 namespace {
-constexpr int kSizeBins = 66;
+constexpr int kSizeBins = 258;    // atom counts 0..256 and "more"
 constexpr int kOrderThreads = 1024;
 
 __global__ __launch_bounds__(kOrderThreads) void size_order_kernel(const int32_t* __restrict__ MACs, int32_t n_mols,
@@ -247,7 +248,7 @@ __global__ __launch_bounds__(kOrderThreads) void size_order_kernel(const int32_t
     __syncthreads();
     for (int m = tid; m < n_mols; m += kOrderThreads) {
         const int n = MACs[m];
-        atomicAdd(&hist[65 - min(max(n, 0), 65)], 1);
+        atomicAdd(&hist[kSizeBins - 1 - min(max(n, 0), kSizeBins - 1)], 1);
     }
     __syncthreads();
     if (tid == 0) {
@@ -260,7 +261,7 @@ __global__ __launch_bounds__(kOrderThreads) void size_order_kernel(const int32_t
     __syncthreads();
     for (int m = tid; m < n_mols; m += kOrderThreads) {
         const int n = MACs[m];
-        order[atomicAdd(&cursor[65 - min(max(n, 0), 65)], 1)] = m;
+        order[atomicAdd(&cursor[kSizeBins - 1 - min(max(n, 0), kSizeBins - 1)], 1)] = m;
     }
 }
 }  // namespace
