@@ -40,23 +40,23 @@ bool aligned16(const khan::Buckets<const T>& g)
 
 // Stream-ordered scratch holding the molecule indices by decreasing size for the one-wavefront kernels.
 // No order (the kernels then take molecules as they come) while the stream is being captured into a graph,
-// for very large or tiny batches, or when the allocation fails.
+// for tiny batches, or when the allocation fails.
 class SizeOrder {
 public:
     SizeOrder(const int32_t* macs, int32_t n_mols, hipStream_t stream) : stream_(stream)
     {
-        if (n_mols < 512 || n_mols > (1 << 20)) return;
+        if (n_mols < 512) return;
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
             (void)hipGetLastError();
             return;
         }
-        if (hipMallocAsync(reinterpret_cast<void**>(&order_), sizeof(int32_t) * static_cast<size_t>(n_mols), stream) != hipSuccess) {
+        if (hipMallocAsync(reinterpret_cast<void**>(&order_), sizeof(int32_t) * (static_cast<size_t>(n_mols) + khan::kSizeOrderScratch), stream) != hipSuccess) {
             (void)hipGetLastError();
             order_ = nullptr;
             return;
         }
-        if (khan::launch_size_order(macs, n_mols, order_, stream) != hipSuccess) {
+        if (khan::launch_size_order(macs, n_mols, order_, order_ + n_mols, stream) != hipSuccess) {
             (void)hipGetLastError();
             (void)hipFreeAsync(order_, stream);
             order_ = nullptr;

@@ -66,8 +66,10 @@ hipError_t launch_mol_offsets(const int32_t* mol_idxs, int64_t n_atoms, int32_t 
 hipError_t launch_ani_sort(const int32_t* A, int64_t n_atoms, int32_t* scatter, int32_t* gather,
                            int32_t* counts4, hipStream_t stream);
 
-// molecule indices by decreasing atom count (one workgroup; meant for up to about a million molecules)
-hipError_t launch_size_order(const int32_t* MACs, int32_t n_mols, int32_t* order, hipStream_t stream);
+// molecule indices by decreasing atom count; `scratch` is kSizeOrderScratch ints (not for use under graph capture:
+// it is cleared with a memset)
+constexpr int kSizeOrderScratch = 2 * 258;
+hipError_t launch_size_order(const int32_t* MACs, int32_t n_mols, int32_t* order, int32_t* scratch, hipStream_t stream);
 
 // ---- charges ----
 template <typename T>

@@ -229,47 +229,77 @@ hipError_t launch_ani_sort(const int32_t* A, int64_t n_atoms, int32_t* scatter, 
 }
 
 // ---- molecules in order of decreasing atom count ----
-// One workgroup sorts the molecule indices by min(atom count, 257), largest first (counting sort with LDS
-// integer atomics; the order inside a size class is whatever the atomics give, which no result depends on).
-// The one-wavefront kernels take molecule order[b] in workgroup b (the workgroup-per-molecule kernels walk the
-// same order with the grid's stride): the dispatcher hands out workgroups in
-// index order, so the expensive molecules start first and the launch does not end on a few long waves.
+// Counting sort of the molecule indices by min(atom count, 257), largest first.  Two passes over the
+// molecules, 1,024 per workgroup: the first adds workgroup histograms (LDS integer atomics) into a global
+// one; the second recomputes its histogram, reserves a range per size class with one global atomic, and
+// places its molecules inside the ranges.  The order inside a size class is whatever the atomics give,
+// which no result depends on.  The one-wavefront kernels take molecule order[b] in workgroup b (the
+// workgroup-per-molecule kernels walk the same order with the grid's stride): the dispatcher hands out
+// workgroups in index order, so the expensive molecules start first and a launch does not end on a few
+// long waves.
 namespace {
 constexpr int kSizeBins = 258;    // atom counts 0..256 and "more"
 constexpr int kOrderThreads = 1024;
 
-__global__ __launch_bounds__(kOrderThreads) void size_order_kernel(const int32_t* __restrict__ MACs, int32_t n_mols,
-                                                                    int32_t* __restrict__ order)
+__device__ __forceinline__ int size_bin(int n) { return kSizeBins - 1 - min(max(n, 0), kSizeBins - 1); }
+
+__global__ __launch_bounds__(kOrderThreads) void size_hist_kernel(const int32_t* __restrict__ MACs, int32_t n_mols,
+                                                                   int32_t* __restrict__ ghist)
 {
     __shared__ int hist[kSizeBins];
-    __shared__ int cursor[kSizeBins];
     const int tid = threadIdx.x;
     if (tid < kSizeBins) hist[tid] = 0;
     __syncthreads();
-    for (int m = tid; m < n_mols; m += kOrderThreads) {
-        const int n = MACs[m];
-        atomicAdd(&hist[kSizeBins - 1 - min(max(n, 0), kSizeBins - 1)], 1);
+    const int m = blockIdx.x * kOrderThreads + tid;
+    if (m < n_mols) atomicAdd(&hist[size_bin(MACs[m])], 1);
+    __syncthreads();
+    if (tid < kSizeBins && hist[tid] > 0) atomicAdd(&ghist[tid], hist[tid]);
+}
+
+__global__ __launch_bounds__(kOrderThreads) void size_place_kernel(const int32_t* __restrict__ MACs, int32_t n_mols,
+                                                                    const int32_t* __restrict__ ghist,
+                                                                    int32_t* __restrict__ gcursor,
+                                                                    int32_t* __restrict__ order)
+{
+    __shared__ int hist[kSizeBins];     // this workgroup's molecules per class, then its cursor inside the range
+    __shared__ int start[kSizeBins];    // first position of the class in the order, then of this workgroup's range
+    const int tid = threadIdx.x;
+    if (tid < kSizeBins) hist[tid] = 0;
+    __syncthreads();
+    const int m = blockIdx.x * kOrderThreads + tid;
+    int bin = 0;
+    if (m < n_mols) {
+        bin = size_bin(MACs[m]);
+        atomicAdd(&hist[bin], 1);
+    }
+    __shared__ int total[kSizeBins];    // molecules per class in the whole batch
+    if (tid < kSizeBins) total[tid] = ghist[tid];
+    __syncthreads();
+    if (tid < kSizeBins) {
+        int run = 0;                    // exclusive prefix: every thread adds up the classes before its own
+        for (int b = 0; b < tid; ++b) run += total[b];
+        start[tid] = run;
     }
     __syncthreads();
-    if (tid == 0) {
-        int run = 0;
-        for (int b = 0; b < kSizeBins; ++b) {
-            cursor[b] = run;
-            run += hist[b];
-        }
+    if (tid < kSizeBins) {
+        const int mine = hist[tid];
+        if (mine > 0) start[tid] += atomicAdd(&gcursor[tid], mine);
+        hist[tid] = 0;
     }
     __syncthreads();
-    for (int m = tid; m < n_mols; m += kOrderThreads) {
-        const int n = MACs[m];
-        order[atomicAdd(&cursor[kSizeBins - 1 - min(max(n, 0), kSizeBins - 1)], 1)] = m;
-    }
+    if (m < n_mols) order[start[bin] + atomicAdd(&hist[bin], 1)] = m;
 }
 }  // namespace
 
-hipError_t launch_size_order(const int32_t* MACs, int32_t n_mols, int32_t* order, hipStream_t stream)
+// `order` holds n_mols entries, `scratch` 2 * 258 entries; both are device memory owned by the caller.
+hipError_t launch_size_order(const int32_t* MACs, int32_t n_mols, int32_t* order, int32_t* scratch, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
-    size_order_kernel<<<dim3(1), dim3(kOrderThreads), 0, stream>>>(MACs, n_mols, order);
+    hipError_t e = hipMemsetAsync(scratch, 0, sizeof(int32_t) * 2 * kSizeBins, stream);
+    if (e != hipSuccess) return e;
+    const unsigned blocks = (static_cast<unsigned>(n_mols) + kOrderThreads - 1) / kOrderThreads;
+    size_hist_kernel<<<dim3(blocks), dim3(kOrderThreads), 0, stream>>>(MACs, n_mols, scratch);
+    size_place_kernel<<<dim3(blocks), dim3(kOrderThreads), 0, stream>>>(MACs, n_mols, scratch, scratch + kSizeBins, order);
     return hipGetLastError();
 }
 
