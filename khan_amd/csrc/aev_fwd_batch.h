@@ -263,24 +263,18 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
     if (total > 0) flush();
 
     // ------------------------------------------------ segments without triples are zeros
-    {
-        const unsigned long long empty = ~nonempty;
-        for (int b = 0; b < nb; ++b) {
-            const unsigned eb = static_cast<unsigned>(empty >> (b * kNumPairBlocks)) & 0x3ffu;
-            if (eb == 0u) continue;
-            const unsigned long long rb = row_of_centre(b);
-            T* row = reinterpret_cast<T*>((static_cast<unsigned long long>(static_cast<unsigned>(uniform(static_cast<int>(rb >> 32)))) << 32) |
-                                                  static_cast<unsigned>(uniform(static_cast<int>(rb & 0xffffffffull)))) + kRadial;
+    // Each segment lane whose segment is empty clears its own 32 values: eight 16-byte stores per lane (or 32
+    // 4-byte ones if the row is not 16-byte aligned), for all centres of the batch at once.
+    if (lane < nb * kNumPairBlocks && cnt == 0) {
+        T* dst = reinterpret_cast<T*>((static_cast<unsigned long long>(seg_row_hi) << 32) | seg_row_lo);
+        if ((seg_row_lo & 15u) == 0u) {
+            constexpr int kPer = 16 / sizeof(T);
 #pragma unroll
-            for (int pp = 0; pp < 5; ++pp) {
-                if (((eb >> (2 * pp)) & 3u) != 0u) {
-                    const int pt = 2 * pp + L.half;
-                    if ((eb >> pt) & 1u) store_global(row + pt * kAngBlock + L.ts, T(0));
-                }
-            }
+            for (int q = 0; q < kAngBlock / kPer; ++q) store_global16(dst + q * kPer);
+        } else {
+            for (int q = 0; q < kAngBlock; ++q) store_global(dst + q, T(0));
         }
     }
-
 }
 
 }  // namespace khan

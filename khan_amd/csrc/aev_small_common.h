@@ -59,6 +59,13 @@ __device__ __forceinline__ void store_global(double* p, double v)
 {
     *((global_double*)(p)) = v;
 }
+// 16 bytes of zeros to a 16-byte aligned global address
+typedef float __attribute__((ext_vector_type(4))) zero_v4f;
+typedef zero_v4f __attribute__((address_space(1))) global_v4f_store;
+__device__ __forceinline__ void store_global16(void* p)
+{
+    *((global_v4f_store*)(p)) = zero_v4f{0.f, 0.f, 0.f, 0.f};
+}
 // sum of the two half-waves, in every lane: swap the upper half of one copy with the lower half of
 // the other (one cross-lane VALU move, no LDS round trip), then add
 __device__ __forceinline__ float half_wave_sum(float v)
