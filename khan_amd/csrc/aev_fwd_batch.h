@@ -32,6 +32,22 @@ struct __align__(16) FwdWaveLds {
     FwdJvpLds<T, kJvp> jvp;
 };
 
+// Padding slots of phase 1 read entry 0 of centre 0's list whatever it holds; their products are cancelled by a
+// zero radial factor, which needs every other factor finite.  Entry 0 is either a partner written by a scan or
+// what this writes once per wavefront before the first batch.
+template <typename T, bool kJvp>
+__device__ __forceinline__ void fwd_lds_init(FwdWaveLds<T, kJvp>& S, int lane)
+{
+    if (lane == 0) {
+        S.nbr[0][0] = Fast<T>::make4(T(0), T(0), T(0), T(0));
+        S.nbr_fc[0][0] = T(0);
+        if constexpr (kJvp) {
+            S.jvp.nbr_p[0][0] = Fast<T>::make4(T(0), T(0), T(0), T(0));
+            S.jvp.nbr_d[0][0] = Fast<T>::make2(T(0), T(0));
+        }
+    }
+}
+
 // Segment table, phases 1 and 2 and the zero fill of empty blocks for centres 0..nb-1 of a batch.
 // `row_of_centre(b)` returns the address of centre b's 384-float output row; it is called by all
 // lanes together, with a per-lane b for the segment table and a wave-uniform b for the zero fill.
@@ -114,17 +130,17 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
         // decode q -> (j,k) inside the centre's type-sorted list
         int bsel = d.packed & 7;
         const int oa = (d.packed >> 3) & 63, ob = (d.packed >> 9) & 63, na = (d.packed >> 15) & 63;
-        // both numberings are decoded and one is selected (no divergent branch).  Same type: pairs jl < kl,
-        // kl-major, q = kl (kl - 1) / 2 + jl; kl = floor((1 + sqrt(8 q + 1)) / 2) is computed with 1.5 under
-        // the root, which keeps the (approximate) hardware square root on the right side of every row
-        // start for q up to several thousand.  Different types: q = kl * n_a + jl.
+        // Different types: q = kl * n_a + jl.  Same type (pairs jl < kl): the rows kl = r + 1 and kl = n_a - r - 1 of the
+        // triangle are laid end to end in one row of length n_a, so the same division serves both numberings:
+        // with (r, col) = divmod(q, n_a), col <= r is the pair (col, r + 1) and col > r the pair (col - r - 1, n_a - r - 1).
         const float qf = static_cast<float>(q);
-        const unsigned kt = static_cast<unsigned>((1.0f + __builtin_amdgcn_sqrtf(fmaf(8.0f, qf, 1.5f))) * 0.5f);
-        const unsigned jt = static_cast<unsigned>(q) - (__umul24(kt, kt - 1u) >> 1);
         const unsigned kr = static_cast<unsigned>((qf + 0.5f) * __builtin_amdgcn_rcpf(static_cast<float>(na)));
         const unsigned jr = static_cast<unsigned>(q) - __umul24(kr, static_cast<unsigned>(na));
-        const bool tri = (d.packed >> 21) & 1;
-        const int kl = static_cast<int>(tri ? kt : kr), jl2 = static_cast<int>(tri ? jt : jr);
+        const unsigned tri = (d.packed >> 21) & 1u;
+        const unsigned k1 = kr + tri;
+        const bool fold = tri && (jr >= k1);
+        const int kl = static_cast<int>(fold ? static_cast<unsigned>(na) - k1 : k1);
+        const int jl2 = static_cast<int>(fold ? jr - k1 : jr);
         int j = oa + jl2, k = ob + kl;
         if (!ok) {
             j = 0;
@@ -163,33 +179,29 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
             }
         }
         const T rho = T(0.5) * (vj.w + vk.w);
-        const T P = T(0.0078125) * fj * fk;
+        // padding slots read entry 0 of centre 0's list (finite, see fwd_lds_init): a zero radial factor,
+        // selected and not multiplied in, cancels their records in phase 2
+        const T P = ok ? T(0.0078125) * fj * fk : T(0);
         T Gf[4], Hf[4];
         T dP = T(0), drho = T(0);
         if constexpr (kJvp) {
             const vec2 dj = S.jvp.nbr_d[bsel][j], dk = S.jvp.nbr_d[bsel][k];
-            dP = T(0.0078125) * (dj.x * fk + fj * dk.x);
+            dP = ok ? T(0.0078125) * (dj.x * fk + fj * dk.x) : T(0);
             drho = T(0.5) * (dj.y + dk.y);
         }
 #pragma unroll
         for (int sidx = 0; sidx < 4; ++sidx) {
             const T dd = rho - static_cast<T>(kA_Rs_f[sidx]);
             const T g = Fast<T>::gauss(static_cast<T>(kA_eta_f), dd);
-            // padding slots read whatever sits in the list: select, do not multiply, so that a
-            // stray NaN cannot reach the sums
-            Gf[sidx] = ok ? g * P : T(0);
-            if constexpr (kJvp) Hf[sidx] = ok ? g * fma(T(-2) * static_cast<T>(kA_eta_f) * dd * drho, P, dP) : T(0);
+            Gf[sidx] = g * P;
+            if constexpr (kJvp) Hf[sidx] = g * fma(T(-2) * static_cast<T>(kA_eta_f) * dd * drho, P, dP);
             else Hf[sidx] = T(0);
         }
-#pragma unroll
-        for (int t = 0; t < 8; ++t) Af[t] = ok ? Af[t] : T(0);
         vec4* recp = reinterpret_cast<vec4*>(S.rec[lane]);
         recp[0] = Fast<T>::make4(Af[0], Af[1], Af[2], Af[3]);
         recp[1] = Fast<T>::make4(Af[4], Af[5], Af[6], Af[7]);
         recp[2] = Fast<T>::make4(Gf[0], Gf[1], Gf[2], Gf[3]);
         if constexpr (kJvp) {
-#pragma unroll
-            for (int t = 0; t < 8; ++t) dAf[t] = ok ? dAf[t] : T(0);
             vec4* rec2p = reinterpret_cast<vec4*>(S.jvp.rec2[lane]);
             rec2p[0] = Fast<T>::make4(dAf[0], dAf[1], dAf[2], dAf[3]);
             rec2p[1] = Fast<T>::make4(dAf[4], dAf[5], dAf[6], dAf[7]);

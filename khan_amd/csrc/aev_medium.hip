@@ -48,6 +48,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
     const float kRadExp = -kR_eta_f * 1.44269504088896340736f;   // exp(-eta d^2) = exp2(kRadExp d^2)
     const int rslot = lane >> 4;                                 // radial walk: entry slot of this 16-lane group
 
+    fwd_lds_init(S, lane);
     __shared__ unsigned long long want[4];
     for_each_molecule_in_range(MACs, n_mols, kMedMin, kMediumMaxAtoms, want, order, [&](int mol) {
         const int n = uniform(MACs[mol]);

@@ -138,6 +138,7 @@ void aev_fwd_small_kernel(
     const int rg_g = G == 4 ? rg : G == 2 ? (rg >> 1) : 0;
     const int rg_s = G == 4 ? 0 : G == 2 ? (rg & 1) : rg;
 
+    fwd_lds_init(S, lane);
     wave_lds_fence();
 
     for (int c0 = 0; c0 < n; c0 += kFB) {
