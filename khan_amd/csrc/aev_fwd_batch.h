@@ -220,6 +220,10 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
             pda = &S.jvp.rec2[L.half][ang_t];
             ph = &S.jvp.rec2[L.half][8 + ang_s];
         }
+        // float: the four lanes of a quad (same theta_t) each read A_t of one of four consecutive pairs, and the
+        // product takes it from the quad lane that holds it: one LDS read of A serves four pairs
+        constexpr bool kQuadA = sizeof(T) == 4 && !kJvp;
+        const T* pa4 = &S.rec[L.half + 2 * ang_s][ang_t];
         unsigned long long mm = starts;
         if (base == 0) {            // the batch's first segment opens here; nothing to close
             cur_lo = static_cast<unsigned>(lane_read(static_cast<int>(d.row_lo), 0));
@@ -230,9 +234,13 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
             T a[8], g[8], da[kJvp ? 8 : 1], h[kJvp ? 8 : 1];
         };
         auto load8 = [&](int q0, Group& v) {
+            if constexpr (kQuadA) {
+                v.a[0] = pa4[q0 * 24];
+                v.a[1] = pa4[(q0 + 4) * 24];
+            }
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
-                v.a[u] = pa[(q0 + u) * 24];
+                if constexpr (!kQuadA) v.a[u] = pa[(q0 + u) * 24];
                 v.g[u] = pg[(q0 + u) * 24];
                 if constexpr (kJvp) {
                     v.da[u] = pda[(q0 + u) * 24];
@@ -255,6 +263,7 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
                     acc = T(0);
                 }
                 if constexpr (kJvp) acc = fma(v.da[u], v.g[u], fma(v.a[u], v.h[u], acc));
+                else if constexpr (kQuadA) acc = fma_quad(v.a[u >> 2], u & 3, v.g[u], acc);
                 else acc = fma(v.a[u], v.g[u], acc);
             }
         };

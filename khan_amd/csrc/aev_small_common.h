@@ -59,6 +59,18 @@ __device__ __forceinline__ void store_global(double* p, double v)
 {
     *((global_double*)(p)) = v;
 }
+// acc + a' * g, where a' is the value of `a` held by lane k of this lane's quad (k is a constant after unrolling).
+// The lane exchange is a modifier of the multiply-add, not an instruction of its own.  `a` must come from
+// memory, not from a vector instruction issued just before (the exchange reads it two cycles early).
+__device__ __forceinline__ float fma_quad(float a, int k, float g, float acc)
+{
+    if (k == 0) asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(acc) : "v"(a), "v"(g));
+    else if (k == 1) asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(acc) : "v"(a), "v"(g));
+    else if (k == 2) asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(acc) : "v"(a), "v"(g));
+    else asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(acc) : "v"(a), "v"(g));
+    return acc;
+}
+__device__ __forceinline__ double fma_quad(double a, int, double g, double acc) { return fma(a, g, acc); }   // float only
 // 16 bytes of zeros to a 16-byte aligned global address
 typedef float __attribute__((ext_vector_type(4))) zero_v4f;
 typedef zero_v4f __attribute__((address_space(1))) global_v4f_store;
