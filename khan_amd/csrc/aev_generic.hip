@@ -28,14 +28,14 @@ __global__ __launch_bounds__(256) void aev_fwd_generic_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs, Buckets<T> out,
-    int min_atoms)
+    int min_atoms, const int32_t* __restrict__ order)
 {
     __shared__ T ang_rows[4][kAngular];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const LaneConsts<T> L = lane_consts<T>(lane);
     T* ang = ang_rows[wave];
     __shared__ unsigned long long want[4];
-    for_each_molecule_in_range(MACs, n_mols, min_atoms, 0x7fffffff, want, nullptr, [&](int mol) {
+    for_each_molecule_in_range(MACs, n_mols, min_atoms, 0x7fffffff, want, order, order ? order + n_mols : nullptr, [&](int mol) {
         const int n = MACs[mol], off = MOs[mol];
         for (int i = wave; i < n; i += 4) {
             T* row = out.p[fold_type(A[off + i])] + static_cast<size_t>(SIs[off + i]) * kFeats;
@@ -51,14 +51,14 @@ __global__ __launch_bounds__(256) void aev_jvp_generic_kernel(
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
     const T* __restrict__ VX, const T* __restrict__ VY, const T* __restrict__ VZ, Buckets<T> out,
-    int min_atoms)
+    int min_atoms, const int32_t* __restrict__ order)
 {
     __shared__ T ang_rows[4][kAngular];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const LaneConsts<T> L = lane_consts<T>(lane);
     T* ang = ang_rows[wave];
     __shared__ unsigned long long want[4];
-    for_each_molecule_in_range(MACs, n_mols, min_atoms, 0x7fffffff, want, nullptr, [&](int mol) {
+    for_each_molecule_in_range(MACs, n_mols, min_atoms, 0x7fffffff, want, order, order ? order + n_mols : nullptr, [&](int mol) {
         const int n = MACs[mol], off = MOs[mol];
         for (int i = wave; i < n; i += 4) {
             T* row = out.p[fold_type(A[off + i])] + static_cast<size_t>(SIs[off + i]) * kFeats;
@@ -73,14 +73,15 @@ __global__ __launch_bounds__(256) void aev_bwd_generic_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
-    Buckets<const T> gin, T* __restrict__ gX, T* __restrict__ gY, T* __restrict__ gZ, int min_atoms)
+    Buckets<const T> gin, T* __restrict__ gX, T* __restrict__ gY, T* __restrict__ gZ, int min_atoms,
+    const int32_t* __restrict__ order)
 {
     __shared__ T g_rows[4][kAngular];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const LaneConsts<T> L = lane_consts<T>(lane);
     T* g_ang = g_rows[wave];
     __shared__ unsigned long long want[4];
-    for_each_molecule_in_range(MACs, n_mols, min_atoms, 0x7fffffff, want, nullptr, [&](int mol) {
+    for_each_molecule_in_range(MACs, n_mols, min_atoms, 0x7fffffff, want, order, order ? order + n_mols : nullptr, [&](int mol) {
         const int n = MACs[mol], off = MOs[mol];
         // every contribution to this molecule's atoms comes from this workgroup: zero them here, then
         // accumulate with atomics (no separate fill pass, nothing to pre-zero for the caller)
@@ -115,10 +116,11 @@ static unsigned generic_grid(int32_t n_mols, int min_atoms)
 template <typename T>
 hipError_t launch_fwd_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
                               const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
-                              const int32_t* SIs, Buckets<T> out, int min_atoms, hipStream_t stream)
+                              const int32_t* SIs, Buckets<T> out, int min_atoms, const int32_t* order,
+                              hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
-    aev_fwd_generic_kernel<T><<<dim3(generic_grid(n_mols, min_atoms)), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, out, min_atoms);
+    aev_fwd_generic_kernel<T><<<dim3(generic_grid(n_mols, min_atoms)), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, out, min_atoms, order);
     return hipGetLastError();
 }
 
@@ -126,10 +128,10 @@ template <typename T>
 hipError_t launch_jvp_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
                               const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
                               const int32_t* SIs, const T* VX, const T* VY, const T* VZ, Buckets<T> out,
-                              int min_atoms, hipStream_t stream)
+                              int min_atoms, const int32_t* order, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
-    aev_jvp_generic_kernel<T><<<dim3(generic_grid(n_mols, min_atoms)), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, VX, VY, VZ, out, min_atoms);
+    aev_jvp_generic_kernel<T><<<dim3(generic_grid(n_mols, min_atoms)), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, VX, VY, VZ, out, min_atoms, order);
     return hipGetLastError();
 }
 
@@ -137,21 +139,21 @@ template <typename T>
 hipError_t launch_bwd_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
                               const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
                               const int32_t* SIs, Buckets<const T> g, T* gX, T* gY, T* gZ,
-                              int64_t n_atoms, int min_atoms, hipStream_t stream)
+                              int64_t n_atoms, int min_atoms, const int32_t* order, hipStream_t stream)
 {
     // the kernel zeroes each molecule's outputs itself before accumulating (the reference zero-fills
     // first, functor_op_cpu.cpp:70-72); no memset node, so the launch is safe to capture in a HIP graph
     (void)n_atoms;
     if (n_mols <= 0) return hipSuccess;
-    aev_bwd_generic_kernel<T><<<dim3(generic_grid(n_mols, min_atoms)), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ, min_atoms);
+    aev_bwd_generic_kernel<T><<<dim3(generic_grid(n_mols, min_atoms)), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ, min_atoms, order);
     return hipGetLastError();
 }
 
-template hipError_t launch_fwd_generic<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<float>, int, hipStream_t);
-template hipError_t launch_fwd_generic<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<double>, int, hipStream_t);
-template hipError_t launch_jvp_generic<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const float*, const float*, const float*, Buckets<float>, int, hipStream_t);
-template hipError_t launch_jvp_generic<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const double*, const double*, const double*, Buckets<double>, int, hipStream_t);
-template hipError_t launch_bwd_generic<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const float>, float*, float*, float*, int64_t, int, hipStream_t);
-template hipError_t launch_bwd_generic<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const double>, double*, double*, double*, int64_t, int, hipStream_t);
+template hipError_t launch_fwd_generic<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<float>, int, const int32_t*, hipStream_t);
+template hipError_t launch_fwd_generic<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<double>, int, const int32_t*, hipStream_t);
+template hipError_t launch_jvp_generic<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const float*, const float*, const float*, Buckets<float>, int, const int32_t*, hipStream_t);
+template hipError_t launch_jvp_generic<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const double*, const double*, const double*, Buckets<double>, int, const int32_t*, hipStream_t);
+template hipError_t launch_bwd_generic<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const float>, float*, float*, float*, int64_t, int, const int32_t*, hipStream_t);
+template hipError_t launch_bwd_generic<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const double>, double*, double*, double*, int64_t, int, const int32_t*, hipStream_t);
 
 }  // namespace khan

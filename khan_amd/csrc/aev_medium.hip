@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
 
     fwd_lds_init(S, lane);
     __shared__ unsigned long long want[4];
-    for_each_molecule_in_range(MACs, n_mols, kMedMin, kMediumMaxAtoms, want, order, [&](int mol) {
+    for_each_molecule_in_range(MACs, n_mols, kMedMin, kMediumMaxAtoms, want, order, order ? order + n_mols : nullptr, [&](int mol) {
         const int n = uniform(MACs[mol]);
         const int off = uniform(MOs[mol]);
 

@@ -38,7 +38,7 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
     Buckets<const float> gin, float* __restrict__ gX, float* __restrict__ gY, float* __restrict__ gZ,
-    const int32_t* __restrict__ order)
+    const int32_t* __restrict__ order, bool walk_in_order)
 {
     __shared__ MedBwdShared M;
     __shared__ BwdPool<float> pools[4];
@@ -50,7 +50,8 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
 
     __shared__ unsigned long long want[4];
-    for_each_molecule_in_range(MACs, n_mols, kMedMin, kMediumMaxAtoms, want, order, [&](int mol) {
+    for_each_molecule_in_range(MACs, n_mols, kMedMin, kMediumMaxAtoms, want, walk_in_order ? order : nullptr,
+                               order ? order + n_mols : nullptr, [&](int mol) {
         const int n = uniform(MACs[mol]);
         const int off = uniform(MOs[mol]);
 
@@ -318,12 +319,12 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
 hipError_t launch_bwd_medium_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
                                  const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
                                  const int32_t* SIs, Buckets<const float> g, float* gX, float* gY,
-                                 float* gZ, const int32_t* order, hipStream_t stream)
+                                 float* gZ, const int32_t* order, bool walk_in_order, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
     // workgroups walk the molecules with the grid's stride and skip those of other sizes
     const unsigned blocks = static_cast<unsigned>(n_mols < 4096 ? n_mols : 4096);
-    aev_bwd_medium_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ, order);
+    aev_bwd_medium_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ, order, walk_in_order);
     return hipGetLastError();
 }
 

@@ -56,7 +56,7 @@ public:
             order_ = nullptr;
             return;
         }
-        if (khan::launch_size_order(macs, n_mols, order_, order_ + n_mols, stream) != hipSuccess) {
+        if (khan::launch_size_order(macs, n_mols, order_, stream) != hipSuccess) {
             (void)hipGetLastError();
             (void)hipFreeAsync(order_, stream);
             order_ = nullptr;
@@ -80,7 +80,7 @@ int forward_dispatch(const float* xs, const float* ys, const float* zs, const in
                      khan::Buckets<float> out, hipStream_t stream)
 {
     if (force_generic())
-        return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, stream));
+        return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, nullptr, stream));
     // molecules of up to 32 atoms: one wavefront each; up to 256: one workgroup each; the rest: general kernel
     SizeOrder order(macs, n_mols, stream);
     int st = hip_status(khan::launch_fwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallPreferredMax,
@@ -89,7 +89,7 @@ int forward_dispatch(const float* xs, const float* ys, const float* zs, const in
     st = hip_status(khan::launch_fwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, out, order.get(), stream));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
-                                                      khan::kMediumMaxAtoms + 1, stream));
+                                                      khan::kMediumMaxAtoms + 1, order.get(), stream));
 }
 
 int forward_dispatch(const double* xs, const double* ys, const double* zs, const int32_t* as,
@@ -97,13 +97,13 @@ int forward_dispatch(const double* xs, const double* ys, const double* zs, const
                      khan::Buckets<double> out, hipStream_t stream)
 {
     if (force_generic())
-        return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, stream));
+        return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, nullptr, stream));
     SizeOrder order(macs, n_mols, stream);
     int st = hip_status(khan::launch_fwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallMaxAtoms,
                                                        order.get(), stream));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
-                                                       khan::kSmallMaxAtoms + 1, stream));
+                                                       khan::kSmallMaxAtoms + 1, order.get(), stream));
 }
 
 int backward_dispatch(const float* xs, const float* ys, const float* zs, const int32_t* as,
@@ -115,15 +115,16 @@ int backward_dispatch(const float* xs, const float* ys, const float* zs, const i
     // (rows are 1,536 bytes, so the bucket's base decides) go through the general kernel, which does not care
     if (force_generic() || !aligned16(g))
         return hip_status(khan::launch_bwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                          n_atoms, 0, stream));
+                                                          n_atoms, 0, nullptr, stream));
     // by molecule size: above 256 atoms the general kernel, 33..256 one workgroup per molecule, up to 32
     // one wavefront per molecule; each kernel defines every gradient of its own molecules
-    int st = hip_status(khan::launch_bwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                        n_atoms, khan::kMediumMaxAtoms + 1, stream));
-    if (st != KHAN_OK) return st;
     SizeOrder order(macs, n_mols, stream);
-    // (the workgroup-per-molecule backward kernel measures slower when it is given the size order)
-    st = hip_status(khan::launch_bwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, nullptr, stream));
+    int st = hip_status(khan::launch_bwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                        n_atoms, khan::kMediumMaxAtoms + 1, order.get(), stream));
+    if (st != KHAN_OK) return st;
+    // (the workgroup-per-molecule backward kernel measures slower when it walks the molecules in size order)
+    st = hip_status(khan::launch_bwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, order.get(), false,
+                                                stream));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_bwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
                                                     khan::kSmallPreferredMax, order.get(), stream));
@@ -136,11 +137,11 @@ int backward_dispatch(const double* xs, const double* ys, const double* zs, cons
 {
     if (force_generic() || !aligned16(g))
         return hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                           n_atoms, 0, stream));
-    int st = hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                         n_atoms, khan::kSmallMaxAtoms + 1, stream));
-    if (st != KHAN_OK) return st;
+                                                           n_atoms, 0, nullptr, stream));
     SizeOrder order(macs, n_mols, stream);
+    int st = hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                         n_atoms, khan::kSmallMaxAtoms + 1, order.get(), stream));
+    if (st != KHAN_OK) return st;
     return hip_status(khan::launch_bwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
                                                      khan::kSmallMaxAtoms, order.get(), stream));
 }
@@ -198,14 +199,14 @@ int featurize_grad_inverse_impl(const T* xs, const T* ys, const T* zs, const int
     khan::Buckets<T> out{{h, c, n, o}};
     if (force_generic())
         return hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, 0,
-                                                      as_stream(stream)));
+                                                      nullptr, as_stream(stream)));
     // molecules of up to 64 atoms: one wavefront each; the rest: general-shape kernel
     SizeOrder order(macs, n_mols, as_stream(stream));
     int st = hip_status(khan::launch_jvp_small<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, order.get(),
                                                   as_stream(stream)));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
-                                                  khan::kSmallMaxAtoms + 1, as_stream(stream)));
+                                                  khan::kSmallMaxAtoms + 1, order.get(), as_stream(stream)));
 }
 
 template <typename T>

@@ -15,14 +15,15 @@ struct Buckets {
 template <typename T>
 hipError_t launch_fwd_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
                               const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
-                              const int32_t* SIs, Buckets<T> out, int min_atoms, hipStream_t stream);
+                              const int32_t* SIs, Buckets<T> out, int min_atoms, const int32_t* order,
+                              hipStream_t stream);
 
 // Jacobian applied to per-atom vectors (VX, VY, VZ): one 384-wide row per atom, laid out like the forward's
 template <typename T>
 hipError_t launch_jvp_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
                               const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
                               const int32_t* SIs, const T* VX, const T* VY, const T* VZ, Buckets<T> out,
-                              int min_atoms, hipStream_t stream);
+                              int min_atoms, const int32_t* order, hipStream_t stream);
 
 // ---- AEV forward for molecules of up to 64 atoms (larger molecules are skipped) ----
 constexpr int kSmallMaxAtoms = 64;      // what one wavefront can hold
@@ -48,13 +49,13 @@ hipError_t launch_fwd_medium_f32(const float* X, const float* Y, const float* Z,
 hipError_t launch_bwd_medium_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
                                  const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
                                  const int32_t* SIs, Buckets<const float> g, float* gX, float* gY,
-                                 float* gZ, const int32_t* order, hipStream_t stream);
+                                 float* gZ, const int32_t* order, bool walk_in_order, hipStream_t stream);
 
 template <typename T>
 hipError_t launch_bwd_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
                               const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
                               const int32_t* SIs, Buckets<const T> g, T* gX, T* gY, T* gZ,
-                              int64_t n_atoms, int min_atoms, hipStream_t stream);
+                              int64_t n_atoms, int min_atoms, const int32_t* order, hipStream_t stream);
 template <typename T>
 hipError_t launch_bwd_small(const T* X, const T* Y, const T* Z, const int32_t* A, const int32_t* MOs,
                             const int32_t* MACs, int32_t n_mols, const int32_t* SIs, Buckets<const T> g,
@@ -66,10 +67,19 @@ hipError_t launch_mol_offsets(const int32_t* mol_idxs, int64_t n_atoms, int32_t 
 hipError_t launch_ani_sort(const int32_t* A, int64_t n_atoms, int32_t* scatter, int32_t* gather,
                            int32_t* counts4, hipStream_t stream);
 
-// molecule indices by decreasing atom count; `scratch` is kSizeOrderScratch ints (not for use under graph capture:
-// it is cleared with a memset)
-constexpr int kSizeOrderScratch = 2 * 258;
-hipError_t launch_size_order(const int32_t* MACs, int32_t n_mols, int32_t* order, int32_t* scratch, hipStream_t stream);
+// Molecule indices by decreasing atom count.  `order` holds n_mols + kSizeOrderScratch ints: the indices, then the
+// number of molecules per size class (kSizeBins entries, class = size_bin(atom count)), then the pass's cursors.
+// Every `order` argument of the launchers above is such an array (or null): the kernels for larger molecules read
+// the class counts behind the indices to leave at once when the batch holds no molecule for them.
+// Not for use under graph capture: the counts are cleared with a memset.
+constexpr int kSizeBins = 258;    // atom counts 0..256 and "more", largest first
+constexpr int kSizeOrderScratch = 2 * kSizeBins;
+__host__ __device__ __forceinline__ int size_bin(int n)
+{
+    const int c = n < 0 ? 0 : n > kSizeBins - 1 ? kSizeBins - 1 : n;
+    return kSizeBins - 1 - c;
+}
+hipError_t launch_size_order(const int32_t* MACs, int32_t n_mols, int32_t* order, hipStream_t stream);
 
 // ---- charges ----
 template <typename T>
@@ -110,13 +120,20 @@ __device__ __forceinline__ void wave_lds_fence()
 // all threads then visit the selected molecules together (body may use __syncthreads).  A launch in
 // which (nearly) every molecule belongs to another kernel therefore costs one load per thread, not a
 // dependent load per molecule.  `want` is shared memory, one word per wavefront of the workgroup.  With
-// `order` (molecule indices by decreasing size) the molecules are visited in that order.
+// `order` (molecule indices by decreasing size) the molecules are visited in that order; with `size_counts`
+// (molecules per size class) a workgroup first checks that the batch holds a molecule in range.
 template <typename Body>
 __device__ __forceinline__ void for_each_molecule_in_range(const int32_t* __restrict__ MACs, int32_t n_mols,
                                                            int lo, int hi, unsigned long long* want,
-                                                           const int32_t* __restrict__ order, Body body)
+                                                           const int32_t* __restrict__ order,
+                                                           const int32_t* __restrict__ size_counts, Body body)
 {
     const int tid = threadIdx.x, nthreads = blockDim.x, nwaves = nthreads >> 6;
+    if (size_counts) {          // molecules per size class: is there anything in [lo, hi] at all?
+        int any = 0;
+        for (int b = size_bin(hi) + tid; b <= size_bin(lo); b += nthreads) any |= size_counts[b];
+        if (!__syncthreads_or(any)) return;
+    }
     for (long long base = blockIdx.x; base < n_mols; base += static_cast<long long>(gridDim.x) * nthreads) {
         const long long m = base + static_cast<long long>(tid) * gridDim.x;
         bool wanted = false;

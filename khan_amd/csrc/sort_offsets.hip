@@ -238,10 +238,7 @@ hipError_t launch_ani_sort(const int32_t* A, int64_t n_atoms, int32_t* scatter, 
 // workgroups in index order, so the expensive molecules start first and a launch does not end on a few
 // long waves.
 namespace {
-constexpr int kSizeBins = 258;    // atom counts 0..256 and "more"
 constexpr int kOrderThreads = 1024;
-
-__device__ __forceinline__ int size_bin(int n) { return kSizeBins - 1 - min(max(n, 0), kSizeBins - 1); }
 
 __global__ __launch_bounds__(kOrderThreads) void size_hist_kernel(const int32_t* __restrict__ MACs, int32_t n_mols,
                                                                    int32_t* __restrict__ ghist)
@@ -291,10 +288,12 @@ __global__ __launch_bounds__(kOrderThreads) void size_place_kernel(const int32_t
 }
 }  // namespace
 
-// `order` holds n_mols entries, `scratch` 2 * 258 entries; both are device memory owned by the caller.
-hipError_t launch_size_order(const int32_t* MACs, int32_t n_mols, int32_t* order, int32_t* scratch, hipStream_t stream)
+// `order` holds n_mols + kSizeOrderScratch entries of device memory owned by the caller: the indices, the class
+// counts, the cursors.
+hipError_t launch_size_order(const int32_t* MACs, int32_t n_mols, int32_t* order, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
+    int32_t* scratch = order + n_mols;
     hipError_t e = hipMemsetAsync(scratch, 0, sizeof(int32_t) * 2 * kSizeBins, stream);
     if (e != hipSuccess) return e;
     const unsigned blocks = (static_cast<unsigned>(n_mols) + kOrderThreads - 1) / kOrderThreads;
