@@ -27,6 +27,10 @@ namespace khan {
 
 namespace {
 
+// radial list entries a lane takes per trip: each type's entries are padded to a multiple of this (times the
+// number of slots), and two measured faster than one, three or four
+constexpr int kRadTrip = 2;
+
 // float: 4 wavefronts per SIMD (LDS 9.8 KB, <= 128 VGPRs); double: 2 (LDS 19.6 KB)
 // With kJvp the kernel computes the Jacobian-vector product instead (featurize_grad_inverse): every term of
 // the forward sums is replaced by its derivative along the per-atom vectors (VX, VY, VZ).
@@ -226,17 +230,17 @@ void aev_fwd_small_kernel(
                 for (int a = 0; a < 4; ++a) {
                     const int cnt_a = a == 0 ? cn.x : a == 1 ? cn.y : a == 2 ? cn.z : cn.w;
                     T acc_r = T(0);
-                    for (int q0 = 0; q0 < mxR[a]; q0 += 4 * rg_ns) {
-                        // four entries of this lane's slot per trip; slot s takes q = s, s+ns, s+2ns, ...
-                        vec2 e[4], ab[4];
+                    for (int q0 = 0; q0 < mxR[a]; q0 += kRadTrip * rg_ns) {
+                        // kRadTrip entries of this lane's slot per trip; slot s takes q = s, s+ns, s+2ns, ...
+                        vec2 e[kRadTrip], ab[kRadTrip];
 #pragma unroll
-                        for (int u = 0; u < 4; ++u) {
+                        for (int u = 0; u < kRadTrip; ++u) {
                             const int at = min(obase + q0 + u * rg_ns + rg_s, W - 1);
                             e[u] = list[at];
                             if constexpr (kJvp) ab[u] = S.jvp.rad_ab[rg_g * W + at];
                         }
 #pragma unroll
-                        for (int u = 0; u < 4; ++u) {
+                        for (int u = 0; u < kRadTrip; ++u) {
                             const T dd = e[u].x - L.rrs;
                             // forward: exp(-eta d^2) f_C; derivative: exp(-eta d^2) (f_C' - 2 eta d f_C) dr
                             T v = Fast<T>::gauss(static_cast<T>(kR_eta_f), dd);
