@@ -185,7 +185,8 @@ template <typename T, typename AddForce>
 __device__ __forceinline__ void bwd_center_generic(const LaneConsts<T>& L, int lane, const T* __restrict__ X,
                                                    const T* __restrict__ Y, const T* __restrict__ Z,
                                                    const int32_t* __restrict__ A, int off, int n, int i,
-                                                   T* g_ang, const T* __restrict__ grow, AddForce add)
+                                                   T* g_ang, const T* __restrict__ grow, AddForce add,
+                                                   bool with_radial = true)
 {
         const T g_rad = grow[lane];                       // upstream for slot (rtype, shell)
         for (int q = lane; q < kAngular; q += 64) g_ang[q] = grow[kRadial + q];
@@ -205,7 +206,8 @@ __device__ __forceinline__ void bwd_center_generic(const LaneConsts<T>& L, int l
             const T dfcA = inA ? cutoff_dfn(pj.r, L.pi_rc_A) : T(0);
 
             // radial: dE/dr_ij = sum_shells g * exp(-eta d^2) * (f_C' - 2 eta d f_C)
-            for (unsigned long long m = wave_ballot(inR); m; m &= m - 1) {
+            // (a caller that has already done the centre's radial pairs passes with_radial = false)
+            for (unsigned long long m = with_radial ? wave_ballot(inR) : 0ull; m; m &= m - 1) {
                 const int b = lowest_bit(m);
                 const Partner<T> J = partner_from_lane(pj, b);
                 const T fb = wave_get(fcR, b), dfb = wave_get(dfcR, b);

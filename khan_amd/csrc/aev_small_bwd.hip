@@ -1,16 +1,16 @@
 // AEV backward (dL/dxyz) for molecules of up to 64 atoms, float32 and float64: one wavefront per molecule.
 //
-// Lanes are sorted by atom type as in the forward kernel.  A first sweep counts the angular partners
-// of every atom; centres are then taken in order of decreasing count, in batches of up to six whose
-// partner lists together fill at most the 64 lanes.  Per batch:
+// Lanes are sorted by atom type as in the forward kernel.  A first sweep over the (centre, partner) pairs,
+// 64 per step, counts the angular partners of every atom and does the radial part: a lane owns one pair,
+// reads the 16 upstream values of the partner's type from the centre's row, sums g e (f_C' - 2 eta d f_C)
+// over the shells, and the pull goes to the partner (one group of lanes at a time, so targets are
+// distinct) and, summed over the group with DPP moves, to the centre.  Centres are then taken in order
+// of decreasing partner count, in batches of up to six whose partner lists together fill at most the 64
+// lanes.  Per batch:
 //   stage    the 320 angular upstream values of each centre's row are fetched with full-line loads
 //            (issued before the scan, so their latency is covered) and laid out in LDS by type pair;
 //   scan     64 (centre, partner) pairs per step; angular partners (unit vector, distance, f_C, f_C')
 //            go to one pooled list, centre after centre;
-//   radial   a lane owns one (centre, partner) pair: it reads the 16 upstream values of the partner's
-//            type from the centre's row, sums g e (f_C' - 2 eta d f_C) over the shells, and the pull
-//            goes to the partner (one group at a time, so targets are distinct) and, summed over the
-//            group with DPP moves, to the centre;
 //   angular  lane = one list entry (centre b, partner j).  It walks the other partners of the same
 //            centre in round-robin order, k = j+1, j+2, ... (mod m): in every round all lanes of a
 //            centre hold distinct j AND distinct k, each unordered pair {j,k} is met exactly once.
@@ -136,10 +136,40 @@ void aev_bwd_small_kernel(
             const vec4 ai = S.atom[min(i, 63)];
             const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
             const T r = sqrt(dx * dx + dy * dy + dz * dz);
-            const bool inA = (i < n) && (jl < n) && (jl != i) && (r < kA_Rc_f);
+            const bool valid = (i < n) && (jl < n) && (jl != i);
+            const bool inA = valid && (r < kA_Rc_f);
             const int cnt = popc64(wave_ballot(inA) & sub_mask);          // in every lane of the group
             const int got = __builtin_amdgcn_ds_bpermute((((lane - s0) << logW) & 63) << 2, cnt);
             if (lane >= s0 && lane < s0 + G) m_mine = got;
+
+            // ---- radial pairs: this lane's (centre, partner) pair over its 16 shells.  Done here, where the
+            // centres come G at a time in lane order, and not per batch, whose last step is rarely full.
+            const T* grow = row_of_lane(min(i, 63));
+            T cfx = T(0), cfy = T(0), cfz = T(0);       // this pair's pull on the centre
+            const bool inR = valid && (r < kR_Rc_f);
+            if (inR) {
+                const T sc = bwd_radial_pair<T>(grow, static_cast<int>(aj.w), r, Fast<T>::rcp(r));   // dE/dr / r
+                cfx = sc * dx;
+                cfy = sc * dy;
+                cfz = sc * dz;
+            }
+            // partner forces: one group per round, so the targets of a round are distinct atoms
+            for (int g = 0; g < G; ++g) {
+                if (inR && grp == g) {
+                    S.force[0][jl] -= cfx;
+                    S.force[1][jl] -= cfy;
+                    S.force[2][jl] -= cfz;
+                }
+            }
+            // the W lanes of a group share their centre: sum inside the group, its last lane adds
+            cfx = group_sum_to_last_lane(cfx, logW);
+            cfy = group_sum_to_last_lane(cfy, logW);
+            cfz = group_sum_to_last_lane(cfz, logW);
+            if (jl == W - 1 && i < n) {
+                S.force[0][i] += cfx;
+                S.force[1][i] += cfy;
+                S.force[2][i] += cfz;
+            }
         }
         const int key = have ? ((m_mine << 6) | (63 - lane)) : -1;
         int rank = 0;
@@ -197,7 +227,6 @@ void aev_bwd_small_kernel(
             const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
             const T r = sqrt(dx * dx + dy * dy + dz * dz);
             const bool valid = centre_ok && (jl < n) && (jl != i);
-            const bool inR = valid && (r < kR_Rc_f);
             const bool inA = valid && (r < kA_Rc_f);
             const unsigned long long mA = wave_ballot(inA);
             const int cntA = popc64(mA & sub_mask);
@@ -216,34 +245,6 @@ void aev_bwd_small_kernel(
                 const unsigned long long ov = wave_ballot(!fits && jl == 0 && centre_ok);
                 for (int g = 0; g < G; ++g)
                     if ((ov >> (g * W)) & 1ull) overflow |= 1u << (b0 + g);
-            }
-
-            // ---- radial pairs: this lane's (centre, partner) pair over its 16 shells
-            const T* grow = row_of_lane(i);
-            T cfx = T(0), cfy = T(0), cfz = T(0);       // this pair's pull on the centre
-            const bool do_rad = inR && fits;              // a centre that does not fit is redone as a whole
-            if (do_rad) {
-                const T sc = bwd_radial_pair<T>(grow, static_cast<int>(aj.w), r, inv);   // dE/dr / r, multiplies (x_i - x_j)
-                cfx = sc * dx;
-                cfy = sc * dy;
-                cfz = sc * dz;
-            }
-            // partner forces: one group per round, so the targets of a round are distinct atoms
-            for (int g = 0; g < G; ++g) {
-                if (do_rad && grp == g) {
-                    S.force[0][jl] -= cfx;
-                    S.force[1][jl] -= cfy;
-                    S.force[2][jl] -= cfz;
-                }
-            }
-            // the W lanes of a group share their centre: sum inside the group, its last lane adds
-            cfx = group_sum_to_last_lane(cfx, logW);
-            cfy = group_sum_to_last_lane(cfy, logW);
-            cfz = group_sum_to_last_lane(cfz, logW);
-            if (jl == W - 1 && centre_ok) {
-                S.force[0][i] += cfx;
-                S.force[1][i] += cfy;
-                S.force[2][i] += cfz;
             }
         }
 
@@ -297,7 +298,8 @@ void aev_bwd_small_kernel(
                                                   atomicAdd(&S.force[0][sl], fx);
                                                   atomicAdd(&S.force[1][sl], fy);
                                                   atomicAdd(&S.force[2][sl], fz);
-                                              });
+                                              },
+                                              false);        // the radial pairs were done in the first sweep
                 }
             }
             wave_lds_fence();
