@@ -37,6 +37,9 @@ WORKLOADS = {
     "organic1024": ("organic", 1024, 4, False),
     "organic16384_f64": ("organic", 16384, 8, True),     # double precision forward + backward + ani_charge
     "boxes4096": ("boxes", 4096, 4, False),              # dense boxes of 64..256 atoms
+    # not a line of the headline metric: energies and coordinate gradients through the atomic networks
+    # (384-128-128-64-1 per type, random weights), the caller either side of the hot path
+    "inference65536": ("organic", 65536, 4, False),
 }
 
 
@@ -125,6 +128,49 @@ def cpu_baseline(batch, sample_mols_fwd, sample_mols_bwd, w=4):
     }
 
 
+def inference_bench(args, batch):
+    """Energy + coordinate-gradient inference: featurize -> per-type networks (rocBLAS products) -> segment sum,
+    then back through the networks and featurize_grad.  One JSON line; the roofline object describes the step's
+    dense layers, which dominate it (their flops against the fp32 matrix peak)."""
+    import numpy as np
+    import torch
+    from khan_amd import model, ops
+    from khan_amd.batching import DeviceBatch
+    dev = torch.device("cuda:0")
+    N, n_mols = batch.n_atoms, batch.n_mols
+    b = DeviceBatch()
+    b.xs, b.ys, b.zs = (torch.from_numpy(v).to(dev) for v in (batch.X, batch.Y, batch.Z))
+    b.atom_types = torch.from_numpy(batch.A).to(dev)
+    b.mol_idxs = torch.from_numpy(batch.mol_idxs).to(dev)
+    b.n_mols = n_mols
+    b.mol_atom_counts, b.mol_offsets = ops.mol_offsets(b.mol_idxs, n_mols)
+    b.scatter_idxs, b.gather_idxs, b.atom_counts = ops.ani_sort(b.atom_types)
+    m = model.AniModel(model.DEFAULT_LAYERS, model.celu, torch.float32, dev, seed=1)
+    for _ in range(args.warmup):
+        m.batch_energies(b, need_grad=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        e, g = m.batch_energies(b, need_grad=True)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    sizes = (384,) + tuple(model.DEFAULT_LAYERS)
+    macs_per_atom = sum(x * y for x, y in zip(sizes[:-1], sizes[1:]))
+    gemm_flops = 2 * macs_per_atom * N * 2            # forward, and the data gradient on the way back
+    print(json.dumps({
+        "metric": "ANI-1 energy + coordinate-gradient inference atoms/sec, fp32, 1 MI355X",
+        "value": N / (ms_per_step * 1e-3), "unit": "atoms/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "inference65536: featurize + 4 atomic networks 384-128-128-64-1 (random weights) + "
+                               "segment sum, gradient back to the coordinates; %d molecules, %d atoms" % (n_mols, N)},
+        "molecules_per_s": n_mols / (ms_per_step * 1e-3),
+        "roofline": {"kernel": "dense layers (rocBLAS)", "bound": "mfma", "achieved": gemm_flops / (ms_per_step * 1e-3) / 1e12,
+                     "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": gemm_flops / (ms_per_step * 1e-3) / 1e12 / FP32_PEAK_TFLOPS, "traffic": None},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -151,6 +197,8 @@ def main():
     kind, n_mols, w, with_charges = WORKLOADS[args.workload]
     tdt = torch.float32 if w == 4 else torch.float64
     batch = datagen.make_batch(kind, n_mols)
+    if args.workload.startswith("inference"):
+        return inference_bench(args, batch)
     N = batch.n_atoms
     counts = batch.work_counts()
     work = algorithmic_work(counts, N, n_mols, w)

@@ -24,7 +24,10 @@ FEATURE_SIZE = 384
 
 # ------------------------------------------------------------------ activation functions (activations.py:63-77)
 def celu(a, alpha=0.1):
-    # a for a >= 0, alpha (exp(a / alpha) - 1) below
+    # a for a >= 0, alpha (exp(a / alpha) - 1) below.  float32: PyTorch's celu, one elementwise kernel forward and
+    # one backward.  float64: spelled out, because that kernel's backward rounds alpha to float (1e-8 off).
+    if a.dtype == torch.float32:
+        return torch.nn.functional.celu(a, alpha)
     return torch.where(a >= 0, a, alpha * torch.expm1(torch.clamp(a, max=0.0) / alpha))
 
 

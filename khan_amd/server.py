@@ -88,13 +88,10 @@ def close_connection(s):
     s.close()
 
 
-def serve(model, host, port, max_connections=None, ready=None):
-    """Accepts connections one at a time and answers requests until the peer closes (energy_server.py:137-190).
-    `max_connections` ends the loop after that many connections (None: forever); `ready`, a threading.Event,
-    is set once the socket listens."""
-    s = connect_socket(host, port, server=True)
-    if ready is not None:
-        ready.set()
+def serve_on(s, model, max_connections=None):
+    """Accepts connections on the listening socket `s` one at a time and answers requests until the peer closes
+    (energy_server.py:137-190).  `max_connections` ends the loop after that many connections (None: forever).
+    Closes `s` on the way out."""
     served = 0
     try:
         while max_connections is None or served < max_connections:
@@ -114,6 +111,10 @@ def serve(model, host, port, max_connections=None, ready=None):
             served += 1
     finally:
         s.close()
+
+
+def serve(model, host, port, max_connections=None):
+    serve_on(connect_socket(host, port, server=True), model, max_connections)
 
 
 def main(argv=None):

@@ -237,11 +237,10 @@ def test_gradient_is_the_derivative_of_the_energy():
 def test_energy_server_round_trip_over_a_socket():
     b, mols = _molecules(n_mols=2, first=11)
     m = _gpu_model(torch.float64, seed=5)
-    ready = threading.Event()
-    port = 50000 + (hash("khan") % 997)
-    th = threading.Thread(target=server.serve, args=(m, "127.0.0.1", port, 1, ready), daemon=True)
+    listening = server.connect_socket("127.0.0.1", 0, server=True)        # port 0: the system picks a free one
+    port = listening.getsockname()[1]
+    th = threading.Thread(target=server.serve_on, args=(listening, m, 1), daemon=True)
     th.start()
-    assert ready.wait(30)
     c = server.connect_socket("127.0.0.1", port, server=False)
     try:
         for k, X in enumerate(mols):
