@@ -55,6 +55,38 @@ __device__ __forceinline__ T bwd_radial_pair(const T* grow, int tj, T r, T inv)
     return Gsum * inv;           // dE/dr / r
 }
 
+// Both directions of a pair at once: centre c with partner j reads row c's block for j's type, centre j with
+// partner c reads row j's block for c's type, and the two share r and with it every shell factor.  The result
+// times (x_c - x_j) is the whole radial force on c from this pair, so that nothing has to be added to j: j
+// receives the same when it is the centre.
+template <typename T>
+__device__ __forceinline__ T bwd_radial_pair_both(const T* grow_c, int tj, const T* grow_j, int tc, T r, T inv)
+{
+    constexpr int kPieces = 16 * sizeof(T) / 16;
+    union {
+        v4f piece[kPieces];
+        T gr[16];
+    } u, w;
+    const global_v4f_ptr gp = (global_v4f_ptr)(grow_c + tj * kNumRRs);
+    const global_v4f_ptr gq = (global_v4f_ptr)(grow_j + tc * kNumRRs);
+#pragma unroll
+    for (int q = 0; q < kPieces; ++q) {
+        u.piece[q] = gp[q];
+        w.piece[q] = gq[q];
+    }
+    T fc, dfc;
+    Fast<T>::cutoff_grad(r, static_cast<T>(kR_Rc_f), fc, dfc);
+    const T m2eta_fc = T(-2) * static_cast<T>(kR_eta_f) * fc;
+    T Gsum = T(0);
+#pragma unroll
+    for (int q = 0; q < kNumRRs; ++q) {
+        const T d = r - static_cast<T>(kR_Rs_f[q]);
+        const T e = Fast<T>::gauss(static_cast<T>(kR_eta_f), d);
+        Gsum = fma((u.gr[q] + w.gr[q]) * e, fma(m2eta_fc, d, dfc), Gsum);
+    }
+    return Gsum * inv;
+}
+
 // The angular part of an upstream row is 320 elements = kRowPieces 16-byte pieces; a wavefront fetches it
 // with kPieceRegs loads per lane (piece r * 64 + lane).
 template <typename T> struct RowStage {

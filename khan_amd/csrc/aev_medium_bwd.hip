@@ -5,8 +5,11 @@
 // then draw centres from a shared counter.  A wavefront collects centres into a batch while their
 // angular partner lists fit the 64 entries of its pool (at most six), and for each centre it takes in:
 //   scan + radial   the centre is tested against the sorted atoms 64 at a time; pairs inside the radial
-//                   cutoff are queued, and whenever 64 are waiting a lane takes one pair, sums
-//                   g e (f_C' - 2 eta d f_C) over the 16 shells, and adds the pull to partner and centre;
+//                   cutoff are queued, and whenever 64 are waiting a lane takes one pair and sums
+//                   g e (f_C' - 2 eta d f_C) over the 16 shells for both directions of the pair (the centre's
+//                   row and the partner's row share every shell factor): that is the pair's whole pull on the
+//                   centre, and nothing is added to the partner, which gets the same as a centre itself
+//                   (per-pair atomic adds to the partners cost a quarter of the kernel);
 // then for the batch:
 //   stage           the 320 angular upstream values of each centre's row go to LDS by type pair;
 //   angular         the round-robin walk shared with the small-molecule kernel: lane = list entry,
@@ -125,13 +128,14 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                 const float4 e = q_d[lane];
                 const int j = q_j[lane];
                 c = q_c[lane];
-                const float* grow = reinterpret_cast<const float*>((static_cast<unsigned long long>(M.row_hi[c]) << 32) | M.row_lo[c]);
+                const float* grow_c = reinterpret_cast<const float*>((static_cast<unsigned long long>(M.row_hi[c]) << 32) | M.row_lo[c]);
+                const float* grow_j = reinterpret_cast<const float*>((static_cast<unsigned long long>(M.row_hi[j]) << 32) | M.row_lo[j]);
                 const float inv = __builtin_amdgcn_rcpf(e.w);
-                const float sc = bwd_radial_pair<float>(grow, type_of(j), e.w, inv);
+                // the pair's pull on the centre from both rows; the partner gets its share when it is the centre
+                const float sc = bwd_radial_pair_both<float>(grow_c, type_of(j), grow_j, type_of(c), e.w, inv);
                 fx = sc * e.x;
                 fy = sc * e.y;
                 fz = sc * e.z;
-                add_force(j, -fx, -fy, -fz);
             }
             // the pairs of one centre are summed in the wave (a handful of centres per 64 pairs) and added once
             unsigned long long todo = wave_ballot(lane < count);
@@ -208,19 +212,8 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                         m_c += popc64(mA[ch]);
                     }
                 }
-                if (m_c > 64) {
-                    // more partners than a pool holds: the general per-centre routine does this centre alone
-                    const int i_orig = uniform(static_cast<int>(M.orig[c]));
-                    radial_drain();                    // the routine uses the staging area as scratch
-                    bwd_center_generic<float>(L, lane, X, Y, Z, A, off, n, i_orig, P.gst, row_of(c),
-                                              [&](int atom, float fx, float fy, float fz) {
-                                                  atomicAdd(&gX[off + atom], fx);
-                                                  atomicAdd(&gY[off + atom], fy);
-                                                  atomicAdd(&gZ[off + atom], fz);
-                                              });
-                    continue;
-                }
-                if (nb > 0 && used + m_c > 64) {       // full: this centre opens the next batch
+                const bool too_many = m_c > 64;        // more partners than a pool holds
+                if (!too_many && nb > 0 && used + m_c > 64) {       // full: this centre opens the next batch
                     pending = c;
                     break;
                 }
@@ -230,7 +223,7 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                 for (int ch = 0; ch < kChunks; ++ch) {
                     if (ch * 64 < n) {
                         const int j = ch * 64 + lane;
-                        if ((mA[ch] >> lane) & 1ull) {
+                        if (!too_many && ((mA[ch] >> lane) & 1ull)) {
                             const int p = pos + popc64(mA[ch] & lt_mask);
                             const float inv = __builtin_amdgcn_rcpf(r[ch]);
                             float fc, dfc;
@@ -268,6 +261,20 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                             qn = rest;
                         }
                     }
+                }
+                if (too_many) {
+                    // the general per-centre routine does this centre's angular part alone (its radial pairs are
+                    // in the queue like everyone's)
+                    const int i_orig = uniform(static_cast<int>(M.orig[c]));
+                    radial_drain();                    // the routine uses the staging area as scratch
+                    bwd_center_generic<float>(L, lane, X, Y, Z, A, off, n, i_orig, P.gst, row_of(c),
+                                              [&](int atom, float fx, float fy, float fz) {
+                                                  atomicAdd(&gX[off + atom], fx);
+                                                  atomicAdd(&gY[off + atom], fy);
+                                                  atomicAdd(&gZ[off + atom], fz);
+                                              },
+                                              false);
+                    continue;
                 }
                 if (lane == nb) {
                     pfv = used;
