@@ -21,6 +21,7 @@ namespace {
 
 constexpr int kMedMin = kSmallPreferredMax + 1;   // smaller molecules run one wavefront each
 constexpr int kRadCap = 64;                   // radial partners kept per centre
+constexpr int kMedRadTrip = 1;                // list entries a lane takes per trip of the radial walk (four slots: 4 entries per trip)
 
 struct __align__(16) MedShared {
     float4 atom[kMediumMaxAtoms];          // x, y, z, type (sorted order)
@@ -152,12 +153,12 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                     for (int a = 0; a < 4; ++a) {
                         const int cnt_a = cR[a];
                         float acc_r = 0.f;
-                        for (int q0 = 0; q0 < cnt_a; q0 += 16) {
-                            float2 e[4];
+                        for (int q0 = 0; q0 < cnt_a; q0 += 4 * kMedRadTrip) {
+                            float2 e[kMedRadTrip];
 #pragma unroll
-                            for (int u = 0; u < 4; ++u) e[u] = S.rad[min(obase + q0 + u * 4 + rslot, kRadCap - 1)];
+                            for (int u = 0; u < kMedRadTrip; ++u) e[u] = S.rad[min(obase + q0 + u * 4 + rslot, kRadCap - 1)];
 #pragma unroll
-                            for (int u = 0; u < 4; ++u) {
+                            for (int u = 0; u < kMedRadTrip; ++u) {
                                 const float dd = e[u].x - L.rrs;
                                 const float v = __builtin_amdgcn_exp2f(kRadExp * dd * dd) * e[u].y;
                                 acc_r += (q0 + u * 4 + rslot < cnt_a) ? v : 0.f;   // entries of other types: select
