@@ -1,4 +1,5 @@
-// AEV forward for molecules of 65 to 256 atoms (float32): one workgroup of four wavefronts per molecule.
+// AEV forward for molecules of up to 256 atoms that are too large for one wavefront (float32 from 33 atoms,
+// float64 from 65; also the float32 Jacobian-vector product from 65): one workgroup of four wavefronts per molecule.
 //
 // The workgroup sorts the molecule's atoms by type into LDS once (256-way counting sort with per-wave
 // ballots).  Each wavefront then takes batches of six centres and runs the same pipeline as the
@@ -19,45 +20,56 @@ namespace khan {
 
 namespace {
 
-constexpr int kMedMin = kSmallPreferredMax + 1;   // smaller molecules run one wavefront each
 constexpr int kRadCap = 64;                   // radial partners kept per centre
 constexpr int kMedRadTrip = 1;                // list entries a lane takes per trip of the radial walk (four slots: 4 entries per trip)
 
+template <typename T, bool kJvp> struct MedVel {};
+template <typename T> struct __align__(16) MedVel<T, true> {
+    typename Fast<T>::vec4 vel[kMediumMaxAtoms];   // the incoming vector of every atom (sorted order)
+};
+
+template <typename T, bool kJvp>
 struct __align__(16) MedShared {
-    float4 atom[kMediumMaxAtoms];          // x, y, z, type (sorted order)
+    typename Fast<T>::vec4 atom[kMediumMaxAtoms];   // x, y, z, type (sorted order)
     unsigned row_lo[kMediumMaxAtoms];      // address of the atom's output row
     unsigned row_hi[kMediumMaxAtoms];
     unsigned short orig[kMediumMaxAtoms];  // sorted position -> index inside the molecule
     int wcount[4][4];                      // atoms of each type held by each wavefront before the sort
+    MedVel<T, kJvp> v;
 };
 
+// With kJvp the kernel computes the Jacobian-vector product instead (featurize_grad_inverse), as the
+// one-wavefront kernel does: list entries also carry (v_i - v_j)/r, the cutoff's derivative and the change of r.
+template <typename T, bool kJvp>
 __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
-    const float* __restrict__ X, const float* __restrict__ Y, const float* __restrict__ Z,
+    const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
-    Buckets<float> out, const int32_t* __restrict__ order)
+    const T* __restrict__ VX, const T* __restrict__ VY, const T* __restrict__ VZ,
+    Buckets<T> out, int min_atoms, const int32_t* __restrict__ order)
 {
-    __shared__ MedShared M;
-    __shared__ FwdWaveLds<float> lds_wave[4];
+    typedef typename Fast<T>::vec4 vec4;
+    typedef typename Fast<T>::vec2 vec2;
+    __shared__ MedShared<T, kJvp> M;
+    __shared__ FwdWaveLds<T, kJvp> lds_wave[4];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = uniform(tid >> 6);
-    FwdWaveLds<float>& S = lds_wave[wave];
-    const LaneConsts<float> L = lane_consts<float>(lane);
+    FwdWaveLds<T, kJvp>& S = lds_wave[wave];
+    const LaneConsts<T> L = lane_consts<T>(lane);
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
-    const float inv_rc_R = 1.0f / kR_Rc_f, inv_rc_A = 1.0f / kA_Rc_f;
-    const float kRadExp = -kR_eta_f * 1.44269504088896340736f;   // exp(-eta d^2) = exp2(kRadExp d^2)
     const int rslot = lane >> 4;                                 // radial walk: entry slot of this 16-lane group
 
     fwd_lds_init(S, lane);
     __shared__ unsigned long long want[4];
-    for_each_molecule_in_range(MACs, n_mols, kMedMin, kMediumMaxAtoms, want, order, order ? order + n_mols : nullptr, [&](int mol) {
+    for_each_molecule_in_range(MACs, n_mols, min_atoms, kMediumMaxAtoms, want, order, order ? order + n_mols : nullptr, [&](int mol) {
         const int n = uniform(MACs[mol]);
         const int off = uniform(MOs[mol]);
 
         // ------------------------------------------------------------ load, sort by type into LDS
         const bool have = tid < n;
-        float x = 0.f, y = 0.f, z = 0.f;
+        T x = T(0), y = T(0), z = T(0);
+        T vx = T(0), vy = T(0), vz = T(0);
         int type = 0;
         unsigned long long rowbits = 0;
         if (have) {
@@ -66,6 +78,11 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
             z = Z[off + tid];
             type = fold_type(A[off + tid]);
             rowbits = reinterpret_cast<unsigned long long>(out.p[type] + static_cast<size_t>(SIs[off + tid]) * kFeats);
+            if constexpr (kJvp) {
+                vx = VX[off + tid];
+                vy = VY[off + tid];
+                vz = VZ[off + tid];
+            }
         }
         unsigned long long tmask[4];
 #pragma unroll
@@ -87,16 +104,17 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
             for (int w = 0; w < wave; ++w) before += M.wcount[w][type];
             const unsigned long long mine = type == 0 ? tmask[0] : type == 1 ? tmask[1] : type == 2 ? tmask[2] : tmask[3];
             const int dest = sel4(type, tbase[0], tbase[1], tbase[2], tbase[3]) + before + popc64(mine & lt_mask);
-            M.atom[dest] = make_float4(x, y, z, __int_as_float(type));
+            M.atom[dest] = Fast<T>::make4(x, y, z, static_cast<T>(type));
             M.row_lo[dest] = static_cast<unsigned>(rowbits & 0xffffffffull);
             M.row_hi[dest] = static_cast<unsigned>(rowbits >> 32);
             M.orig[dest] = static_cast<unsigned short>(tid);
+            if constexpr (kJvp) M.v.vel[dest] = Fast<T>::make4(vx, vy, vz, T(0));
         }
         __syncthreads();
-        auto row_of = [&](int sorted_idx) -> float* {            // wave-uniform index
+        auto row_of = [&](int sorted_idx) -> T* {            // wave-uniform index
             const unsigned lo = static_cast<unsigned>(uniform(static_cast<int>(M.row_lo[sorted_idx])));
             const unsigned hi = static_cast<unsigned>(uniform(static_cast<int>(M.row_hi[sorted_idx])));
-            return reinterpret_cast<float*>((static_cast<unsigned long long>(hi) << 32) | lo);
+            return reinterpret_cast<T*>((static_cast<unsigned long long>(hi) << 32) | lo);
         };
 
         // ------------------------------------------------------------ batches of six centres per wavefront
@@ -106,35 +124,61 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
 
             for (int b = 0; b < nb; ++b) {
                 const int i = c0 + b;
-                const float4 ai = M.atom[i];
+                const vec4 ai = M.atom[i];
                 int posR = 0, posA = 0;                 // list lengths so far (wave-uniform)
                 int cR[4] = {0, 0, 0, 0}, cA[4] = {0, 0, 0, 0};
                 for (int jc = 0; jc < n; jc += 64) {
                     const int j = jc + lane;
-                    const float4 aj = M.atom[min(j, kMediumMaxAtoms - 1)];
-                    const float dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
-                    const float r = sqrtf(dx * dx + dy * dy + dz * dz);
+                    const int jj = min(j, kMediumMaxAtoms - 1);
+                    const vec4 aj = M.atom[jj];
+                    const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
+                    const T r = sqrt(dx * dx + dy * dy + dz * dz);
                     const bool valid = (j < n) && (j != i);
                     const bool inR = valid && (r < kR_Rc_f);
                     const bool inA = valid && (r < kA_Rc_f);
                     const unsigned long long mR = wave_ballot(inR), mA = wave_ballot(inA);
-                    const int tj = __float_as_int(aj.w);
+                    const int tj = static_cast<int>(aj.w);
 #pragma unroll
                     for (int a = 0; a < 4; ++a) {
                         const unsigned long long ta = wave_ballot(tj == a);
                         cR[a] += popc64(mR & ta);
                         cA[a] += popc64(mA & ta);
                     }
+                    const T inv = Fast<T>::rcp(r);
+                    T wx = T(0), wy = T(0), wz = T(0), rd = T(0);        // v_centre - v_partner, and d r along it
+                    if constexpr (kJvp) {
+                        const vec4 vi = M.v.vel[i], vjv = M.v.vel[jj];
+                        wx = vi.x - vjv.x;
+                        wy = vi.y - vjv.y;
+                        wz = vi.z - vjv.z;
+                        rd = (dx * wx + dy * wy + dz * wz) * inv;
+                    }
                     if (inR) {
                         const int p = posR + popc64(mR & lt_mask);
-                        if (p < kRadCap) S.rad[p] = make_float2(r, cutoff_poly(r * inv_rc_R));
+                        if (p < kRadCap) {
+                            if constexpr (kJvp) {
+                                T fc, dfc;
+                                Fast<T>::cutoff_grad(r, static_cast<T>(kR_Rc_f), fc, dfc);
+                                S.rad[p] = Fast<T>::make2(r, fc);
+                                S.jvp.rad_ab[p] = Fast<T>::make2(dfc * rd, T(-2) * static_cast<T>(kR_eta_f) * fc * rd);
+                            } else {
+                                S.rad[p] = Fast<T>::make2(r, Fast<T>::cutoff(r, static_cast<T>(kR_Rc_f)));
+                            }
+                        }
                     }
                     if (inA) {
                         const int p = posA + popc64(mA & lt_mask);
                         if (p < kCapA) {
-                            const float inv = __builtin_amdgcn_rcpf(r);
-                            S.nbr[b][p] = make_float4(dx * inv, dy * inv, dz * inv, r);
-                            S.nbr_fc[b][p] = cutoff_poly(r * inv_rc_A);
+                            S.nbr[b][p] = Fast<T>::make4(dx * inv, dy * inv, dz * inv, r);
+                            if constexpr (kJvp) {
+                                T fc, dfc;
+                                Fast<T>::cutoff_grad(r, static_cast<T>(kA_Rc_f), fc, dfc);
+                                S.nbr_fc[b][p] = fc;
+                                S.jvp.nbr_p[b][p] = Fast<T>::make4(wx * inv, wy * inv, wz * inv, rd * inv);
+                                S.jvp.nbr_d[b][p] = Fast<T>::make2(dfc * rd, rd);
+                            } else {
+                                S.nbr_fc[b][p] = Fast<T>::cutoff(r, static_cast<T>(kA_Rc_f));
+                            }
                         }
                     }
                     posR += popc64(mR);
@@ -147,21 +191,28 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
 
                 // ---- radial features of this centre: lanes = (slot of 4) x (shell)
                 if (fits) {
-                    float* row = row_of(i);
+                    T* row = row_of(i);
                     int obase = 0;
 #pragma unroll
                     for (int a = 0; a < 4; ++a) {
                         const int cnt_a = cR[a];
-                        float acc_r = 0.f;
+                        T acc_r = T(0);
                         for (int q0 = 0; q0 < cnt_a; q0 += 4 * kMedRadTrip) {
-                            float2 e[kMedRadTrip];
-#pragma unroll
-                            for (int u = 0; u < kMedRadTrip; ++u) e[u] = S.rad[min(obase + q0 + u * 4 + rslot, kRadCap - 1)];
+                            vec2 e[kMedRadTrip], ab[kMedRadTrip];
 #pragma unroll
                             for (int u = 0; u < kMedRadTrip; ++u) {
-                                const float dd = e[u].x - L.rrs;
-                                const float v = __builtin_amdgcn_exp2f(kRadExp * dd * dd) * e[u].y;
-                                acc_r += (q0 + u * 4 + rslot < cnt_a) ? v : 0.f;   // entries of other types: select
+                                const int at = min(obase + q0 + u * 4 + rslot, kRadCap - 1);
+                                e[u] = S.rad[at];
+                                if constexpr (kJvp) ab[u] = S.jvp.rad_ab[at];
+                            }
+#pragma unroll
+                            for (int u = 0; u < kMedRadTrip; ++u) {
+                                const T dd = e[u].x - L.rrs;
+                                // forward: exp(-eta d^2) f_C; derivative: exp(-eta d^2) (f_C' - 2 eta d f_C) dr
+                                T v = Fast<T>::gauss(static_cast<T>(kR_eta_f), dd);
+                                if constexpr (kJvp) v *= fma(ab[u].y, dd, ab[u].x);
+                                else v *= e[u].y;
+                                acc_r += (q0 + u * 4 + rslot < cnt_a) ? v : T(0);   // entries of other types: select
                             }
                         }
                         acc_r += __shfl_xor(acc_r, 16, 64);
@@ -174,7 +225,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
             }
 
             // ------------------------------------------------ segment table, phases 1 and 2, zero fill
-            fwd_angular_batch<float, false>(S, L, lane, nb, [&](int b) -> unsigned long long {
+            fwd_angular_batch<T, kJvp>(S, L, lane, nb, [&](int b) -> unsigned long long {
                 const int idx = min(c0 + b, kMediumMaxAtoms - 1);
                 return (static_cast<unsigned long long>(M.row_hi[idx]) << 32) | M.row_lo[idx];
             });
@@ -185,8 +236,12 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                 for (int b = 0; b < nb; ++b) {
                     if (overflow & (1u << b)) {
                         const int i_orig = uniform(static_cast<int>(M.orig[c0 + b]));
-                        fwd_center_generic<float>(L, lane, X, Y, Z, A, off, n, i_orig,
-                                                  reinterpret_cast<float*>(S.rec), row_of(c0 + b));
+                        if constexpr (kJvp)
+                            jvp_center_generic<T>(L, lane, X, Y, Z, A, VX, VY, VZ, off, n, i_orig,
+                                                  reinterpret_cast<T*>(S.rec), row_of(c0 + b));
+                        else
+                            fwd_center_generic<T>(L, lane, X, Y, Z, A, off, n, i_orig,
+                                                  reinterpret_cast<T*>(S.rec), row_of(c0 + b));
                     }
                 }
                 wave_lds_fence();
@@ -198,15 +253,32 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
 
 }  // namespace
 
-hipError_t launch_fwd_medium_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
-                                 const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
-                                 const int32_t* SIs, Buckets<float> out, const int32_t* order, hipStream_t stream)
+template <typename T>
+hipError_t launch_fwd_medium(const T* X, const T* Y, const T* Z, const int32_t* A,
+                             const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                             const int32_t* SIs, Buckets<T> out, int min_atoms, const int32_t* order, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
     // workgroups walk the molecules with the grid's stride and skip those of other sizes
     const unsigned blocks = static_cast<unsigned>(n_mols < 4096 ? n_mols : 4096);
-    aev_fwd_medium_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, out, order);
+    aev_fwd_medium_kernel<T, false><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, nullptr, nullptr,
+                                                                        nullptr, out, min_atoms, order);
     return hipGetLastError();
 }
+
+hipError_t launch_jvp_medium_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
+                                 const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                                 const int32_t* SIs, const float* VX, const float* VY, const float* VZ,
+                                 Buckets<float> out, int min_atoms, const int32_t* order, hipStream_t stream)
+{
+    if (n_mols <= 0) return hipSuccess;
+    const unsigned blocks = static_cast<unsigned>(n_mols < 4096 ? n_mols : 4096);
+    aev_fwd_medium_kernel<float, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, VX, VY, VZ,
+                                                                            out, min_atoms, order);
+    return hipGetLastError();
+}
+
+template hipError_t launch_fwd_medium<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<float>, int, const int32_t*, hipStream_t);
+template hipError_t launch_fwd_medium<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<double>, int, const int32_t*, hipStream_t);
 
 }  // namespace khan

@@ -86,7 +86,8 @@ int forward_dispatch(const float* xs, const float* ys, const float* zs, const in
     int st = hip_status(khan::launch_fwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallPreferredMax,
                                                       order.get(), stream));
     if (st != KHAN_OK) return st;
-    st = hip_status(khan::launch_fwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, out, order.get(), stream));
+    st = hip_status(khan::launch_fwd_medium<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallPreferredMax + 1,
+                                                   order.get(), stream));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
                                                       khan::kMediumMaxAtoms + 1, order.get(), stream));
@@ -102,8 +103,12 @@ int forward_dispatch(const double* xs, const double* ys, const double* zs, const
     int st = hip_status(khan::launch_fwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallMaxAtoms,
                                                        order.get(), stream));
     if (st != KHAN_OK) return st;
+    // 65..256 atoms: one workgroup each (in float64 a one-wavefront kernel keeps molecules of up to 64 atoms)
+    st = hip_status(khan::launch_fwd_medium<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallMaxAtoms + 1,
+                                                    order.get(), stream));
+    if (st != KHAN_OK) return st;
     return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
-                                                       khan::kSmallMaxAtoms + 1, order.get(), stream));
+                                                       khan::kMediumMaxAtoms + 1, order.get(), stream));
 }
 
 int backward_dispatch(const float* xs, const float* ys, const float* zs, const int32_t* as,
@@ -200,13 +205,20 @@ int featurize_grad_inverse_impl(const T* xs, const T* ys, const T* zs, const int
     if (force_generic())
         return hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, 0,
                                                       nullptr, as_stream(stream)));
-    // molecules of up to 64 atoms: one wavefront each; the rest: general-shape kernel
+    // molecules of up to 64 atoms: one wavefront each; 65..256 in float32: one workgroup each; the rest: general-shape kernel
     SizeOrder order(macs, n_mols, as_stream(stream));
     int st = hip_status(khan::launch_jvp_small<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, order.get(),
                                                   as_stream(stream)));
     if (st != KHAN_OK) return st;
+    int generic_from = khan::kSmallMaxAtoms + 1;
+    if constexpr (sizeof(T) == 4) {
+        st = hip_status(khan::launch_jvp_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
+                                                    khan::kSmallMaxAtoms + 1, order.get(), as_stream(stream)));
+        if (st != KHAN_OK) return st;
+        generic_from = khan::kMediumMaxAtoms + 1;
+    }
     return hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
-                                                  khan::kSmallMaxAtoms + 1, order.get(), as_stream(stream)));
+                                                  generic_from, order.get(), as_stream(stream)));
 }
 
 template <typename T>
