@@ -1,5 +1,5 @@
-// AEV backward (dL/dxyz) for molecules of 65 to 256 atoms, float32: one workgroup of four wavefronts
-// per molecule.
+// AEV backward (dL/dxyz) for molecules of up to 256 atoms that are too large for one wavefront (float32 from
+// 33 atoms, float64 from 65): one workgroup of four wavefronts per molecule.
 //
 // The workgroup sorts the atoms by type into LDS once and zeroes the molecule's outputs.  Wavefronts
 // then draw centres from a shared counter.  A wavefront collects centres into a batch while their
@@ -24,11 +24,11 @@ namespace khan {
 
 namespace {
 
-constexpr int kMedMin = kSmallPreferredMax + 1;   // smaller molecules run one wavefront each
 constexpr int kChunks = kMediumMaxAtoms / 64;
 
+template <typename T>
 struct __align__(16) MedBwdShared {
-    float4 atom[kMediumMaxAtoms];          // x, y, z, type (sorted order)
+    typename Fast<T>::vec4 atom[kMediumMaxAtoms];   // x, y, z, type (sorted order)
     unsigned row_lo[kMediumMaxAtoms];      // address of the atom's upstream row
     unsigned row_hi[kMediumMaxAtoms];
     unsigned short orig[kMediumMaxAtoms];  // sorted position -> index inside the molecule
@@ -36,31 +36,33 @@ struct __align__(16) MedBwdShared {
     int next;                              // next centre (sorted position) to hand out
 };
 
+template <typename T>
 __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
-    const float* __restrict__ X, const float* __restrict__ Y, const float* __restrict__ Z,
+    const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
-    Buckets<const float> gin, float* __restrict__ gX, float* __restrict__ gY, float* __restrict__ gZ,
+    Buckets<const T> gin, T* __restrict__ gX, T* __restrict__ gY, T* __restrict__ gZ, int min_atoms,
     const int32_t* __restrict__ order, bool walk_in_order)
 {
-    __shared__ MedBwdShared M;
-    __shared__ BwdPool<float> pools[4];
+    typedef typename Fast<T>::vec4 vec4;
+    __shared__ MedBwdShared<T> M;
+    __shared__ BwdPool<T> pools[4];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = uniform(tid >> 6);
-    BwdPool<float>& P = pools[wave];
-    const LaneConsts<float> L = lane_consts<float>(lane);
+    BwdPool<T>& P = pools[wave];
+    const LaneConsts<T> L = lane_consts<T>(lane);
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
 
     __shared__ unsigned long long want[4];
-    for_each_molecule_in_range(MACs, n_mols, kMedMin, kMediumMaxAtoms, want, walk_in_order ? order : nullptr,
+    for_each_molecule_in_range(MACs, n_mols, min_atoms, kMediumMaxAtoms, want, walk_in_order ? order : nullptr,
                                order ? order + n_mols : nullptr, [&](int mol) {
         const int n = uniform(MACs[mol]);
         const int off = uniform(MOs[mol]);
 
         // ------------------------------------------------------------ load, sort by type into LDS, zero outputs
         const bool have = tid < n;
-        float x = 0.f, y = 0.f, z = 0.f;
+        T x = T(0), y = T(0), z = T(0);
         int type = 0;
         unsigned long long rowbits = 0;
         if (have) {
@@ -69,9 +71,9 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
             z = Z[off + tid];
             type = fold_type(A[off + tid]);
             rowbits = reinterpret_cast<unsigned long long>(gin.p[type] + static_cast<size_t>(SIs[off + tid]) * kFeats);
-            gX[off + tid] = 0.f;
-            gY[off + tid] = 0.f;
-            gZ[off + tid] = 0.f;
+            gX[off + tid] = T(0);
+            gY[off + tid] = T(0);
+            gZ[off + tid] = T(0);
         }
         unsigned long long tmask[4];
 #pragma unroll
@@ -93,7 +95,7 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
             for (int w = 0; w < wave; ++w) before += M.wcount[w][type];
             const unsigned long long mine = type == 0 ? tmask[0] : type == 1 ? tmask[1] : type == 2 ? tmask[2] : tmask[3];
             const int dest = sel4(type, tbase[0], tbase[1], tbase[2], tbase[3]) + before + popc64(mine & lt_mask);
-            M.atom[dest] = make_float4(x, y, z, __int_as_float(type));
+            M.atom[dest] = Fast<T>::make4(x, y, z, static_cast<T>(type));
             M.row_lo[dest] = static_cast<unsigned>(rowbits & 0xffffffffull);
             M.row_hi[dest] = static_cast<unsigned>(rowbits >> 32);
             M.orig[dest] = static_cast<unsigned short>(tid);
@@ -101,12 +103,12 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
         __syncthreads();       // sorted arrays complete; the zeroed outputs are visible before any atomic add
         const int tb1 = tbase[1], tb2 = tbase[2], tb3 = tbase[3];
         auto type_of = [&](int sorted_idx) { return (sorted_idx >= tb1) + (sorted_idx >= tb2) + (sorted_idx >= tb3); };
-        auto row_of = [&](int sorted_idx) -> const float* {            // wave-uniform index
+        auto row_of = [&](int sorted_idx) -> const T* {            // wave-uniform index
             const unsigned lo = static_cast<unsigned>(uniform(static_cast<int>(M.row_lo[sorted_idx])));
             const unsigned hi = static_cast<unsigned>(uniform(static_cast<int>(M.row_hi[sorted_idx])));
-            return reinterpret_cast<const float*>((static_cast<unsigned long long>(hi) << 32) | lo);
+            return reinterpret_cast<const T*>((static_cast<unsigned long long>(hi) << 32) | lo);
         };
-        auto add_force = [&](int sorted_idx, float fx, float fy, float fz) {   // per-lane target
+        auto add_force = [&](int sorted_idx, T fx, T fy, T fz) {   // per-lane target
             const int g = off + M.orig[sorted_idx];
             atomicAdd(&gX[g], fx);
             atomicAdd(&gY[g], fy);
@@ -117,22 +119,22 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
         // pairs of a large molecule lie inside the radial cutoff, so evaluating them where they are found
         // would leave most lanes idle.  The queue lives in the pool's staging area, which is free while a
         // batch is being collected; it is emptied before the batch's upstream rows are staged.
-        float4* const q_d = reinterpret_cast<float4*>(P.gst);                      // 128 x (dx, dy, dz, r)
+        vec4* const q_d = reinterpret_cast<vec4*>(P.gst);                          // 128 x (dx, dy, dz, r)
         unsigned short* const q_j = reinterpret_cast<unsigned short*>(q_d + 128);  // partner (sorted position)
         unsigned short* const q_c = q_j + 128;                                     // centre (sorted position)
         int qn = 0;
         auto radial_work_off = [&](int count) {      // entries 0..count-1, count <= 64
-            float fx = 0.f, fy = 0.f, fz = 0.f;
+            T fx = T(0), fy = T(0), fz = T(0);
             int c = -1;
             if (lane < count) {
-                const float4 e = q_d[lane];
+                const vec4 e = q_d[lane];
                 const int j = q_j[lane];
                 c = q_c[lane];
-                const float* grow_c = reinterpret_cast<const float*>((static_cast<unsigned long long>(M.row_hi[c]) << 32) | M.row_lo[c]);
-                const float* grow_j = reinterpret_cast<const float*>((static_cast<unsigned long long>(M.row_hi[j]) << 32) | M.row_lo[j]);
-                const float inv = __builtin_amdgcn_rcpf(e.w);
+                const T* grow_c = reinterpret_cast<const T*>((static_cast<unsigned long long>(M.row_hi[c]) << 32) | M.row_lo[c]);
+                const T* grow_j = reinterpret_cast<const T*>((static_cast<unsigned long long>(M.row_hi[j]) << 32) | M.row_lo[j]);
+                const T inv = Fast<T>::rcp(e.w);
                 // the pair's pull on the centre from both rows; the partner gets its share when it is the centre
-                const float sc = bwd_radial_pair_both<float>(grow_c, type_of(j), grow_j, type_of(c), e.w, inv);
+                const T sc = bwd_radial_pair_both<T>(grow_c, type_of(j), grow_j, type_of(c), e.w, inv);
                 fx = sc * e.x;
                 fy = sc * e.y;
                 fz = sc * e.z;
@@ -143,9 +145,9 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                 const int c0 = lane_read(c, lowest_bit(todo));
                 const bool mine = c == c0;
                 todo &= ~wave_ballot(mine);
-                const float sx = group_sum_to_last_lane(mine ? fx : 0.f, 6);
-                const float sy = group_sum_to_last_lane(mine ? fy : 0.f, 6);
-                const float sz = group_sum_to_last_lane(mine ? fz : 0.f, 6);
+                const T sx = group_sum_to_last_lane(mine ? fx : T(0), 6);
+                const T sy = group_sum_to_last_lane(mine ? fy : T(0), 6);
+                const T sz = group_sum_to_last_lane(mine ? fz : T(0), 6);
                 if (lane == 63) add_force(c0, sx, sy, sz);
             }
         };
@@ -155,7 +157,7 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                 const int take = min(qn, 64);
                 radial_work_off(take);
                 const int rest = qn - take;
-                float4 e = make_float4(0.f, 0.f, 0.f, 1.f);
+                vec4 e = Fast<T>::make4(T(0), T(0), T(0), T(1));
                 unsigned short ej = 0, ec = 0;
                 if (lane < rest) {
                     e = q_d[64 + lane];
@@ -178,7 +180,7 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
             // ------------------------------------------------ collect a batch of centres
             int nb = 0, used = 0;
             int pfv = 0, cv = 0;   // lane k: first pool slot and sorted position of centre k of the batch
-            P.facc[lane] = make_float4(0.f, 0.f, 0.f, 0.f);
+            P.facc[lane] = Fast<T>::make4(T(0), T(0), T(0), T(0));
             while (nb < kB) {
                 int c = pending;
                 pending = -1;
@@ -188,24 +190,24 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                     c = uniform(drawn);
                 }
                 if (c >= n) break;
-                const float4 ai = M.atom[c];
+                const vec4 ai = M.atom[c];
                 // first pass over the partners: who is inside the cutoffs
-                float dx[kChunks], dy[kChunks], dz[kChunks], r[kChunks];
+                T dx[kChunks], dy[kChunks], dz[kChunks], r[kChunks];
                 unsigned long long mA[kChunks], mR[kChunks];
                 int m_c = 0;
 #pragma unroll
                 for (int ch = 0; ch < kChunks; ++ch) {
                     mA[ch] = 0ull;
                     mR[ch] = 0ull;
-                    dx[ch] = dy[ch] = dz[ch] = 0.f;
-                    r[ch] = 1.f;
+                    dx[ch] = dy[ch] = dz[ch] = T(0);
+                    r[ch] = T(1);
                     if (ch * 64 < n) {
                         const int j = ch * 64 + lane;
-                        const float4 aj = M.atom[j];
+                        const vec4 aj = M.atom[j];
                         dx[ch] = ai.x - aj.x;
                         dy[ch] = ai.y - aj.y;
                         dz[ch] = ai.z - aj.z;
-                        r[ch] = sqrtf(dx[ch] * dx[ch] + dy[ch] * dy[ch] + dz[ch] * dz[ch]);
+                        r[ch] = sqrt(dx[ch] * dx[ch] + dy[ch] * dy[ch] + dz[ch] * dz[ch]);
                         const bool valid = (j < n) && (j != c);
                         mR[ch] = wave_ballot(valid && (r[ch] < kR_Rc_f));
                         mA[ch] = wave_ballot(valid && (r[ch] < kA_Rc_f));
@@ -225,17 +227,17 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                         const int j = ch * 64 + lane;
                         if (!too_many && ((mA[ch] >> lane) & 1ull)) {
                             const int p = pos + popc64(mA[ch] & lt_mask);
-                            const float inv = __builtin_amdgcn_rcpf(r[ch]);
-                            float fc, dfc;
-                            Fast<float>::cutoff_grad(r[ch], kA_Rc_f, fc, dfc);
-                            P.nbr[p] = make_float4(dx[ch] * inv, dy[ch] * inv, dz[ch] * inv, r[ch]);
-                            P.nbr_fc[p] = make_float2(fc, dfc);
+                            const T inv = Fast<T>::rcp(r[ch]);
+                            T fc, dfc;
+                            Fast<T>::cutoff_grad(r[ch], static_cast<T>(kA_Rc_f), fc, dfc);
+                            P.nbr[p] = Fast<T>::make4(dx[ch] * inv, dy[ch] * inv, dz[ch] * inv, r[ch]);
+                            P.nbr_fc[p] = Fast<T>::make2(fc, dfc);
                             P.nbr_idx[p] = static_cast<unsigned char>(j);
                         }
                         pos += popc64(mA[ch]);
                         if ((mR[ch] >> lane) & 1ull) {
                             const int p = qn + popc64(mR[ch] & lt_mask);
-                            q_d[p] = make_float4(dx[ch], dy[ch], dz[ch], r[ch]);
+                            q_d[p] = Fast<T>::make4(dx[ch], dy[ch], dz[ch], r[ch]);
                             q_j[p] = static_cast<unsigned short>(j);
                             q_c[p] = static_cast<unsigned short>(c);
                         }
@@ -244,7 +246,7 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                             wave_lds_fence();
                             radial_work_off(64);
                             const int rest = qn - 64;
-                            float4 e = make_float4(0.f, 0.f, 0.f, 1.f);
+                            vec4 e = Fast<T>::make4(T(0), T(0), T(0), T(1));
                             unsigned short ej = 0, ec = 0;
                             if (lane < rest) {
                                 e = q_d[64 + lane];
@@ -267,8 +269,8 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                     // in the queue like everyone's)
                     const int i_orig = uniform(static_cast<int>(M.orig[c]));
                     radial_drain();                    // the routine uses the staging area as scratch
-                    bwd_center_generic<float>(L, lane, X, Y, Z, A, off, n, i_orig, P.gst, row_of(c),
-                                              [&](int atom, float fx, float fy, float fz) {
+                    bwd_center_generic<T>(L, lane, X, Y, Z, A, off, n, i_orig, P.gst, row_of(c),
+                                              [&](int atom, T fx, T fy, T fz) {
                                                   atomicAdd(&gX[off + atom], fx);
                                                   atomicAdd(&gY[off + atom], fy);
                                                   atomicAdd(&gZ[off + atom], fz);
@@ -289,7 +291,7 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
 
             // ---- the angular upstream blocks of the batch's rows go to LDS (80 x 16 bytes per row)
             {
-                RowStage<float> stage;
+                RowStage<T> stage;
                 stage.fetch(lane, nb, [&](int b) { return row_of(lane_read(cv, b)); });
                 stage.store(P, lane, nb);
             }
@@ -304,15 +306,15 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
             const int bs = live ? b : 0;
             const int pb = sel6(bs, 0, pf1, pf2, pf3, pf4, pf5);
             const int m = sel6(bs, pf1, pf2, pf3, pf4, pf5, pf6) - pb;
-            const float4 f = bwd_angular_rounds<float>(P, lane, live, bs, pb, m, type_of);
+            const vec4 f = bwd_angular_rounds<T>(P, lane, live, bs, pb, m, type_of);
 
             // ------------------------------------------------ gather
             if (live) add_force(P.nbr_idx[lane], f.x, f.y, f.z);
             for (int bb = 0; bb < nb; ++bb) {
                 const bool mine = live && (bs == bb);
-                const float sx = group_sum_to_last_lane(mine ? f.x : 0.f, 6);
-                const float sy = group_sum_to_last_lane(mine ? f.y : 0.f, 6);
-                const float sz = group_sum_to_last_lane(mine ? f.z : 0.f, 6);
+                const T sx = group_sum_to_last_lane(mine ? f.x : T(0), 6);
+                const T sy = group_sum_to_last_lane(mine ? f.y : T(0), 6);
+                const T sz = group_sum_to_last_lane(mine ? f.z : T(0), 6);
                 if (lane == 63) add_force(lane_read(cv, bb), -sx, -sy, -sz);
             }
             wave_lds_fence();
@@ -323,16 +325,21 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
 
 }  // namespace
 
-hipError_t launch_bwd_medium_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
-                                 const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
-                                 const int32_t* SIs, Buckets<const float> g, float* gX, float* gY,
-                                 float* gZ, const int32_t* order, bool walk_in_order, hipStream_t stream)
+template <typename T>
+hipError_t launch_bwd_medium(const T* X, const T* Y, const T* Z, const int32_t* A,
+                             const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                             const int32_t* SIs, Buckets<const T> g, T* gX, T* gY,
+                             T* gZ, int min_atoms, const int32_t* order, bool walk_in_order, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
     // workgroups walk the molecules with the grid's stride and skip those of other sizes
     const unsigned blocks = static_cast<unsigned>(n_mols < 4096 ? n_mols : 4096);
-    aev_bwd_medium_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ, order, walk_in_order);
+    aev_bwd_medium_kernel<T><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ, min_atoms,
+                                                                  order, walk_in_order);
     return hipGetLastError();
 }
+
+template hipError_t launch_bwd_medium<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const float>, float*, float*, float*, int, const int32_t*, bool, hipStream_t);
+template hipError_t launch_bwd_medium<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const double>, double*, double*, double*, int, const int32_t*, bool, hipStream_t);
 
 }  // namespace khan

@@ -128,8 +128,8 @@ int backward_dispatch(const float* xs, const float* ys, const float* zs, const i
                                                         n_atoms, khan::kMediumMaxAtoms + 1, order.get(), stream));
     if (st != KHAN_OK) return st;
     // (the workgroup-per-molecule backward kernel measures slower when it walks the molecules in size order)
-    st = hip_status(khan::launch_bwd_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, order.get(), false,
-                                                stream));
+    st = hip_status(khan::launch_bwd_medium<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                   khan::kSmallPreferredMax + 1, order.get(), false, stream));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_bwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
                                                     khan::kSmallPreferredMax, order.get(), stream));
@@ -145,7 +145,10 @@ int backward_dispatch(const double* xs, const double* ys, const double* zs, cons
                                                            n_atoms, 0, nullptr, stream));
     SizeOrder order(macs, n_mols, stream);
     int st = hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                         n_atoms, khan::kSmallMaxAtoms + 1, order.get(), stream));
+                                                         n_atoms, khan::kMediumMaxAtoms + 1, order.get(), stream));
+    if (st != KHAN_OK) return st;
+    st = hip_status(khan::launch_bwd_medium<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                    khan::kSmallMaxAtoms + 1, order.get(), false, stream));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_bwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
                                                      khan::kSmallMaxAtoms, order.get(), stream));

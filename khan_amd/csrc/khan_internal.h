@@ -52,10 +52,11 @@ hipError_t launch_jvp_medium_f32(const float* X, const float* Y, const float* Z,
                                  const int32_t* SIs, const float* VX, const float* VY, const float* VZ,
                                  Buckets<float> out, int min_atoms, const int32_t* order, hipStream_t stream);
 
-hipError_t launch_bwd_medium_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
-                                 const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
-                                 const int32_t* SIs, Buckets<const float> g, float* gX, float* gY,
-                                 float* gZ, const int32_t* order, bool walk_in_order, hipStream_t stream);
+template <typename T>
+hipError_t launch_bwd_medium(const T* X, const T* Y, const T* Z, const int32_t* A,
+                             const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                             const int32_t* SIs, Buckets<const T> g, T* gX, T* gY,
+                             T* gZ, int min_atoms, const int32_t* order, bool walk_in_order, hipStream_t stream);
 
 template <typename T>
 hipError_t launch_bwd_generic(const T* X, const T* Y, const T* Z, const int32_t* A,
