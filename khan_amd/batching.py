@@ -4,6 +4,9 @@
 batch is their concatenation plus, per atom, the index of its molecule inside the batch; the last
 batch is not padded (dataset.py:118-183).
 
+`PackedDataset` holds the same data packed once into flat arrays and assembles a batch with a native,
+multi-threaded gather (csrc/host_batch.c) instead of one numpy operation per molecule.
+
 `DeviceFeeder` is what the reference does with a feed dict and a staging queue
 (khan/training/trainer_multi_tower.py:767-792, 291-303), done for one GPU with PyTorch as the memory
 and stream plumbing: it splits a batch into the flat arrays the ops take (xs, ys, zs, atom types,
@@ -11,9 +14,39 @@ molecule indices), copies them through pinned host buffers with asynchronous hos
 side stream, runs `mol_offsets` and `ani_sort` on the device, and keeps one batch in flight while the
 caller works on the previous one.
 """
+import ctypes
 import math
+import os
 
 import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+HOST_LIB_PATH = os.path.join(_HERE, "csrc", "libkhan_host.so")
+_host_lib = None
+
+
+def _host():
+    """The native batch assembler (csrc/host_batch.c); no GPU code in it."""
+    global _host_lib
+    if _host_lib is None:
+        if not os.path.exists(HOST_LIB_PATH):
+            raise RuntimeError("%s is missing: run `python -m khan_amd.build`" % HOST_LIB_PATH)
+        lib = ctypes.CDLL(HOST_LIB_PATH)
+        vp, i64 = ctypes.c_void_p, ctypes.c_int64
+        lib.khan_host_batch_offsets.restype = i64
+        lib.khan_host_batch_offsets.argtypes = [vp, i64, vp, i64, vp]
+        for name in ("khan_host_gather_f32", "khan_host_gather_f64"):
+            fn = getattr(lib, name)
+            fn.restype = None
+            fn.argtypes = [vp, vp, vp, vp, vp, vp, i64, vp, vp, vp, vp, vp, vp, ctypes.c_int]
+        lib.khan_host_gather_rows3_f64.restype = None
+        lib.khan_host_gather_rows3_f64.argtypes = [vp, vp, vp, i64, vp, vp, ctypes.c_int]
+        _host_lib = lib
+    return _host_lib
+
+
+def _np_ptr(a):
+    return ctypes.c_void_p(a.ctypes.data)
 
 
 class RawDataset:
@@ -56,6 +89,97 @@ class RawDataset:
             mol_grads = None
             if self.all_grads is not None:
                 mol_grads = np.concatenate([np.asarray(self.all_grads[p]) for p in sel], axis=0)
+            yield mol_Xs, mol_ids, mol_yts, mol_grads
+
+
+class PackedDataset:
+    """The same data set packed once into flat arrays: every atom's type and coordinates end to end plus the
+    molecule offsets.  A batch is then gathered by a native routine (parallel over molecules) straight into the
+    flat arrays the ops take, instead of one numpy operation per molecule; `iterate` still yields the
+    reference's tuples.  Coordinates are kept in `dtype`, the precision the featurizer will run in."""
+
+    def __init__(self, all_Xs, all_ys=None, all_grads=None, dtype=np.float32, n_threads=None):
+        counts = np.array([len(m) for m in all_Xs], dtype=np.int64)
+        self.offsets = np.zeros(len(counts) + 1, dtype=np.int64)
+        np.cumsum(counts, out=self.offsets[1:])
+        flat = np.concatenate([np.asarray(m, dtype=np.float64).reshape(-1, 4) for m in all_Xs], axis=0) \
+            if len(counts) else np.zeros((0, 4))
+        self.dtype = np.dtype(dtype)
+        self.types = np.ascontiguousarray(flat[:, 0]).astype(np.int32)
+        self.x, self.y, self.z = (np.ascontiguousarray(flat[:, k], dtype=self.dtype) for k in (1, 2, 3))
+        self.ys = None if all_ys is None else np.asarray(all_ys)
+        if self.ys is not None and len(self.ys) != len(counts):
+            raise ValueError("all_ys must have one entry per molecule")
+        self.grads = None
+        if all_grads is not None:
+            if len(all_grads) != len(counts):
+                raise ValueError("all_grads must have one entry per molecule")
+            self.grads = np.ascontiguousarray(np.concatenate([np.asarray(g, dtype=np.float64).reshape(-1, 3)
+                                                              for g in all_grads], axis=0)) if len(counts) else np.zeros((0, 3))
+        self.n_threads = int(n_threads) if n_threads else min(16, os.cpu_count() or 1)
+
+    @classmethod
+    def from_raw(cls, raw, dtype=np.float32, n_threads=None):
+        return cls(raw.all_Xs, raw.all_ys, raw.all_grads, dtype, n_threads)
+
+    def num_mols(self):
+        return self.offsets.size - 1
+
+    def num_batches(self, batch_size):
+        return math.ceil(self.num_mols() / batch_size)
+
+    def batch_atoms(self, sel):
+        """-> (per-molecule offsets inside the batch [len(sel) + 1], number of atoms) for molecules `sel`."""
+        sel = np.ascontiguousarray(sel, dtype=np.int64)
+        out_off = np.empty(sel.size + 1, dtype=np.int64)
+        n = _host().khan_host_batch_offsets(_np_ptr(self.offsets), self.num_mols(), _np_ptr(sel), sel.size, _np_ptr(out_off))
+        if n < 0:
+            raise IndexError("molecule index out of range")
+        return sel, out_off, int(n)
+
+    def gather_into(self, sel, out_off, xs, ys, zs, types, mol_ids):
+        """Fills the first out_off[-1] elements of the given flat arrays (numpy views, e.g. of pinned tensors)."""
+        for a, dt in ((xs, self.dtype), (ys, self.dtype), (zs, self.dtype), (types, np.int32), (mol_ids, np.int32)):
+            if a.dtype != dt or not a.flags["C_CONTIGUOUS"] or a.size < out_off[-1]:
+                raise ValueError("destination arrays must be contiguous, of the data set's types, and large enough")
+        fn = _host().khan_host_gather_f32 if self.dtype == np.float32 else _host().khan_host_gather_f64
+        fn(_np_ptr(self.offsets), _np_ptr(self.types), _np_ptr(self.x), _np_ptr(self.y), _np_ptr(self.z), _np_ptr(sel),
+           sel.size, _np_ptr(out_off), _np_ptr(xs), _np_ptr(ys), _np_ptr(zs), _np_ptr(types), _np_ptr(mol_ids), self.n_threads)
+
+    def gather(self, sel):
+        """-> (xs, ys, zs, atom types, molecule index per atom) of the batch made of molecules `sel`."""
+        sel, out_off, n = self.batch_atoms(sel)
+        xs, ys, zs = (np.empty(n, dtype=self.dtype) for _ in range(3))
+        types, mol_ids = np.empty(n, dtype=np.int32), np.empty(n, dtype=np.int32)
+        self.gather_into(sel, out_off, xs, ys, zs, types, mol_ids)
+        return xs, ys, zs, types, mol_ids
+
+    def gather_grads(self, sel, out_off):
+        out = np.empty((int(out_off[-1]), 3), dtype=np.float64)
+        _host().khan_host_gather_rows3_f64(_np_ptr(self.offsets), _np_ptr(self.grads), _np_ptr(sel), sel.size,
+                                           _np_ptr(out_off), _np_ptr(out), self.n_threads)
+        return out
+
+    def selections(self, batch_size, shuffle, rng=None):
+        """The molecule indices of every batch, in order (the last batch is not padded)."""
+        rng = np.random.default_rng() if rng is None else rng
+        perm = np.arange(self.num_mols(), dtype=np.int64)
+        if shuffle:
+            rng.shuffle(perm)
+        for batch_idx in range(self.num_batches(batch_size)):
+            yield perm[batch_idx * batch_size:min((batch_idx + 1) * batch_size, self.num_mols())]
+
+    def iterate(self, batch_size, shuffle, fuzz=None, rng=None):
+        """Same tuples as RawDataset.iterate: (mol_Xs [N,4] float64, mol_ids, mol_yts or None, mol_grads or None)."""
+        rng = np.random.default_rng() if rng is None else rng
+        for sel in self.selections(batch_size, shuffle, rng):
+            sel, out_off, n = self.batch_atoms(sel)
+            xs, ys, zs, types, mol_ids = self.gather(sel)
+            mol_Xs = np.stack([types.astype(np.float64), xs.astype(np.float64), ys.astype(np.float64), zs.astype(np.float64)], axis=1)
+            if fuzz is not None:
+                mol_Xs[:, 1:4] += rng.uniform(-fuzz, fuzz, (n, 3))
+            mol_yts = None if self.ys is None else list(self.ys[sel])
+            mol_grads = None if self.grads is None else self.gather_grads(sel, out_off)
             yield mol_Xs, mol_ids, mol_yts, mol_grads
 
 
@@ -114,9 +238,9 @@ class DeviceFeeder:
             self._pinned[slot] = cur
         return cur
 
-    def _enqueue(self, slot, item):
+    def _fill_from_tuple(self, slot, item):
+        """Reference-style tuple -> staging set; returns (n atoms, n molecules, labels, gradients)."""
         import torch
-        from . import ops
         mol_Xs, mol_ids, mol_yts, mol_grads = item
         xs, ys, zs, types, mids = split_columns(mol_Xs, mol_ids, self.dtype)
         n = xs.size
@@ -129,6 +253,32 @@ class DeviceFeeder:
         st["xyz"][2, :n] = torch.from_numpy(zs)
         st["ints"][0, :n] = torch.from_numpy(types)
         st["ints"][1, :n] = torch.from_numpy(mids)
+        return n, n_mols, mol_yts, mol_grads
+
+    def _fill_from_packed(self, slot, sel):
+        """Molecule selection of a PackedDataset -> staging set, gathered natively into the pinned buffers."""
+        ds = self.dataset
+        sel, out_off, n = ds.batch_atoms(sel)
+        st = self._staging(slot, n)
+        if self._events[slot] is not None:
+            self._events[slot].synchronize()
+        xyz, ints = st["xyz"].numpy(), st["ints"].numpy()
+        ds.gather_into(sel, out_off, xyz[0], xyz[1], xyz[2], ints[0], ints[1])
+        if self.fuzz is not None:
+            rng = np.random.default_rng() if self.rng is None else self.rng
+            xyz[:, :n] += rng.uniform(-self.fuzz, self.fuzz, (3, n)).astype(xyz.dtype)
+        labels = None if ds.ys is None else ds.ys[sel]            # an array here (a list from a RawDataset)
+        grads = None if ds.grads is None else ds.gather_grads(sel, out_off)
+        return n, sel.size, labels, grads
+
+    def _enqueue(self, slot, item):
+        import torch
+        from . import ops
+        if isinstance(self.dataset, PackedDataset):
+            n, n_mols, mol_yts, mol_grads = self._fill_from_packed(slot, item)
+        else:
+            n, n_mols, mol_yts, mol_grads = self._fill_from_tuple(slot, item)
+        st = self._pinned[slot]
         b = DeviceBatch()
         with torch.cuda.stream(self.stream):
             # each row of the staging arrays is contiguous pinned memory: five asynchronous copies
@@ -149,7 +299,13 @@ class DeviceFeeder:
         return b
 
     def __iter__(self):
-        it = self.dataset.iterate(self.batch_size, self.shuffle, self.fuzz, self.rng)
+        if isinstance(self.dataset, PackedDataset):
+            if self.dataset.dtype != np.dtype(self.dtype):
+                raise TypeError("the packed data set holds %s coordinates, the feeder was asked for %s"
+                                % (self.dataset.dtype, np.dtype(self.dtype)))
+            it = self.dataset.selections(self.batch_size, self.shuffle, self.rng)
+        else:
+            it = self.dataset.iterate(self.batch_size, self.shuffle, self.fuzz, self.rng)
         slot, ahead = 0, None
         for item in it:
             nxt = self._enqueue(slot, item)

@@ -2,6 +2,7 @@
 
   khan_amd/csrc/libkhan_aev.so      HIP kernels + C ABI, compiled for gfx950 with hipcc
   khan_amd/csrc/libkhan_datagen.so  host-only synthetic batch generator (gcc)
+  khan_amd/csrc/libkhan_host.so     host-only batch assembly (gcc, OpenMP)
 
 Run as ``python -m khan_amd.build`` or through ``__graft_entry__.build()``.
 """
@@ -67,8 +68,15 @@ def build_datagen():
     return out
 
 
+def build_host():
+    out = os.path.join(CSRC, "libkhan_host.so")
+    _run(["gcc", "-std=gnu99", "-O2", "-fPIC", "-fopenmp", "-fvisibility=hidden", "-shared", "-o", out,
+          os.path.join(CSRC, "host_batch.c")])
+    return out
+
+
 def build_all():
-    return [build_hip(), build_datagen()]
+    return [build_hip(), build_datagen(), build_host()]
 
 
 if __name__ == "__main__":

@@ -20,10 +20,13 @@ def _ensure_built():
         subprocess.run(["make", "-C", os.path.join(ROOT, "oracle"), "all"], check=True)
     datagen_so = os.path.join(ROOT, "khan_amd", "csrc", "libkhan_datagen.so")
     aev_so = os.path.join(ROOT, "khan_amd", "csrc", "libkhan_aev.so")
-    if not os.path.exists(datagen_so) or not os.path.exists(aev_so):
+    host_so = os.path.join(ROOT, "khan_amd", "csrc", "libkhan_host.so")
+    if not os.path.exists(datagen_so) or not os.path.exists(aev_so) or not os.path.exists(host_so):
         from khan_amd import build
         if not os.path.exists(datagen_so):
             build.build_datagen()
+        if not os.path.exists(host_so):
+            build.build_host()
         if not os.path.exists(aev_so):
             build.build_hip()
 

@@ -85,3 +85,71 @@ def test_device_feeder_feeds_the_featurizer():
         assert np.all(np.abs(got - ref) <= 1e-6 + 1e-5 * np.abs(ref))
         seen += k
     assert seen == 41
+
+
+# ------------------------------------------------------------------------------- packed data set (native gather)
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_packed_dataset_yields_what_the_raw_one_yields(dtype):
+    mols = _molecules(29, seed=11)
+    ys = [float(3 * k) for k in range(len(mols))]
+    grads = [np.random.default_rng(k).normal(size=(len(m), 3)) for k, m in enumerate(mols)]
+    raw = batching.RawDataset(mols, ys, grads)
+    packed = batching.PackedDataset.from_raw(raw, dtype=dtype, n_threads=3)
+    assert packed.num_mols() == 29 and packed.num_batches(8) == 4
+    for shuffle in (False, True):
+        a = list(raw.iterate(8, shuffle, rng=np.random.default_rng(5)))
+        b = list(packed.iterate(8, shuffle, rng=np.random.default_rng(5)))
+        assert len(a) == len(b) == 4
+        for (Xa, ia, ya, ga), (Xb, ib, yb, gb) in zip(a, b):
+            # coordinates pass through the data set's precision (the generator's are float32 values)
+            assert Xb.dtype == np.float64 and np.array_equal(Xa.astype(dtype), Xb.astype(dtype))
+            assert ib.dtype == np.int32 and np.array_equal(ia, ib)
+            assert ya == yb and np.array_equal(ga, gb)
+
+
+def test_packed_dataset_gather_edge_cases():
+    mols = _molecules(7, seed=2)
+    packed = batching.PackedDataset(mols, dtype=np.float64)
+    xs, ys, zs, types, ids = packed.gather([6, 0, 0, 3])               # any order, repeats allowed
+    want = np.concatenate([mols[6], mols[0], mols[0], mols[3]], axis=0)
+    assert np.array_equal(xs, want[:, 1]) and np.array_equal(zs, want[:, 3]) and np.array_equal(types, want[:, 0].astype(np.int32))
+    assert np.array_equal(ids, np.repeat(np.arange(4), [len(mols[6]), len(mols[0]), len(mols[0]), len(mols[3])]))
+    assert packed.gather([])[0].size == 0
+    with pytest.raises(IndexError):
+        packed.gather([7])
+    with pytest.raises(IndexError):
+        packed.gather([-1])
+    sel, off, n = packed.batch_atoms([1, 2])
+    small = np.empty(n - 1, dtype=np.float64)
+    with pytest.raises(ValueError):
+        packed.gather_into(sel, off, small, small, small, np.empty(n, np.int32), np.empty(n, np.int32))
+    assert batching.PackedDataset([]).num_mols() == 0 and list(batching.PackedDataset([]).iterate(4, False)) == []
+    fuzzed = next(iter(packed.iterate(7, False, fuzz=0.02, rng=np.random.default_rng(1))))[0]
+    plain = next(iter(packed.iterate(7, False)))[0]
+    d = np.abs(fuzzed[:, 1:] - plain[:, 1:])
+    assert np.array_equal(fuzzed[:, 0], plain[:, 0]) and 0.0 < d.max() <= 0.02
+
+
+@pytest.mark.gpu
+def test_device_feeder_from_a_packed_dataset_matches_the_raw_one():
+    torch = pytest.importorskip("torch")
+    mols = _molecules(53, seed=80)
+    labels = [float(k) for k in range(len(mols))]
+    grads = [np.full((len(m), 3), k, dtype=np.float64) for k, m in enumerate(mols)]
+    raw = batching.RawDataset(mols, labels, grads)
+    packed = batching.PackedDataset.from_raw(raw, dtype=np.float32)
+    for shuffle in (False, True):
+        fa = batching.DeviceFeeder(raw, 20, shuffle=shuffle, rng=np.random.default_rng(9))
+        fb = batching.DeviceFeeder(packed, 20, shuffle=shuffle, rng=np.random.default_rng(9))
+        n_batches = 0
+        for a, b in zip(fa, fb):
+            a.wait()
+            b.wait()
+            for name in ("xs", "ys", "zs", "atom_types", "mol_idxs", "mol_atom_counts", "mol_offsets", "scatter_idxs",
+                         "gather_idxs", "atom_counts", "grads"):
+                assert torch.equal(getattr(a, name), getattr(b, name)), name
+            assert a.n_mols == b.n_mols and a.labels == list(b.labels)
+            n_batches += 1
+        assert n_batches == 3
+    with pytest.raises(TypeError):
+        list(batching.DeviceFeeder(packed, 20, dtype=np.float64))
