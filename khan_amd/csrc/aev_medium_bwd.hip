@@ -333,7 +333,9 @@ hipError_t launch_bwd_medium(const T* X, const T* Y, const T* Z, const int32_t* 
 {
     if (n_mols <= 0) return hipSuccess;
     // workgroups walk the molecules with the grid's stride and skip those of other sizes
-    const unsigned blocks = static_cast<unsigned>(n_mols < 4096 ? n_mols : 4096);
+    // (in float64 the working set lets one workgroup run per CU: a smaller grid costs less when it only skips)
+    const int32_t cap = sizeof(T) == 4 ? 4096 : 1024;
+    const unsigned blocks = static_cast<unsigned>(n_mols < cap ? n_mols : cap);
     aev_bwd_medium_kernel<T><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ, min_atoms,
                                                                   order, walk_in_order);
     return hipGetLastError();

@@ -8,11 +8,13 @@
 // khan/training/trainer_multi_tower.py:112-119); it is the closed form
 //     dL/dx_i = g_m K q_i sum_{j != i} q_j d/dr[(1 - f_C)/r] (x_i - x_j)/r.
 //
-// One wavefront per molecule, one lane per atom i (strided for molecules above 64 atoms); every lane
-// walks all partners j, whose loads are wave-uniform.  Each output element is written once by its
-// own lane: no atomics and no pre-zeroing.
-#include "khan_internal.h"
-#include "khan_params.h"
+// One wavefront per molecule.  Up to 64 atoms a step evaluates 64 (i, j) pairs at once -- 4 atoms i x 16
+// partners j for molecules of up to 16 atoms, 2 x 32 up to 32, 1 x 64 above -- with the partners' data
+// held in the lanes, and the sums over j are in-wave DPP reductions (a lane per atom i walking all j
+// would leave four fifths of the lanes idle on a 12-atom molecule).  Above 64 atoms a lane takes the
+// atoms i = lane, lane + 64, ... and walks all partners j, whose loads are wave-uniform.  Each output
+// element is written once: no atomics and no pre-zeroing.
+#include "aev_small_common.h"
 
 namespace khan {
 
@@ -45,6 +47,26 @@ __global__ __launch_bounds__(256) void charge_energy_kernel(
     const T rc = static_cast<T>(kR_Rc_f), pi_rc = static_cast<T>(kPi / static_cast<double>(kR_Rc_f));
     const T K = static_cast<T>(kChargeK_f);
     T acc = T(0);
+    if (n <= 64) {
+        const int logW = n <= 16 ? 4 : n <= 32 ? 5 : 6;
+        const int W = 1 << logW, G = 64 >> logW;
+        const int grp = lane >> logW, jl = lane & (W - 1);
+        const bool jok = jl < n;
+        const T xj = jok ? X[off + jl] : T(0), yj = jok ? Y[off + jl] : T(0), zj = jok ? Z[off + jl] : T(0),
+                qj = jok ? Q[off + jl] : T(0);
+        for (int i0 = 0; i0 < n; i0 += G) {
+            const int i = i0 + grp;                      // lane i of the first group holds atom i
+            const T xi = __shfl(xj, i & 63, 64), yi = __shfl(yj, i & 63, 64), zi = __shfl(zj, i & 63, 64),
+                    qi = __shfl(qj, i & 63, 64);
+            const bool valid = (i < n) && jok && (jl > i);
+            T u, du;
+            pair_terms(valid ? xi - xj : T(1), valid ? yi - yj : T(0), valid ? zi - zj : T(0), pi_rc, rc, u, du);
+            acc += valid ? K * qi * qj * u : T(0);
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) E[mol] = acc;
+        return;
+    }
     for (int i0 = 0; i0 < n; i0 += 64) {
         const int i = i0 + lane;
         const bool active = i < n;
@@ -75,6 +97,38 @@ __global__ __launch_bounds__(256) void charge_grad_kernel(
     const int n = MACs[mol], off = MOs[mol];
     const T rc = static_cast<T>(kR_Rc_f), pi_rc = static_cast<T>(kPi / static_cast<double>(kR_Rc_f));
     const T gK = grads[mol] * static_cast<T>(kChargeK_f);
+    if (n <= 64) {
+        const int logW = n <= 16 ? 4 : n <= 32 ? 5 : 6;
+        const int W = 1 << logW, G = 64 >> logW;
+        const int grp = lane >> logW, jl = lane & (W - 1);
+        const bool jok = jl < n;
+        const T xj = jok ? X[off + jl] : T(0), yj = jok ? Y[off + jl] : T(0), zj = jok ? Z[off + jl] : T(0),
+                qj = jok ? Q[off + jl] : T(0);
+        for (int i0 = 0; i0 < n; i0 += G) {
+            const int i = i0 + grp;                      // lane i of the first group holds atom i
+            const T xi = __shfl(xj, i & 63, 64), yi = __shfl(yj, i & 63, 64), zi = __shfl(zj, i & 63, 64),
+                    qi = __shfl(qj, i & 63, 64);
+            const bool valid = (i < n) && jok && (jl != i);
+            const T dx = valid ? xi - xj : T(1), dy = valid ? yi - yj : T(0), dz = valid ? zi - zj : T(0);
+            T u, du;
+            pair_terms(dx, dy, dz, pi_rc, rc, u, du);
+            const T w = valid ? qj * du : T(0);
+            // sums over the W partners of the group end up in its last lane
+            const T dq = group_sum_to_last_lane(valid ? qj * u : T(0), logW);
+            const T fx = group_sum_to_last_lane(w * dx, logW);
+            const T fy = group_sum_to_last_lane(w * dy, logW);
+            const T fz = group_sum_to_last_lane(w * dz, logW);
+            if (jl == W - 1 && i < n) {
+                if (q_grads) q_grads[off + i] = gK * dq;
+                if (gX) {
+                    gX[off + i] = gK * qi * fx;
+                    gY[off + i] = gK * qi * fy;
+                    gZ[off + i] = gK * qi * fz;
+                }
+            }
+        }
+        return;
+    }
     for (int i = lane; i < n; i += 64) {
         const T xi = X[off + i], yi = Y[off + i], zi = Z[off + i], qi = Q[off + i];
         T dq = T(0), fx = T(0), fy = T(0), fz = T(0);
