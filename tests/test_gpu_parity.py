@@ -268,6 +268,47 @@ def test_edge_shapes(ops):
     check_forward_backward(ops, Case(xyz[:, 0], xyz[:, 1], xyz[:, 2], A, mi, len(mols)))
 
 
+def _boundary_case():
+    """One random box per atom count next to every limit the dispatch and the kernels know: scan shapes
+    (16 / 17, 32 / 33), one wavefront (64 / 65), one workgroup (256 / 257), in mixed order."""
+    rng = np.random.default_rng(21)
+    mols = []
+    for n in (33, 16, 257, 64, 17, 256, 32, 65, 1, 2):
+        side = (n / 0.09) ** (1 / 3)
+        pts = []
+        while len(pts) < n:
+            p = rng.uniform(0, side, 3)
+            if all(np.linalg.norm(p - q) >= 0.9 for q in pts):
+                pts.append(p)
+        mols.append((rng.integers(0, 4, n), np.array(pts)))
+    A = np.concatenate([m[0] for m in mols]).astype(np.int32)
+    xyz = np.concatenate([m[1] for m in mols]).astype(np.float32).astype(np.float64)
+    mi = np.concatenate([np.full(len(m[0]), k) for k, m in enumerate(mols)]).astype(np.int32)
+    return Case(xyz[:, 0], xyz[:, 1], xyz[:, 2], A, mi, len(mols))
+
+
+def test_size_class_boundaries(ops):
+    say("case: molecules of 16/17, 32/33, 64/65, 256/257 atoms: features, gradients, grad-inverse, charges")
+    c = _boundary_case()
+    check_forward_backward(ops, c)
+    _check_grad_inverse(ops, c)
+    q = np.random.default_rng(3).normal(0.0, 0.3, c.N)
+    gm = np.random.default_rng(4).standard_normal(c.n_mols)
+    E64 = ob.ani_charge(c.X, c.Y, c.Z, q, c.MOs, c.MACs, dtype=np.float64)
+    Eabs = ob.ani_charge(c.X, c.Y, c.Z, np.abs(q), c.MOs, c.MACs, dtype=np.float64)
+    dq64 = ob.ani_charge_grad(c.X, c.Y, c.Z, q, c.MOs, c.MACs, gm, dtype=np.float64)
+    dx64 = np.stack(ob.ani_charge_grad_xyz(c.X, c.Y, c.Z, q, c.MOs, c.MACs, gm, dtype=np.float64), axis=1)
+    mos, macs = dev(c.MOs), dev(c.MACs)
+    for ndt, rtol in ((np.float32, F32_RTOL), (np.float64, F64_RTOL)):
+        X, Y, Z, Q, G = dev(c.X, ndt), dev(c.Y, ndt), dev(c.Z, ndt), dev(q, ndt), dev(gm, ndt)
+        assert_close("charge energy %s" % ndt.__name__, host(ops.ani_charge(X, Y, Z, Q, mos, macs)), E64, rtol, 0.0,
+                     scale=np.maximum(Eabs, 1e-300))
+        qg, gx, gy, gz = ops.ani_charge_grad_xyz(X, Y, Z, Q, mos, macs, G)
+        assert_close("charge dE/dq %s" % ndt.__name__, host(qg), dq64, rtol, 0.0, scale=mol_scale(dq64, c.MOs, c.MACs))
+        assert_close("charge dE/dxyz %s" % ndt.__name__, host(torch.stack([gx, gy, gz], dim=1)), dx64, rtol, 0.0,
+                     scale=mol_scale(dx64, c.MOs, c.MACs))
+
+
 def test_empty_batch(ops):
     say("case: empty batch (0 atoms, 0 molecules)")
     e32 = torch.empty(0, dtype=torch.float32, device="cuda:0")
