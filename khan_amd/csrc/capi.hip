@@ -40,12 +40,13 @@ bool aligned16(const khan::Buckets<const T>& g)
 
 // Stream-ordered scratch holding the molecule indices by decreasing size for the one-wavefront kernels.
 // No order (the kernels then take molecules as they come) while the stream is being captured into a graph,
-// for tiny batches, or when the allocation fails.
+// for small batches, or when the allocation fails.
 class SizeOrder {
 public:
     SizeOrder(const int32_t* macs, int32_t n_mols, hipStream_t stream) : stream_(stream)
     {
-        if (n_mols < 512) return;
+        // below a few thousand molecules every wavefront of the launch is resident at once and the order buys nothing
+        if (n_mols < 2048) return;
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
             (void)hipGetLastError();
