@@ -50,7 +50,7 @@ __device__ __forceinline__ void fwd_lds_init(FwdWaveLds<T, kJvp>& S, int lane)
 
 // Segment table, phases 1 and 2 and the zero fill of empty blocks for centres 0..nb-1 of a batch.
 // `row_of_centre(b)` returns the address of centre b's 384-float output row; it is called by all
-// lanes together, with a per-lane b for the segment table and a wave-uniform b for the zero fill.
+// lanes together, with a per-lane b.
 // With kJvp the same sums are formed for the derivative of every term along the atoms' incoming vectors:
 // d(A_t G_s P) = dA_t (G_s P) + A_t (dG_s P + G_s dP), two products per record instead of one.
 template <typename T, bool kJvp, typename RowOfCentre>

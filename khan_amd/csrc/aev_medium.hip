@@ -8,7 +8,7 @@
 //            cutoff are appended to a (r, f_C) list, partners inside the angular cutoff to the centre's
 //            list of unit vectors.  Chunks are consecutive ranges of the sorted order, so both lists
 //            stay sorted by type.
-//   radial   lanes = (slot of 4) x (shell): a centre's list is walked type by type, sixteen entries per
+//   radial   lanes = (slot of 4) x (shell): a centre's list is walked type by type, four entries per
 //            trip, and 16 finished floats per type go straight to the row.
 //   angular  segment table, triple-per-lane factors and the (theta_t, Rs_s) accumulation of the shared
 //            batch routine.

@@ -9,15 +9,17 @@
 //            Partners inside the radial cutoff go to a (r, f_C) list, partners inside the angular
 //            cutoff to a per-centre list of unit vectors, both compacted with ballot + popcount.
 //   radial   lanes = (group of 16) x (shell): a group walks one centre's radial list type by type,
-//            four entries per trip, and stores 16 finished floats per (centre, type).
+//            two entries per trip, and stores 16 finished floats per (centre, type).
 //   phase 1  the triples (centre; j<k) of the six centres are enumerated in (centre, type-pair)
 //            order, each segment padded to an even length, and dealt one per lane.  A lane computes
 //            what depends on the triple alone: the 8 angular factors (1+cos(theta-theta_t))^8 and the
 //            4 radial factors 2^-7 f_C f_C exp(-eta (rho-Rs_s)^2).  12 floats go to LDS.
-//   phase 2  lanes = (half, theta_t, Rs_s).  The halves take alternate records; a lane reads A_t and
-//            G_s of its record and does one FMA into a register.  Segment boundaries are a bit mask
+//   phase 2  lanes = (half, theta_t, Rs_s).  The halves take alternate records; a lane reads G_s of its
+//            record (and, in float, one A_t per four records, shared inside its quad) and does one FMA
+//            into a register.  Segment boundaries are a bit mask
 //            held in scalar registers; at a boundary the halves are added and 32 floats are stored
-//            straight to the row in HBM.  Segments without triples are stored as zeros at the end.
+//            straight to the row in HBM.  Segments without triples are cleared by their lanes of the
+//            segment table.
 // No atomics and no pre-zeroed output.  A centre with more than 32 angular neighbours (the 3.1 A
 // sphere holds about 25 atoms at the densest packings tested) is redone by the general-shape
 // per-centre routine.  Semantics: gpu_featurizer/kernel_cpu.cpp:406-537.
@@ -31,10 +33,10 @@ namespace {
 // number of slots), and two measured faster than one, three or four
 constexpr int kRadTrip = 2;
 
-// float: 4 wavefronts per SIMD (LDS 9.8 KB, <= 128 VGPRs); double: 2 (LDS 19.6 KB)
 // With kJvp the kernel computes the Jacobian-vector product instead (featurize_grad_inverse): every term of
 // the forward sums is replaced by its derivative along the per-atom vectors (VX, VY, VZ).
-// float: 4 wavefronts per SIMD (LDS 9.8 KB, <= 128 VGPRs); double or kJvp: 2 (LDS 19 KB); both: 1.
+// float: 4 wavefronts per SIMD (LDS 9.8 KB, <= 128 VGPRs; the kernel loses a fifth of its speed at three);
+// double or kJvp: 2 (LDS 19 KB); both: 1.
 template <typename T, bool kJvp>
 __global__ __launch_bounds__(64 * kWavesPerBlock)
 __attribute__((amdgpu_waves_per_eu((sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1), (sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1))))
