@@ -265,22 +265,37 @@ void aev_bwd_small_kernel(
             const int self = live ? lane : 0;
             // -------------------------------------------- gather: partners get their slot, the centre minus the sum
             const int atom = S.pool.nbr_idx[self];
-            for (int bb = 0; bb < nb; ++bb) {
-                if (uniform(pf[bb + 1] - pf[bb]) == 0) continue;
-                const bool mine = live && (bs == bb);
-                if (mine) {
-                    S.force[0][atom] += f.x;
-                    S.force[1][atom] += f.y;
-                    S.force[2][atom] += f.z;
+            // one add-scan over the lanes per component: a centre's list is a run of lanes, its sum the
+            // difference of two prefix values (lane b takes centre b's)
+            const T px = group_sum_to_last_lane(live ? f.x : T(0), 6);
+            const T py = group_sum_to_last_lane(live ? f.y : T(0), 6);
+            const T pz = group_sum_to_last_lane(live ? f.z : T(0), 6);
+            {
+                const int lo = sel6(min(lane, kB - 1), pf[0], pf[1], pf[2], pf[3], pf[4], pf[5]);
+                const int hi = sel6(min(lane, kB - 1), pf[1], pf[2], pf[3], pf[4], pf[5], pf[6]);
+                const int at_hi = max(hi - 1, 0) << 2, at_lo = max(lo - 1, 0) << 2;
+                T sx = lane_fetch(px, at_hi), sy = lane_fetch(py, at_hi), sz = lane_fetch(pz, at_hi);
+                const T qx = lane_fetch(px, at_lo), qy = lane_fetch(py, at_lo), qz = lane_fetch(pz, at_lo);
+                if (lo > 0) {
+                    sx -= qx;
+                    sy -= qy;
+                    sz -= qz;
                 }
-                const T sx = group_sum_to_last_lane(mine ? f.x : T(0), 6);
-                const T sy = group_sum_to_last_lane(mine ? f.y : T(0), 6);
-                const T sz = group_sum_to_last_lane(mine ? f.z : T(0), 6);
-                if (lane == 63) {
-                    const int i_b = lane_read(cord, min(c0 + bb, 63));
+                const int i_b = __builtin_amdgcn_ds_bpermute(min(c0 + lane, 63) << 2, cord);
+                if (lane < nb && hi > lo) {          // the centres of a batch are distinct atoms
                     S.force[0][i_b] -= sx;
                     S.force[1][i_b] -= sy;
                     S.force[2][i_b] -= sz;
+                }
+            }
+            wave_lds_fence();
+            // partners: one centre at a time, so the atoms of a pass are distinct
+            for (int bb = 0; bb < nb; ++bb) {
+                if (uniform(pf[bb + 1] - pf[bb]) == 0) continue;
+                if (live && (bs == bb)) {
+                    S.force[0][atom] += f.x;
+                    S.force[1][atom] += f.y;
+                    S.force[2][atom] += f.z;
                 }
                 wave_lds_fence();
             }

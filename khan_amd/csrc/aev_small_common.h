@@ -143,6 +143,18 @@ __device__ __forceinline__ double dpp_take_f(double v)
     const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(b >> 32), kCtrl, kRowMask, 0xf, false));
     return __longlong_as_double(static_cast<long long>((static_cast<unsigned long long>(hi) << 32) | lo));
 }
+// the value lane (byte_index / 4) holds (per-lane source; every lane takes part)
+__device__ __forceinline__ float lane_fetch(float v, int byte_index)
+{
+    return __int_as_float(__builtin_amdgcn_ds_bpermute(byte_index, __float_as_int(v)));
+}
+__device__ __forceinline__ double lane_fetch(double v, int byte_index)
+{
+    const long long b = __double_as_longlong(v);
+    const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(byte_index, static_cast<int>(b)));
+    const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(byte_index, static_cast<int>(b >> 32)));
+    return __longlong_as_double(static_cast<long long>((static_cast<unsigned long long>(hi) << 32) | lo));
+}
 __device__ __forceinline__ double group_sum_to_last_lane(double v, int log_group)
 {
     v += dpp_take_f<0x111, 0xf>(v);
