@@ -139,16 +139,23 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                 fy = sc * e.y;
                 fz = sc * e.z;
             }
-            // the pairs of one centre are summed in the wave (a handful of centres per 64 pairs) and added once
-            unsigned long long todo = wave_ballot(lane < count);
-            while (todo) {
-                const int c0 = lane_read(c, lowest_bit(todo));
-                const bool mine = c == c0;
-                todo &= ~wave_ballot(mine);
-                const T sx = group_sum_to_last_lane(mine ? fx : T(0), 6);
-                const T sy = group_sum_to_last_lane(mine ? fy : T(0), 6);
-                const T sz = group_sum_to_last_lane(mine ? fz : T(0), 6);
-                if (lane == 63) add_force(c0, sx, sy, sz);
+            // The pairs of one centre are a run of lanes (the queue is filled centre after centre): one add-scan
+            // per component, and the last lane of every run adds the difference of two prefix values to its
+            // centre -- one atomic per centre and component, issued for all centres of the step at once.
+            const T px = group_sum_to_last_lane(fx, 6), py = group_sum_to_last_lane(fy, 6), pz = group_sum_to_last_lane(fz, 6);
+            const int c_prev = __builtin_amdgcn_ds_bpermute(max(lane - 1, 0) << 2, c);
+            const int c_next = __builtin_amdgcn_ds_bpermute(min(lane + 1, 63) << 2, c);
+            const bool in_q = lane < count;
+            const unsigned long long starts = wave_ballot(in_q && (lane == 0 || c_prev != c));
+            const bool run_end = in_q && (lane == count - 1 || c_next != c);
+            // first lane of this lane's run: the highest start at or below the lane
+            const unsigned long long below = starts & ((lane == 63) ? ~0ull : ((2ull << lane) - 1ull));
+            const int first = below ? 63 - __clzll(static_cast<long long>(below)) : 0;
+            const int at = max(first - 1, 0) << 2;
+            const T qx = lane_fetch(px, at), qy = lane_fetch(py, at), qz = lane_fetch(pz, at);
+            if (run_end) {
+                const bool whole = first == 0;
+                add_force(c, whole ? px : px - qx, whole ? py : py - qy, whole ? pz : pz - qz);
             }
         };
         auto radial_drain = [&]() {
@@ -310,12 +317,23 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
 
             // ------------------------------------------------ gather
             if (live) add_force(P.nbr_idx[lane], f.x, f.y, f.z);
-            for (int bb = 0; bb < nb; ++bb) {
-                const bool mine = live && (bs == bb);
-                const T sx = group_sum_to_last_lane(mine ? f.x : T(0), 6);
-                const T sy = group_sum_to_last_lane(mine ? f.y : T(0), 6);
-                const T sz = group_sum_to_last_lane(mine ? f.z : T(0), 6);
-                if (lane == 63) add_force(lane_read(cv, bb), -sx, -sy, -sz);
+            {
+                // a centre's list is a run of lanes: its sum is the difference of two values of an add-scan,
+                // and lane b adds centre b's
+                const T px = group_sum_to_last_lane(live ? f.x : T(0), 6);
+                const T py = group_sum_to_last_lane(live ? f.y : T(0), 6);
+                const T pz = group_sum_to_last_lane(live ? f.z : T(0), 6);
+                const int lo = __builtin_amdgcn_ds_bpermute(min(lane, 63) << 2, pfv);          // pfv of lane b = first slot of centre b
+                const int hi = __builtin_amdgcn_ds_bpermute(min(lane + 1, 63) << 2, pfv);
+                const int at_hi = max(hi - 1, 0) << 2, at_lo = max(lo - 1, 0) << 2;
+                T sx = lane_fetch(px, at_hi), sy = lane_fetch(py, at_hi), sz = lane_fetch(pz, at_hi);
+                const T qx = lane_fetch(px, at_lo), qy = lane_fetch(py, at_lo), qz = lane_fetch(pz, at_lo);
+                if (lo > 0) {
+                    sx -= qx;
+                    sy -= qy;
+                    sz -= qz;
+                }
+                if (lane < nb && hi > lo) add_force(cv, -sx, -sy, -sz);      // cv of lane b = centre b
             }
             wave_lds_fence();
         }
