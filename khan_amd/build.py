@@ -62,6 +62,79 @@ def build_hip(jobs=4):
     return out
 
 
+DPP_SOURCES = ["aev_small.hip", "aev_medium.hip"]     # translation units that use fma_quad (aev_small_common.h)
+
+
+def check_dpp_operands(asm_text, name="<asm>"):
+    """The multiply-add with a lane-exchange operand (written as inline asm, which the compiler's hazard
+    handling does not look into) needs two wait states between a vector instruction that writes the exchanged
+    register and itself.  Checks every use in the generated code: none of the two instructions before it -- on
+    the fall-through path and before every branch to a label in between -- may be a vector instruction that
+    writes that register.  Raises on a violation (the remedy is an `s_nop 1` in front of the instruction)."""
+    import re
+    lines = [l.strip() for l in asm_text.split("\n")]
+    code = [(i, l) for i, l in enumerate(lines) if l and not l.startswith((";", ".", "//")) or re.match(r"^\.LBB\d+_\d+:", l or "")]
+    is_label = lambda l: re.match(r"^\.LBB\d+_\d+:", l) is not None
+    branches = {}
+    for k, (_, l) in enumerate(code):
+        m = re.match(r"^s_c?branch\S*\s+(\.LBB\d+_\d+)", l)
+        if m:
+            branches.setdefault(m.group(1) + ":", []).append(k)
+
+    def writes(l, reg):
+        m = re.match(r"^(v_\S+)\s+([^,\s]+)", l)
+        if not m or m.group(1).startswith(("v_cmp", "v_readlane", "v_readfirstlane")):
+            return False
+        dst = m.group(2)
+        r = re.match(r"^v\[(\d+):(\d+)\]$", dst)
+        n = int(reg[1:])
+        if r:
+            return int(r.group(1)) <= n <= int(r.group(2))
+        return dst == reg
+
+    def hazard_before(k, reg, budget):
+        """True if a vector write of `reg` lies within `budget` instructions before position k on any path."""
+        j = k - 1
+        while budget > 0 and j >= 0:
+            l = code[j][1]
+            if is_label(l):
+                for b in branches.get(l.split()[0], []):
+                    if hazard_before(b, reg, budget):
+                        return True
+                j -= 1
+                continue
+            if writes(l, reg):
+                return True
+            budget -= 1
+            j -= 1
+        return False
+
+    uses = 0
+    for k, (i, l) in enumerate(code):
+        m = re.match(r"^v_fmac_f32_dpp\s+v\d+,\s*(v\d+),", l)
+        if m:
+            uses += 1
+            if hazard_before(k, m.group(1), 2):
+                raise RuntimeError("%s line %d: a vector instruction writes %s within two instructions of its "
+                                   "lane-exchange read" % (name, i + 1, m.group(1)))
+    return uses
+
+
+def check_dpp_sources():
+    """Compiles the translation units that use the lane-exchange multiply-add to assembly and checks them."""
+    hipcc = _hipcc()
+    total = 0
+    for src in DPP_SOURCES:
+        cmd = [hipcc] + [f for f in HIPCC_FLAGS if f != "-Wall"] + ["-S", "--cuda-device-only", "-o", "-", os.path.join(CSRC, src)]
+        print("+", " ".join(cmd), flush=True)
+        out = subprocess.run(cmd, check=True, capture_output=True, text=True).stdout
+        total += check_dpp_operands(out, src)
+    if total == 0:
+        raise RuntimeError("no lane-exchange multiply-add found in %s: the check looks at the wrong files" % DPP_SOURCES)
+    print("lane-exchange operands: %d uses checked" % total, flush=True)
+    return total
+
+
 def build_datagen():
     out = os.path.join(CSRC, "libkhan_datagen.so")
     _run(["gcc", "-std=gnu99", "-O2", "-fPIC", "-shared", "-o", out, os.path.join(CSRC, "datagen.c"), "-lm"])
@@ -76,7 +149,9 @@ def build_host():
 
 
 def build_all():
-    return [build_hip(), build_datagen(), build_host()]
+    outs = [build_hip(), build_datagen(), build_host()]
+    check_dpp_sources()
+    return outs
 
 
 if __name__ == "__main__":

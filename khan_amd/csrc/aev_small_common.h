@@ -62,13 +62,14 @@ __device__ __forceinline__ void store_global(double* p, double v)
 // acc + a' * g, where a' is the value of `a` held by lane k of this lane's quad (k is a constant after unrolling).
 // The lane exchange is a modifier of the multiply-add, not an instruction of its own.  It reads `a` early: two
 // wait states have to lie between a vector instruction that writes `a` and this one, and the compiler does not
-// see inside the asm, so they are part of it (about 1 % of the forward kernel; the exchange saves 2 %).
+// see inside the asm.  `a` comes from an LDS read here, never from a vector instruction; the build checks the
+// generated code for that (khan_amd/build.py: check_dpp_operands) instead of paying two idle cycles per use.
 __device__ __forceinline__ float fma_quad(float a, int k, float g, float acc)
 {
-    if (k == 0) asm("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(acc) : "v"(a), "v"(g));
-    else if (k == 1) asm("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(acc) : "v"(a), "v"(g));
-    else if (k == 2) asm("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(acc) : "v"(a), "v"(g));
-    else asm("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(acc) : "v"(a), "v"(g));
+    if (k == 0) asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(acc) : "v"(a), "v"(g));
+    else if (k == 1) asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(acc) : "v"(a), "v"(g));
+    else if (k == 2) asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(acc) : "v"(a), "v"(g));
+    else asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(acc) : "v"(a), "v"(g));
     return acc;
 }
 __device__ __forceinline__ double fma_quad(double a, int, double g, double acc) { return fma(a, g, acc); }   // float only

@@ -113,3 +113,20 @@ def test_normal_stream_is_position_keyed():
     part = datagen.normal(1500, 0.3, datagen.TAG_CHARGES, first=2100)
     assert np.array_equal(full[2100:3600], part)
     assert abs(full.std() - 0.3) < 0.02 and abs(full.mean()) < 0.02
+
+
+def test_build_check_of_the_lane_exchange_operand():
+    """khan_amd.build.check_dpp_operands guards the one inline-asm instruction of the kernels: it has to see a
+    vector write of the exchanged register within two instructions, on the fall-through path and through a
+    branch, and to accept code that keeps the distance."""
+    from khan_amd import build
+    use = "\tv_fmac_f32_dpp v90, v2, v42 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n"
+    good = "\tds_read_b32 v2, v7\n\ts_waitcnt lgkmcnt(0)\n" + use + "\tv_mov_b32_e32 v3, v9\n\ts_nop 0\n\ts_nop 0\n" + use.replace("v2", "v3")
+    assert build.check_dpp_operands(good) == 2
+    with pytest.raises(RuntimeError):
+        build.check_dpp_operands("\tv_mov_b32_e32 v2, v9\n\ts_nop 0\n" + use)
+    with pytest.raises(RuntimeError):       # a register pair that covers the operand
+        build.check_dpp_operands("\tv_lshlrev_b64 v[2:3], 1, v[8:9]\n" + use)
+    with pytest.raises(RuntimeError):       # the write sits before a branch to a label just ahead of the use
+        build.check_dpp_operands("\tv_mov_b32_e32 v2, v9\n\ts_branch .LBB0_7\n.LBB0_5:\n\ts_nop 0\n\ts_nop 0\n.LBB0_7:\n" + use)
+    assert build.check_dpp_operands("\tv_mov_b32_e32 v90, 0\n" + use) == 1      # writing the accumulator is fine
