@@ -309,6 +309,34 @@ def test_size_class_boundaries(ops):
                      scale=mol_scale(dx64, c.MOs, c.MACs))
 
 
+def test_mixed_sizes_in_one_ordered_batch(ops):
+    say("case: 2,326 molecules of every size class in one batch, shuffled (the size order and the per-class counts are active)")
+    rng = np.random.default_rng(5)
+    org = datagen.make_batch("organic", 2300)
+    box = datagen.make_batch("boxes", 24)
+    mols = []
+    for b in (org, box):
+        for m in range(b.n_mols):
+            sl = slice(b.MOs[m], b.MOs[m] + b.MACs[m])
+            mols.append((b.A[sl], np.stack([b.X[sl], b.Y[sl], b.Z[sl]], axis=1)))
+    for n in (257, 300):                                  # beyond one workgroup
+        side = (n / 0.08) ** (1 / 3)
+        pts = []
+        while len(pts) < n:
+            p = rng.uniform(0, side, 3)
+            if all(np.linalg.norm(p - q) >= 0.9 for q in pts):
+                pts.append(p)
+        mols.append((rng.integers(0, 4, n).astype(np.int32), np.array(pts, dtype=np.float32)))
+    mols = [mols[i] for i in rng.permutation(len(mols))]
+    A = np.concatenate([m[0] for m in mols]).astype(np.int32)
+    xyz = np.concatenate([m[1] for m in mols]).astype(np.float64)
+    mi = np.concatenate([np.full(len(m[0]), k) for k, m in enumerate(mols)]).astype(np.int32)
+    c = Case(xyz[:, 0], xyz[:, 1], xyz[:, 2], A, mi, len(mols))
+    assert c.n_mols >= 2048                               # the dispatcher orders batches from 2,048 molecules on
+    check_forward_backward(ops, c)
+    _check_grad_inverse(ops, c)
+
+
 def test_empty_batch(ops):
     say("case: empty batch (0 atoms, 0 molecules)")
     e32 = torch.empty(0, dtype=torch.float32, device="cuda:0")
