@@ -771,7 +771,9 @@ def test_forward_backward_replay_from_a_hip_graph(ops):
     # no host synchronisation), so they can be captured once and replayed; every replay is checked against
     # the eager result, with eager work and synchronisations in between
     say("case: HIP graph capture and replay of forward + backward")
-    b = datagen.make_batch("organic", 512, first_mol=900)
+    # enough molecules for the eager calls to take the size order (skipped under capture, where nothing may be
+    # allocated): the captured launches walk the molecules in batch order and must give the same rows
+    b = datagen.make_batch("organic", 2100, first_mol=900)
     big = datagen.make_batch("boxes", 2)               # brings the medium-molecule kernels into the graph
     X = np.concatenate([b.X, big.X]); Y = np.concatenate([b.Y, big.Y]); Z = np.concatenate([b.Z, big.Z])
     A = np.concatenate([b.A, big.A])
