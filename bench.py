@@ -42,6 +42,8 @@ WORKLOADS = {
     # not a line of the headline metric: energies and coordinate gradients through the atomic networks
     # (384-128-128-64-1 per type, random weights), the caller either side of the hot path
     "inference65536": ("organic", 65536, 4, False),
+    # not a line of the headline metric either: featurize_grad_inverse (the Jacobian applied to per-atom vectors)
+    "grad_inverse65536": ("organic", 65536, 4, False),
 }
 
 
@@ -173,6 +175,46 @@ def inference_bench(args, batch):
     }))
 
 
+def grad_inverse_bench(args, batch):
+    """featurize_grad_inverse on the organic batch: one JSON line; algorithmic bytes are the forward's plus the
+    three incoming vectors."""
+    import torch
+    from khan_amd import ops
+    dev = torch.device("cuda:0")
+    N, n_mols = batch.n_atoms, batch.n_mols
+    X, Y, Z = (torch.from_numpy(v).to(dev) for v in (batch.X, batch.Y, batch.Z))
+    A = torch.from_numpy(batch.A).to(dev)
+    macs, mos = ops.mol_offsets(torch.from_numpy(batch.mol_idxs).to(dev), n_mols)
+    sc, ga, ac = ops.ani_sort(A)
+    acs = ac.cpu()
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(7)
+    v = [torch.randn(N, device=dev, generator=gen) for _ in range(3)]
+    for _ in range(args.warmup):
+        ops.featurize_grad_inverse(X, Y, Z, A, mos, macs, sc, acs, *v)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        out = ops.featurize_grad_inverse(X, Y, Z, A, mos, macs, sc, acs, *v)
+    e1.record()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    launch_ms = e0.elapsed_time(e1) / args.steps
+    nbytes = N * (384 * 4 + 6 * 4 + 8) + 8 * n_mols
+    print(json.dumps({
+        "metric": "AEV grad-inverse (Jacobian-vector product) atoms/sec, fp32, 1 MI355X",
+        "value": N / (ms_per_step * 1e-3), "unit": "atoms/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "grad_inverse65536: featurize_grad_inverse, %d molecules, %d atoms" % (n_mols, N)},
+        "roofline": {"kernel": "aev_fwd_small_kernel<float, true>", "bound": "hbm", "achieved": nbytes / (launch_ms * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (launch_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "launch_ms": launch_ms, "algorithmic_bytes": nbytes},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -201,6 +243,8 @@ def main():
     batch = datagen.make_batch(kind, n_mols)
     if args.workload.startswith("inference"):
         return inference_bench(args, batch)
+    if args.workload.startswith("grad_inverse"):
+        return grad_inverse_bench(args, batch)
     N = batch.n_atoms
     counts = batch.work_counts()
     work = algorithmic_work(counts, N, n_mols, w)

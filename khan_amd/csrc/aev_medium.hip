@@ -274,7 +274,8 @@ hipError_t launch_jvp_medium_f32(const float* X, const float* Y, const float* Z,
                                  Buckets<float> out, int min_atoms, const int32_t* order, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
-    const unsigned blocks = static_cast<unsigned>(n_mols < 4096 ? n_mols : 4096);
+    // (one workgroup per CU with this working set: a smaller grid costs less when it only skips)
+    const unsigned blocks = static_cast<unsigned>(n_mols < 1024 ? n_mols : 1024);
     aev_fwd_medium_kernel<float, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, VX, VY, VZ,
                                                                             out, min_atoms, order);
     return hipGetLastError();
