@@ -78,7 +78,7 @@ hipError_t launch_ani_sort(const int32_t* A, int64_t n_atoms, int32_t* scatter, 
 // number of molecules per size class (kSizeBins entries, class = size_bin(atom count)), then the pass's cursors.
 // Every `order` argument of the launchers above is such an array (or null): the kernels for larger molecules read
 // the class counts behind the indices to leave at once when the batch holds no molecule for them.
-// Not for use under graph capture: the counts are cleared with a memset.
+// Kernels only (the counts are cleared by a small kernel), so the sequence can be recorded into a graph.
 constexpr int kSizeBins = 258;    // atom counts 0..256 and "more", largest first
 constexpr int kSizeOrderScratch = 2 * kSizeBins;
 __host__ __device__ __forceinline__ int size_bin(int n)

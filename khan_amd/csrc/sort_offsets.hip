@@ -193,6 +193,13 @@ __global__ void zero_counts_kernel(int32_t* counts4)
     if (threadIdx.x < 4) counts4[threadIdx.x] = 0;
 }
 
+// clears the class counts and cursors behind a size order (a kernel and not a memset node, so that the
+// sequence can be recorded into a graph)
+__global__ __launch_bounds__(kSizeOrderScratch) void size_clear_kernel(int32_t* __restrict__ scratch)
+{
+    scratch[threadIdx.x] = 0;
+}
+
 }  // namespace
 
 hipError_t launch_mol_offsets(const int32_t* mol_idxs, int64_t n_atoms, int32_t n_mols,
@@ -294,8 +301,7 @@ hipError_t launch_size_order(const int32_t* MACs, int32_t n_mols, int32_t* order
 {
     if (n_mols <= 0) return hipSuccess;
     int32_t* scratch = order + n_mols;
-    hipError_t e = hipMemsetAsync(scratch, 0, sizeof(int32_t) * 2 * kSizeBins, stream);
-    if (e != hipSuccess) return e;
+    size_clear_kernel<<<dim3(1), dim3(kSizeOrderScratch), 0, stream>>>(scratch);
     const unsigned blocks = (static_cast<unsigned>(n_mols) + kOrderThreads - 1) / kOrderThreads;
     size_hist_kernel<<<dim3(blocks), dim3(kOrderThreads), 0, stream>>>(MACs, n_mols, scratch);
     size_place_kernel<<<dim3(blocks), dim3(kOrderThreads), 0, stream>>>(MACs, n_mols, scratch, scratch + kSizeBins, order);
