@@ -76,6 +76,21 @@ int khan_featurize_f64(const double *xs, const double *ys, const double *zs, con
                        double *h_feat, double *c_feat, double *n_feat, double *o_feat,
                        const int32_t *acs_host, khan_stream_t stream);
 
+/* khan_featurize_f32 for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments,
+ * same results.  khan_featurize_f32 takes its scratch buffer (the molecule indices in order of decreasing
+ * size, one int per molecule + 516) from the stream-ordered allocator on every call; this one keeps it in a
+ * fixed array inside the library's code object (4.2 MB per GPU, held until the process ends) and calls no
+ * hipMalloc, hipFree or other allocating routine.  More than KHAN_FEATURIZE_NOALLOC_MAX_MOLS molecules:
+ * KHAN_ERR_TOO_LARGE, nothing launched.  Every call on a GPU uses that GPU's one array: calls that overlap
+ * on one GPU (two streams, two threads) race; calls on one stream are ordered and safe.  The first call on
+ * a device looks the array's address up (hipGetSymbolAddress); make that call outside graph capture. */
+#define KHAN_FEATURIZE_NOALLOC_MAX_MOLS (1 << 20)
+int khan_featurize_f32_noalloc(const float *xs, const float *ys, const float *zs, const int32_t *as,
+                               const int32_t *mos, const int32_t *macs, int32_t n_mols,
+                               const int32_t *sis, float *h_feat, float *c_feat, float *n_feat,
+                               float *o_feat, const int32_t *acs_host, khan_stream_t stream);
+
 /* FeaturizeGrad (op: gpu_featurizer/ani_op.cpp:200-221; functor: functor_op.h:27-47,
  * functor_op_cpu.cpp:46-83; kernel: kernel_cpu.cpp:217-366 -- CPU-only in the reference).
  * in : the Featurize inputs, then the upstream gradients h_grads..o_grads laid out like its outputs

@@ -36,6 +36,7 @@ _SIGNATURES = {
     "khan_ani_sort": (ctypes.c_int, [_ptr, ctypes.c_int64, _ptr, _ptr, _ptr, _ptr]),
     "khan_featurize_f32": (ctypes.c_int, _featurize_sig()),
     "khan_featurize_f64": (ctypes.c_int, _featurize_sig()),
+    "khan_featurize_f32_noalloc": (ctypes.c_int, _featurize_sig()),
     "khan_featurize_grad_f32": (ctypes.c_int, _featurize_grad_sig()),
     "khan_featurize_grad_f64": (ctypes.c_int, _featurize_grad_sig()),
     "khan_featurize_grad_inverse_f32": (ctypes.c_int, _featurize_grad_sig()),

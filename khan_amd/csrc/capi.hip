@@ -1,14 +1,43 @@
 // extern "C" surface of libkhan_aev.so: argument checks and dispatch to the kernel launchers.
 #include <cstdlib>
+#include <mutex>
 #include <string>
 
 #include "../../include/khan_aev.h"
 #include "khan_internal.h"
 #include "khan_params.h"
 
+// Size order of khan_featurize_f32_noalloc: the molecule indices by decreasing atom count, then the class counts
+// and cursors (khan::launch_size_order).  One copy per GPU, held until the process ends.  In host code this name
+// is a stand-in, not a device address: host code uses the pointer that noalloc_scratch() returns.
+static __device__ __align__(256) int32_t scratch[KHAN_FEATURIZE_NOALLOC_MAX_MOLS + khan::kSizeOrderScratch];
+
 namespace {
 
 thread_local std::string g_last_hip_error;
+
+// Device address of `scratch` on the current device, looked up once per device with that device current.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+int32_t* g_scratch_ptr[kMaxDevices] = {};
+
+hipError_t noalloc_scratch(int32_t** ptr)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = static_cast<int32_t*>(p);
+    }
+    *ptr = g_scratch_ptr[dev];
+    return hipSuccess;
+}
 
 int hip_status(hipError_t e)
 {
@@ -78,38 +107,36 @@ private:
 
 int forward_dispatch(const float* xs, const float* ys, const float* zs, const int32_t* as,
                      const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
-                     khan::Buckets<float> out, hipStream_t stream)
+                     khan::Buckets<float> out, const int32_t* order, hipStream_t stream)
 {
     if (force_generic())
         return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, nullptr, stream));
     // molecules of up to 32 atoms: one wavefront each; up to 256: one workgroup each; the rest: general kernel
-    SizeOrder order(macs, n_mols, stream);
     int st = hip_status(khan::launch_fwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallPreferredMax,
-                                                      order.get(), stream));
+                                                      order, stream));
     if (st != KHAN_OK) return st;
     st = hip_status(khan::launch_fwd_medium<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallPreferredMax + 1,
-                                                   order.get(), stream));
+                                                   order, stream));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
-                                                      khan::kMediumMaxAtoms + 1, order.get(), stream));
+                                                      khan::kMediumMaxAtoms + 1, order, stream));
 }
 
 int forward_dispatch(const double* xs, const double* ys, const double* zs, const int32_t* as,
                      const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
-                     khan::Buckets<double> out, hipStream_t stream)
+                     khan::Buckets<double> out, const int32_t* order, hipStream_t stream)
 {
     if (force_generic())
         return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, nullptr, stream));
-    SizeOrder order(macs, n_mols, stream);
     int st = hip_status(khan::launch_fwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallMaxAtoms,
-                                                       order.get(), stream));
+                                                       order, stream));
     if (st != KHAN_OK) return st;
     // 65..256 atoms: one workgroup each (in float64 a one-wavefront kernel keeps molecules of up to 64 atoms)
     st = hip_status(khan::launch_fwd_medium<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallMaxAtoms + 1,
-                                                    order.get(), stream));
+                                                    order, stream));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
-                                                       khan::kMediumMaxAtoms + 1, order.get(), stream));
+                                                       khan::kMediumMaxAtoms + 1, order, stream));
 }
 
 int backward_dispatch(const float* xs, const float* ys, const float* zs, const int32_t* as,
@@ -155,21 +182,37 @@ int backward_dispatch(const double* xs, const double* ys, const double* zs, cons
                                                      khan::kSmallMaxAtoms, order.get(), stream));
 }
 
+// argument checks of featurize; KHAN_OK with *run == false means a successful no-op
 template <typename T>
-int featurize_impl(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
-                   const int32_t* macs, int32_t n_mols, const int32_t* sis, T* h, T* c, T* n, T* o,
-                   const int32_t* acs_host, khan_stream_t stream)
+int featurize_check(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
+                    const int32_t* macs, int32_t n_mols, const int32_t* sis, T* h, T* c, T* n, T* o,
+                    const int32_t* acs_host, bool* run)
 {
+    *run = false;
     if (n_mols < 0 || !acs_host) return KHAN_ERR_INVALID_ARG;
     if (n_mols == 0) return KHAN_OK;
     const int64_t n_atoms = static_cast<int64_t>(acs_host[0]) + acs_host[1] + acs_host[2] + acs_host[3];
     if (acs_host[0] < 0 || acs_host[1] < 0 || acs_host[2] < 0 || acs_host[3] < 0) return KHAN_ERR_INVALID_ARG;
     if (n_atoms == 0) return KHAN_OK;
+    if (n_atoms > INT32_MAX) return KHAN_ERR_TOO_LARGE;
     if (!xs || !ys || !zs || !as || !mos || !macs || !sis) return KHAN_ERR_INVALID_ARG;
     if ((acs_host[0] && !h) || (acs_host[1] && !c) || (acs_host[2] && !n) || (acs_host[3] && !o))
         return KHAN_ERR_INVALID_ARG;
+    *run = true;
+    return KHAN_OK;
+}
+
+template <typename T>
+int featurize_impl(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
+                   const int32_t* macs, int32_t n_mols, const int32_t* sis, T* h, T* c, T* n, T* o,
+                   const int32_t* acs_host, khan_stream_t stream)
+{
+    bool run;
+    const int st = featurize_check(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, &run);
+    if (st != KHAN_OK || !run) return st;
     khan::Buckets<T> out{{h, c, n, o}};
-    return forward_dispatch(xs, ys, zs, as, mos, macs, n_mols, sis, out, as_stream(stream));
+    SizeOrder order(macs, n_mols, as_stream(stream));
+    return forward_dispatch(xs, ys, zs, as, mos, macs, n_mols, sis, out, order.get(), as_stream(stream));
 }
 
 template <typename T>
@@ -320,6 +363,30 @@ int khan_featurize_f64(const double* xs, const double* ys, const double* zs, con
                        khan_stream_t stream)
 {
     return featurize_impl<double>(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, stream);
+}
+
+// khan_featurize_f32 without any allocation: the size order goes to the file-scope array above.
+int khan_featurize_f32_noalloc(const float* xs, const float* ys, const float* zs, const int32_t* as,
+                               const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
+                               float* h, float* c, float* n, float* o, const int32_t* acs_host,
+                               khan_stream_t stream)
+{
+    bool run;
+    const int st = featurize_check(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, &run);
+    if (st != KHAN_OK || !run) return st;
+    if (n_mols > KHAN_FEATURIZE_NOALLOC_MAX_MOLS) {
+        g_last_hip_error = "khan_featurize_f32_noalloc: more molecules than its fixed scratch holds (KHAN_FEATURIZE_NOALLOC_MAX_MOLS)";
+        return KHAN_ERR_TOO_LARGE;
+    }
+    int32_t* order = nullptr;
+    hipError_t e = noalloc_scratch(&order);
+    if (e != hipSuccess) return hip_status(e);
+    // the class counts and cursors behind the indices keep the last call's values: launch_size_order clears them
+    // with a kernel first; the indices are all rewritten
+    e = khan::launch_size_order(macs, n_mols, order, as_stream(stream));
+    if (e != hipSuccess) return hip_status(e);
+    khan::Buckets<float> out{{h, c, n, o}};
+    return forward_dispatch(xs, ys, zs, as, mos, macs, n_mols, sis, out, order, as_stream(stream));
 }
 
 int khan_featurize_grad_f32(const float* xs, const float* ys, const float* zs, const int32_t* as,

@@ -1,0 +1,71 @@
+"""khan_featurize_f32_noalloc (the entry point that allocates nothing) against khan_featurize_f32, through the
+C ABI, on two calls in a row, the second with a smaller input: both run the same kernels and differ only in
+where the size order of the molecules lives, so the outputs must be identical bit for bit.  The first batch
+is also checked against the CPU oracle.  Collected last (file name): a failure here hides nothing else."""
+import ctypes
+import sys
+
+import numpy as np
+import pytest
+
+from khan_amd import datagen
+from oracle import binding as ob
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def _call(lib, name, t, acs, out):
+    p = lambda x: ctypes.c_void_p(x.data_ptr() if x.numel() else None)
+    bounds = np.concatenate([[0], np.cumsum(acs)]) * 384
+    buckets = [out[bounds[k]:bounds[k + 1]] for k in range(4)]
+    acs_c = (ctypes.c_int32 * 4)(*[int(v) for v in acs])
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    return getattr(lib, name)(p(t["X"]), p(t["Y"]), p(t["Z"]), p(t["A"]), p(t["mos"]), p(t["macs"]),
+                              t["macs"].numel(), p(t["sc"]), p(buckets[0]), p(buckets[1]), p(buckets[2]),
+                              p(buckets[3]), acs_c, stream)
+
+
+def _batch(kind, n_mols, first_mol):
+    b = datagen.make_batch(kind, n_mols, first_mol=first_mol)
+    sc, _, ac = ob.ani_sort(b.A)
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")
+    t = {"X": d(b.X), "Y": d(b.Y), "Z": d(b.Z), "A": d(b.A), "mos": d(b.MOs), "macs": d(b.MACs), "sc": d(sc)}
+    return b, sc, ac, t
+
+
+def test_no_alloc_entry_point_matches_featurize_on_two_calls_in_a_row():
+    assert torch.cuda.is_available()
+    from khan_amd import _lib
+    lib = _lib.load()
+    # 4,096 then 2,500 molecules (both large enough for the size order to be used), then a batch below that
+    # threshold; the boxes put molecules into the kernels for larger sizes, which read the class counts
+    for kind, n_mols, first in (("organic", 4096, 0), ("organic", 2500, 5000), ("boxes", 40, 0), ("organic", 64, 9000)):
+        b, sc, ac, t = _batch(kind, n_mols, first)
+        say("   no-alloc entry point: %s, %d molecules, %d atoms" % (kind, n_mols, b.n_atoms))
+        ref_out = torch.full((b.n_atoms * 384,), -1.0, dtype=torch.float32, device="cuda:0")
+        new_out = torch.full((b.n_atoms * 384,), -2.0, dtype=torch.float32, device="cuda:0")
+        assert _call(lib, "khan_featurize_f32", t, ac, ref_out) == 0
+        assert _call(lib, "khan_featurize_f32_noalloc", t, ac, new_out) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(ref_out, new_out), "the two entry points differ"
+        if first == 0 and kind == "organic":
+            ref = np.concatenate(ob.featurize(b.X, b.Y, b.Z, b.A, b.MOs, b.MACs, sc, ac, dtype=np.float64))
+            got = new_out.cpu().numpy().astype(np.float64)
+            assert np.all(np.abs(got - ref) <= 1e-6 + 1e-5 * np.abs(ref)), "no-alloc entry point vs the oracle"
+
+
+def test_no_alloc_entry_point_rejects_what_its_scratch_cannot_hold():
+    from khan_amd import _lib
+    lib = _lib.load()
+    acs = (ctypes.c_int32 * 4)(1, 0, 0, 0)
+    one = ctypes.c_void_p(16)      # never dereferenced: the size check comes before any launch
+    too_many = (1 << 20) + 1
+    st = lib.khan_featurize_f32_noalloc(one, one, one, one, one, one, too_many, one, one, one, one, one, acs, None)
+    assert st == 3 and b"scratch" in lib.khan_last_hip_error()
+    assert lib.khan_featurize_f32_noalloc(None, None, None, None, None, None, 0, None, None, None, None, None, acs, None) == 0
