@@ -7,7 +7,16 @@
  * DEVICE pointers unless the name ends in _host.  Work is enqueued on `stream` (a hipStream_t passed
  * as void*; NULL is the default stream) and the call returns without synchronising.  The library
  * keeps no state between calls, never frees or retains caller memory, and writes every element of
- * every output (outputs need not be zeroed by the caller).
+ * every output (outputs need not be zeroed by the caller), provided that the molecules cover every
+ * atom: sum(macs) = number of atoms.  Rows and gradients of atoms that belong to no molecule are left
+ * untouched, except in a batch with atoms and no molecule at all (n_mols = 0), whose outputs are
+ * zeros, as in the reference (functor_op_cpu.cpp:31-38, 68-72).
+ *
+ * Device memory: ordinary (coarse-grained) allocations from hipMalloc / a framework's allocator.  The
+ * gradient kernels for molecules of more than 32 atoms (float32; 64 in float64) add to x/y/z_grads
+ * with hardware floating-point atomics, which fine-grained or host-coherent memory does not support
+ * (the adds would be lost), and whose order varies: those gradients differ from run to run in the
+ * last bits.  Everything else is bit-reproducible.
  *
  * Return value: KHAN_OK, or a KHAN_ERR_* code; khan_status_string() describes it.  Nothing here
  * calls exit().  An empty batch (0 atoms, 0 molecules) is a successful no-op: the reference trainer
@@ -162,6 +171,26 @@ int khan_ani_charge_grad_xyz_f64(const double *xs, const double *ys, const doubl
                                  int32_t n_mols, const double *grads, double *q_grads,
                                  double *x_grads, double *y_grads, double *z_grads,
                                  khan_stream_t stream);
+
+/* Plain Coulomb sums, E_m = k sum_{i<j in m} q_i q_j / r_ij, and their gradients: the charge kernels with
+ * the damping (1 - f_C) switched off and the constant chosen by the caller (k = 1 for charges in e and
+ * distances in the unit the energy is wanted in).  No reference counterpart: khan's own op is the damped,
+ * K-scaled form above (ani_charges.cpp:58-71); this is the bare sum for callers who want it.
+ * khan_coulomb_grad: grads[n_mols] upstream; out q_grads[n_atoms] (may be NULL) and x/y/z_grads[n_atoms]. */
+int khan_coulomb_f32(const float *xs, const float *ys, const float *zs, const float *qs,
+                     const int32_t *mos, const int32_t *macs, int32_t n_mols, float k,
+                     float *energies, khan_stream_t stream);
+int khan_coulomb_f64(const double *xs, const double *ys, const double *zs, const double *qs,
+                     const int32_t *mos, const int32_t *macs, int32_t n_mols, double k,
+                     double *energies, khan_stream_t stream);
+int khan_coulomb_grad_f32(const float *xs, const float *ys, const float *zs, const float *qs,
+                          const int32_t *mos, const int32_t *macs, int32_t n_mols,
+                          const float *grads, float k, float *q_grads, float *x_grads,
+                          float *y_grads, float *z_grads, khan_stream_t stream);
+int khan_coulomb_grad_f64(const double *xs, const double *ys, const double *zs, const double *qs,
+                          const int32_t *mos, const int32_t *macs, int32_t n_mols,
+                          const double *grads, double k, double *q_grads, double *x_grads,
+                          double *y_grads, double *z_grads, khan_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -47,6 +47,10 @@ _SIGNATURES = {
     "khan_ani_charge_grad_f64": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32, _ptr, _ptr, _ptr]),
     "khan_ani_charge_grad_xyz_f32": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32] + [_ptr] * 6),
     "khan_ani_charge_grad_xyz_f64": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32] + [_ptr] * 6),
+    "khan_coulomb_f32": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32, ctypes.c_float, _ptr, _ptr]),
+    "khan_coulomb_f64": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32, ctypes.c_double, _ptr, _ptr]),
+    "khan_coulomb_grad_f32": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32, _ptr, ctypes.c_float] + [_ptr] * 5),
+    "khan_coulomb_grad_f64": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32, _ptr, ctypes.c_double] + [_ptr] * 5),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

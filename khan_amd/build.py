@@ -57,6 +57,8 @@ def build_hip(jobs=4):
     for p in procs:
         if p.wait() != 0:
             raise RuntimeError("hipcc failed")
+    # the generated code of the inline-asm users is checked before anything is linked: no library without it
+    check_dpp_sources()
     out = os.path.join(CSRC, "libkhan_aev.so")
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs)
     return out
@@ -66,57 +68,92 @@ DPP_SOURCES = ["aev_small.hip", "aev_medium.hip"]     # translation units that u
 
 
 def check_dpp_operands(asm_text, name="<asm>"):
-    """The multiply-add with a lane-exchange operand (written as inline asm, which the compiler's hazard
-    handling does not look into) needs two wait states between a vector instruction that writes the exchanged
-    register and itself.  Checks every use in the generated code: none of the two instructions before it -- on
-    the fall-through path and before every branch to a label in between -- may be a vector instruction that
-    writes that register.  Raises on a violation (the remedy is an `s_nop 1` in front of the instruction)."""
+    """The multiply-add with a lane-exchange operand (v_fmac_f32_dpp, written as inline asm, which the compiler's
+    hazard handling does not look into) reads its exchanged register early: two wait states have to lie between a
+    vector instruction that writes that register and the multiply-add, and five between a vector instruction
+    that writes EXEC (v_cmpx) and it.  Checks every use in the generated code, on the fall-through path and
+    backwards through every branch to a label in between.  Every vector destination counts (register ranges,
+    both operands of the swap instructions); `s_nop N` counts as N + 1 wait states, any other instruction as one.
+    Raises on a violation (the remedy is an `s_nop` in front of the instruction)."""
     import re
-    lines = [l.strip() for l in asm_text.split("\n")]
-    code = [(i, l) for i, l in enumerate(lines) if l and not l.startswith((";", ".", "//")) or re.match(r"^\.LBB\d+_\d+:", l or "")]
-    is_label = lambda l: re.match(r"^\.LBB\d+_\d+:", l) is not None
+    label_re = re.compile(r"^(\.LBB\d+_\d+):")
+    code = []
+    for i, raw in enumerate(asm_text.split("\n")):
+        l = raw.split(";")[0].strip()            # drop comments (also the ';;#ASMSTART' markers)
+        if not l or l.startswith("//"):
+            continue
+        if label_re.match(l) or not l.startswith("."):
+            code.append((i, l))
+    is_label = lambda l: label_re.match(l) is not None
     branches = {}
     for k, (_, l) in enumerate(code):
         m = re.match(r"^s_c?branch\S*\s+(\.LBB\d+_\d+)", l)
         if m:
-            branches.setdefault(m.group(1) + ":", []).append(k)
+            branches.setdefault(m.group(1), []).append(k)
 
-    def writes(l, reg):
-        m = re.match(r"^(v_\S+)\s+([^,\s]+)", l)
-        if not m or m.group(1).startswith(("v_cmp", "v_readlane", "v_readfirstlane")):
-            return False
-        dst = m.group(2)
-        r = re.match(r"^v\[(\d+):(\d+)\]$", dst)
-        n = int(reg[1:])
-        if r:
-            return int(r.group(1)) <= n <= int(r.group(2))
-        return dst == reg
+    two_dest = ("v_swap_b32", "v_permlane32_swap", "v_permlane16_swap")
 
-    def hazard_before(k, reg, budget):
-        """True if a vector write of `reg` lies within `budget` instructions before position k on any path."""
+    def vgpr_dests(l):
+        """VGPR numbers a vector-ALU instruction writes."""
+        m = re.match(r"^(v_\S+)\s+(.*)$", l)
+        if not m:
+            return set()
+        op, args = m.group(1), [a.strip() for a in m.group(2).split(",")]
+        if op.startswith(("v_cmp", "v_readlane", "v_readfirstlane")):
+            return set()
+        out = set()
+        for a in args[:2 if op.startswith(two_dest) else 1]:
+            r = re.match(r"^v\[(\d+):(\d+)\]", a)
+            if r:
+                out.update(range(int(r.group(1)), int(r.group(2)) + 1))
+            else:
+                r = re.match(r"^v(\d+)\b", a)
+                if r:
+                    out.add(int(r.group(1)))
+        return out
+
+    def writes_exec(l):
+        return l.startswith("v_cmpx") or re.match(r"^v_\S+\s+exec\b", l) is not None
+
+    def wait_states(l):
+        m = re.match(r"^s_nop\s+(\d+)", l)
+        return int(m.group(1)) + 1 if m else 1
+
+    def hazard_before(k, pred, budget, seen):
+        """True if an instruction satisfying `pred` lies within `budget` wait states before position k on any path."""
         j = k - 1
         while budget > 0 and j >= 0:
             l = code[j][1]
             if is_label(l):
-                for b in branches.get(l.split()[0], []):
-                    if hazard_before(b, reg, budget):
-                        return True
+                lab = label_re.match(l).group(1)
+                for b in branches.get(lab, []):
+                    if (b, budget) not in seen:
+                        seen.add((b, budget))
+                        # the branch itself is an instruction on that path
+                        if hazard_before(b, pred, budget - 1, seen):
+                            return True
                 j -= 1
                 continue
-            if writes(l, reg):
+            if re.match(r"^s_branch\b", l):
+                return False                     # nothing falls through an unconditional branch
+            if pred(l):
                 return True
-            budget -= 1
+            budget -= wait_states(l)
             j -= 1
         return False
 
     uses = 0
     for k, (i, l) in enumerate(code):
-        m = re.match(r"^v_fmac_f32_dpp\s+v\d+,\s*(v\d+),", l)
+        m = re.match(r"^v_fmac_f32_dpp\s+v\d+,\s*v(\d+),", l)
         if m:
             uses += 1
-            if hazard_before(k, m.group(1), 2):
-                raise RuntimeError("%s line %d: a vector instruction writes %s within two instructions of its "
-                                   "lane-exchange read" % (name, i + 1, m.group(1)))
+            reg = int(m.group(1))
+            if hazard_before(k, lambda x: reg in vgpr_dests(x), 2, set()):
+                raise RuntimeError("%s line %d: a vector instruction writes v%d within two wait states of its "
+                                   "lane-exchange read" % (name, i + 1, reg))
+            if hazard_before(k, writes_exec, 5, set()):
+                raise RuntimeError("%s line %d: a vector instruction writes EXEC within five wait states of a "
+                                   "lane-exchange multiply-add" % (name, i + 1))
     return uses
 
 
@@ -124,10 +161,15 @@ def check_dpp_sources():
     """Compiles the translation units that use the lane-exchange multiply-add to assembly and checks them."""
     hipcc = _hipcc()
     total = 0
+    procs = []
     for src in DPP_SOURCES:
         cmd = [hipcc] + [f for f in HIPCC_FLAGS if f != "-Wall"] + ["-S", "--cuda-device-only", "-o", "-", os.path.join(CSRC, src)]
         print("+", " ".join(cmd), flush=True)
-        out = subprocess.run(cmd, check=True, capture_output=True, text=True).stdout
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True)))
+    for src, p in procs:
+        out, _ = p.communicate()
+        if p.returncode != 0:
+            raise RuntimeError("hipcc -S failed on " + src)
         total += check_dpp_operands(out, src)
     if total == 0:
         raise RuntimeError("no lane-exchange multiply-add found in %s: the check looks at the wrong files" % DPP_SOURCES)
@@ -149,9 +191,7 @@ def build_host():
 
 
 def build_all():
-    outs = [build_hip(), build_datagen(), build_host()]
-    check_dpp_sources()
-    return outs
+    return [build_hip(), build_datagen(), build_host()]
 
 
 if __name__ == "__main__":

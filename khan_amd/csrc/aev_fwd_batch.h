@@ -155,7 +155,9 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
         const T cx = vj.y * vk.z - vj.z * vk.y;
         const T cy = vj.z * vk.x - vj.x * vk.z;
         const T cz = vj.x * vk.y - vj.y * vk.x;
-        const T s = Fast<T>::sqrt_(cx * cx + cy * cy + cz * cz);
+        // clamped to [0, 1] like c: a coincident partner (unit vector 0/0) then gives c = -1, s = 0, the angle pi
+        // that the reference arrives at through fmax/fmin/acos (kernel_cpu.cpp:514-517)
+        const T s = Fast<T>::sqrt_(fmin(fmax(cx * cx + cy * cy + cz * cz, T(0)), T(1)));
         T Af[8], dAf[8];
         T dc = T(0), cot = T(0);
         if constexpr (kJvp) {

@@ -160,7 +160,9 @@ __device__ __forceinline__ void fwd_center_generic(const LaneConsts<T>& L, int l
                         const T cx = J.dy * K.dz - J.dz * K.dy;
                         const T cy = J.dz * K.dx - J.dx * K.dz;
                         const T cz = J.dx * K.dy - J.dy * K.dx;
-                        const T s = Real<T>::sqrt_(cx * cx + cy * cy + cz * cz) * inv;
+                        // (a coincident partner makes c and s 0/0: the clamps turn them into -1 and 0, the angle pi the
+                        // reference arrives at through fmax/fmin/acos, kernel_cpu.cpp:514-517)
+                        const T s = fmin(fmax(Real<T>::sqrt_(cx * cx + cy * cy + cz * cz) * inv, T(0)), T(1));
                         const T base = T(1) + c * L.ct + s * L.st;
                         const T b2 = base * base, b4 = b2 * b2, b8 = b4 * b4;
                         const T dav = (J.r + K.r) * T(0.5) - L.ars;
@@ -198,8 +200,8 @@ __device__ __forceinline__ void bwd_center_generic(const LaneConsts<T>& L, int l
             const int j = jc + lane;
             const Partner<T> pj = scan_partner(X, Y, Z, A, off, j, n, xi, yi, zi);
             const bool valid = (j < n) && (j != i);
-            const bool inR = valid && (pj.r < L.R_Rc);
-            const bool inA = valid && (pj.r < L.A_Rc);
+            const bool inR = valid && (pj.r < L.R_Rc) && (pj.r > T(0));      // no derivative for a coincident atom
+            const bool inA = valid && (pj.r < L.A_Rc) && (pj.r > T(0));
             const T fcR = inR ? cutoff_fn(pj.r, L.pi_rc_R) : T(0);
             const T dfcR = inR ? cutoff_dfn(pj.r, L.pi_rc_R) : T(0);
             const T fcA = inA ? cutoff_fn(pj.r, L.pi_rc_A) : T(0);
@@ -242,7 +244,7 @@ __device__ __forceinline__ void bwd_center_generic(const LaneConsts<T>& L, int l
                     } else {
                         const int k = kc + lane;
                         pk = scan_partner(X, Y, Z, A, off, k, n, xi, yi, zi);
-                        kin = (k < n) && (k != i) && (pk.r < L.A_Rc);
+                        kin = (k < n) && (k != i) && (pk.r < L.A_Rc) && (pk.r > T(0));
                         fcK = kin ? cutoff_fn(pk.r, L.pi_rc_A) : T(0);
                         dfcK = kin ? cutoff_dfn(pk.r, L.pi_rc_A) : T(0);
                     }
@@ -346,7 +348,7 @@ __device__ __forceinline__ void jvp_center_generic(const LaneConsts<T>& L, int l
         auto scan_extra = [&](const Partner<T>& p, int j) {
             Extra e;
             e.wx = e.wy = e.wz = e.rd = T(0);
-            if (j < n) {
+            if (j < n && p.r > T(0)) {
                 e.wx = vxi - VX[off + j];
                 e.wy = vyi - VY[off + j];
                 e.wz = vzi - VZ[off + j];
@@ -368,8 +370,8 @@ __device__ __forceinline__ void jvp_center_generic(const LaneConsts<T>& L, int l
             const Partner<T> pj = scan_partner(X, Y, Z, A, off, j, n, xi, yi, zi);
             const Extra ej = scan_extra(pj, j);
             const bool valid = (j < n) && (j != i);
-            const bool inR = valid && (pj.r < L.R_Rc);
-            const bool inA = valid && (pj.r < L.A_Rc);
+            const bool inR = valid && (pj.r < L.R_Rc) && (pj.r > T(0));      // no derivative for a coincident atom
+            const bool inA = valid && (pj.r < L.A_Rc) && (pj.r > T(0));
             const T fcR = inR ? cutoff_fn(pj.r, L.pi_rc_R) : T(0);
             const T dfcR = inR ? cutoff_dfn(pj.r, L.pi_rc_R) : T(0);
             const T fcA = inA ? cutoff_fn(pj.r, L.pi_rc_A) : T(0);
@@ -409,7 +411,7 @@ __device__ __forceinline__ void jvp_center_generic(const LaneConsts<T>& L, int l
                         const int k = kc + lane;
                         pk = scan_partner(X, Y, Z, A, off, k, n, xi, yi, zi);
                         ek = scan_extra(pk, k);
-                        kin = (k < n) && (k != i) && (pk.r < L.A_Rc);
+                        kin = (k < n) && (k != i) && (pk.r < L.A_Rc) && (pk.r > T(0));
                         fcK = kin ? cutoff_fn(pk.r, L.pi_rc_A) : T(0);
                         dfcK = kin ? cutoff_dfn(pk.r, L.pi_rc_A) : T(0);
                     }

@@ -134,8 +134,9 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                     const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
                     const T r = sqrt(dx * dx + dy * dy + dz * dz);
                     const bool valid = (j < n) && (j != i);
-                    const bool inR = valid && (r < kR_Rc_f);
-                    const bool inA = valid && (r < kA_Rc_f);
+                    // r = 0, a coincident atom: no part in derivatives; in the features as the reference has it
+                    const bool inR = valid && (r < kR_Rc_f) && (!kJvp || r > T(0));
+                    const bool inA = valid && (r < kA_Rc_f) && (!kJvp || r > T(0));
                     const unsigned long long mR = wave_ballot(inR), mA = wave_ballot(inA);
                     const int tj = static_cast<int>(aj.w);
 #pragma unroll

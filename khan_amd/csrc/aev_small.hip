@@ -161,8 +161,10 @@ void aev_fwd_small_kernel(
             const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
             const T r = sqrt(dx * dx + dy * dy + dz * dz);
             const bool valid = centre_ok && (jl < n) && (jl != i);
-            const bool inR = valid && (r < kR_Rc_f);
-            const bool inA = valid && (r < kA_Rc_f);
+            // a coincident atom (r = 0) has no direction: it takes no part in any derivative.  In the features it
+            // counts as the reference counts it: its cosine is 0/0, which the clamp turns into -1 (kernel_cpu.cpp:514-516)
+            const bool inR = valid && (r < kR_Rc_f) && (!kJvp || r > T(0));
+            const bool inA = valid && (r < kA_Rc_f) && (!kJvp || r > T(0));
             const unsigned long long mR = wave_ballot(inR), mA = wave_ballot(inA);
             const bool fits = popc64(mA & sub_mask) <= kCapA;
             T wx = T(0), wy = T(0), wz = T(0), rd = T(0);        // v_centre - v_partner, and d r along it

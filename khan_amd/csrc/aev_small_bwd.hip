@@ -137,7 +137,7 @@ void aev_bwd_small_kernel(
             const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
             const T r = sqrt(dx * dx + dy * dy + dz * dz);
             const bool valid = (i < n) && (jl < n) && (jl != i);
-            const bool inA = valid && (r < kA_Rc_f);
+            const bool inA = valid && (r < kA_Rc_f) && (r > T(0));     // r = 0: a coincident atom exerts no force
             const int cnt = popc64(wave_ballot(inA) & sub_mask);          // in every lane of the group
             const int got = __builtin_amdgcn_ds_bpermute((((lane - s0) << logW) & 63) << 2, cnt);
             if (lane >= s0 && lane < s0 + G) m_mine = got;
@@ -146,7 +146,7 @@ void aev_bwd_small_kernel(
             // centres come G at a time in lane order, and not per batch, whose last step is rarely full.
             const T* grow = row_of_lane(min(i, 63));
             T cfx = T(0), cfy = T(0), cfz = T(0);       // this pair's pull on the centre
-            const bool inR = valid && (r < kR_Rc_f);
+            const bool inR = valid && (r < kR_Rc_f) && (r > T(0));
             if (inR) {
                 const T sc = bwd_radial_pair<T>(grow, static_cast<int>(aj.w), r, Fast<T>::rcp(r));   // dE/dr / r
                 cfx = sc * dx;
@@ -227,7 +227,7 @@ void aev_bwd_small_kernel(
             const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
             const T r = sqrt(dx * dx + dy * dy + dz * dz);
             const bool valid = centre_ok && (jl < n) && (jl != i);
-            const bool inA = valid && (r < kA_Rc_f);
+            const bool inA = valid && (r < kA_Rc_f) && (r > T(0));
             const unsigned long long mA = wave_ballot(inA);
             const int cntA = popc64(mA & sub_mask);
             const bool fits = cntA == room;       // the list has the length the first sweep counted

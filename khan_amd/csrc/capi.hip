@@ -182,19 +182,34 @@ int backward_dispatch(const double* xs, const double* ys, const double* zs, cons
                                                      khan::kSmallMaxAtoms, order.get(), stream));
 }
 
-// argument checks of featurize; KHAN_OK with *run == false means a successful no-op
+// zeros to the four buckets (a batch with atoms but no molecule: the reference zero-fills its outputs before it
+// looks at the molecules, functor_op_cpu.cpp:31-38)
+template <typename T>
+int zero_buckets(T* h, T* c, T* n, T* o, const int32_t* acs_host, hipStream_t stream)
+{
+    T* p[4] = {h, c, n, o};
+    for (int t = 0; t < 4; ++t) {
+        if (acs_host[t] > 0 && !p[t]) return KHAN_ERR_INVALID_ARG;
+        const int st = hip_status(khan::launch_zero<T>(p[t], static_cast<int64_t>(acs_host[t]) * khan::kFeats, stream));
+        if (st != KHAN_OK) return st;
+    }
+    return KHAN_OK;
+}
+
+// Argument checks of featurize and featurize_grad_inverse, and the batches that need no AEV kernel: KHAN_OK with
+// *run == false means the call is complete (nothing to do, or rows of zeros written for atoms without a molecule).
 template <typename T>
 int featurize_check(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
                     const int32_t* macs, int32_t n_mols, const int32_t* sis, T* h, T* c, T* n, T* o,
-                    const int32_t* acs_host, bool* run)
+                    const int32_t* acs_host, hipStream_t stream, bool* run)
 {
     *run = false;
     if (n_mols < 0 || !acs_host) return KHAN_ERR_INVALID_ARG;
-    if (n_mols == 0) return KHAN_OK;
-    const int64_t n_atoms = static_cast<int64_t>(acs_host[0]) + acs_host[1] + acs_host[2] + acs_host[3];
     if (acs_host[0] < 0 || acs_host[1] < 0 || acs_host[2] < 0 || acs_host[3] < 0) return KHAN_ERR_INVALID_ARG;
+    const int64_t n_atoms = static_cast<int64_t>(acs_host[0]) + acs_host[1] + acs_host[2] + acs_host[3];
     if (n_atoms == 0) return KHAN_OK;
     if (n_atoms > INT32_MAX) return KHAN_ERR_TOO_LARGE;
+    if (n_mols == 0) return zero_buckets(h, c, n, o, acs_host, stream);
     if (!xs || !ys || !zs || !as || !mos || !macs || !sis) return KHAN_ERR_INVALID_ARG;
     if ((acs_host[0] && !h) || (acs_host[1] && !c) || (acs_host[2] && !n) || (acs_host[3] && !o))
         return KHAN_ERR_INVALID_ARG;
@@ -208,7 +223,7 @@ int featurize_impl(const T* xs, const T* ys, const T* zs, const int32_t* as, con
                    const int32_t* acs_host, khan_stream_t stream)
 {
     bool run;
-    const int st = featurize_check(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, &run);
+    const int st = featurize_check(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, as_stream(stream), &run);
     if (st != KHAN_OK || !run) return st;
     khan::Buckets<T> out{{h, c, n, o}};
     SizeOrder order(macs, n_mols, as_stream(stream));
@@ -227,7 +242,15 @@ int featurize_grad_impl(const T* xs, const T* ys, const T* zs, const int32_t* as
     if (n_atoms == 0) return KHAN_OK;
     if (n_atoms > INT32_MAX) return KHAN_ERR_TOO_LARGE;
     if (!gx || !gy || !gz) return KHAN_ERR_INVALID_ARG;
-    if (n_mols > 0 && (!xs || !ys || !zs || !as || !mos || !macs || !sis)) return KHAN_ERR_INVALID_ARG;
+    // atoms but no molecules: nothing contributes; the reference zero-fills its outputs first (functor_op_cpu.cpp:68-72)
+    if (n_mols == 0) {
+        for (T* g : {gx, gy, gz}) {
+            const int st = hip_status(khan::launch_zero<T>(g, n_atoms, as_stream(stream)));
+            if (st != KHAN_OK) return st;
+        }
+        return KHAN_OK;
+    }
+    if (!xs || !ys || !zs || !as || !mos || !macs || !sis) return KHAN_ERR_INVALID_ARG;
     if ((acs_host[0] && !gh) || (acs_host[1] && !gc) || (acs_host[2] && !gn) || (acs_host[3] && !go))
         return KHAN_ERR_INVALID_ARG;
     khan::Buckets<const T> g{{gh, gc, gn, go}};
@@ -240,14 +263,10 @@ int featurize_grad_inverse_impl(const T* xs, const T* ys, const T* zs, const int
                                 const T* vy, const T* vz, T* h, T* c, T* n, T* o,
                                 const int32_t* acs_host, khan_stream_t stream)
 {
-    if (n_mols < 0 || !acs_host) return KHAN_ERR_INVALID_ARG;
-    if (n_mols == 0) return KHAN_OK;
-    if (acs_host[0] < 0 || acs_host[1] < 0 || acs_host[2] < 0 || acs_host[3] < 0) return KHAN_ERR_INVALID_ARG;
-    const int64_t n_atoms = static_cast<int64_t>(acs_host[0]) + acs_host[1] + acs_host[2] + acs_host[3];
-    if (n_atoms == 0) return KHAN_OK;
-    if (!xs || !ys || !zs || !as || !mos || !macs || !sis || !vx || !vy || !vz) return KHAN_ERR_INVALID_ARG;
-    if ((acs_host[0] && !h) || (acs_host[1] && !c) || (acs_host[2] && !n) || (acs_host[3] && !o))
-        return KHAN_ERR_INVALID_ARG;
+    bool run;
+    const int chk = featurize_check(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, as_stream(stream), &run);
+    if (chk != KHAN_OK || !run) return chk;
+    if (!vx || !vy || !vz) return KHAN_ERR_INVALID_ARG;
     khan::Buckets<T> out{{h, c, n, o}};
     if (force_generic())
         return hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, 0,
@@ -270,24 +289,24 @@ int featurize_grad_inverse_impl(const T* xs, const T* ys, const T* zs, const int
 
 template <typename T>
 int charge_impl(const T* xs, const T* ys, const T* zs, const T* qs, const int32_t* mos,
-                const int32_t* macs, int32_t n_mols, T* e, khan_stream_t stream)
+                const int32_t* macs, int32_t n_mols, bool damped, T k, T* e, khan_stream_t stream)
 {
     if (n_mols < 0) return KHAN_ERR_INVALID_ARG;
     if (n_mols == 0) return KHAN_OK;
     if (!xs || !ys || !zs || !qs || !mos || !macs || !e) return KHAN_ERR_INVALID_ARG;
-    return hip_status(khan::launch_charge_energy<T>(xs, ys, zs, qs, mos, macs, n_mols, e, as_stream(stream)));
+    return hip_status(khan::launch_charge_energy<T>(xs, ys, zs, qs, mos, macs, n_mols, damped, k, e, as_stream(stream)));
 }
 
 template <typename T>
 int charge_grad_impl(const T* xs, const T* ys, const T* zs, const T* qs, const int32_t* mos,
-                     const int32_t* macs, int32_t n_mols, const T* grads, T* qg, T* gx, T* gy, T* gz,
+                     const int32_t* macs, int32_t n_mols, const T* grads, bool damped, T k, T* qg, T* gx, T* gy, T* gz,
                      bool want_xyz, khan_stream_t stream)
 {
     if (n_mols < 0) return KHAN_ERR_INVALID_ARG;
     if (n_mols == 0) return KHAN_OK;
     if (!xs || !ys || !zs || !qs || !mos || !macs || !grads) return KHAN_ERR_INVALID_ARG;
     if (want_xyz ? (!gx || !gy || !gz) : !qg) return KHAN_ERR_INVALID_ARG;
-    return hip_status(khan::launch_charge_grad<T>(xs, ys, zs, qs, mos, macs, n_mols, grads, qg,
+    return hip_status(khan::launch_charge_grad<T>(xs, ys, zs, qs, mos, macs, n_mols, grads, damped, k, qg,
                                                   want_xyz ? gx : nullptr, gy, gz, as_stream(stream)));
 }
 
@@ -372,7 +391,7 @@ int khan_featurize_f32_noalloc(const float* xs, const float* ys, const float* zs
                                khan_stream_t stream)
 {
     bool run;
-    const int st = featurize_check(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, &run);
+    const int st = featurize_check(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, as_stream(stream), &run);
     if (st != KHAN_OK || !run) return st;
     if (n_mols > KHAN_FEATURIZE_NOALLOC_MAX_MOLS) {
         g_last_hip_error = "khan_featurize_f32_noalloc: more molecules than its fixed scratch holds (KHAN_FEATURIZE_NOALLOC_MAX_MOLS)";
@@ -431,27 +450,27 @@ int khan_ani_charge_f32(const float* xs, const float* ys, const float* zs, const
                         const int32_t* mos, const int32_t* macs, int32_t n_mols, float* e,
                         khan_stream_t stream)
 {
-    return charge_impl<float>(xs, ys, zs, qs, mos, macs, n_mols, e, stream);
+    return charge_impl<float>(xs, ys, zs, qs, mos, macs, n_mols, true, khan::kChargeK_f, e, stream);
 }
 int khan_ani_charge_f64(const double* xs, const double* ys, const double* zs, const double* qs,
                         const int32_t* mos, const int32_t* macs, int32_t n_mols, double* e,
                         khan_stream_t stream)
 {
-    return charge_impl<double>(xs, ys, zs, qs, mos, macs, n_mols, e, stream);
+    return charge_impl<double>(xs, ys, zs, qs, mos, macs, n_mols, true, static_cast<double>(khan::kChargeK_f), e, stream);
 }
 
 int khan_ani_charge_grad_f32(const float* xs, const float* ys, const float* zs, const float* qs,
                              const int32_t* mos, const int32_t* macs, int32_t n_mols,
                              const float* grads, float* q_grads, khan_stream_t stream)
 {
-    return charge_grad_impl<float>(xs, ys, zs, qs, mos, macs, n_mols, grads, q_grads, nullptr, nullptr,
+    return charge_grad_impl<float>(xs, ys, zs, qs, mos, macs, n_mols, grads, true, khan::kChargeK_f, q_grads, nullptr, nullptr,
                                    nullptr, false, stream);
 }
 int khan_ani_charge_grad_f64(const double* xs, const double* ys, const double* zs, const double* qs,
                              const int32_t* mos, const int32_t* macs, int32_t n_mols,
                              const double* grads, double* q_grads, khan_stream_t stream)
 {
-    return charge_grad_impl<double>(xs, ys, zs, qs, mos, macs, n_mols, grads, q_grads, nullptr, nullptr,
+    return charge_grad_impl<double>(xs, ys, zs, qs, mos, macs, n_mols, grads, true, static_cast<double>(khan::kChargeK_f), q_grads, nullptr, nullptr,
                                     nullptr, false, stream);
 }
 
@@ -460,14 +479,38 @@ int khan_ani_charge_grad_xyz_f32(const float* xs, const float* ys, const float* 
                                  const float* grads, float* q_grads, float* gx, float* gy, float* gz,
                                  khan_stream_t stream)
 {
-    return charge_grad_impl<float>(xs, ys, zs, qs, mos, macs, n_mols, grads, q_grads, gx, gy, gz, true, stream);
+    return charge_grad_impl<float>(xs, ys, zs, qs, mos, macs, n_mols, grads, true, khan::kChargeK_f, q_grads, gx, gy, gz, true, stream);
 }
 int khan_ani_charge_grad_xyz_f64(const double* xs, const double* ys, const double* zs,
                                  const double* qs, const int32_t* mos, const int32_t* macs,
                                  int32_t n_mols, const double* grads, double* q_grads, double* gx,
                                  double* gy, double* gz, khan_stream_t stream)
 {
-    return charge_grad_impl<double>(xs, ys, zs, qs, mos, macs, n_mols, grads, q_grads, gx, gy, gz, true, stream);
+    return charge_grad_impl<double>(xs, ys, zs, qs, mos, macs, n_mols, grads, true, static_cast<double>(khan::kChargeK_f), q_grads, gx, gy, gz, true, stream);
+}
+
+// Plain Coulomb sums: the charge kernels with the cutoff function switched off and the constant given by the caller.
+int khan_coulomb_f32(const float* xs, const float* ys, const float* zs, const float* qs, const int32_t* mos,
+                     const int32_t* macs, int32_t n_mols, float k, float* e, khan_stream_t stream)
+{
+    return charge_impl<float>(xs, ys, zs, qs, mos, macs, n_mols, false, k, e, stream);
+}
+int khan_coulomb_f64(const double* xs, const double* ys, const double* zs, const double* qs, const int32_t* mos,
+                     const int32_t* macs, int32_t n_mols, double k, double* e, khan_stream_t stream)
+{
+    return charge_impl<double>(xs, ys, zs, qs, mos, macs, n_mols, false, k, e, stream);
+}
+int khan_coulomb_grad_f32(const float* xs, const float* ys, const float* zs, const float* qs, const int32_t* mos,
+                          const int32_t* macs, int32_t n_mols, const float* grads, float k, float* q_grads,
+                          float* gx, float* gy, float* gz, khan_stream_t stream)
+{
+    return charge_grad_impl<float>(xs, ys, zs, qs, mos, macs, n_mols, grads, false, k, q_grads, gx, gy, gz, true, stream);
+}
+int khan_coulomb_grad_f64(const double* xs, const double* ys, const double* zs, const double* qs, const int32_t* mos,
+                          const int32_t* macs, int32_t n_mols, const double* grads, double k, double* q_grads,
+                          double* gx, double* gy, double* gz, khan_stream_t stream)
+{
+    return charge_grad_impl<double>(xs, ys, zs, qs, mos, macs, n_mols, grads, false, k, q_grads, gx, gy, gz, true, stream);
 }
 
 }  // extern "C"

@@ -20,32 +20,33 @@ namespace khan {
 
 namespace {
 
-template <typename T>
+// kDamped = false drops the cutoff function: plain Coulomb pairs q_i q_j / r (the reference's op is the damped form)
+template <typename T, bool kDamped>
 __device__ __forceinline__ void pair_terms(T dx, T dy, T dz, T pi_rc, T rc, T& u, T& dudr_over_r)
 {
     const T r = Real<T>::sqrt_(dx * dx + dy * dy + dz * dz);
     T fc = T(0), dfc = T(0);
-    if (r <= rc) {
+    if (kDamped && r <= rc) {
         fc = cutoff_fn(r, pi_rc);
         dfc = cutoff_dfn(r, pi_rc);
     }
-    const T inv = T(1) / r;
+    // coincident atoms (r = 0): (1 - f_C)/r -> 0 there, and the pair has no direction to pull along
+    const T inv = r > T(0) ? T(1) / r : T(0);
     u = (T(1) - fc) * inv;                            // (1 - f_C) / r
     dudr_over_r = (-dfc * inv - u * inv) * inv;       // d/dr[(1-f_C)/r] / r
 }
 
-template <typename T>
+template <typename T, bool kDamped>
 __global__ __launch_bounds__(256) void charge_energy_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const T* __restrict__ Q, const int32_t* __restrict__ MOs, const int32_t* __restrict__ MACs,
-    int32_t n_mols, T* __restrict__ E)
+    int32_t n_mols, T K, T* __restrict__ E)
 {
     const int lane = threadIdx.x & 63;
     const int64_t mol = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
     if (mol >= n_mols) return;
     const int n = MACs[mol], off = MOs[mol];
     const T rc = static_cast<T>(kR_Rc_f), pi_rc = static_cast<T>(kPi / static_cast<double>(kR_Rc_f));
-    const T K = static_cast<T>(kChargeK_f);
     T acc = T(0);
     if (n <= 64) {
         const int logW = n <= 16 ? 4 : n <= 32 ? 5 : 6;
@@ -60,7 +61,7 @@ __global__ __launch_bounds__(256) void charge_energy_kernel(
                     qi = __shfl(qj, i & 63, 64);
             const bool valid = (i < n) && jok && (jl > i);
             T u, du;
-            pair_terms(valid ? xi - xj : T(1), valid ? yi - yj : T(0), valid ? zi - zj : T(0), pi_rc, rc, u, du);
+            pair_terms<T, kDamped>(valid ? xi - xj : T(1), valid ? yi - yj : T(0), valid ? zi - zj : T(0), pi_rc, rc, u, du);
             acc += valid ? K * qi * qj * u : T(0);
         }
         acc = wave_sum(acc);
@@ -75,7 +76,7 @@ __global__ __launch_bounds__(256) void charge_energy_kernel(
         for (int j = i0 + 1; j < n; ++j) {
             if (active && j > i) {
                 T u, du;
-                pair_terms(xi - X[off + j], yi - Y[off + j], zi - Z[off + j], pi_rc, rc, u, du);
+                pair_terms<T, kDamped>(xi - X[off + j], yi - Y[off + j], zi - Z[off + j], pi_rc, rc, u, du);
                 acc += K * qi * Q[off + j] * u;
             }
         }
@@ -84,11 +85,11 @@ __global__ __launch_bounds__(256) void charge_energy_kernel(
     if (lane == 0) E[mol] = acc;
 }
 
-template <typename T>
+template <typename T, bool kDamped>
 __global__ __launch_bounds__(256) void charge_grad_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const T* __restrict__ Q, const int32_t* __restrict__ MOs, const int32_t* __restrict__ MACs,
-    int32_t n_mols, const T* __restrict__ grads, T* __restrict__ q_grads, T* __restrict__ gX,
+    int32_t n_mols, const T* __restrict__ grads, T K, T* __restrict__ q_grads, T* __restrict__ gX,
     T* __restrict__ gY, T* __restrict__ gZ)
 {
     const int lane = threadIdx.x & 63;
@@ -96,7 +97,7 @@ __global__ __launch_bounds__(256) void charge_grad_kernel(
     if (mol >= n_mols) return;
     const int n = MACs[mol], off = MOs[mol];
     const T rc = static_cast<T>(kR_Rc_f), pi_rc = static_cast<T>(kPi / static_cast<double>(kR_Rc_f));
-    const T gK = grads[mol] * static_cast<T>(kChargeK_f);
+    const T gK = grads[mol] * K;
     if (n <= 64) {
         const int logW = n <= 16 ? 4 : n <= 32 ? 5 : 6;
         const int W = 1 << logW, G = 64 >> logW;
@@ -111,7 +112,7 @@ __global__ __launch_bounds__(256) void charge_grad_kernel(
             const bool valid = (i < n) && jok && (jl != i);
             const T dx = valid ? xi - xj : T(1), dy = valid ? yi - yj : T(0), dz = valid ? zi - zj : T(0);
             T u, du;
-            pair_terms(dx, dy, dz, pi_rc, rc, u, du);
+            pair_terms<T, kDamped>(dx, dy, dz, pi_rc, rc, u, du);
             const T w = valid ? qj * du : T(0);
             // sums over the W partners of the group end up in its last lane
             const T dq = group_sum_to_last_lane(valid ? qj * u : T(0), logW);
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(256) void charge_grad_kernel(
             if (j == i) continue;
             const T dx = xi - X[off + j], dy = yi - Y[off + j], dz = zi - Z[off + j];
             T u, du;
-            pair_terms(dx, dy, dz, pi_rc, rc, u, du);
+            pair_terms<T, kDamped>(dx, dy, dz, pi_rc, rc, u, du);
             const T qj = Q[off + j];
             dq += qj * u;
             const T w = qj * du;
@@ -157,28 +158,30 @@ __global__ __launch_bounds__(256) void charge_grad_kernel(
 
 template <typename T>
 hipError_t launch_charge_energy(const T* X, const T* Y, const T* Z, const T* Q, const int32_t* MOs,
-                                const int32_t* MACs, int32_t n_mols, T* E, hipStream_t stream)
+                                const int32_t* MACs, int32_t n_mols, bool damped, T K, T* E, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
     const unsigned blocks = (static_cast<unsigned>(n_mols) + 3u) / 4u;
-    charge_energy_kernel<T><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, E);
+    if (damped) charge_energy_kernel<T, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, K, E);
+    else charge_energy_kernel<T, false><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, K, E);
     return hipGetLastError();
 }
 
 template <typename T>
 hipError_t launch_charge_grad(const T* X, const T* Y, const T* Z, const T* Q, const int32_t* MOs,
-                              const int32_t* MACs, int32_t n_mols, const T* grads, T* q_grads,
+                              const int32_t* MACs, int32_t n_mols, const T* grads, bool damped, T K, T* q_grads,
                               T* gX, T* gY, T* gZ, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
     const unsigned blocks = (static_cast<unsigned>(n_mols) + 3u) / 4u;
-    charge_grad_kernel<T><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, q_grads, gX, gY, gZ);
+    if (damped) charge_grad_kernel<T, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, q_grads, gX, gY, gZ);
+    else charge_grad_kernel<T, false><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, q_grads, gX, gY, gZ);
     return hipGetLastError();
 }
 
-template hipError_t launch_charge_energy<float>(const float*, const float*, const float*, const float*, const int32_t*, const int32_t*, int32_t, float*, hipStream_t);
-template hipError_t launch_charge_energy<double>(const double*, const double*, const double*, const double*, const int32_t*, const int32_t*, int32_t, double*, hipStream_t);
-template hipError_t launch_charge_grad<float>(const float*, const float*, const float*, const float*, const int32_t*, const int32_t*, int32_t, const float*, float*, float*, float*, float*, hipStream_t);
-template hipError_t launch_charge_grad<double>(const double*, const double*, const double*, const double*, const int32_t*, const int32_t*, int32_t, const double*, double*, double*, double*, double*, hipStream_t);
+template hipError_t launch_charge_energy<float>(const float*, const float*, const float*, const float*, const int32_t*, const int32_t*, int32_t, bool, float, float*, hipStream_t);
+template hipError_t launch_charge_energy<double>(const double*, const double*, const double*, const double*, const int32_t*, const int32_t*, int32_t, bool, double, double*, hipStream_t);
+template hipError_t launch_charge_grad<float>(const float*, const float*, const float*, const float*, const int32_t*, const int32_t*, int32_t, const float*, bool, float, float*, float*, float*, float*, hipStream_t);
+template hipError_t launch_charge_grad<double>(const double*, const double*, const double*, const double*, const int32_t*, const int32_t*, int32_t, const double*, bool, double, double*, double*, double*, double*, hipStream_t);
 
 }  // namespace khan

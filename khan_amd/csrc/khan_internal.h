@@ -88,13 +88,17 @@ __host__ __device__ __forceinline__ int size_bin(int n)
 }
 hipError_t launch_size_order(const int32_t* MACs, int32_t n_mols, int32_t* order, hipStream_t stream);
 
-// ---- charges ----
+// zeros to an array of n elements (outputs that no molecule covers)
+template <typename T>
+hipError_t launch_zero(T* a, int64_t n, hipStream_t stream);
+
+// ---- charges: pair energy K q_i q_j (1 - f_C(r)) / r; damped = false drops f_C (plain Coulomb) ----
 template <typename T>
 hipError_t launch_charge_energy(const T* X, const T* Y, const T* Z, const T* Q, const int32_t* MOs,
-                                const int32_t* MACs, int32_t n_mols, T* E, hipStream_t stream);
+                                const int32_t* MACs, int32_t n_mols, bool damped, T K, T* E, hipStream_t stream);
 template <typename T>
 hipError_t launch_charge_grad(const T* X, const T* Y, const T* Z, const T* Q, const int32_t* MOs,
-                              const int32_t* MACs, int32_t n_mols, const T* grads, T* q_grads,
+                              const int32_t* MACs, int32_t n_mols, const T* grads, bool damped, T K, T* q_grads,
                               T* gX, T* gY, T* gZ, hipStream_t stream);
 
 // ---- wavefront helpers (64 lanes) ----

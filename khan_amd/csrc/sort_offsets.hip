@@ -200,7 +200,26 @@ __global__ __launch_bounds__(kSizeOrderScratch) void size_clear_kernel(int32_t* 
     scratch[threadIdx.x] = 0;
 }
 
+// zeros for outputs that no molecule covers (a kernel, not a memset node: see size_clear_kernel)
+template <typename T>
+__global__ __launch_bounds__(256) void zero_fill_kernel(T* __restrict__ a, int64_t n)
+{
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * 256)
+        a[i] = T(0);
+}
+
 }  // namespace
+
+template <typename T>
+hipError_t launch_zero(T* a, int64_t n, hipStream_t stream)
+{
+    if (n <= 0) return hipSuccess;
+    const int64_t want = (n + 255) / 256;
+    zero_fill_kernel<T><<<dim3(static_cast<unsigned>(want < 8192 ? want : 8192)), dim3(256), 0, stream>>>(a, n);
+    return hipGetLastError();
+}
+template hipError_t launch_zero<float>(float*, int64_t, hipStream_t);
+template hipError_t launch_zero<double>(double*, int64_t, hipStream_t);
 
 hipError_t launch_mol_offsets(const int32_t* mol_idxs, int64_t n_atoms, int32_t n_mols,
                               int32_t* MACs, int32_t* MOs, hipStream_t stream)

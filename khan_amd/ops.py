@@ -219,3 +219,31 @@ def ani_charge_grad_xyz(xs, ys, zs, qs, mos, macs, grads):
     _lib.check(fn(_p(xs), _p(ys), _p(zs), _p(qs), _p(mos), _p(macs), mos.numel(), _p(grads), _p(qg),
                   _p(gx), _p(gy), _p(gz), _stream()))
     return qg, gx, gy, gz
+
+
+def coulomb(xs, ys, zs, qs, mos, macs, k=1.0):
+    """-> energies[n_mols] = k * sum_{i<j} q_i q_j / r_ij: the charge kernel without the reference's damping
+    and constant (the reference's op is `ani_charge`)."""
+    lib = _lib.load()
+    dt, _ = _check_charge(xs, ys, zs, qs, mos, macs)
+    e = torch.empty(mos.numel(), dtype=dt, device=xs.device)
+    fn = getattr(lib, "khan_coulomb_" + _SUFFIX[dt])
+    _lib.check(fn(_p(xs), _p(ys), _p(zs), _p(qs), _p(mos), _p(macs), mos.numel(), float(k), _p(e), _stream()))
+    return e
+
+
+def coulomb_grad(xs, ys, zs, qs, mos, macs, grads, k=1.0):
+    """-> (q_grads, x_grads, y_grads, z_grads) of `coulomb`, weighted by grads[n_mols]."""
+    lib = _lib.load()
+    dt, n = _check_charge(xs, ys, zs, qs, mos, macs)
+    grads = _dev(grads, dt, "grads")
+    if grads.numel() != mos.numel():
+        raise ValueError("grads must have one element per molecule")
+    qg = torch.zeros(n, dtype=dt, device=xs.device)
+    gx = torch.zeros(n, dtype=dt, device=xs.device)
+    gy = torch.zeros_like(gx)
+    gz = torch.zeros_like(gx)
+    fn = getattr(lib, "khan_coulomb_grad_" + _SUFFIX[dt])
+    _lib.check(fn(_p(xs), _p(ys), _p(zs), _p(qs), _p(mos), _p(macs), mos.numel(), _p(grads), float(k), _p(qg),
+                  _p(gx), _p(gy), _p(gz), _stream()))
+    return qg, gx, gy, gz

@@ -130,3 +130,19 @@ def test_build_check_of_the_lane_exchange_operand():
     with pytest.raises(RuntimeError):       # the write sits before a branch to a label just ahead of the use
         build.check_dpp_operands("\tv_mov_b32_e32 v2, v9\n\ts_branch .LBB0_7\n.LBB0_5:\n\ts_nop 0\n\ts_nop 0\n.LBB0_7:\n" + use)
     assert build.check_dpp_operands("\tv_mov_b32_e32 v90, 0\n" + use) == 1      # writing the accumulator is fine
+    with pytest.raises(RuntimeError):       # the second destination of a swap
+        build.check_dpp_operands("\tv_permlane32_swap_b32_e32 v88, v2\n\ts_nop 0\n" + use)
+    with pytest.raises(RuntimeError):       # a vector write of EXEC needs five wait states
+        build.check_dpp_operands("\tv_cmpx_gt_u32_e32 32, v0\n\ts_nop 3\n" + use)
+    assert build.check_dpp_operands("\tv_cmpx_gt_u32_e32 32, v0\n\ts_nop 4\n" + use) == 1
+    assert build.check_dpp_operands("\tv_mov_b32_e32 v2, v9\n\ts_nop 1\n" + use) == 1     # s_nop 1 = two wait states
+    # the write sits in a block that ends in an unconditional branch elsewhere: it does not reach the use
+    assert build.check_dpp_operands("\tv_mov_b32_e32 v2, v9\n\ts_branch .LBB0_9\n.LBB0_5:\n" + use) == 1
+
+
+def test_the_library_cannot_be_built_without_the_lane_exchange_check():
+    """build_hip() runs the check before it links, so every way of producing libkhan_aev.so goes through it."""
+    import inspect
+    from khan_amd import build
+    src = inspect.getsource(build.build_hip)
+    assert src.index("check_dpp_sources()") < src.index('"-shared"')

@@ -68,4 +68,5 @@ def test_no_alloc_entry_point_rejects_what_its_scratch_cannot_hold():
     too_many = (1 << 20) + 1
     st = lib.khan_featurize_f32_noalloc(one, one, one, one, one, one, too_many, one, one, one, one, one, acs, None)
     assert st == 3 and b"scratch" in lib.khan_last_hip_error()
-    assert lib.khan_featurize_f32_noalloc(None, None, None, None, None, None, 0, None, None, None, None, None, acs, None) == 0
+    acs0 = (ctypes.c_int32 * 4)(0, 0, 0, 0)
+    assert lib.khan_featurize_f32_noalloc(None, None, None, None, None, None, 0, None, None, None, None, None, acs0, None) == 0
