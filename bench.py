@@ -2,7 +2,7 @@
 """Benchmark of the ANI-1 featurization hot path on one MI355X.
 
 One "step" = one pass of the hot path over one synthetic batch that is already resident in HBM:
-    mol_offsets + ani_sort  ->  featurize (float32 forward)  ->  featurize_grad (float32 backward)
+    mol_offsets + ani_sort + size_order  ->  featurize (float32 forward)  ->  featurize_grad (float32 backward)
 on the 65,536-molecule organic batch (the configuration the headline metric is quoted on).  The sort runs one
 batch ahead of the passes that use it (its four atom counts have to reach the host first), as a feeder would
 run it; every step still holds exactly one sort, one forward and one backward pass.
@@ -25,12 +25,9 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3       # MI355X vector FP32, published
 FP64_PEAK_TFLOPS = 78.6
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the same
-# counter reads for a plain 64 MiB copy); the summaries and commands are under profiles/.
-MEASURED_TRAFFIC = {
-    ("organic65536", "fwd"): 1255.2e6,
-    ("organic65536", "bwd"): 1252.7e6,
-}
+# roofline.traffic (HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) comes from the record
+# profiles/hbm_traffic.json through khan_amd.profiling: an entry measured on other kernel sources than the ones in
+# the tree is reported as stale (traffic null), never passed on.
 
 # name: (generator, molecules, float width in bytes, charges kernels in the step)
 WORKLOADS = {
@@ -95,7 +92,9 @@ def cpu_baseline(batch, sample_mols_fwd, sample_mols_bwd, w=4):
     # the same kernels sharded by molecule over the host cores (one slice of molecules per thread; the
     # reference runs one CPU tower per core this way, gdb8.py:73-76)
     import concurrent.futures
-    threads = max(1, min(16, os.cpu_count() or 1))
+    # a one-GPU box gives a job 16 host cores whatever os.cpu_count() shows there: at most that many threads
+    host_cores = os.cpu_count() or 1
+    threads = max(1, min(16, host_cores))
 
     def shards(n_mols):
         per = max(1, n_mols // threads)
@@ -128,7 +127,11 @@ def cpu_baseline(batch, sample_mols_fwd, sample_mols_bwd, w=4):
         "fwd_atoms_per_s": 1.0 / t_fwd,
         "bwd_atoms_per_s": 1.0 / t_bwd,
         "all_cores": {"value": 1.0 / (tf_all + tb_all), "unit": "atoms/s", "cores": threads,
-                      "sample": "the same kernels sharded by molecule, one slice per thread"},
+                      "host_cpu_count": host_cores,
+                      "sample": "the same kernels sharded by molecule, one slice per thread; %d threads = the job's "
+                                "share of the host (os.cpu_count() reports %d); forward: wall time of the pool; "
+                                "gradient: the slowest thread's timer (the scatter of its upstream rows is outside it)"
+                                % (threads, host_cores)},
     }
 
 
@@ -295,12 +298,13 @@ def main():
             m0.record()
         macs, mos = ops.mol_offsets(mol_idxs, n_mols)
         sc, ga, ac = ops.ani_sort(A)
+        order = ops.size_order(macs)       # largest molecules first: once per batch, shared by both passes
         if timed:
             m1.record()
         acs_pinned[slot].copy_(ac, non_blocking=True)
         done = torch.cuda.Event()
         done.record()
-        return {"macs": macs, "mos": mos, "sc": sc, "slot": slot, "done": done, "marks": (m0, m1)}
+        return {"macs": macs, "mos": mos, "sc": sc, "order": order, "slot": slot, "done": done, "marks": (m0, m1)}
 
     state = {"cur": None, "n": 0}
 
@@ -312,7 +316,7 @@ def main():
         nxt = enqueue_sort(state["n"] & 1, timed)           # the next batch's sort, ahead of this batch's passes
         cur["done"].synchronize()                           # this batch's counts: copied a step ago
         acs = acs_pinned[cur["slot"]].clone()
-        macs, mos, sc = cur["macs"], cur["mos"], cur["sc"]
+        macs, mos, sc, order = cur["macs"], cur["mos"], cur["sc"], cur["order"]
         # events sit directly around each op, on the stream the kernels are launched on
         marks = [torch.cuda.Event(enable_timing=True) for _ in range(4)] if timed else None
         grads, start = [], 0
@@ -321,11 +325,11 @@ def main():
             start += c
         if timed:
             marks[0].record()
-        feats = ops.featurize(X, Y, Z, A, mos, macs, sc, acs)
+        feats = ops.featurize(X, Y, Z, A, mos, macs, sc, acs, order=order)
         if timed:
             marks[1].record()
             marks[2].record()
-        gx, gy, gz = ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *grads)
+        gx, gy, gz = ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *grads, order=order)
         if timed:
             marks[3].record()
         if with_charges:     # energy, then its gradient with respect to charges and coordinates
@@ -357,6 +361,8 @@ def main():
     dom_flops = work["flops_" + dom]
     achieved = dom_bytes / (ms[dom] * 1e-3) / 1e9
     valu_peak = FP32_PEAK_TFLOPS if w == 4 else FP64_PEAK_TFLOPS
+    from khan_amd import profiling
+    traffic, traffic_stale, traffic_entry = profiling.measured_traffic(args.workload, dom)
     roofline = {
         "kernel": "aev_bwd" if dom == "bwd" else "aev_fwd",
         "bound": "hbm",
@@ -364,7 +370,10 @@ def main():
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": achieved / HBM_PEAK_GBS,
-        "traffic": MEASURED_TRAFFIC.get((args.workload, dom)),
+        "traffic": traffic,
+        "traffic_stale": traffic_stale,
+        "traffic_source": "profiles/hbm_traffic.json entry %s/%s (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a 64 MiB copy)"
+                          % (args.workload, dom) if traffic_entry else None,
         "launch_ms": ms[dom],
         "algorithmic_bytes": dom_bytes,
         "valu_frac": dom_flops / (ms[dom] * 1e-3) / 1e12 / valu_peak,
@@ -391,8 +400,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": "%s: ani_sort + AEV forward + AEV backward%s, %d molecules, %d atoms" % (
             args.workload, " + ani_charge energy and gradients" if with_charges else "", n_mols, N), "n_mols": n_mols, "n_atoms": N, "work_counts": counts,
-            "feeding": "each step enqueues the next batch's mol_offsets + ani_sort (and the copy of its 4 atom counts to the "
-                       "host) ahead of the current batch's forward and backward"},
+            "feeding": "each step enqueues the next batch's mol_offsets + ani_sort + size_order (and the copy of its 4 atom "
+                       "counts to the host) ahead of the current batch's forward and backward, which share that order"},
         "molecules_per_s": n_mols / (ms_per_step * 1e-3),
         "roofline": roofline,
     }

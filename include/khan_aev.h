@@ -138,6 +138,53 @@ int khan_featurize_grad_inverse_f64(const double *xs, const double *ys, const do
                                     double *c_grads, double *n_grads, double *o_grads,
                                     const int32_t *acs_host, khan_stream_t stream);
 
+/* Size order of a batch, computed once and shared by the passes.  No reference counterpart (the reference's
+ * CUDA grid takes the molecules as they come, functor_op_gpu.cu:82-85).  The AEV kernels start the largest
+ * molecules first; every khan_featurize* / khan_featurize_grad* call above works this order out for itself in a
+ * stream-ordered scratch allocation (and goes without it while its stream is being captured into a graph).
+ * khan_size_order writes it into caller memory instead -- order[n_mols + KHAN_SIZE_ORDER_EXTRA] int32, device:
+ * the molecule indices by decreasing atom count, then per-size-class counts -- and the *_ordered entry points
+ * take it as an argument: the same results bit for bit, one order per batch instead of one per call, no
+ * allocation, and usable under graph capture.  `order` may be NULL (molecules are then taken in batch order). */
+#define KHAN_SIZE_ORDER_EXTRA 516
+int khan_size_order(const int32_t *macs, int32_t n_mols, int32_t *order, khan_stream_t stream);
+int khan_featurize_ordered_f32(const float *xs, const float *ys, const float *zs, const int32_t *as,
+                               const int32_t *mos, const int32_t *macs, int32_t n_mols,
+                               const int32_t *sis, float *h_feat, float *c_feat, float *n_feat,
+                               float *o_feat, const int32_t *acs_host, const int32_t *order,
+                               khan_stream_t stream);
+int khan_featurize_ordered_f64(const double *xs, const double *ys, const double *zs, const int32_t *as,
+                               const int32_t *mos, const int32_t *macs, int32_t n_mols,
+                               const int32_t *sis, double *h_feat, double *c_feat, double *n_feat,
+                               double *o_feat, const int32_t *acs_host, const int32_t *order,
+                               khan_stream_t stream);
+int khan_featurize_grad_ordered_f32(const float *xs, const float *ys, const float *zs,
+                                    const int32_t *as, const int32_t *mos, const int32_t *macs,
+                                    int32_t n_mols, const int32_t *sis, const float *h_grads,
+                                    const float *c_grads, const float *n_grads, const float *o_grads,
+                                    float *x_grads, float *y_grads, float *z_grads,
+                                    const int32_t *acs_host, const int32_t *order, khan_stream_t stream);
+int khan_featurize_grad_ordered_f64(const double *xs, const double *ys, const double *zs,
+                                    const int32_t *as, const int32_t *mos, const int32_t *macs,
+                                    int32_t n_mols, const int32_t *sis, const double *h_grads,
+                                    const double *c_grads, const double *n_grads, const double *o_grads,
+                                    double *x_grads, double *y_grads, double *z_grads,
+                                    const int32_t *acs_host, const int32_t *order, khan_stream_t stream);
+int khan_featurize_grad_inverse_ordered_f32(const float *xs, const float *ys, const float *zs,
+                                            const int32_t *as, const int32_t *mos, const int32_t *macs,
+                                            int32_t n_mols, const int32_t *sis, const float *x_grads,
+                                            const float *y_grads, const float *z_grads, float *h_grads,
+                                            float *c_grads, float *n_grads, float *o_grads,
+                                            const int32_t *acs_host, const int32_t *order,
+                                            khan_stream_t stream);
+int khan_featurize_grad_inverse_ordered_f64(const double *xs, const double *ys, const double *zs,
+                                            const int32_t *as, const int32_t *mos, const int32_t *macs,
+                                            int32_t n_mols, const int32_t *sis, const double *x_grads,
+                                            const double *y_grads, const double *z_grads,
+                                            double *h_grads, double *c_grads, double *n_grads,
+                                            double *o_grads, const int32_t *acs_host,
+                                            const int32_t *order, khan_stream_t stream);
+
 /* AniCharge (gpu_featurizer/ani_charges.cpp:45-52 registration, 58-71 charge_energy, 81-119 Compute;
  * CUDA twin ani_charges_gpu.cu:70-128).
  * in : xs, ys, zs, qs [n_atoms]; mos, macs [n_mols]      out: charge_energies[n_mols] */

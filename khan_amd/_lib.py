@@ -27,6 +27,10 @@ def _featurize_grad_sig():
         ctypes.POINTER(ctypes.c_int32), _ptr]
 
 
+def _ordered(sig):
+    return sig[:-1] + [_ptr, _ptr]        # ..., acs_host, order, stream
+
+
 _SIGNATURES = {
     "khan_feature_size": (ctypes.c_int32, []),
     "khan_status_string": (ctypes.c_char_p, [ctypes.c_int]),
@@ -41,6 +45,13 @@ _SIGNATURES = {
     "khan_featurize_grad_f64": (ctypes.c_int, _featurize_grad_sig()),
     "khan_featurize_grad_inverse_f32": (ctypes.c_int, _featurize_grad_sig()),
     "khan_featurize_grad_inverse_f64": (ctypes.c_int, _featurize_grad_sig()),
+    "khan_size_order": (ctypes.c_int, [_ptr, ctypes.c_int32, _ptr, _ptr]),
+    "khan_featurize_ordered_f32": (ctypes.c_int, _ordered(_featurize_sig())),
+    "khan_featurize_ordered_f64": (ctypes.c_int, _ordered(_featurize_sig())),
+    "khan_featurize_grad_ordered_f32": (ctypes.c_int, _ordered(_featurize_grad_sig())),
+    "khan_featurize_grad_ordered_f64": (ctypes.c_int, _ordered(_featurize_grad_sig())),
+    "khan_featurize_grad_inverse_ordered_f32": (ctypes.c_int, _ordered(_featurize_grad_sig())),
+    "khan_featurize_grad_inverse_ordered_f64": (ctypes.c_int, _ordered(_featurize_grad_sig())),
     "khan_ani_charge_f32": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32, _ptr, _ptr]),
     "khan_ani_charge_f64": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32, _ptr, _ptr]),
     "khan_ani_charge_grad_f32": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32, _ptr, _ptr, _ptr]),

@@ -244,7 +244,10 @@ class DeviceFeeder:
         mol_Xs, mol_ids, mol_yts, mol_grads = item
         xs, ys, zs, types, mids = split_columns(mol_Xs, mol_ids, self.dtype)
         n = xs.size
-        n_mols = int(mids[-1]) + 1 if n else 0
+        # one molecule per label: trailing molecules without atoms still count (mol_ids alone would drop them)
+        n_mols = len(mol_yts) if mol_yts is not None else (int(mids[-1]) + 1 if n else 0)
+        if n and int(mids[-1]) >= n_mols:
+            raise ValueError("mol_ids names molecule %d but the batch has %d labels" % (int(mids[-1]), n_mols))
         st = self._staging(slot, n)
         if self._events[slot] is not None:
             self._events[slot].synchronize()          # the previous copy out of this staging set has finished

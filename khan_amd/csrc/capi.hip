@@ -142,7 +142,7 @@ int forward_dispatch(const double* xs, const double* ys, const double* zs, const
 int backward_dispatch(const float* xs, const float* ys, const float* zs, const int32_t* as,
                       const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
                       khan::Buckets<const float> g, float* gx, float* gy, float* gz, int64_t n_atoms,
-                      hipStream_t stream)
+                      const int32_t* order, hipStream_t stream)
 {
     // the specialised kernels fetch upstream rows in 16-byte pieces; buckets that are not 16-byte aligned
     // (rows are 1,536 bytes, so the bucket's base decides) go through the general kernel, which does not care
@@ -151,35 +151,33 @@ int backward_dispatch(const float* xs, const float* ys, const float* zs, const i
                                                           n_atoms, 0, nullptr, stream));
     // by molecule size: above 256 atoms the general kernel, 33..256 one workgroup per molecule, up to 32
     // one wavefront per molecule; each kernel defines every gradient of its own molecules
-    SizeOrder order(macs, n_mols, stream);
     int st = hip_status(khan::launch_bwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                        n_atoms, khan::kMediumMaxAtoms + 1, order.get(), stream));
+                                                        n_atoms, khan::kMediumMaxAtoms + 1, order, stream));
     if (st != KHAN_OK) return st;
     // (the workgroup-per-molecule backward kernel measures slower when it walks the molecules in size order)
     st = hip_status(khan::launch_bwd_medium<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                   khan::kSmallPreferredMax + 1, order.get(), false, stream));
+                                                   khan::kSmallPreferredMax + 1, order, false, stream));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_bwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                    khan::kSmallPreferredMax, order.get(), stream));
+                                                    khan::kSmallPreferredMax, order, stream));
 }
 
 int backward_dispatch(const double* xs, const double* ys, const double* zs, const int32_t* as,
                       const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
                       khan::Buckets<const double> g, double* gx, double* gy, double* gz, int64_t n_atoms,
-                      hipStream_t stream)
+                      const int32_t* order, hipStream_t stream)
 {
     if (force_generic() || !aligned16(g))
         return hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
                                                            n_atoms, 0, nullptr, stream));
-    SizeOrder order(macs, n_mols, stream);
     int st = hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                         n_atoms, khan::kMediumMaxAtoms + 1, order.get(), stream));
+                                                         n_atoms, khan::kMediumMaxAtoms + 1, order, stream));
     if (st != KHAN_OK) return st;
     st = hip_status(khan::launch_bwd_medium<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                    khan::kSmallMaxAtoms + 1, order.get(), false, stream));
+                                                    khan::kSmallMaxAtoms + 1, order, false, stream));
     if (st != KHAN_OK) return st;
     return hip_status(khan::launch_bwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                     khan::kSmallMaxAtoms, order.get(), stream));
+                                                     khan::kSmallMaxAtoms, order, stream));
 }
 
 // zeros to the four buckets (a batch with atoms but no molecule: the reference zero-fills its outputs before it
@@ -220,12 +218,15 @@ int featurize_check(const T* xs, const T* ys, const T* zs, const int32_t* as, co
 template <typename T>
 int featurize_impl(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
                    const int32_t* macs, int32_t n_mols, const int32_t* sis, T* h, T* c, T* n, T* o,
-                   const int32_t* acs_host, khan_stream_t stream)
+                   const int32_t* acs_host, khan_stream_t stream, const int32_t* caller_order = nullptr,
+                   bool own_order = true)
 {
     bool run;
     const int st = featurize_check(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, as_stream(stream), &run);
     if (st != KHAN_OK || !run) return st;
     khan::Buckets<T> out{{h, c, n, o}};
+    if (!own_order)       // the caller's size order (or none): nothing is allocated
+        return forward_dispatch(xs, ys, zs, as, mos, macs, n_mols, sis, out, caller_order, as_stream(stream));
     SizeOrder order(macs, n_mols, as_stream(stream));
     return forward_dispatch(xs, ys, zs, as, mos, macs, n_mols, sis, out, order.get(), as_stream(stream));
 }
@@ -234,7 +235,8 @@ template <typename T>
 int featurize_grad_impl(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
                         const int32_t* macs, int32_t n_mols, const int32_t* sis, const T* gh,
                         const T* gc, const T* gn, const T* go, T* gx, T* gy, T* gz,
-                        const int32_t* acs_host, khan_stream_t stream)
+                        const int32_t* acs_host, khan_stream_t stream, const int32_t* caller_order = nullptr,
+                        bool own_order = true)
 {
     if (n_mols < 0 || !acs_host) return KHAN_ERR_INVALID_ARG;
     if (acs_host[0] < 0 || acs_host[1] < 0 || acs_host[2] < 0 || acs_host[3] < 0) return KHAN_ERR_INVALID_ARG;
@@ -254,14 +256,18 @@ int featurize_grad_impl(const T* xs, const T* ys, const T* zs, const int32_t* as
     if ((acs_host[0] && !gh) || (acs_host[1] && !gc) || (acs_host[2] && !gn) || (acs_host[3] && !go))
         return KHAN_ERR_INVALID_ARG;
     khan::Buckets<const T> g{{gh, gc, gn, go}};
-    return backward_dispatch(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, n_atoms, as_stream(stream));
+    if (!own_order)
+        return backward_dispatch(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, n_atoms, caller_order, as_stream(stream));
+    SizeOrder order(macs, n_mols, as_stream(stream));
+    return backward_dispatch(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, n_atoms, order.get(), as_stream(stream));
 }
 
 template <typename T>
 int featurize_grad_inverse_impl(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
                                 const int32_t* macs, int32_t n_mols, const int32_t* sis, const T* vx,
                                 const T* vy, const T* vz, T* h, T* c, T* n, T* o,
-                                const int32_t* acs_host, khan_stream_t stream)
+                                const int32_t* acs_host, khan_stream_t stream, const int32_t* caller_order = nullptr,
+                                bool own_order = true)
 {
     bool run;
     const int chk = featurize_check(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, as_stream(stream), &run);
@@ -272,19 +278,20 @@ int featurize_grad_inverse_impl(const T* xs, const T* ys, const T* zs, const int
         return hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, 0,
                                                       nullptr, as_stream(stream)));
     // molecules of up to 64 atoms: one wavefront each; 65..256 in float32: one workgroup each; the rest: general-shape kernel
-    SizeOrder order(macs, n_mols, as_stream(stream));
-    int st = hip_status(khan::launch_jvp_small<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, order.get(),
+    SizeOrder made(own_order ? macs : nullptr, own_order ? n_mols : 0, as_stream(stream));
+    const int32_t* order = own_order ? made.get() : caller_order;
+    int st = hip_status(khan::launch_jvp_small<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, order,
                                                   as_stream(stream)));
     if (st != KHAN_OK) return st;
     int generic_from = khan::kSmallMaxAtoms + 1;
     if constexpr (sizeof(T) == 4) {
         st = hip_status(khan::launch_jvp_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
-                                                    khan::kSmallMaxAtoms + 1, order.get(), as_stream(stream)));
+                                                    khan::kSmallMaxAtoms + 1, order, as_stream(stream)));
         if (st != KHAN_OK) return st;
         generic_from = khan::kMediumMaxAtoms + 1;
     }
     return hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
-                                                  generic_from, order.get(), as_stream(stream)));
+                                                  generic_from, order, as_stream(stream)));
 }
 
 template <typename T>
@@ -315,6 +322,14 @@ int charge_grad_impl(const T* xs, const T* ys, const T* zs, const T* qs, const i
 extern "C" {
 
 int32_t khan_feature_size(void) { return khan::kFeats; }
+
+int khan_size_order(const int32_t* macs, int32_t n_mols, int32_t* order, khan_stream_t stream)
+{
+    if (n_mols < 0) return KHAN_ERR_INVALID_ARG;
+    if (!order) return KHAN_ERR_INVALID_ARG;
+    if (n_mols > 0 && !macs) return KHAN_ERR_INVALID_ARG;
+    return hip_status(khan::launch_size_order(macs, n_mols, order, as_stream(stream)));
+}
 
 const char* khan_status_string(int status)
 {
@@ -511,6 +526,58 @@ int khan_coulomb_grad_f64(const double* xs, const double* ys, const double* zs, 
                           double* gx, double* gy, double* gz, khan_stream_t stream)
 {
     return charge_grad_impl<double>(xs, ys, zs, qs, mos, macs, n_mols, grads, false, k, q_grads, gx, gy, gz, true, stream);
+}
+
+// The AEV passes on a size order that the caller computed once for the batch (khan_size_order): nothing is allocated.
+int khan_featurize_ordered_f32(const float* xs, const float* ys, const float* zs, const int32_t* as,
+                               const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
+                               float* h, float* c, float* n, float* o, const int32_t* acs_host,
+                               const int32_t* order, khan_stream_t stream)
+{
+    return featurize_impl<float>(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, stream, order, false);
+}
+int khan_featurize_ordered_f64(const double* xs, const double* ys, const double* zs, const int32_t* as,
+                               const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
+                               double* h, double* c, double* n, double* o, const int32_t* acs_host,
+                               const int32_t* order, khan_stream_t stream)
+{
+    return featurize_impl<double>(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, stream, order, false);
+}
+int khan_featurize_grad_ordered_f32(const float* xs, const float* ys, const float* zs, const int32_t* as,
+                                    const int32_t* mos, const int32_t* macs, int32_t n_mols,
+                                    const int32_t* sis, const float* gh, const float* gc, const float* gn,
+                                    const float* go, float* gx, float* gy, float* gz,
+                                    const int32_t* acs_host, const int32_t* order, khan_stream_t stream)
+{
+    return featurize_grad_impl<float>(xs, ys, zs, as, mos, macs, n_mols, sis, gh, gc, gn, go, gx, gy, gz,
+                                      acs_host, stream, order, false);
+}
+int khan_featurize_grad_ordered_f64(const double* xs, const double* ys, const double* zs, const int32_t* as,
+                                    const int32_t* mos, const int32_t* macs, int32_t n_mols,
+                                    const int32_t* sis, const double* gh, const double* gc, const double* gn,
+                                    const double* go, double* gx, double* gy, double* gz,
+                                    const int32_t* acs_host, const int32_t* order, khan_stream_t stream)
+{
+    return featurize_grad_impl<double>(xs, ys, zs, as, mos, macs, n_mols, sis, gh, gc, gn, go, gx, gy, gz,
+                                       acs_host, stream, order, false);
+}
+int khan_featurize_grad_inverse_ordered_f32(const float* xs, const float* ys, const float* zs, const int32_t* as,
+                                            const int32_t* mos, const int32_t* macs, int32_t n_mols,
+                                            const int32_t* sis, const float* x_grads, const float* y_grads,
+                                            const float* z_grads, float* h, float* c, float* n, float* o,
+                                            const int32_t* acs_host, const int32_t* order, khan_stream_t stream)
+{
+    return featurize_grad_inverse_impl<float>(xs, ys, zs, as, mos, macs, n_mols, sis, x_grads, y_grads, z_grads,
+                                              h, c, n, o, acs_host, stream, order, false);
+}
+int khan_featurize_grad_inverse_ordered_f64(const double* xs, const double* ys, const double* zs, const int32_t* as,
+                                            const int32_t* mos, const int32_t* macs, int32_t n_mols,
+                                            const int32_t* sis, const double* x_grads, const double* y_grads,
+                                            const double* z_grads, double* h, double* c, double* n, double* o,
+                                            const int32_t* acs_host, const int32_t* order, khan_stream_t stream)
+{
+    return featurize_grad_inverse_impl<double>(xs, ys, zs, as, mos, macs, n_mols, sis, x_grads, y_grads, z_grads,
+                                               h, c, n, o, acs_host, stream, order, false);
 }
 
 }  // extern "C"

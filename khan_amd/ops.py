@@ -82,6 +82,27 @@ def ani_sort(atomic_numbers):
     return scatter, gather, counts
 
 
+SIZE_ORDER_EXTRA = 516
+
+
+def size_order(macs):
+    """-> int32[n_mols + 516]: the molecule indices by decreasing atom count and the per-size-class counts, to be
+    passed as `order=` to featurize / featurize_grad / featurize_grad_inverse of the same batch (computed once
+    per batch instead of once per call; the calls then allocate nothing and can be captured into a graph)."""
+    lib = _lib.load()
+    macs = _dev(macs, torch.int32, "macs")
+    order = torch.empty(macs.numel() + SIZE_ORDER_EXTRA, dtype=torch.int32, device=macs.device)
+    _lib.check(lib.khan_size_order(_p(macs), macs.numel(), _p(order), _stream()))
+    return order
+
+
+def _order_arg(order, macs):
+    order = _dev(order, torch.int32, "order")
+    if order.numel() != macs.numel() + SIZE_ORDER_EXTRA:
+        raise ValueError("order must come from size_order(macs) of this batch")
+    return order
+
+
 def _check_common(xs, ys, zs, as_, mos, macs, sis):
     dt = _float_dtype(xs)
     _dev(xs, dt, "xs"); _dev(ys, dt, "ys"); _dev(zs, dt, "zs")
@@ -95,7 +116,7 @@ def _check_common(xs, ys, zs, as_, mos, macs, sis):
     return dt, n
 
 
-def featurize(xs, ys, zs, as_, mos, macs, sis, acs):
+def featurize(xs, ys, zs, as_, mos, macs, sis, acs, order=None):
     """-> (h_feat, c_feat, n_feat, o_feat), flat tensors of acs[t]*384 elements.
 
     The four outputs are consecutive slices of one allocation, so
@@ -111,13 +132,16 @@ def featurize(xs, ys, zs, as_, mos, macs, sis, acs):
     for c in acs_v:
         outs.append(packed[start * FEATURE_SIZE:(start + c) * FEATURE_SIZE])
         start += c
-    fn = getattr(lib, "khan_featurize_" + _SUFFIX[dt])
-    _lib.check(fn(_p(xs), _p(ys), _p(zs), _p(as_), _p(mos), _p(macs), mos.numel(), _p(sis),
-                  _p(outs[0]), _p(outs[1]), _p(outs[2]), _p(outs[3]), acs_c, _stream()))
+    args = (_p(xs), _p(ys), _p(zs), _p(as_), _p(mos), _p(macs), mos.numel(), _p(sis),
+            _p(outs[0]), _p(outs[1]), _p(outs[2]), _p(outs[3]), acs_c)
+    if order is None:
+        _lib.check(getattr(lib, "khan_featurize_" + _SUFFIX[dt])(*args, _stream()))
+    else:
+        _lib.check(getattr(lib, "khan_featurize_ordered_" + _SUFFIX[dt])(*args, _p(_order_arg(order, macs)), _stream()))
     return tuple(outs)
 
 
-def featurize_grad(xs, ys, zs, as_, mos, macs, sis, acs, h_grads, c_grads, n_grads, o_grads):
+def featurize_grad(xs, ys, zs, as_, mos, macs, sis, acs, h_grads, c_grads, n_grads, o_grads, order=None):
     """-> (x_grads, y_grads, z_grads), each [n_atoms] in original atom order."""
     lib = _lib.load()
     dt, n = _check_common(xs, ys, zs, as_, mos, macs, sis)
@@ -133,14 +157,16 @@ def featurize_grad(xs, ys, zs, as_, mos, macs, sis, acs, h_grads, c_grads, n_gra
     gx = torch.empty(n, dtype=dt, device=xs.device)
     gy = torch.empty_like(gx)
     gz = torch.empty_like(gx)
-    fn = getattr(lib, "khan_featurize_grad_" + _SUFFIX[dt])
-    _lib.check(fn(_p(xs), _p(ys), _p(zs), _p(as_), _p(mos), _p(macs), mos.numel(), _p(sis),
-                  _p(grads[0]), _p(grads[1]), _p(grads[2]), _p(grads[3]), _p(gx), _p(gy), _p(gz),
-                  acs_c, _stream()))
+    args = (_p(xs), _p(ys), _p(zs), _p(as_), _p(mos), _p(macs), mos.numel(), _p(sis),
+            _p(grads[0]), _p(grads[1]), _p(grads[2]), _p(grads[3]), _p(gx), _p(gy), _p(gz), acs_c)
+    if order is None:
+        _lib.check(getattr(lib, "khan_featurize_grad_" + _SUFFIX[dt])(*args, _stream()))
+    else:
+        _lib.check(getattr(lib, "khan_featurize_grad_ordered_" + _SUFFIX[dt])(*args, _p(_order_arg(order, macs)), _stream()))
     return gx, gy, gz
 
 
-def featurize_grad_inverse(xs, ys, zs, as_, mos, macs, sis, acs, x_grads, y_grads, z_grads):
+def featurize_grad_inverse(xs, ys, zs, as_, mos, macs, sis, acs, x_grads, y_grads, z_grads, order=None):
     """-> (h_grads, c_grads, n_grads, o_grads) laid out like `featurize`'s outputs: the Jacobian of the
     features applied to one vector per atom, row_i[f] = sum_a dAEV_i[f]/dxyz_a . (x,y,z)_grads[a].
     It is the gradient of `featurize_grad` with respect to its upstream gradients
@@ -161,10 +187,12 @@ def featurize_grad_inverse(xs, ys, zs, as_, mos, macs, sis, acs, x_grads, y_grad
     for c in acs_v:
         outs.append(packed[start * FEATURE_SIZE:(start + c) * FEATURE_SIZE])
         start += c
-    fn = getattr(lib, "khan_featurize_grad_inverse_" + _SUFFIX[dt])
-    _lib.check(fn(_p(xs), _p(ys), _p(zs), _p(as_), _p(mos), _p(macs), mos.numel(), _p(sis),
-                  _p(vs[0]), _p(vs[1]), _p(vs[2]), _p(outs[0]), _p(outs[1]), _p(outs[2]), _p(outs[3]),
-                  acs_c, _stream()))
+    args = (_p(xs), _p(ys), _p(zs), _p(as_), _p(mos), _p(macs), mos.numel(), _p(sis),
+            _p(vs[0]), _p(vs[1]), _p(vs[2]), _p(outs[0]), _p(outs[1]), _p(outs[2]), _p(outs[3]), acs_c)
+    if order is None:
+        _lib.check(getattr(lib, "khan_featurize_grad_inverse_" + _SUFFIX[dt])(*args, _stream()))
+    else:
+        _lib.check(getattr(lib, "khan_featurize_grad_inverse_ordered_" + _SUFFIX[dt])(*args, _p(_order_arg(order, macs)), _stream()))
     return tuple(outs)
 
 

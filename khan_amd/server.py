@@ -88,6 +88,33 @@ def close_connection(s):
     s.close()
 
 
+def receive_request(conn, idle_s=0.25):
+    """One JSON request from a connection that has no framing (the reference reads a single recv of up to 1 MB,
+    client_server.py:29-34, which cuts a request that arrives in several segments): reads until the text parses
+    as JSON, the peer closes, MAX_BYTES are in, or nothing more arrives for `idle_s` seconds after a partial
+    message.  Returns the text ('' when the peer closed without sending); bytes that are not valid UTF-8 come
+    back as a text that does not parse, so the caller answers with an error instead of dying."""
+    buf = b""
+    conn.settimeout(None)
+    try:
+        while len(buf) < MAX_BYTES:
+            try:
+                chunk = conn.recv(MAX_BYTES - len(buf))
+            except socket.timeout:
+                break
+            if not chunk:
+                break
+            buf += chunk
+            try:
+                json.loads(buf.decode(ENCODING))
+                break                                   # a complete request
+            except (UnicodeDecodeError, ValueError):
+                conn.settimeout(idle_s)                 # wait a little for the rest
+    finally:
+        conn.settimeout(None)
+    return buf.decode(ENCODING, errors="replace")
+
+
 def serve_on(s, model, max_connections=None):
     """Accepts connections on the listening socket `s` one at a time and answers requests until the peer closes
     (energy_server.py:137-190).  `max_connections` ends the loop after that many connections (None: forever).
@@ -98,14 +125,16 @@ def serve_on(s, model, max_connections=None):
             conn, _ = s.accept()
             try:
                 while True:
-                    text = receive(conn)
+                    text = receive_request(conn)
                     if not text:
                         break
                     try:
                         reply = handle_request(model, text)
-                    except (ValueError, KeyError) as e:        # malformed request: say so, keep serving
+                    except (ValueError, KeyError, TypeError, IndexError) as e:   # malformed request: say so, keep serving
                         reply = json.dumps({"error": str(e)})
                     send(conn, reply)
+            except OSError:
+                pass                                            # the peer went away mid-request: next connection
             finally:
                 conn.close()
             served += 1

@@ -87,6 +87,21 @@ def test_device_feeder_feeds_the_featurizer():
     assert seen == 41
 
 
+@pytest.mark.gpu
+def test_device_feeder_keeps_trailing_molecules_without_atoms():
+    """A batch whose last molecules have no atoms still has one molecule per label (the molecule ids of the atoms
+    alone would end at the last non-empty one)."""
+    pytest.importorskip("torch")
+    mols = _molecules(5, seed=61) + [np.zeros((0, 4)), np.zeros((0, 4))]
+    ds = batching.RawDataset(mols, [float(k) for k in range(len(mols))])
+    batches = list(batching.DeviceFeeder(ds, batch_size=7, dtype=np.float32))
+    assert len(batches) == 1
+    b = batches[0].wait()
+    assert b.n_mols == 7 and len(b.labels) == 7
+    assert b.mol_atom_counts.cpu().tolist() == [len(m) for m in mols]
+    assert b.mol_offsets.cpu().tolist()[-2:] == [sum(len(m) for m in mols)] * 2
+
+
 # ------------------------------------------------------------------------------- packed data set (native gather)
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_packed_dataset_yields_what_the_raw_one_yields(dtype):

@@ -930,8 +930,8 @@ def test_gradient_error_per_element_beside_the_references_own_functor(ops):
     the sum; the bar here is that the HIP kernels are at least as close to the float64 oracle as the reference's
     functor of the same precision, quantile by quantile, and that the worst per-element ratios stay where they
     were measured (stated in the assertions)."""
-    say("case: per-element gradient error, HIP vs the reference's own functor, 1,024 organic molecules")
-    c = Case.from_batch(datagen.make_batch("organic", 1024))
+    say("case: per-element gradient error, HIP vs the reference's own functor, 256 organic molecules")
+    c = Case.from_batch(datagen.make_batch("organic", 256))
     macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
     acs = ac.cpu()
     upb = c.upstream()
@@ -977,8 +977,8 @@ def test_forward_backward_replay_from_a_hip_graph(ops):
     # no host synchronisation), so they can be captured once and replayed; every replay is checked against
     # the eager result, with eager work and synchronisations in between
     say("case: HIP graph capture and replay of forward + backward")
-    # enough molecules for the eager calls to take the size order (skipped under capture, where nothing may be
-    # allocated): the captured launches walk the molecules in batch order and must give the same rows
+    # enough molecules for the eager calls to take the size order (which they allocate, so they go without it under
+    # capture); the captured calls are given a caller-owned order and must produce the same rows
     b = datagen.make_batch("organic", 2100, first_mol=900)
     big = datagen.make_batch("boxes", 2)               # brings the medium-molecule kernels into the graph
     X = np.concatenate([b.X, big.X]); Y = np.concatenate([b.Y, big.Y]); Z = np.concatenate([b.Z, big.Z])
@@ -1006,10 +1006,14 @@ def test_forward_backward_replay_from_a_hip_graph(ops):
     torch.cuda.current_stream().wait_stream(side)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
-        f_out = ops.featurize(Xd, Yd, Zd, Ad, mos, macs, sc, acs)
-        g_out = ops.featurize_grad(Xd, Yd, Zd, Ad, mos, macs, sc, acs, *gb)
+        # with a caller-owned size order the captured launches walk the molecules largest first, as eager calls do;
+        # the order itself is part of the graph (kernels only: its counts are cleared by a kernel, not a memset node)
+        order = ops.size_order(macs)
+        f_out = ops.featurize(Xd, Yd, Zd, Ad, mos, macs, sc, acs, order=order)
+        g_out = ops.featurize_grad(Xd, Yd, Zd, Ad, mos, macs, sc, acs, *gb, order=order)
     f_cat = lambda: torch.cat(f_out)
     for replay in range(4):
+        order.zero_()                                  # a stale order would send every workgroup to molecule 0
         for t in f_out:
             t.fill_(-1.0)                              # eager work between replays
         for t in g_out:

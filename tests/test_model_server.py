@@ -157,6 +157,47 @@ def test_wire_format():
             server.parse_request(bad)
 
 
+def test_serve_loop_survives_split_requests_and_bytes_that_are_not_text(monkeypatch):
+    """The socket protocol has no framing: a request may arrive in several segments, and a peer may send bytes
+    that are not UTF-8.  The loop reassembles the first and answers the second with an error; it never dies."""
+    import socket
+    import time
+    seen = []
+
+    def fake_handle(model_, text):
+        seen.append(text)
+        return json.dumps({"n": len(json.loads(text)["X"])})
+
+    monkeypatch.setattr(server, "handle_request", fake_handle)
+    listening = server.connect_socket("127.0.0.1", 0, server=True)
+    port = listening.getsockname()[1]
+    th = threading.Thread(target=server.serve_on, args=(listening, None, 2), daemon=True)
+    th.start()
+    big = json.dumps({"X": [[0, 0.1 * k, 0.0, 0.0] for k in range(3000)]})
+    c = server.connect_socket("127.0.0.1", port, server=False)
+    c.setsockopt(socket.IPPROTO_TCP, socket.TCP_NODELAY, 1)
+    try:
+        c.sendall(big[:1000].encode())                 # a request in three segments
+        time.sleep(0.05)
+        c.sendall(big[1000:50000].encode())
+        time.sleep(0.05)
+        c.sendall(big[50000:].encode())
+        assert json.loads(server.receive(c)) == {"n": 3000}
+        c.sendall(b"\xff\xfe{not text")                # not UTF-8, not JSON
+        assert "error" in json.loads(server.receive(c))
+    finally:
+        server.close_connection(c)
+    c2 = server.connect_socket("127.0.0.1", port, server=False)     # the loop is still serving
+    try:
+        server.send(c2, json.dumps({"X": [[0, 0, 0, 0]]}))
+        assert json.loads(server.receive(c2)) == {"n": 1}
+    finally:
+        server.close_connection(c2)
+    th.join(30)
+    assert not th.is_alive()
+    assert seen[0] == big
+
+
 # ------------------------------------------------------------------------------------------- GPU
 def _gpu_model(dtype, seed=7, layers=model.DEFAULT_LAYERS):
     m = model.AniModel(layers, model.celu, dtype, "cuda:0", seed=seed)
