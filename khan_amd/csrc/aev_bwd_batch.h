@@ -28,6 +28,21 @@ __device__ __forceinline__ int sel6(int b, int v0, int v1, int v2, int v3, int v
     return b == 0 ? v0 : b == 1 ? v1 : b == 2 ? v2 : b == 3 ? v3 : b == 4 ? v4 : v5;
 }
 
+// sum over the 16 shells of g_q e_q (f_C' - 2 eta d_q f_C), e_q = exp(-eta d_q^2), d_q = r - Rs_q
+template <typename T>
+__device__ __forceinline__ T radial_shell_sum(const T (&g)[16], T r, T fc, T dfc)
+{
+    const T m2eta_fc = T(-2) * static_cast<T>(kR_eta_f) * fc;
+    T Gsum = T(0);
+#pragma unroll
+    for (int q = 0; q < kNumRRs; ++q) {
+        const T d = r - static_cast<T>(kR_Rs_f[q]);
+        const T e = Fast<T>::gauss(static_cast<T>(kR_eta_f), d);
+        Gsum = fma(g[q] * e, fma(m2eta_fc, d, dfc), Gsum);   // g e (f_C' - 2 eta d f_C)
+    }
+    return Gsum;
+}
+
 // Radial part of one (centre, partner) pair: sum over the 16 shells of g e (f_C' - 2 eta d f_C), divided
 // by r.  The result times (x_i - x_j) is the pair's pull on the centre (and minus that on the partner).
 // `grow` is the centre's upstream row, `tj` the partner's type, `inv` = 1/r.
@@ -44,15 +59,7 @@ __device__ __forceinline__ T bwd_radial_pair(const T* grow, int tj, T r, T inv)
     for (int q = 0; q < kPieces; ++q) u.piece[q] = gp[q];
     T fc, dfc;
     Fast<T>::cutoff_grad(r, static_cast<T>(kR_Rc_f), fc, dfc);
-    const T m2eta_fc = T(-2) * static_cast<T>(kR_eta_f) * fc;
-    T Gsum = T(0);
-#pragma unroll
-    for (int q = 0; q < kNumRRs; ++q) {
-        const T d = r - static_cast<T>(kR_Rs_f[q]);
-        const T e = Fast<T>::gauss(static_cast<T>(kR_eta_f), d);
-        Gsum = fma(u.gr[q] * e, fma(m2eta_fc, d, dfc), Gsum);   // g e (f_C' - 2 eta d f_C)
-    }
-    return Gsum * inv;           // dE/dr / r
+    return radial_shell_sum<T>(u.gr, r, fc, dfc) * inv;           // dE/dr / r
 }
 
 // Both directions of a pair at once: centre c with partner j reads row c's block for j's type, centre j with
@@ -76,15 +83,9 @@ __device__ __forceinline__ T bwd_radial_pair_both(const T* grow_c, int tj, const
     }
     T fc, dfc;
     Fast<T>::cutoff_grad(r, static_cast<T>(kR_Rc_f), fc, dfc);
-    const T m2eta_fc = T(-2) * static_cast<T>(kR_eta_f) * fc;
-    T Gsum = T(0);
 #pragma unroll
-    for (int q = 0; q < kNumRRs; ++q) {
-        const T d = r - static_cast<T>(kR_Rs_f[q]);
-        const T e = Fast<T>::gauss(static_cast<T>(kR_eta_f), d);
-        Gsum = fma((u.gr[q] + w.gr[q]) * e, fma(m2eta_fc, d, dfc), Gsum);
-    }
-    return Gsum * inv;
+    for (int q = 0; q < kNumRRs; ++q) u.gr[q] += w.gr[q];
+    return radial_shell_sum<T>(u.gr, r, fc, dfc) * inv;
 }
 
 // The angular part of an upstream row is 320 elements = kRowPieces 16-byte pieces; a wavefront fetches it
@@ -129,25 +130,32 @@ template <typename T> struct RowStage {
     }
 };
 
-// Angular walk of a batch.  Lane = list entry `lane` of the pool, belonging to centre `bs` of the batch
-// whose list starts at slot `pb` and has `m` entries (`live` = the lane has an entry).  In round d the
-// entry pairs with entry (e + d) mod m of the same centre; after m/2 rounds every unordered pair has
-// been visited once.  The force on the partner k goes to pool.facc[k] by plain read-add-write (the k of a
-// centre are distinct within a round); the force on the lane's own entry is kept in registers.
-// Returns the lane's total: pool.facc[lane] + own (zero for lanes without an entry).
+// Copies of a batch's list that share the rounds: a pool of at most 32 (16) entries is walked by two (four)
+// lanes per entry, lane = copy * span + entry, and copy h takes the rounds d = 1 + h, 1 + h + R, ...
+__device__ __forceinline__ int round_copies(int total) { return total <= 16 ? 4 : total <= 32 ? 2 : 1; }
+
+// Angular walk of a batch.  Lane = copy `copy` (of `copies`, a power of two; `span` = 64 / copies lanes each) of
+// list entry `entry` of the pool, belonging to centre `bs` of the batch whose list starts at slot `pb` and has `m`
+// entries (`live` = the lane has an entry).  In round d the entry pairs with entry (e + d) mod m of the same
+// centre; after m/2 rounds every unordered pair has been visited once.  The force on the partner k goes to
+// the copy's own pool.facc[copy * span + k] by plain read-add-write (the k of a centre are distinct within a round);
+// the force on the lane's own entry is kept in registers.
+// Returns the entry's total over all copies, in every copy's lane (zero for lanes without an entry).
 // `type_of(sorted position)` gives an atom's type.
 template <typename T, typename TypeOf>
-__device__ __forceinline__ typename Fast<T>::vec4 bwd_angular_rounds(BwdPool<T>& pool, int lane, bool live, int bs, int pb, int m,
-                                                     TypeOf type_of)
+__device__ __forceinline__ typename Fast<T>::vec4 bwd_angular_rounds(BwdPool<T>& pool, int entry, int copy, int copies, bool live,
+                                                     int bs, int pb, int m, TypeOf type_of)
 {
     typedef typename Fast<T>::vec4 vec4;
     typedef typename Fast<T>::vec2 vec2;
-    const int e = live ? lane - pb : 0;
-    // rounds: d = 1 .. (m-1)/2 for every lane; when m is even one more round for the lower half
+    const int e = live ? entry - pb : 0;
+    const int span = 64 / copies;
+    const int mine = copy * span;          // this copy's slots of pool.facc
+    // rounds: d = 1 .. (m-1)/2 for every entry; when m is even one more round for the lower half
     const int full = (m - 1) >> 1;
     const int rounds = live ? full + ((((m & 1) == 0) && (e < (m >> 1))) ? 1 : 0) : 0;
     const int max_rounds = wave_max(rounds);
-    const int self = live ? lane : 0;
+    const int self = live ? entry : 0;
     const vec4 vj = pool.nbr[self];
     const vec2 fj = pool.nbr_fc[self];
     const int tj = type_of(pool.nbr_idx[self]);
@@ -155,7 +163,8 @@ __device__ __forceinline__ typename Fast<T>::vec4 bwd_angular_rounds(BwdPool<T>&
     const T* gbase = &pool.gst[bs * kNumPairBlocks * kBlockStride];
     T ajx = T(0), ajy = T(0), ajz = T(0);           // force on j, kept in registers
 
-    for (int d = 1; d <= max_rounds; ++d) {
+    for (int d0 = 1; d0 <= max_rounds; d0 += copies) {           // uniform trip count; copy h is at round d0 + h
+        const int d = d0 + copy;
         const bool act = d <= rounds;
         int k = e + d;
         k -= (k >= m) ? m : 0;
@@ -189,14 +198,22 @@ __device__ __forceinline__ typename Fast<T>::vec4 bwd_angular_rounds(BwdPool<T>&
             }
             // X_s = sum_t g_ts A_t and Y_s = sum_t g_ts dA_t/dcos (without its factor 8)
             T Xs[4] = {T(0), T(0), T(0), T(0)}, Ys[4] = {T(0), T(0), T(0), T(0)};
+            T bases[8];
+            theta_bases<T>(c, s, bases);
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
                 const T ct = static_cast<T>(kCosTheta[t]), st = static_cast<T>(kSinTheta[t]);
-                const T bs1 = fma(s, st, fma(c, ct, T(1)));       // 1 + cos(theta - theta_t)
+                const T bs1 = bases[t];                              // 1 + cos(theta - theta_t)
                 const T b2 = bs1 * bs1, b4 = b2 * b2;
                 const T Am1 = b4 * b2 * bs1;                         // ^7
                 const T At = Am1 * bs1;                              // ^8
-                const T dAt = Am1 * fma(-c_over_s, st, ct);         // (d/dcos) / 8
+                // (d/dcos) / 8 = Am1 (cos theta_t - cot sin theta_t); theta_0 = 0 exactly; in float theta_2 and theta_6
+                // are pi/2 and 3 pi/2 to 8e-8, which leaves -cot and +cot (theta_4's sine stays: cot is unbounded)
+                T dAt;
+                if (t == 0) dAt = Am1;
+                else if (sizeof(T) == 4 && t == 2) dAt = -c_over_s * Am1;
+                else if (sizeof(T) == 4 && t == 6) dAt = c_over_s * Am1;
+                else dAt = Am1 * fma(-c_over_s, st, ct);
                 Xs[0] = fma(g[t].x, At, Xs[0]);
                 Xs[1] = fma(g[t].y, At, Xs[1]);
                 Xs[2] = fma(g[t].z, At, Xs[2]);
@@ -223,19 +240,29 @@ __device__ __forceinline__ typename Fast<T>::vec4 bwd_angular_rounds(BwdPool<T>&
             ajy = fma(-Fj, vj.y, fma(-ij, fma(-c, vj.y, vk.y), ajy));
             ajz = fma(-Fj, vj.z, fma(-ij, fma(-c, vj.z, vk.z), ajz));
             // force on k: in a round every lane of a centre holds a different k
-            vec4 fk_acc = pool.facc[ks];
+            vec4 fk_acc = pool.facc[mine + ks];
             fk_acc.x = fma(-Fk, vk.x, fma(-ik, fma(-c, vk.x, vj.x), fk_acc.x));
             fk_acc.y = fma(-Fk, vk.y, fma(-ik, fma(-c, vk.y, vj.y), fk_acc.y));
             fk_acc.z = fma(-Fk, vk.z, fma(-ik, fma(-c, vk.z, vj.z), fk_acc.z));
-            pool.facc[ks] = fk_acc;
+            pool.facc[mine + ks] = fk_acc;
         }
         wave_lds_fence();
     }
 
-    vec4 f = pool.facc[self];
+    vec4 f = pool.facc[mine + self];
     f.x = live ? f.x + ajx : T(0);
     f.y = live ? f.y + ajy : T(0);
     f.z = live ? f.z + ajz : T(0);
+    if (copies >= 2) {
+        f.x += __shfl_xor(f.x, 32, 64);
+        f.y += __shfl_xor(f.y, 32, 64);
+        f.z += __shfl_xor(f.z, 32, 64);
+    }
+    if (copies == 4) {
+        f.x += __shfl_xor(f.x, 16, 64);
+        f.y += __shfl_xor(f.y, 16, 64);
+        f.z += __shfl_xor(f.z, 16, 64);
+    }
     return f;
 }
 

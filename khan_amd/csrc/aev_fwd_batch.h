@@ -20,12 +20,12 @@ template <typename T> struct __align__(16) FwdJvpLds<T, true> {
 // LDS working set of one wavefront
 template <typename T, bool kJvp = false>
 struct __align__(16) FwdWaveLds {
-    typename Fast<T>::vec4 atom[64];          // x, y, z, type (sorted order)
     typename Fast<T>::vec4 nbr[kFB][kCapA];    // unit vector (centre minus partner)/r, and r
     T nbr_fc[kFB][kCapA];                      // f_C(r, A_Rc)
     typename Fast<T>::vec2 rad[64];           // (r, f_C(r, R_Rc)); group g of a scan step owns [g*W, (g+1)*W)
     T rec[64][12];                            // phase-1 records: A_0..7, G_0..3
     SegDesc seg[64];                          // non-empty segments of the batch, in order
+    unsigned long long segrow[64];            // where each of them puts its 32 output values
     unsigned bits[kBitWords];                 // bit per triple slot: a segment starts here
     int nA[kFB][4];                            // angular partners per type, per centre of the batch
     int nR[4][4];                             // radial partners per type, per group of the scan step
@@ -68,7 +68,8 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
     const int ang_t = L.ts >> 2, ang_s = L.ts & 3;
 
     // ------------------------------------------------ segment table of the batch
-    int cnt = 0, packed = 0;
+    int cnt = 0;
+    SegDesc mine = {0u, 0u, 0u, 0u};
     unsigned seg_row_lo = 0, seg_row_hi = 0;          // where the segment's 32 floats go
     {
         // row of the segment's centre (every lane takes part: the lookup may be a lane exchange)
@@ -85,7 +86,11 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
         const int ob = sel4(seg_bt, 0, nn.x, nn.x + nn.y, nn.x + nn.y + nn.z);
         const bool same = seg_a == seg_bt;
         cnt = same ? (__mul24(na, na - 1) >> 1) : __mul24(na, nbt);
-        packed = seg_b | (oa << 3) | (ob << 9) | (na << 15) | (same ? (1 << 21) : 0) | (seg_pt << 22);
+        mine.aj = static_cast<unsigned>((seg_b * kCapA + oa) * static_cast<int>(sizeof(vec4)));
+        mine.ak = static_cast<unsigned>((seg_b * kCapA + ob) * static_cast<int>(sizeof(vec4)));
+        // floor(2^15 / n_a) + 1 (the reciprocal is within an ulp, and 2^15 / n_a is never that close below an integer)
+        const unsigned magic = static_cast<unsigned>(32768.0f * __builtin_amdgcn_rcpf(static_cast<float>(max(na, 1)))) + 1u;
+        mine.div = magic | (static_cast<unsigned>(na) << 16) | (same ? (1u << 24) : 0u);
     }
     const int padded = (cnt + 1) & ~1;
     const int incl = scan_add(padded);
@@ -95,12 +100,10 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
     for (int w = lane; w < kBitWords; w += 64) S.bits[w] = 0u;
     wave_lds_fence();
     if (cnt > 0) {
-        SegDesc d;
-        d.start_cnt = start | (cnt << 12);
-        d.packed = packed;
-        d.row_lo = seg_row_lo;
-        d.row_hi = seg_row_hi;
-        S.seg[popc64(nonempty & lt_mask)] = d;
+        mine.start_cnt = static_cast<unsigned>(start) | (static_cast<unsigned>(cnt) << 16);
+        const int at = popc64(nonempty & lt_mask);
+        S.seg[at] = mine;
+        S.segrow[at] = (static_cast<unsigned long long>(seg_row_hi) << 32) | seg_row_lo;
         atomicOr(&S.bits[start >> 5], 1u << (start & 31));
     }
     wave_lds_fence();
@@ -122,33 +125,33 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
         const unsigned long long starts = (static_cast<unsigned long long>(w1) << 32) | w0;
         const int ord = carry + popc64(starts & (lt_mask | lane_bit)) - 1;
         carry += popc64(starts);
-        const SegDesc d = S.seg[max(ord, 0)];
+        const int seg_at = max(ord, 0);
+        const SegDesc d = S.seg[seg_at];
+        const unsigned long long d_row = S.segrow[seg_at];
+        const unsigned d_row_lo = static_cast<unsigned>(d_row), d_row_hi = static_cast<unsigned>(d_row >> 32);
         const int slot = base + lane;
-        const int q = slot - (d.start_cnt & 0xfff);
-        const bool ok = (slot < total) && (q >= 0) && (q < (d.start_cnt >> 12));
+        const unsigned q = static_cast<unsigned>(slot) - (d.start_cnt & 0xffffu);     // "negative" = huge
+        const bool ok = (slot < total) && (q < (d.start_cnt >> 16));
 
         // decode q -> (j,k) inside the centre's type-sorted list
-        int bsel = d.packed & 7;
-        const int oa = (d.packed >> 3) & 63, ob = (d.packed >> 9) & 63, na = (d.packed >> 15) & 63;
         // Different types: q = kl * n_a + jl.  Same type (pairs jl < kl): the rows kl = r + 1 and kl = n_a - r - 1 of the
         // triangle are laid end to end in one row of length n_a, so the same division serves both numberings:
         // with (r, col) = divmod(q, n_a), col <= r is the pair (col, r + 1) and col > r the pair (col - r - 1, n_a - r - 1).
-        const float qf = static_cast<float>(q);
-        const unsigned kr = static_cast<unsigned>((qf + 0.5f) * __builtin_amdgcn_rcpf(static_cast<float>(na)));
-        const unsigned jr = static_cast<unsigned>(q) - __umul24(kr, static_cast<unsigned>(na));
-        const unsigned tri = (d.packed >> 21) & 1u;
+        const unsigned na = (d.div >> 16) & 0xffu, tri = d.div >> 24;
+        const unsigned kr = __umul24(q, d.div & 0xffffu) >> 15;
+        const unsigned jr = q - __umul24(kr, na);
         const unsigned k1 = kr + tri;
         const bool fold = tri && (jr >= k1);
-        const int kl = static_cast<int>(fold ? static_cast<unsigned>(na) - k1 : k1);
-        const int jl2 = static_cast<int>(fold ? jr - k1 : jr);
-        int j = oa + jl2, k = ob + kl;
-        if (!ok) {
-            j = 0;
-            k = 0;
-            bsel = 0;
-        }
-        const vec4 vj = S.nbr[bsel][j], vk = S.nbr[bsel][k];
-        const T fj = S.nbr_fc[bsel][j], fk = S.nbr_fc[bsel][k];
+        const unsigned kl = fold ? na - k1 : k1;
+        const unsigned jl2 = fold ? jr - k1 : jr;
+        // byte offsets of the two list entries (padding slots take entry 0 of the first list)
+        constexpr unsigned kEntry = sizeof(vec4), kPerT = sizeof(vec4) / sizeof(T);
+        const unsigned bj = ok ? d.aj + jl2 * kEntry : 0u;
+        const unsigned bk = ok ? d.ak + kl * kEntry : 0u;
+        const char* const nbr_bytes = reinterpret_cast<const char*>(&S.nbr[0][0]);
+        const char* const fc_bytes = reinterpret_cast<const char*>(&S.nbr_fc[0][0]);
+        const vec4 vj = *reinterpret_cast<const vec4*>(nbr_bytes + bj), vk = *reinterpret_cast<const vec4*>(nbr_bytes + bk);
+        const T fj = *reinterpret_cast<const T*>(fc_bytes + bj / kPerT), fk = *reinterpret_cast<const T*>(fc_bytes + bk / kPerT);
 
         T c = vj.x * vk.x + vj.y * vk.y + vj.z * vk.z;
         c = fmin(fmax(c, T(-1)), T(1));
@@ -162,14 +165,17 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
         T dc = T(0), cot = T(0);
         if constexpr (kJvp) {
             // d cos = u_k.p_j + u_j.p_k - c (alpha_j + alpha_k), p = (v_i - v_partner)/r, alpha = u.p
-            const vec4 pj = S.jvp.nbr_p[bsel][j], pk = S.jvp.nbr_p[bsel][k];
+            const char* const p_bytes = reinterpret_cast<const char*>(&S.jvp.nbr_p[0][0]);
+            const vec4 pj = *reinterpret_cast<const vec4*>(p_bytes + bj), pk = *reinterpret_cast<const vec4*>(p_bytes + bk);
             dc = (vk.x * pj.x + vk.y * pj.y + vk.z * pj.z) + (vj.x * pk.x + vj.y * pk.y + vj.z * pk.z) - c * (pj.w + pk.w);
             cot = c * s * Fast<T>::rcp(s * s + Real<T>::kCotEps);     // c/s, zero on the line (cusp of the angle)
         }
+        T bases[8];
+        theta_bases<T>(c, s, bases);
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
             const T ct = static_cast<T>(kCosTheta[t]), st = static_cast<T>(kSinTheta[t]);
-            const T base = fma(s, st, fma(c, ct, T(1)));
+            const T base = bases[t];
             if constexpr (kJvp) {
                 const T b2 = base * base, b4 = b2 * b2;
                 const T Am1 = b4 * b2 * base;
@@ -187,7 +193,8 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
         T Gf[4], Hf[4];
         T dP = T(0), drho = T(0);
         if constexpr (kJvp) {
-            const vec2 dj = S.jvp.nbr_d[bsel][j], dk = S.jvp.nbr_d[bsel][k];
+            const char* const d_bytes = reinterpret_cast<const char*>(&S.jvp.nbr_d[0][0]);
+            const vec2 dj = *reinterpret_cast<const vec2*>(d_bytes + bj / 2u), dk = *reinterpret_cast<const vec2*>(d_bytes + bk / 2u);
             dP = ok ? T(0.0078125) * (dj.x * fk + fj * dk.x) : T(0);
             drho = T(0.5) * (dj.y + dk.y);
         }
@@ -228,8 +235,8 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
         const T* pa4 = &S.rec[L.half + 2 * ang_s][ang_t];
         unsigned long long mm = starts;
         if (base == 0) {            // the batch's first segment opens here; nothing to close
-            cur_lo = static_cast<unsigned>(lane_read(static_cast<int>(d.row_lo), 0));
-            cur_hi = static_cast<unsigned>(lane_read(static_cast<int>(d.row_hi), 0));
+            cur_lo = static_cast<unsigned>(lane_read(static_cast<int>(d_row_lo), 0));
+            cur_hi = static_cast<unsigned>(lane_read(static_cast<int>(d_row_hi), 0));
             mm &= ~1ull;
         }
         struct Group {
@@ -260,8 +267,8 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
                     flush();
                     int first = 2 * (q0 + u);
                     asm volatile("" : "+s"(first));      // keeps the lane reads inside this branch
-                    cur_lo = static_cast<unsigned>(lane_read(static_cast<int>(d.row_lo), first));
-                    cur_hi = static_cast<unsigned>(lane_read(static_cast<int>(d.row_hi), first));
+                    cur_lo = static_cast<unsigned>(lane_read(static_cast<int>(d_row_lo), first));
+                    cur_hi = static_cast<unsigned>(lane_read(static_cast<int>(d_row_hi), first));
                     acc = T(0);
                 }
                 if constexpr (kJvp) acc = fma(v.da[u], v.g[u], fma(v.a[u], v.h[u], acc));

@@ -308,12 +308,15 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
             const int pf1 = lane_read(pfv, 1), pf2 = lane_read(pfv, 2), pf3 = lane_read(pfv, 3),
                       pf4 = lane_read(pfv, 4), pf5 = lane_read(pfv, 5), pf6 = lane_read(pfv, 6);
             const int total = used;
-            const int b = (lane >= pf1) + (lane >= pf2) + (lane >= pf3) + (lane >= pf4) + (lane >= pf5);
-            const bool live = lane < total;
-            const int bs = live ? b : 0;
+            // a short pool is walked by two or four lanes per entry, which share its rounds
+            const int copies = round_copies(total), span = 64 / copies;
+            const int entry = lane & (span - 1), copy = lane / span;
+            const int b = (entry >= pf1) + (entry >= pf2) + (entry >= pf3) + (entry >= pf4) + (entry >= pf5);
+            const int bs = entry < total ? b : 0;
             const int pb = sel6(bs, 0, pf1, pf2, pf3, pf4, pf5);
             const int m = sel6(bs, pf1, pf2, pf3, pf4, pf5, pf6) - pb;
-            const vec4 f = bwd_angular_rounds<T>(P, lane, live, bs, pb, m, type_of);
+            const vec4 f = bwd_angular_rounds<T>(P, entry, copy, copies, entry < total, bs, pb, m, type_of);
+            const bool live = lane < total;       // from here on one lane per entry again
 
             // ------------------------------------------------ gather
             if (live) add_force(P.nbr_idx[lane], f.x, f.y, f.z);

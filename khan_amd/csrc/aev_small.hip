@@ -51,7 +51,7 @@ void aev_fwd_small_kernel(
     typedef typename Fast<T>::vec2 vec2;
     __shared__ FwdWaveLds<T, kJvp> lds_all[kWavesPerBlock];
     const int lane = threadIdx.x & 63;
-    const int wave = uniform(threadIdx.x >> 6);
+    const int wave = kWavesPerBlock == 1 ? 0 : uniform(threadIdx.x >> 6);    // a constant LDS base with one wavefront per workgroup
     const int slot = blockIdx.x * kWavesPerBlock + wave;
     if (slot >= n_mols) return;
     const int mol = order ? uniform(order[slot]) : slot;      // largest molecules first when an order is given
@@ -108,7 +108,6 @@ void aev_fwd_small_kernel(
     orig = lane_push(dest, orig);
     const int rp_lo = lane_push(dest, static_cast<int>(rowbits & 0xffffffffull));
     const int rp_hi = lane_push(dest, static_cast<int>(rowbits >> 32));
-    S.atom[lane] = Fast<T>::make4(x, y, z, static_cast<T>(type));
     if constexpr (kJvp) {
         vx = lane_push(dest, vx);
         vy = lane_push(dest, vy);
@@ -143,6 +142,9 @@ void aev_fwd_small_kernel(
     const int rg_ns = 4 / G;                                   // 1, 2 or 4
     const int rg_g = G == 4 ? rg : G == 2 ? (rg >> 1) : 0;
     const int rg_s = G == 4 ? 0 : G == 2 ? (rg & 1) : rg;
+    // the sorted atoms stay in the lanes' registers: the partner this lane tests in every scan step, once; the
+    // step's centres by lane exchange
+    const T xj = lane_fetch(x, jl << 2), yj = lane_fetch(y, jl << 2), zj = lane_fetch(z, jl << 2);
 
     fwd_lds_init(S, lane);
     wave_lds_fence();
@@ -156,9 +158,8 @@ void aev_fwd_small_kernel(
             const int b = b0 + grp;                      // centre-in-batch of this lane's group
             const int i = c0 + b;
             const bool centre_ok = b < nb;
-            const vec4 ai = S.atom[centre_ok ? i : 0];
-            const vec4 aj = S.atom[jl];
-            const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
+            const int ci = (centre_ok ? i : 0) << 2;
+            const T dx = lane_fetch(x, ci) - xj, dy = lane_fetch(y, ci) - yj, dz = lane_fetch(z, ci) - zj;
             const T r = sqrt(dx * dx + dy * dy + dz * dz);
             const bool valid = centre_ok && (jl < n) && (jl != i);
             // a coincident atom (r = 0) has no direction: it takes no part in any derivative.  In the features it

@@ -256,12 +256,17 @@ void aev_bwd_small_kernel(
         {
             const int4 m03 = *reinterpret_cast<const int4*>(&S.nM[0]);
             const int4 m47 = *reinterpret_cast<const int4*>(&S.nM[4]);
-            const int b = (lane >= pf[1]) + (lane >= pf[2]) + (lane >= pf[3]) + (lane >= pf[4]) + (lane >= pf[5]);
-            const int bs = lane < total ? b : 0;
+            // a short pool is walked by two or four lanes per entry, which share its rounds
+            const int copies = round_copies(total), span = 64 / copies;
+            const int entry = lane & (span - 1), copy = lane / span;
+            const int b = (entry >= pf[1]) + (entry >= pf[2]) + (entry >= pf[3]) + (entry >= pf[4]) + (entry >= pf[5]);
+            const int bs = entry < total ? b : 0;
             const int pb = sel6(bs, pf[0], pf[1], pf[2], pf[3], pf[4], pf[5]);
             const int m = sel6(bs, m03.x, m03.y, m03.z, m03.w, m47.x, m47.y);   // 0 for a centre that did not fit
+            const vec4 fall = bwd_angular_rounds<T>(S.pool, entry, copy, copies, (entry < total) && (m > 0), bs, pb, m, type_of);
+            // from here on one lane per entry again
             const bool live = (lane < total) && (m > 0);
-            const vec4 f = bwd_angular_rounds<T>(S.pool, lane, live, bs, pb, m, type_of);
+            const vec4 f = fall;
             const int self = live ? lane : 0;
             // -------------------------------------------- gather: partners get their slot, the centre minus the sum
             const int atom = S.pool.nbr_idx[self];

@@ -12,11 +12,14 @@ constexpr int kB = 6;          // centres per batch: 6 x 10 type pairs = 60 segm
 constexpr int kCapA = 32;      // angular neighbours kept per centre
 constexpr int kBitWords = 96;  // 6 centres x (496 triples + padding) fit in 96 x 32 slot bits
 
+// One (centre, type pair) segment of a batch's triples, laid out so that a lane decodes its triple with few
+// instructions: fields sit on byte / half-word boundaries (the operand selects of the vector instructions read them
+// in place) and the list offsets are byte offsets, ready to be added to.
 struct __align__(16) SegDesc {
-    int start_cnt;       // first triple slot of the segment inside the batch (even, low 12 bits) | triples << 12
-    int packed;          // centre-in-batch | offset of type a | offset of type b | n_a | a==b | pair index
-    unsigned row_lo;     // address of the segment's 32 output floats
-    unsigned row_hi;
+    unsigned start_cnt;  // first triple slot of the segment inside the batch (even, low 16 bits) | triples << 16
+    unsigned aj;         // byte offset, inside the batch's neighbour lists, of the centre's first entry of type a
+    unsigned ak;         // the same for type b
+    unsigned div;        // floor(2^15 / n_a) + 1 (low 16 bits: q / n_a = q * that >> 15 for q < 1024) | n_a << 16 | (a == b) << 24
 };
 
 
@@ -175,6 +178,32 @@ __device__ __forceinline__ float group_sum_to_last_lane(float v, int log_group)
     if (log_group >= 5) v += dpp_take_f<0x142, 0xa>(v);
     if (log_group >= 6) v += dpp_take_f<0x143, 0xc>(v);
     return v;
+}
+
+// 1 + cos(theta - theta_t) for the eight theta_t = t pi/4, from c = cos(theta) and s = sin(theta) >= 0.
+// double: each from the table's cos/sin of the float-rounded theta_t, as the 1e-12 tolerance needs.
+// float: theta_0 = 0 is exact; theta_2, theta_4 and theta_6 are within 9e-8 of pi/2, pi and 3 pi/2, so their values are
+// 1 + s, 1 - c and 1 - s to 9e-8; theta_1 and theta_5 are within 7e-8 of pi/4 and 5 pi/4 and share
+// p = (c + s)/sqrt(2): 12 instructions instead of 16, the values within 1e-7 of the table's (a few percent of
+// the tolerance after the eighth power).  theta_3 and theta_7 (the latter 1.5e-7 off) keep their table entries.
+template <typename T>
+__device__ __forceinline__ void theta_bases(T c, T s, T (&b)[8])
+{
+    if constexpr (sizeof(T) == 4) {
+        const T p = T(0.70710678118654752) * (c + s);
+        b[0] = T(1) + c;
+        b[4] = T(1) - c;
+        b[2] = T(1) + s;
+        b[6] = T(1) - s;
+        b[1] = T(1) + p;
+        b[5] = T(1) - p;
+        b[3] = fma(s, static_cast<T>(kSinTheta[3]), fma(c, static_cast<T>(kCosTheta[3]), T(1)));
+        b[7] = fma(s, static_cast<T>(kSinTheta[7]), fma(c, static_cast<T>(kCosTheta[7]), T(1)));
+    } else {
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+            b[t] = fma(s, static_cast<T>(kSinTheta[t]), fma(c, static_cast<T>(kCosTheta[t]), T(1)));
+    }
 }
 
 template <typename T>
