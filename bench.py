@@ -289,21 +289,28 @@ def main():
     # queue does, the feeder side runs one batch ahead: a step enqueues the sort of the NEXT batch (same synthetic
     # data) and the asynchronous copy of its counts into pinned memory, then the forward and backward passes of the
     # current batch, whose counts arrived a step ago.  Every step does one sort, one forward and one backward.
-    acs_pinned = [torch.empty(4, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+    # [0:4] the atom counts of ani_sort, [4:8] the size-class counts behind the size order
+    counts_pinned = [torch.empty(8, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+    main_stream = torch.cuda.current_stream()
+    feed_stream = torch.cuda.Stream()          # default priority; the feeder side of the pipeline, as in khan_amd.batching
 
     def enqueue_sort(slot, timed):
         m0 = m1 = None
-        if timed:
-            m0, m1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            m0.record()
-        macs, mos = ops.mol_offsets(mol_idxs, n_mols)
-        sc, ga, ac = ops.ani_sort(A)
-        order = ops.size_order(macs)       # largest molecules first: once per batch, shared by both passes
-        if timed:
-            m1.record()
-        acs_pinned[slot].copy_(ac, non_blocking=True)
-        done = torch.cuda.Event()
-        done.record()
+        with torch.cuda.stream(feed_stream):
+            if timed:
+                m0, m1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                m0.record()
+            macs, mos = ops.mol_offsets(mol_idxs, n_mols)
+            sc, ga, ac = ops.ani_sort(A)
+            order = ops.size_order(macs)       # largest molecules first: once per batch, shared by both passes
+            if timed:
+                m1.record()
+            counts_pinned[slot][0:4].copy_(ac, non_blocking=True)
+            counts_pinned[slot][4:8].copy_(order[-4:], non_blocking=True)
+            done = torch.cuda.Event()
+            done.record()
+            for t in (macs, mos, sc, ga, ac, order):
+                t.record_stream(main_stream)   # allocated on the feeder's stream, read by the passes on the main one
         return {"macs": macs, "mos": mos, "sc": sc, "order": order, "slot": slot, "done": done, "marks": (m0, m1)}
 
     state = {"cur": None, "n": 0}
@@ -315,7 +322,9 @@ def main():
         state["n"] += 1
         nxt = enqueue_sort(state["n"] & 1, timed)           # the next batch's sort, ahead of this batch's passes
         cur["done"].synchronize()                           # this batch's counts: copied a step ago
-        acs = acs_pinned[cur["slot"]].clone()
+        main_stream.wait_event(cur["done"])
+        acs = counts_pinned[cur["slot"]][0:4].clone()
+        classes = counts_pinned[cur["slot"]][4:8].clone()
         macs, mos, sc, order = cur["macs"], cur["mos"], cur["sc"], cur["order"]
         # events sit directly around each op, on the stream the kernels are launched on
         marks = [torch.cuda.Event(enable_timing=True) for _ in range(4)] if timed else None
@@ -325,11 +334,11 @@ def main():
             start += c
         if timed:
             marks[0].record()
-        feats = ops.featurize(X, Y, Z, A, mos, macs, sc, acs, order=order)
+        feats = ops.featurize(X, Y, Z, A, mos, macs, sc, acs, order=order, size_classes=classes)
         if timed:
             marks[1].record()
             marks[2].record()
-        gx, gy, gz = ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *grads, order=order)
+        gx, gy, gz = ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *grads, order=order, size_classes=classes)
         if timed:
             marks[3].record()
         if with_charges:     # energy, then its gradient with respect to charges and coordinates
@@ -401,7 +410,9 @@ def main():
         "config": {"workload": "%s: ani_sort + AEV forward + AEV backward%s, %d molecules, %d atoms" % (
             args.workload, " + ani_charge energy and gradients" if with_charges else "", n_mols, N), "n_mols": n_mols, "n_atoms": N, "work_counts": counts,
             "feeding": "each step enqueues the next batch's mol_offsets + ani_sort + size_order (and the copy of its 4 atom "
-                       "counts to the host) ahead of the current batch's forward and backward, which share that order"},
+                       "counts and 4 size-class counts to the host) on a feeder stream, ahead of the current batch's "
+                       "forward and backward on the main stream, which share that order and launch only the kernels "
+                       "whose size class is present"},
         "molecules_per_s": n_mols / (ms_per_step * 1e-3),
         "roofline": roofline,
     }

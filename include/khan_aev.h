@@ -88,7 +88,7 @@ int khan_featurize_f64(const double *xs, const double *ys, const double *zs, con
 /* khan_featurize_f32 for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments,
  * same results.  khan_featurize_f32 takes its scratch buffer (the molecule indices in order of decreasing
- * size, one int per molecule + 516) from the stream-ordered allocator on every call; this one keeps it in a
+ * size, one int per molecule + 520) from the stream-ordered allocator on every call; this one keeps it in a
  * fixed array inside the library's code object (4.2 MB per GPU, held until the process ends) and calls no
  * hipMalloc, hipFree or other allocating routine.  More than KHAN_FEATURIZE_NOALLOC_MAX_MOLS molecules:
  * KHAN_ERR_TOO_LARGE, nothing launched.  Every call on a GPU uses that GPU's one array: calls that overlap
@@ -143,47 +143,54 @@ int khan_featurize_grad_inverse_f64(const double *xs, const double *ys, const do
  * molecules first; every khan_featurize* / khan_featurize_grad* call above works this order out for itself in a
  * stream-ordered scratch allocation (and goes without it while its stream is being captured into a graph).
  * khan_size_order writes it into caller memory instead -- order[n_mols + KHAN_SIZE_ORDER_EXTRA] int32, device:
- * the molecule indices by decreasing atom count, then per-size-class counts -- and the *_ordered entry points
- * take it as an argument: the same results bit for bit, one order per batch instead of one per call, no
- * allocation, and usable under graph capture.  `order` may be NULL (molecules are then taken in batch order). */
-#define KHAN_SIZE_ORDER_EXTRA 516
+ * the molecule indices by decreasing atom count, then per-size counts, and in its last four elements the number
+ * of molecules of up to 32 atoms, of 33..64, of 65..256 and of more -- and the *_ordered entry points take it as
+ * an argument: the same results bit for bit, one order per batch instead of one per call, no allocation, and
+ * usable under graph capture.  `order` may be NULL (molecules are then taken in batch order).
+ * size_classes_host (HOST memory, may be NULL) is a copy of those last four elements: a caller that brings them
+ * to the host anyway -- as it does the four atom counts of khan_ani_sort -- spares every pass the launches of
+ * the kernels whose size class is empty in this batch (with NULL every kernel is launched and leaves by itself). */
+#define KHAN_SIZE_ORDER_EXTRA 520
 int khan_size_order(const int32_t *macs, int32_t n_mols, int32_t *order, khan_stream_t stream);
 int khan_featurize_ordered_f32(const float *xs, const float *ys, const float *zs, const int32_t *as,
                                const int32_t *mos, const int32_t *macs, int32_t n_mols,
                                const int32_t *sis, float *h_feat, float *c_feat, float *n_feat,
                                float *o_feat, const int32_t *acs_host, const int32_t *order,
-                               khan_stream_t stream);
+                               const int32_t *size_classes_host, khan_stream_t stream);
 int khan_featurize_ordered_f64(const double *xs, const double *ys, const double *zs, const int32_t *as,
                                const int32_t *mos, const int32_t *macs, int32_t n_mols,
                                const int32_t *sis, double *h_feat, double *c_feat, double *n_feat,
                                double *o_feat, const int32_t *acs_host, const int32_t *order,
-                               khan_stream_t stream);
+                               const int32_t *size_classes_host, khan_stream_t stream);
 int khan_featurize_grad_ordered_f32(const float *xs, const float *ys, const float *zs,
                                     const int32_t *as, const int32_t *mos, const int32_t *macs,
                                     int32_t n_mols, const int32_t *sis, const float *h_grads,
                                     const float *c_grads, const float *n_grads, const float *o_grads,
                                     float *x_grads, float *y_grads, float *z_grads,
-                                    const int32_t *acs_host, const int32_t *order, khan_stream_t stream);
+                                    const int32_t *acs_host, const int32_t *order,
+                                    const int32_t *size_classes_host, khan_stream_t stream);
 int khan_featurize_grad_ordered_f64(const double *xs, const double *ys, const double *zs,
                                     const int32_t *as, const int32_t *mos, const int32_t *macs,
                                     int32_t n_mols, const int32_t *sis, const double *h_grads,
                                     const double *c_grads, const double *n_grads, const double *o_grads,
                                     double *x_grads, double *y_grads, double *z_grads,
-                                    const int32_t *acs_host, const int32_t *order, khan_stream_t stream);
+                                    const int32_t *acs_host, const int32_t *order,
+                                    const int32_t *size_classes_host, khan_stream_t stream);
 int khan_featurize_grad_inverse_ordered_f32(const float *xs, const float *ys, const float *zs,
                                             const int32_t *as, const int32_t *mos, const int32_t *macs,
                                             int32_t n_mols, const int32_t *sis, const float *x_grads,
                                             const float *y_grads, const float *z_grads, float *h_grads,
                                             float *c_grads, float *n_grads, float *o_grads,
                                             const int32_t *acs_host, const int32_t *order,
-                                            khan_stream_t stream);
+                                            const int32_t *size_classes_host, khan_stream_t stream);
 int khan_featurize_grad_inverse_ordered_f64(const double *xs, const double *ys, const double *zs,
                                             const int32_t *as, const int32_t *mos, const int32_t *macs,
                                             int32_t n_mols, const int32_t *sis, const double *x_grads,
                                             const double *y_grads, const double *z_grads,
                                             double *h_grads, double *c_grads, double *n_grads,
                                             double *o_grads, const int32_t *acs_host,
-                                            const int32_t *order, khan_stream_t stream);
+                                            const int32_t *order, const int32_t *size_classes_host,
+                                            khan_stream_t stream);
 
 /* AniCharge (gpu_featurizer/ani_charges.cpp:45-52 registration, 58-71 charge_energy, 81-119 Compute;
  * CUDA twin ani_charges_gpu.cu:70-128).

@@ -28,7 +28,7 @@ def _featurize_grad_sig():
 
 
 def _ordered(sig):
-    return sig[:-1] + [_ptr, _ptr]        # ..., acs_host, order, stream
+    return sig[:-1] + [_ptr, ctypes.POINTER(ctypes.c_int32), _ptr]        # ..., acs_host, order, size_classes_host, stream
 
 
 _SIGNATURES = {

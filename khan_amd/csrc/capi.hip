@@ -105,79 +105,76 @@ private:
     hipStream_t stream_;
 };
 
-int forward_dispatch(const float* xs, const float* ys, const float* zs, const int32_t* as,
-                     const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
-                     khan::Buckets<float> out, const int32_t* order, hipStream_t stream)
+// Which kernels have work.  `classes` (host memory, null = not known: launch everything) holds the number of molecules
+// of up to 32 atoms, of 33..64, of 65..256 and of more, as khan_size_order leaves them behind the order.
+struct SizeClasses {
+    bool known;
+    int32_t n[khan::kSizeClasses];
+    explicit SizeClasses(const int32_t* host) : known(host != nullptr)
+    {
+        for (int c = 0; c < khan::kSizeClasses; ++c) n[c] = host ? host[c] : 1;
+    }
+    // any molecule with lo <= atom count <= hi (lo, hi on class boundaries)?
+    bool any(int lo, int hi) const
+    {
+        if (!known) return true;
+        static const int first[khan::kSizeClasses] = {0, 33, 65, 257};
+        for (int c = 0; c < khan::kSizeClasses; ++c) {
+            const int last = c + 1 < khan::kSizeClasses ? first[c + 1] - 1 : INT32_MAX;
+            if (first[c] >= lo && last <= hi && n[c] > 0) return true;
+        }
+        return false;
+    }
+};
+
+// forward: one wavefront per molecule up to 32 atoms (float32; 64 in float64), one workgroup up to 256, the
+// general kernel above
+template <typename T>
+int forward_dispatch(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
+                     const int32_t* macs, int32_t n_mols, const int32_t* sis, khan::Buckets<T> out,
+                     const int32_t* order, const int32_t* classes_host, hipStream_t stream)
 {
     if (force_generic())
-        return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, nullptr, stream));
-    // molecules of up to 32 atoms: one wavefront each; up to 256: one workgroup each; the rest: general kernel
-    int st = hip_status(khan::launch_fwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallPreferredMax,
-                                                      order, stream));
-    if (st != KHAN_OK) return st;
-    st = hip_status(khan::launch_fwd_medium<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallPreferredMax + 1,
-                                                   order, stream));
-    if (st != KHAN_OK) return st;
-    return hip_status(khan::launch_fwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
-                                                      khan::kMediumMaxAtoms + 1, order, stream));
+        return hip_status(khan::launch_fwd_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, nullptr, stream));
+    constexpr int small_max = sizeof(T) == 4 ? khan::kSmallPreferredMax : khan::kSmallMaxAtoms;
+    const SizeClasses cls(classes_host);
+    int st = KHAN_OK;
+    if (cls.any(0, small_max))
+        st = hip_status(khan::launch_fwd_small<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out, small_max, order, stream));
+    if (st == KHAN_OK && cls.any(small_max + 1, khan::kMediumMaxAtoms))
+        st = hip_status(khan::launch_fwd_medium<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out, small_max + 1, order, stream));
+    if (st == KHAN_OK && cls.any(khan::kMediumMaxAtoms + 1, INT32_MAX))
+        st = hip_status(khan::launch_fwd_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
+                                                    khan::kMediumMaxAtoms + 1, order, stream));
+    return st;
 }
 
-int forward_dispatch(const double* xs, const double* ys, const double* zs, const int32_t* as,
-                     const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
-                     khan::Buckets<double> out, const int32_t* order, hipStream_t stream)
-{
-    if (force_generic())
-        return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, nullptr, stream));
-    int st = hip_status(khan::launch_fwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallMaxAtoms,
-                                                       order, stream));
-    if (st != KHAN_OK) return st;
-    // 65..256 atoms: one workgroup each (in float64 a one-wavefront kernel keeps molecules of up to 64 atoms)
-    st = hip_status(khan::launch_fwd_medium<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out, khan::kSmallMaxAtoms + 1,
-                                                    order, stream));
-    if (st != KHAN_OK) return st;
-    return hip_status(khan::launch_fwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
-                                                       khan::kMediumMaxAtoms + 1, order, stream));
-}
-
-int backward_dispatch(const float* xs, const float* ys, const float* zs, const int32_t* as,
-                      const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
-                      khan::Buckets<const float> g, float* gx, float* gy, float* gz, int64_t n_atoms,
-                      const int32_t* order, hipStream_t stream)
+// backward: the same split; each kernel defines every gradient of its own molecules
+template <typename T>
+int backward_dispatch(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
+                      const int32_t* macs, int32_t n_mols, const int32_t* sis, khan::Buckets<const T> g,
+                      T* gx, T* gy, T* gz, int64_t n_atoms, const int32_t* order, const int32_t* classes_host,
+                      hipStream_t stream)
 {
     // the specialised kernels fetch upstream rows in 16-byte pieces; buckets that are not 16-byte aligned
     // (rows are 1,536 bytes, so the bucket's base decides) go through the general kernel, which does not care
     if (force_generic() || !aligned16(g))
-        return hip_status(khan::launch_bwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                          n_atoms, 0, nullptr, stream));
-    // by molecule size: above 256 atoms the general kernel, 33..256 one workgroup per molecule, up to 32
-    // one wavefront per molecule; each kernel defines every gradient of its own molecules
-    int st = hip_status(khan::launch_bwd_generic<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                        n_atoms, khan::kMediumMaxAtoms + 1, order, stream));
-    if (st != KHAN_OK) return st;
+        return hip_status(khan::launch_bwd_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                      n_atoms, 0, nullptr, stream));
+    constexpr int small_max = sizeof(T) == 4 ? khan::kSmallPreferredMax : khan::kSmallMaxAtoms;
+    const SizeClasses cls(classes_host);
+    int st = KHAN_OK;
+    if (cls.any(khan::kMediumMaxAtoms + 1, INT32_MAX))
+        st = hip_status(khan::launch_bwd_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                    n_atoms, khan::kMediumMaxAtoms + 1, order, stream));
     // (the workgroup-per-molecule backward kernel measures slower when it walks the molecules in size order)
-    st = hip_status(khan::launch_bwd_medium<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                   khan::kSmallPreferredMax + 1, order, false, stream));
-    if (st != KHAN_OK) return st;
-    return hip_status(khan::launch_bwd_small<float>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                    khan::kSmallPreferredMax, order, stream));
-}
-
-int backward_dispatch(const double* xs, const double* ys, const double* zs, const int32_t* as,
-                      const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
-                      khan::Buckets<const double> g, double* gx, double* gy, double* gz, int64_t n_atoms,
-                      const int32_t* order, hipStream_t stream)
-{
-    if (force_generic() || !aligned16(g))
-        return hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                           n_atoms, 0, nullptr, stream));
-    int st = hip_status(khan::launch_bwd_generic<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                         n_atoms, khan::kMediumMaxAtoms + 1, order, stream));
-    if (st != KHAN_OK) return st;
-    st = hip_status(khan::launch_bwd_medium<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                    khan::kSmallMaxAtoms + 1, order, false, stream));
-    if (st != KHAN_OK) return st;
-    return hip_status(khan::launch_bwd_small<double>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                     khan::kSmallMaxAtoms, order, stream));
+    if (st == KHAN_OK && cls.any(small_max + 1, khan::kMediumMaxAtoms))
+        st = hip_status(khan::launch_bwd_medium<T>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                   small_max + 1, order, false, stream));
+    if (st == KHAN_OK && cls.any(0, small_max))
+        st = hip_status(khan::launch_bwd_small<T>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                  small_max, order, stream));
+    return st;
 }
 
 // zeros to the four buckets (a batch with atoms but no molecule: the reference zero-fills its outputs before it
@@ -219,16 +216,16 @@ template <typename T>
 int featurize_impl(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
                    const int32_t* macs, int32_t n_mols, const int32_t* sis, T* h, T* c, T* n, T* o,
                    const int32_t* acs_host, khan_stream_t stream, const int32_t* caller_order = nullptr,
-                   bool own_order = true)
+                   const int32_t* classes_host = nullptr, bool own_order = true)
 {
     bool run;
     const int st = featurize_check(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, as_stream(stream), &run);
     if (st != KHAN_OK || !run) return st;
     khan::Buckets<T> out{{h, c, n, o}};
     if (!own_order)       // the caller's size order (or none): nothing is allocated
-        return forward_dispatch(xs, ys, zs, as, mos, macs, n_mols, sis, out, caller_order, as_stream(stream));
+        return forward_dispatch<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out, caller_order, classes_host, as_stream(stream));
     SizeOrder order(macs, n_mols, as_stream(stream));
-    return forward_dispatch(xs, ys, zs, as, mos, macs, n_mols, sis, out, order.get(), as_stream(stream));
+    return forward_dispatch<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out, order.get(), nullptr, as_stream(stream));
 }
 
 template <typename T>
@@ -236,7 +233,7 @@ int featurize_grad_impl(const T* xs, const T* ys, const T* zs, const int32_t* as
                         const int32_t* macs, int32_t n_mols, const int32_t* sis, const T* gh,
                         const T* gc, const T* gn, const T* go, T* gx, T* gy, T* gz,
                         const int32_t* acs_host, khan_stream_t stream, const int32_t* caller_order = nullptr,
-                        bool own_order = true)
+                        const int32_t* classes_host = nullptr, bool own_order = true)
 {
     if (n_mols < 0 || !acs_host) return KHAN_ERR_INVALID_ARG;
     if (acs_host[0] < 0 || acs_host[1] < 0 || acs_host[2] < 0 || acs_host[3] < 0) return KHAN_ERR_INVALID_ARG;
@@ -257,9 +254,10 @@ int featurize_grad_impl(const T* xs, const T* ys, const T* zs, const int32_t* as
         return KHAN_ERR_INVALID_ARG;
     khan::Buckets<const T> g{{gh, gc, gn, go}};
     if (!own_order)
-        return backward_dispatch(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, n_atoms, caller_order, as_stream(stream));
+        return backward_dispatch<T>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, n_atoms, caller_order, classes_host,
+                                    as_stream(stream));
     SizeOrder order(macs, n_mols, as_stream(stream));
-    return backward_dispatch(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, n_atoms, order.get(), as_stream(stream));
+    return backward_dispatch<T>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, n_atoms, order.get(), nullptr, as_stream(stream));
 }
 
 template <typename T>
@@ -267,7 +265,7 @@ int featurize_grad_inverse_impl(const T* xs, const T* ys, const T* zs, const int
                                 const int32_t* macs, int32_t n_mols, const int32_t* sis, const T* vx,
                                 const T* vy, const T* vz, T* h, T* c, T* n, T* o,
                                 const int32_t* acs_host, khan_stream_t stream, const int32_t* caller_order = nullptr,
-                                bool own_order = true)
+                                const int32_t* classes_host = nullptr, bool own_order = true)
 {
     bool run;
     const int chk = featurize_check(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, as_stream(stream), &run);
@@ -280,18 +278,22 @@ int featurize_grad_inverse_impl(const T* xs, const T* ys, const T* zs, const int
     // molecules of up to 64 atoms: one wavefront each; 65..256 in float32: one workgroup each; the rest: general-shape kernel
     SizeOrder made(own_order ? macs : nullptr, own_order ? n_mols : 0, as_stream(stream));
     const int32_t* order = own_order ? made.get() : caller_order;
-    int st = hip_status(khan::launch_jvp_small<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, order,
+    const SizeClasses cls(own_order ? nullptr : classes_host);
+    int st = KHAN_OK;
+    if (cls.any(0, khan::kSmallMaxAtoms))
+        st = hip_status(khan::launch_jvp_small<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, order,
                                                   as_stream(stream)));
-    if (st != KHAN_OK) return st;
     int generic_from = khan::kSmallMaxAtoms + 1;
     if constexpr (sizeof(T) == 4) {
-        st = hip_status(khan::launch_jvp_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
-                                                    khan::kSmallMaxAtoms + 1, order, as_stream(stream)));
-        if (st != KHAN_OK) return st;
+        if (st == KHAN_OK && cls.any(khan::kSmallMaxAtoms + 1, khan::kMediumMaxAtoms))
+            st = hip_status(khan::launch_jvp_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
+                                                        khan::kSmallMaxAtoms + 1, order, as_stream(stream)));
         generic_from = khan::kMediumMaxAtoms + 1;
     }
-    return hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
-                                                  generic_from, order, as_stream(stream)));
+    if (st == KHAN_OK && cls.any(generic_from, INT32_MAX))
+        st = hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
+                                                    generic_from, order, as_stream(stream)));
+    return st;
 }
 
 template <typename T>
@@ -420,7 +422,7 @@ int khan_featurize_f32_noalloc(const float* xs, const float* ys, const float* zs
     e = khan::launch_size_order(macs, n_mols, order, as_stream(stream));
     if (e != hipSuccess) return hip_status(e);
     khan::Buckets<float> out{{h, c, n, o}};
-    return forward_dispatch(xs, ys, zs, as, mos, macs, n_mols, sis, out, order, as_stream(stream));
+    return forward_dispatch<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, order, nullptr, as_stream(stream));
 }
 
 int khan_featurize_grad_f32(const float* xs, const float* ys, const float* zs, const int32_t* as,
@@ -532,52 +534,58 @@ int khan_coulomb_grad_f64(const double* xs, const double* ys, const double* zs, 
 int khan_featurize_ordered_f32(const float* xs, const float* ys, const float* zs, const int32_t* as,
                                const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
                                float* h, float* c, float* n, float* o, const int32_t* acs_host,
-                               const int32_t* order, khan_stream_t stream)
+                               const int32_t* order, const int32_t* size_classes_host,
+        khan_stream_t stream)
 {
-    return featurize_impl<float>(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, stream, order, false);
+    return featurize_impl<float>(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, stream, order, size_classes_host, false);
 }
 int khan_featurize_ordered_f64(const double* xs, const double* ys, const double* zs, const int32_t* as,
                                const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
                                double* h, double* c, double* n, double* o, const int32_t* acs_host,
-                               const int32_t* order, khan_stream_t stream)
+                               const int32_t* order, const int32_t* size_classes_host,
+        khan_stream_t stream)
 {
-    return featurize_impl<double>(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, stream, order, false);
+    return featurize_impl<double>(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, stream, order, size_classes_host, false);
 }
 int khan_featurize_grad_ordered_f32(const float* xs, const float* ys, const float* zs, const int32_t* as,
                                     const int32_t* mos, const int32_t* macs, int32_t n_mols,
                                     const int32_t* sis, const float* gh, const float* gc, const float* gn,
                                     const float* go, float* gx, float* gy, float* gz,
-                                    const int32_t* acs_host, const int32_t* order, khan_stream_t stream)
+                                    const int32_t* acs_host, const int32_t* order, const int32_t* size_classes_host,
+        khan_stream_t stream)
 {
     return featurize_grad_impl<float>(xs, ys, zs, as, mos, macs, n_mols, sis, gh, gc, gn, go, gx, gy, gz,
-                                      acs_host, stream, order, false);
+                                      acs_host, stream, order, size_classes_host, false);
 }
 int khan_featurize_grad_ordered_f64(const double* xs, const double* ys, const double* zs, const int32_t* as,
                                     const int32_t* mos, const int32_t* macs, int32_t n_mols,
                                     const int32_t* sis, const double* gh, const double* gc, const double* gn,
                                     const double* go, double* gx, double* gy, double* gz,
-                                    const int32_t* acs_host, const int32_t* order, khan_stream_t stream)
+                                    const int32_t* acs_host, const int32_t* order, const int32_t* size_classes_host,
+        khan_stream_t stream)
 {
     return featurize_grad_impl<double>(xs, ys, zs, as, mos, macs, n_mols, sis, gh, gc, gn, go, gx, gy, gz,
-                                       acs_host, stream, order, false);
+                                       acs_host, stream, order, size_classes_host, false);
 }
 int khan_featurize_grad_inverse_ordered_f32(const float* xs, const float* ys, const float* zs, const int32_t* as,
                                             const int32_t* mos, const int32_t* macs, int32_t n_mols,
                                             const int32_t* sis, const float* x_grads, const float* y_grads,
                                             const float* z_grads, float* h, float* c, float* n, float* o,
-                                            const int32_t* acs_host, const int32_t* order, khan_stream_t stream)
+                                            const int32_t* acs_host, const int32_t* order, const int32_t* size_classes_host,
+        khan_stream_t stream)
 {
     return featurize_grad_inverse_impl<float>(xs, ys, zs, as, mos, macs, n_mols, sis, x_grads, y_grads, z_grads,
-                                              h, c, n, o, acs_host, stream, order, false);
+                                              h, c, n, o, acs_host, stream, order, size_classes_host, false);
 }
 int khan_featurize_grad_inverse_ordered_f64(const double* xs, const double* ys, const double* zs, const int32_t* as,
                                             const int32_t* mos, const int32_t* macs, int32_t n_mols,
                                             const int32_t* sis, const double* x_grads, const double* y_grads,
                                             const double* z_grads, double* h, double* c, double* n, double* o,
-                                            const int32_t* acs_host, const int32_t* order, khan_stream_t stream)
+                                            const int32_t* acs_host, const int32_t* order, const int32_t* size_classes_host,
+        khan_stream_t stream)
 {
     return featurize_grad_inverse_impl<double>(xs, ys, zs, as, mos, macs, n_mols, sis, x_grads, y_grads, z_grads,
-                                               h, c, n, o, acs_host, stream, order, false);
+                                               h, c, n, o, acs_host, stream, order, size_classes_host, false);
 }
 
 }  // extern "C"

@@ -75,12 +75,15 @@ hipError_t launch_ani_sort(const int32_t* A, int64_t n_atoms, int32_t* scatter, 
                            int32_t* counts4, hipStream_t stream);
 
 // Molecule indices by decreasing atom count.  `order` holds n_mols + kSizeOrderScratch ints: the indices, then the
-// number of molecules per size class (kSizeBins entries, class = size_bin(atom count)), then the pass's cursors.
+// number of molecules per size (kSizeBins entries, bin = size_bin(atom count)), then the pass's cursors, then the
+// number of molecules of up to 32 atoms, of 33..64, of 65..256 and of more (kSizeClasses entries: what a host needs
+// to know which kernels have work).
 // Every `order` argument of the launchers above is such an array (or null): the kernels for larger molecules read
 // the class counts behind the indices to leave at once when the batch holds no molecule for them.
 // Kernels only (the counts are cleared by a small kernel), so the sequence can be recorded into a graph.
 constexpr int kSizeBins = 258;    // atom counts 0..256 and "more", largest first
-constexpr int kSizeOrderScratch = 2 * kSizeBins;
+constexpr int kSizeClasses = 4;
+constexpr int kSizeOrderScratch = 2 * kSizeBins + kSizeClasses;
 __host__ __device__ __forceinline__ int size_bin(int n)
 {
     const int c = n < 0 ? 0 : n > kSizeBins - 1 ? kSizeBins - 1 : n;

@@ -311,6 +311,14 @@ __global__ __launch_bounds__(kOrderThreads) void size_place_kernel(const int32_t
     }
     __syncthreads();
     if (m < n_mols) order[start[bin] + atomicAdd(&hist[bin], 1)] = m;
+    // the four totals that tell a host which kernels have work (behind the cursors)
+    if (blockIdx.x == 0 && tid < kSizeClasses) {
+        const int lo = tid == 0 ? 0 : tid == 1 ? 33 : tid == 2 ? 65 : 257;          // atom counts of the class
+        const int hi = tid == 0 ? 32 : tid == 1 ? 64 : tid == 2 ? 256 : 257;
+        int sum = 0;
+        for (int b = size_bin(hi); b <= size_bin(lo); ++b) sum += total[b];
+        gcursor[kSizeBins + tid] = sum;
+    }
 }
 }  // namespace
 

@@ -82,13 +82,15 @@ def ani_sort(atomic_numbers):
     return scatter, gather, counts
 
 
-SIZE_ORDER_EXTRA = 516
+SIZE_ORDER_EXTRA = 520
 
 
 def size_order(macs):
-    """-> int32[n_mols + 516]: the molecule indices by decreasing atom count and the per-size-class counts, to be
+    """-> int32[n_mols + 520]: the molecule indices by decreasing atom count and the per-size counts, to be
     passed as `order=` to featurize / featurize_grad / featurize_grad_inverse of the same batch (computed once
-    per batch instead of once per call; the calls then allocate nothing and can be captured into a graph)."""
+    per batch instead of once per call; the calls then allocate nothing and can be captured into a graph).
+    Its last four elements (`order[-4:]`) count the molecules of up to 32, 33..64, 65..256 and more atoms: copied
+    to the host and passed as `size_classes=`, they spare the passes the launches of kernels without work."""
     lib = _lib.load()
     macs = _dev(macs, torch.int32, "macs")
     order = torch.empty(macs.numel() + SIZE_ORDER_EXTRA, dtype=torch.int32, device=macs.device)
@@ -101,6 +103,16 @@ def _order_arg(order, macs):
     if order.numel() != macs.numel() + SIZE_ORDER_EXTRA:
         raise ValueError("order must come from size_order(macs) of this batch")
     return order
+
+
+def _classes_arg(size_classes):
+    """host copy of order[-4:] (a CPU tensor or 4 ints), or None"""
+    if size_classes is None:
+        return None
+    vals = [int(v) for v in (size_classes.tolist() if isinstance(size_classes, torch.Tensor) else size_classes)]
+    if len(vals) != 4:
+        raise ValueError("size_classes must hold 4 counts")
+    return (ctypes.c_int32 * 4)(*vals)
 
 
 def _check_common(xs, ys, zs, as_, mos, macs, sis):
@@ -116,7 +128,7 @@ def _check_common(xs, ys, zs, as_, mos, macs, sis):
     return dt, n
 
 
-def featurize(xs, ys, zs, as_, mos, macs, sis, acs, order=None):
+def featurize(xs, ys, zs, as_, mos, macs, sis, acs, order=None, size_classes=None):
     """-> (h_feat, c_feat, n_feat, o_feat), flat tensors of acs[t]*384 elements.
 
     The four outputs are consecutive slices of one allocation, so
@@ -137,11 +149,11 @@ def featurize(xs, ys, zs, as_, mos, macs, sis, acs, order=None):
     if order is None:
         _lib.check(getattr(lib, "khan_featurize_" + _SUFFIX[dt])(*args, _stream()))
     else:
-        _lib.check(getattr(lib, "khan_featurize_ordered_" + _SUFFIX[dt])(*args, _p(_order_arg(order, macs)), _stream()))
+        _lib.check(getattr(lib, "khan_featurize_ordered_" + _SUFFIX[dt])(*args, _p(_order_arg(order, macs)), _classes_arg(size_classes), _stream()))
     return tuple(outs)
 
 
-def featurize_grad(xs, ys, zs, as_, mos, macs, sis, acs, h_grads, c_grads, n_grads, o_grads, order=None):
+def featurize_grad(xs, ys, zs, as_, mos, macs, sis, acs, h_grads, c_grads, n_grads, o_grads, order=None, size_classes=None):
     """-> (x_grads, y_grads, z_grads), each [n_atoms] in original atom order."""
     lib = _lib.load()
     dt, n = _check_common(xs, ys, zs, as_, mos, macs, sis)
@@ -162,11 +174,11 @@ def featurize_grad(xs, ys, zs, as_, mos, macs, sis, acs, h_grads, c_grads, n_gra
     if order is None:
         _lib.check(getattr(lib, "khan_featurize_grad_" + _SUFFIX[dt])(*args, _stream()))
     else:
-        _lib.check(getattr(lib, "khan_featurize_grad_ordered_" + _SUFFIX[dt])(*args, _p(_order_arg(order, macs)), _stream()))
+        _lib.check(getattr(lib, "khan_featurize_grad_ordered_" + _SUFFIX[dt])(*args, _p(_order_arg(order, macs)), _classes_arg(size_classes), _stream()))
     return gx, gy, gz
 
 
-def featurize_grad_inverse(xs, ys, zs, as_, mos, macs, sis, acs, x_grads, y_grads, z_grads, order=None):
+def featurize_grad_inverse(xs, ys, zs, as_, mos, macs, sis, acs, x_grads, y_grads, z_grads, order=None, size_classes=None):
     """-> (h_grads, c_grads, n_grads, o_grads) laid out like `featurize`'s outputs: the Jacobian of the
     features applied to one vector per atom, row_i[f] = sum_a dAEV_i[f]/dxyz_a . (x,y,z)_grads[a].
     It is the gradient of `featurize_grad` with respect to its upstream gradients
@@ -192,7 +204,7 @@ def featurize_grad_inverse(xs, ys, zs, as_, mos, macs, sis, acs, x_grads, y_grad
     if order is None:
         _lib.check(getattr(lib, "khan_featurize_grad_inverse_" + _SUFFIX[dt])(*args, _stream()))
     else:
-        _lib.check(getattr(lib, "khan_featurize_grad_inverse_ordered_" + _SUFFIX[dt])(*args, _p(_order_arg(order, macs)), _stream()))
+        _lib.check(getattr(lib, "khan_featurize_grad_inverse_ordered_" + _SUFFIX[dt])(*args, _p(_order_arg(order, macs)), _classes_arg(size_classes), _stream()))
     return tuple(outs)
 
 

@@ -337,6 +337,67 @@ def test_mixed_sizes_in_one_ordered_batch(ops):
     _check_grad_inverse(ops, c)
 
 
+def test_size_order_workspace_and_size_classes(ops):
+    """khan_size_order: a permutation of the molecules by decreasing atom count, followed by the per-size counts and the
+    four size-class totals; the *_ordered entry points with that order -- and with a host copy of the class totals,
+    which lets them skip the kernels without work -- give what the plain entry points give."""
+    say("case: caller-owned size order, size classes, ordered entry points")
+    rng = np.random.default_rng(17)
+    for label, parts in (("organic only", [("organic", 2200)]), ("organic + boxes", [("organic", 2100), ("boxes", 5)]),
+                         ("boxes only", [("boxes", 7)])):
+        mols = []
+        for kind, k in parts:
+            b = datagen.make_batch(kind, k)
+            for m in range(b.n_mols):
+                sl = slice(b.MOs[m], b.MOs[m] + b.MACs[m])
+                mols.append((b.A[sl], np.stack([b.X[sl], b.Y[sl], b.Z[sl]], axis=1)))
+        if label == "organic + boxes":                   # one molecule for the general-shape kernel, and an empty one
+            n = 270
+            side = (n / 0.08) ** (1 / 3)
+            pts = []
+            while len(pts) < n:
+                p = rng.uniform(0, side, 3)
+                if all(np.linalg.norm(p - q) >= 0.9 for q in pts):
+                    pts.append(p)
+            mols.append((rng.integers(0, 4, n).astype(np.int32), np.array(pts, dtype=np.float32)))
+            mols.append((np.zeros(0, dtype=np.int32), np.zeros((0, 3), dtype=np.float32)))
+        mols = [mols[i] for i in rng.permutation(len(mols))]
+        A = np.concatenate([m[0] for m in mols]).astype(np.int32)
+        xyz = np.concatenate([m[1] for m in mols]).astype(np.float64)
+        mi = np.concatenate([np.full(len(m[0]), k) for k, m in enumerate(mols)]).astype(np.int32)
+        c = Case(xyz[:, 0], xyz[:, 1], xyz[:, 2], A, mi, len(mols))
+        macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+        acs = ac.cpu()
+        order = ops.size_order(macs)
+        o = host(order)
+        perm, classes = o[:c.n_mols], o[-4:]
+        assert np.array_equal(np.sort(perm), np.arange(c.n_mols)), label
+        sizes = c.MACs[perm]
+        assert np.all(np.minimum(sizes[:-1], 257) >= np.minimum(sizes[1:], 257)), "largest first"
+        want = [int((c.MACs <= 32).sum()), int(((c.MACs > 32) & (c.MACs <= 64)).sum()),
+                int(((c.MACs > 64) & (c.MACs <= 256)).sum()), int((c.MACs > 256).sum())]
+        assert classes.tolist() == want, (label, classes.tolist(), want)
+        say("   %s: %d molecules, size classes %s" % (label, c.n_mols, want))
+        Ad = dev(c.A)
+        upb = c.upstream()
+        for tdt, ndt in ((torch.float32, np.float32), (torch.float64, np.float64)):
+            X, Y, Z = dev(c.X, ndt), dev(c.Y, ndt), dev(c.Z, ndt)
+            gb = [dev(u, ndt) for u in upb]
+            v = [dev(np.random.default_rng(k).standard_normal(c.N), ndt) for k in range(3)]
+            f0 = torch.cat(ops.featurize(X, Y, Z, Ad, mos, macs, sc, acs))
+            g0 = torch.stack(ops.featurize_grad(X, Y, Z, Ad, mos, macs, sc, acs, *gb))
+            j0 = torch.cat(ops.featurize_grad_inverse(X, Y, Z, Ad, mos, macs, sc, acs, *v))
+            for cls in (None, classes):
+                f1 = torch.cat(ops.featurize(X, Y, Z, Ad, mos, macs, sc, acs, order=order, size_classes=cls))
+                g1 = torch.stack(ops.featurize_grad(X, Y, Z, Ad, mos, macs, sc, acs, *gb, order=order, size_classes=cls))
+                j1 = torch.cat(ops.featurize_grad_inverse(X, Y, Z, Ad, mos, macs, sc, acs, *v, order=order, size_classes=cls))
+                assert torch.equal(f0, f1) and torch.equal(j0, j1), (label, ndt, cls is None)
+                # molecules above one wavefront add their forces with atomics: equal up to the order of the additions
+                assert torch.allclose(g0, g1, rtol=1e-5 if ndt == np.float32 else 1e-12, atol=1e-5 if ndt == np.float32 else 1e-12)
+                one_wave = torch.from_numpy(c.MACs[c.mol_idxs] <= 32).to("cuda:0")
+                assert torch.equal(g0[:, one_wave], g1[:, one_wave])
+
+
 def test_empty_batch(ops):
     say("case: empty batch (0 atoms, 0 molecules)")
     e32 = torch.empty(0, dtype=torch.float32, device="cuda:0")
