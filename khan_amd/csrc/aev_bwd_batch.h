@@ -102,8 +102,11 @@ template <typename T> struct RowStage {
     {
 #pragma unroll
         for (int b = 0; b < kB; ++b) {
+            // Registers of centres beyond nb and of pieces beyond the row are never stored.  They are declared written
+            // without an instruction: left unset they are "undefined" to the compiler, whose handling of that cost 30
+            // registers here, and filling them with zeros costs 48 moves per batch.
 #pragma unroll
-            for (int r = 0; r < kPieceRegs; ++r) st[b][r] = v4f{0.f, 0.f, 0.f, 0.f};
+            for (int r = 0; r < kPieceRegs; ++r) asm volatile("" : "=v"(st[b][r]));
             if (b < nb) {
                 const global_v4f_ptr rowp = (global_v4f_ptr)(row_of(b) + kRadial);
 #pragma unroll

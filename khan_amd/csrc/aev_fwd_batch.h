@@ -8,35 +8,36 @@ namespace khan {
 
 // LDS working set of one wavefront
 // what the Jacobian-vector variant keeps on top of the forward working set
-template <typename T, bool kJvp> struct FwdJvpLds {};
-template <typename T> struct __align__(16) FwdJvpLds<T, true> {
+template <typename T, bool kJvp, int kNB> struct FwdJvpLds {};
+template <typename T, int kNB> struct __align__(16) FwdJvpLds<T, true, kNB> {
     typename Fast<T>::vec4 vel[64];               // the incoming vector of every atom (sorted order)
-    typename Fast<T>::vec4 nbr_p[kFB][kCapA];      // (v_centre - v_partner)/r, and its component along the unit vector
-    typename Fast<T>::vec2 nbr_d[kFB][kCapA];      // f_C'(r) dr, and dr = change of the distance along the vectors
+    typename Fast<T>::vec4 nbr_p[kNB][kCapA];      // (v_centre - v_partner)/r, and its component along the unit vector
+    typename Fast<T>::vec2 nbr_d[kNB][kCapA];      // f_C'(r) dr, and dr = change of the distance along the vectors
     typename Fast<T>::vec2 rad_ab[64];            // radial entries: f_C' dr, and -2 eta f_C dr
     T rec2[64][12];                               // phase-1 records: dA_0..7, H_0..3
 };
 
-// LDS working set of one wavefront
-template <typename T, bool kJvp = false>
+// LDS working set of one wavefront, for batches of kNB centres
+template <typename T, bool kJvp = false, int kNB = kFB>
 struct __align__(16) FwdWaveLds {
-    typename Fast<T>::vec4 nbr[kFB][kCapA];    // unit vector (centre minus partner)/r, and r
-    T nbr_fc[kFB][kCapA];                      // f_C(r, A_Rc)
+    static constexpr int kCentres = kNB;
+    typename Fast<T>::vec4 nbr[kNB][kCapA];    // unit vector (centre minus partner)/r, and r
+    T nbr_fc[kNB][kCapA];                      // f_C(r, A_Rc)
     typename Fast<T>::vec2 rad[64];           // (r, f_C(r, R_Rc)); group g of a scan step owns [g*W, (g+1)*W)
     T rec[64][12];                            // phase-1 records: A_0..7, G_0..3
     SegDesc seg[64];                          // non-empty segments of the batch, in order
     unsigned long long segrow[64];            // where each of them puts its 32 output values
-    unsigned bits[kBitWords];                 // bit per triple slot: a segment starts here
-    int nA[kFB][4];                            // angular partners per type, per centre of the batch
+    unsigned bits[bit_words(kNB)];            // bit per triple slot: a segment starts here
+    int nA[kNB][4];                            // angular partners per type, per centre of the batch
     int nR[4][4];                             // radial partners per type, per group of the scan step
-    FwdJvpLds<T, kJvp> jvp;
+    FwdJvpLds<T, kJvp, kNB> jvp;
 };
 
 // Padding slots of phase 1 read entry 0 of centre 0's list whatever it holds; their products are cancelled by a
 // zero radial factor, which needs every other factor finite.  Entry 0 is either a partner written by a scan or
 // what this writes once per wavefront before the first batch.
-template <typename T, bool kJvp>
-__device__ __forceinline__ void fwd_lds_init(FwdWaveLds<T, kJvp>& S, int lane)
+template <typename T, bool kJvp, int kNB>
+__device__ __forceinline__ void fwd_lds_init(FwdWaveLds<T, kJvp, kNB>& S, int lane)
 {
     if (lane == 0) {
         S.nbr[0][0] = Fast<T>::make4(T(0), T(0), T(0), T(0));
@@ -48,15 +49,16 @@ __device__ __forceinline__ void fwd_lds_init(FwdWaveLds<T, kJvp>& S, int lane)
     }
 }
 
-// Segment table, phases 1 and 2 and the zero fill of empty blocks for centres 0..nb-1 of a batch.
+// Segment table, phases 1 and 2 and the zero fill of empty blocks for centres 0..nb-1 of a batch (nb <= kNB <= 6).
 // `row_of_centre(b)` returns the address of centre b's 384-float output row; it is called by all
 // lanes together, with a per-lane b.
 // With kJvp the same sums are formed for the derivative of every term along the atoms' incoming vectors:
 // d(A_t G_s P) = dA_t (G_s P) + A_t (dG_s P + G_s dP), two products per record instead of one.
-template <typename T, bool kJvp, typename RowOfCentre>
-__device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const LaneConsts<T>& L, int lane, int nb,
+template <typename T, bool kJvp, int kNB, typename RowOfCentre>
+__device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB>& S, const LaneConsts<T>& L, int lane, int nb,
                                                   RowOfCentre row_of_centre)
 {
+    static_assert(kNB * kNumPairBlocks <= 64, "one segment-table lane per (centre, type pair)");
     typedef typename Fast<T>::vec4 vec4;
     typedef typename Fast<T>::vec2 vec2;
     const unsigned long long lane_bit = 1ull << lane;
@@ -73,7 +75,7 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
     unsigned seg_row_lo = 0, seg_row_hi = 0;          // where the segment's 32 floats go
     {
         // row of the segment's centre (every lane takes part: the lookup may be a lane exchange)
-        const unsigned long long rowp = row_of_centre(min(seg_b, kFB - 1)) +
+        const unsigned long long rowp = row_of_centre(min(seg_b, kNB - 1)) +
                                         static_cast<unsigned long long>((kRadial + seg_pt * kAngBlock) * sizeof(T));
         seg_row_lo = static_cast<unsigned>(rowp);
         seg_row_hi = static_cast<unsigned>(rowp >> 32);
@@ -97,7 +99,7 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp>& S, const 
     const int start = incl - padded;
     const int total = lane_read(incl, 63);            // triple slots in this batch (even)
     const unsigned long long nonempty = wave_ballot(cnt > 0);
-    for (int w = lane; w < kBitWords; w += 64) S.bits[w] = 0u;
+    for (int w = lane; w < bit_words(kNB); w += 64) S.bits[w] = 0u;
     wave_lds_fence();
     if (cnt > 0) {
         mine.start_cnt = static_cast<unsigned>(start) | (static_cast<unsigned>(cnt) << 16);

@@ -233,12 +233,10 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                     if (ch * 64 < n) {
                         const int j = ch * 64 + lane;
                         if (!too_many && ((mA[ch] >> lane) & 1ull)) {
+                            // the entry as found; unit vector and cutoff are worked out once per centre below, on
+                            // the compacted list, not once per chunk on every lane
                             const int p = pos + popc64(mA[ch] & lt_mask);
-                            const T inv = Fast<T>::rcp(r[ch]);
-                            T fc, dfc;
-                            Fast<T>::cutoff_grad(r[ch], static_cast<T>(kA_Rc_f), fc, dfc);
-                            P.nbr[p] = Fast<T>::make4(dx[ch] * inv, dy[ch] * inv, dz[ch] * inv, r[ch]);
-                            P.nbr_fc[p] = Fast<T>::make2(fc, dfc);
+                            P.nbr[p] = Fast<T>::make4(dx[ch], dy[ch], dz[ch], r[ch]);
                             P.nbr_idx[p] = static_cast<unsigned char>(j);
                         }
                         pos += popc64(mA[ch]);
@@ -269,6 +267,17 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                             wave_lds_fence();
                             qn = rest;
                         }
+                    }
+                }
+                if (!too_many) {
+                    wave_lds_fence();
+                    if (lane < m_c) {
+                        const vec4 d = P.nbr[used + lane];
+                        const T inv = Fast<T>::rcp(d.w);
+                        T fc, dfc;
+                        Fast<T>::cutoff_grad(d.w, static_cast<T>(kA_Rc_f), fc, dfc);
+                        P.nbr[used + lane] = Fast<T>::make4(d.x * inv, d.y * inv, d.z * inv, d.w);
+                        P.nbr_fc[used + lane] = Fast<T>::make2(fc, dfc);
                     }
                 }
                 if (too_many) {

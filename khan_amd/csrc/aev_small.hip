@@ -264,7 +264,7 @@ void aev_fwd_small_kernel(
         }
 
         // ------------------------------------------------ segment table, phases 1 and 2, zero fill
-        fwd_angular_batch<T, kJvp>(S, L, lane, nb, [&](int b) -> unsigned long long {
+        fwd_angular_batch(S, L, lane, nb, [&](int b) -> unsigned long long {
             const int cl = min(c0 + b, 63);
             const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(cl << 2, rp_lo));
             const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(cl << 2, rp_hi));

@@ -7,10 +7,12 @@ namespace khan {
 // One wavefront per workgroup: molecules differ a lot in cost, and a workgroup's LDS is only released when
 // its slowest wavefront ends, so wider workgroups leave wave slots idle.
 constexpr int kWavesPerBlock = 1;
-constexpr int kFB = 6;         // centres per batch of the forward kernels
+constexpr int kFB = 6;         // centres per batch of the one-wavefront forward kernels
 constexpr int kB = 6;          // centres per batch: 6 x 10 type pairs = 60 segment lanes
 constexpr int kCapA = 32;      // angular neighbours kept per centre
-constexpr int kBitWords = 96;  // 6 centres x (496 triples + padding) fit in 96 x 32 slot bits
+// words of slot bits for a batch of n centres: at most 496 triples and 10 padding slots each, one bit per slot, and
+// one word beyond the last step's (96 for six centres)
+constexpr int bit_words(int n) { return (n * 506 + 31) / 32 + 1; }
 
 // One (centre, type pair) segment of a batch's triples, laid out so that a lane decodes its triple with few
 // instructions: fields sit on byte / half-word boundaries (the operand selects of the vector instructions read them
