@@ -41,6 +41,9 @@ WORKLOADS = {
     "inference65536": ("organic", 65536, 4, False),
     # not a line of the headline metric either: featurize_grad_inverse (the Jacobian applied to per-atom vectors)
     "grad_inverse65536": ("organic", 65536, 4, False),
+    # nor these: the charge kernels alone (energy, then dE/dq and dE/dxyz), float64
+    "charges_boxes4096_f64": ("boxes", 4096, 8, True),
+    "charges_organic16384_f64": ("organic", 16384, 8, True),
 }
 
 
@@ -218,6 +221,56 @@ def grad_inverse_bench(args, batch):
     }))
 
 
+def charges_bench(args, batch, w):
+    """ani_charge + ani_charge_grad_xyz (energy, dE/dq, dE/dxyz) on a resident batch: one JSON line.  Contract figures:
+    20 C flops for the energy, 45 C for energy + both gradients (C = unordered pairs), N 8w + M (w + 8) bytes."""
+    import torch
+    from khan_amd import datagen, ops
+    dev = torch.device("cuda:0")
+    tdt = torch.float32 if w == 4 else torch.float64
+    N, n_mols = batch.n_atoms, batch.n_mols
+    X, Y, Z = (torch.from_numpy(v).to(dev).to(tdt) for v in (batch.X, batch.Y, batch.Z))
+    Q = torch.from_numpy(datagen.charges(N)).to(dev).to(tdt)
+    macs, mos = ops.mol_offsets(torch.from_numpy(batch.mol_idxs).to(dev), n_mols)
+    ones = torch.ones(n_mols, dtype=tdt, device=dev)
+    C = batch.work_counts()["C"]
+    for _ in range(args.warmup):
+        ops.ani_charge(X, Y, Z, Q, mos, macs)
+        ops.ani_charge_grad_xyz(X, Y, Z, Q, mos, macs, ones)
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    t_e = t_g = 0.0
+    t0 = time.perf_counter()
+    marks = []
+    for _ in range(args.steps):
+        m = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        m[0].record()
+        e = ops.ani_charge(X, Y, Z, Q, mos, macs)
+        m[1].record()
+        g = ops.ani_charge_grad_xyz(X, Y, Z, Q, mos, macs, ones)
+        m[2].record()
+        marks.append(m)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    t_e = sum(m[0].elapsed_time(m[1]) for m in marks) / args.steps
+    t_g = sum(m[1].elapsed_time(m[2]) for m in marks) / args.steps
+    nbytes = N * 8 * w + n_mols * (w + 8)
+    peak = FP32_PEAK_TFLOPS if w == 4 else FP64_PEAK_TFLOPS
+    print(json.dumps({
+        "metric": "ani_charge energy + gradients atoms/sec, fp%d, 1 MI355X" % (8 * w),
+        "value": N / (ms_per_step * 1e-3), "unit": "atoms/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if w == 4 else "f64", "data": "synthetic",
+        "config": {"workload": "%s: ani_charge + ani_charge_grad_xyz, %d molecules, %d atoms, %d pairs" % (
+            args.workload, n_mols, N, C)},
+        "molecules_per_s": n_mols / (ms_per_step * 1e-3),
+        "roofline": {"kernel": "charge kernels", "bound": "hbm", "achieved": nbytes / ((t_e + t_g) * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / ((t_e + t_g) * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "energy_ms": t_e, "gradients_ms": t_g, "algorithmic_bytes": nbytes,
+                     "valu_frac": 45.0 * C / ((t_e + t_g) * 1e-3) / 1e12 / peak, "valu_peak_tflops": peak},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -248,6 +301,8 @@ def main():
         return inference_bench(args, batch)
     if args.workload.startswith("grad_inverse"):
         return grad_inverse_bench(args, batch)
+    if args.workload.startswith("charges_"):
+        return charges_bench(args, batch, w)
     N = batch.n_atoms
     counts = batch.work_counts()
     work = algorithmic_work(counts, N, n_mols, w)

@@ -11,8 +11,9 @@
 // One wavefront per molecule.  Up to 64 atoms a step evaluates 64 (i, j) pairs at once -- 4 atoms i x 16
 // partners j for molecules of up to 16 atoms, 2 x 32 up to 32, 1 x 64 above -- with the partners' data
 // held in the lanes, and the sums over j are in-wave DPP reductions (a lane per atom i walking all j
-// would leave four fifths of the lanes idle on a 12-atom molecule).  Above 64 atoms a lane takes the
-// atoms i = lane, lane + 64, ... and walks all partners j, whose loads are wave-uniform.  Each output
+// would leave four fifths of the lanes idle on a 12-atom molecule).  Molecules of 65 to 256 atoms go to a
+// second kernel that tiles the molecule through LDS (charge_tile_kernel below).  Above 256 atoms a lane takes
+// the atoms i = lane, lane + 64, ... and walks all partners j, whose loads are wave-uniform.  Each output
 // element is written once: no atomics and no pre-zeroing.
 #include "aev_small_common.h"
 
@@ -46,6 +47,7 @@ __global__ __launch_bounds__(256) void charge_energy_kernel(
     const int64_t mol = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
     if (mol >= n_mols) return;
     const int n = MACs[mol], off = MOs[mol];
+    if (n > kSmallMaxAtoms && n <= kMediumMaxAtoms) return;      // the tile kernel's
     const T rc = static_cast<T>(kR_Rc_f), pi_rc = static_cast<T>(kPi / static_cast<double>(kR_Rc_f));
     T acc = T(0);
     if (n <= 64) {
@@ -96,6 +98,7 @@ __global__ __launch_bounds__(256) void charge_grad_kernel(
     const int64_t mol = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
     if (mol >= n_mols) return;
     const int n = MACs[mol], off = MOs[mol];
+    if (n > kSmallMaxAtoms && n <= kMediumMaxAtoms) return;      // the tile kernel's
     const T rc = static_cast<T>(kR_Rc_f), pi_rc = static_cast<T>(kPi / static_cast<double>(kR_Rc_f));
     const T gK = grads[mol] * K;
     if (n <= 64) {
@@ -154,6 +157,111 @@ __global__ __launch_bounds__(256) void charge_grad_kernel(
     }
 }
 
+
+// Molecules of 65 to 256 atoms: one wavefront per molecule, the molecule (x, y, z, q) tiled through LDS.
+// A lane owns the atoms i = lane, lane + 64, ... (at most four).  In round d it pairs each of them with atom
+// j = (i + d) mod n, read from the tile: after (n-1)/2 rounds (plus half a round when n is even) every
+// unordered pair has been evaluated exactly once -- half the pair evaluations of a walk over all j != i, with all
+// lanes busy.  In a round the partners j of all atoms are distinct, so what a pair contributes to its partner
+// (dE/dq_j and the force on j) is added to the partner's slot in LDS by plain read-add-write, without atomics,
+// while the atom's own side stays in registers.  Every output element is written once.
+template <typename T, bool kGrad> struct ChargeTile;
+template <typename T> struct __align__(16) ChargeTile<T, false> {
+    typename Fast<T>::vec4 in[kMediumMaxAtoms];     // x, y, z, q
+};
+template <typename T> struct __align__(16) ChargeTile<T, true> {
+    typename Fast<T>::vec4 in[kMediumMaxAtoms];     // x, y, z, q
+    typename Fast<T>::vec4 acc[kMediumMaxAtoms];    // partner side: force x, y, z and dE/dq
+};
+
+template <typename T, bool kDamped, bool kGrad>
+__global__ __launch_bounds__(64) void charge_tile_kernel(
+    const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
+    const T* __restrict__ Q, const int32_t* __restrict__ MOs, const int32_t* __restrict__ MACs,
+    int32_t n_mols, const T* __restrict__ grads, T K, T* __restrict__ E, T* __restrict__ q_grads,
+    T* __restrict__ gX, T* __restrict__ gY, T* __restrict__ gZ)
+{
+    typedef typename Fast<T>::vec4 vec4;
+    constexpr int kOwn = kMediumMaxAtoms / 64;      // atoms per lane
+    __shared__ ChargeTile<T, kGrad> S;
+    const int lane = threadIdx.x;
+    const T rc = static_cast<T>(kR_Rc_f), pi_rc = static_cast<T>(kPi / static_cast<double>(kR_Rc_f));
+    for (int mol = blockIdx.x; mol < n_mols; mol += gridDim.x) {
+        const int n = uniform(MACs[mol]);
+        if (n <= kSmallMaxAtoms || n > kMediumMaxAtoms) continue;
+        const int off = uniform(MOs[mol]);
+        vec4 own[kOwn];
+        T fx[kOwn], fy[kOwn], fz[kOwn], dq[kOwn];
+#pragma unroll
+        for (int k = 0; k < kOwn; ++k) {
+            const int i = lane + 64 * k;
+            own[k] = Fast<T>::make4(T(0), T(0), T(0), T(0));
+            fx[k] = fy[k] = fz[k] = dq[k] = T(0);
+            if (i < n) {
+                own[k] = Fast<T>::make4(X[off + i], Y[off + i], Z[off + i], Q[off + i]);
+                S.in[i] = own[k];
+                if constexpr (kGrad) S.acc[i] = Fast<T>::make4(T(0), T(0), T(0), T(0));
+            }
+        }
+        wave_lds_fence();
+        const int half = (n - 1) >> 1;
+        const int rounds = half + (((n & 1) == 0) ? 1 : 0);
+        T e_acc = T(0);
+        for (int d = 1; d <= rounds; ++d) {
+#pragma unroll
+            for (int k = 0; k < kOwn; ++k) {
+                const int i = lane + 64 * k;
+                const bool act = (i < n) && (d <= half || i < (n >> 1));     // the half round: the lower half only
+                int j = i + d;
+                j -= (j >= n) ? n : 0;
+                const vec4 aj = S.in[act ? j : 0];
+                const T dx = act ? own[k].x - aj.x : T(1), dy = act ? own[k].y - aj.y : T(0), dz = act ? own[k].z - aj.z : T(0);
+                T u, du;
+                pair_terms<T, kDamped>(dx, dy, dz, pi_rc, rc, u, du);
+                if constexpr (!kGrad) {
+                    e_acc += act ? own[k].w * aj.w * u : T(0);
+                } else {
+                    if (act) {
+                        dq[k] = fma(aj.w, u, dq[k]);
+                        const T wq = own[k].w * aj.w * du;       // q_i q_j d/dr[(1-f_C)/r] / r
+                        fx[k] = fma(wq, dx, fx[k]);
+                        fy[k] = fma(wq, dy, fy[k]);
+                        fz[k] = fma(wq, dz, fz[k]);
+                        vec4 pa = S.acc[j];                      // distinct j across the lanes of this step
+                        pa.x = fma(-wq, dx, pa.x);
+                        pa.y = fma(-wq, dy, pa.y);
+                        pa.z = fma(-wq, dz, pa.z);
+                        pa.w = fma(own[k].w, u, pa.w);
+                        S.acc[j] = pa;
+                    }
+                    wave_lds_fence();                            // the next step may touch slots written here
+                }
+            }
+        }
+        if constexpr (!kGrad) {
+            e_acc = wave_sum(e_acc);
+            if (lane == 0) E[mol] = K * e_acc;
+        } else {
+            const T gK = grads[mol] * K;
+#pragma unroll
+            for (int k = 0; k < kOwn; ++k) {
+                const int i = lane + 64 * k;
+                if (i < n) {
+                    const vec4 pa = S.acc[i];
+                    if (q_grads) q_grads[off + i] = gK * (dq[k] + pa.w);
+                    if (gX) {
+                        // the force sums carry q_i already (wq = q_i q_j ...)
+                        gX[off + i] = gK * (fx[k] + pa.x);
+                        gY[off + i] = gK * (fy[k] + pa.y);
+                        gZ[off + i] = gK * (fz[k] + pa.z);
+                    }
+                }
+            }
+        }
+        wave_lds_fence();        // the next molecule reuses the tile
+    }
+}
+
 }  // namespace
 
 template <typename T>
@@ -162,8 +270,17 @@ hipError_t launch_charge_energy(const T* X, const T* Y, const T* Z, const T* Q, 
 {
     if (n_mols <= 0) return hipSuccess;
     const unsigned blocks = (static_cast<unsigned>(n_mols) + 3u) / 4u;
-    if (damped) charge_energy_kernel<T, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, K, E);
-    else charge_energy_kernel<T, false><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, K, E);
+    // molecules of 65..256 atoms are the tile kernel's, everything else the first kernel's (each leaves the other's alone)
+    const unsigned tile_blocks = static_cast<unsigned>(n_mols < 8192 ? n_mols : 8192);
+    if (damped) {
+        charge_energy_kernel<T, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, K, E);
+        charge_tile_kernel<T, true, false><<<dim3(tile_blocks), dim3(64), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, nullptr, K, E,
+                                                                                   nullptr, nullptr, nullptr, nullptr);
+    } else {
+        charge_energy_kernel<T, false><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, K, E);
+        charge_tile_kernel<T, false, false><<<dim3(tile_blocks), dim3(64), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, nullptr, K, E,
+                                                                                    nullptr, nullptr, nullptr, nullptr);
+    }
     return hipGetLastError();
 }
 
@@ -174,8 +291,16 @@ hipError_t launch_charge_grad(const T* X, const T* Y, const T* Z, const T* Q, co
 {
     if (n_mols <= 0) return hipSuccess;
     const unsigned blocks = (static_cast<unsigned>(n_mols) + 3u) / 4u;
-    if (damped) charge_grad_kernel<T, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, q_grads, gX, gY, gZ);
-    else charge_grad_kernel<T, false><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, q_grads, gX, gY, gZ);
+    const unsigned tile_blocks = static_cast<unsigned>(n_mols < 8192 ? n_mols : 8192);
+    if (damped) {
+        charge_grad_kernel<T, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, q_grads, gX, gY, gZ);
+        charge_tile_kernel<T, true, true><<<dim3(tile_blocks), dim3(64), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, nullptr,
+                                                                                  q_grads, gX, gY, gZ);
+    } else {
+        charge_grad_kernel<T, false><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, q_grads, gX, gY, gZ);
+        charge_tile_kernel<T, false, true><<<dim3(tile_blocks), dim3(64), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, nullptr,
+                                                                                   q_grads, gX, gY, gZ);
+    }
     return hipGetLastError();
 }
 
