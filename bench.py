@@ -155,15 +155,20 @@ def inference_bench(args, batch):
     b.n_mols = n_mols
     b.mol_atom_counts, b.mol_offsets = ops.mol_offsets(b.mol_idxs, n_mols)
     b.scatter_idxs, b.gather_idxs, b.atom_counts = ops.ani_sort(b.atom_types)
-    m = model.AniModel(model.DEFAULT_LAYERS, model.celu, torch.float32, dev, seed=1)
-    for _ in range(args.warmup):
-        m.batch_energies(b, need_grad=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        e, g = m.batch_energies(b, need_grad=True)
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    def timed(first_layer_kernel):
+        m = model.AniModel(model.DEFAULT_LAYERS, model.celu, torch.float32, dev, seed=1, first_layer_kernel=first_layer_kernel)
+        for _ in range(args.warmup):
+            m.batch_energies(b, need_grad=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            e, g = m.batch_energies(b, need_grad=True)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps * 1e3, e, g
+
+    ms_library, e_lib, g_lib = timed(False)      # every dense layer a library (rocBLAS) product
+    ms_per_step, e_k, g_k = timed(True)          # first layer in this package's matrix-core kernel
+    agree = float((e_k - e_lib).abs().max() / e_lib.abs().max())
     sizes = (384,) + tuple(model.DEFAULT_LAYERS)
     macs_per_atom = sum(x * y for x, y in zip(sizes[:-1], sizes[1:]))
     gemm_flops = 2 * macs_per_atom * N * 2            # forward, and the data gradient on the way back
@@ -175,7 +180,9 @@ def inference_bench(args, batch):
         "config": {"workload": "inference65536: featurize + 4 atomic networks 384-128-128-64-1 (random weights) + "
                                "segment sum, gradient back to the coordinates; %d molecules, %d atoms" % (n_mols, N)},
         "molecules_per_s": n_mols / (ms_per_step * 1e-3),
-        "roofline": {"kernel": "dense layers (rocBLAS)", "bound": "mfma", "achieved": gemm_flops / (ms_per_step * 1e-3) / 1e12,
+        "first_layer": {"kernel_ms_per_step": ms_per_step, "library_ms_per_step": ms_library,
+                        "max_relative_energy_difference": agree},
+        "roofline": {"kernel": "dense layers (first: khan_dense_first_f32, others: rocBLAS)", "bound": "mfma", "achieved": gemm_flops / (ms_per_step * 1e-3) / 1e12,
                      "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": gemm_flops / (ms_per_step * 1e-3) / 1e12 / FP32_PEAK_TFLOPS, "traffic": None},
     }))

@@ -226,6 +226,20 @@ int khan_ani_charge_grad_xyz_f64(const double *xs, const double *ys, const doubl
                                  double *x_grads, double *y_grads, double *z_grads,
                                  khan_stream_t stream);
 
+/* First dense layer of the per-type atomic networks, right behind the featurizer (khan/model/nn.py:38-68: matmul +
+ * bias + activation per atom type; activation CELU, khan/model/activations.py:63-65, or none):
+ *     out_t[r, :] = act(rows_t[r, :] . W_t + b_t),  t = H, C, N, O,  one launch for the four types.
+ * Every *_host4 argument is a HOST array of four DEVICE pointers: rows_t [acs[t], 384] (the featurizer's buckets,
+ * 16-byte aligned), wt_t [128, 384] = the layer's [384, 128] weights TRANSPOSED (16-byte aligned), bias_t [128],
+ * out_t [acs[t], 128].  float32 in, float32 accumulation on the matrix cores.  The layer width is fixed at 128
+ * (the reference's default network, energy_server.py:121); other widths are the caller's matrix library's. */
+#define KHAN_ACT_NONE 0
+#define KHAN_ACT_CELU 1
+int khan_dense_first_f32(const float *const *rows_host4, const int32_t *acs_host,
+                         const float *const *wt_host4, const float *const *bias_host4,
+                         int32_t activation, float alpha, float *const *out_host4,
+                         khan_stream_t stream);
+
 /* Plain Coulomb sums, E_m = k sum_{i<j in m} q_i q_j / r_ij, and their gradients: the charge kernels with
  * the damping (1 - f_C) switched off and the constant chosen by the caller (k = 1 for charges in e and
  * distances in the unit the energy is wanted in).  No reference counterpart: khan's own op is the damped,

@@ -73,6 +73,49 @@ class _AniCharge(torch.autograd.Function):
         return None, None, None, ops.ani_charge_grad(*args), None, None
 
 
+class _DenseFirst(torch.autograd.Function):
+    """act(rows_t . W_t + b_t) for the four atom types through `ops.dense_first` (float32, width 128, CELU or no
+    activation).  Backward: plain matrix products; the activation's derivative comes from the saved outputs
+    (CELU: 1 for out >= 0, out / alpha + 1 = exp(z / alpha) below)."""
+
+    @staticmethod
+    def forward(ctx, acs_host, activation, alpha, *tensors):
+        feats, ws, bs = tensors[0:4], tensors[4:8], tensors[8:12]
+        outs = ops.dense_first([f.detach() for f in feats], acs_host, [w.detach().t().contiguous() for w in ws],
+                               [b.detach() for b in bs], activation, alpha)
+        ctx.save_for_backward(*feats, *ws, *outs)
+        ctx.activation, ctx.alpha = activation, alpha
+        return outs
+
+    @staticmethod
+    def backward(ctx, *gouts):
+        saved = ctx.saved_tensors
+        feats, ws, outs = saved[0:4], saved[4:8], saved[8:12]
+        gf, gw, gb = [], [], []
+        for t in range(4):
+            g = gouts[t]
+            if g is None or outs[t].numel() == 0:
+                gf.append(torch.zeros_like(feats[t]) if ctx.needs_input_grad[3 + t] else None)
+                gw.append(torch.zeros_like(ws[t]) if ctx.needs_input_grad[7 + t] else None)
+                gb.append(torch.zeros(ws[t].shape[1], dtype=ws[t].dtype, device=ws[t].device) if ctx.needs_input_grad[11 + t] else None)
+                continue
+            if ctx.activation == ops.ACT_CELU:
+                # one elementwise kernel: CELU is ELU with input scale 1 / alpha, differentiated from its result
+                g = torch.ops.aten.elu_backward(g.contiguous(), ctx.alpha, 1.0, 1.0 / ctx.alpha, True, outs[t])
+            rows = feats[t].reshape(-1, ops.FEATURE_SIZE)
+            gf.append((g @ ws[t].t()).reshape(feats[t].shape) if ctx.needs_input_grad[3 + t] else None)
+            gw.append(rows.t() @ g if ctx.needs_input_grad[7 + t] else None)
+            gb.append(g.sum(dim=0) if ctx.needs_input_grad[11 + t] else None)
+        return (None, None, None) + tuple(gf) + tuple(gw) + tuple(gb)
+
+
+def dense_first(atom_type_features, acs_host, weights, biases, activation=ops.ACT_CELU, alpha=0.1):
+    """Differentiable first dense layer of the four atomic networks: four flat feature buckets, four [384, 128]
+    weights, four [128] biases -> four [n_t, 128] activations (float32)."""
+    return _DenseFirst.apply([int(v) for v in acs_host], int(activation), float(alpha),
+                             *atom_type_features, *weights, *biases)
+
+
 def featurize(xs, ys, zs, as_, mos, macs, sis, acs):
     """Differentiable `featurize`: -> (h_feat, c_feat, n_feat, o_feat); gradients flow to xs, ys, zs."""
     return _Featurize.apply(xs, ys, zs, as_, mos, macs, sis, acs)

@@ -506,6 +506,28 @@ int khan_ani_charge_grad_xyz_f64(const double* xs, const double* ys, const doubl
     return charge_grad_impl<double>(xs, ys, zs, qs, mos, macs, n_mols, grads, true, static_cast<double>(khan::kChargeK_f), q_grads, gx, gy, gz, true, stream);
 }
 
+int khan_dense_first_f32(const float* const* rows_host4, const int32_t* acs_host, const float* const* wt_host4,
+                         const float* const* bias_host4, int32_t activation, float alpha, float* const* out_host4,
+                         khan_stream_t stream)
+{
+    if (!rows_host4 || !acs_host || !wt_host4 || !bias_host4 || !out_host4) return KHAN_ERR_INVALID_ARG;
+    if (activation != KHAN_ACT_NONE && activation != KHAN_ACT_CELU) return KHAN_ERR_INVALID_ARG;
+    if (activation == KHAN_ACT_CELU && !(alpha > 0.0f)) return KHAN_ERR_INVALID_ARG;
+    int64_t total = 0;
+    for (int t = 0; t < 4; ++t) {
+        if (acs_host[t] < 0) return KHAN_ERR_INVALID_ARG;
+        if (acs_host[t] > 0 && (!rows_host4[t] || !wt_host4[t] || !bias_host4[t] || !out_host4[t])) return KHAN_ERR_INVALID_ARG;
+        // 16-byte loads of rows and weights
+        if (acs_host[t] > 0 && ((reinterpret_cast<uintptr_t>(rows_host4[t]) | reinterpret_cast<uintptr_t>(wt_host4[t])) & 15u))
+            return KHAN_ERR_INVALID_ARG;
+        total += acs_host[t];
+    }
+    if (total == 0) return KHAN_OK;
+    if (total > INT32_MAX) return KHAN_ERR_TOO_LARGE;
+    return hip_status(khan::launch_dense_first(rows_host4, acs_host, wt_host4, bias_host4, activation == KHAN_ACT_CELU, alpha,
+                                               out_host4, as_stream(stream)));
+}
+
 // Plain Coulomb sums: the charge kernels with the cutoff function switched off and the constant given by the caller.
 int khan_coulomb_f32(const float* xs, const float* ys, const float* zs, const float* qs, const int32_t* mos,
                      const int32_t* macs, int32_t n_mols, float k, float* e, khan_stream_t stream)

@@ -95,6 +95,12 @@ hipError_t launch_size_order(const int32_t* MACs, int32_t n_mols, int32_t* order
 template <typename T>
 hipError_t launch_zero(T* a, int64_t n, hipStream_t stream);
 
+// ---- first dense layer behind the featurizer: out_t = act(rows_t . W_t + b_t) for the four types, float32 ----
+// rows[t]: [n[t], 384]; wt[t]: [128, 384] (the weights transposed); bias[t]: [128]; out[t]: [n[t], 128]
+hipError_t launch_dense_first(const float* const rows[4], const int32_t n[4], const float* const wt[4],
+                              const float* const bias[4], bool celu, float alpha, float* const out[4],
+                              hipStream_t stream);
+
 // ---- charges: pair energy K q_i q_j (1 - f_C(r)) / r; damped = false drops f_C (plain Coulomb) ----
 template <typename T>
 hipError_t launch_charge_energy(const T* X, const T* Y, const T* Z, const T* Q, const int32_t* MOs,

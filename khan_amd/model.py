@@ -6,7 +6,8 @@ save_numpy / load_numpy (451-499), predict (655-678), coordinate_gradients (580-
 features -> per-type networks -> gather -> segment_sum (+ ani_charge) of lines 306-385.
 
 The featurizer, its gradient and the charge energy are the HIP kernels of this package (through
-`khan_amd.autograd`).  The dense layers are plain matrix products: PyTorch's (rocBLAS) here.  Parameter
+`khan_amd.autograd`).  The first dense layer (float32, width 128, CELU) runs in this package's matrix-core kernel
+right behind the featurizer (`ops.dense_first`); the other layers are plain matrix products: PyTorch's (rocBLAS).  Parameter
 names are the reference's TensorFlow variable names, `<prefix>W_<type>_<in>x<out>_l<k>:0` and
 `<prefix>b_...` (nn.py:41-60), so a checkpoint written by the reference's `save_numpy` loads unchanged;
 whatever else such a file holds (optimizer slots, learning rate, moving averages) is ignored.
@@ -71,7 +72,9 @@ class MoleculeNN:
     """Four atomic networks (H, C, N, O) mapping feature rows to one number per atom."""
 
     def __init__(self, layer_sizes=DEFAULT_LAYERS, activation_fn=celu, dtype=torch.float32, device="cpu",
-                 prefix="near_", seed=None):
+                 prefix="near_", seed=None, first_layer_kernel=True):
+        self.first_layer_kernel = bool(first_layer_kernel)
+        self.weights_need_grad = False      # set it to differentiate through the first layer's weights (training)
         layer_sizes = tuple(int(v) for v in layer_sizes)
         if layer_sizes[-1] != 1:
             raise ValueError("the last layer must have size 1")
@@ -91,19 +94,39 @@ class MoleculeNN:
     def parameters(self):
         return [self.params[k] for k in self.params]
 
-    def atom_type_outputs(self, type_idx, feats):
-        """[n_t, 384] feature rows of one type -> [n_t] network outputs."""
+    def atom_type_outputs(self, type_idx, feats, first_layer_done=False):
+        """[n_t, 384] feature rows of one type -> [n_t] network outputs (`first_layer_done`: `feats` are the first
+        layer's activations already)."""
         rows = self.names[TYPE_MAP[type_idx]]
         a = feats
         for k, (wn, bn, _, _) in enumerate(rows):
+            if first_layer_done and k == 0:
+                continue
             a = torch.addmm(self.params[bn], a, self.params[wn])
             if k != len(rows) - 1:
                 a = self.activation_fn(a)
         return a.reshape(-1)
 
+    def fused_first_layer(self):
+        """True when the first layer can run in this package's matrix-core kernel (`ops.dense_first`): float32 on the
+        GPU, width 128, CELU with its default alpha, at least two layers."""
+        return (self.first_layer_kernel and self.dtype == torch.float32 and self.device.type == "cuda"
+                and self.layer_sizes[1] == 128 and len(self.layer_sizes) > 2 and self.activation_fn is celu)
+
     def atom_outputs(self, atom_type_features, gather_idxs):
         """Per-type flat feature buckets -> one number per atom in the batch's atom order (nn.py:176-177)."""
-        outs = [self.atom_type_outputs(t, f.reshape(-1, FEATURE_SIZE)) for t, f in enumerate(atom_type_features)]
+        if self.fused_first_layer():
+            from . import autograd
+            acs = [f.numel() // FEATURE_SIZE for f in atom_type_features]
+            first = [self.names[t][0] for t in TYPE_MAP]
+            # inference: the weights are constants here (a custom autograd function cannot tell that only the
+            # coordinates' gradient was asked for, and would form the weights' gradient, a second product, every time)
+            par = (lambda k: self.params[k]) if self.weights_need_grad else (lambda k: self.params[k].detach())
+            a1 = autograd.dense_first(atom_type_features, acs, [par(r[0]) for r in first],
+                                      [par(r[1]) for r in first], alpha=0.1)
+            outs = [self.atom_type_outputs(t, a1[t], first_layer_done=True) for t in range(4)]
+        else:
+            outs = [self.atom_type_outputs(t, f.reshape(-1, FEATURE_SIZE)) for t, f in enumerate(atom_type_features)]
         return torch.cat(outs)[gather_idxs.long()]
 
 
@@ -111,13 +134,13 @@ class AniModel:
     """Near-field network, optional charge network with the pairwise charge energy, and their checkpoint."""
 
     def __init__(self, layer_sizes=DEFAULT_LAYERS, activation_fn=celu, dtype=torch.float32, device="cuda:0",
-                 fit_charges=False, seed=None):
+                 fit_charges=False, seed=None, first_layer_kernel=True):
         self.dtype, self.device = dtype, torch.device(device)
-        self.near = MoleculeNN(layer_sizes, activation_fn, dtype, device, "near_", seed)
+        self.near = MoleculeNN(layer_sizes, activation_fn, dtype, device, "near_", seed, first_layer_kernel)
         self.charge = None
         if fit_charges:
             self.charge = MoleculeNN(layer_sizes, activation_fn, dtype, device, "charge_",
-                                     None if seed is None else seed + 1)
+                                     None if seed is None else seed + 1, first_layer_kernel)
 
     # -------------------------------------------------------------------------------------- checkpoint
     def named_parameters(self):

@@ -287,3 +287,29 @@ def coulomb_grad(xs, ys, zs, qs, mos, macs, grads, k=1.0):
     _lib.check(fn(_p(xs), _p(ys), _p(zs), _p(qs), _p(mos), _p(macs), mos.numel(), _p(grads), float(k), _p(qg),
                   _p(gx), _p(gy), _p(gz), _stream()))
     return qg, gx, gy, gz
+
+
+ACT_NONE, ACT_CELU = 0, 1
+
+
+def dense_first(atom_type_features, acs, weights_t, biases, activation=ACT_CELU, alpha=0.1):
+    """First dense layer of the four atomic networks on the featurizer's buckets, float32, one launch:
+    -> four [acs[t], 128] tensors act(rows_t . W_t + b_t).  `weights_t[t]` is W_t TRANSPOSED, [128, 384]."""
+    lib = _lib.load()
+    acs_c, acs_v = _acs_host(acs)
+    rows, wts, bs, outs = [], [], [], []
+    for t in range(4):
+        r = _dev(atom_type_features[t].reshape(-1), torch.float32, "features")
+        if r.numel() != acs_v[t] * FEATURE_SIZE:
+            raise ValueError("bucket %d has %d elements, expected %d" % (t, r.numel(), acs_v[t] * FEATURE_SIZE))
+        w = weights_t[t]
+        if tuple(w.shape) != (128, FEATURE_SIZE) or w.dtype != torch.float32 or not w.is_contiguous() or not w.is_cuda:
+            raise ValueError("weights_t[%d] must be a contiguous float32 CUDA tensor of shape [128, 384]" % t)
+        b = _dev(biases[t], torch.float32, "bias")
+        if b.numel() != 128:
+            raise ValueError("bias %d must have 128 elements" % t)
+        rows.append(r); wts.append(w); bs.append(b)
+        outs.append(torch.empty((acs_v[t], 128), dtype=torch.float32, device=r.device))
+    arr = lambda ts: (ctypes.c_void_p * 4)(*[t.data_ptr() if t.numel() else None for t in ts])
+    _lib.check(lib.khan_dense_first_f32(arr(rows), acs_c, arr(wts), arr(bs), int(activation), float(alpha), arr(outs), _stream()))
+    return tuple(outs)

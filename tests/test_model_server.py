@@ -275,6 +275,46 @@ def test_gradient_is_the_derivative_of_the_energy():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("activation", ["celu", "none"])
+def test_first_dense_layer_kernel_matches_the_oracle(activation):
+    """khan_dense_first_f32 (the first layer of the four atomic networks on the featurizer's buckets, matrix cores,
+    one launch) against oracle/nn_ref.py's layer 1 in float64 (khan/model/nn.py:38-68), on real feature rows:
+    row counts on and off the 128-row tile size, an empty type, and the float32 library product beside it."""
+    from khan_amd import ops
+    b, _ = _molecules(n_mols=300, first=3)
+    dev = "cuda:0"
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    A = b.A.copy()
+    A[A == 2] = 1                                   # no nitrogen: an empty bucket
+    macs, mos = ops.mol_offsets(d(b.mol_idxs), b.n_mols)
+    sc, ga, ac = ops.ani_sort(d(A))
+    acs = ac.cpu()
+    feats = ops.featurize(d(b.X), d(b.Y), d(b.Z), d(A), mos, macs, sc, acs)
+    assert acs.tolist()[2] == 0 and min(acs.tolist()[:2]) > 128
+    rng = np.random.default_rng(4)
+    Ws = [rng.standard_normal((384, 128)) * (2.0 / 512) ** 0.5 for _ in range(4)]
+    bs = [rng.standard_normal(128) * 0.1 for _ in range(4)]
+    wt = [d(W.T.astype(np.float32)) for W in Ws]
+    bt = [d(v.astype(np.float32)) for v in bs]
+    act = ops.ACT_CELU if activation == "celu" else ops.ACT_NONE
+    outs = ops.dense_first(feats, acs, wt, bt, activation=act, alpha=0.1)
+    for t in range(4):
+        rows = feats[t].reshape(-1, 384).cpu().numpy().astype(np.float64)
+        z = rows @ Ws[t].astype(np.float32).astype(np.float64) + bs[t].astype(np.float32).astype(np.float64)
+        want = nn_ref._celu(z) if activation == "celu" else z
+        got = outs[t].cpu().numpy().astype(np.float64)
+        assert got.shape == want.shape
+        if want.size == 0:
+            continue
+        # float32 products summed over 384 terms: the bound scales with the sum of the terms' magnitudes
+        mag = np.abs(rows) @ np.abs(Ws[t]) + np.abs(bs[t])
+        assert np.all(np.abs(got - want) <= 1e-6 * mag + 1e-7), (t, np.abs(got - want).max())
+        lib = torch.addmm(bt[t], feats[t].reshape(-1, 384), wt[t].t())
+        lib = torch.nn.functional.celu(lib, 0.1) if activation == "celu" else lib
+        assert np.all(np.abs(lib.cpu().numpy() - want) <= 1e-6 * mag + 1e-7)
+
+
+@pytest.mark.gpu
 def test_energy_server_round_trip_over_a_socket():
     b, mols = _molecules(n_mols=2, first=11)
     m = _gpu_model(torch.float64, seed=5)
