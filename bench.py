@@ -288,7 +288,12 @@ def main():
     ap.add_argument("--traffic-probe", choices=("fwd", "bwd"), default=None,
                     help="counter-collection mode: launch that pass twice, then a plain 64 MiB device copy of "
                          "known traffic (scales FETCH_SIZE / WRITE_SIZE), print nothing else and exit")
+    ap.add_argument("--phase2", choices=("vector", "matrix"), default="vector",
+                    help="matrix: measure the variant of the small-molecule forward kernel that sums the angular "
+                         "records on the matrix cores (sets KHAN_AEV_PHASE2 before the library's first launch)")
     args = ap.parse_args()
+    if args.phase2 == "matrix":
+        os.environ["KHAN_AEV_PHASE2"] = "matrix"
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; the path shards by molecule with no exchange, "
                  "but no multi-GPU launch is part of this run (got --gpus %d)" % args.gpus)
@@ -478,6 +483,8 @@ def main():
         "molecules_per_s": n_mols / (ms_per_step * 1e-3),
         "roofline": roofline,
     }
+    if args.phase2 != "vector":
+        result["config"]["forward_phase2"] = args.phase2 + " cores (measurement variant, not the default kernel)"
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(batch, min(n_mols, 8192) if kind == "organic" else 32, min(n_mols, 4096) if kind == "organic" else 8, w)
     print(json.dumps(result))

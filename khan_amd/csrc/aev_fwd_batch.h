@@ -54,11 +54,17 @@ __device__ __forceinline__ void fwd_lds_init(FwdWaveLds<T, kJvp, kNB>& S, int la
 // lanes together, with a per-lane b.
 // With kJvp the same sums are formed for the derivative of every term along the atoms' incoming vectors:
 // d(A_t G_s P) = dA_t (G_s P) + A_t (dG_s P + G_s dP), two products per record instead of one.
-template <typename T, bool kJvp, int kNB, typename RowOfCentre>
+//
+// kMatrixPhase2 (float, forward only) sums the records on the matrix cores instead of the vector ALU: the sum over a
+// segment's records of A_t G_s is the product of an 8 x K by a K x 4 matrix, and v_mfma_f32_16x16x4_f32 takes four
+// records (K = 4) per instruction, using an 8 x 4 corner of its 16 x 16 result.  The variant exists to be measured
+// against the vector form; the launcher selects it on request only.
+template <bool kMatrixPhase2, typename T, bool kJvp, int kNB, typename RowOfCentre>
 __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB>& S, const LaneConsts<T>& L, int lane, int nb,
                                                   RowOfCentre row_of_centre)
 {
     static_assert(kNB * kNumPairBlocks <= 64, "one segment-table lane per (centre, type pair)");
+    static_assert(!kMatrixPhase2 || (sizeof(T) == 4 && !kJvp), "the matrix-core phase 2 is float, forward only");
     typedef typename Fast<T>::vec4 vec4;
     typedef typename Fast<T>::vec2 vec2;
     const unsigned long long lane_bit = 1ull << lane;
@@ -119,6 +125,17 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB>& S, c
         const T tot = half_wave_sum(acc);
         T* dst = reinterpret_cast<T*>((static_cast<unsigned long long>(cur_hi) << 32) | cur_lo);
         if (lane < 32) store_global(dst + lane, tot);
+    };
+    // matrix-core form: result element (theta_t, Rs_s) of the open segment is register t % 4 of lane 16 (t / 4) + s
+    typedef float mfma_acc __attribute__((ext_vector_type(4)));
+    mfma_acc macc = {0.f, 0.f, 0.f, 0.f};
+    auto flush_matrix = [&]() {
+        T* dst = reinterpret_cast<T*>((static_cast<unsigned long long>(cur_hi) << 32) | cur_lo);
+        if (lane < 32 && (lane & 15) < 4) {
+            T* p = dst + (lane >> 4) * 16 + (lane & 15);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) store_global(p + 4 * v, static_cast<T>(macc[v]));
+        }
     };
 
     for (int base = 0; base < total; base += 64) {
@@ -220,6 +237,63 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB>& S, c
         }
         wave_lds_fence();
 
+        if constexpr (kMatrixPhase2) {
+            // phase 2 on the matrix cores, four records per instruction.  Operand A (16 x 4): lane 16 k + i supplies
+            // row i of record k, operand B (4 x 16): lane 16 k + j column j of record k.  Rows 0-7 are A_0..7 and
+            // columns 0-3 are G_0..3; the other rows and columns take whatever follows in the record buffer, which
+            // only reaches result elements outside the 8 x 4 corner.  Segments start at even records: a start in
+            // the middle of a group splits it into two instructions, each with the other half's rows zeroed.
+            const int nrec = min(64, total - base);
+            const int ngroups = (nrec + 3) >> 2;           // records past `total` are zeros
+            const float* pm = &S.rec[0][0] + (lane >> 4) * 12 + (lane & 15);
+            unsigned long long mm = starts;
+            if (base == 0) {
+                cur_lo = static_cast<unsigned>(lane_read(static_cast<int>(d_row_lo), 0));
+                cur_hi = static_cast<unsigned>(lane_read(static_cast<int>(d_row_hi), 0));
+                mm &= ~1ull;
+            }
+            auto open_at = [&](int first) {
+                asm volatile("" : "+s"(first));
+                cur_lo = static_cast<unsigned>(lane_read(static_cast<int>(d_row_lo), first));
+                cur_hi = static_cast<unsigned>(lane_read(static_cast<int>(d_row_hi), first));
+                macc = mfma_acc{0.f, 0.f, 0.f, 0.f};
+            };
+            for (int g0 = 0; g0 < ngroups; g0 += 4) {
+                float av[4], bv[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    av[u] = pm[(g0 + u) * 48];
+                    bv[u] = pm[(g0 + u) * 48 + 8];
+                }
+                const unsigned m16 = static_cast<unsigned>(mm) & 0xffffu;
+                mm >>= 16;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (g0 + u < ngroups) {
+                        const unsigned m4 = (m16 >> (4 * u)) & 5u;
+                        if (__builtin_expect(m4 != 0u, 0)) {
+                            if (m4 & 1u) {
+                                flush_matrix();
+                                open_at(4 * (g0 + u));
+                            }
+                            if (m4 & 4u) {
+                                macc = __builtin_amdgcn_mfma_f32_16x16x4f32(lane < 32 ? av[u] : 0.f, bv[u], macc, 0, 0, 0);
+                                flush_matrix();
+                                open_at(4 * (g0 + u) + 2);
+                                macc = __builtin_amdgcn_mfma_f32_16x16x4f32(lane < 32 ? 0.f : av[u], bv[u], macc, 0, 0, 0);
+                            } else {
+                                macc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], bv[u], macc, 0, 0, 0);
+                            }
+                        } else {
+                            macc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], bv[u], macc, 0, 0, 0);
+                        }
+                    }
+                }
+            }
+            wave_lds_fence();
+            continue;
+        }
+
         // phase 2: lane = (half, theta_t, Rs_s); the halves take alternate records.  Records past
         // `total` in the last step are zeros, so whole groups of eight pairs can always be run.
         const int npairs = min(64, total - base) >> 1;
@@ -292,7 +366,10 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB>& S, c
         }
         wave_lds_fence();
     }
-    if (total > 0) flush();
+    if (total > 0) {
+        if constexpr (kMatrixPhase2) flush_matrix();
+        else flush();
+    }
 
     // ------------------------------------------------ segments without triples are zeros
     // Each segment lane whose segment is empty clears its own 32 values: eight 16-byte stores per lane (or 32

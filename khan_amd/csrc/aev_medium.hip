@@ -259,7 +259,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
             }
 
             // ------------------------------------------------ segment table, phases 1 and 2, zero fill
-            fwd_angular_batch(S, L, lane, nb, [&](int b) -> unsigned long long {
+            fwd_angular_batch<false>(S, L, lane, nb, [&](int b) -> unsigned long long {
                 const int idx = min(c0 + b, kMediumMaxAtoms - 1);
                 return (static_cast<unsigned long long>(M.row_hi[idx]) << 32) | M.row_lo[idx];
             });

@@ -23,6 +23,8 @@
 // No atomics and no pre-zeroed output.  A centre with more than 32 angular neighbours (the 3.1 A
 // sphere holds about 25 atoms at the densest packings tested) is redone by the general-shape
 // per-centre routine.  Semantics: gpu_featurizer/kernel_cpu.cpp:406-537.
+#include <cstdlib>
+#include <cstring>
 #include "aev_fwd_batch.h"
 
 namespace khan {
@@ -37,7 +39,7 @@ constexpr int kRadTrip = 2;
 // the forward sums is replaced by its derivative along the per-atom vectors (VX, VY, VZ).
 // float: 4 wavefronts per SIMD (LDS 9.8 KB, <= 128 VGPRs; the kernel loses a fifth of its speed at three);
 // double or kJvp: 2 (LDS 19 KB); both: 1.
-template <typename T, bool kJvp>
+template <typename T, bool kJvp, bool kMatrixPhase2 = false>
 __global__ __launch_bounds__(64 * kWavesPerBlock)
 __attribute__((amdgpu_waves_per_eu((sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1), (sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1))))
 void aev_fwd_small_kernel(
@@ -264,7 +266,7 @@ void aev_fwd_small_kernel(
         }
 
         // ------------------------------------------------ segment table, phases 1 and 2, zero fill
-        fwd_angular_batch(S, L, lane, nb, [&](int b) -> unsigned long long {
+        fwd_angular_batch<kMatrixPhase2>(S, L, lane, nb, [&](int b) -> unsigned long long {
             const int cl = min(c0 + b, 63);
             const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(cl << 2, rp_lo));
             const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(cl << 2, rp_hi));
@@ -299,6 +301,19 @@ hipError_t launch_fwd_small(const T* X, const T* Y, const T* Z, const int32_t* A
 {
     if (n_mols <= 0) return hipSuccess;
     const unsigned blocks = (static_cast<unsigned>(n_mols) + kWavesPerBlock - 1u) / kWavesPerBlock;
+    if constexpr (sizeof(T) == 4) {
+        // KHAN_AEV_PHASE2=matrix (read once) selects the variant that sums the angular records on the matrix cores;
+        // it is slower than the default and kept for measurement
+        static const bool matrix_phase2 = [] {
+            const char* v = std::getenv("KHAN_AEV_PHASE2");
+            return v != nullptr && std::strcmp(v, "matrix") == 0;
+        }();
+        if (matrix_phase2) {
+            aev_fwd_small_kernel<T, false, true><<<dim3(blocks), dim3(64 * kWavesPerBlock), 0, stream>>>(
+                X, Y, Z, A, MOs, MACs, n_mols, SIs, nullptr, nullptr, nullptr, out, max_atoms < 64 ? max_atoms : 64, order);
+            return hipGetLastError();
+        }
+    }
     aev_fwd_small_kernel<T, false><<<dim3(blocks), dim3(64 * kWavesPerBlock), 0, stream>>>(
         X, Y, Z, A, MOs, MACs, n_mols, SIs, nullptr, nullptr, nullptr, out, max_atoms < 64 ? max_atoms : 64, order);
     return hipGetLastError();
