@@ -6,7 +6,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "csrc", "libkhan_aev.so")
+# KHAN_AEV_LIBRARY names another build of the same library (the measurement builds of khan_amd.build)
+LIB_PATH = os.environ.get("KHAN_AEV_LIBRARY") or os.path.join(_HERE, "csrc", "libkhan_aev.so")
 
 _c_i32p = ctypes.c_void_p   # all tensor arguments are raw device addresses
 _ptr = ctypes.c_void_p

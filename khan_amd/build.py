@@ -5,6 +5,7 @@
   khan_amd/csrc/libkhan_host.so     host-only batch assembly (gcc, OpenMP)
 
 Run as ``python -m khan_amd.build`` or through ``__graft_entry__.build()``.
+``python -m khan_amd.build --stage-variants`` builds the three measurement libraries of `build_stage_variants`.
 """
 import os
 import shutil
@@ -38,15 +39,17 @@ def _hipcc():
     return exe
 
 
-def build_hip(jobs=4):
-    """Compile every HIP translation unit for gfx950 and link libkhan_aev.so."""
+def build_hip(jobs=4, defines=(), out_dir=None, check=True):
+    """Compile every HIP translation unit for gfx950 and link libkhan_aev.so (into `out_dir`, default csrc/)."""
     hipcc = _hipcc()
+    out_dir = out_dir or CSRC
+    os.makedirs(out_dir, exist_ok=True)
     objs = []
     procs = []
     for src in HIP_SOURCES:
-        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+        obj = os.path.join(out_dir, src.replace(".hip", ".o"))
         objs.append(obj)
-        cmd = [hipcc] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc] + HIPCC_FLAGS + ["-D" + d for d in defines] + ["-c", os.path.join(CSRC, src), "-o", obj]
         print("+", " ".join(cmd), flush=True)
         procs.append(subprocess.Popen(cmd))
         if len(procs) >= jobs:
@@ -58,10 +61,26 @@ def build_hip(jobs=4):
         if p.wait() != 0:
             raise RuntimeError("hipcc failed")
     # the generated code of the inline-asm users is checked before anything is linked: no library without it
-    check_dpp_sources()
-    out = os.path.join(CSRC, "libkhan_aev.so")
+    if check:
+        check_dpp_sources(defines)
+    out = os.path.join(out_dir, "libkhan_aev.so")
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs)
     return out
+
+
+STAGE_BUILDS = os.path.join(CSRC, "stage_builds")
+
+
+def stage_variant_path(skip):
+    return os.path.join(STAGE_BUILDS, "skip%d" % skip, "libkhan_aev.so")
+
+
+def build_stage_variants():
+    """Measurement builds of libkhan_aev.so with a stage of the AEV kernels compiled out (KHAN_PROFILE_SKIP = 1:
+    no angular part, 2: no radial part, 3: neither), for `python -m khan_amd.profiling stages`.  Their results are
+    wrong by design; they are loaded only when KHAN_AEV_LIBRARY names them."""
+    return [build_hip(defines=("KHAN_PROFILE_SKIP=%d" % k,), out_dir=os.path.dirname(stage_variant_path(k)))
+            for k in (1, 2, 3)]
 
 
 DPP_SOURCES = ["aev_small.hip", "aev_medium.hip"]     # translation units that use fma_quad (aev_small_common.h)
@@ -157,13 +176,14 @@ def check_dpp_operands(asm_text, name="<asm>"):
     return uses
 
 
-def check_dpp_sources():
+def check_dpp_sources(defines=()):
     """Compiles the translation units that use the lane-exchange multiply-add to assembly and checks them."""
     hipcc = _hipcc()
     total = 0
     procs = []
     for src in DPP_SOURCES:
-        cmd = [hipcc] + [f for f in HIPCC_FLAGS if f != "-Wall"] + ["-S", "--cuda-device-only", "-o", "-", os.path.join(CSRC, src)]
+        cmd = ([hipcc] + [f for f in HIPCC_FLAGS if f != "-Wall"] + ["-D" + d for d in defines] +
+               ["-S", "--cuda-device-only", "-o", "-", os.path.join(CSRC, src)])
         print("+", " ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True)))
     for src, p in procs:
@@ -171,7 +191,7 @@ def check_dpp_sources():
         if p.returncode != 0:
             raise RuntimeError("hipcc -S failed on " + src)
         total += check_dpp_operands(out, src)
-    if total == 0:
+    if total == 0 and not defines:       # a measurement build may have compiled every use out
         raise RuntimeError("no lane-exchange multiply-add found in %s: the check looks at the wrong files" % DPP_SOURCES)
     print("lane-exchange operands: %d uses checked" % total, flush=True)
     return total
@@ -195,5 +215,8 @@ def build_all():
 
 
 if __name__ == "__main__":
-    build_all()
+    if "--stage-variants" in sys.argv[1:]:
+        build_stage_variants()
+    else:
+        build_all()
     sys.exit(0)

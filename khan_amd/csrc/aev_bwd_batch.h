@@ -157,7 +157,7 @@ __device__ __forceinline__ typename Fast<T>::vec4 bwd_angular_rounds(BwdPool<T>&
     // rounds: d = 1 .. (m-1)/2 for every entry; when m is even one more round for the lower half
     const int full = (m - 1) >> 1;
     const int rounds = live ? full + ((((m & 1) == 0) && (e < (m >> 1))) ? 1 : 0) : 0;
-    const int max_rounds = wave_max(rounds);
+    const int max_rounds = kSkipAngular ? 0 : wave_max(rounds);
     const int self = live ? entry : 0;
     const vec4 vj = pool.nbr[self];
     const vec2 fj = pool.nbr_fc[self];

@@ -103,7 +103,7 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB>& S, c
     const int padded = (cnt + 1) & ~1;
     const int incl = scan_add(padded);
     const int start = incl - padded;
-    const int total = lane_read(incl, 63);            // triple slots in this batch (even)
+    const int total = kSkipAngular ? 0 : lane_read(incl, 63);            // triple slots in this batch (even)
     const unsigned long long nonempty = wave_ballot(cnt > 0);
     for (int w = lane; w < bit_words(kNB); w += 64) S.bits[w] = 0u;
     wave_lds_fence();

@@ -231,7 +231,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                     for (int a = 0; a < 4; ++a) {
                         const int cnt_a = cR[a];
                         T acc_r = T(0);
-                        for (int q0 = 0; q0 < cnt_a; q0 += 4 * kMedRadTrip) {
+                        for (int q0 = 0; q0 < (kSkipRadial ? 0 : cnt_a); q0 += 4 * kMedRadTrip) {
                             vec2 e[kMedRadTrip], ab[kMedRadTrip];
 #pragma unroll
                             for (int u = 0; u < kMedRadTrip; ++u) {

@@ -237,7 +237,7 @@ void aev_fwd_small_kernel(
                 for (int a = 0; a < 4; ++a) {
                     const int cnt_a = a == 0 ? cn.x : a == 1 ? cn.y : a == 2 ? cn.z : cn.w;
                     T acc_r = T(0);
-                    for (int q0 = 0; q0 < mxR[a]; q0 += kRadTrip * rg_ns) {
+                    for (int q0 = 0; q0 < (kSkipRadial ? 0 : mxR[a]); q0 += kRadTrip * rg_ns) {
                         // kRadTrip entries of this lane's slot per trip; slot s takes q = s, s+ns, s+2ns, ...
                         vec2 e[kRadTrip], ab[kRadTrip];
 #pragma unroll

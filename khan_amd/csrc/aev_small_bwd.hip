@@ -146,7 +146,7 @@ void aev_bwd_small_kernel(
             // centres come G at a time in lane order, and not per batch, whose last step is rarely full.
             const T* grow = row_of_lane(min(i, 63));
             T cfx = T(0), cfy = T(0), cfz = T(0);       // this pair's pull on the centre
-            const bool inR = valid && (r < kR_Rc_f) && (r > T(0));
+            const bool inR = !kSkipRadial && valid && (r < kR_Rc_f) && (r > T(0));
             if (inR) {
                 const T sc = bwd_radial_pair<T>(grow, static_cast<int>(aj.w), r, Fast<T>::rcp(r));   // dE/dr / r
                 cfx = sc * dx;

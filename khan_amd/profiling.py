@@ -14,6 +14,10 @@ Refreshing an entry (on a GPU box; four counter passes, one counter each, each a
 
 `bench.py --traffic-probe` launches the pass twice and then a plain 64 MiB device-to-device copy whose traffic is
 known; the counters of the pass are scaled by what they read for that copy.
+
+Time by stage (`python -m khan_amd.profiling stages --workload W`): the passes are timed on the default library and on
+three measurement builds with the angular part, the radial part or both compiled out
+(`python -m khan_amd.build --stage-variants`, built beforehand); differences of those times are the stages.
 """
 import csv
 import glob
@@ -137,6 +141,85 @@ def refresh(workload, directory):
     return out
 
 
+BENCH_SHAPES = {"organic65536": ("organic", 65536), "organic16384": ("organic", 16384), "organic1024": ("organic", 1024),
+                "boxes4096": ("boxes", 4096)}
+
+
+def time_passes(workload, repeats=20):
+    """Average time of the forward and of the backward pass (ms) of a bench workload on the library this process
+    loaded, each pass launched with the batch's size order and size classes as bench.py does."""
+    import torch
+    from . import datagen, ops
+    kind, n_mols = BENCH_SHAPES[workload[:-4] if workload.endswith("_f64") else workload]
+    tdt = torch.float64 if workload.endswith("_f64") else torch.float32
+    b = datagen.make_batch(kind, n_mols)
+    dev = torch.device("cuda:0")
+    X, Y, Z = (torch.from_numpy(v).to(dev).to(tdt) for v in (b.X, b.Y, b.Z))
+    A = torch.from_numpy(b.A).to(dev)
+    macs, mos = ops.mol_offsets(torch.from_numpy(b.mol_idxs).to(dev), b.n_mols)
+    sc, ga, ac = ops.ani_sort(A)
+    acs = ac.cpu()
+    order = ops.size_order(macs)
+    classes = order[-4:].cpu()
+    up = torch.randn(b.n_atoms * 384, dtype=tdt, device=dev)
+    g, s0 = [], 0
+    for c in acs.tolist():
+        g.append(up[s0 * 384:(s0 + c) * 384])
+        s0 += c
+    out = {}
+    passes = (("fwd", lambda: ops.featurize(X, Y, Z, A, mos, macs, sc, acs, order=order, size_classes=classes)),
+              ("bwd", lambda: ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *g, order=order, size_classes=classes)))
+    for _ in range(30):            # the first milliseconds of a process run below the clock the rest runs at
+        for name, fn in passes:
+            fn()
+    for name, fn in passes:
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(repeats):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        out[name] = e0.elapsed_time(e1) / repeats
+    return out
+
+
+def stage_times(workload):
+    """Time of the passes with the angular part, the radial part or both compiled out (the measurement builds of
+    khan_amd.build.build_stage_variants), each library in a process of its own.  Returns {build: {fwd, bwd}}."""
+    from . import build
+    res = {}
+    for name, skip in (("full", 0), ("no angular part", 1), ("no radial part", 2), ("neither (skeleton)", 3)):
+        env = dict(os.environ)
+        env.pop("KHAN_AEV_LIBRARY", None)
+        if skip:
+            lib = build.stage_variant_path(skip)
+            if not os.path.exists(lib):
+                raise RuntimeError(lib + " is missing: python -m khan_amd.build --stage-variants")
+            env["KHAN_AEV_LIBRARY"] = lib
+        r = subprocess.run([sys.executable, "-m", "khan_amd.profiling", "time", "--workload", workload],
+                           env=env, cwd=ROOT, capture_output=True, text=True, timeout=300)
+        if r.returncode != 0:
+            raise RuntimeError("timing %s failed: %s" % (name, r.stderr[-2000:]))
+        res[name] = json.loads(r.stdout.strip().splitlines()[-1])
+    return res
+
+
+def print_stage_table(workload, res):
+    full = res["full"]
+    print("workload %s, kernel sources digest %s; ms per pass (HIP events, 20 launches after 30 warm-up passes)" % (workload, kernel_sources_digest()))
+    print("| build | forward | backward |")
+    print("|---|---|---|")
+    for name, r in res.items():
+        print("| %s | %.3f | %.3f |" % (name, r["fwd"], r["bwd"]))
+    print("| => angular part (full - no angular) | %.3f (%.0f %%) | %.3f (%.0f %%) |" % tuple(
+        x for w in ("fwd", "bwd") for x in (full[w] - res["no angular part"][w], 100 * (full[w] - res["no angular part"][w]) / full[w])))
+    print("| => radial part (full - no radial) | %.3f (%.0f %%) | %.3f (%.0f %%) |" % tuple(
+        x for w in ("fwd", "bwd") for x in (full[w] - res["no radial part"][w], 100 * (full[w] - res["no radial part"][w]) / full[w])))
+    print("| => skeleton (sort, scan, lists, staging, segment tables, stores) | %.3f (%.0f %%) | %.3f (%.0f %%) |" % tuple(
+        x for w in ("fwd", "bwd") for x in (res["neither (skeleton)"][w], 100 * res["neither (skeleton)"][w] / full[w])))
+
+
 def main(argv=None):
     import argparse
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
@@ -145,10 +228,19 @@ def main(argv=None):
     t.add_argument("--workload", required=True)
     t.add_argument("--dir", required=True, help="directory holding fwd_fetch/ fwd_write/ bwd_fetch/ bwd_write/")
     sub.add_parser("digest", help="print the digest of the kernel sources in the tree")
+    st = sub.add_parser("stages", help="time by stage of the AEV passes, from the measurement builds "
+                                       "(python -m khan_amd.build --stage-variants)")
+    st.add_argument("--workload", required=True, choices=sorted(BENCH_SHAPES) + [k + "_f64" for k in sorted(BENCH_SHAPES)])
+    tm = sub.add_parser("time", help="time the two passes on the library this process loads; prints one JSON line")
+    tm.add_argument("--workload", required=True)
     sub.add_parser("show", help="print the record and which entries are stale")
     args = ap.parse_args(argv)
     if args.cmd == "digest":
         print(kernel_sources_digest())
+    elif args.cmd == "time":
+        print(json.dumps(time_passes(args.workload)))
+    elif args.cmd == "stages":
+        print_stage_table(args.workload, stage_times(args.workload))
     elif args.cmd == "show":
         d = kernel_sources_digest()
         for k, e in sorted(load_records().items()):
