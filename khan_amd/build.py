@@ -39,7 +39,7 @@ def _hipcc():
     return exe
 
 
-def build_hip(jobs=4, defines=(), out_dir=None, check=True):
+def build_hip(jobs=4, defines=(), out_dir=None):
     """Compile every HIP translation unit for gfx950 and link libkhan_aev.so (into `out_dir`, default csrc/)."""
     hipcc = _hipcc()
     out_dir = out_dir or CSRC
@@ -61,8 +61,7 @@ def build_hip(jobs=4, defines=(), out_dir=None, check=True):
         if p.wait() != 0:
             raise RuntimeError("hipcc failed")
     # the generated code of the inline-asm users is checked before anything is linked: no library without it
-    if check:
-        check_dpp_sources(defines)
+    check_dpp_sources(defines)
     out = os.path.join(out_dir, "libkhan_aev.so")
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs)
     return out

@@ -145,4 +145,5 @@ def test_the_library_cannot_be_built_without_the_lane_exchange_check():
     import inspect
     from khan_amd import build
     src = inspect.getsource(build.build_hip)
-    assert src.index("check_dpp_sources()") < src.index('"-shared"')
+    assert src.index("check_dpp_sources(defines)") < src.index('"-shared"')
+    assert "check=" not in src and "if check" not in src          # no switch that skips it
