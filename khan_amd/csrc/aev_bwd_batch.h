@@ -28,38 +28,87 @@ __device__ __forceinline__ int sel6(int b, int v0, int v1, int v2, int v3, int v
     return b == 0 ? v0 : b == 1 ? v1 : b == 2 ? v2 : b == 3 ? v3 : b == 4 ? v4 : v5;
 }
 
-// sum over the 16 shells of g_q e_q (f_C' - 2 eta d_q f_C), e_q = exp(-eta d_q^2), d_q = r - Rs_q
-template <typename T>
-__device__ __forceinline__ T radial_shell_sum(const T (&g)[16], T r, T fc, T dfc)
+// sum over the shells of g_q e_q (f_C' - 2 eta d_q f_C), e_q = exp(-eta d_q^2), d_q = r - Rs_q, for kN shells whose
+// radii are rs[0..kN)
+template <typename T, int kN>
+__device__ __forceinline__ T radial_shell_sum(const T (&g)[kN], const T (&rs)[kN], T r, T fc, T dfc)
 {
     const T m2eta_fc = T(-2) * static_cast<T>(kR_eta_f) * fc;
     T Gsum = T(0);
 #pragma unroll
-    for (int q = 0; q < kNumRRs; ++q) {
-        const T d = r - static_cast<T>(kR_Rs_f[q]);
+    for (int q = 0; q < kN; ++q) {
+        const T d = r - rs[q];
         const T e = Fast<T>::gauss(static_cast<T>(kR_eta_f), d);
         Gsum = fma(g[q] * e, fma(m2eta_fc, d, dfc), Gsum);   // g e (f_C' - 2 eta d f_C)
     }
     return Gsum;
 }
 
-// Radial part of one (centre, partner) pair: sum over the 16 shells of g e (f_C' - 2 eta d f_C), divided
+// Which shells a pair at distance r needs.  double: all 16.  float: the nine nearest to r -- a shell more than 4.5
+// spacings (1.15 A) away contributes exp(-16 * 1.15^2) = 6e-10 times a factor that grows no faster than 2 eta d,
+// in all less than 1e-8 of the largest term of the sum for every r below the cutoff: an order below the rounding of
+// the float sum itself.  The window is [q0, q0 + 9) with q0 = clamp(nearest - 4, 0, 7).
+template <typename T> struct ShellWindow {
+    static constexpr int kShells = kNumRRs;
+    static __device__ __forceinline__ int first(T) { return 0; }
+};
+template <> struct ShellWindow<float> {
+    static constexpr int kShells = 9;
+    static __device__ __forceinline__ int first(float r)
+    {
+        constexpr float kInvSpacing = 1.0f / 0.25625f;          // Rs_q = 0.5 + 0.25625 q
+        const int nearest = __float2int_rn((r - 0.5f) * kInvSpacing);
+        return min(max(nearest - 4, 0), kNumRRs - kShells);
+    }
+};
+
+typedef float v4f_dword_aligned __attribute__((ext_vector_type(4), aligned(4)));
+typedef const __attribute__((address_space(1))) v4f_dword_aligned* global_v4f_unaligned_ptr;
+typedef const __attribute__((address_space(1))) float* global_float_ptr;
+
+// the window's upstream values g[q0 .. q0 + kShells) of a 16-shell block, and the shells' radii
+template <typename T>
+__device__ __forceinline__ void load_shell_window(const T* block, int q0, T (&g)[ShellWindow<T>::kShells],
+                                                  T (&rs)[ShellWindow<T>::kShells])
+{
+    if constexpr (sizeof(T) == 4) {
+        // nine floats from a 4-byte-aligned address: two 16-byte loads and one of 4 bytes
+        const global_v4f_unaligned_ptr gp = (global_v4f_unaligned_ptr)(block + q0);
+        const v4f_dword_aligned a = gp[0], b = gp[1];
+        g[0] = a.x; g[1] = a.y; g[2] = a.z; g[3] = a.w;
+        g[4] = b.x; g[5] = b.y; g[6] = b.z; g[7] = b.w;
+        g[8] = ((global_float_ptr)(block + q0))[8];
+#pragma unroll
+        for (int q = 0; q < 9; ++q) rs[q] = kR_Rs_f[q0 + q];
+    } else {
+        constexpr int kPieces = 16 * sizeof(T) / 16;          // 16-byte loads for the 16 upstream values
+        union {
+            v4f piece[kPieces];
+            T gr[16];
+        } u;
+        const global_v4f_ptr gp = (global_v4f_ptr)block;
+#pragma unroll
+        for (int q = 0; q < kPieces; ++q) u.piece[q] = gp[q];
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            g[q] = u.gr[q];
+            rs[q] = static_cast<T>(kR_Rs_f[q]);
+        }
+    }
+}
+
+// Radial part of one (centre, partner) pair: sum over the shells of g e (f_C' - 2 eta d f_C), divided
 // by r.  The result times (x_i - x_j) is the pair's pull on the centre (and minus that on the partner).
 // `grow` is the centre's upstream row, `tj` the partner's type, `inv` = 1/r.
 template <typename T>
 __device__ __forceinline__ T bwd_radial_pair(const T* grow, int tj, T r, T inv)
 {
-    constexpr int kPieces = 16 * sizeof(T) / 16;          // 16-byte loads for the 16 upstream values
-    union {
-        v4f piece[kPieces];
-        T gr[16];
-    } u;
-    const global_v4f_ptr gp = (global_v4f_ptr)(grow + tj * kNumRRs);
-#pragma unroll
-    for (int q = 0; q < kPieces; ++q) u.piece[q] = gp[q];
+    constexpr int kN = ShellWindow<T>::kShells;
+    T g[kN], rs[kN];
+    load_shell_window<T>(grow + tj * kNumRRs, ShellWindow<T>::first(r), g, rs);
     T fc, dfc;
     Fast<T>::cutoff_grad(r, static_cast<T>(kR_Rc_f), fc, dfc);
-    return radial_shell_sum<T>(u.gr, r, fc, dfc) * inv;           // dE/dr / r
+    return radial_shell_sum<T, kN>(g, rs, r, fc, dfc) * inv;           // dE/dr / r
 }
 
 // Both directions of a pair at once: centre c with partner j reads row c's block for j's type, centre j with
@@ -69,23 +118,16 @@ __device__ __forceinline__ T bwd_radial_pair(const T* grow, int tj, T r, T inv)
 template <typename T>
 __device__ __forceinline__ T bwd_radial_pair_both(const T* grow_c, int tj, const T* grow_j, int tc, T r, T inv)
 {
-    constexpr int kPieces = 16 * sizeof(T) / 16;
-    union {
-        v4f piece[kPieces];
-        T gr[16];
-    } u, w;
-    const global_v4f_ptr gp = (global_v4f_ptr)(grow_c + tj * kNumRRs);
-    const global_v4f_ptr gq = (global_v4f_ptr)(grow_j + tc * kNumRRs);
-#pragma unroll
-    for (int q = 0; q < kPieces; ++q) {
-        u.piece[q] = gp[q];
-        w.piece[q] = gq[q];
-    }
+    constexpr int kN = ShellWindow<T>::kShells;
+    T g[kN], w[kN], rs[kN];
+    const int q0 = ShellWindow<T>::first(r);
+    load_shell_window<T>(grow_c + tj * kNumRRs, q0, g, rs);
+    load_shell_window<T>(grow_j + tc * kNumRRs, q0, w, rs);
     T fc, dfc;
     Fast<T>::cutoff_grad(r, static_cast<T>(kR_Rc_f), fc, dfc);
 #pragma unroll
-    for (int q = 0; q < kNumRRs; ++q) u.gr[q] += w.gr[q];
-    return radial_shell_sum<T>(u.gr, r, fc, dfc) * inv;
+    for (int q = 0; q < kN; ++q) g[q] += w[q];
+    return radial_shell_sum<T, kN>(g, rs, r, fc, dfc) * inv;
 }
 
 // The angular part of an upstream row is 320 elements = kRowPieces 16-byte pieces; a wavefront fetches it

@@ -136,7 +136,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                     const int jj = min(j, kMediumMaxAtoms - 1);
                     const vec4 aj = M.atom[jj];
                     const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
-                    const T r = sqrt(dx * dx + dy * dy + dz * dz);
+                    const T r = Fast<T>::sqrt_rn(dx * dx + dy * dy + dz * dz);
                     const bool valid = (j < n) && (j != i);
                     // r = 0, a coincident atom: no part in derivatives; in the features as the reference has it
                     const bool inR = valid && (r < kR_Rc_f) && (!kJvp || r > T(0));

@@ -214,7 +214,7 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
                         dx[ch] = ai.x - aj.x;
                         dy[ch] = ai.y - aj.y;
                         dz[ch] = ai.z - aj.z;
-                        r[ch] = sqrt(dx[ch] * dx[ch] + dy[ch] * dy[ch] + dz[ch] * dz[ch]);
+                        r[ch] = Fast<T>::sqrt_rn(dx[ch] * dx[ch] + dy[ch] * dy[ch] + dz[ch] * dz[ch]);
                         const bool valid = (j < n) && (j != c);
                         mR[ch] = wave_ballot(!kSkipRadial && valid && (r[ch] < kR_Rc_f) && (r[ch] > T(0)));     // r = 0: a coincident atom exerts no force
                         mA[ch] = wave_ballot(valid && (r[ch] < kA_Rc_f) && (r[ch] > T(0)));

@@ -162,7 +162,7 @@ void aev_fwd_small_kernel(
             const bool centre_ok = b < nb;
             const int ci = (centre_ok ? i : 0) << 2;
             const T dx = lane_fetch(x, ci) - xj, dy = lane_fetch(y, ci) - yj, dz = lane_fetch(z, ci) - zj;
-            const T r = sqrt(dx * dx + dy * dy + dz * dz);
+            const T r = Fast<T>::sqrt_rn(dx * dx + dy * dy + dz * dz);
             const bool valid = centre_ok && (jl < n) && (jl != i);
             // a coincident atom (r = 0) has no direction: it takes no part in any derivative.  In the features it
             // counts as the reference counts it: its cosine is 0/0, which the clamp turns into -1 (kernel_cpu.cpp:514-516)

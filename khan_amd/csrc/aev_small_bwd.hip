@@ -135,7 +135,7 @@ void aev_bwd_small_kernel(
             const int i = s0 + grp;
             const vec4 ai = S.atom[min(i, 63)];
             const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
-            const T r = sqrt(dx * dx + dy * dy + dz * dz);
+            const T r = Fast<T>::sqrt_rn(dx * dx + dy * dy + dz * dz);
             const bool valid = (i < n) && (jl < n) && (jl != i);
             const bool inA = valid && (r < kA_Rc_f) && (r > T(0));     // r = 0: a coincident atom exerts no force
             const int cnt = popc64(wave_ballot(inA) & sub_mask);          // in every lane of the group
@@ -225,7 +225,7 @@ void aev_bwd_small_kernel(
             const int room = sel6(cb, pf[1], pf[2], pf[3], pf[4], pf[5], pf[6]) - base;
             const vec4 ai = S.atom[i];
             const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
-            const T r = sqrt(dx * dx + dy * dy + dz * dz);
+            const T r = Fast<T>::sqrt_rn(dx * dx + dy * dy + dz * dz);
             const bool valid = centre_ok && (jl < n) && (jl != i);
             const bool inA = valid && (r < kA_Rc_f) && (r > T(0));
             const unsigned long long mA = wave_ballot(inA);

@@ -269,6 +269,17 @@ template <> struct Fast<float> {
     static __device__ __forceinline__ float4 make4(float a, float b, float c, float d) { return make_float4(a, b, c, d); }
     static __device__ __forceinline__ float2 make2(float a, float b) { return make_float2(a, b); }
     static __device__ __forceinline__ float sqrt_(float x) { return __builtin_amdgcn_sqrtf(x); }
+    // Square root to half an ulp (the distances: their rounding is what limits the float results) without the
+    // library routine's scaling for denormals and its two trial roundings: the hardware's reciprocal square root
+    // (1 ulp) and one Newton step, whose fused residual x - s^2 is exact.  The reciprocal is capped so that
+    // x = 0 gives 0 and not 0 * inf.  6 instructions instead of 14.
+    static __device__ __forceinline__ float sqrt_rn(float x)
+    {
+        const float y = fminf(__builtin_amdgcn_rsqf(x), 1.0e18f);
+        const float s = x * y;
+        const float e = fmaf(-s, s, x);
+        return fmaf(e, 0.5f * y, s);
+    }
     static __device__ __forceinline__ float rcp(float x) { return __builtin_amdgcn_rcpf(x); }
     // exp(-eta d^2)
     static __device__ __forceinline__ float gauss(float eta, float d) { return __builtin_amdgcn_exp2f((-eta * 1.44269504088896340736f) * d * d); }
@@ -284,6 +295,7 @@ template <> struct Fast<double> {
     static __device__ __forceinline__ double4 make4(double a, double b, double c, double d) { return make_double4(a, b, c, d); }
     static __device__ __forceinline__ double2 make2(double a, double b) { return make_double2(a, b); }
     static __device__ __forceinline__ double sqrt_(double x) { return sqrt(x); }
+    static __device__ __forceinline__ double sqrt_rn(double x) { return sqrt(x); }
     static __device__ __forceinline__ double rcp(double x) { return 1.0 / x; }
     static __device__ __forceinline__ double gauss(double eta, double d) { return exp(-eta * d * d); }
     static __device__ __forceinline__ double cutoff(double r, double rc) { return 0.5 * cos(kPi / rc * r) + 0.5; }
