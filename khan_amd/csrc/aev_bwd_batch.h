@@ -14,12 +14,13 @@ constexpr int kBlockStride = 36;   // elements between staged 32-element blocks:
 
 // per-wavefront LDS of a batch: the centres' angular partner lists laid end to end (at most 64 entries)
 // and their rows' angular upstream values
-template <typename T>
+template <typename T, int kNB = kB>
 struct __align__(16) BwdPool {
+    static constexpr int kCentres = kNB;          // centres per batch
     typename Fast<T>::vec4 nbr[64];               // unit vector (centre minus partner)/r, and r
     typename Fast<T>::vec4 facc[64];              // force on each list entry from its centre's row
     typename Fast<T>::vec2 nbr_fc[64];            // f_C(r, A_Rc) and its derivative in r
-    T gst[kB * kNumPairBlocks * kBlockStride];    // staged upstream blocks [centre][type pair][32]
+    T gst[kNB * kNumPairBlocks * kBlockStride];   // staged upstream blocks [centre][type pair][32]
     unsigned char nbr_idx[64];                    // sorted position of the partner
 };
 
@@ -132,18 +133,18 @@ __device__ __forceinline__ T bwd_radial_pair_both(const T* grow_c, int tj, const
 
 // The angular part of an upstream row is 320 elements = kRowPieces 16-byte pieces; a wavefront fetches it
 // with kPieceRegs loads per lane (piece r * 64 + lane).
-template <typename T> struct RowStage {
+template <typename T, int kNB = kB> struct RowStage {
     static constexpr int kPerPiece = 16 / sizeof(T);                  // elements in a 16-byte piece
     static constexpr int kRowPieces = kAngular / kPerPiece;           // 80 (float) or 160 (double)
     static constexpr int kPieceRegs = (kRowPieces + 63) / 64;         // 2 or 3
-    v4f st[kB][kPieceRegs];
+    v4f st[kNB][kPieceRegs];
 
     // issues the loads for the rows of centres 0..nb-1; row_of(b) is wave-uniform
     template <typename RowOf>
     __device__ __forceinline__ void fetch(int lane, int nb, RowOf row_of)
     {
 #pragma unroll
-        for (int b = 0; b < kB; ++b) {
+        for (int b = 0; b < kNB; ++b) {
             // Registers of centres beyond nb and of pieces beyond the row are never stored.  They are declared written
             // without an instruction: left unset they are "undefined" to the compiler, whose handling of that cost 30
             // registers here, and filling them with zeros costs 48 moves per batch.
@@ -158,10 +159,10 @@ template <typename T> struct RowStage {
         }
     }
     // writes the fetched pieces into the pool, one 32-element block per type pair
-    __device__ __forceinline__ void store(BwdPool<T>& pool, int lane, int nb) const
+    __device__ __forceinline__ void store(BwdPool<T, kNB>& pool, int lane, int nb) const
     {
 #pragma unroll
-        for (int b = 0; b < kB; ++b) {
+        for (int b = 0; b < kNB; ++b) {
             if (b < nb) {
 #pragma unroll
                 for (int r = 0; r < kPieceRegs; ++r) {
@@ -187,8 +188,8 @@ __device__ __forceinline__ int round_copies(int total) { return total <= 16 ? 4 
 // the force on the lane's own entry is kept in registers.
 // Returns the entry's total over all copies, in every copy's lane (zero for lanes without an entry).
 // `type_of(sorted position)` gives an atom's type.
-template <typename T, typename TypeOf>
-__device__ __forceinline__ typename Fast<T>::vec4 bwd_angular_rounds(BwdPool<T>& pool, int entry, int copy, int copies, bool live,
+template <typename T, int kNB, typename TypeOf>
+__device__ __forceinline__ typename Fast<T>::vec4 bwd_angular_rounds(BwdPool<T, kNB>& pool, int entry, int copy, int copies, bool live,
                                                      int bs, int pb, int m, TypeOf type_of)
 {
     typedef typename Fast<T>::vec4 vec4;

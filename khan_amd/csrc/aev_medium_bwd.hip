@@ -25,6 +25,10 @@ namespace khan {
 namespace {
 
 constexpr int kChunks = kMediumMaxAtoms / 64;
+// centres per batch.  float: four, so that the pools of the four wavefronts leave room for four workgroups on a CU
+// (LDS 39.6 KB; 128 registers) -- the shorter batches fill fewer lanes, the fourth wavefront per SIMD hides more;
+// double: six, one workgroup per CU either way.
+template <typename T> constexpr int kMedBwdCentres = sizeof(T) == 4 ? 4 : kB;
 
 template <typename T>
 struct __align__(16) MedBwdShared {
@@ -37,7 +41,8 @@ struct __align__(16) MedBwdShared {
 };
 
 template <typename T>
-__global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 4 : 1, sizeof(T) == 4 ? 4 : 1)))
+void aev_bwd_medium_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
@@ -46,11 +51,12 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
 {
     typedef typename Fast<T>::vec4 vec4;
     __shared__ MedBwdShared<T> M;
-    __shared__ BwdPool<T> pools[4];
+    constexpr int kMB = kMedBwdCentres<T>;
+    __shared__ BwdPool<T, kMB> pools[4];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = uniform(tid >> 6);
-    BwdPool<T>& P = pools[wave];
+    BwdPool<T, kMB>& P = pools[wave];
     const LaneConsts<T> L = lane_consts<T>(lane);
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
 
@@ -188,7 +194,7 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
             int nb = 0, used = 0;
             int pfv = 0, cv = 0;   // lane k: first pool slot and sorted position of centre k of the batch
             P.facc[lane] = Fast<T>::make4(T(0), T(0), T(0), T(0));
-            while (nb < kB) {
+            while (nb < kMB) {
                 int c = pending;
                 pending = -1;
                 if (c < 0) {
@@ -307,7 +313,7 @@ __global__ __launch_bounds__(256) void aev_bwd_medium_kernel(
 
             // ---- the angular upstream blocks of the batch's rows go to LDS (80 x 16 bytes per row)
             {
-                RowStage<T> stage;
+                RowStage<T, kMB> stage;
                 stage.fetch(lane, nb, [&](int b) { return row_of(lane_read(cv, b)); });
                 stage.store(P, lane, nb);
             }
