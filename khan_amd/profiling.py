@@ -34,13 +34,13 @@ COPY_BYTES = 64 * 1024 * 1024
 
 # the kernel that dominates each pass of each bench workload (substring of the name rocprofv3 prints)
 DOMINANT = {
-    ("organic65536", "fwd"): "aev_fwd_small_kernel<float, false>",
+    ("organic65536", "fwd"): "aev_fwd_small_kernel<float, false, false>",
     ("organic65536", "bwd"): "aev_bwd_small_kernel<float>",
-    ("organic16384", "fwd"): "aev_fwd_small_kernel<float, false>",
+    ("organic16384", "fwd"): "aev_fwd_small_kernel<float, false, false>",
     ("organic16384", "bwd"): "aev_bwd_small_kernel<float>",
-    ("organic1024", "fwd"): "aev_fwd_small_kernel<float, false>",
+    ("organic1024", "fwd"): "aev_fwd_small_kernel<float, false, false>",
     ("organic1024", "bwd"): "aev_bwd_small_kernel<float>",
-    ("organic16384_f64", "fwd"): "aev_fwd_small_kernel<double, false>",
+    ("organic16384_f64", "fwd"): "aev_fwd_small_kernel<double, false, false>",
     ("organic16384_f64", "bwd"): "aev_bwd_small_kernel<double>",
     ("boxes4096", "fwd"): "aev_fwd_medium_kernel<float, false>",
     ("boxes4096", "bwd"): "aev_bwd_medium_kernel<float>",
