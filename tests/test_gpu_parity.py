@@ -970,6 +970,50 @@ def test_gradient_against_central_differences_on_64_molecules(ops):
 
 
 
+def test_radial_gradient_at_every_distance(ops):
+    """The float32 backward kernels sum the radial shells nearest to the pair's distance only (nine of sixteen): pairs
+    at 240 distances from 0.04 A to beyond the cutoff, alone (one-wavefront kernel) and inside a 70-atom molecule
+    whose other atoms are out of reach (workgroup-per-molecule kernel), against the float64 oracle, which sums all
+    sixteen.  Also a third atom at an angle, so that the window edges are met together with angular terms."""
+    say("case: pair distances 0.04 .. 4.7 A, float32 radial window against the oracle's full sum")
+    rng = np.random.default_rng(21)
+    dists = np.concatenate([np.linspace(0.04, 4.7, 200), 0.5 + 0.25625 * (np.arange(16) + 0.5), 0.5 + 0.25625 * np.arange(16),
+                            [4.5999, 4.6, 4.6001, 3.0999, 3.1, 3.1001, 1e-3, 2e-2]])
+    mols = []
+    for k, d in enumerate(dists):
+        u = rng.standard_normal(3)
+        u /= np.linalg.norm(u)
+        t = rng.integers(0, 4, 3)
+        v = np.cross(u, rng.standard_normal(3))
+        v /= np.linalg.norm(v)
+        third = 0.8 * d * (0.3 * u + 0.95 * v) + 1e-3
+        mols.append((t.astype(np.int32), np.stack([np.zeros(3), d * u, third])))            # 3 atoms
+        if k % 4 == 0:                                                                       # the same pair in a large molecule
+            far = np.stack([np.array([20.0 + 12.0 * (i % 8), 12.0 * (i // 8), 40.0]) for i in range(67)])
+            mols.append((np.concatenate([t, rng.integers(0, 4, 67)]).astype(np.int32),
+                         np.concatenate([np.stack([np.zeros(3), d * u, third]), far])))
+    A = np.concatenate([m[0] for m in mols])
+    xyz = np.concatenate([m[1] for m in mols])
+    mol_idxs = np.concatenate([np.full(len(m[0]), i, dtype=np.int32) for i, m in enumerate(mols)])
+    c = Case(xyz[:, 0], xyz[:, 1], xyz[:, 2], A, mol_idxs, len(mols))
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+    acs = ac.cpu()
+    upb = c.upstream(seed=22)
+    g64 = c.oracle_grad(upb)
+    assert np.all(np.isfinite(g64))
+    S = mol_scale(g64, c.MOs, c.MACs)
+    Ad = dev(c.A)
+    for tdt, ndt, rtol, atol in ((torch.float32, np.float32, F32_RTOL, F32_ATOL), (torch.float64, np.float64, F64_RTOL, 0.0)):
+        X, Y, Z = dev(c.X, ndt), dev(c.Y, ndt), dev(c.Z, ndt)
+        gx, gy, gz = ops.featurize_grad(X, Y, Z, Ad, mos, macs, sc, acs, *[dev(x, ndt) for x in upb])
+        gg = host(torch.stack([gx, gy, gz], dim=1))
+        assert_close("gradient %s, %d molecules" % (np.dtype(ndt).name, len(mols)), gg, g64, rtol, atol, scale=S)
+        # the forces of a molecule add up to nothing (sum over a molecule of mixed-sign components: on its scale)
+        for m in range(0, len(mols), 37):
+            s_ = slice(c.MOs[m], c.MOs[m] + c.MACs[m])
+            assert np.abs(gg[s_].sum(axis=0)).max() <= (2e-5 if ndt == np.float32 else 1e-11) * max(float(S[c.MOs[m]].max()), 1e-30)
+
+
 def _ratio_quantiles(name, got, ref, rtol, atol):
     """Per-element |got - ref| / (atol + rtol |ref|) -- the tolerance as BASELINE words it, every component on
     its own -- as quantiles; non-finite entries of `got` are left out and counted."""
