@@ -1015,7 +1015,7 @@ def test_radial_gradient_at_every_distance(ops):
 
 
 def _ratio_quantiles(name, got, ref, rtol, atol):
-    """Per-element |got - ref| / (atol + rtol |ref|) -- the tolerance as BASELINE words it, every component on
+    """Per-element |got - ref| / (atol + rtol |ref|) -- the tolerance taken component by component, every component on
     its own -- as quantiles; non-finite entries of `got` are left out and counted."""
     got, ref = np.asarray(got, dtype=np.float64), np.asarray(ref, dtype=np.float64)
     ok = np.isfinite(got)
@@ -1027,7 +1027,7 @@ def _ratio_quantiles(name, got, ref, rtol, atol):
 
 
 def test_gradient_error_per_element_beside_the_references_own_functor(ops):
-    """How much the per-molecule scale in the gradient tolerance relaxes BASELINE's per-element wording
+    """How much the per-molecule scale in the gradient tolerance relaxes a per-element reading of the same tolerance
     (float32 1e-5 relative / 1e-6 absolute; float64 1e-12 relative), measured: the per-element error ratio of
     the HIP gradients against the float64 oracle, beside the same ratio for the reference's own functor
     (gpu_featurizer/kernel_cpu.cpp:217-366 compiled in place, float32 and float64, finite entries only).  A
