@@ -13,6 +13,7 @@ else this repo's CPU port) timed on a bounded sample of the same batch.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload organic65536|organic16384_f64|boxes4096|...]
 """
 import argparse
+import collections
 import json
 import os
 import sys
@@ -376,11 +377,13 @@ def main():
             counts_pinned[slot][4:8].copy_(order[-4:], non_blocking=True)
             done = torch.cuda.Event()
             done.record()
-            for t in (macs, mos, sc, ga, ac, order):
-                t.record_stream(main_stream)   # allocated on the feeder's stream, read by the passes on the main one
+        # macs, mos, sc and order are allocated on the feeder's stream and read by the passes on the main one: the
+        # step keeps them alive until an event behind its passes has completed (`in_use` below).  Telling the
+        # allocator instead (record_stream) costs an event packet per array on the main stream at every step boundary.
         return {"macs": macs, "mos": mos, "sc": sc, "order": order, "slot": slot, "done": done, "marks": (m0, m1)}
 
     state = {"cur": None, "n": 0}
+    in_use = collections.deque()      # (event behind a step's passes, that step's arrays)
 
     def step(timed):
         if state["cur"] is None:
@@ -410,9 +413,17 @@ def main():
         gx, gy, gz = ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *grads, order=order, size_classes=classes)
         if timed:
             marks[2].record()
+        behind = marks[2] if timed else None
         if with_charges:     # energy, then its gradient with respect to charges and coordinates
             e = ops.ani_charge(X, Y, Z, Q, mos, macs)
             qg = ops.ani_charge_grad_xyz(X, Y, Z, Q, mos, macs, ones_m)
+            behind = None
+        if behind is None:
+            behind = torch.cuda.Event()
+            behind.record()
+        in_use.append((behind, cur))
+        while in_use and in_use[0][0].query():
+            in_use.popleft()
         state["cur"] = nxt
         return (nxt["marks"], marks), (feats, gx, gy, gz)
 
