@@ -147,3 +147,50 @@ def test_the_library_cannot_be_built_without_the_lane_exchange_check():
     src = inspect.getsource(build.build_hip)
     assert src.index("check_dpp_sources(defines)") < src.index('"-shared"')
     assert "check=" not in src and "if check" not in src          # no switch that skips it
+
+
+def test_traffic_record_is_tied_to_the_kernel_sources(tmp_path, monkeypatch):
+    """bench.py reports roofline.traffic from the record only while the record's digest matches the kernel sources in
+    the tree; a record measured on other sources comes back as stale (bytes None), a missing one as absent."""
+    import json
+    from khan_amd import profiling
+    d = profiling.kernel_sources_digest()
+    assert len(d) == 16 and d == profiling.kernel_sources_digest()
+    rec = tmp_path / "hbm_traffic.json"
+    monkeypatch.setattr(profiling, "RECORD", str(rec))
+    assert profiling.measured_traffic("organic65536", "bwd") == (None, False, None)
+    entry = {"bytes": 123.0, "sources_digest": d, "kernel": "k", "fetch_bytes": 100.0, "write_bytes": 23.0}
+    rec.write_text(json.dumps({"organic65536/bwd": entry, "organic65536/fwd": dict(entry, sources_digest="0" * 16)}))
+    b, stale, e = profiling.measured_traffic("organic65536", "bwd")
+    assert (b, stale) == (123.0, False) and e["kernel"] == "k"
+    b, stale, e = profiling.measured_traffic("organic65536", "fwd")
+    assert b is None and stale and e is not None
+
+
+def test_the_committed_traffic_record_names_the_dominant_kernels():
+    """Every entry of profiles/hbm_traffic.json belongs to a (workload, pass) whose dominant kernel is known, and
+    carries the pieces its total is made of."""
+    from khan_amd import profiling
+    rec = profiling.load_records()
+    assert rec, "profiles/hbm_traffic.json is missing or empty"
+    for key, e in rec.items():
+        workload, which = key.split("/")
+        assert profiling.DOMINANT[(workload, which)] == e["kernel"], key
+        assert abs(e["fetch_bytes"] + e["write_bytes"] - e["bytes"]) <= 1e-6 * e["bytes"]
+        assert 1.9 < e["fetch_scale"] < 2.1 and 0.95 < e["write_scale"] < 1.05      # what a 64 MiB copy reads on this part
+
+
+def test_measurement_builds_are_not_the_default_library(monkeypatch):
+    """KHAN_AEV_LIBRARY, and nothing else, makes the package load another build of the library."""
+    import importlib
+    from khan_amd import build
+    monkeypatch.delenv("KHAN_AEV_LIBRARY", raising=False)
+    from khan_amd import _lib
+    m = importlib.reload(_lib)
+    assert m.LIB_PATH.endswith(os.path.join("khan_amd", "csrc", "libkhan_aev.so"))
+    for k in (1, 2, 3):
+        assert "stage_builds" in build.stage_variant_path(k) and build.stage_variant_path(k) != m.LIB_PATH
+    monkeypatch.setenv("KHAN_AEV_LIBRARY", build.stage_variant_path(3))
+    assert importlib.reload(_lib).LIB_PATH == build.stage_variant_path(3)
+    monkeypatch.delenv("KHAN_AEV_LIBRARY")
+    importlib.reload(_lib)
