@@ -149,13 +149,9 @@ def inference_bench(args, batch):
     from khan_amd.batching import DeviceBatch
     dev = torch.device("cuda:0")
     N, n_mols = batch.n_atoms, batch.n_mols
-    b = DeviceBatch()
-    b.xs, b.ys, b.zs = (torch.from_numpy(v).to(dev) for v in (batch.X, batch.Y, batch.Z))
-    b.atom_types = torch.from_numpy(batch.A).to(dev)
-    b.mol_idxs = torch.from_numpy(batch.mol_idxs).to(dev)
-    b.n_mols = n_mols
-    b.mol_atom_counts, b.mol_offsets = ops.mol_offsets(b.mol_idxs, n_mols)
-    b.scatter_idxs, b.gather_idxs, b.atom_counts = ops.ani_sort(b.atom_types)
+    xs, ys, zs = (torch.from_numpy(v).to(dev) for v in (batch.X, batch.Y, batch.Z))
+    b = DeviceBatch.from_device_arrays(xs, ys, zs, torch.from_numpy(batch.A).to(dev),
+                                       torch.from_numpy(batch.mol_idxs).to(dev), n_mols)
     def timed(first_layer_kernel):
         m = model.AniModel(model.DEFAULT_LAYERS, model.celu, torch.float32, dev, seed=1, first_layer_kernel=first_layer_kernel)
         for _ in range(args.warmup):

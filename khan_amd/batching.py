@@ -196,7 +196,39 @@ class DeviceBatch:
     """One batch resident on the GPU, with everything `featurize` needs."""
 
     __slots__ = ("xs", "ys", "zs", "atom_types", "mol_idxs", "n_mols", "mol_atom_counts", "mol_offsets",
-                 "scatter_idxs", "gather_idxs", "atom_counts", "labels", "grads", "ready")
+                 "scatter_idxs", "gather_idxs", "atom_counts", "size_order", "counts_pinned", "labels", "grads", "ready")
+
+    def host_counts(self):
+        """-> (atoms per type [4], the size order on the device, molecules per size class [4] on the host): what the
+        host has to know before it can launch the passes.  One 32-byte copy, enqueued by the feeder behind the
+        sort; this waits for it."""
+        self.ready.synchronize()
+        return self.counts_pinned[0:4].tolist(), self.size_order, self.counts_pinned[4:8].clone()
+
+    @classmethod
+    def from_device_arrays(cls, xs, ys, zs, atom_types, mol_idxs, n_mols):
+        """A batch from arrays that are on the GPU already: runs `mol_offsets`, `ani_sort` and `size_order` on the
+        current stream and enqueues the copy of the counts."""
+        import torch
+        from . import ops
+        b = cls()
+        b.xs, b.ys, b.zs, b.atom_types, b.mol_idxs, b.n_mols = xs, ys, zs, atom_types, mol_idxs, n_mols
+        b.labels = b.grads = None
+        b.finish_on_current_stream()
+        return b
+
+    def finish_on_current_stream(self):
+        """Offsets, type sort, size order and the copy of the counts for the arrays already in place; records `ready`."""
+        import torch
+        from . import ops
+        self.mol_atom_counts, self.mol_offsets = ops.mol_offsets(self.mol_idxs, self.n_mols)
+        self.scatter_idxs, self.gather_idxs, self.atom_counts = ops.ani_sort(self.atom_types)
+        self.size_order = ops.size_order(self.mol_atom_counts)
+        self.counts_pinned = torch.empty(8, dtype=torch.int32, pin_memory=True)     # from the pinned-memory cache
+        self.counts_pinned[0:4].copy_(self.atom_counts, non_blocking=True)
+        self.counts_pinned[4:8].copy_(self.size_order[-4:], non_blocking=True)
+        self.ready = torch.cuda.Event()
+        self.ready.record()
 
     def wait(self):
         """Makes the current stream wait for the copies and the sort of this batch."""
@@ -204,7 +236,7 @@ class DeviceBatch:
         cur = torch.cuda.current_stream()
         cur.wait_event(self.ready)
         for name in ("xs", "ys", "zs", "atom_types", "mol_idxs", "mol_atom_counts", "mol_offsets", "scatter_idxs",
-                     "gather_idxs", "atom_counts", "grads"):
+                     "gather_idxs", "atom_counts", "size_order", "grads"):
             t = getattr(self, name)
             if t is not None:
                 t.record_stream(cur)       # the memory was allocated on the feeder's stream
@@ -291,14 +323,11 @@ class DeviceFeeder:
             copied.record(self.stream)
             self._events[slot] = copied
             b.n_mols = n_mols
-            b.mol_atom_counts, b.mol_offsets = ops.mol_offsets(b.mol_idxs, n_mols)
-            b.scatter_idxs, b.gather_idxs, b.atom_counts = ops.ani_sort(b.atom_types)
             b.labels = mol_yts
             b.grads = None
             if mol_grads is not None:
                 b.grads = torch.from_numpy(np.ascontiguousarray(mol_grads, dtype=self.dtype)).to(self.device)
-            b.ready = torch.cuda.Event()
-            b.ready.record(self.stream)
+            b.finish_on_current_stream()          # the feeder's stream is current here
         return b
 
     def __iter__(self):

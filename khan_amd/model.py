@@ -113,6 +113,16 @@ class MoleculeNN:
         return (self.first_layer_kernel and self.dtype == torch.float32 and self.device.type == "cuda"
                 and self.layer_sizes[1] == 128 and len(self.layer_sizes) > 2 and self.activation_fn is celu)
 
+    def first_layer_transposed(self):
+        """The four first-layer weights transposed ([128, 384], k contiguous), as `ops.dense_first` takes them; kept
+        until a weight is written again."""
+        ws = [self.params[self.names[t][0][0]] for t in TYPE_MAP]
+        key = tuple((w.data_ptr(), w._version) for w in ws)
+        if getattr(self, "_wt_key", None) != key:
+            self._wt = [w.detach().t().contiguous() for w in ws]
+            self._wt_key = key
+        return self._wt
+
     def atom_outputs(self, atom_type_features, gather_idxs):
         """Per-type flat feature buckets -> one number per atom in the batch's atom order (nn.py:176-177)."""
         if self.fused_first_layer():
@@ -123,11 +133,14 @@ class MoleculeNN:
             # coordinates' gradient was asked for, and would form the weights' gradient, a second product, every time)
             par = (lambda k: self.params[k]) if self.weights_need_grad else (lambda k: self.params[k].detach())
             a1 = autograd.dense_first(atom_type_features, acs, [par(r[0]) for r in first],
-                                      [par(r[1]) for r in first], alpha=0.1)
+                                      [par(r[1]) for r in first], alpha=0.1,
+                                      weights_t=self.first_layer_transposed())
             outs = [self.atom_type_outputs(t, a1[t], first_layer_done=True) for t in range(4)]
         else:
             outs = [self.atom_type_outputs(t, f.reshape(-1, FEATURE_SIZE)) for t, f in enumerate(atom_type_features)]
-        return torch.cat(outs)[gather_idxs.long()]
+        # gather_idxs is a permutation: index_select's backward is a scatter-add, where indexing with [] sorts the
+        # indices first (a merge sort of n atoms in every backward pass)
+        return torch.index_select(torch.cat(outs), 0, gather_idxs.long())
 
 
 class AniModel:
@@ -181,8 +194,9 @@ class AniModel:
         xs, ys, zs = b.xs, b.ys, b.zs
         if need_grad:
             xs, ys, zs = (t.detach().clone().requires_grad_(True) for t in (xs, ys, zs))
-        acs = b.atom_counts.cpu().tolist()
-        feats = autograd.featurize(xs, ys, zs, b.atom_types, b.mol_offsets, b.mol_atom_counts, b.scatter_idxs, acs)
+        acs, order, classes = b.host_counts()
+        feats = autograd.featurize(xs, ys, zs, b.atom_types, b.mol_offsets, b.mol_atom_counts, b.scatter_idxs, acs,
+                                   order=order, size_classes=classes)
         atom_e = self.near.atom_outputs(feats, b.gather_idxs)
         energies = torch.zeros(b.n_mols, dtype=self.dtype, device=self.device)
         energies.index_add_(0, b.mol_idxs.long(), atom_e)                 # segment_sum over molecules
