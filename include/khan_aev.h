@@ -240,6 +240,20 @@ int khan_dense_first_f32(const float *const *rows_host4, const int32_t *acs_host
                          int32_t activation, float alpha, float *const *out_host4,
                          khan_stream_t stream);
 
+/* Any dense layer of the per-type networks, forward or on the way back (khan/model/nn.py:38-68 and its gradient
+ * with respect to the layer's input, which the reference leaves to TensorFlow's matmul gradient), one launch for
+ * the four types:
+ *     out_t[r, :] = act(in_t'[r, :] . W_t + b_t),   in_t' = in_t, or in_t .* CELU'(z) with CELU(z) = deriv_of_t.
+ * in_t [n_t, k], wt_t [n_out, k] (the summed index contiguous), bias_t [n_out] or bias_host4 = NULL, deriv_of_t
+ * [n_t, k] or deriv_of_host4 = NULL, out_t [n_t, n_out]; k a multiple of 32, n_out a multiple of 64; in, deriv_of and
+ * wt 16-byte aligned.  Forward of a layer with weights W [k, n_out]: wt = W transposed, bias, activation.  Data
+ * gradient of a layer with weights W [k_l, n_l] and CELU outputs h: in = d/dh [n_t, n_l], deriv_of = h, wt = W
+ * as it is (k = n_l, n_out = k_l), no bias, no activation.  float32 in, float32 accumulation on the matrix cores. */
+int khan_dense_f32(const float *const *rows_host4, const int32_t *n_host4, int32_t k, int32_t n_out,
+                   const float *const *wt_host4, const float *const *bias_host4, int32_t activation,
+                   float alpha, const float *const *deriv_of_host4, float *const *out_host4,
+                   khan_stream_t stream);
+
 /* Plain Coulomb sums, E_m = k sum_{i<j in m} q_i q_j / r_ij, and their gradients: the charge kernels with
  * the damping (1 - f_C) switched off and the constant chosen by the caller (k = 1 for charges in e and
  * distances in the unit the energy is wanted in).  No reference counterpart: khan's own op is the damped,

@@ -76,49 +76,61 @@ class _AniCharge(torch.autograd.Function):
         return None, None, None, ops.ani_charge_grad(*args), None, None
 
 
-class _DenseFirst(torch.autograd.Function):
-    """act(rows_t . W_t + b_t) for the four atom types through `ops.dense_first` (float32, width 128, CELU or no
-    activation).  Backward: plain matrix products; the activation's derivative comes from the saved outputs
-    (CELU: 1 for out >= 0, out / alpha + 1 = exp(z / alpha) below)."""
+class _Dense(torch.autograd.Function):
+    """act(in_t . W_t + b_t) for the four atom types through `ops.dense` (float32; CELU or no activation), forward on
+    the matrix-core kernel and the data gradient too: d/d in = (g .* act'(out)) . W^T, with the activation's derivative
+    taken from the saved outputs inside the kernel (CELU: 1 for out >= 0, out / alpha + 1 = exp(z / alpha) below)."""
 
     @staticmethod
-    def forward(ctx, acs_host, activation, alpha, weights_t, *tensors):
-        feats, ws, bs = tensors[0:4], tensors[4:8], tensors[8:12]
+    def forward(ctx, activation, alpha, weights_t, *tensors):
+        xs, ws, bs = tensors[0:4], tensors[4:8], tensors[8:12]
+        k = ws[0].shape[0]
         if weights_t is None:
             weights_t = [w.detach().t().contiguous() for w in ws]
-        outs = ops.dense_first([f.detach() for f in feats], acs_host, weights_t, [b.detach() for b in bs], activation, alpha)
-        ctx.save_for_backward(*feats, *ws, *outs)
+        outs = ops.dense([x.detach().reshape(-1, k) for x in xs], weights_t, [b.detach() for b in bs], activation, alpha)
+        ctx.save_for_backward(*xs, *ws, *outs)
         ctx.activation, ctx.alpha = activation, alpha
         return outs
 
     @staticmethod
     def backward(ctx, *gouts):
         saved = ctx.saved_tensors
-        feats, ws, outs = saved[0:4], saved[4:8], saved[8:12]
-        gf, gw, gb = [], [], []
-        for t in range(4):
-            g = gouts[t]
-            if g is None or outs[t].numel() == 0:
-                gf.append(torch.zeros_like(feats[t]) if ctx.needs_input_grad[4 + t] else None)
-                gw.append(torch.zeros_like(ws[t]) if ctx.needs_input_grad[8 + t] else None)
-                gb.append(torch.zeros(ws[t].shape[1], dtype=ws[t].dtype, device=ws[t].device) if ctx.needs_input_grad[12 + t] else None)
-                continue
-            if ctx.activation == ops.ACT_CELU:
-                # one elementwise kernel: CELU is ELU with input scale 1 / alpha, differentiated from its result
-                g = torch.ops.aten.elu_backward(g.contiguous(), ctx.alpha, 1.0, 1.0 / ctx.alpha, True, outs[t])
-            rows = feats[t].reshape(-1, ops.FEATURE_SIZE)
-            gf.append((g @ ws[t].t()).reshape(feats[t].shape) if ctx.needs_input_grad[4 + t] else None)
-            gw.append(rows.t() @ g if ctx.needs_input_grad[8 + t] else None)
-            gb.append(g.sum(dim=0) if ctx.needs_input_grad[12 + t] else None)
-        return (None, None, None, None) + tuple(gf) + tuple(gw) + tuple(gb)
+        xs, ws, outs = saved[0:4], saved[4:8], saved[8:12]
+        k, n_out = ws[0].shape
+        celu_act = ctx.activation == ops.ACT_CELU
+        gs = [torch.zeros_like(outs[t]) if gouts[t] is None else gouts[t].contiguous() for t in range(4)]
+        gx = (None,) * 4
+        if any(ctx.needs_input_grad[3:7]):
+            # one launch for the four types: in = g, the derivative from the saved activations, W as it is
+            gx = ops.dense(gs, [w.detach() for w in ws], None, ops.ACT_NONE, ctx.alpha, deriv_of=outs if celu_act else None)
+            gx = tuple(g.reshape(xs[t].shape) if ctx.needs_input_grad[3 + t] else None for t, g in enumerate(gx))
+        gw, gb = [None] * 4, [None] * 4
+        if any(ctx.needs_input_grad[7:15]):
+            for t in range(4):
+                g = gs[t]
+                if celu_act:     # CELU is ELU with input scale 1 / alpha, differentiated from its result
+                    g = torch.ops.aten.elu_backward(g, ctx.alpha, 1.0, 1.0 / ctx.alpha, True, outs[t])
+                if ctx.needs_input_grad[7 + t]:
+                    gw[t] = xs[t].reshape(-1, k).t() @ g
+                if ctx.needs_input_grad[11 + t]:
+                    gb[t] = g.sum(dim=0)
+        return (None, None, None) + tuple(gx) + tuple(gw) + tuple(gb)
+
+
+def dense(inputs, weights, biases, activation=ops.ACT_CELU, alpha=0.1, weights_t=None):
+    """Differentiable dense layer of the four atomic networks: four inputs ([n_t, k], or flat buckets of n_t * k), four
+    [k, n_out] weights, four [n_out] biases -> four [n_t, n_out] activations (float32; k a multiple of 32, n_out of 64).
+    `weights_t`: the four weights transposed ([n_out, k], contiguous), if the caller keeps them; otherwise they are
+    transposed here on every call."""
+    return _Dense.apply(int(activation), float(alpha), weights_t, *inputs, *weights, *biases)
 
 
 def dense_first(atom_type_features, acs_host, weights, biases, activation=ops.ACT_CELU, alpha=0.1, weights_t=None):
-    """Differentiable first dense layer of the four atomic networks: four flat feature buckets, four [384, 128]
-    weights, four [128] biases -> four [n_t, 128] activations (float32).  `weights_t`: the four weights transposed
-    ([128, 384], contiguous), if the caller keeps them; otherwise they are transposed here on every call."""
-    return _DenseFirst.apply([int(v) for v in acs_host], int(activation), float(alpha), weights_t,
-                             *atom_type_features, *weights, *biases)
+    """The first dense layer on the featurizer's four flat buckets: `dense` with k = 384."""
+    for f, c in zip(atom_type_features, acs_host):
+        if f.numel() != int(c) * ops.FEATURE_SIZE:
+            raise ValueError("a bucket of %d elements for %d atoms" % (f.numel(), int(c)))
+    return dense(atom_type_features, weights, biases, activation, alpha, weights_t)
 
 
 def featurize(xs, ys, zs, as_, mos, macs, sis, acs, order=None, size_classes=None):

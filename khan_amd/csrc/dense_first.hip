@@ -1,18 +1,23 @@
-// First dense layer of the per-type atomic networks, right behind the featurizer:
-//     out[r, :] = act(rows[r, :] . W + b),   rows [n, 384] feature rows of one atom type, W [384, 128], b [128]
-// (reference: khan/model/nn.py:38-68 -- tf.matmul + bias + activation per type -- with the CELU of
-// khan/model/activations.py:63-65 as activation, or none).  float32 in, float32 accumulation on the matrix cores
+// Dense layers of the per-type atomic networks on the matrix cores:
+//     out[r, :] = act(in'[r, :] . W + b),   in' = in, or in .* CELU'(value) taken from a layer's own activations,
+// for the four atom types in one launch (reference: khan/model/nn.py:38-68 -- tf.matmul + bias + activation per
+// type -- with the CELU of khan/model/activations.py:63-65 as activation, or none).  The first form is a layer's
+// forward pass (the first layer right behind the featurizer: in = the 384-wide feature rows); the second is the data
+// gradient of a layer on the way back (in = the gradient with respect to the layer's activations, W = the layer's
+// weights read the other way round, no bias, no activation).  float32 in, float32 accumulation
 // (v_mfma_f32_32x32x2_f32): the same arithmetic as a float32 matrix product, in another summation order.
 //
-// One workgroup of four wavefronts owns a 128-row x 128-column tile of the output of one type; every wavefront a
-// 64 x 64 quarter of it = 2 x 2 matrix-core blocks of 32 x 32, whose 64 accumulator registers stay in the lanes
-// for the whole K = 384 loop.  K is walked in chunks of 32: a chunk of the rows (128 x 32) and of the transposed
-// weights (128 x 32) is staged in LDS through registers, double buffered, so the global loads of chunk c+1 are in
-// flight while chunk c is multiplied.  In LDS both tiles are [row or column][k] with the k run padded from 32 to 36
-// floats: a lane reads four consecutive k of its row with one 16-byte read, conflict-free.  A matrix-core step
-// multiplies two k per block: the lower half of the wavefront supplies k = 8q + t, the upper half k = 8q + 4 + t
-// (t = 0..3 from one 16-byte read each), which covers every k of the chunk once -- a sum does not care about its order.
-// The four types are one launch: a workgroup finds its type and tile from the per-type tile counts.
+// One workgroup of four wavefronts owns a tile of 128 rows x kTileCols columns of the output of one type.  With 128
+// columns every wavefront has a 64 x 64 quarter of it = 2 x 2 matrix-core blocks of 32 x 32; with 64 columns (the third
+// layer's width) a 32 x 64 strip = 1 x 2 blocks.  The accumulators stay in the lanes for the whole K loop.  K is
+// walked in chunks of 32: a chunk of the rows (128 x 32) and of the transposed weights (kTileCols x 32) is staged in LDS
+// through registers, double buffered, so the global loads of chunk c+1 are in flight while chunk c is multiplied; the
+// multiplication by the activation's derivative happens in those registers.  In LDS both tiles are [row or column][k]
+// with the k run padded from 32 to 36 floats: a lane reads four consecutive k of its row with one 16-byte read,
+// conflict-free.  A matrix-core step multiplies two k per block: the lower half of the wavefront supplies k = 8q + t,
+// the upper half k = 8q + 4 + t (t = 0..3 from one 16-byte read each), which covers every k of the chunk once -- a
+// sum does not care about its order.  A workgroup finds its type, row tile and column tile from the per-type tile
+// counts; the column tiles of one row tile are neighbours in the grid, so the rows they share come from L2.
 #include "khan_internal.h"
 #include "khan_params.h"
 
@@ -20,8 +25,6 @@ namespace khan {
 
 namespace {
 
-constexpr int kDenseIn = kFeats;       // 384
-constexpr int kDenseOut = 128;
 constexpr int kTileRows = 128;
 constexpr int kChunk = 32;             // k per staging step
 constexpr int kPad = 36;               // floats per staged row: 32 + 4 (bank rotation for 16-byte reads)
@@ -30,139 +33,410 @@ typedef float v4 __attribute__((ext_vector_type(4)));
 typedef float v16 __attribute__((ext_vector_type(16)));
 
 struct DenseArgs {
-    const float* rows[4];      // [n_t, 384] per type
-    const float* wt[4];        // [128, 384]: the layer's weights transposed (k contiguous)
-    const float* bias[4];      // [128]
-    float* out[4];             // [n_t, 128]
+    const float* rows[4];      // [n_t, k] per type
+    const float* deriv[4];     // [n_t, k] activations whose CELU derivative multiplies the rows, or null
+    const float* wt[4];        // [n_out, k]: the weights with the summed index contiguous
+    const float* bias[4];      // [n_out], or null
+    float* out[4];             // [n_t, n_out]
     int n[4];                  // rows per type
-    int tile_end[4];           // running sum of the per-type tile counts
+    int tile_end[4];           // running sum of the per-type (row tile x column tile) counts
+    int k, n_out, col_tiles;
 };
 
+template <int kTileCols>
 struct __align__(16) DenseLds {
     float a[2][kTileRows][kPad];       // rows tile, double buffered
-    float b[2][kDenseOut][kPad];       // transposed-weights tile
+    float b[2][kTileCols][kPad];       // transposed-weights tile
 };
 
-template <bool kCelu>
-__global__ __launch_bounds__(256) void dense_first_kernel(DenseArgs args, float alpha, float inv_alpha)
+// kK: the summed width when it is one of the network's (384, 128, 64: the chunk loop is then known to the compiler),
+// 0 for any other multiple of 32 (taken from the arguments)
+template <int kTileCols, int kK, bool kCelu, bool kDeriv>
+__global__ __launch_bounds__(256) void dense_kernel(DenseArgs args, float alpha, float inv_alpha)
 {
-    __shared__ DenseLds S;
+    constexpr int kWaveRows = kTileCols == 128 ? 64 : 32;      // rows of a wavefront's part of the tile
+    constexpr int kBI = kWaveRows / 32;                        // its matrix-core blocks down (2 or 1); across: 2
+    constexpr int kBPieces = kTileCols * (kChunk / 4) / 256;   // 16-byte pieces of the weight chunk per thread (4 or 2)
+    __shared__ DenseLds<kTileCols> S;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    // type and tile of this workgroup
+    // type, row tile and column tile of this workgroup
     const int blk = blockIdx.x;
     const int t = (blk >= args.tile_end[0]) + (blk >= args.tile_end[1]) + (blk >= args.tile_end[2]);
-    const int tile = blk - (t == 0 ? 0 : args.tile_end[t - 1]);
-    const int n = args.n[t];
+    const int rel = blk - (t == 0 ? 0 : args.tile_end[t - 1]);
+    const int tile = rel / args.col_tiles, ctile = rel - tile * args.col_tiles;
+    const int n = args.n[t], K = kK > 0 ? kK : args.k;
     const float* __restrict__ rows = args.rows[t];
-    const float* __restrict__ wt = args.wt[t];
-    const int row0 = tile * kTileRows;
+    const float* __restrict__ deriv = args.deriv[t];
+    const float* __restrict__ wt = args.wt[t] + static_cast<size_t>(ctile) * kTileCols * K;
+    const int row0 = tile * kTileRows, col0 = ctile * kTileCols;
 
-    // staging: a chunk of each tile is 128 x 32 floats = 1,024 pieces of 16 bytes, four per thread:
-    // piece p = tid + 256 u -> tile row p / 8, k offset (p % 8) * 4
-    v4 ra[4], rb[4];
+    // staging: a chunk of the rows tile is 128 x 32 floats = 1,024 pieces of 16 bytes, four per thread:
+    // piece p = tid + 256 u -> tile row p / 8, k offset (p % 8) * 4; the weight chunk likewise (kTileCols rows)
+    v4 ra[4], rb[kBPieces];
     auto fetch = [&](int chunk) {
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int p = tid + 256 * u;
             const int r = p >> 3, k4 = (p & 7) << 2;
-            const int gr = row0 + r;
-            ra[u] = v4{0.f, 0.f, 0.f, 0.f};
-            if (gr < n) ra[u] = *reinterpret_cast<const v4*>(rows + static_cast<size_t>(gr) * kDenseIn + chunk * kChunk + k4);
-            rb[u] = *reinterpret_cast<const v4*>(wt + static_cast<size_t>(r) * kDenseIn + chunk * kChunk + k4);
+            // rows past the end of the type read its last row: their products are never stored, and a load that is
+            // not under a condition needs no merge with a default afterwards (which would wait for it on the spot)
+            const int gr = min(row0 + r, n - 1);
+            const size_t at = static_cast<size_t>(gr) * K + chunk * kChunk + k4;
+            ra[u] = *reinterpret_cast<const v4*>(rows + at);
+            if constexpr (kDeriv) {
+                // CELU'(z) from CELU(z) = h: 1 for h >= 0, exp(z / alpha) = h / alpha + 1 below
+                const v4 h = *reinterpret_cast<const v4*>(deriv + at);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ra[u][e] *= h[e] >= 0.f ? 1.0f : fmaf(h[e], inv_alpha, 1.0f);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kBPieces; ++u) {
+            const int p = tid + 256 * u;
+            const int r = p >> 3, k4 = (p & 7) << 2;
+            rb[u] = *reinterpret_cast<const v4*>(wt + static_cast<size_t>(r) * K + chunk * kChunk + k4);
         }
     };
     auto stage = [&](int buf) {
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int p = tid + 256 * u;
-            const int r = p >> 3, k4 = (p & 7) << 2;
-            *reinterpret_cast<v4*>(&S.a[buf][r][k4]) = ra[u];
-            *reinterpret_cast<v4*>(&S.b[buf][r][k4]) = rb[u];
+            *reinterpret_cast<v4*>(&S.a[buf][p >> 3][(p & 7) << 2]) = ra[u];
+        }
+#pragma unroll
+        for (int u = 0; u < kBPieces; ++u) {
+            const int p = tid + 256 * u;
+            *reinterpret_cast<v4*>(&S.b[buf][p >> 3][(p & 7) << 2]) = rb[u];
         }
     };
 
-    // this wavefront's 64 x 64 quarter: rows wr*64.., columns wc*64..; two blocks of 32 each way
-    const int wr = wave >> 1, wc = wave & 1;
+    // this wavefront's part: 128 columns -> rows wr*64.., columns wc*64..; 64 columns -> rows wave*32.., all columns
+    const int wr = kTileCols == 128 ? (wave >> 1) : wave, wc = kTileCols == 128 ? (wave & 1) : 0;
     const int l32 = lane & 31, half = lane >> 5;
-    v16 acc[2][2];
+    v16 acc[kBI][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < kBI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    constexpr int kChunks = kDenseIn / kChunk;      // 12
+    const int chunks = K / kChunk;
     fetch(0);
     stage(0);
     __syncthreads();
-    for (int c = 0; c < kChunks; ++c) {
+    for (int c = 0; c < chunks; ++c) {
         const int buf = c & 1;
-        if (c + 1 < kChunks) fetch(c + 1);          // in flight while this chunk is multiplied
+        if (c + 1 < chunks) fetch(c + 1);          // in flight while this chunk is multiplied
 #pragma unroll
         for (int q = 0; q < kChunk / 8; ++q) {
             // four consecutive k of this lane's row / column: k = 8q + 4 half + (0..3)
-            v4 av[2], bv[2];
+            v4 av[kBI], bv[2];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) av[i] = *reinterpret_cast<const v4*>(&S.a[buf][wr * 64 + i * 32 + l32][q * 8 + half * 4]);
+            for (int i = 0; i < kBI; ++i) av[i] = *reinterpret_cast<const v4*>(&S.a[buf][wr * kWaveRows + i * 32 + l32][q * 8 + half * 4]);
 #pragma unroll
             for (int j = 0; j < 2; ++j) bv[j] = *reinterpret_cast<const v4*>(&S.b[buf][wc * 64 + j * 32 + l32][q * 8 + half * 4]);
 #pragma unroll
             for (int e = 0; e < 4; ++e)
 #pragma unroll
-                for (int i = 0; i < 2; ++i)
+                for (int i = 0; i < kBI; ++i)
 #pragma unroll
                     for (int j = 0; j < 2; ++j)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i][e], bv[j][e], acc[i][j], 0, 0, 0);
         }
-        if (c + 1 < kChunks) {
+        if (c + 1 < chunks) {
             stage(buf ^ 1);                          // the other buffer: nobody reads it during this chunk
             __syncthreads();
         }
     }
 
     // epilogue: bias, activation, store.  Accumulator e of block (i, j) is output row
-    // wr*64 + i*32 + 8 (e / 4) + 4 half + e % 4, column wc*64 + j*32 + l32.
+    // wr*kWaveRows + i*32 + 8 (e / 4) + 4 half + e % 4, column wc*64 + j*32 + l32 of the tile.
+    // The bias is waited for once, before the first store: a wait inside a conditional store would also wait for
+    // the stores before it (loads and stores share one counter), one by one -- 64 stores, each at full latency.
     const float* __restrict__ bias = args.bias[t];
     float* __restrict__ out = args.out[t];
+    const int n_out = args.n_out;
+    float bj[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        const int col = wc * 64 + j * 32 + l32;
-        const float bj = bias[col];
+        bj[j] = bias ? bias[col0 + wc * 64 + j * 32 + l32] : 0.f;
+        asm volatile("" : "+v"(bj[j]));          // the bias is in its register from here on: the one wait happens here
+    }
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+    for (int j = 0; j < 2; ++j) {
+        const int col = col0 + wc * 64 + j * 32 + l32;
+#pragma unroll
+        for (int i = 0; i < kBI; ++i) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int r = row0 + wr * 64 + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
-                float v = acc[i][j][e] + bj;
+                const int r = row0 + wr * kWaveRows + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                float v = acc[i][j][e] + bj[j];
                 if (kCelu) v = v >= 0.f ? v : alpha * (__expf(v * inv_alpha) - 1.0f);
-                if (r < n) out[static_cast<size_t>(r) * kDenseOut + col] = v;
+                if (r < n) out[static_cast<size_t>(r) * n_out + col] = v;
             }
         }
     }
 }
 
+// The same product for the network's own widths (kK = 384, 128 or 64: an even number of chunks), as a pipeline that
+// does not drain between tiles.  The grid is as many workgroups as stay resident; a workgroup takes tiles blk,
+// blk + grid, ... and walks their chunks as one sequence of steps.  At step s it issues the global loads of step s + 2
+// into one of two register sets, multiplies step s out of LDS, then stages the registers of step s + 1 -- loaded a
+// whole step ago -- into the other LDS buffer.  So the first chunk of the next tile arrives while this tile is still
+// being multiplied, and its epilogue's stores drain under the next tile's products: with K = 128 a tile is only four
+// chunks long, and starting every tile cold cost a third of the kernel.
+template <int kTileCols, int kK, bool kCelu, bool kDeriv>
+__global__ __launch_bounds__(256) void dense_pipe_kernel(DenseArgs args, int total_tiles, float alpha, float inv_alpha)
+{
+    constexpr int kWaveRows = kTileCols == 128 ? 64 : 32;
+    constexpr int kBI = kWaveRows / 32;
+    constexpr int kBPieces = kTileCols * (kChunk / 4) / 256;
+    constexpr int kChunks = kK / kChunk;
+    static_assert(kChunks % 2 == 0, "two register sets alternate by step: a tile must be an even number of steps");
+    __shared__ DenseLds<kTileCols> S;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int stride = gridDim.x;
+
+    struct Cursor {                 // where the next loads come from: a tile (or none) and a chunk of it
+        const float* rows;
+        const float* deriv;
+        const float* wt;
+        int row0, n, chunk, tile;
+        bool live;
+    };
+    struct TileOut {                // what the epilogue of a tile needs
+        float* out;
+        int row0, col0, n;
+        float bj[2];                // the bias of this lane's two columns, loaded when the tile starts
+    };
+    auto decode_loads = [&](int id, Cursor& c) {
+        const int t = (id >= args.tile_end[0]) + (id >= args.tile_end[1]) + (id >= args.tile_end[2]);
+        const int rel = id - (t == 0 ? 0 : args.tile_end[t - 1]);
+        const int tile = rel / args.col_tiles, ctile = rel - tile * args.col_tiles;
+        c.rows = args.rows[t];
+        c.deriv = args.deriv[t];
+        c.wt = args.wt[t] + static_cast<size_t>(ctile) * kTileCols * kK;
+        c.row0 = tile * kTileRows;
+        c.n = args.n[t];
+    };
+    auto decode_out = [&](int id, TileOut& o) {
+        const int t = (id >= args.tile_end[0]) + (id >= args.tile_end[1]) + (id >= args.tile_end[2]);
+        const int rel = id - (t == 0 ? 0 : args.tile_end[t - 1]);
+        const int tile = rel / args.col_tiles, ctile = rel - tile * args.col_tiles;
+        o.out = args.out[t];
+        o.row0 = tile * kTileRows;
+        o.col0 = ctile * kTileCols;
+        o.n = args.n[t];
+        const float* bias = args.bias[t];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) o.bj[j] = bias ? bias[o.col0 + (kTileCols == 128 ? (wave & 1) : 0) * 64 + j * 32 + (lane & 31)] : 0.f;
+    };
+
+    v4 ra[2][4], rb[2][kBPieces];
+    auto fetch = [&](const Cursor& c, v4 (&a)[4], v4 (&b)[kBPieces]) {
+        if (!c.live) return;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int p = tid + 256 * u;
+            const int r = p >> 3, k4 = (p & 7) << 2;
+            const int gr = min(c.row0 + r, c.n - 1);       // past the end: the last row again, never stored
+            const size_t at = static_cast<size_t>(gr) * kK + c.chunk * kChunk + k4;
+            a[u] = *reinterpret_cast<const v4*>(c.rows + at);
+            if constexpr (kDeriv) {
+                const v4 h = *reinterpret_cast<const v4*>(c.deriv + at);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) a[u][e] *= h[e] >= 0.f ? 1.0f : fmaf(h[e], inv_alpha, 1.0f);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kBPieces; ++u) {
+            const int p = tid + 256 * u;
+            const int r = p >> 3, k4 = (p & 7) << 2;
+            b[u] = *reinterpret_cast<const v4*>(c.wt + static_cast<size_t>(r) * kK + c.chunk * kChunk + k4);
+        }
+    };
+    auto stage = [&](int buf, const v4 (&a)[4], const v4 (&b)[kBPieces]) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int p = tid + 256 * u;
+            *reinterpret_cast<v4*>(&S.a[buf][p >> 3][(p & 7) << 2]) = a[u];
+        }
+#pragma unroll
+        for (int u = 0; u < kBPieces; ++u) {
+            const int p = tid + 256 * u;
+            *reinterpret_cast<v4*>(&S.b[buf][p >> 3][(p & 7) << 2]) = b[u];
+        }
+    };
+
+    const int wr = kTileCols == 128 ? (wave >> 1) : wave, wc = kTileCols == 128 ? (wave & 1) : 0;
+    const int l32 = lane & 31, half = lane >> 5;
+    v16 acc[kBI][2];
+    auto clear = [&]() {
+#pragma unroll
+        for (int i = 0; i < kBI; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    };
+    auto multiply = [&](int buf) {
+#pragma unroll
+        for (int q = 0; q < kChunk / 8; ++q) {
+            v4 av[kBI], bv[2];
+#pragma unroll
+            for (int i = 0; i < kBI; ++i) av[i] = *reinterpret_cast<const v4*>(&S.a[buf][wr * kWaveRows + i * 32 + l32][q * 8 + half * 4]);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) bv[j] = *reinterpret_cast<const v4*>(&S.b[buf][wc * 64 + j * 32 + l32][q * 8 + half * 4]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int i = 0; i < kBI; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i][e], bv[j][e], acc[i][j], 0, 0, 0);
+        }
+    };
+    auto epilogue = [&](TileOut& o) {
+        // the bias (loaded when the tile started) is waited for once, before the first store (see dense_kernel)
+        const int n_out = args.n_out;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) asm volatile("" : "+v"(o.bj[j]));
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int col = o.col0 + wc * 64 + j * 32 + l32;
+#pragma unroll
+            for (int i = 0; i < kBI; ++i) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int r = o.row0 + wr * kWaveRows + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                    float v = acc[i][j][e] + o.bj[j];
+                    if (kCelu) v = v >= 0.f ? v : alpha * (__expf(v * inv_alpha) - 1.0f);
+                    if (r < o.n) o.out[static_cast<size_t>(r) * n_out + col] = v;
+                }
+            }
+        }
+    };
+
+    // the load cursor runs two steps ahead of the multiplication
+    Cursor cu;
+    cu.tile = blockIdx.x;
+    cu.chunk = 0;
+    cu.live = cu.tile < total_tiles;
+    if (!cu.live) return;
+    decode_loads(cu.tile, cu);
+    auto advance = [&]() {          // one step further
+        if (++cu.chunk == kChunks) {
+            cu.chunk = 0;
+            cu.tile += stride;
+            cu.live = cu.tile < total_tiles;
+            if (cu.live) decode_loads(cu.tile, cu);
+        }
+    };
+    // prologue: step 0 into LDS buffer 0, step 1 into register set 1
+    fetch(cu, ra[0], rb[0]);
+    advance();
+    fetch(cu, ra[1], rb[1]);
+    advance();
+    stage(0, ra[0], rb[0]);
+    __syncthreads();
+    clear();
+    for (int tile = blockIdx.x; tile < total_tiles; tile += stride) {
+        const bool more = tile + stride < total_tiles;
+        TileOut cur;
+        decode_out(tile, cur);
+        for (int c = 0; c < kChunks; c += 2) {
+            // even step: LDS buffer 0 is multiplied, set 0 loads two steps ahead, set 1 (one step ahead) is staged
+            fetch(cu, ra[0], rb[0]);
+            advance();
+            multiply(0);
+            stage(1, ra[1], rb[1]);
+            __syncthreads();
+            // odd step
+            fetch(cu, ra[1], rb[1]);
+            advance();
+            multiply(1);
+            if (c + 2 < kChunks || more) {           // something follows: the first chunk of the next tile, at a tile's end
+                stage(0, ra[0], rb[0]);
+                __syncthreads();
+            }
+        }
+        epilogue(cur);
+        clear();
+    }
+}
+
+template <int kTileCols, int kK>
+hipError_t launch_tiles_k(const DenseArgs& a, int run, bool celu, bool deriv, float alpha, hipStream_t stream)
+{
+    const float inv_alpha = 1.0f / alpha;
+    // the widths of the reference's default network 384-128-128-64-1, forward and backward
+    if constexpr ((kTileCols == 128 && kK > 0) || (kTileCols == 64 && kK == 128)) {
+        // the pipelined kernel: as many workgroups as stay resident (two per CU at 72 KB of LDS, three at 54 KB)
+        int device = 0, cus = 0;
+        if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0)
+            cus = 256;
+        const int resident = cus * (kTileCols == 128 ? 2 : 2);
+        const dim3 pgrid(static_cast<unsigned>(run < resident ? run : resident)), pblock(256);
+        if (celu && !deriv) dense_pipe_kernel<kTileCols, kK, true, false><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
+        else if (!celu && !deriv) dense_pipe_kernel<kTileCols, kK, false, false><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
+        else if (!celu && deriv) dense_pipe_kernel<kTileCols, kK, false, true><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
+        else dense_pipe_kernel<kTileCols, kK, true, true><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
+        return hipGetLastError();
+    }
+    const dim3 grid(static_cast<unsigned>(run)), block(256);
+    if (celu && !deriv) dense_kernel<kTileCols, 0, true, false><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
+    else if (!celu && !deriv) dense_kernel<kTileCols, 0, false, false><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
+    else if (!celu && deriv) dense_kernel<kTileCols, 0, false, true><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
+    else dense_kernel<kTileCols, 0, true, true><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
+    return hipGetLastError();
+}
+
+template <int kTileCols>
+hipError_t launch_tiles(const DenseArgs& a, int run, bool celu, bool deriv, float alpha, hipStream_t stream)
+{
+    if (a.k == 384) return launch_tiles_k<kTileCols, 384>(a, run, celu, deriv, alpha, stream);
+    if (a.k == 128) return launch_tiles_k<kTileCols, 128>(a, run, celu, deriv, alpha, stream);
+    if (a.k == 64) return launch_tiles_k<kTileCols, 64>(a, run, celu, deriv, alpha, stream);
+    return launch_tiles_k<kTileCols, 0>(a, run, celu, deriv, alpha, stream);
+}
+
 }  // namespace
+
+// k: a multiple of 32; n_out: a multiple of 64.  bias and deriv_of may be null (as arrays, or entry by entry).
+hipError_t launch_dense(const float* const rows[4], const int32_t n[4], int32_t k, int32_t n_out,
+                        const float* const wt[4], const float* const bias[4], bool celu, float alpha,
+                        const float* const deriv_of[4], float* const out[4], hipStream_t stream)
+{
+    DenseArgs a;
+    const int tile_cols = (n_out % 128 == 0) ? 128 : 64;
+    a.k = k;
+    a.n_out = n_out;
+    a.col_tiles = n_out / tile_cols;
+    int64_t run = 0;
+    bool deriv = false;
+    for (int t = 0; t < 4; ++t) {
+        a.rows[t] = rows[t];
+        a.deriv[t] = deriv_of ? deriv_of[t] : nullptr;
+        a.wt[t] = wt[t];
+        a.bias[t] = bias ? bias[t] : nullptr;
+        a.out[t] = out[t];
+        a.n[t] = n[t];
+        if (n[t] > 0 && a.deriv[t]) deriv = true;
+        run += static_cast<int64_t>((n[t] + kTileRows - 1) / kTileRows) * a.col_tiles;
+        a.tile_end[t] = static_cast<int>(run);
+    }
+    if (run == 0) return hipSuccess;
+    if (run > INT32_MAX) return hipErrorInvalidValue;
+    if (tile_cols == 128) return launch_tiles<128>(a, static_cast<int>(run), celu, deriv, alpha, stream);
+    return launch_tiles<64>(a, static_cast<int>(run), celu, deriv, alpha, stream);
+}
 
 hipError_t launch_dense_first(const float* const rows[4], const int32_t n[4], const float* const wt[4],
                               const float* const bias[4], bool celu, float alpha, float* const out[4],
                               hipStream_t stream)
 {
-    DenseArgs a;
-    int run = 0;
-    for (int t = 0; t < 4; ++t) {
-        a.rows[t] = rows[t];
-        a.wt[t] = wt[t];
-        a.bias[t] = bias[t];
-        a.out[t] = out[t];
-        a.n[t] = n[t];
-        run += (n[t] + kTileRows - 1) / kTileRows;
-        a.tile_end[t] = run;
-    }
-    if (run == 0) return hipSuccess;
-    if (celu) dense_first_kernel<true><<<dim3(static_cast<unsigned>(run)), dim3(256), 0, stream>>>(a, alpha, 1.0f / alpha);
-    else dense_first_kernel<false><<<dim3(static_cast<unsigned>(run)), dim3(256), 0, stream>>>(a, alpha, 1.0f);
-    return hipGetLastError();
+    return launch_dense(rows, n, kFeats, 128, wt, bias, celu, alpha, nullptr, out, stream);
 }
 
 }  // namespace khan

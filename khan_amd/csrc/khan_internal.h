@@ -97,6 +97,9 @@ hipError_t launch_zero(T* a, int64_t n, hipStream_t stream);
 
 // ---- first dense layer behind the featurizer: out_t = act(rows_t . W_t + b_t) for the four types, float32 ----
 // rows[t]: [n[t], 384]; wt[t]: [128, 384] (the weights transposed); bias[t]: [128]; out[t]: [n[t], 128]
+hipError_t launch_dense(const float* const rows[4], const int32_t n[4], int32_t k, int32_t n_out,
+                        const float* const wt[4], const float* const bias[4], bool celu, float alpha,
+                        const float* const deriv_of[4], float* const out[4], hipStream_t stream);
 hipError_t launch_dense_first(const float* const rows[4], const int32_t n[4], const float* const wt[4],
                               const float* const bias[4], bool celu, float alpha, float* const out[4],
                               hipStream_t stream);

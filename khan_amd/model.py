@@ -6,8 +6,10 @@ save_numpy / load_numpy (451-499), predict (655-678), coordinate_gradients (580-
 features -> per-type networks -> gather -> segment_sum (+ ani_charge) of lines 306-385.
 
 The featurizer, its gradient and the charge energy are the HIP kernels of this package (through
-`khan_amd.autograd`).  The first dense layer (float32, width 128, CELU) runs in this package's matrix-core kernel
-right behind the featurizer (`ops.dense_first`); the other layers are plain matrix products: PyTorch's (rocBLAS).  Parameter
+`khan_amd.autograd`).  In float32 the dense layers with CELU (all but the last of the reference's default network) run in
+this package's matrix-core kernel (`ops.dense`: bias and activation in the product's epilogue, the activation's
+derivative in the prologue of the data gradient), the first one right behind the featurizer; the last layer and every
+float64 layer are plain matrix products: PyTorch's (rocBLAS).  Parameter
 names are the reference's TensorFlow variable names, `<prefix>W_<type>_<in>x<out>_l<k>:0` and
 `<prefix>b_...` (nn.py:41-60), so a checkpoint written by the reference's `save_numpy` loads unchanged;
 whatever else such a file holds (optimizer slots, learning rate, moving averages) is ignored.
@@ -74,7 +76,7 @@ class MoleculeNN:
     def __init__(self, layer_sizes=DEFAULT_LAYERS, activation_fn=celu, dtype=torch.float32, device="cpu",
                  prefix="near_", seed=None, first_layer_kernel=True):
         self.first_layer_kernel = bool(first_layer_kernel)
-        self.weights_need_grad = False      # set it to differentiate through the first layer's weights (training)
+        self.weights_need_grad = False      # set it to differentiate through the kernel layers' weights (training)
         layer_sizes = tuple(int(v) for v in layer_sizes)
         if layer_sizes[-1] != 1:
             raise ValueError("the last layer must have size 1")
@@ -94,48 +96,57 @@ class MoleculeNN:
     def parameters(self):
         return [self.params[k] for k in self.params]
 
-    def atom_type_outputs(self, type_idx, feats, first_layer_done=False):
-        """[n_t, 384] feature rows of one type -> [n_t] network outputs (`first_layer_done`: `feats` are the first
-        layer's activations already)."""
+    def atom_type_outputs(self, type_idx, feats, layers_done=0):
+        """[n_t, 384] feature rows of one type -> [n_t] network outputs (`layers_done`: `feats` are the activations of
+        that many leading layers already)."""
         rows = self.names[TYPE_MAP[type_idx]]
         a = feats
         for k, (wn, bn, _, _) in enumerate(rows):
-            if first_layer_done and k == 0:
+            if k < layers_done:
                 continue
             a = torch.addmm(self.params[bn], a, self.params[wn])
             if k != len(rows) - 1:
                 a = self.activation_fn(a)
         return a.reshape(-1)
 
-    def fused_first_layer(self):
-        """True when the first layer can run in this package's matrix-core kernel (`ops.dense_first`): float32 on the
-        GPU, width 128, CELU with its default alpha, at least two layers."""
-        return (self.first_layer_kernel and self.dtype == torch.float32 and self.device.type == "cuda"
-                and self.layer_sizes[1] == 128 and len(self.layer_sizes) > 2 and self.activation_fn is celu)
-
-    def first_layer_transposed(self):
-        """The four first-layer weights transposed ([128, 384], k contiguous), as `ops.dense_first` takes them; kept
-        until a weight is written again."""
-        ws = [self.params[self.names[t][0][0]] for t in TYPE_MAP]
+    def layer_transposed(self, k):
+        """The four weights of layer k transposed ([out, in], the summed index contiguous), as `ops.dense` takes them;
+        kept until a weight is written again."""
+        ws = [self.params[self.names[t][k][0]] for t in TYPE_MAP]
         key = tuple((w.data_ptr(), w._version) for w in ws)
-        if getattr(self, "_wt_key", None) != key:
-            self._wt = [w.detach().t().contiguous() for w in ws]
-            self._wt_key = key
-        return self._wt
+        cache = self.__dict__.setdefault("_wt_cache", {})
+        if k not in cache or cache[k][0] != key:
+            cache[k] = (key, [w.detach().t().contiguous() for w in ws])
+        return cache[k][1]
+
+    def kernel_layers(self):
+        """How many leading layers run in this package's matrix-core kernel (`ops.dense`): float32 on the GPU, CELU
+        with its default alpha, input width a multiple of 32 and output width a multiple of 64 -- for the reference's
+        default network 384-128-128-64-1 all but the last."""
+        if not (self.first_layer_kernel and self.dtype == torch.float32 and self.device.type == "cuda"
+                and self.activation_fn is celu):
+            return 0
+        n = 0
+        for x, y in zip(self.layer_sizes[:-2], self.layer_sizes[1:-1]):      # the last layer has no activation
+            if x % 32 or y % 64:
+                break
+            n += 1
+        return n
 
     def atom_outputs(self, atom_type_features, gather_idxs):
         """Per-type flat feature buckets -> one number per atom in the batch's atom order (nn.py:176-177)."""
-        if self.fused_first_layer():
+        nk = self.kernel_layers()
+        if nk > 0:
             from . import autograd
-            acs = [f.numel() // FEATURE_SIZE for f in atom_type_features]
-            first = [self.names[t][0] for t in TYPE_MAP]
             # inference: the weights are constants here (a custom autograd function cannot tell that only the
             # coordinates' gradient was asked for, and would form the weights' gradient, a second product, every time)
             par = (lambda k: self.params[k]) if self.weights_need_grad else (lambda k: self.params[k].detach())
-            a1 = autograd.dense_first(atom_type_features, acs, [par(r[0]) for r in first],
-                                      [par(r[1]) for r in first], alpha=0.1,
-                                      weights_t=self.first_layer_transposed())
-            outs = [self.atom_type_outputs(t, a1[t], first_layer_done=True) for t in range(4)]
+            a = atom_type_features
+            for k in range(nk):
+                rows = [self.names[t][k] for t in TYPE_MAP]
+                a = autograd.dense(a, [par(r[0]) for r in rows], [par(r[1]) for r in rows], alpha=0.1,
+                                   weights_t=self.layer_transposed(k))
+            outs = [self.atom_type_outputs(t, a[t], layers_done=nk) for t in range(4)]
         else:
             outs = [self.atom_type_outputs(t, f.reshape(-1, FEATURE_SIZE)) for t, f in enumerate(atom_type_features)]
         # gather_idxs is a permutation: index_select's backward is a scatter-add, where indexing with [] sorts the

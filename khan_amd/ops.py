@@ -292,6 +292,47 @@ def coulomb_grad(xs, ys, zs, qs, mos, macs, grads, k=1.0):
 ACT_NONE, ACT_CELU = 0, 1
 
 
+def dense(inputs, weights_nk, biases=None, activation=ACT_NONE, alpha=0.1, deriv_of=None):
+    """A dense layer of the four atomic networks, forward or on the way back, float32, one launch:
+    -> four [n_t, n_out] tensors act(in_t' . W_t + b_t), with in_t' = inputs[t] ([n_t, k]) or, with `deriv_of`, inputs[t]
+    times the CELU derivative taken from the activations deriv_of[t] ([n_t, k]).  `weights_nk[t]` is [n_out, k]
+    (the summed index contiguous): a layer's weights transposed for its forward pass, the weights as they are for
+    its data gradient.  k a multiple of 32, n_out a multiple of 64."""
+    lib = _lib.load()
+    n_out, k = (int(v) for v in weights_nk[0].shape)
+    rows, ders, wts, bs, outs, ns = [], [], [], [], [], []
+
+    def matrix(x, name):
+        if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dtype != torch.float32:
+            raise TypeError("%s must be a float32 CUDA tensor" % name)
+        if x.dim() != 2 or x.shape[1] != k or not x.is_contiguous():
+            raise ValueError("%s must be a contiguous [n, %d] tensor, got %s" % (name, k, tuple(x.shape)))
+        return x
+
+    for t in range(4):
+        r = matrix(inputs[t], "inputs[%d]" % t)
+        w = weights_nk[t]
+        if tuple(w.shape) != (n_out, k) or w.dtype != torch.float32 or not w.is_contiguous() or not w.is_cuda:
+            raise ValueError("weights_nk[%d] must be a contiguous float32 CUDA tensor of shape [%d, %d]" % (t, n_out, k))
+        if deriv_of is not None:
+            d = matrix(deriv_of[t], "deriv_of[%d]" % t)
+            if d.shape[0] != r.shape[0]:
+                raise ValueError("deriv_of[%d] must be shaped like inputs[%d]" % (t, t))
+            ders.append(d)
+        if biases is not None:
+            b = _dev(biases[t], torch.float32, "bias")
+            if b.numel() != n_out:
+                raise ValueError("bias %d must have %d elements" % (t, n_out))
+            bs.append(b)
+        rows.append(r); wts.append(w); ns.append(int(r.shape[0]))
+        outs.append(torch.empty((r.shape[0], n_out), dtype=torch.float32, device=r.device))
+    arr = lambda ts: (ctypes.c_void_p * 4)(*[t.data_ptr() if t.numel() else None for t in ts])
+    _lib.check(lib.khan_dense_f32(arr(rows), (ctypes.c_int32 * 4)(*ns), k, n_out, arr(wts),
+                                  arr(bs) if biases is not None else None, int(activation), float(alpha),
+                                  arr(ders) if deriv_of is not None else None, arr(outs), _stream()))
+    return tuple(outs)
+
+
 def dense_first(atom_type_features, acs, weights_t, biases, activation=ACT_CELU, alpha=0.1):
     """First dense layer of the four atomic networks on the featurizer's buckets, float32, one launch:
     -> four [acs[t], 128] tensors act(rows_t . W_t + b_t).  `weights_t[t]` is W_t TRANSPOSED, [128, 384]."""

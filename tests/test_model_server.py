@@ -315,6 +315,53 @@ def test_first_dense_layer_kernel_matches_the_oracle(activation):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("k,n_out", [(128, 128), (128, 64), (64, 128), (128, 384), (384, 128)])
+def test_dense_kernel_shapes_forward_and_data_gradient(k, n_out):
+    """khan_dense_f32 for every (input width, output width) the default network 384-128-128-64-1 needs, forward
+    (bias + CELU) and as the data gradient of a layer (rows times CELU' taken from saved activations, weights read the
+    other way round): against float64 numpy, row counts on and off the 128-row tile, an empty type."""
+    from khan_amd import ops
+    dev = "cuda:0"
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a.astype(np.float32))).to(dev)
+    rng = np.random.default_rng(k * 1000 + n_out)
+    ns = [0, 1, 128, 300]
+    xs = [rng.standard_normal((n, k)) for n in ns]
+    hs = [rng.standard_normal((n, k)) * 0.2 for n in ns]           # activations the derivative is taken from
+    Wt = [rng.standard_normal((n_out, k)) * (2.0 / (k + n_out)) ** 0.5 for _ in range(4)]
+    bs = [rng.standard_normal(n_out) * 0.1 for _ in range(4)]
+    f32 = lambda a: a.astype(np.float32).astype(np.float64)
+    fwd = ops.dense([d(x) for x in xs], [d(w) for w in Wt], [d(v) for v in bs], ops.ACT_CELU, 0.1)
+    lin = ops.dense([d(x) for x in xs], [d(w) for w in Wt], None, ops.ACT_NONE, 0.1)
+    bwd = ops.dense([d(x) for x in xs], [d(w) for w in Wt], None, ops.ACT_NONE, 0.1, deriv_of=[d(h) for h in hs])
+    for t in range(4):
+        x, h, w, b_ = f32(xs[t]), f32(hs[t]), f32(Wt[t]), f32(bs[t])
+        mag = np.abs(x) @ np.abs(w.T) + np.abs(b_)
+        for name, got, want in (("forward", fwd[t], nn_ref._celu(x @ w.T + b_)), ("plain", lin[t], x @ w.T),
+                                ("data gradient", bwd[t], (x * np.where(h >= 0, 1.0, h / 0.1 + 1.0)) @ w.T)):
+            got = got.cpu().numpy().astype(np.float64)
+            assert got.shape == want.shape == (ns[t], n_out), (name, t)
+            if want.size:
+                assert np.all(np.isfinite(got)) and np.all(np.abs(got - want) <= 2e-6 * mag + 1e-7), (name, t, np.abs(got - want).max())
+
+
+@pytest.mark.gpu
+def test_kernel_layers_agree_with_library_layers_in_energy_and_gradient():
+    """The float32 model with its CELU layers in khan_dense_f32 against the same model with every layer a library
+    product: energies and coordinate gradients of 200 molecules."""
+    b, mols = _molecules(n_mols=200, first=40)
+    ys = [0.0] * len(mols)
+    res = []
+    for kernel in (True, False):
+        m = model.AniModel(model.DEFAULT_LAYERS, model.celu, torch.float32, "cuda:0", seed=9, first_layer_kernel=kernel)
+        assert m.near.kernel_layers() == (3 if kernel else 0)
+        rd = RawDataset(mols, ys)
+        res.append((np.asarray(m.predict(rd, batch_size=64)), np.concatenate(list(m.coordinate_gradients(rd, batch_size=64)), axis=0)))
+    (e1, g1), (e0, g0) = res
+    assert np.abs(e1 - e0).max() <= 2e-5 * max(1.0, np.abs(e0).max())
+    assert np.abs(g1 - g0).max() <= 2e-4 * max(1e-3, np.abs(g0).max())
+
+
+@pytest.mark.gpu
 def test_energy_server_round_trip_over_a_socket():
     b, mols = _molecules(n_mols=2, first=11)
     m = _gpu_model(torch.float64, seed=5)
