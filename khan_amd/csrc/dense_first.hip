@@ -186,12 +186,18 @@ __global__ __launch_bounds__(256) void dense_kernel(DenseArgs args, float alpha,
 // whole step ago -- into the other LDS buffer.  So the first chunk of the next tile arrives while this tile is still
 // being multiplied, and its epilogue's stores drain under the next tile's products: with K = 128 a tile is only four
 // chunks long, and starting every tile cold cost a third of the kernel.
-template <int kTileCols, int kK, bool kCelu, bool kDeriv>
-__global__ __launch_bounds__(256) void dense_pipe_kernel(DenseArgs args, int total_tiles, float alpha, float inv_alpha)
+// kThreads: 512 for the 128-column tile (eight wavefronts, 4 down x 2 across, 32 x 64 each; two workgroups per CU are
+// four wavefronts per SIMD, which need 128 registers or fewer), 256 for the 64-column tile (four wavefronts, 4 x 1).
+template <int kTileCols, int kThreads, int kK, bool kCelu, bool kDeriv>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kThreads / 128, kThreads / 128)))
+void dense_pipe_kernel(DenseArgs args, int total_tiles, float alpha, float inv_alpha)
 {
-    constexpr int kWaveRows = kTileCols == 128 ? 64 : 32;
+    constexpr int kAcross = kTileCols / 64;                    // wavefronts across the tile
+    constexpr int kWaveRows = kTileRows / (kThreads / 64 / kAcross);
+    static_assert(kWaveRows == 32, "one 32-row block down, two across per wavefront");
     constexpr int kBI = kWaveRows / 32;
-    constexpr int kBPieces = kTileCols * (kChunk / 4) / 256;
+    constexpr int kAPieces = kTileRows * (kChunk / 4) / kThreads;    // 16-byte pieces of the rows chunk per thread
+    constexpr int kBPieces = kTileCols * (kChunk / 4) / kThreads;    // and of the weight chunk
     constexpr int kChunks = kK / kChunk;
     static_assert(kChunks % 2 == 0, "two register sets alternate by step: a tile must be an even number of steps");
     __shared__ DenseLds<kTileCols> S;
@@ -230,15 +236,15 @@ __global__ __launch_bounds__(256) void dense_pipe_kernel(DenseArgs args, int tot
         o.n = args.n[t];
         const float* bias = args.bias[t];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) o.bj[j] = bias ? bias[o.col0 + (kTileCols == 128 ? (wave & 1) : 0) * 64 + j * 32 + (lane & 31)] : 0.f;
+        for (int j = 0; j < 2; ++j) o.bj[j] = bias ? bias[o.col0 + (kAcross == 2 ? (wave & 1) : 0) * 64 + j * 32 + (lane & 31)] : 0.f;
     };
 
-    v4 ra[2][4], rb[2][kBPieces];
-    auto fetch = [&](const Cursor& c, v4 (&a)[4], v4 (&b)[kBPieces]) {
+    v4 ra[2][kAPieces], rb[2][kBPieces];
+    auto fetch = [&](const Cursor& c, v4 (&a)[kAPieces], v4 (&b)[kBPieces]) {
         if (!c.live) return;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int p = tid + 256 * u;
+        for (int u = 0; u < kAPieces; ++u) {
+            const int p = tid + kThreads * u;
             const int r = p >> 3, k4 = (p & 7) << 2;
             const int gr = min(c.row0 + r, c.n - 1);       // past the end: the last row again, never stored
             const size_t at = static_cast<size_t>(gr) * kK + c.chunk * kChunk + k4;
@@ -251,25 +257,25 @@ __global__ __launch_bounds__(256) void dense_pipe_kernel(DenseArgs args, int tot
         }
 #pragma unroll
         for (int u = 0; u < kBPieces; ++u) {
-            const int p = tid + 256 * u;
+            const int p = tid + kThreads * u;
             const int r = p >> 3, k4 = (p & 7) << 2;
             b[u] = *reinterpret_cast<const v4*>(c.wt + static_cast<size_t>(r) * kK + c.chunk * kChunk + k4);
         }
     };
-    auto stage = [&](int buf, const v4 (&a)[4], const v4 (&b)[kBPieces]) {
+    auto stage = [&](int buf, const v4 (&a)[kAPieces], const v4 (&b)[kBPieces]) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int p = tid + 256 * u;
+        for (int u = 0; u < kAPieces; ++u) {
+            const int p = tid + kThreads * u;
             *reinterpret_cast<v4*>(&S.a[buf][p >> 3][(p & 7) << 2]) = a[u];
         }
 #pragma unroll
         for (int u = 0; u < kBPieces; ++u) {
-            const int p = tid + 256 * u;
+            const int p = tid + kThreads * u;
             *reinterpret_cast<v4*>(&S.b[buf][p >> 3][(p & 7) << 2]) = b[u];
         }
     };
 
-    const int wr = kTileCols == 128 ? (wave >> 1) : wave, wc = kTileCols == 128 ? (wave & 1) : 0;
+    const int wr = kAcross == 2 ? (wave >> 1) : wave, wc = kAcross == 2 ? (wave & 1) : 0;
     const int l32 = lane & 31, half = lane >> 5;
     v16 acc[kBI][2];
     auto clear = [&]() {
@@ -376,12 +382,13 @@ hipError_t launch_tiles_k(const DenseArgs& a, int run, bool celu, bool deriv, fl
         int device = 0, cus = 0;
         if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0)
             cus = 256;
-        const int resident = cus * (kTileCols == 128 ? 2 : 2);
-        const dim3 pgrid(static_cast<unsigned>(run < resident ? run : resident)), pblock(256);
-        if (celu && !deriv) dense_pipe_kernel<kTileCols, kK, true, false><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
-        else if (!celu && !deriv) dense_pipe_kernel<kTileCols, kK, false, false><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
-        else if (!celu && deriv) dense_pipe_kernel<kTileCols, kK, false, true><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
-        else dense_pipe_kernel<kTileCols, kK, true, true><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
+        constexpr int kThreads = kTileCols == 128 ? 512 : 256;
+        const int resident = cus * 2;
+        const dim3 pgrid(static_cast<unsigned>(run < resident ? run : resident)), pblock(kThreads);
+        if (celu && !deriv) dense_pipe_kernel<kTileCols, kThreads, kK, true, false><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
+        else if (!celu && !deriv) dense_pipe_kernel<kTileCols, kThreads, kK, false, false><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
+        else if (!celu && deriv) dense_pipe_kernel<kTileCols, kThreads, kK, false, true><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
+        else dense_pipe_kernel<kTileCols, kThreads, kK, true, true><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
         return hipGetLastError();
     }
     const dim3 grid(static_cast<unsigned>(run)), block(256);
