@@ -140,8 +140,9 @@ def cpu_baseline(batch, sample_mols_fwd, sample_mols_bwd, w=4):
 
 
 def inference_bench(args, batch):
-    """Energy + coordinate-gradient inference: featurize -> per-type networks (rocBLAS products) -> segment sum,
-    then back through the networks and featurize_grad.  One JSON line; the roofline object describes the step's
+    """Energy + coordinate-gradient inference: featurize -> per-type networks -> segment sum, then back through the
+    networks and featurize_grad; timed with every layer a library (rocBLAS) product and with the CELU layers in this
+    package's matrix-core kernel.  One JSON line; the roofline object describes the step's
     dense layers, which dominate it (their flops against the fp32 matrix peak)."""
     import numpy as np
     import torch
@@ -164,7 +165,7 @@ def inference_bench(args, batch):
         return (time.perf_counter() - t0) / args.steps * 1e3, e, g
 
     ms_library, e_lib, g_lib = timed(False)      # every dense layer a library (rocBLAS) product
-    ms_per_step, e_k, g_k = timed(True)          # first layer in this package's matrix-core kernel
+    ms_per_step, e_k, g_k = timed(True)          # CELU layers, forward and backward, in this package's matrix-core kernel
     agree = float((e_k - e_lib).abs().max() / e_lib.abs().max())
     sizes = (384,) + tuple(model.DEFAULT_LAYERS)
     macs_per_atom = sum(x * y for x, y in zip(sizes[:-1], sizes[1:]))
@@ -179,7 +180,7 @@ def inference_bench(args, batch):
         "molecules_per_s": n_mols / (ms_per_step * 1e-3),
         "first_layer": {"kernel_ms_per_step": ms_per_step, "library_ms_per_step": ms_library,
                         "max_relative_energy_difference": agree},
-        "roofline": {"kernel": "dense layers (first: khan_dense_first_f32, others: rocBLAS)", "bound": "mfma", "achieved": gemm_flops / (ms_per_step * 1e-3) / 1e12,
+        "roofline": {"kernel": "dense layers (CELU layers forward and backward: khan_dense_f32; last layer: rocBLAS)", "bound": "mfma", "achieved": gemm_flops / (ms_per_step * 1e-3) / 1e12,
                      "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": gemm_flops / (ms_per_step * 1e-3) / 1e12 / FP32_PEAK_TFLOPS, "traffic": None},
     }))
