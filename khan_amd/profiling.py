@@ -48,12 +48,13 @@ DOMINANT = {
 
 
 def kernel_sources_digest():
-    """sha256 over the kernel sources (csrc/*.hip, csrc/*.h, the build flags), 16 hex digits."""
+    """sha256 over the sources of the AEV kernels the record is about (csrc/aev_*.hip, csrc/aev_*.h, the two shared
+    headers, the build flags), 16 hex digits."""
     from . import build
     h = hashlib.sha256()
     csrc = os.path.join(HERE, "csrc")
     for name in sorted(os.listdir(csrc)):
-        if name.endswith((".hip", ".h")):
+        if (name.startswith("aev_") and name.endswith((".hip", ".h"))) or name in ("khan_internal.h", "khan_params.h"):
             h.update(name.encode())
             with open(os.path.join(csrc, name), "rb") as f:
                 h.update(f.read())
