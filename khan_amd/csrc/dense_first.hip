@@ -372,6 +372,20 @@ void dense_pipe_kernel(DenseArgs args, int total_tiles, float alpha, float inv_a
     }
 }
 
+// compute units of the current device (looked up once per device)
+int compute_units()
+{
+    static int cached[64] = {};
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
+    int cus = __atomic_load_n(&cached[device], __ATOMIC_RELAXED);
+    if (cus == 0) {
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) cus = 256;
+        __atomic_store_n(&cached[device], cus, __ATOMIC_RELAXED);
+    }
+    return cus;
+}
+
 template <int kTileCols, int kK>
 hipError_t launch_tiles_k(const DenseArgs& a, int run, bool celu, bool deriv, float alpha, hipStream_t stream)
 {
@@ -379,9 +393,7 @@ hipError_t launch_tiles_k(const DenseArgs& a, int run, bool celu, bool deriv, fl
     // the widths of the reference's default network 384-128-128-64-1, forward and backward
     if constexpr ((kTileCols == 128 && kK > 0) || (kTileCols == 64 && kK == 128)) {
         // the pipelined kernel: as many workgroups as stay resident (two per CU at 72 KB of LDS, three at 54 KB)
-        int device = 0, cus = 0;
-        if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0)
-            cus = 256;
+        const int cus = compute_units();
         constexpr int kThreads = kTileCols == 128 ? 512 : 256;
         const int resident = cus * 2;
         const dim3 pgrid(static_cast<unsigned>(run < resident ? run : resident)), pblock(kThreads);
