@@ -49,9 +49,9 @@ struct __align__(16) DenseLds {
     float b[2][kTileCols][kPad];       // transposed-weights tile
 };
 
-// kK: the summed width when it is one of the network's (384, 128, 64: the chunk loop is then known to the compiler),
-// 0 for any other multiple of 32 (taken from the arguments)
-template <int kTileCols, int kK, bool kCelu, bool kDeriv>
+// The plain form, one tile per workgroup, for any summed width that is a multiple of 32 (the widths of the
+// reference's default network take the pipelined kernel below).
+template <int kTileCols, bool kCelu, bool kDeriv>
 __global__ __launch_bounds__(256) void dense_kernel(DenseArgs args, float alpha, float inv_alpha)
 {
     constexpr int kWaveRows = kTileCols == 128 ? 64 : 32;      // rows of a wavefront's part of the tile
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void dense_kernel(DenseArgs args, float alpha,
     const int t = (blk >= args.tile_end[0]) + (blk >= args.tile_end[1]) + (blk >= args.tile_end[2]);
     const int rel = blk - (t == 0 ? 0 : args.tile_end[t - 1]);
     const int tile = rel / args.col_tiles, ctile = rel - tile * args.col_tiles;
-    const int n = args.n[t], K = kK > 0 ? kK : args.k;
+    const int n = args.n[t], K = args.k;
     const float* __restrict__ rows = args.rows[t];
     const float* __restrict__ deriv = args.deriv[t];
     const float* __restrict__ wt = args.wt[t] + static_cast<size_t>(ctile) * kTileCols * K;
@@ -404,10 +404,10 @@ hipError_t launch_tiles_k(const DenseArgs& a, int run, bool celu, bool deriv, fl
         return hipGetLastError();
     }
     const dim3 grid(static_cast<unsigned>(run)), block(256);
-    if (celu && !deriv) dense_kernel<kTileCols, 0, true, false><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
-    else if (!celu && !deriv) dense_kernel<kTileCols, 0, false, false><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
-    else if (!celu && deriv) dense_kernel<kTileCols, 0, false, true><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
-    else dense_kernel<kTileCols, 0, true, true><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
+    if (celu && !deriv) dense_kernel<kTileCols, true, false><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
+    else if (!celu && !deriv) dense_kernel<kTileCols, false, false><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
+    else if (!celu && deriv) dense_kernel<kTileCols, false, true><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
+    else dense_kernel<kTileCols, true, true><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
     return hipGetLastError();
 }
 

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from khan_amd import datagen, model, server
+from khan_amd import autograd, datagen, model, server
 from khan_amd.batching import RawDataset
 from oracle import nn_ref
 
@@ -359,6 +359,31 @@ def test_kernel_layers_agree_with_library_layers_in_energy_and_gradient():
     (e1, g1), (e0, g0) = res
     assert np.abs(e1 - e0).max() <= 2e-5 * max(1.0, np.abs(e0).max())
     assert np.abs(g1 - g0).max() <= 2e-4 * max(1e-3, np.abs(g0).max())
+
+
+@pytest.mark.gpu
+def test_kernel_layers_give_the_library_layers_weight_gradients():
+    """Training through the kernel layers (`weights_need_grad`): d sum(energies) / d every weight and bias against
+    the same model with library layers, on one batch; a network of other widths (384-192-64-1) goes through the plain kernel."""
+    from khan_amd.batching import DeviceBatch
+    b, _ = _molecules(n_mols=120, first=7)
+    dev = "cuda:0"
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    batch = DeviceBatch.from_device_arrays(d(b.X), d(b.Y), d(b.Z), d(b.A), d(b.mol_idxs), b.n_mols)
+    for layers in (model.DEFAULT_LAYERS, (192, 64, 1)):
+        grads = []
+        for kernel in (True, False):
+            m = model.AniModel(layers, model.celu, torch.float32, dev, seed=3, first_layer_kernel=kernel)
+            m.near.weights_need_grad = True
+            assert m.near.kernel_layers() == ((len(layers) - 1) if kernel else 0)
+            names = sorted(m.near.params)
+            feats = autograd.featurize(batch.xs, batch.ys, batch.zs, batch.atom_types, batch.mol_offsets,
+                                       batch.mol_atom_counts, batch.scatter_idxs, batch.host_counts()[0])
+            atom_e = m.near.atom_outputs(feats, batch.gather_idxs)
+            gs = torch.autograd.grad(atom_e.sum(), [m.near.params[k] for k in names])
+            grads.append([g.cpu().numpy().astype(np.float64) for g in gs])
+        for name, g1, g0 in zip(names, grads[0], grads[1]):
+            assert np.abs(g1 - g0).max() <= 2e-4 * max(1e-6, np.abs(g0).max()), (layers, name, np.abs(g1 - g0).max())
 
 
 @pytest.mark.gpu
