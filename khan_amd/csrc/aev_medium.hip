@@ -2,7 +2,7 @@
 // float64 from 65; also the float32 Jacobian-vector product from 65): one workgroup of four wavefronts per molecule.
 //
 // The workgroup sorts the molecule's atoms by type into LDS once (256-way counting sort with per-wave
-// ballots).  Each wavefront then takes batches of six centres and runs the same pipeline as the
+// ballots).  Each wavefront then takes batches of four or six centres (see kNB below) and runs the same pipeline as the
 // one-wavefront-per-molecule kernel on them:
 //   scan     a centre is tested against the sorted atoms 64 at a time; partners inside the radial
 //            cutoff are appended to a (r, f_C) list, partners inside the angular cutoff to the centre's
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
             return reinterpret_cast<T*>((static_cast<unsigned long long>(hi) << 32) | lo);
         };
 
-        // ------------------------------------------------------------ batches of six centres per wavefront
+        // ------------------------------------------------------------ batches of kNB centres per wavefront
         for (int c0 = wave * kNB; c0 < n; c0 += 4 * kNB) {
             const int nb = min(kNB, n - c0);
             unsigned overflow = 0;

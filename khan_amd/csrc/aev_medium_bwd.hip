@@ -3,10 +3,10 @@
 //
 // The workgroup sorts the atoms by type into LDS once and zeroes the molecule's outputs.  Wavefronts
 // then draw centres from a shared counter.  A wavefront collects centres into a batch while their
-// angular partner lists fit the 64 entries of its pool (at most six), and for each centre it takes in:
+// angular partner lists fit the 64 entries of its pool (at most four in float, six in double), and for each centre it takes in:
 //   scan + radial   the centre is tested against the sorted atoms 64 at a time; pairs inside the radial
 //                   cutoff are queued, and whenever 64 are waiting a lane takes one pair and sums
-//                   g e (f_C' - 2 eta d f_C) over the 16 shells for both directions of the pair (the centre's
+//                   g e (f_C' - 2 eta d f_C) over the shells (float: the nine nearest to r) for both directions of the pair (the centre's
 //                   row and the partner's row share every shell factor): that is the pair's whole pull on the
 //                   centre, and nothing is added to the partner, which gets the same as a centre itself
 //                   (per-pair atomic adds to the partners cost a quarter of the kernel);

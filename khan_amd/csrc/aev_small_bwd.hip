@@ -142,7 +142,7 @@ void aev_bwd_small_kernel(
             const int got = __builtin_amdgcn_ds_bpermute((((lane - s0) << logW) & 63) << 2, cnt);
             if (lane >= s0 && lane < s0 + G) m_mine = got;
 
-            // ---- radial pairs: this lane's (centre, partner) pair over its 16 shells.  Done here, where the
+            // ---- radial pairs: this lane's (centre, partner) pair over its shells (float: the nine nearest to r).  Done here, where the
             // centres come G at a time in lane order, and not per batch, whose last step is rarely full.
             const T* grow = row_of_lane(min(i, 63));
             T cfx = T(0), cfy = T(0), cfz = T(0);       // this pair's pull on the centre

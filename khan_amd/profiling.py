@@ -47,17 +47,26 @@ DOMINANT = {
 }
 
 
+def _code_only(text):
+    """Source text without comments and with runs of white space collapsed: what the digest is taken over, so that
+    rewording a comment does not make a measurement stale."""
+    import re
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", " ", text)
+    return " ".join(text.split())
+
+
 def kernel_sources_digest():
-    """sha256 over the sources of the AEV kernels the record is about (csrc/aev_*.hip, csrc/aev_*.h, the two shared
-    headers, the build flags), 16 hex digits."""
+    """sha256 over the code (comments left out) of the AEV kernels the record is about (csrc/aev_*.hip, csrc/aev_*.h,
+    the two shared headers) and the build flags, 16 hex digits."""
     from . import build
     h = hashlib.sha256()
     csrc = os.path.join(HERE, "csrc")
     for name in sorted(os.listdir(csrc)):
         if (name.startswith("aev_") and name.endswith((".hip", ".h"))) or name in ("khan_internal.h", "khan_params.h"):
             h.update(name.encode())
-            with open(os.path.join(csrc, name), "rb") as f:
-                h.update(f.read())
+            with open(os.path.join(csrc, name), "r") as f:
+                h.update(_code_only(f.read()).encode())
     h.update(" ".join(build.HIPCC_FLAGS).encode())
     return h.hexdigest()[:16]
 
