@@ -30,16 +30,21 @@ namespace khan {
 
 namespace {
 
+// centres per batch.  float: six (the pool of 64 entries is what ends most batches).  double: four -- the staged
+// upstream rows are twice the size, and with four the working set (20.4 KB) lets eight wavefronts share a CU instead
+// of six, which is worth more than the fuller pools of six-centre batches (organic molecules: 0.53 -> 0.44 ms).
+template <typename T> constexpr int kSmallBwdCentres = sizeof(T) == 8 ? 4 : kB;
+
 template <typename T>
 struct __align__(16) BwdLds {
     typename Fast<T>::vec4 atom[64];     // x, y, z, type (sorted order)
-    BwdPool<T> pool;                     // partner lists and staged upstream values of the batch
+    BwdPool<T, kSmallBwdCentres<T>> pool;   // partner lists and staged upstream values of the batch
     T force[3][64];                      // dL/dx, dL/dy, dL/dz per sorted atom
     int nM[8];                           // angular partners per centre of the batch
     unsigned char inv[64];               // original atom index -> sorted lane
 };
 
-// float: 3 wavefronts per SIMD (LDS 13.2 KB); double: 1 (LDS 26 KB, twice the registers)
+// float: 3 wavefronts per SIMD (LDS 13.2 KB); double: 2 (LDS 20.4 KB, twice the registers)
 template <typename T>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 3 : 1, sizeof(T) == 4 ? 3 : 2)))
 void aev_bwd_small_kernel(
@@ -180,7 +185,7 @@ void aev_bwd_small_kernel(
     }
 
     for (int c0 = 0, nb = 0; c0 < n; c0 += nb) {
-        // centres of this batch: up to kB, lists fitting the 64 lanes; pf[b] = first list slot of centre b
+        // centres of this batch: up to kSmallBwdCentres, lists fitting the 64 lanes; pf[b] = first list slot of centre b
         int pf[kB + 1];
         {
             bool open = true;
@@ -190,7 +195,7 @@ void aev_bwd_small_kernel(
 #pragma unroll
             for (int k = 0; k < kB; ++k) {
                 int m = 0;
-                if (open && c0 + k < n) {
+                if (open && k < kSmallBwdCentres<T> && c0 + k < n) {
                     m = lane_read(m_at, min(c0 + k, 63));
                     if (k > 0 && tot + m > 64) {
                         open = false;
@@ -209,7 +214,7 @@ void aev_bwd_small_kernel(
         unsigned overflow = 0;
 
         // ---- fetch the angular upstream blocks of the batch's rows (80 x 16 bytes per row)
-        RowStage<T> stage;
+        RowStage<T, kSmallBwdCentres<T>> stage;
         stage.fetch(lane, nb, [&](int b) { return row_of(lane_read(cord, min(c0 + b, 63))); });
         S.pool.facc[lane] = Fast<T>::make4(T(0), T(0), T(0), T(0));
         if (lane < 8) S.nM[lane] = 0;
