@@ -5,7 +5,7 @@
 // reads the 16 upstream values of the partner's type from the centre's row, sums g e (f_C' - 2 eta d f_C)
 // over the shells, and the pull goes to the partner (one group of lanes at a time, so targets are
 // distinct) and, summed over the group with DPP moves, to the centre.  Centres are then taken in order
-// of decreasing partner count, in batches of up to six whose partner lists together fill at most the 64
+// of decreasing partner count, in batches of up to six (four in float64) whose partner lists together fill at most the 64
 // lanes.  Per batch:
 //   stage    the 320 angular upstream values of each centre's row are fetched with full-line loads
 //            (issued before the scan, so their latency is covered) and laid out in LDS by type pair;
