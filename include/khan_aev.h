@@ -254,6 +254,29 @@ int khan_dense_f32(const float *const *rows_host4, const int32_t *n_host4, int32
                    float alpha, const float *const *deriv_of_host4, float *const *out_host4,
                    khan_stream_t stream);
 
+/* The last hidden layer of the per-type networks together with the output layer behind it (khan/model/nn.py:38-68
+ * with layer sizes (..., 64, 1): the output layer is a matmul to one column plus bias, no activation), one launch
+ * for the four types:
+ *     out_t[r, :] = act(in_t[r, :] . W_t + b_t),    head_out_t[r] = out_t[r, :] . head_w_t + head_b_t[0].
+ * Arguments as khan_dense_f32, with n_out = 64; head_w_t [64], head_b_t [1] or head_b_host4 = NULL, head_out_t [n_t].
+ * out_t is still written: the way back needs the activations. */
+int khan_dense_head_f32(const float *const *rows_host4, const int32_t *n_host4, int32_t k, int32_t n_out,
+                        const float *const *wt_host4, const float *const *bias_host4, int32_t activation,
+                        float alpha, const float *const *head_w_host4, const float *const *head_b_host4,
+                        float *const *out_host4, float *const *head_out_host4, khan_stream_t stream);
+
+/* The way back through the output layer and the last hidden layer (the gradient TensorFlow derives for
+ * nn.py:38-68), one launch for the four types: given scale_t[r] = d/d head_out_t[r],
+ *     out_t[r, :] = (scale_t[r] head_w_t[:] .* CELU'(z)) . W_t^T,   CELU(z) = deriv_of_t (the layer's activations),
+ * the gradient with respect to the last hidden layer's input.  scale_t [n_t], head_w_t [k] (16-byte aligned),
+ * deriv_of_t [n_t, k], wt_t [n_out, k] = the layer's weights as stored (k = the layer's width, n_out = its input
+ * width: the convention of khan_dense_f32's data gradient), out_t [n_t, n_out].  The outer product is formed in
+ * registers; no [n_t, k] gradient matrix is written or read. */
+int khan_dense_head_grad_f32(const float *const *scale_host4, const float *const *head_w_host4,
+                             const int32_t *n_host4, int32_t k, int32_t n_out, const float *const *wt_host4,
+                             float alpha, const float *const *deriv_of_host4, float *const *out_host4,
+                             khan_stream_t stream);
+
 /* Plain Coulomb sums, E_m = k sum_{i<j in m} q_i q_j / r_ij, and their gradients: the charge kernels with
  * the damping (1 - f_C) switched off and the constant chosen by the caller (k = 1 for charges in e and
  * distances in the unit the energy is wanted in).  No reference counterpart: khan's own op is the damped,

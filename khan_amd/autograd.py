@@ -125,6 +125,64 @@ def dense(inputs, weights, biases, activation=ops.ACT_CELU, alpha=0.1, weights_t
     return _Dense.apply(int(activation), float(alpha), weights_t, *inputs, *weights, *biases)
 
 
+class _DenseHead(torch.autograd.Function):
+    """The last hidden layer (width 64) and the output layer (64 -> 1, no activation) of the four atomic networks in
+    one launch each way (`ops.dense_head`, `ops.dense_head_grad`): -> four [n_t] vectors of atomic values.  On the way
+    back the gradient with respect to the hidden activations, g_t[r] * w_out_t[c], is never materialised for the data
+    gradient; the weight gradients (when asked for) are library products."""
+
+    @staticmethod
+    def forward(ctx, activation, alpha, weights_t, *tensors):
+        xs, ws, bs, hws, hbs = tensors[0:4], tensors[4:8], tensors[8:12], tensors[12:16], tensors[16:20]
+        k = ws[0].shape[0]
+        if weights_t is None:
+            weights_t = [w.detach().t().contiguous() for w in ws]
+        outs, heads = ops.dense_head([x.detach().reshape(-1, k) for x in xs], weights_t, [b.detach() for b in bs],
+                                     [w.detach() for w in hws], [b.detach() for b in hbs], activation, alpha)
+        ctx.save_for_backward(*xs, *ws, *hws, *outs)
+        ctx.activation, ctx.alpha = activation, alpha
+        return heads
+
+    @staticmethod
+    def backward(ctx, *gheads):
+        saved = ctx.saved_tensors
+        xs, ws, hws, outs = saved[0:4], saved[4:8], saved[8:12], saved[12:16]
+        k, n_out = ws[0].shape
+        celu_act = ctx.activation == ops.ACT_CELU
+        gs = [torch.zeros(outs[t].shape[0], dtype=outs[t].dtype, device=outs[t].device) if gheads[t] is None
+              else gheads[t].contiguous() for t in range(4)]
+        gx = (None,) * 4
+        if any(ctx.needs_input_grad[3:7]):
+            if celu_act:
+                gx = ops.dense_head_grad(gs, [w.detach() for w in hws], [w.detach() for w in ws], outs, ctx.alpha)
+            else:
+                gx = ops.dense([gs[t][:, None] * hws[t].detach().reshape(1, -1) for t in range(4)], [w.detach() for w in ws])
+            gx = tuple(g.reshape(xs[t].shape) if ctx.needs_input_grad[3 + t] else None for t, g in enumerate(gx))
+        gw, gb, ghw, ghb = [None] * 4, [None] * 4, [None] * 4, [None] * 4
+        if any(ctx.needs_input_grad[7:23]):
+            for t in range(4):
+                if ctx.needs_input_grad[15 + t]:
+                    ghw[t] = (outs[t].t() @ gs[t]).reshape(hws[t].shape)
+                if ctx.needs_input_grad[19 + t]:
+                    ghb[t] = gs[t].sum().reshape(1)
+                if ctx.needs_input_grad[7 + t] or ctx.needs_input_grad[11 + t]:
+                    g = gs[t][:, None] * hws[t].detach().reshape(1, -1)
+                    if celu_act:
+                        g = torch.ops.aten.elu_backward(g, ctx.alpha, 1.0, 1.0 / ctx.alpha, True, outs[t])
+                    if ctx.needs_input_grad[7 + t]:
+                        gw[t] = xs[t].reshape(-1, k).t() @ g
+                    if ctx.needs_input_grad[11 + t]:
+                        gb[t] = g.sum(dim=0)
+        return (None, None, None) + tuple(gx) + tuple(gw) + tuple(gb) + tuple(ghw) + tuple(ghb)
+
+
+def dense_head(inputs, weights, biases, head_weights, head_biases, activation=ops.ACT_CELU, alpha=0.1, weights_t=None):
+    """Differentiable last hidden layer + output layer of the four atomic networks: four inputs [n_t, k], four
+    [k, 64] weights, four [64] biases, four [64, 1] output-layer weights, four [1] output-layer biases -> four [n_t]
+    vectors (float32; k a multiple of 32)."""
+    return _DenseHead.apply(int(activation), float(alpha), weights_t, *inputs, *weights, *biases, *head_weights, *head_biases)
+
+
 def dense_first(atom_type_features, acs_host, weights, biases, activation=ops.ACT_CELU, alpha=0.1, weights_t=None):
     """The first dense layer on the featurizer's four flat buckets: `dense` with k = 384."""
     for f, c in zip(atom_type_features, acs_host):

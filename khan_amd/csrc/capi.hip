@@ -555,6 +555,55 @@ int khan_dense_f32(const float* const* rows_host4, const int32_t* n_host4, int32
                                          alpha, deriv_of_host4, out_host4, as_stream(stream)));
 }
 
+int khan_dense_head_f32(const float* const* rows_host4, const int32_t* n_host4, int32_t k, int32_t n_out,
+                        const float* const* wt_host4, const float* const* bias_host4, int32_t activation, float alpha,
+                        const float* const* head_w_host4, const float* const* head_b_host4, float* const* out_host4,
+                        float* const* head_out_host4, khan_stream_t stream)
+{
+    if (!rows_host4 || !n_host4 || !wt_host4 || !head_w_host4 || !out_host4 || !head_out_host4) return KHAN_ERR_INVALID_ARG;
+    if (activation != KHAN_ACT_NONE && activation != KHAN_ACT_CELU) return KHAN_ERR_INVALID_ARG;
+    if (activation == KHAN_ACT_CELU && !(alpha > 0.0f)) return KHAN_ERR_INVALID_ARG;
+    if (k <= 0 || k % 32 != 0 || n_out != 64) return KHAN_ERR_INVALID_ARG;
+    int64_t total = 0;
+    for (int t = 0; t < 4; ++t) {
+        if (n_host4[t] < 0) return KHAN_ERR_INVALID_ARG;
+        if (n_host4[t] == 0) continue;
+        if (!rows_host4[t] || !wt_host4[t] || !head_w_host4[t] || !out_host4[t] || !head_out_host4[t]) return KHAN_ERR_INVALID_ARG;
+        if (bias_host4 && !bias_host4[t]) return KHAN_ERR_INVALID_ARG;
+        if (head_b_host4 && !head_b_host4[t]) return KHAN_ERR_INVALID_ARG;
+        if ((reinterpret_cast<uintptr_t>(rows_host4[t]) | reinterpret_cast<uintptr_t>(wt_host4[t])) & 15u) return KHAN_ERR_INVALID_ARG;
+        total += n_host4[t];
+    }
+    if (total == 0) return KHAN_OK;
+    if (total > INT32_MAX) return KHAN_ERR_TOO_LARGE;
+    return hip_status(khan::launch_dense_head(rows_host4, n_host4, k, n_out, wt_host4, bias_host4, activation == KHAN_ACT_CELU,
+                                              alpha, head_w_host4, head_b_host4, out_host4, head_out_host4, as_stream(stream)));
+}
+
+int khan_dense_head_grad_f32(const float* const* scale_host4, const float* const* head_w_host4, const int32_t* n_host4,
+                             int32_t k, int32_t n_out, const float* const* wt_host4, float alpha,
+                             const float* const* deriv_of_host4, float* const* out_host4, khan_stream_t stream)
+{
+    if (!scale_host4 || !head_w_host4 || !n_host4 || !wt_host4 || !deriv_of_host4 || !out_host4) return KHAN_ERR_INVALID_ARG;
+    if (!(alpha > 0.0f)) return KHAN_ERR_INVALID_ARG;
+    if (k <= 0 || k % 32 != 0 || n_out <= 0 || n_out % 64 != 0) return KHAN_ERR_INVALID_ARG;
+    int64_t total = 0;
+    for (int t = 0; t < 4; ++t) {
+        if (n_host4[t] < 0) return KHAN_ERR_INVALID_ARG;
+        if (n_host4[t] == 0) continue;
+        if (!scale_host4[t] || !head_w_host4[t] || !wt_host4[t] || !deriv_of_host4[t] || !out_host4[t]) return KHAN_ERR_INVALID_ARG;
+        // 16-byte loads of the output layer's weights, the activations and the weights
+        if ((reinterpret_cast<uintptr_t>(head_w_host4[t]) | reinterpret_cast<uintptr_t>(wt_host4[t]) |
+             reinterpret_cast<uintptr_t>(deriv_of_host4[t])) & 15u)
+            return KHAN_ERR_INVALID_ARG;
+        total += n_host4[t];
+    }
+    if (total == 0) return KHAN_OK;
+    if (total > INT32_MAX) return KHAN_ERR_TOO_LARGE;
+    return hip_status(khan::launch_dense_head_grad(scale_host4, head_w_host4, n_host4, k, n_out, wt_host4, alpha, deriv_of_host4,
+                                                   out_host4, as_stream(stream)));
+}
+
 // Plain Coulomb sums: the charge kernels with the cutoff function switched off and the constant given by the caller.
 int khan_coulomb_f32(const float* xs, const float* ys, const float* zs, const float* qs, const int32_t* mos,
                      const int32_t* macs, int32_t n_mols, float k, float* e, khan_stream_t stream)

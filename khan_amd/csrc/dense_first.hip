@@ -18,6 +18,12 @@
 // the upper half k = 8q + 4 + t (t = 0..3 from one 16-byte read each), which covers every k of the chunk once -- a
 // sum does not care about its order.  A workgroup finds its type, row tile and column tile from the per-type tile
 // counts; the column tiles of one row tile are neighbours in the grid, so the rows they share come from L2.
+//
+// Two extras fold the networks' output layer (n -> 1, no activation: nn.py:38-68 with the last entry of the layer
+// sizes) into its neighbour.  kHead (64-column tile): the epilogue also forms head_out[r] = out[r, :] . head_w + head_b,
+// a sum over the tile's 64 columns = over the 32 lanes that hold a row's values.  kRank1: on the way back the
+// gradient with respect to the last hidden layer's activations is the outer product scale[r] * head_w[c]; the
+// staging builds it in registers instead of reading a matrix that something else would have had to write.
 #include "khan_internal.h"
 #include "khan_params.h"
 
@@ -41,7 +47,80 @@ struct DenseArgs {
     int n[4];                  // rows per type
     int tile_end[4];           // running sum of the per-type (row tile x column tile) counts
     int k, n_out, col_tiles;
+    const float* head_w[4];    // kHead: [n_out] weights of the output layer; kRank1: [k], the same weights on the way back
+    const float* head_b[4];    // kHead: one float, or null
+    float* head_out[4];        // kHead: [n_t]
+    const float* scale[4];     // kRank1: [n_t], the gradient with respect to each row's output value
 };
+
+// sum over the 32 lanes of each half of the wavefront; lanes 16-31 and 48-63 hold the result
+__device__ __forceinline__ float half_sum_to_upper_row(float v)
+{
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));   // row_ror:8
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false));   // row_ror:4
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false));   // row_ror:2
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false));   // row_ror:1
+    // rows 1 and 3 add lane 15 of the row before them (rows 0 and 2 add the zero given as old value)
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xa, 0xf, false));   // row_bcast:15
+    return v;
+}
+
+// Rows of a staging piece built from the outer product scale[row] * head_w[k..k+3]
+__device__ __forceinline__ v4 rank1_piece(const float* __restrict__ scale, const float* __restrict__ head_w, int row, int k)
+{
+    const float sc = scale[row];
+    const v4 w = *reinterpret_cast<const v4*>(head_w + k);
+    return v4{sc * w[0], sc * w[1], sc * w[2], sc * w[3]};
+}
+
+// Epilogue of one tile for one wavefront: bias, activation, store; with kHead (one wavefront holds all 64 columns of
+// its 32 rows) also the output layer's value of every row.  Accumulator e of block (i, j) is output row
+// row_base + i*32 + 8 (e / 4) + 4 half + e % 4, column col_base + j*32 + l32.
+// The bias is waited for once, before the first store: a wait inside a conditional store would also wait for
+// the stores before it (loads and stores share one counter), one by one -- 64 stores, each at full latency.
+template <bool kCelu, bool kHead, int kBI>
+__device__ __forceinline__ void tile_epilogue(const v16 (&acc)[kBI][2], float (&bj)[2], float (&hw)[2], const float* head_b,
+                                              float* __restrict__ out, float* __restrict__ head_out, int n, int n_out,
+                                              int row_base, int col_base, int l32, int half, float alpha, float inv_alpha)
+{
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        asm volatile("" : "+v"(bj[j]));          // in its register from here on: the one wait happens here
+        if constexpr (kHead) asm volatile("" : "+v"(hw[j]));
+    }
+    float hb = 0.f;
+    if constexpr (kHead) {
+        hb = head_b ? *head_b : 0.f;
+        asm volatile("" : "+v"(hb));
+    }
+#pragma unroll
+    for (int i = 0; i < kBI; ++i) {
+        float dot[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) dot[e] = 0.f;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int col = col_base + j * 32 + l32;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int r = row_base + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                float v = acc[i][j][e] + bj[j];
+                if (kCelu) v = v >= 0.f ? v : alpha * (__expf(v * inv_alpha) - 1.0f);
+                if (r < n) out[static_cast<size_t>(r) * n_out + col] = v;
+                if constexpr (kHead) dot[e] = fmaf(v, hw[j], dot[e]);
+            }
+        }
+        if constexpr (kHead) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const float tot = half_sum_to_upper_row(dot[e]) + hb;
+                const int r = row_base + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                if (l32 == 16 + e && r < n) head_out[r] = tot;        // lane 16 + e of each half stores row e's value
+            }
+        }
+    }
+}
+
 
 template <int kTileCols>
 struct __align__(16) DenseLds {
@@ -51,9 +130,10 @@ struct __align__(16) DenseLds {
 
 // The plain form, one tile per workgroup, for any summed width that is a multiple of 32 (the widths of the
 // reference's default network take the pipelined kernel below).
-template <int kTileCols, bool kCelu, bool kDeriv>
+template <int kTileCols, bool kCelu, bool kDeriv, bool kHead, bool kRank1>
 __global__ __launch_bounds__(256) void dense_kernel(DenseArgs args, float alpha, float inv_alpha)
 {
+    static_assert(!kHead || kTileCols == 64, "the output layer's sum runs over one wavefront's 64 columns");
     constexpr int kWaveRows = kTileCols == 128 ? 64 : 32;      // rows of a wavefront's part of the tile
     constexpr int kBI = kWaveRows / 32;                        // its matrix-core blocks down (2 or 1); across: 2
     constexpr int kBPieces = kTileCols * (kChunk / 4) / 256;   // 16-byte pieces of the weight chunk per thread (4 or 2)
@@ -82,7 +162,8 @@ __global__ __launch_bounds__(256) void dense_kernel(DenseArgs args, float alpha,
             // not under a condition needs no merge with a default afterwards (which would wait for it on the spot)
             const int gr = min(row0 + r, n - 1);
             const size_t at = static_cast<size_t>(gr) * K + chunk * kChunk + k4;
-            ra[u] = *reinterpret_cast<const v4*>(rows + at);
+            if constexpr (kRank1) ra[u] = rank1_piece(args.scale[t], args.head_w[t], gr, chunk * kChunk + k4);
+            else ra[u] = *reinterpret_cast<const v4*>(rows + at);
             if constexpr (kDeriv) {
                 // CELU'(z) from CELU(z) = h: 1 for h >= 0, exp(z / alpha) = h / alpha + 1 below
                 const v4 h = *reinterpret_cast<const v4*>(deriv + at);
@@ -150,33 +231,15 @@ __global__ __launch_bounds__(256) void dense_kernel(DenseArgs args, float alpha,
         }
     }
 
-    // epilogue: bias, activation, store.  Accumulator e of block (i, j) is output row
-    // wr*kWaveRows + i*32 + 8 (e / 4) + 4 half + e % 4, column wc*64 + j*32 + l32 of the tile.
-    // The bias is waited for once, before the first store: a wait inside a conditional store would also wait for
-    // the stores before it (loads and stores share one counter), one by one -- 64 stores, each at full latency.
     const float* __restrict__ bias = args.bias[t];
-    float* __restrict__ out = args.out[t];
-    const int n_out = args.n_out;
-    float bj[2];
+    float bj[2], hw[2] = {0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         bj[j] = bias ? bias[col0 + wc * 64 + j * 32 + l32] : 0.f;
-        asm volatile("" : "+v"(bj[j]));          // the bias is in its register from here on: the one wait happens here
+        if constexpr (kHead) hw[j] = args.head_w[t][col0 + j * 32 + l32];
     }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int col = col0 + wc * 64 + j * 32 + l32;
-#pragma unroll
-        for (int i = 0; i < kBI; ++i) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int r = row0 + wr * kWaveRows + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
-                float v = acc[i][j][e] + bj[j];
-                if (kCelu) v = v >= 0.f ? v : alpha * (__expf(v * inv_alpha) - 1.0f);
-                if (r < n) out[static_cast<size_t>(r) * n_out + col] = v;
-            }
-        }
-    }
+    tile_epilogue<kCelu, kHead, kBI>(acc, bj, hw, args.head_b[t], args.out[t], args.head_out[t], n, args.n_out,
+                                     row0 + wr * kWaveRows, col0 + wc * 64, l32, half, alpha, inv_alpha);
 }
 
 // The same product for the network's own widths (kK = 384, 128 or 64: an even number of chunks), as a pipeline that
@@ -188,10 +251,11 @@ __global__ __launch_bounds__(256) void dense_kernel(DenseArgs args, float alpha,
 // chunks long, and starting every tile cold cost a third of the kernel.
 // kThreads: 512 for the 128-column tile (eight wavefronts, 4 down x 2 across, 32 x 64 each; two workgroups per CU are
 // four wavefronts per SIMD, which need 128 registers or fewer), 256 for the 64-column tile (four wavefronts, 4 x 1).
-template <int kTileCols, int kThreads, int kK, bool kCelu, bool kDeriv>
+template <int kTileCols, int kThreads, int kK, bool kCelu, bool kDeriv, bool kHead, bool kRank1>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kThreads / 128, kThreads / 128)))
 void dense_pipe_kernel(DenseArgs args, int total_tiles, float alpha, float inv_alpha)
 {
+    static_assert(!kHead || kTileCols == 64, "the output layer's sum runs over one wavefront's 64 columns");
     constexpr int kAcross = kTileCols / 64;                    // wavefronts across the tile
     constexpr int kWaveRows = kTileRows / (kThreads / 64 / kAcross);
     static_assert(kWaveRows == 32, "one 32-row block down, two across per wavefront");
@@ -205,7 +269,8 @@ void dense_pipe_kernel(DenseArgs args, int total_tiles, float alpha, float inv_a
     const int stride = gridDim.x;
 
     struct Cursor {                 // where the next loads come from: a tile (or none) and a chunk of it
-        const float* rows;
+        const float* rows;          // kRank1: the per-row factors
+        const float* head_w;
         const float* deriv;
         const float* wt;
         int row0, n, chunk, tile;
@@ -213,14 +278,18 @@ void dense_pipe_kernel(DenseArgs args, int total_tiles, float alpha, float inv_a
     };
     struct TileOut {                // what the epilogue of a tile needs
         float* out;
+        float* head_out;
+        const float* head_b;
         int row0, col0, n;
         float bj[2];                // the bias of this lane's two columns, loaded when the tile starts
+        float hw[2];                // kHead: the output layer's weights of those columns
     };
     auto decode_loads = [&](int id, Cursor& c) {
         const int t = (id >= args.tile_end[0]) + (id >= args.tile_end[1]) + (id >= args.tile_end[2]);
         const int rel = id - (t == 0 ? 0 : args.tile_end[t - 1]);
         const int tile = rel / args.col_tiles, ctile = rel - tile * args.col_tiles;
-        c.rows = args.rows[t];
+        c.rows = kRank1 ? args.scale[t] : args.rows[t];
+        c.head_w = args.head_w[t];
         c.deriv = args.deriv[t];
         c.wt = args.wt[t] + static_cast<size_t>(ctile) * kTileCols * kK;
         c.row0 = tile * kTileRows;
@@ -236,7 +305,13 @@ void dense_pipe_kernel(DenseArgs args, int total_tiles, float alpha, float inv_a
         o.n = args.n[t];
         const float* bias = args.bias[t];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) o.bj[j] = bias ? bias[o.col0 + (kAcross == 2 ? (wave & 1) : 0) * 64 + j * 32 + (lane & 31)] : 0.f;
+        for (int j = 0; j < 2; ++j) {
+            o.bj[j] = bias ? bias[o.col0 + (kAcross == 2 ? (wave & 1) : 0) * 64 + j * 32 + (lane & 31)] : 0.f;
+            o.hw[j] = 0.f;
+            if constexpr (kHead) o.hw[j] = args.head_w[t][o.col0 + j * 32 + (lane & 31)];
+        }
+        o.head_out = args.head_out[t];
+        o.head_b = args.head_b[t];
     };
 
     v4 ra[2][kAPieces], rb[2][kBPieces];
@@ -248,7 +323,8 @@ void dense_pipe_kernel(DenseArgs args, int total_tiles, float alpha, float inv_a
             const int r = p >> 3, k4 = (p & 7) << 2;
             const int gr = min(c.row0 + r, c.n - 1);       // past the end: the last row again, never stored
             const size_t at = static_cast<size_t>(gr) * kK + c.chunk * kChunk + k4;
-            a[u] = *reinterpret_cast<const v4*>(c.rows + at);
+            if constexpr (kRank1) a[u] = rank1_piece(c.rows, c.head_w, gr, c.chunk * kChunk + k4);
+            else a[u] = *reinterpret_cast<const v4*>(c.rows + at);
             if constexpr (kDeriv) {
                 const v4 h = *reinterpret_cast<const v4*>(c.deriv + at);
 #pragma unroll
@@ -304,24 +380,8 @@ void dense_pipe_kernel(DenseArgs args, int total_tiles, float alpha, float inv_a
         }
     };
     auto epilogue = [&](TileOut& o) {
-        // the bias (loaded when the tile started) is waited for once, before the first store (see dense_kernel)
-        const int n_out = args.n_out;
-#pragma unroll
-        for (int j = 0; j < 2; ++j) asm volatile("" : "+v"(o.bj[j]));
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int col = o.col0 + wc * 64 + j * 32 + l32;
-#pragma unroll
-            for (int i = 0; i < kBI; ++i) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const int r = o.row0 + wr * kWaveRows + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
-                    float v = acc[i][j][e] + o.bj[j];
-                    if (kCelu) v = v >= 0.f ? v : alpha * (__expf(v * inv_alpha) - 1.0f);
-                    if (r < o.n) o.out[static_cast<size_t>(r) * n_out + col] = v;
-                }
-            }
-        }
+        tile_epilogue<kCelu, kHead, kBI>(acc, o.bj, o.hw, o.head_b, o.out, o.head_out, o.n, args.n_out,
+                                         o.row0 + wr * kWaveRows, o.col0 + wc * 64, l32, half, alpha, inv_alpha);
     };
 
     // the load cursor runs two steps ahead of the multiplication
@@ -386,8 +446,10 @@ int compute_units()
     return cus;
 }
 
+enum class Extra { kNone, kHead, kRank1 };
+
 template <int kTileCols, int kK>
-hipError_t launch_tiles_k(const DenseArgs& a, int run, bool celu, bool deriv, float alpha, hipStream_t stream)
+hipError_t launch_tiles_k(const DenseArgs& a, int run, bool celu, bool deriv, Extra extra, float alpha, hipStream_t stream)
 {
     const float inv_alpha = 1.0f / alpha;
     // the widths of the reference's default network 384-128-128-64-1, forward and backward
@@ -397,27 +459,58 @@ hipError_t launch_tiles_k(const DenseArgs& a, int run, bool celu, bool deriv, fl
         constexpr int kThreads = kTileCols == 128 ? 512 : 256;
         const int resident = cus * 2;
         const dim3 pgrid(static_cast<unsigned>(run < resident ? run : resident)), pblock(kThreads);
-        if (celu && !deriv) dense_pipe_kernel<kTileCols, kThreads, kK, true, false><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
-        else if (!celu && !deriv) dense_pipe_kernel<kTileCols, kThreads, kK, false, false><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
-        else if (!celu && deriv) dense_pipe_kernel<kTileCols, kThreads, kK, false, true><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
-        else dense_pipe_kernel<kTileCols, kThreads, kK, true, true><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
+        if (extra == Extra::kRank1) dense_pipe_kernel<kTileCols, kThreads, kK, false, true, false, true><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
+        else if (extra == Extra::kHead) {
+            if constexpr (kTileCols == 64) {
+                if (celu) dense_pipe_kernel<64, kThreads, kK, true, false, true, false><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
+                else dense_pipe_kernel<64, kThreads, kK, false, false, true, false><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
+            } else return hipErrorInvalidValue;
+        }
+        else if (celu && !deriv) dense_pipe_kernel<kTileCols, kThreads, kK, true, false, false, false><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
+        else if (!celu && !deriv) dense_pipe_kernel<kTileCols, kThreads, kK, false, false, false, false><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
+        else if (!celu && deriv) dense_pipe_kernel<kTileCols, kThreads, kK, false, true, false, false><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
+        else dense_pipe_kernel<kTileCols, kThreads, kK, true, true, false, false><<<pgrid, pblock, 0, stream>>>(a, run, alpha, inv_alpha);
         return hipGetLastError();
     }
     const dim3 grid(static_cast<unsigned>(run)), block(256);
-    if (celu && !deriv) dense_kernel<kTileCols, true, false><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
-    else if (!celu && !deriv) dense_kernel<kTileCols, false, false><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
-    else if (!celu && deriv) dense_kernel<kTileCols, false, true><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
-    else dense_kernel<kTileCols, true, true><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
+    if (extra == Extra::kRank1) dense_kernel<kTileCols, false, true, false, true><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
+    else if (extra == Extra::kHead) {
+        if constexpr (kTileCols == 64) {
+            if (celu) dense_kernel<64, true, false, true, false><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
+            else dense_kernel<64, false, false, true, false><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
+        } else return hipErrorInvalidValue;
+    }
+    else if (celu && !deriv) dense_kernel<kTileCols, true, false, false, false><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
+    else if (!celu && !deriv) dense_kernel<kTileCols, false, false, false, false><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
+    else if (!celu && deriv) dense_kernel<kTileCols, false, true, false, false><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
+    else dense_kernel<kTileCols, true, true, false, false><<<grid, block, 0, stream>>>(a, alpha, inv_alpha);
     return hipGetLastError();
 }
 
 template <int kTileCols>
-hipError_t launch_tiles(const DenseArgs& a, int run, bool celu, bool deriv, float alpha, hipStream_t stream)
+hipError_t launch_tiles(const DenseArgs& a, int run, bool celu, bool deriv, Extra extra, float alpha, hipStream_t stream)
 {
-    if (a.k == 384) return launch_tiles_k<kTileCols, 384>(a, run, celu, deriv, alpha, stream);
-    if (a.k == 128) return launch_tiles_k<kTileCols, 128>(a, run, celu, deriv, alpha, stream);
-    if (a.k == 64) return launch_tiles_k<kTileCols, 64>(a, run, celu, deriv, alpha, stream);
-    return launch_tiles_k<kTileCols, 0>(a, run, celu, deriv, alpha, stream);
+    if (a.k == 384) return launch_tiles_k<kTileCols, 384>(a, run, celu, deriv, extra, alpha, stream);
+    if (a.k == 128) return launch_tiles_k<kTileCols, 128>(a, run, celu, deriv, extra, alpha, stream);
+    if (a.k == 64) return launch_tiles_k<kTileCols, 64>(a, run, celu, deriv, extra, alpha, stream);
+    return launch_tiles_k<kTileCols, 0>(a, run, celu, deriv, extra, alpha, stream);
+}
+
+// fills the tile bookkeeping and launches
+hipError_t launch_filled(DenseArgs& a, const int32_t n[4], bool celu, bool deriv, Extra extra, float alpha, hipStream_t stream)
+{
+    const int tile_cols = (a.n_out % 128 == 0) ? 128 : 64;
+    a.col_tiles = a.n_out / tile_cols;
+    int64_t run = 0;
+    for (int t = 0; t < 4; ++t) {
+        a.n[t] = n[t];
+        run += static_cast<int64_t>((n[t] + kTileRows - 1) / kTileRows) * a.col_tiles;
+        a.tile_end[t] = static_cast<int>(run);
+    }
+    if (run == 0) return hipSuccess;
+    if (run > INT32_MAX) return hipErrorInvalidValue;
+    if (tile_cols == 128) return launch_tiles<128>(a, static_cast<int>(run), celu, deriv, extra, alpha, stream);
+    return launch_tiles<64>(a, static_cast<int>(run), celu, deriv, extra, alpha, stream);
 }
 
 }  // namespace
@@ -427,12 +520,9 @@ hipError_t launch_dense(const float* const rows[4], const int32_t n[4], int32_t 
                         const float* const wt[4], const float* const bias[4], bool celu, float alpha,
                         const float* const deriv_of[4], float* const out[4], hipStream_t stream)
 {
-    DenseArgs a;
-    const int tile_cols = (n_out % 128 == 0) ? 128 : 64;
+    DenseArgs a = {};
     a.k = k;
     a.n_out = n_out;
-    a.col_tiles = n_out / tile_cols;
-    int64_t run = 0;
     bool deriv = false;
     for (int t = 0; t < 4; ++t) {
         a.rows[t] = rows[t];
@@ -440,15 +530,52 @@ hipError_t launch_dense(const float* const rows[4], const int32_t n[4], int32_t 
         a.wt[t] = wt[t];
         a.bias[t] = bias ? bias[t] : nullptr;
         a.out[t] = out[t];
-        a.n[t] = n[t];
         if (n[t] > 0 && a.deriv[t]) deriv = true;
-        run += static_cast<int64_t>((n[t] + kTileRows - 1) / kTileRows) * a.col_tiles;
-        a.tile_end[t] = static_cast<int>(run);
     }
-    if (run == 0) return hipSuccess;
-    if (run > INT32_MAX) return hipErrorInvalidValue;
-    if (tile_cols == 128) return launch_tiles<128>(a, static_cast<int>(run), celu, deriv, alpha, stream);
-    return launch_tiles<64>(a, static_cast<int>(run), celu, deriv, alpha, stream);
+    return launch_filled(a, n, celu, deriv, Extra::kNone, alpha, stream);
+}
+
+// The last hidden layer (n_out = 64) together with the output layer behind it:
+// out[t] = act(rows[t] . W + b) as above, and head_out[t][r] = out[t][r, :] . head_w[t] + head_b[t][0].
+hipError_t launch_dense_head(const float* const rows[4], const int32_t n[4], int32_t k, int32_t n_out,
+                             const float* const wt[4], const float* const bias[4], bool celu, float alpha,
+                             const float* const head_w[4], const float* const head_b[4], float* const out[4],
+                             float* const head_out[4], hipStream_t stream)
+{
+    if (n_out != 64) return hipErrorInvalidValue;
+    DenseArgs a = {};
+    a.k = k;
+    a.n_out = n_out;
+    for (int t = 0; t < 4; ++t) {
+        a.rows[t] = rows[t];
+        a.wt[t] = wt[t];
+        a.bias[t] = bias ? bias[t] : nullptr;
+        a.out[t] = out[t];
+        a.head_w[t] = head_w[t];
+        a.head_b[t] = head_b ? head_b[t] : nullptr;
+        a.head_out[t] = head_out[t];
+    }
+    return launch_filled(a, n, celu, false, Extra::kHead, alpha, stream);
+}
+
+// The way back through the output layer and the last hidden layer (weights W [n_out, k] as stored, CELU outputs h):
+// out[t] = (scale[t][r] * head_w[t][c] * CELU'(h[t][r, c])) . W^T-as-stored, i.e. the gradient with respect to the
+// last hidden layer's input, given the gradient `scale` with respect to each row's output value.
+hipError_t launch_dense_head_grad(const float* const scale[4], const float* const head_w[4], const int32_t n[4], int32_t k,
+                                  int32_t n_out, const float* const wt[4], float alpha, const float* const deriv_of[4],
+                                  float* const out[4], hipStream_t stream)
+{
+    DenseArgs a = {};
+    a.k = k;
+    a.n_out = n_out;
+    for (int t = 0; t < 4; ++t) {
+        a.scale[t] = scale[t];
+        a.head_w[t] = head_w[t];
+        a.deriv[t] = deriv_of[t];
+        a.wt[t] = wt[t];
+        a.out[t] = out[t];
+    }
+    return launch_filled(a, n, false, true, Extra::kRank1, alpha, stream);
 }
 
 hipError_t launch_dense_first(const float* const rows[4], const int32_t n[4], const float* const wt[4],

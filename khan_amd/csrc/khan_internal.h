@@ -100,6 +100,15 @@ hipError_t launch_zero(T* a, int64_t n, hipStream_t stream);
 hipError_t launch_dense(const float* const rows[4], const int32_t n[4], int32_t k, int32_t n_out,
                         const float* const wt[4], const float* const bias[4], bool celu, float alpha,
                         const float* const deriv_of[4], float* const out[4], hipStream_t stream);
+// the last hidden layer (n_out = 64) with the output layer folded into its epilogue: head_out[t][r] = out[t][r, :] . head_w[t] + head_b[t][0]
+hipError_t launch_dense_head(const float* const rows[4], const int32_t n[4], int32_t k, int32_t n_out,
+                             const float* const wt[4], const float* const bias[4], bool celu, float alpha,
+                             const float* const head_w[4], const float* const head_b[4], float* const out[4],
+                             float* const head_out[4], hipStream_t stream);
+// and the way back: rows built from scale[t][r] * head_w[t][c] * CELU'(deriv_of[t][r, c])
+hipError_t launch_dense_head_grad(const float* const scale[4], const float* const head_w[4], const int32_t n[4], int32_t k,
+                                  int32_t n_out, const float* const wt[4], float alpha, const float* const deriv_of[4],
+                                  float* const out[4], hipStream_t stream);
 hipError_t launch_dense_first(const float* const rows[4], const int32_t n[4], const float* const wt[4],
                               const float* const bias[4], bool celu, float alpha, float* const out[4],
                               hipStream_t stream);

@@ -122,7 +122,8 @@ class MoleculeNN:
     def kernel_layers(self):
         """How many leading layers run in this package's matrix-core kernel (`ops.dense`): float32 on the GPU, CELU
         with its default alpha, input width a multiple of 32 and output width a multiple of 64 -- for the reference's
-        default network 384-128-128-64-1 all but the last."""
+        default network 384-128-128-64-1 all but the last, which `atom_outputs` folds into the launch of the one
+        before it (`ops.dense_head`)."""
         if not (self.first_layer_kernel and self.dtype == torch.float32 and self.device.type == "cuda"
                 and self.activation_fn is celu):
             return 0
@@ -142,11 +143,20 @@ class MoleculeNN:
             # coordinates' gradient was asked for, and would form the weights' gradient, a second product, every time)
             par = (lambda k: self.params[k]) if self.weights_need_grad else (lambda k: self.params[k].detach())
             a = atom_type_features
-            for k in range(nk):
+            # the output layer rides in the last hidden layer's launch when that layer is a kernel layer of width 64
+            fuse_head = nk == len(self.layer_sizes) - 2 and self.layer_sizes[-2] == 64
+            for k in range(nk - 1 if fuse_head else nk):
                 rows = [self.names[t][k] for t in TYPE_MAP]
                 a = autograd.dense(a, [par(r[0]) for r in rows], [par(r[1]) for r in rows], alpha=0.1,
                                    weights_t=self.layer_transposed(k))
-            outs = [self.atom_type_outputs(t, a[t], layers_done=nk) for t in range(4)]
+            if fuse_head:
+                rows = [self.names[t][nk - 1] for t in TYPE_MAP]
+                head = [self.names[t][nk] for t in TYPE_MAP]
+                outs = autograd.dense_head(a, [par(r[0]) for r in rows], [par(r[1]) for r in rows],
+                                           [par(r[0]) for r in head], [par(r[1]) for r in head], alpha=0.1,
+                                           weights_t=self.layer_transposed(nk - 1))
+            else:
+                outs = [self.atom_type_outputs(t, a[t], layers_done=nk) for t in range(4)]
         else:
             outs = [self.atom_type_outputs(t, f.reshape(-1, FEATURE_SIZE)) for t, f in enumerate(atom_type_features)]
         # gather_idxs is a permutation: index_select's backward is a scatter-add, where indexing with [] sorts the

@@ -301,21 +301,11 @@ def dense(inputs, weights_nk, biases=None, activation=ACT_NONE, alpha=0.1, deriv
     lib = _lib.load()
     n_out, k = (int(v) for v in weights_nk[0].shape)
     rows, ders, wts, bs, outs, ns = [], [], [], [], [], []
-
-    def matrix(x, name):
-        if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dtype != torch.float32:
-            raise TypeError("%s must be a float32 CUDA tensor" % name)
-        if x.dim() != 2 or x.shape[1] != k or not x.is_contiguous():
-            raise ValueError("%s must be a contiguous [n, %d] tensor, got %s" % (name, k, tuple(x.shape)))
-        return x
-
     for t in range(4):
-        r = matrix(inputs[t], "inputs[%d]" % t)
-        w = weights_nk[t]
-        if tuple(w.shape) != (n_out, k) or w.dtype != torch.float32 or not w.is_contiguous() or not w.is_cuda:
-            raise ValueError("weights_nk[%d] must be a contiguous float32 CUDA tensor of shape [%d, %d]" % (t, n_out, k))
+        r = _dense_matrix(inputs[t], k, "inputs[%d]" % t)
+        wts.append(_dense_weights(weights_nk[t], n_out, k, "weights_nk[%d]" % t))
         if deriv_of is not None:
-            d = matrix(deriv_of[t], "deriv_of[%d]" % t)
+            d = _dense_matrix(deriv_of[t], k, "deriv_of[%d]" % t)
             if d.shape[0] != r.shape[0]:
                 raise ValueError("deriv_of[%d] must be shaped like inputs[%d]" % (t, t))
             ders.append(d)
@@ -324,12 +314,91 @@ def dense(inputs, weights_nk, biases=None, activation=ACT_NONE, alpha=0.1, deriv
             if b.numel() != n_out:
                 raise ValueError("bias %d must have %d elements" % (t, n_out))
             bs.append(b)
-        rows.append(r); wts.append(w); ns.append(int(r.shape[0]))
+        rows.append(r); ns.append(int(r.shape[0]))
         outs.append(torch.empty((r.shape[0], n_out), dtype=torch.float32, device=r.device))
-    arr = lambda ts: (ctypes.c_void_p * 4)(*[t.data_ptr() if t.numel() else None for t in ts])
-    _lib.check(lib.khan_dense_f32(arr(rows), (ctypes.c_int32 * 4)(*ns), k, n_out, arr(wts),
-                                  arr(bs) if biases is not None else None, int(activation), float(alpha),
-                                  arr(ders) if deriv_of is not None else None, arr(outs), _stream()))
+    _lib.check(lib.khan_dense_f32(_ptr4(rows), (ctypes.c_int32 * 4)(*ns), k, n_out, _ptr4(wts),
+                                  _ptr4(bs) if biases is not None else None, int(activation), float(alpha),
+                                  _ptr4(ders) if deriv_of is not None else None, _ptr4(outs), _stream()))
+    return tuple(outs)
+
+
+def _dense_matrix(x, k, name):
+    if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dtype != torch.float32:
+        raise TypeError("%s must be a float32 CUDA tensor" % name)
+    if x.dim() != 2 or x.shape[1] != k or not x.is_contiguous():
+        raise ValueError("%s must be a contiguous [n, %d] tensor, got %s" % (name, k, tuple(x.shape)))
+    return x
+
+
+def _dense_weights(w, n_out, k, name):
+    if tuple(w.shape) != (n_out, k) or w.dtype != torch.float32 or not w.is_contiguous() or not w.is_cuda:
+        raise ValueError("%s must be a contiguous float32 CUDA tensor of shape [%d, %d]" % (name, n_out, k))
+    return w
+
+
+def _ptr4(ts):
+    return (ctypes.c_void_p * 4)(*[t.data_ptr() if t.numel() else None for t in ts])
+
+
+def dense_head(inputs, weights_nk, biases, head_weights, head_biases=None, activation=ACT_CELU, alpha=0.1):
+    """The last hidden layer of the four atomic networks (width 64) with the output layer (64 -> 1, no activation)
+    folded into the same launch, float32: -> (outs, head_outs), outs[t] = act(inputs[t] . W_t + b_t) as `dense`
+    gives it ([n_t, 64]; the way back needs it) and head_outs[t][r] = outs[t][r, :] . head_weights[t] + head_biases[t]
+    ([n_t]).  `weights_nk[t]` is [64, k]; `head_weights[t]` has 64 elements, `head_biases[t]` one."""
+    lib = _lib.load()
+    n_out, k = (int(v) for v in weights_nk[0].shape)
+    if n_out != 64:
+        raise ValueError("the fused output layer needs a last hidden layer of width 64, got %d" % n_out)
+    rows, wts, bs, hws, hbs, outs, houts, ns = [], [], [], [], [], [], [], []
+    for t in range(4):
+        r = _dense_matrix(inputs[t], k, "inputs[%d]" % t)
+        wts.append(_dense_weights(weights_nk[t], n_out, k, "weights_nk[%d]" % t))
+        if biases is not None:
+            b = _dev(biases[t], torch.float32, "bias")
+            if b.numel() != n_out:
+                raise ValueError("bias %d must have %d elements" % (t, n_out))
+            bs.append(b)
+        hw = _dev(head_weights[t].reshape(-1), torch.float32, "head_weights")
+        if hw.numel() != n_out:
+            raise ValueError("head_weights[%d] must have %d elements" % (t, n_out))
+        hws.append(hw)
+        if head_biases is not None:
+            hb = _dev(head_biases[t].reshape(-1), torch.float32, "head_biases")
+            if hb.numel() != 1:
+                raise ValueError("head_biases[%d] must have one element" % t)
+            hbs.append(hb)
+        rows.append(r); ns.append(int(r.shape[0]))
+        outs.append(torch.empty((r.shape[0], n_out), dtype=torch.float32, device=r.device))
+        houts.append(torch.empty((r.shape[0],), dtype=torch.float32, device=r.device))
+    _lib.check(lib.khan_dense_head_f32(_ptr4(rows), (ctypes.c_int32 * 4)(*ns), k, n_out, _ptr4(wts),
+                                       _ptr4(bs) if biases is not None else None, int(activation), float(alpha),
+                                       _ptr4(hws), _ptr4(hbs) if head_biases is not None else None, _ptr4(outs),
+                                       _ptr4(houts), _stream()))
+    return tuple(outs), tuple(houts)
+
+
+def dense_head_grad(scales, head_weights, weights_nk, deriv_of, alpha=0.1):
+    """The way back through the output layer and the last hidden layer, float32, one launch: given scales[t] ([n_t],
+    the gradient with respect to each row's output value), -> four [n_t, n_out] tensors
+    (scales[t][:, None] * head_weights[t][None, :] * CELU'(z)) . W_t, CELU(z) = deriv_of[t] ([n_t, k], the hidden
+    layer's activations); `weights_nk[t]` is [n_out, k], the hidden layer's weights as stored (input width x layer
+    width).  The outer product is formed inside the kernel."""
+    lib = _lib.load()
+    n_out, k = (int(v) for v in weights_nk[0].shape)
+    scs, hws, wts, ders, outs, ns = [], [], [], [], [], []
+    for t in range(4):
+        d = _dense_matrix(deriv_of[t], k, "deriv_of[%d]" % t)
+        sc = _dev(scales[t].reshape(-1), torch.float32, "scales")
+        if sc.numel() != d.shape[0]:
+            raise ValueError("scales[%d] must have %d elements" % (t, d.shape[0]))
+        hw = _dev(head_weights[t].reshape(-1), torch.float32, "head_weights")
+        if hw.numel() != k:
+            raise ValueError("head_weights[%d] must have %d elements" % (t, k))
+        wts.append(_dense_weights(weights_nk[t], n_out, k, "weights_nk[%d]" % t))
+        scs.append(sc); hws.append(hw); ders.append(d); ns.append(int(d.shape[0]))
+        outs.append(torch.empty((d.shape[0], n_out), dtype=torch.float32, device=d.device))
+    _lib.check(lib.khan_dense_head_grad_f32(_ptr4(scs), _ptr4(hws), (ctypes.c_int32 * 4)(*ns), k, n_out, _ptr4(wts),
+                                            float(alpha), _ptr4(ders), _ptr4(outs), _stream()))
     return tuple(outs)
 
 

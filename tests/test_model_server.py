@@ -345,6 +345,58 @@ def test_dense_kernel_shapes_forward_and_data_gradient(k, n_out):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("k", [128, 192, 64])
+def test_output_layer_folded_into_the_last_hidden_layer(k):
+    """khan_dense_head_f32 / khan_dense_head_grad_f32 (the 64 -> 1 output layer inside the launch of the 64-wide layer
+    before it, both ways) against float64 numpy: row counts on and off the 128-row tile, an empty type, with and
+    without the output layer's bias, and no activation in the hidden layer."""
+    from khan_amd import ops
+    dev = "cuda:0"
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a.astype(np.float32))).to(dev)
+    rng = np.random.default_rng(7000 + k)
+    ns = [300, 0, 129, 1]
+    xs = [rng.standard_normal((n, k)) for n in ns]
+    Wt = [rng.standard_normal((64, k)) * (2.0 / (k + 64)) ** 0.5 for _ in range(4)]
+    bs = [rng.standard_normal(64) * 0.1 for _ in range(4)]
+    hw = [rng.standard_normal(64) * 0.2 for _ in range(4)]
+    hb = [rng.standard_normal(1) for _ in range(4)]
+    f32 = lambda a: a.astype(np.float32).astype(np.float64)
+    for act, with_hb in ((ops.ACT_CELU, True), (ops.ACT_CELU, False), (ops.ACT_NONE, True)):
+        outs, heads = ops.dense_head([d(x) for x in xs], [d(w) for w in Wt], [d(v) for v in bs], [d(v) for v in hw],
+                                     [d(v) for v in hb] if with_hb else None, act, 0.1)
+        plain = ops.dense([d(x) for x in xs], [d(w) for w in Wt], [d(v) for v in bs], act, 0.1)
+        for t in range(4):
+            x, w, b_, v, c = f32(xs[t]), f32(Wt[t]), f32(bs[t]), f32(hw[t]), f32(hb[t])
+            z = x @ w.T + b_
+            h = nn_ref._celu(z) if act == ops.ACT_CELU else z
+            want = h @ v + (c[0] if with_hb else 0.0)
+            assert torch.equal(outs[t], plain[t]), t                      # the hidden activations are the plain layer's
+            got = heads[t].cpu().numpy().astype(np.float64)
+            assert got.shape == (ns[t],)
+            if ns[t]:
+                mag = (np.abs(x) @ np.abs(w.T) + np.abs(b_)) @ np.abs(v) + abs(c[0])
+                assert np.all(np.isfinite(got)) and np.all(np.abs(got - want) <= 2e-6 * mag + 1e-7), (t, np.abs(got - want).max())
+    # the way back: scale[r] * head_w[c] * CELU'(h[r, c]), times the hidden layer's weights as stored ([n_in, 64])
+    n_in = 128
+    Wst = [rng.standard_normal((n_in, 64)) * (2.0 / (n_in + 64)) ** 0.5 for _ in range(4)]
+    hs = [rng.standard_normal((n, 64)) * 0.2 for n in ns]
+    sc = [rng.standard_normal(n) for n in ns]
+    got4 = ops.dense_head_grad([d(v) for v in sc], [d(v) for v in hw], [d(w) for w in Wst], [d(h) for h in hs], 0.1)
+    two_step = ops.dense([d(sc[t][:, None] * hw[t][None, :]) for t in range(4)], [d(w) for w in Wst], None, ops.ACT_NONE, 0.1,
+                         deriv_of=[d(h) for h in hs])
+    for t in range(4):
+        s_, v, h, w = f32(sc[t]), f32(hw[t]), f32(hs[t]), f32(Wst[t])
+        up = s_[:, None] * v[None, :] * np.where(h >= 0, 1.0, h / 0.1 + 1.0)
+        want = up @ w.T
+        got = got4[t].cpu().numpy().astype(np.float64)
+        assert got.shape == (ns[t], n_in)
+        if ns[t]:
+            mag = np.abs(up) @ np.abs(w.T)
+            assert np.all(np.isfinite(got)) and np.all(np.abs(got - want) <= 2e-6 * mag + 1e-7), (t, np.abs(got - want).max())
+            assert np.all(np.abs(got - two_step[t].cpu().numpy()) <= 2e-6 * mag + 1e-7)
+
+
+@pytest.mark.gpu
 def test_kernel_layers_agree_with_library_layers_in_energy_and_gradient():
     """The float32 model with its CELU layers in khan_dense_f32 against the same model with every layer a library
     product: energies and coordinate gradients of 200 molecules."""
