@@ -8,36 +8,35 @@ namespace khan {
 
 // LDS working set of one wavefront
 // what the Jacobian-vector variant keeps on top of the forward working set
-template <typename T, bool kJvp, int kNB> struct FwdJvpLds {};
-template <typename T, int kNB> struct __align__(16) FwdJvpLds<T, true, kNB> {
+template <typename T, bool kJvp, int kNB, int kRadN> struct FwdJvpLds {};
+template <typename T, int kNB, int kRadN> struct __align__(16) FwdJvpLds<T, true, kNB, kRadN> {
     typename Fast<T>::vec4 vel[64];               // the incoming vector of every atom (sorted order)
     typename Fast<T>::vec4 nbr_p[kNB][kCapA];      // (v_centre - v_partner)/r, and its component along the unit vector
     typename Fast<T>::vec2 nbr_d[kNB][kCapA];      // f_C'(r) dr, and dr = change of the distance along the vectors
-    typename Fast<T>::vec2 rad_ab[64];            // radial entries: f_C' dr, and -2 eta f_C dr
+    typename Fast<T>::vec2 rad_ab[kRadN];         // radial entries: f_C' dr, and -2 eta f_C dr
     T rec2[64][12];                               // phase-1 records: dA_0..7, H_0..3
 };
 
 // LDS working set of one wavefront, for batches of kNB centres
-template <typename T, bool kJvp = false, int kNB = kFB>
+template <typename T, bool kJvp = false, int kNB = kFB, int kRadN = 64>
 struct __align__(16) FwdWaveLds {
     static constexpr int kCentres = kNB;
     typename Fast<T>::vec4 nbr[kNB][kCapA];    // unit vector (centre minus partner)/r, and r
     T nbr_fc[kNB][kCapA];                      // f_C(r, A_Rc)
-    typename Fast<T>::vec2 rad[64];           // (r, f_C(r, R_Rc)); group g of a scan step owns [g*W, (g+1)*W)
+    typename Fast<T>::vec2 rad[kRadN];        // (r, f_C(r, R_Rc)) of the radial partners of a scan step's centres
     T rec[64][12];                            // phase-1 records: A_0..7, G_0..3
     SegDesc seg[64];                          // non-empty segments of the batch, in order
     unsigned long long segrow[64];            // where each of them puts its 32 output values
     unsigned bits[bit_words(kNB)];            // bit per triple slot: a segment starts here
     int nA[kNB][4];                            // angular partners per type, per centre of the batch
-    int nR[4][4];                             // radial partners per type, per group of the scan step
-    FwdJvpLds<T, kJvp, kNB> jvp;
+    FwdJvpLds<T, kJvp, kNB, kRadN> jvp;
 };
 
 // Padding slots of phase 1 read entry 0 of centre 0's list whatever it holds; their products are cancelled by a
 // zero radial factor, which needs every other factor finite.  Entry 0 is either a partner written by a scan or
 // what this writes once per wavefront before the first batch.
-template <typename T, bool kJvp, int kNB>
-__device__ __forceinline__ void fwd_lds_init(FwdWaveLds<T, kJvp, kNB>& S, int lane)
+template <typename T, bool kJvp, int kNB, int kRadN>
+__device__ __forceinline__ void fwd_lds_init(FwdWaveLds<T, kJvp, kNB, kRadN>& S, int lane)
 {
     if (lane == 0) {
         S.nbr[0][0] = Fast<T>::make4(T(0), T(0), T(0), T(0));
@@ -59,8 +58,8 @@ __device__ __forceinline__ void fwd_lds_init(FwdWaveLds<T, kJvp, kNB>& S, int la
 // segment's records of A_t G_s is the product of an 8 x K by a K x 4 matrix, and v_mfma_f32_16x16x4_f32 takes four
 // records (K = 4) per instruction, using an 8 x 4 corner of its 16 x 16 result.  The variant exists to be measured
 // against the vector form; the launcher selects it on request only.
-template <bool kMatrixPhase2, typename T, bool kJvp, int kNB, typename RowOfCentre>
-__device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB>& S, const LaneConsts<T>& L, int lane, int nb,
+template <bool kMatrixPhase2, typename T, bool kJvp, int kNB, int kRadN, typename RowOfCentre>
+__device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB, kRadN>& S, const LaneConsts<T>& L, int lane, int nb,
                                                   RowOfCentre row_of_centre)
 {
     static_assert(kNB * kNumPairBlocks <= 64, "one segment-table lane per (centre, type pair)");

@@ -34,6 +34,10 @@ namespace {
 // radial list entries a lane takes per trip: each type's entries are padded to a multiple of this (times the
 // number of slots), and two measured faster than one, three or four
 constexpr int kRadTrip = 2;
+// Entries of the radial lists of one scan step.  A group's list has a fixed place for every partner type, each as
+// long as the molecule's number of atoms of that type rounded up to a whole trip of the walk: 16 + 4, 32 + 12 or
+// 64 + 28 entries per group for 4, 2 or 1 groups.
+constexpr int kRadSlots = 96;
 
 // With kJvp the kernel computes the Jacobian-vector product instead (featurize_grad_inverse): every term of
 // the forward sums is replaced by its derivative along the per-atom vectors (VX, VY, VZ).
@@ -51,7 +55,7 @@ void aev_fwd_small_kernel(
 {
     typedef typename Fast<T>::vec4 vec4;
     typedef typename Fast<T>::vec2 vec2;
-    __shared__ FwdWaveLds<T, kJvp> lds_all[kWavesPerBlock];
+    __shared__ FwdWaveLds<T, kJvp, kFB, kRadSlots> lds_all[kWavesPerBlock];
     const int lane = threadIdx.x & 63;
     const int wave = kWavesPerBlock == 1 ? 0 : uniform(threadIdx.x >> 6);    // a constant LDS base with one wavefront per workgroup
     const int slot = blockIdx.x * kWavesPerBlock + wave;
@@ -60,7 +64,7 @@ void aev_fwd_small_kernel(
     const int n = uniform(MACs[mol]);
     const int off = uniform(MOs[mol]);
     if (n <= 0 || n > max_atoms) return;          // larger molecules belong to other kernels (max_atoms <= 64)
-    FwdWaveLds<T, kJvp>& S = lds_all[wave];
+    FwdWaveLds<T, kJvp, kFB, kRadSlots>& S = lds_all[wave];
     const LaneConsts<T> L = lane_consts<T>(lane);
     const unsigned long long lane_bit = 1ull << lane;
     const unsigned long long lt_mask = lane_bit - 1ull;
@@ -144,6 +148,19 @@ void aev_fwd_small_kernel(
     const int rg_ns = 4 / G;                                   // 1, 2 or 4
     const int rg_g = G == 4 ? rg : G == 2 ? (rg >> 1) : 0;
     const int rg_s = G == 4 ? 0 : G == 2 ? (rg & 1) : rg;
+    // Radial lists: type a's entries of a group start at rbase[a] whatever the centre, and the list is cleared before
+    // every step, so the walk reads whole trips without asking how many entries a centre has: an entry that was not
+    // written has f_C = 0.  A partner's place is rbase[its type] + the number of in-range partners of that type
+    // before it in its group.
+    const int rad_unit = kRadTrip * rg_ns;
+    const int rad_stride = kRadSlots >> (6 - logW);             // entries per group: 24, 48 or 96
+    int rbase[4];
+    rbase[0] = 0;
+#pragma unroll
+    for (int a = 1; a < 4; ++a) rbase[a] = rbase[a - 1] + ((tcount[a - 1] + rad_unit - 1) & -rad_unit);
+    const int tj = __builtin_amdgcn_ds_bpermute(jl << 2, type);
+    const int rad_pos0 = grp * rad_stride + sel4(tj, rbase[0], rbase[1], rbase[2], rbase[3]);
+    const unsigned long long rad_mask = lt_mask & (~0ull << ((grp * W + sel4(tj, tbase[0], tbase[1], tbase[2], tbase[3])) & 63));
     // the sorted atoms stay in the lanes' registers: the partner this lane tests in every scan step, once; the
     // step's centres by lane exchange
     const T xj = lane_fetch(x, jl << 2), yj = lane_fetch(y, jl << 2), zj = lane_fetch(z, jl << 2);
@@ -161,6 +178,10 @@ void aev_fwd_small_kernel(
             const int i = c0 + b;
             const bool centre_ok = b < nb;
             const int ci = (centre_ok ? i : 0) << 2;
+            for (int e = lane; e < kRadSlots; e += 64) {
+                S.rad[e] = Fast<T>::make2(T(0), T(0));
+                if constexpr (kJvp) S.jvp.rad_ab[e] = Fast<T>::make2(T(0), T(0));
+            }
             const T dx = lane_fetch(x, ci) - xj, dy = lane_fetch(y, ci) - yj, dz = lane_fetch(z, ci) - zj;
             const T r = Fast<T>::sqrt_rn(dx * dx + dy * dy + dz * dz);
             const bool valid = centre_ok && (jl < n) && (jl != i);
@@ -180,7 +201,7 @@ void aev_fwd_small_kernel(
                 rd = (dx * wx + dy * wy + dz * wz) * inv;
             }
             if (inR) {
-                const int pos = grp * W + popc64(mR & ltg_mask);
+                const int pos = rad_pos0 + popc64(mR & rad_mask);
                 if constexpr (kJvp) {
                     T fc, dfc;
                     Fast<T>::cutoff_grad(r, static_cast<T>(kR_Rc_f), fc, dfc);
@@ -214,7 +235,6 @@ void aev_fwd_small_kernel(
                 const int cb = b0 + cl_g;
                 cntR = popc64(mR & cl_mask);
                 if (cb < nb) S.nA[cb][cl_a] = (popc64(mA & cl_sub) <= kCapA) ? popc64(mA & cl_mask) : 0;
-                S.nR[cl_g][cl_a] = cntR;
             }
             // largest radial count of each type over the groups of this step (lanes 0..15 hold them)
             int mx = cntR;
@@ -225,41 +245,36 @@ void aev_fwd_small_kernel(
 
             // ---- radial features of the G centres of this step
             {
-                const int4 cn = *reinterpret_cast<const int4*>(S.nR[rg_g]);
-                const vec2* list = &S.rad[rg_g * W];
+                const vec2* list = &S.rad[rg_g * rad_stride + rg_s];
                 const int cb = b0 + rg_g;
                 const int ci = min(c0 + cb, 63);
                 const unsigned rlo = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(ci << 2, rp_lo));
                 const unsigned rhi = static_cast<unsigned>(__builtin_amdgcn_ds_bpermute(ci << 2, rp_hi));
                 T* row = reinterpret_cast<T*>((static_cast<unsigned long long>(rhi) << 32) | rlo);
-                int obase = 0;
 #pragma unroll
                 for (int a = 0; a < 4; ++a) {
-                    const int cnt_a = a == 0 ? cn.x : a == 1 ? cn.y : a == 2 ? cn.z : cn.w;
                     T acc_r = T(0);
-                    for (int q0 = 0; q0 < (kSkipRadial ? 0 : mxR[a]); q0 += kRadTrip * rg_ns) {
+                    const vec2* pl = list + rbase[a];
+                    for (int q0 = 0; q0 < (kSkipRadial ? 0 : mxR[a]); q0 += rad_unit) {
                         // kRadTrip entries of this lane's slot per trip; slot s takes q = s, s+ns, s+2ns, ...
                         vec2 e[kRadTrip], ab[kRadTrip];
 #pragma unroll
                         for (int u = 0; u < kRadTrip; ++u) {
-                            const int at = min(obase + q0 + u * rg_ns + rg_s, W - 1);
-                            e[u] = list[at];
-                            if constexpr (kJvp) ab[u] = S.jvp.rad_ab[rg_g * W + at];
+                            e[u] = pl[q0 + u * rg_ns];
+                            if constexpr (kJvp) ab[u] = S.jvp.rad_ab[rg_g * rad_stride + rg_s + rbase[a] + q0 + u * rg_ns];
                         }
 #pragma unroll
                         for (int u = 0; u < kRadTrip; ++u) {
                             const T dd = e[u].x - L.rrs;
                             // forward: exp(-eta d^2) f_C; derivative: exp(-eta d^2) (f_C' - 2 eta d f_C) dr
-                            T v = Fast<T>::gauss(static_cast<T>(kR_eta_f), dd);
-                            if constexpr (kJvp) v *= fma(ab[u].y, dd, ab[u].x);
-                            else v *= e[u].y;
-                            acc_r += (q0 + u * rg_ns + rg_s < cnt_a) ? v : T(0);   // stale entries: select
+                            const T v = Fast<T>::gauss(static_cast<T>(kR_eta_f), dd);
+                            if constexpr (kJvp) acc_r = fma(v, fma(ab[u].y, dd, ab[u].x), acc_r);
+                            else acc_r = fma(v, e[u].y, acc_r);
                         }
                     }
                     if (rg_ns >= 2) acc_r += __shfl_xor(acc_r, 16, 64);
                     if (rg_ns == 4) acc_r += __shfl_xor(acc_r, 32, 64);
                     if (rg_s == 0 && cb < nb) store_global(row + a * kNumRRs + (lane & 15), acc_r);
-                    obase += cnt_a;
                 }
             }
             wave_lds_fence();
