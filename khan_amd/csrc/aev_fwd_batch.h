@@ -104,7 +104,9 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB, kRadN
     const int start = incl - padded;
     const int total = kSkipAngular ? 0 : lane_read(incl, 63);            // triple slots in this batch (even)
     const unsigned long long nonempty = wave_ballot(cnt > 0);
-    for (int w = lane; w < bit_words(kNB); w += 64) S.bits[w] = 0u;
+    // (lanes past the last word write the last word again: no loop, no branch)
+#pragma unroll
+    for (int w0 = 0; w0 < bit_words(kNB); w0 += 64) S.bits[min(w0 + lane, bit_words(kNB) - 1)] = 0u;
     wave_lds_fence();
     if (cnt > 0) {
         mine.start_cnt = static_cast<unsigned>(start) | (static_cast<unsigned>(cnt) << 16);

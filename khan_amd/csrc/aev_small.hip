@@ -178,9 +178,13 @@ void aev_fwd_small_kernel(
             const int i = c0 + b;
             const bool centre_ok = b < nb;
             const int ci = (centre_ok ? i : 0) << 2;
-            for (int e = lane; e < kRadSlots; e += 64) {
-                S.rad[e] = Fast<T>::make2(T(0), T(0));
-                if constexpr (kJvp) S.jvp.rad_ab[e] = Fast<T>::make2(T(0), T(0));
+            // clears the lists: every lane two entries (the upper half of the wavefront repeats the lower half's second one)
+            static_assert(kRadSlots == 96, "64 + 32 entries");
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int at = e == 0 ? lane : 64 + (lane & 31);
+                S.rad[at] = Fast<T>::make2(T(0), T(0));
+                if constexpr (kJvp) S.jvp.rad_ab[at] = Fast<T>::make2(T(0), T(0));
             }
             const T dx = lane_fetch(x, ci) - xj, dy = lane_fetch(y, ci) - yj, dz = lane_fetch(z, ci) - zj;
             const T r = Fast<T>::sqrt_rn(dx * dx + dy * dy + dz * dz);

@@ -667,6 +667,43 @@ def test_crowded_centres_take_the_fallback(ops):
     check_forward_backward(ops, c)
 
 
+def test_radial_lists_at_their_fullest(ops):
+    # The one-wavefront forward kernel gives every partner type a place of its own in a centre's radial list, each
+    # rounded up to a whole trip of the walk.  Fullest lists: molecules of exactly 16, 32 and 64 atoms (the three scan
+    # shapes) with an odd number of atoms of every type, packed so that every atom is inside every other atom's
+    # radial cutoff; beside them single-type molecules and one with a type that no atom has.
+    say("case: radial lists at their fullest (16 / 32 / 64 atoms, odd type counts, everything inside the cutoff)")
+    rng = np.random.default_rng(77)
+    mols = []
+    for counts in ((5, 5, 3, 3), (9, 9, 7, 7), (17, 17, 15, 15), (1, 1, 1, 13), (16, 0, 0, 0), (0, 31, 1, 0), (3, 0, 5, 7)):
+        n = sum(counts)
+        types = rng.permutation(np.repeat(np.arange(4), counts))
+        if n < 64:
+            mols.append((types, _packed_ball(rng, n, 2.25, 0.8)))
+        else:
+            # 64 atoms on a sphere of 4.58 A diameter: 63 radial partners each, and no more than 32 inside the
+            # angular cutoff, so that the lists are used and not the fallback for crowded centres
+            pts = []
+            while len(pts) < n:
+                v = rng.standard_normal(3)
+                v *= 2.29 / np.linalg.norm(v)
+                if all(np.linalg.norm(v - q) >= 0.8 for q in pts):
+                    pts.append(v)
+            pts = np.array(pts)
+            dm = np.linalg.norm(pts[:, None] - pts[None], axis=2)
+            assert ((dm < 3.1) & (dm > 0)).sum(axis=1).max() <= 32
+            mols.append((types, pts))
+    A = np.concatenate([m[0] for m in mols]).astype(np.int32)
+    xyz = np.concatenate([m[1] for m in mols])
+    mi = np.concatenate([np.full(len(m[0]), k) for k, m in enumerate(mols)]).astype(np.int32)
+    for types, p in mols:
+        dm = np.linalg.norm(p[:, None] - p[None], axis=2)
+        assert dm.max() < 4.6                       # the premise: every pair is a radial pair
+    c = Case(xyz[:, 0], xyz[:, 1], xyz[:, 2], A, mi, len(mols))
+    check_forward_backward(ops, c)
+    _check_grad_inverse(ops, c)
+
+
 # ----------------------------------------------------------------------------- full-size batch
 def test_full_size_batch_properties(ops):
     # 65,536 molecules (the benchmark batch) in float32: properties that need no oracle at full size, plus
