@@ -24,6 +24,8 @@
 // a sum over the tile's 64 columns = over the 32 lanes that hold a row's values.  kRank1: on the way back the
 // gradient with respect to the last hidden layer's activations is the outer product scale[r] * head_w[c]; the
 // staging builds it in registers instead of reading a matrix that something else would have had to write.
+#include <cstdlib>
+#include <cstring>
 #include "khan_internal.h"
 #include "khan_params.h"
 
@@ -432,6 +434,204 @@ void dense_pipe_kernel(DenseArgs args, int total_tiles, float alpha, float inv_a
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The same float32 product on the bfloat16 matrix instructions, which run sixteen times as fast as the float32 ones.
+// Every float32 operand is split exactly into three bfloat16 values, x = x1 + x2 + x3 (8 + 8 + 8 significant bits:
+// x1 = bf16(x), x2 = bf16(x - x1), x3 = bf16(x - x1 - x2); both differences are exact in float32), and of the nine
+// partial products of x w the six largest are formed, each an exact 16-bit product accumulated in float32:
+//     x w ~ x1 w1 + x1 w2 + x2 w1 + x2 w2 + x1 w3 + x3 w1.
+// What is left out (x2 w3 + x3 w2 + x3 w3) is below 2^-23 |x w| (measured: 3e-9 of sum |x| |w| on a 384-term sum, against
+// 3e-7 for the rounding of the float32 accumulation itself), so the result is a float32 matrix product to float32
+// accuracy: six matrix instructions of 32 x 32 x 16 in place of eight of 32 x 32 x 2, at 32 instead of 64 cycles each.
+// The splitting happens while a chunk is staged (rows: after the activation's derivative has been multiplied in; the
+// weights likewise, in every workgroup: no second copy of the weights has to be kept).  In LDS a chunk is three planes
+// of [row or column][32 k] bfloat16, rows 80 bytes apart (16-byte reads without bank conflicts).
+// Eight wavefronts (128 columns) or four (64 columns) per workgroup, 32 rows x 64 columns each; one LDS buffer: the next
+// chunk's global loads are in flight during the products, and the workgroups that share a CU alternate.
+constexpr int kSplitStride = 40;       // bfloat16 elements between staged rows: 32 + 8
+
+typedef unsigned u2v __attribute__((ext_vector_type(2)));
+typedef unsigned u4v __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f2v __attribute__((ext_vector_type(2)));
+
+template <int kTileCols>
+struct __align__(16) SplitLds {
+    unsigned short a[3][kTileRows][kSplitStride];
+    unsigned short b[3][kTileCols][kSplitStride];
+};
+
+// two floats -> their three bfloat16 parts, each pair packed into one register (first value in the low half)
+__device__ __forceinline__ void split_pair(float x0, float x1, unsigned& p1, unsigned& p2, unsigned& p3)
+{
+    p1 = __builtin_bit_cast(unsigned, __builtin_convertvector(f2v{x0, x1}, bf16x2));
+    const float r0 = x0 - __uint_as_float(p1 << 16), r1 = x1 - __uint_as_float(p1 & 0xffff0000u);
+    p2 = __builtin_bit_cast(unsigned, __builtin_convertvector(f2v{r0, r1}, bf16x2));
+    const float s0 = r0 - __uint_as_float(p2 << 16), s1 = r1 - __uint_as_float(p2 & 0xffff0000u);
+    p3 = __builtin_bit_cast(unsigned, __builtin_convertvector(f2v{s0, s1}, bf16x2));
+}
+
+template <int kTileCols, bool kCelu, bool kDeriv, bool kHead, bool kRank1>
+__global__ __launch_bounds__(kTileCols * 4) void dense_split_kernel(DenseArgs args, int row_tiles, float alpha, float inv_alpha)
+{
+    static_assert(!kHead || kTileCols == 64, "the output layer's sum runs over one wavefront's 64 columns");
+    constexpr int kThreads = kTileCols * 4;                          // 512 or 256: one wavefront per 32 rows x 64 columns
+    constexpr int kAPieces = kTileRows * (kChunk / 4) / kThreads;    // 16-byte pieces of the rows chunk per thread (2 or 4)
+    constexpr int kBPieces = kTileCols * (kChunk / 4) / kThreads;    // and of the weight chunk (2)
+    __shared__ SplitLds<kTileCols> S;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K = args.k, chunks = K / kChunk, col_tiles = args.col_tiles;
+    // row tiles of the four types, counted through: tile_end holds (row tiles x column tiles) sums
+    const int rt_end0 = args.tile_end[0] / col_tiles, rt_end1 = args.tile_end[1] / col_tiles, rt_end2 = args.tile_end[2] / col_tiles;
+
+    // A workgroup takes row tiles blk, blk + grid, ... and for each walks the column tiles and their chunks as one
+    // sequence of steps; the loads of a step are issued during the products of the step before, also across the end
+    // of a tile, so that only the very first chunk is waited for.
+    struct Cursor {
+        const float* rows;          // kRank1: the per-row factors
+        const float* head_w;
+        const float* deriv;
+        const float* wt;            // the type's weights (column tile 0)
+        int row0, n, t;
+        int rt, ctile, chunk;
+        bool live;
+    };
+    auto open_row_tile = [&](Cursor& c) {
+        c.live = c.rt < row_tiles;
+        if (!c.live) return;
+        const int t = (c.rt >= rt_end0) + (c.rt >= rt_end1) + (c.rt >= rt_end2);
+        const int first = t == 0 ? 0 : t == 1 ? rt_end0 : t == 2 ? rt_end1 : rt_end2;
+        c.t = t;
+        c.rows = kRank1 ? args.scale[t] : args.rows[t];
+        c.head_w = args.head_w[t];
+        c.deriv = args.deriv[t];
+        c.wt = args.wt[t];
+        c.row0 = (c.rt - first) * kTileRows;
+        c.n = args.n[t];
+        c.ctile = 0;
+        c.chunk = 0;
+    };
+    auto advance = [&](Cursor& c) {
+        if (++c.chunk < chunks) return;
+        c.chunk = 0;
+        if (++c.ctile < col_tiles) return;
+        c.rt += static_cast<int>(gridDim.x);
+        open_row_tile(c);
+    };
+
+    v4 ra[kAPieces], rb[kBPieces];
+    auto fetch = [&](const Cursor& c) {
+#pragma unroll
+        for (int u = 0; u < kAPieces; ++u) {
+            const int p = tid + kThreads * u;
+            const int r = p >> 3, k4 = (p & 7) << 2;
+            const int gr = min(c.row0 + r, c.n - 1);            // past the end: the last row again, never stored
+            const size_t at = static_cast<size_t>(gr) * K + c.chunk * kChunk + k4;
+            if constexpr (kRank1) ra[u] = rank1_piece(c.rows, c.head_w, gr, c.chunk * kChunk + k4);
+            else ra[u] = *reinterpret_cast<const v4*>(c.rows + at);
+            if constexpr (kDeriv) {
+                const v4 h = *reinterpret_cast<const v4*>(c.deriv + at);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ra[u][e] *= h[e] >= 0.f ? 1.0f : fmaf(h[e], inv_alpha, 1.0f);
+            }
+        }
+        const float* wt = c.wt + static_cast<size_t>(c.ctile) * kTileCols * K;
+#pragma unroll
+        for (int u = 0; u < kBPieces; ++u) {
+            const int p = tid + kThreads * u;
+            const int r = p >> 3, k4 = (p & 7) << 2;
+            rb[u] = *reinterpret_cast<const v4*>(wt + static_cast<size_t>(r) * K + c.chunk * kChunk + k4);
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int u = 0; u < kAPieces; ++u) {
+            const int p = tid + kThreads * u;
+            const int r = p >> 3, k4 = (p & 7) << 2;
+            unsigned lo[3], hi[3];
+            split_pair(ra[u][0], ra[u][1], lo[0], lo[1], lo[2]);
+            split_pair(ra[u][2], ra[u][3], hi[0], hi[1], hi[2]);
+#pragma unroll
+            for (int q = 0; q < 3; ++q) *reinterpret_cast<u2v*>(&S.a[q][r][k4]) = u2v{lo[q], hi[q]};
+        }
+#pragma unroll
+        for (int u = 0; u < kBPieces; ++u) {
+            const int p = tid + kThreads * u;
+            const int r = p >> 3, k4 = (p & 7) << 2;
+            unsigned lo[3], hi[3];
+            split_pair(rb[u][0], rb[u][1], lo[0], lo[1], lo[2]);
+            split_pair(rb[u][2], rb[u][3], hi[0], hi[1], hi[2]);
+#pragma unroll
+            for (int q = 0; q < 3; ++q) *reinterpret_cast<u2v*>(&S.b[q][r][k4]) = u2v{lo[q], hi[q]};
+        }
+    };
+
+    // this wavefront's part: rows wr*32.., columns wc*64.. (two 32 x 32 blocks across)
+    const int wr = kTileCols == 128 ? (wave >> 1) : wave, wc = kTileCols == 128 ? (wave & 1) : 0;
+    const int l32 = lane & 31, half = lane >> 5;
+    v16 acc[1][2];
+    auto clear = [&]() {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[0][j][e] = 0.f;
+    };
+    clear();
+
+    Cursor load;                 // the step whose loads are in registers
+    load.rt = static_cast<int>(blockIdx.x);
+    open_row_tile(load);
+    if (!load.live) return;
+    fetch(load);
+    for (;;) {
+        // the tile that the staged chunk belongs to (for its epilogue)
+        const int t = load.t, row0 = load.row0, n = load.n, ctile = load.ctile;
+        const bool last_chunk = load.chunk == chunks - 1;
+        stage();                                     // the chunk fetched during the previous products
+        __syncthreads();
+        advance(load);
+        if (load.live) fetch(load);                  // in flight while this chunk is multiplied
+#pragma unroll
+        for (int q = 0; q < kChunk / 16; ++q) {
+            // eight consecutive k of this lane's row / column: k = 16 q + 8 half + (0..7)
+            bf16x8 av[3], bv[2][3];
+#pragma unroll
+            for (int m = 0; m < 3; ++m) {
+                av[m] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u4v*>(&S.a[m][wr * 32 + l32][q * 16 + half * 8]));
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    bv[j][m] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u4v*>(&S.b[m][wc * 64 + j * 32 + l32][q * 16 + half * 8]));
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                // smallest partial products first
+                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[2], bv[j][0], acc[0][j], 0, 0, 0);
+                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][2], acc[0][j], 0, 0, 0);
+                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[j][1], acc[0][j], 0, 0, 0);
+                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[j][0], acc[0][j], 0, 0, 0);
+                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][1], acc[0][j], 0, 0, 0);
+                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][0], acc[0][j], 0, 0, 0);
+            }
+        }
+        __syncthreads();                             // everyone has read the chunk before it is overwritten
+        if (last_chunk) {
+            const int col0 = ctile * kTileCols;
+            const float* __restrict__ bias = args.bias[t];
+            float bj[2], hw[2] = {0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                bj[j] = bias ? bias[col0 + wc * 64 + j * 32 + l32] : 0.f;
+                if constexpr (kHead) hw[j] = args.head_w[t][col0 + j * 32 + l32];
+            }
+            tile_epilogue<kCelu, kHead, 1>(acc, bj, hw, args.head_b[t], args.out[t], args.head_out[t], n, args.n_out,
+                                           row0 + wr * 32, col0 + wc * 64, l32, half, alpha, inv_alpha);
+            clear();
+            if (!load.live) break;
+        }
+    }
+}
+
 // compute units of the current device (looked up once per device)
 int compute_units()
 {
@@ -448,10 +648,40 @@ int compute_units()
 
 enum class Extra { kNone, kHead, kRank1 };
 
+// KHAN_DENSE_MATRIX (read once): "bf16x3" selects the products on the bfloat16 matrix instructions with three-way split
+// operands, "f32" the float32 matrix instructions
+bool split_products()
+{
+    static const bool on = [] {
+        const char* v = std::getenv("KHAN_DENSE_MATRIX");
+        return v != nullptr && std::strcmp(v, "bf16x3") == 0;
+    }();
+    return on;
+}
+
 template <int kTileCols, int kK>
 hipError_t launch_tiles_k(const DenseArgs& a, int run, bool celu, bool deriv, Extra extra, float alpha, hipStream_t stream)
 {
     const float inv_alpha = 1.0f / alpha;
+    if (split_products()) {
+        constexpr int kThreads = kTileCols * 4;
+        // as many workgroups as stay resident (61 / 46 KB of LDS: two / three per CU), each walking row tiles
+        const int row_tiles = run / a.col_tiles;
+        const int resident = compute_units() * (kTileCols == 128 ? 2 : 3);
+        const dim3 grid(static_cast<unsigned>(row_tiles < resident ? row_tiles : resident)), block(kThreads);
+        if (extra == Extra::kRank1) dense_split_kernel<kTileCols, false, true, false, true><<<grid, block, 0, stream>>>(a, row_tiles, alpha, inv_alpha);
+        else if (extra == Extra::kHead) {
+            if constexpr (kTileCols == 64) {
+                if (celu) dense_split_kernel<64, true, false, true, false><<<grid, block, 0, stream>>>(a, row_tiles, alpha, inv_alpha);
+                else dense_split_kernel<64, false, false, true, false><<<grid, block, 0, stream>>>(a, row_tiles, alpha, inv_alpha);
+            } else return hipErrorInvalidValue;
+        }
+        else if (celu && !deriv) dense_split_kernel<kTileCols, true, false, false, false><<<grid, block, 0, stream>>>(a, row_tiles, alpha, inv_alpha);
+        else if (!celu && !deriv) dense_split_kernel<kTileCols, false, false, false, false><<<grid, block, 0, stream>>>(a, row_tiles, alpha, inv_alpha);
+        else if (!celu && deriv) dense_split_kernel<kTileCols, false, true, false, false><<<grid, block, 0, stream>>>(a, row_tiles, alpha, inv_alpha);
+        else dense_split_kernel<kTileCols, true, true, false, false><<<grid, block, 0, stream>>>(a, row_tiles, alpha, inv_alpha);
+        return hipGetLastError();
+    }
     // the widths of the reference's default network 384-128-128-64-1, forward and backward
     if constexpr ((kTileCols == 128 && kK > 0) || (kTileCols == 64 && kK == 128)) {
         // the pipelined kernel: as many workgroups as stay resident (two per CU at 72 KB of LDS, three at 54 KB)
