@@ -180,7 +180,12 @@ def inference_bench(args, batch):
         "molecules_per_s": n_mols / (ms_per_step * 1e-3),
         "first_layer": {"kernel_ms_per_step": ms_per_step, "library_ms_per_step": ms_library,
                         "max_relative_energy_difference": agree},
-        "roofline": {"kernel": "dense layers (CELU layers forward and backward: khan_dense_f32; last layer: rocBLAS)", "bound": "mfma", "achieved": gemm_flops / (ms_per_step * 1e-3) / 1e12,
+        "dense_products": "float32 operands split exactly into three bfloat16 parts, six partial products per pair on "
+                          "v_mfma_f32_32x32x16_bf16, float32 accumulation (KHAN_DENSE_MATRIX=f32 selects "
+                          "v_mfma_f32_32x32x2_f32)" if os.environ.get("KHAN_DENSE_MATRIX") != "f32" else "v_mfma_f32_32x32x2_f32",
+        "roofline": {"kernel": "dense layers, forward and data gradient (khan_dense_f32, khan_dense_head_f32, "
+                               "khan_dense_head_grad_f32): float32-equivalent flops of the whole step against the float32 matrix peak",
+                     "bound": "mfma", "achieved": gemm_flops / (ms_per_step * 1e-3) / 1e12,
                      "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": gemm_flops / (ms_per_step * 1e-3) / 1e12 / FP32_PEAK_TFLOPS, "traffic": None},
     }))

@@ -4,8 +4,11 @@
 // type -- with the CELU of khan/model/activations.py:63-65 as activation, or none).  The first form is a layer's
 // forward pass (the first layer right behind the featurizer: in = the 384-wide feature rows); the second is the data
 // gradient of a layer on the way back (in = the gradient with respect to the layer's activations, W = the layer's
-// weights read the other way round, no bias, no activation).  float32 in, float32 accumulation
-// (v_mfma_f32_32x32x2_f32): the same arithmetic as a float32 matrix product, in another summation order.
+// weights read the other way round, no bias, no activation).  float32 in, float32 accumulation: the arithmetic of a
+// float32 matrix product, in another summation order.  Two forms of the products: on the float32 matrix instructions
+// (v_mfma_f32_32x32x2_f32; dense_kernel and dense_pipe_kernel, described first), and -- the default -- on the bfloat16
+// matrix instructions with every float32 operand split exactly into three bfloat16 parts (dense_split_kernel, further
+// down), which gives the same result to float32 accuracy in less than half the matrix time.
 //
 // One workgroup of four wavefronts owns a tile of 128 rows x kTileCols columns of the output of one type.  With 128
 // columns every wavefront has a 64 x 64 quarter of it = 2 x 2 matrix-core blocks of 32 x 32; with 64 columns (the third
@@ -648,13 +651,13 @@ int compute_units()
 
 enum class Extra { kNone, kHead, kRank1 };
 
-// KHAN_DENSE_MATRIX (read once): "bf16x3" selects the products on the bfloat16 matrix instructions with three-way split
-// operands, "f32" the float32 matrix instructions
+// The products run on the bfloat16 matrix instructions with three-way split operands (dense_split_kernel) unless
+// KHAN_DENSE_MATRIX=f32 (read once) asks for the float32 matrix instructions.
 bool split_products()
 {
     static const bool on = [] {
         const char* v = std::getenv("KHAN_DENSE_MATRIX");
-        return v != nullptr && std::strcmp(v, "bf16x3") == 0;
+        return !(v != nullptr && std::strcmp(v, "f32") == 0);
     }();
     return on;
 }
