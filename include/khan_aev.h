@@ -232,7 +232,12 @@ int khan_ani_charge_grad_xyz_f64(const double *xs, const double *ys, const doubl
  * Every *_host4 argument is a HOST array of four DEVICE pointers: rows_t [acs[t], 384] (the featurizer's buckets,
  * 16-byte aligned), wt_t [128, 384] = the layer's [384, 128] weights TRANSPOSED (16-byte aligned), bias_t [128],
  * out_t [acs[t], 128].  float32 in, float32 accumulation on the matrix cores.  The layer width is fixed at 128
- * (the reference's default network, energy_server.py:121); other widths are the caller's matrix library's. */
+ * (the reference's default network, energy_server.py:121); khan_dense_f32 takes other widths.
+ * All khan_dense_* entry points compute the float32 product to float32 accuracy.  By default the partial products
+ * are formed on the bfloat16 matrix instructions, every float32 operand split exactly into three bfloat16 parts and
+ * the six largest of the nine partial products accumulated in float32 (what is dropped is below 2^-23 of a product);
+ * KHAN_DENSE_MATRIX=f32 in the environment (read once per process) selects the float32 matrix instructions.  With the
+ * split products a non-finite input gives NaN where a float32 product would give +-inf. */
 #define KHAN_ACT_NONE 0
 #define KHAN_ACT_CELU 1
 int khan_dense_first_f32(const float *const *rows_host4, const int32_t *acs_host,
