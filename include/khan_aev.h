@@ -282,6 +282,22 @@ int khan_dense_head_grad_f32(const float *const *scale_host4, const float *const
                              float alpha, const float *const *deriv_of_host4, float *const *out_host4,
                              khan_stream_t stream);
 
+/* Per-molecule sums of the atomic networks' outputs: e[m] = sum over the atoms g of molecule m of
+ * out_{as[g]}[sis[g]] -- the gather to the batch's atom order and the segment sum by molecule of the reference
+ * (khan/model/nn.py:165-177; trainer_multi_tower.py:350) in one launch, without the gathered copy, each molecule's
+ * sum formed in a fixed order (the same bits on every run).  out_host4: a HOST array of four DEVICE pointers, the
+ * per-type vectors [acs[t]] (an empty type's pointer may be NULL); as, sis [n_atoms]; mos, macs, e [n_mols]. */
+int khan_mol_energy_f32(const float *const *out_host4, const int32_t *as, const int32_t *sis, const int32_t *mos,
+                        const int32_t *macs, int32_t n_mols, float *e, khan_stream_t stream);
+int khan_mol_energy_f64(const double *const *out_host4, const int32_t *as, const int32_t *sis, const int32_t *mos,
+                        const int32_t *macs, int32_t n_mols, double *e, khan_stream_t stream);
+/* The way back: grad_t[sis[g]] = e_grads[m] for every atom g of molecule m (every element of the four vectors that
+ * belongs to an atom of a molecule is written). */
+int khan_mol_energy_grad_f32(const float *e_grads, const int32_t *as, const int32_t *sis, const int32_t *mos,
+                             const int32_t *macs, int32_t n_mols, float *const *grad_host4, khan_stream_t stream);
+int khan_mol_energy_grad_f64(const double *e_grads, const int32_t *as, const int32_t *sis, const int32_t *mos,
+                             const int32_t *macs, int32_t n_mols, double *const *grad_host4, khan_stream_t stream);
+
 /* Plain Coulomb sums, E_m = k sum_{i<j in m} q_i q_j / r_ij, and their gradients: the charge kernels with
  * the damping (1 - f_C) switched off and the constant chosen by the caller (k = 1 for charges in e and
  * distances in the unit the energy is wanted in).  No reference counterpart: khan's own op is the damped,

@@ -183,6 +183,29 @@ def dense_head(inputs, weights, biases, head_weights, head_biases, activation=op
     return _DenseHead.apply(int(activation), float(alpha), weights_t, *inputs, *weights, *biases, *head_weights, *head_biases)
 
 
+class _MolEnergy(torch.autograd.Function):
+    """Per-molecule sums of the four per-type output vectors (`ops.mol_energy`); the way back hands every atom's
+    entry its molecule's gradient (`ops.mol_energy_grad`)."""
+
+    @staticmethod
+    def forward(ctx, atom_types, sis, mos, macs, *outs):
+        ctx.save_for_backward(atom_types, sis, mos, macs)
+        ctx.counts = [int(o.numel()) for o in outs]
+        ctx.shapes = [o.shape for o in outs]
+        return ops.mol_energy([o.detach() for o in outs], atom_types, sis, mos, macs)
+
+    @staticmethod
+    def backward(ctx, ge):
+        atom_types, sis, mos, macs = ctx.saved_tensors
+        gs = ops.mol_energy_grad(ge.contiguous(), atom_types, sis, mos, macs, ctx.counts)
+        return (None, None, None, None) + tuple(g.reshape(sh) for g, sh in zip(gs, ctx.shapes))
+
+
+def mol_energy(type_outputs, atom_types, sis, mos, macs):
+    """Differentiable per-molecule sums of the four per-type network outputs: -> [n_mols]."""
+    return _MolEnergy.apply(atom_types, sis, mos, macs, *type_outputs)
+
+
 def dense_first(atom_type_features, acs_host, weights, biases, activation=ops.ACT_CELU, alpha=0.1, weights_t=None):
     """The first dense layer on the featurizer's four flat buckets: `dense` with k = 384."""
     for f, c in zip(atom_type_features, acs_host):

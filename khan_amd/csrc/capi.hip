@@ -321,6 +321,32 @@ int charge_grad_impl(const T* xs, const T* ys, const T* zs, const T* qs, const i
 
 }  // namespace
 
+// Per-molecule sums of the per-type network outputs, and the way back (khan_mol_energy_*).
+template <typename T>
+static int mol_energy_impl(const T* const* out_host4, const int32_t* as, const int32_t* sis, const int32_t* mos,
+                           const int32_t* macs, int32_t n_mols, T* e, khan_stream_t stream)
+{
+    if (n_mols < 0) return KHAN_ERR_INVALID_ARG;
+    if (n_mols == 0) return KHAN_OK;
+    if (!out_host4 || !as || !sis || !mos || !macs || !e) return KHAN_ERR_INVALID_ARG;
+    khan::Buckets<const T> in;
+    for (int t = 0; t < 4; ++t) in.p[t] = out_host4[t];
+    return hip_status(khan::launch_mol_sum<T>(in, as, sis, mos, macs, n_mols, e, as_stream(stream)));
+}
+
+template <typename T>
+static int mol_energy_grad_impl(const T* e_grads, const int32_t* as, const int32_t* sis, const int32_t* mos,
+                                const int32_t* macs, int32_t n_mols, T* const* grad_host4, khan_stream_t stream)
+{
+    if (n_mols < 0) return KHAN_ERR_INVALID_ARG;
+    if (n_mols == 0) return KHAN_OK;
+    if (!grad_host4 || !as || !sis || !mos || !macs || !e_grads) return KHAN_ERR_INVALID_ARG;
+    khan::Buckets<T> out;
+    for (int t = 0; t < 4; ++t) out.p[t] = grad_host4[t];
+    return hip_status(khan::launch_mol_sum_grad<T>(e_grads, as, sis, mos, macs, n_mols, out, as_stream(stream)));
+}
+
+
 extern "C" {
 
 int32_t khan_feature_size(void) { return khan::kFeats; }
@@ -602,6 +628,28 @@ int khan_dense_head_grad_f32(const float* const* scale_host4, const float* const
     if (total > INT32_MAX) return KHAN_ERR_TOO_LARGE;
     return hip_status(khan::launch_dense_head_grad(scale_host4, head_w_host4, n_host4, k, n_out, wt_host4, alpha, deriv_of_host4,
                                                    out_host4, as_stream(stream)));
+}
+
+// Per-molecule sums of the per-type network outputs, and the way back.
+int khan_mol_energy_f32(const float* const* out_host4, const int32_t* as, const int32_t* sis, const int32_t* mos,
+                        const int32_t* macs, int32_t n_mols, float* e, khan_stream_t stream)
+{
+    return mol_energy_impl<float>(out_host4, as, sis, mos, macs, n_mols, e, stream);
+}
+int khan_mol_energy_f64(const double* const* out_host4, const int32_t* as, const int32_t* sis, const int32_t* mos,
+                        const int32_t* macs, int32_t n_mols, double* e, khan_stream_t stream)
+{
+    return mol_energy_impl<double>(out_host4, as, sis, mos, macs, n_mols, e, stream);
+}
+int khan_mol_energy_grad_f32(const float* e_grads, const int32_t* as, const int32_t* sis, const int32_t* mos,
+                             const int32_t* macs, int32_t n_mols, float* const* grad_host4, khan_stream_t stream)
+{
+    return mol_energy_grad_impl<float>(e_grads, as, sis, mos, macs, n_mols, grad_host4, stream);
+}
+int khan_mol_energy_grad_f64(const double* e_grads, const int32_t* as, const int32_t* sis, const int32_t* mos,
+                             const int32_t* macs, int32_t n_mols, double* const* grad_host4, khan_stream_t stream)
+{
+    return mol_energy_grad_impl<double>(e_grads, as, sis, mos, macs, n_mols, grad_host4, stream);
 }
 
 // Plain Coulomb sums: the charge kernels with the cutoff function switched off and the constant given by the caller.

@@ -95,6 +95,14 @@ hipError_t launch_size_order(const int32_t* MACs, int32_t n_mols, int32_t* order
 template <typename T>
 hipError_t launch_zero(T* a, int64_t n, hipStream_t stream);
 
+// per-molecule sums of the four per-type output vectors (atom g's value is bucket[as[g]][sis[g]]), and the way back
+template <typename T>
+hipError_t launch_mol_sum(Buckets<const T> in, const int32_t* A, const int32_t* SIs, const int32_t* MOs, const int32_t* MACs,
+                          int32_t n_mols, T* e, hipStream_t stream);
+template <typename T>
+hipError_t launch_mol_sum_grad(const T* e_grad, const int32_t* A, const int32_t* SIs, const int32_t* MOs, const int32_t* MACs,
+                               int32_t n_mols, Buckets<T> out, hipStream_t stream);
+
 // ---- first dense layer behind the featurizer: out_t = act(rows_t . W_t + b_t) for the four types, float32 ----
 // rows[t]: [n[t], 384]; wt[t]: [128, 384] (the weights transposed); bias[t]: [128]; out[t]: [n[t], 128]
 hipError_t launch_dense(const float* const rows[4], const int32_t n[4], int32_t k, int32_t n_out,

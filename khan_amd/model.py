@@ -136,6 +136,12 @@ class MoleculeNN:
 
     def atom_outputs(self, atom_type_features, gather_idxs):
         """Per-type flat feature buckets -> one number per atom in the batch's atom order (nn.py:176-177)."""
+        # gather_idxs is a permutation: index_select's backward is a scatter-add, where indexing with [] sorts the
+        # indices first (a merge sort of n atoms in every backward pass)
+        return torch.index_select(torch.cat(self.type_outputs(atom_type_features)), 0, gather_idxs.long())
+
+    def type_outputs(self, atom_type_features):
+        """Per-type flat feature buckets -> the four per-type output vectors [acs[t]] (nn.py:165-175)."""
         nk = self.kernel_layers()
         if nk > 0:
             from . import autograd
@@ -159,9 +165,7 @@ class MoleculeNN:
                 outs = [self.atom_type_outputs(t, a[t], layers_done=nk) for t in range(4)]
         else:
             outs = [self.atom_type_outputs(t, f.reshape(-1, FEATURE_SIZE)) for t, f in enumerate(atom_type_features)]
-        # gather_idxs is a permutation: index_select's backward is a scatter-add, where indexing with [] sorts the
-        # indices first (a merge sort of n atoms in every backward pass)
-        return torch.index_select(torch.cat(outs), 0, gather_idxs.long())
+        return list(outs)
 
 
 class AniModel:
@@ -218,9 +222,9 @@ class AniModel:
         acs, order, classes = b.host_counts()
         feats = autograd.featurize(xs, ys, zs, b.atom_types, b.mol_offsets, b.mol_atom_counts, b.scatter_idxs, acs,
                                    order=order, size_classes=classes)
-        atom_e = self.near.atom_outputs(feats, b.gather_idxs)
-        energies = torch.zeros(b.n_mols, dtype=self.dtype, device=self.device)
-        energies.index_add_(0, b.mol_idxs.long(), atom_e)                 # segment_sum over molecules
+        # the networks' outputs summed by molecule straight from the four per-type vectors (nn.py:165-177 in one launch)
+        energies = autograd.mol_energy(self.near.type_outputs(feats), b.atom_types, b.scatter_idxs, b.mol_offsets,
+                                       b.mol_atom_counts)
         if self.charge is not None:
             qs = self.charge.atom_outputs(feats, b.gather_idxs)
             energies = energies + autograd.ani_charge(xs, ys, zs, qs.contiguous(), b.mol_offsets, b.mol_atom_counts)

@@ -261,6 +261,43 @@ def ani_charge_grad_xyz(xs, ys, zs, qs, mos, macs, grads):
     return qg, gx, gy, gz
 
 
+def mol_energy(type_outputs, atom_types, sis, mos, macs):
+    """Per-molecule sums of the four per-type output vectors (`type_outputs[t]` is [acs[t]], float32 or float64; atom
+    g's value is type_outputs[as[g]][sis[g]]) -> [n_mols]: the reference's gather to atom order + segment_sum by
+    molecule (khan/model/nn.py:165-177) in one launch, summed in a fixed order."""
+    lib = _lib.load()
+    dt = type_outputs[0].dtype
+    if dt not in _SUFFIX:
+        raise TypeError("type_outputs must be float32 or float64, got %s" % dt)
+    outs = [_dev(o.reshape(-1), dt, "type_outputs[%d]" % t) for t, o in enumerate(type_outputs)]
+    if len(outs) != 4:
+        raise ValueError("type_outputs must hold the four per-type vectors")
+    a, s_, mo, ma = (_dev(v, torch.int32, n) for v, n in ((atom_types, "atom_types"), (sis, "sis"), (mos, "mos"), (macs, "macs")))
+    if sum(o.numel() for o in outs) != a.numel() or s_.numel() != a.numel() or mo.numel() != ma.numel():
+        raise ValueError("the four vectors must hold one value per atom, and mos / macs one entry per molecule")
+    e = torch.empty(ma.numel(), dtype=dt, device=a.device)
+    fn = getattr(lib, "khan_mol_energy_" + _SUFFIX[dt])
+    _lib.check(fn(_ptr4(outs), _p(a), _p(s_), _p(mo), _p(ma), ma.numel(), _p(e), _stream()))
+    return e
+
+
+def mol_energy_grad(e_grads, atom_types, sis, mos, macs, acs):
+    """The way back through `mol_energy`: -> four vectors [acs[t]] with grad_t[sis[g]] = e_grads[molecule of g]."""
+    lib = _lib.load()
+    dt = e_grads.dtype
+    if dt not in _SUFFIX:
+        raise TypeError("e_grads must be float32 or float64, got %s" % dt)
+    eg = _dev(e_grads, dt, "e_grads")
+    a, s_, mo, ma = (_dev(v, torch.int32, n) for v, n in ((atom_types, "atom_types"), (sis, "sis"), (mos, "mos"), (macs, "macs")))
+    counts = _acs_host(acs)[1]
+    if sum(counts) != a.numel() or s_.numel() != a.numel() or mo.numel() != ma.numel() or eg.numel() != ma.numel():
+        raise ValueError("acs must add up to the number of atoms, and e_grads / mos / macs hold one entry per molecule")
+    outs = [torch.zeros(c, dtype=dt, device=a.device) for c in counts]       # atoms outside every molecule keep 0
+    fn = getattr(lib, "khan_mol_energy_grad_" + _SUFFIX[dt])
+    _lib.check(fn(_p(eg), _p(a), _p(s_), _p(mo), _p(ma), ma.numel(), _ptr4(outs), _stream()))
+    return tuple(outs)
+
+
 def coulomb(xs, ys, zs, qs, mos, macs, k=1.0):
     """-> energies[n_mols] = k * sum_{i<j} q_i q_j / r_ij: the charge kernel without the reference's damping
     and constant (the reference's op is `ani_charge`)."""

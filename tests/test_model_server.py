@@ -397,6 +397,53 @@ def test_output_layer_folded_into_the_last_hidden_layer(k):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "float64"])
+def test_molecule_sums_of_the_type_outputs_and_the_way_back(dtype):
+    """khan_mol_energy / khan_mol_energy_grad (the gather to atom order + segment sum by molecule of nn.py:165-177 in one
+    launch) against numpy: organic molecules with an empty molecule in the middle and a type outside 0..3 (counted as O,
+    as the sort does); the sums are the same bits on every call, and the autograd wiring returns the way back."""
+    from khan_amd import ops, autograd, datagen
+    dev = "cuda:0"
+    tdt = getattr(torch, dtype)
+    b = datagen.make_batch("organic", 300)
+    A = b.A.copy()
+    A[7] = 9                                         # out of range: the O bucket
+    mol_idxs = b.mol_idxs.copy()
+    mol_idxs[mol_idxs >= 150] += 1                   # molecule 150 is empty
+    n_mols = b.n_mols + 1
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    macs, mos = ops.mol_offsets(d(mol_idxs), n_mols)
+    sc, ga, ac = ops.ani_sort(d(A))
+    acs = [int(v) for v in ac.cpu().tolist()]
+    rng = np.random.default_rng(5)
+    outs = [rng.standard_normal(c) for c in acs]
+    t_of = np.minimum(np.where(A < 0, 3, A), 3)
+    sis = sc.cpu().numpy()
+    per_atom = np.array([outs[t_of[g]][sis[g]] for g in range(len(A))])
+    want = np.zeros(n_mols)
+    np.add.at(want, mol_idxs, per_atom)
+    touts = [d(o).to(tdt) for o in outs]
+    e = ops.mol_energy(touts, d(A), sc, mos, macs)
+    tol = 1e-5 if dtype == "float32" else 1e-13
+    mag = np.zeros(n_mols)
+    np.add.at(mag, mol_idxs, np.abs(per_atom))
+    assert e.shape == (n_mols,) and np.all(np.abs(e.cpu().numpy() - want) <= tol * mag + 1e-30)
+    assert float(e[150]) == 0.0
+    assert torch.equal(e, ops.mol_energy(touts, d(A), sc, mos, macs))             # fixed summation order
+    ge = rng.standard_normal(n_mols)
+    gs = ops.mol_energy_grad(d(ge).to(tdt), d(A), sc, mos, macs, acs)
+    for t in range(4):
+        wg = np.zeros(acs[t])
+        sel = t_of == t
+        wg[sis[sel]] = ge[mol_idxs[sel]]
+        assert np.array_equal(gs[t].cpu().numpy(), wg.astype(getattr(np, dtype)))
+    leaves = [o.clone().requires_grad_(True) for o in touts]
+    (autograd.mol_energy(leaves, d(A), sc, mos, macs) * d(ge).to(tdt)).sum().backward()
+    for t in range(4):
+        assert torch.equal(leaves[t].grad, gs[t])
+
+
+@pytest.mark.gpu
 def test_kernel_layers_agree_with_library_layers_in_energy_and_gradient():
     """The float32 model with its CELU layers in khan_dense_f32 against the same model with every layer a library
     product: energies and coordinate gradients of 200 molecules."""
