@@ -230,7 +230,7 @@ class AniModel:
             energies = energies + autograd.ani_charge(xs, ys, zs, qs.contiguous(), b.mol_offsets, b.mol_atom_counts)
         if not need_grad:
             return energies.detach(), None
-        gx, gy, gz = torch.autograd.grad(energies.sum(), (xs, ys, zs))
+        gx, gy, gz = torch.autograd.grad(energies, (xs, ys, zs), grad_outputs=torch.ones_like(energies))
         return energies.detach(), torch.stack((gx, gy, gz), dim=1)
 
     def _feeder(self, dataset, batch_size):

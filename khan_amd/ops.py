@@ -292,7 +292,8 @@ def mol_energy_grad(e_grads, atom_types, sis, mos, macs, acs):
     counts = _acs_host(acs)[1]
     if sum(counts) != a.numel() or s_.numel() != a.numel() or mo.numel() != ma.numel() or eg.numel() != ma.numel():
         raise ValueError("acs must add up to the number of atoms, and e_grads / mos / macs hold one entry per molecule")
-    outs = [torch.zeros(c, dtype=dt, device=a.device) for c in counts]       # atoms outside every molecule keep 0
+    # one cleared array cut into the four vectors (atoms outside every molecule keep 0)
+    outs = list(torch.zeros(sum(counts), dtype=dt, device=a.device).split(counts))
     fn = getattr(lib, "khan_mol_energy_grad_" + _SUFFIX[dt])
     _lib.check(fn(_p(eg), _p(a), _p(s_), _p(mo), _p(ma), ma.numel(), _ptr4(outs), _stream()))
     return tuple(outs)
