@@ -488,9 +488,14 @@ __global__ __launch_bounds__(kTileCols * 4) void dense_split_kernel(DenseArgs ar
     // row tiles of the four types, counted through: tile_end holds (row tiles x column tiles) sums
     const int rt_end0 = args.tile_end[0] / col_tiles, rt_end1 = args.tile_end[1] / col_tiles, rt_end2 = args.tile_end[2] / col_tiles;
 
-    // A workgroup takes row tiles blk, blk + grid, ... and for each walks the column tiles and their chunks as one
-    // sequence of steps; the loads of a step are issued during the products of the step before, also across the end
-    // of a tile, so that only the very first chunk is waited for.
+    // A workgroup keeps one column tile and walks row tiles, their chunks as one sequence of steps; the loads of a step
+    // are issued during the products of the step before, also across the end of a tile, so that only the very first
+    // chunk is waited for.  Which tiles: workgroups are dealt to the eight XCDs in turn (workgroup w runs on XCD
+    // w % 8), and each XCD has an L2 of its own.  The column tiles of one row tile share its rows, so they go to
+    // workgroups of the same XCD that start together and do the same amount of work: w = 8 q + x takes column tile
+    // q % col_tiles of the row tiles x + 8 (q / col_tiles) + k * stride.  The rows then come from HBM once and from
+    // L2 for the other column tiles (the first layer's data gradient has three: its fetches were three times its
+    // inputs when one workgroup took the column tiles of a row tile one after the other).
     struct Cursor {
         const float* rows;          // kRank1: the per-row factors
         const float* head_w;
@@ -512,14 +517,13 @@ __global__ __launch_bounds__(kTileCols * 4) void dense_split_kernel(DenseArgs ar
         c.wt = args.wt[t];
         c.row0 = (c.rt - first) * kTileRows;
         c.n = args.n[t];
-        c.ctile = 0;
         c.chunk = 0;
     };
+    const int wg_x = static_cast<int>(blockIdx.x) & 7, wg_q = static_cast<int>(blockIdx.x) >> 3;
+    const int rt_stride = (static_cast<int>(gridDim.x) >> 3) / col_tiles * 8;       // the grid is a multiple of 8 col_tiles
     auto advance = [&](Cursor& c) {
         if (++c.chunk < chunks) return;
-        c.chunk = 0;
-        if (++c.ctile < col_tiles) return;
-        c.rt += static_cast<int>(gridDim.x);
+        c.rt += rt_stride;
         open_row_tile(c);
     };
 
@@ -583,7 +587,8 @@ __global__ __launch_bounds__(kTileCols * 4) void dense_split_kernel(DenseArgs ar
     clear();
 
     Cursor load;                 // the step whose loads are in registers
-    load.rt = static_cast<int>(blockIdx.x);
+    load.rt = wg_x + 8 * (wg_q / col_tiles);
+    load.ctile = wg_q % col_tiles;
     open_row_tile(load);
     if (!load.live) return;
     fetch(load);
@@ -669,9 +674,15 @@ hipError_t launch_tiles_k(const DenseArgs& a, int run, bool celu, bool deriv, Ex
     if (split_products()) {
         constexpr int kThreads = kTileCols * 4;
         // as many workgroups as stay resident (61 / 46 KB of LDS: two / three per CU), each walking row tiles
+        // (the grid is a multiple of 8 x column tiles: see the kernel)
         const int row_tiles = run / a.col_tiles;
         const int resident = compute_units() * (kTileCols == 128 ? 2 : 3);
-        const dim3 grid(static_cast<unsigned>(row_tiles < resident ? row_tiles : resident)), block(kThreads);
+        const int unit = 8 * a.col_tiles;
+        int groups = resident / unit;                     // row tiles in flight per XCD
+        const int needed = (row_tiles + 7) / 8;
+        if (groups > needed) groups = needed;
+        if (groups < 1) groups = 1;
+        const dim3 grid(static_cast<unsigned>(groups * unit)), block(kThreads);
         if (extra == Extra::kRank1) dense_split_kernel<kTileCols, false, true, false, true><<<grid, block, 0, stream>>>(a, row_tiles, alpha, inv_alpha);
         else if (extra == Extra::kHead) {
             if constexpr (kTileCols == 64) {
