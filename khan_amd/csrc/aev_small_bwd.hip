@@ -5,7 +5,7 @@
 // reads the 16 upstream values of the partner's type from the centre's row, sums g e (f_C' - 2 eta d f_C)
 // over the shells, and the pull goes to the partner (one group of lanes at a time, so targets are
 // distinct) and, summed over the group with DPP moves, to the centre.  Centres are then taken in order
-// of decreasing partner count, in batches of up to six (four in float64) whose partner lists together fill at most the 64
+// of decreasing partner count, in batches of up to four whose partner lists together fill at most the 64
 // lanes.  Per batch:
 //   stage    the 320 angular upstream values of each centre's row are fetched with full-line loads
 //            (issued before the scan, so their latency is covered) and laid out in LDS by type pair;
@@ -30,23 +30,22 @@ namespace khan {
 
 namespace {
 
-// centres per batch.  float: six (the pool of 64 entries is what ends most batches).  double: four -- the staged
-// upstream rows are twice the size, and with four the working set (20.4 KB) lets eight wavefronts share a CU instead
-// of six, which is worth more than the fuller pools of six-centre batches (organic molecules: 0.53 -> 0.44 ms).
-template <typename T> constexpr int kSmallBwdCentres = sizeof(T) == 8 ? 4 : kB;
+// centres per batch: four.  Six would fill the pools of 64 entries better (8 % fewer rounds), but the staged upstream
+// rows are most of the working set: with four it is 10.2 KB (float) or 20.4 KB (double) and sixteen (eight) wavefronts
+// share a CU instead of twelve (six), which is worth more (organic molecules: float 0.68 -> 0.63 ms, double 0.53 -> 0.44 ms).
+template <typename T> constexpr int kSmallBwdCentres = 4;
 
 template <typename T>
 struct __align__(16) BwdLds {
-    typename Fast<T>::vec4 atom[64];     // x, y, z, type (sorted order)
+    typename Fast<T>::vec4 atom[64];     // x, y, z of the atom at this sorted position; w = its type + 4 * (the sorted position of the atom whose index in the molecule is this slot's)
     BwdPool<T, kSmallBwdCentres<T>> pool;   // partner lists and staged upstream values of the batch
     T force[3][64];                      // dL/dx, dL/dy, dL/dz per sorted atom
     int nM[8];                           // angular partners per centre of the batch
-    unsigned char inv[64];               // original atom index -> sorted lane
 };
 
-// float: 3 wavefronts per SIMD (LDS 13.2 KB); double: 2 (LDS 20.4 KB, twice the registers)
+// float: 4 wavefronts per SIMD (LDS 10.2 KB, 127 registers); double: 2 (LDS 20.4 KB, twice the registers)
 template <typename T>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 3 : 1, sizeof(T) == 4 ? 3 : 2)))
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 4 : 1, sizeof(T) == 4 ? 4 : 2)))
 void aev_bwd_small_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
@@ -96,7 +95,6 @@ void aev_bwd_small_kernel(
             dest = sel4(type, tbase[0], tbase[1], tbase[2], tbase[3]) + popc64(mine & lt_mask);
         }
     }
-    S.inv[lane] = static_cast<unsigned char>(dest);
     x = lane_push(dest, x);
     y = lane_push(dest, y);
     z = lane_push(dest, z);
@@ -104,7 +102,7 @@ void aev_bwd_small_kernel(
     orig = lane_push(dest, orig);
     const int rp_lo = lane_push(dest, static_cast<int>(rowbits & 0xffffffffull));
     const int rp_hi = lane_push(dest, static_cast<int>(rowbits >> 32));
-    S.atom[lane] = Fast<T>::make4(x, y, z, static_cast<T>(type));
+    S.atom[lane] = Fast<T>::make4(x, y, z, static_cast<T>(type + 4 * dest));     // dest: where the atom with index `lane` went
     S.force[0][lane] = T(0);
     S.force[1][lane] = T(0);
     S.force[2][lane] = T(0);
@@ -128,6 +126,7 @@ void aev_bwd_small_kernel(
     auto type_of = [&](int sorted_lane) { return (sorted_lane >= tb1) + (sorted_lane >= tb2) + (sorted_lane >= tb3); };
     wave_lds_fence();
     const vec4 aj = S.atom[jl];      // the partner this lane tests in every scan step
+    const int aj_type = static_cast<int>(aj.w) & 3;
 
     // ------------------------------------------------------------ order of the centres
     // Angular partner count of every atom, then centres in order of decreasing count: a batch of
@@ -153,7 +152,7 @@ void aev_bwd_small_kernel(
             T cfx = T(0), cfy = T(0), cfz = T(0);       // this pair's pull on the centre
             const bool inR = !kSkipRadial && valid && (r < kR_Rc_f) && (r > T(0));
             if (inR) {
-                const T sc = bwd_radial_pair<T>(grow, static_cast<int>(aj.w), r, Fast<T>::rcp(r));   // dE/dr / r
+                const T sc = bwd_radial_pair<T>(grow, aj_type, r, Fast<T>::rcp(r));   // dE/dr / r
                 cfx = sc * dx;
                 cfy = sc * dy;
                 cfz = sc * dz;
@@ -319,7 +318,7 @@ void aev_bwd_small_kernel(
                     const int i_orig = lane_read(orig, i_b);
                     bwd_center_generic<T>(L, lane, X, Y, Z, A, off, n, i_orig, S.pool.gst, row_of(i_b),
                                               [&](int atom, T fx, T fy, T fz) {
-                                                  const int sl = S.inv[atom];
+                                                  const int sl = static_cast<int>(S.atom[atom].w) >> 2;
                                                   atomicAdd(&S.force[0][sl], fx);
                                                   atomicAdd(&S.force[1][sl], fy);
                                                   atomicAdd(&S.force[2][sl], fz);
