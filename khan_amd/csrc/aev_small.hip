@@ -45,7 +45,7 @@ constexpr int kRadSlots = 96;
 // double or kJvp: 2 (LDS 19 KB); both: 1.
 template <typename T, bool kJvp, bool kMatrixPhase2 = false>
 __global__ __launch_bounds__(64 * kWavesPerBlock)
-__attribute__((amdgpu_waves_per_eu((sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1), (sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1))))
+__attribute__((amdgpu_waves_per_eu((sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1), (sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1) + ((kJvp && sizeof(T) == 4) ? 1 : 0))))
 void aev_fwd_small_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
@@ -55,7 +55,9 @@ void aev_fwd_small_kernel(
 {
     typedef typename Fast<T>::vec4 vec4;
     typedef typename Fast<T>::vec2 vec2;
-    __shared__ FwdWaveLds<T, kJvp, kFB, kRadSlots> lds_all[kWavesPerBlock];
+    // centres per batch: six; four in the float Jacobian-vector kernel, whose working set then lets ten wavefronts share a CU instead of eight
+    constexpr int kNB = (kJvp && sizeof(T) == 4) ? 4 : kFB;
+    __shared__ FwdWaveLds<T, kJvp, kNB, kRadSlots> lds_all[kWavesPerBlock];
     const int lane = threadIdx.x & 63;
     const int wave = kWavesPerBlock == 1 ? 0 : uniform(threadIdx.x >> 6);    // a constant LDS base with one wavefront per workgroup
     const int slot = blockIdx.x * kWavesPerBlock + wave;
@@ -64,7 +66,7 @@ void aev_fwd_small_kernel(
     const int n = uniform(MACs[mol]);
     const int off = uniform(MOs[mol]);
     if (n <= 0 || n > max_atoms) return;          // larger molecules belong to other kernels (max_atoms <= 64)
-    FwdWaveLds<T, kJvp, kFB, kRadSlots>& S = lds_all[wave];
+    FwdWaveLds<T, kJvp, kNB, kRadSlots>& S = lds_all[wave];
     const LaneConsts<T> L = lane_consts<T>(lane);
     const unsigned long long lane_bit = 1ull << lane;
     const unsigned long long lt_mask = lane_bit - 1ull;
@@ -168,8 +170,8 @@ void aev_fwd_small_kernel(
     fwd_lds_init(S, lane);
     wave_lds_fence();
 
-    for (int c0 = 0; c0 < n; c0 += kFB) {
-        const int nb = min(kFB, n - c0);
+    for (int c0 = 0; c0 < n; c0 += kNB) {
+        const int nb = min(kNB, n - c0);
         unsigned overflow = 0;
 
         // ------------------------------------------------ scan steps: G centres x W partners
