@@ -42,6 +42,7 @@ WORKLOADS = {
     "inference65536": ("organic", 65536, 4, False),
     # not a line of the headline metric either: featurize_grad_inverse (the Jacobian applied to per-atom vectors)
     "grad_inverse65536": ("organic", 65536, 4, False),
+    "grad_inverse_boxes4096": ("boxes", 4096, 4, False),
     # nor these: the charge kernels alone (energy, then dE/dq and dE/dxyz), float64
     "charges_boxes4096_f64": ("boxes", 4096, 8, True),
     "charges_organic16384_f64": ("organic", 16384, 8, True),
@@ -224,7 +225,7 @@ def grad_inverse_bench(args, batch):
         "value": N / (ms_per_step * 1e-3), "unit": "atoms/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "grad_inverse65536: featurize_grad_inverse, %d molecules, %d atoms" % (n_mols, N)},
+        "config": {"workload": "%s: featurize_grad_inverse, %d molecules, %d atoms" % (args.workload, n_mols, N)},
         "roofline": {"kernel": "aev_fwd_small_kernel<float, true>", "bound": "hbm", "achieved": nbytes / (launch_ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (launch_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "traffic": None, "launch_ms": launch_ms, "algorithmic_bytes": nbytes},
