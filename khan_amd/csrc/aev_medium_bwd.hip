@@ -3,7 +3,7 @@
 //
 // The workgroup sorts the atoms by type into LDS once and zeroes the molecule's outputs.  Wavefronts
 // then draw centres from a shared counter.  A wavefront collects centres into a batch while their
-// angular partner lists fit the 64 entries of its pool (at most four in float, six in double), and for each centre it takes in:
+// angular partner lists fit the 64 entries of its pool (at most four), and for each centre it takes in:
 //   scan + radial   the centre is tested against the sorted atoms 64 at a time; pairs inside the radial
 //                   cutoff are queued, and whenever 64 are waiting a lane takes one pair and sums
 //                   g e (f_C' - 2 eta d f_C) over the shells (float: the nine nearest to r) for both directions of the pair (the centre's
@@ -25,10 +25,11 @@ namespace khan {
 namespace {
 
 constexpr int kChunks = kMediumMaxAtoms / 64;
-// centres per batch.  float: four, so that the pools of the four wavefronts leave room for four workgroups on a CU
-// (LDS 39.6 KB; 128 registers) -- the shorter batches fill fewer lanes, the fourth wavefront per SIMD hides more;
-// double: six, one workgroup per CU either way.
-template <typename T> constexpr int kMedBwdCentres = sizeof(T) == 4 ? 4 : kB;
+// centres per batch: four, so that the pools of the four wavefronts leave room for four workgroups on a CU in float
+// (LDS 39.6 KB; 128 registers) and two in double (76 KB; 256 registers) -- the shorter batches fill fewer lanes, the
+// additional wavefronts per SIMD hide more (dense boxes: float 4 % faster than six-centre batches at three workgroups,
+// double 23 % faster than at one).
+template <typename T> constexpr int kMedBwdCentres = 4;
 
 template <typename T>
 struct __align__(16) MedBwdShared {
@@ -41,7 +42,7 @@ struct __align__(16) MedBwdShared {
 };
 
 template <typename T>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 4 : 1, sizeof(T) == 4 ? 4 : 1)))
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 4 : 2, sizeof(T) == 4 ? 4 : 2)))
 void aev_bwd_medium_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
