@@ -459,10 +459,10 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f2v __attribute__((ext_vector_type(2)));
 
-template <int kTileCols>
+template <int kTileCols, int kCT>
 struct __align__(16) SplitLds {
     unsigned short a[3][kTileRows][kSplitStride];
-    unsigned short b[3][kTileCols][kSplitStride];
+    unsigned short b[kCT][3][kTileCols][kSplitStride];
 };
 
 // two floats -> their three bfloat16 parts, each pair packed into one register (first value in the low half)
@@ -475,18 +475,22 @@ __device__ __forceinline__ void split_pair(float x0, float x1, unsigned& p1, uns
     p3 = __builtin_bit_cast(unsigned, __builtin_convertvector(f2v{s0, s1}, bf16x2));
 }
 
-template <int kTileCols, bool kCelu, bool kDeriv, bool kHead, bool kRank1>
+// kCT: column tiles that one workgroup multiplies at once (1, or all 3 of a 384-wide output: the rows are then staged
+// and split once for the three, a step holds three times the products between its barriers, and one workgroup of eight
+// wavefronts fills a CU -- 120 KB of LDS, 96 accumulator registers per lane).
+template <int kTileCols, bool kCelu, bool kDeriv, bool kHead, bool kRank1, int kCT = 1>
 __global__ __launch_bounds__(kTileCols * 4) void dense_split_kernel(DenseArgs args, int row_tiles, float alpha, float inv_alpha)
 {
     static_assert(!kHead || kTileCols == 64, "the output layer's sum runs over one wavefront's 64 columns");
     constexpr int kThreads = kTileCols * 4;                          // 512 or 256: one wavefront per 32 rows x 64 columns
     constexpr int kAPieces = kTileRows * (kChunk / 4) / kThreads;    // 16-byte pieces of the rows chunk per thread (2 or 4)
     constexpr int kBPieces = kTileCols * (kChunk / 4) / kThreads;    // and of the weight chunk (2)
-    __shared__ SplitLds<kTileCols> S;
+    static_assert(kCT == 1 || (kTileCols == 128 && !kHead), "several column tiles at once: 128-column tiles, no output layer");
+    __shared__ SplitLds<kTileCols, kCT> S;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int K = args.k, chunks = K / kChunk, col_tiles = args.col_tiles;
+    const int K = args.k, chunks = K / kChunk, col_tiles = args.col_tiles / kCT;     // column tiles as the workgroups see them
     // row tiles of the four types, counted through: tile_end holds (row tiles x column tiles) sums
-    const int rt_end0 = args.tile_end[0] / col_tiles, rt_end1 = args.tile_end[1] / col_tiles, rt_end2 = args.tile_end[2] / col_tiles;
+    const int rt_end0 = args.tile_end[0] / args.col_tiles, rt_end1 = args.tile_end[1] / args.col_tiles, rt_end2 = args.tile_end[2] / args.col_tiles;
 
     // A workgroup keeps one column tile and walks row tiles, their chunks as one sequence of steps; the loads of a step
     // are issued during the products of the step before, also across the end of a tile, so that only the very first
@@ -527,7 +531,7 @@ __global__ __launch_bounds__(kTileCols * 4) void dense_split_kernel(DenseArgs ar
         open_row_tile(c);
     };
 
-    v4 ra[kAPieces], rb[kBPieces];
+    v4 ra[kAPieces], rb[kCT][kBPieces];
     auto fetch = [&](const Cursor& c) {
 #pragma unroll
         for (int u = 0; u < kAPieces; ++u) {
@@ -543,12 +547,15 @@ __global__ __launch_bounds__(kTileCols * 4) void dense_split_kernel(DenseArgs ar
                 for (int e = 0; e < 4; ++e) ra[u][e] *= h[e] >= 0.f ? 1.0f : fmaf(h[e], inv_alpha, 1.0f);
             }
         }
-        const float* wt = c.wt + static_cast<size_t>(c.ctile) * kTileCols * K;
 #pragma unroll
-        for (int u = 0; u < kBPieces; ++u) {
-            const int p = tid + kThreads * u;
-            const int r = p >> 3, k4 = (p & 7) << 2;
-            rb[u] = *reinterpret_cast<const v4*>(wt + static_cast<size_t>(r) * K + c.chunk * kChunk + k4);
+        for (int ct = 0; ct < kCT; ++ct) {
+            const float* wt = c.wt + static_cast<size_t>(c.ctile * kCT + ct) * kTileCols * K;
+#pragma unroll
+            for (int u = 0; u < kBPieces; ++u) {
+                const int p = tid + kThreads * u;
+                const int r = p >> 3, k4 = (p & 7) << 2;
+                rb[ct][u] = *reinterpret_cast<const v4*>(wt + static_cast<size_t>(r) * K + c.chunk * kChunk + k4);
+            }
         }
     };
     auto stage = [&]() {
@@ -563,26 +570,31 @@ __global__ __launch_bounds__(kTileCols * 4) void dense_split_kernel(DenseArgs ar
             for (int q = 0; q < 3; ++q) *reinterpret_cast<u2v*>(&S.a[q][r][k4]) = u2v{lo[q], hi[q]};
         }
 #pragma unroll
-        for (int u = 0; u < kBPieces; ++u) {
-            const int p = tid + kThreads * u;
-            const int r = p >> 3, k4 = (p & 7) << 2;
-            unsigned lo[3], hi[3];
-            split_pair(rb[u][0], rb[u][1], lo[0], lo[1], lo[2]);
-            split_pair(rb[u][2], rb[u][3], hi[0], hi[1], hi[2]);
+        for (int ct = 0; ct < kCT; ++ct) {
 #pragma unroll
-            for (int q = 0; q < 3; ++q) *reinterpret_cast<u2v*>(&S.b[q][r][k4]) = u2v{lo[q], hi[q]};
+            for (int u = 0; u < kBPieces; ++u) {
+                const int p = tid + kThreads * u;
+                const int r = p >> 3, k4 = (p & 7) << 2;
+                unsigned lo[3], hi[3];
+                split_pair(rb[ct][u][0], rb[ct][u][1], lo[0], lo[1], lo[2]);
+                split_pair(rb[ct][u][2], rb[ct][u][3], hi[0], hi[1], hi[2]);
+#pragma unroll
+                for (int q = 0; q < 3; ++q) *reinterpret_cast<u2v*>(&S.b[ct][q][r][k4]) = u2v{lo[q], hi[q]};
+            }
         }
     };
 
     // this wavefront's part: rows wr*32.., columns wc*64.. (two 32 x 32 blocks across)
     const int wr = kTileCols == 128 ? (wave >> 1) : wave, wc = kTileCols == 128 ? (wave & 1) : 0;
     const int l32 = lane & 31, half = lane >> 5;
-    v16 acc[1][2];
+    v16 acc[kCT][1][2];
     auto clear = [&]() {
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int ct = 0; ct < kCT; ++ct)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[0][j][e] = 0.f;
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[ct][0][j][e] = 0.f;
     };
     clear();
 
@@ -603,37 +615,45 @@ __global__ __launch_bounds__(kTileCols * 4) void dense_split_kernel(DenseArgs ar
 #pragma unroll
         for (int q = 0; q < kChunk / 16; ++q) {
             // eight consecutive k of this lane's row / column: k = 16 q + 8 half + (0..7)
-            bf16x8 av[3], bv[2][3];
+            bf16x8 av[3];
 #pragma unroll
-            for (int m = 0; m < 3; ++m) {
+            for (int m = 0; m < 3; ++m)
                 av[m] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u4v*>(&S.a[m][wr * 32 + l32][q * 16 + half * 8]));
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    bv[j][m] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u4v*>(&S.b[m][wc * 64 + j * 32 + l32][q * 16 + half * 8]));
-            }
+            for (int ct = 0; ct < kCT; ++ct) {
+                bf16x8 bv[2][3];
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                // smallest partial products first
-                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[2], bv[j][0], acc[0][j], 0, 0, 0);
-                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][2], acc[0][j], 0, 0, 0);
-                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[j][1], acc[0][j], 0, 0, 0);
-                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[j][0], acc[0][j], 0, 0, 0);
-                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][1], acc[0][j], 0, 0, 0);
-                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][0], acc[0][j], 0, 0, 0);
+                for (int m = 0; m < 3; ++m)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        bv[j][m] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u4v*>(&S.b[ct][m][wc * 64 + j * 32 + l32][q * 16 + half * 8]));
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    // smallest partial products first
+                    acc[ct][0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[2], bv[j][0], acc[ct][0][j], 0, 0, 0);
+                    acc[ct][0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][2], acc[ct][0][j], 0, 0, 0);
+                    acc[ct][0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[j][1], acc[ct][0][j], 0, 0, 0);
+                    acc[ct][0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[j][0], acc[ct][0][j], 0, 0, 0);
+                    acc[ct][0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][1], acc[ct][0][j], 0, 0, 0);
+                    acc[ct][0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][0], acc[ct][0][j], 0, 0, 0);
+                }
             }
         }
         __syncthreads();                             // everyone has read the chunk before it is overwritten
         if (last_chunk) {
-            const int col0 = ctile * kTileCols;
-            const float* __restrict__ bias = args.bias[t];
-            float bj[2], hw[2] = {0.f, 0.f};
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                bj[j] = bias ? bias[col0 + wc * 64 + j * 32 + l32] : 0.f;
-                if constexpr (kHead) hw[j] = args.head_w[t][col0 + j * 32 + l32];
+            for (int ct = 0; ct < kCT; ++ct) {
+                const int col0 = (ctile * kCT + ct) * kTileCols;
+                const float* __restrict__ bias = args.bias[t];
+                float bj[2], hw[2] = {0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    bj[j] = bias ? bias[col0 + wc * 64 + j * 32 + l32] : 0.f;
+                    if constexpr (kHead) hw[j] = args.head_w[t][col0 + j * 32 + l32];
+                }
+                tile_epilogue<kCelu, kHead, 1>(acc[ct], bj, hw, args.head_b[t], args.out[t], args.head_out[t], n, args.n_out,
+                                               row0 + wr * 32, col0 + wc * 64, l32, half, alpha, inv_alpha);
             }
-            tile_epilogue<kCelu, kHead, 1>(acc, bj, hw, args.head_b[t], args.out[t], args.head_out[t], n, args.n_out,
-                                           row0 + wr * 32, col0 + wc * 64, l32, half, alpha, inv_alpha);
             clear();
             if (!load.live) break;
         }
@@ -672,6 +692,22 @@ hipError_t launch_tiles_k(const DenseArgs& a, int run, bool celu, bool deriv, Ex
 {
     const float inv_alpha = 1.0f / alpha;
     if (split_products()) {
+        if constexpr (kTileCols == 128) {
+            if (a.col_tiles == 3 && extra == Extra::kNone) {
+                // the three column tiles of a 384-wide output at once: one workgroup per CU
+                const int row_tiles = run / a.col_tiles;
+                int groups = compute_units() / 8;
+                const int needed = (row_tiles + 7) / 8;
+                if (groups > needed) groups = needed;
+                if (groups < 1) groups = 1;
+                const dim3 grid(static_cast<unsigned>(groups * 8)), block(512);
+                if (celu && !deriv) dense_split_kernel<128, true, false, false, false, 3><<<grid, block, 0, stream>>>(a, row_tiles, alpha, inv_alpha);
+                else if (!celu && !deriv) dense_split_kernel<128, false, false, false, false, 3><<<grid, block, 0, stream>>>(a, row_tiles, alpha, inv_alpha);
+                else if (!celu && deriv) dense_split_kernel<128, false, true, false, false, 3><<<grid, block, 0, stream>>>(a, row_tiles, alpha, inv_alpha);
+                else dense_split_kernel<128, true, true, false, false, 3><<<grid, block, 0, stream>>>(a, row_tiles, alpha, inv_alpha);
+                return hipGetLastError();
+            }
+        }
         constexpr int kThreads = kTileCols * 4;
         // as many workgroups as stay resident (61 / 46 KB of LDS: two / three per CU), each walking row tiles
         // (the grid is a multiple of 8 x column tiles: see the kernel)
