@@ -59,6 +59,22 @@ def test_status_codes_without_touching_the_gpu():
     assert lib.khan_ani_sort(n, -1, n, n, n, n) == 1
     assert lib.khan_ani_charge_grad_f64(n, n, n, n, n, n, 3, n, n, n) == 1
     assert lib.khan_mol_offsets(n, 1 << 40, 1, n, n, n) == 3
+    # the entry points behind the networks: the sums by molecule and the dense layers
+    four = (ctypes.c_void_p * 4)(None, None, None, None)
+    n4 = (ctypes.c_int32 * 4)(0, 0, 0, 0)
+    one4 = (ctypes.c_int32 * 4)(1, 0, 0, 0)
+    assert lib.khan_mol_energy_f32(four, n, n, n, n, 0, n, n) == 0
+    assert lib.khan_mol_energy_f64(four, n, n, n, n, 2, n, n) == 1
+    assert lib.khan_mol_energy_f32(None, n, n, n, n, 2, n, n) == 1
+    assert lib.khan_mol_energy_grad_f32(n, n, n, n, n, -1, four, n) == 1
+    assert lib.khan_mol_energy_grad_f64(n, n, n, n, n, 0, four, n) == 0
+    assert lib.khan_dense_f32(four, n4, 128, 128, four, None, 1, 0.1, None, four, n) == 0          # no rows: nothing to do
+    assert lib.khan_dense_f32(four, one4, 128, 128, four, None, 1, 0.1, None, four, n) == 1        # rows without pointers
+    assert lib.khan_dense_f32(four, n4, 100, 128, four, None, 1, 0.1, None, four, n) == 1          # width not a multiple of 32
+    assert lib.khan_dense_f32(four, n4, 128, 128, four, None, 1, 0.0, None, four, n) == 1          # CELU needs alpha > 0
+    assert lib.khan_dense_head_f32(four, n4, 128, 128, four, None, 1, 0.1, four, None, four, four, n) == 1   # the output layer sits behind 64 columns
+    assert lib.khan_dense_head_f32(four, n4, 128, 64, four, None, 1, 0.1, four, None, four, four, n) == 0
+    assert lib.khan_dense_head_grad_f32(four, four, one4, 64, 128, four, 0.1, four, four, n) == 1
     assert b"invalid" in lib.khan_status_string(1)
 
 
