@@ -1,0 +1,82 @@
+"""KHAN_AEV_FORCE_GENERIC=1 (read once per process by libkhan_aev.so) routes every molecule through the general-shape
+kernels (workgroup per molecule, wavefront per centre), which otherwise only see molecules of more than 256 atoms and
+the centres whose lists overflow.  Features, gradients and the Jacobian-vector product of organic molecules and dense
+boxes from those kernels are checked against the float64 oracle at the tolerances of test_gpu_parity.py; the variable is
+read at the first launch, so the run is a child process."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from khan_amd import datagen
+from oracle import binding as ob
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+CHILD = r"""
+import sys
+import numpy as np, torch
+sys.path.insert(0, sys.argv[1])
+from khan_amd import datagen, ops
+kind, n_mols, out = sys.argv[2], int(sys.argv[3]), sys.argv[4]
+b = datagen.make_batch(kind, n_mols)
+d = "cuda:0"
+res = {}
+A = torch.from_numpy(b.A).to(d)
+macs, mos = ops.mol_offsets(torch.from_numpy(b.mol_idxs).to(d), b.n_mols)
+sc, ga, ac = ops.ani_sort(A)
+acs = ac.cpu()
+up = np.random.default_rng(11).standard_normal((b.n_atoms, 384))
+v = np.random.default_rng(12).standard_normal((3, b.n_atoms))
+counts = [int(c) for c in acs.tolist()]
+for name, dt in (("f32", np.float32), ("f64", np.float64)):
+    X, Y, Z = (torch.from_numpy(a.astype(dt)).to(d) for a in (b.X, b.Y, b.Z))
+    f = ops.featurize(X, Y, Z, A, mos, macs, sc, acs)
+    res["feat_" + name] = torch.cat(f).cpu().numpy()
+    # upstream rows in bucket order: row of atom g is bucket row gather_idxs[g]
+    bucket = torch.empty((b.n_atoms, 384), dtype=X.dtype, device=d)
+    bucket[ga.long()] = torch.from_numpy(up.astype(dt)).to(d)
+    gb = [t.reshape(-1) for t in bucket.split(counts)]
+    g = ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *gb)
+    res["grad_" + name] = torch.stack(g, 1).cpu().numpy()
+    j = ops.featurize_grad_inverse(X, Y, Z, A, mos, macs, sc, acs, *[torch.from_numpy(v[c].astype(dt)).to(d) for c in range(3)])
+    res["jvp_" + name] = torch.cat(j).cpu().numpy()
+torch.cuda.synchronize()
+np.savez(out, **res)
+"""
+
+
+@pytest.mark.parametrize("kind,n_mols", [("organic", 96), ("boxes", 2)])
+def test_general_shape_kernels_match_the_oracle(tmp_path, kind, n_mols):
+    b = datagen.make_batch(kind, n_mols)
+    MACs, MOs = ob.mol_offsets(b.mol_idxs, b.n_mols)
+    sc, ga, ac = ob.ani_sort(b.A)
+    up = np.random.default_rng(11).standard_normal((b.n_atoms, 384))
+    v = np.random.default_rng(12).standard_normal((3, b.n_atoms))
+    feat = np.concatenate(ob.featurize(b.X, b.Y, b.Z, b.A, MOs, MACs, sc, ac, dtype=np.float64))
+    upb = ob.scatter_rows(up, b.A, sc, ac)
+    grad = np.stack(ob.featurize_grad(b.X, b.Y, b.Z, b.A, MOs, MACs, sc, ac, upb, dtype=np.float64), 1)
+    jvp = np.concatenate(ob.featurize_grad_inverse(b.X, b.Y, b.Z, b.A, MOs, MACs, sc, ac, v[0], v[1], v[2], dtype=np.float64))
+    out = str(tmp_path / "generic.npz")
+    env = dict(os.environ)
+    env["KHAN_AEV_FORCE_GENERIC"] = "1"
+    print("child: KHAN_AEV_FORCE_GENERIC=1, %s %d molecules" % (kind, n_mols), flush=True)
+    subprocess.run([sys.executable, "-c", CHILD, ROOT, kind, str(n_mols), out], env=env, check=True, timeout=300)
+    got = np.load(out)
+    gscale = np.zeros_like(grad)
+    for m in range(b.n_mols):
+        s = slice(MOs[m], MOs[m] + MACs[m])
+        gscale[s] = np.abs(grad[s]).max()
+    jscale = np.abs(jvp).max()
+    for name, rtol, atol in (("f32", 1e-5, 1e-6), ("f64", 1e-12, 1e-15)):
+        f = got["feat_" + name].astype(np.float64).reshape(-1)
+        assert np.all(np.abs(f - feat.reshape(-1)) <= atol + rtol * np.abs(feat.reshape(-1))), ("features", name)
+        g = got["grad_" + name].astype(np.float64)
+        assert np.all(np.abs(g - grad) <= atol + rtol * np.maximum(np.abs(grad), gscale)), ("gradient", name)
+        j = got["jvp_" + name].astype(np.float64).reshape(-1)
+        assert np.all(np.abs(j - jvp.reshape(-1)) <= atol + rtol * np.maximum(np.abs(jvp.reshape(-1)), jscale)), ("jvp", name)
