@@ -43,6 +43,7 @@ WORKLOADS = {
     # not a line of the headline metric either: featurize_grad_inverse (the Jacobian applied to per-atom vectors)
     "grad_inverse65536": ("organic", 65536, 4, False),
     "grad_inverse_boxes4096": ("boxes", 4096, 4, False),
+    "grad_inverse_boxes4096_f64": ("boxes", 4096, 8, False),
     # nor these: the charge kernels alone (energy, then dE/dq and dE/dxyz), float64
     "charges_boxes4096_f64": ("boxes", 4096, 8, True),
     "charges_organic16384_f64": ("organic", 16384, 8, True),
@@ -192,21 +193,22 @@ def inference_bench(args, batch):
     }))
 
 
-def grad_inverse_bench(args, batch):
-    """featurize_grad_inverse on the organic batch: one JSON line; algorithmic bytes are the forward's plus the
+def grad_inverse_bench(args, batch, w, kind):
+    """featurize_grad_inverse on the batch: one JSON line; algorithmic bytes are the forward's plus the
     three incoming vectors."""
     import torch
     from khan_amd import ops
     dev = torch.device("cuda:0")
     N, n_mols = batch.n_atoms, batch.n_mols
-    X, Y, Z = (torch.from_numpy(v).to(dev) for v in (batch.X, batch.Y, batch.Z))
+    tdt, tname = (torch.float32, "float") if w == 4 else (torch.float64, "double")
+    X, Y, Z = (torch.from_numpy(v).to(dev).to(tdt) for v in (batch.X, batch.Y, batch.Z))
     A = torch.from_numpy(batch.A).to(dev)
     macs, mos = ops.mol_offsets(torch.from_numpy(batch.mol_idxs).to(dev), n_mols)
     sc, ga, ac = ops.ani_sort(A)
     acs = ac.cpu()
     gen = torch.Generator(device=dev)
     gen.manual_seed(7)
-    v = [torch.randn(N, device=dev, generator=gen) for _ in range(3)]
+    v = [torch.randn(N, device=dev, generator=gen, dtype=tdt) for _ in range(3)]
     for _ in range(args.warmup):
         ops.featurize_grad_inverse(X, Y, Z, A, mos, macs, sc, acs, *v)
     torch.cuda.synchronize()
@@ -219,14 +221,15 @@ def grad_inverse_bench(args, batch):
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
     launch_ms = e0.elapsed_time(e1) / args.steps
-    nbytes = N * (384 * 4 + 6 * 4 + 8) + 8 * n_mols
+    nbytes = N * (384 * w + 6 * w + 8) + 8 * n_mols
+    kernel = "aev_fwd_%s_kernel<%s, true>" % ("small" if kind == "organic" else "medium", tname)
     print(json.dumps({
-        "metric": "AEV grad-inverse (Jacobian-vector product) atoms/sec, fp32, 1 MI355X",
+        "metric": "AEV grad-inverse (Jacobian-vector product) atoms/sec, fp%d, 1 MI355X" % (8 * w),
         "value": N / (ms_per_step * 1e-3), "unit": "atoms/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f%d" % (8 * w),
         "data": "synthetic",
         "config": {"workload": "%s: featurize_grad_inverse, %d molecules, %d atoms" % (args.workload, n_mols, N)},
-        "roofline": {"kernel": "aev_fwd_small_kernel<float, true>", "bound": "hbm", "achieved": nbytes / (launch_ms * 1e-3) / 1e9,
+        "roofline": {"kernel": kernel, "bound": "hbm", "achieved": nbytes / (launch_ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (launch_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "traffic": None, "launch_ms": launch_ms, "algorithmic_bytes": nbytes},
     }))
@@ -316,7 +319,7 @@ def main():
     if args.workload.startswith("inference"):
         return inference_bench(args, batch)
     if args.workload.startswith("grad_inverse"):
-        return grad_inverse_bench(args, batch)
+        return grad_inverse_bench(args, batch, w, kind)
     if args.workload.startswith("charges_"):
         return charges_bench(args, batch, w)
     N = batch.n_atoms

@@ -53,8 +53,9 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
     __shared__ MedShared<T, kJvp> M;
     // Batches of four centres in float32: the forward kernel's working set then lets four workgroups share a CU
     // (LDS 39.9 KB each) instead of three, which measured 21 % faster on dense boxes, and the Jacobian-vector kernel's
-    // two (75 KB each) instead of one; the float64 forward kernel keeps batches of six.
-    constexpr int kNB = sizeof(T) == 4 ? 4 : kFB;
+    // two (75 KB each) instead of one; the float64 forward kernel keeps batches of six, and the float64 Jacobian-vector
+    // kernel takes batches of four (134 KB, one workgroup per CU; six measured the same at 157 KB of the CU's 160).
+    constexpr int kNB = (sizeof(T) == 4 || kJvp) ? 4 : kFB;
     __shared__ FwdWaveLds<T, kJvp, kNB> lds_wave[4];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -302,20 +303,25 @@ hipError_t launch_fwd_medium(const T* X, const T* Y, const T* Z, const int32_t* 
     return hipGetLastError();
 }
 
-hipError_t launch_jvp_medium_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
-                                 const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
-                                 const int32_t* SIs, const float* VX, const float* VY, const float* VZ,
-                                 Buckets<float> out, int min_atoms, const int32_t* order, hipStream_t stream)
+template <typename T>
+hipError_t launch_jvp_medium(const T* X, const T* Y, const T* Z, const int32_t* A,
+                             const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                             const int32_t* SIs, const T* VX, const T* VY, const T* VZ,
+                             Buckets<T> out, int min_atoms, const int32_t* order, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
-    // (one workgroup per CU with this working set: a smaller grid costs less when it only skips)
-    const unsigned blocks = static_cast<unsigned>(n_mols < 1024 ? n_mols : 1024);
-    aev_fwd_medium_kernel<float, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, VX, VY, VZ,
-                                                                            out, min_atoms, order);
+    // (two workgroups per CU in float32, one in float64: a smaller grid costs less when it only skips)
+    const int32_t cap = sizeof(T) == 4 ? 1024 : 512;
+    const unsigned blocks = static_cast<unsigned>(n_mols < cap ? n_mols : cap);
+    aev_fwd_medium_kernel<T, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, VX, VY, VZ,
+                                                                       out, min_atoms, order);
     return hipGetLastError();
 }
 
 template hipError_t launch_fwd_medium<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<float>, int, const int32_t*, hipStream_t);
 template hipError_t launch_fwd_medium<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<double>, int, const int32_t*, hipStream_t);
+
+template hipError_t launch_jvp_medium<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const float*, const float*, const float*, Buckets<float>, int, const int32_t*, hipStream_t);
+template hipError_t launch_jvp_medium<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const double*, const double*, const double*, Buckets<double>, int, const int32_t*, hipStream_t);
 
 }  // namespace khan

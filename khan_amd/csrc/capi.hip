@@ -275,7 +275,7 @@ int featurize_grad_inverse_impl(const T* xs, const T* ys, const T* zs, const int
     if (force_generic())
         return hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, 0,
                                                       nullptr, as_stream(stream)));
-    // molecules of up to 64 atoms: one wavefront each; 65..256 in float32: one workgroup each; the rest: general-shape kernel
+    // molecules of up to 64 atoms: one wavefront each; 65..256: one workgroup each; the rest: general-shape kernel
     SizeOrder made(own_order ? macs : nullptr, own_order ? n_mols : 0, as_stream(stream));
     const int32_t* order = own_order ? made.get() : caller_order;
     const SizeClasses cls(own_order ? nullptr : classes_host);
@@ -283,13 +283,10 @@ int featurize_grad_inverse_impl(const T* xs, const T* ys, const T* zs, const int
     if (cls.any(0, khan::kSmallMaxAtoms))
         st = hip_status(khan::launch_jvp_small<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, order,
                                                   as_stream(stream)));
-    int generic_from = khan::kSmallMaxAtoms + 1;
-    if constexpr (sizeof(T) == 4) {
-        if (st == KHAN_OK && cls.any(khan::kSmallMaxAtoms + 1, khan::kMediumMaxAtoms))
-            st = hip_status(khan::launch_jvp_medium_f32(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
-                                                        khan::kSmallMaxAtoms + 1, order, as_stream(stream)));
-        generic_from = khan::kMediumMaxAtoms + 1;
-    }
+    if (st == KHAN_OK && cls.any(khan::kSmallMaxAtoms + 1, khan::kMediumMaxAtoms))
+        st = hip_status(khan::launch_jvp_medium<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
+                                                   khan::kSmallMaxAtoms + 1, order, as_stream(stream)));
+    const int generic_from = khan::kMediumMaxAtoms + 1;
     if (st == KHAN_OK && cls.any(generic_from, INT32_MAX))
         st = hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
                                                     generic_from, order, as_stream(stream)));

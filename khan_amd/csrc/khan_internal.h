@@ -46,11 +46,12 @@ template <typename T>
 hipError_t launch_fwd_medium(const T* X, const T* Y, const T* Z, const int32_t* A,
                              const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
                              const int32_t* SIs, Buckets<T> out, int min_atoms, const int32_t* order, hipStream_t stream);
-// the same kernel as Jacobian-vector product (float32 only: in float64 its working set exceeds the LDS)
-hipError_t launch_jvp_medium_f32(const float* X, const float* Y, const float* Z, const int32_t* A,
-                                 const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
-                                 const int32_t* SIs, const float* VX, const float* VY, const float* VZ,
-                                 Buckets<float> out, int min_atoms, const int32_t* order, hipStream_t stream);
+// the same kernel as Jacobian-vector product
+template <typename T>
+hipError_t launch_jvp_medium(const T* X, const T* Y, const T* Z, const int32_t* A,
+                             const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                             const int32_t* SIs, const T* VX, const T* VY, const T* VZ,
+                             Buckets<T> out, int min_atoms, const int32_t* order, hipStream_t stream);
 
 template <typename T>
 hipError_t launch_bwd_medium(const T* X, const T* Y, const T* Z, const int32_t* A,

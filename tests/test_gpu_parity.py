@@ -830,11 +830,13 @@ def test_grad_inverse_organic_and_boxes(ops):
     _check_grad_inverse(ops, Case(x, y, z, a, mi, 2))
 
 
-def test_grad_inverse_adjoint_identity_and_uniform_vector(ops):
+@pytest.mark.parametrize("kind,n_mols,first", [("organic", 512, 2000), ("boxes", 3, 40)])
+def test_grad_inverse_adjoint_identity_and_uniform_vector(ops, kind, n_mols, first):
     # on the device, in float64: <u, J v> = <J^T u, v> with J^T u from featurize_grad, and J applied to a
-    # uniform vector (the reference's only test input, test_kernel.py:363-400) is zero
-    say("case: featurize_grad_inverse adjoint identity, 512 molecules")
-    c = Case.from_batch(datagen.make_batch("organic", 512, first_mol=2000))
+    # uniform vector (the reference's only test input, test_kernel.py:363-400) is zero; the boxes go through the
+    # workgroup-per-molecule kernels on both sides
+    say("case: featurize_grad_inverse adjoint identity, %d %s molecules" % (n_mols, kind))
+    c = Case.from_batch(datagen.make_batch(kind, n_mols, first_mol=first))
     macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
     acs = ac.cpu()
     X, Y, Z, A = dev(c.X, np.float64), dev(c.Y, np.float64), dev(c.Z, np.float64), dev(c.A)
