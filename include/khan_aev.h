@@ -75,7 +75,11 @@ int khan_ani_sort(const int32_t *atomic_numbers, int64_t n_atoms, int32_t *scatt
  * in : xs, ys, zs [n_atoms]; as [n_atoms]; mos, macs [n_mols]; sis = scatter_idxs [n_atoms];
  *      acs_host[4] = atom_counts in HOST memory (the reference declares it HostMemory, ani_op.cpp:333)
  * out: h_feat[acs[0]*384], c_feat[acs[1]*384], n_feat[acs[2]*384], o_feat[acs[3]*384], row-major;
- *      the row of atom g is bucket[as[g]] + sis[g]*384. */
+ *      the row of atom g is bucket[as[g]] + sis[g]*384.
+ * Scratch, from the stream-ordered allocator on every call: the molecule indices in order of decreasing size, and,
+ * for molecules of more than 256 atoms, a sorted copy of the atoms (24 bytes per atom of the batch in float32, 40 in
+ * float64).  While the stream is being captured into a graph neither is taken: molecules then run in the order given,
+ * and those of more than 256 atoms in slower kernels that need no scratch. */
 int khan_featurize_f32(const float *xs, const float *ys, const float *zs, const int32_t *as,
                        const int32_t *mos, const int32_t *macs, int32_t n_mols, const int32_t *sis,
                        float *h_feat, float *c_feat, float *n_feat, float *o_feat,
@@ -93,7 +97,8 @@ int khan_featurize_f64(const double *xs, const double *ys, const double *zs, con
  * hipMalloc, hipFree or other allocating routine.  More than KHAN_FEATURIZE_NOALLOC_MAX_MOLS molecules:
  * KHAN_ERR_TOO_LARGE, nothing launched.  Every call on a GPU uses that GPU's one array: calls that overlap
  * on one GPU (two streams, two threads) race; calls on one stream are ordered and safe.  The first call on
- * a device looks the array's address up (hipGetSymbolAddress); make that call outside graph capture. */
+ * a device looks the array's address up (hipGetSymbolAddress); make that call outside graph capture.
+ * Molecules of more than 256 atoms run in the kernels that need no scratch (slower than khan_featurize_f32's). */
 #define KHAN_FEATURIZE_NOALLOC_MAX_MOLS (1 << 20)
 int khan_featurize_f32_noalloc(const float *xs, const float *ys, const float *zs, const int32_t *as,
                                const int32_t *mos, const int32_t *macs, int32_t n_mols,

@@ -15,6 +15,7 @@
 // Rows are written once, without atomics.  A centre with more than 32 angular or 64 radial partners is
 // redone by the general per-centre routine.  Semantics: gpu_featurizer/kernel_cpu.cpp:406-537.
 #include "aev_fwd_batch.h"
+#include "aev_large.h"
 
 namespace khan {
 
@@ -28,7 +29,7 @@ template <typename T> struct __align__(16) MedVel<T, true> {
     typename Fast<T>::vec4 vel[kMediumMaxAtoms];   // the incoming vector of every atom (sorted order)
 };
 
-template <typename T, bool kJvp>
+template <typename T, bool kJvp, bool kLarge = false>
 struct __align__(16) MedShared {
     typename Fast<T>::vec4 atom[kMediumMaxAtoms];   // x, y, z, type (sorted order)
     unsigned row_lo[kMediumMaxAtoms];      // address of the atom's output row
@@ -37,20 +38,28 @@ struct __align__(16) MedShared {
     int wcount[4][4];                      // atoms of each type held by each wavefront before the sort
     MedVel<T, kJvp> v;
 };
+// above 256 atoms the sorted atoms are in device memory (aev_large.h); what stays here are the output rows of the
+// centres of each wavefront's batch
+template <typename T, bool kJvp>
+struct __align__(16) MedShared<T, kJvp, true> {
+    unsigned long long row[4][8];
+};
 
 // With kJvp the kernel computes the Jacobian-vector product instead (featurize_grad_inverse), as the
 // one-wavefront kernel does: list entries also carry (v_i - v_j)/r, the cutoff's derivative and the change of r.
-template <typename T, bool kJvp>
+// With kLarge the kernel takes the molecules of more than 256 atoms: the atoms come type-sorted from `sorted`, and
+// the workgroups of one grid column (blockIdx.y = 0 .. gridDim.y - 1) share a molecule's centres batch by batch.
+template <typename T, bool kJvp, bool kLarge = false>
 __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
     const T* __restrict__ VX, const T* __restrict__ VY, const T* __restrict__ VZ,
-    Buckets<T> out, int min_atoms, const int32_t* __restrict__ order)
+    Buckets<T> out, int min_atoms, const int32_t* __restrict__ order, const SortedAtoms<T> sorted)
 {
     typedef typename Fast<T>::vec4 vec4;
     typedef typename Fast<T>::vec2 vec2;
-    __shared__ MedShared<T, kJvp> M;
+    __shared__ MedShared<T, kJvp, kLarge> M;
     // Batches of four centres in float32: the forward kernel's working set then lets four workgroups share a CU
     // (LDS 39.9 KB each) instead of three, which measured 21 % faster on dense boxes, and the Jacobian-vector kernel's
     // two (75 KB each) instead of one; the float64 forward kernel keeps batches of six, and the float64 Jacobian-vector
@@ -67,11 +76,12 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
 
     fwd_lds_init(S, lane);
     __shared__ unsigned long long want[4];
-    for_each_molecule_in_range(MACs, n_mols, min_atoms, kMediumMaxAtoms, want, order, order ? order + n_mols : nullptr, [&](int mol) {
+    for_each_molecule_in_range(MACs, n_mols, min_atoms, kLarge ? INT32_MAX : kMediumMaxAtoms, want, order, order ? order + n_mols : nullptr, [&](int mol) {
         const int n = uniform(MACs[mol]);
         const int off = uniform(MOs[mol]);
 
         // ------------------------------------------------------------ load, sort by type into LDS
+        if constexpr (!kLarge) {
         const bool have = tid < n;
         T x = T(0), y = T(0), z = T(0);
         T vx = T(0), vy = T(0), vz = T(0);
@@ -116,26 +126,61 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
             if constexpr (kJvp) M.v.vel[dest] = Fast<T>::make4(vx, vy, vz, T(0));
         }
         __syncthreads();
+        }
+        const int last_atom = (kLarge ? n : kMediumMaxAtoms) - 1;
+        auto atom_at = [&](int sorted_idx) -> vec4 {
+            if constexpr (kLarge) return sorted.atom[off + sorted_idx];
+            else return M.atom[sorted_idx];
+        };
+        auto vel_at = [&](int sorted_idx) -> vec4 {
+            if constexpr (!kJvp) return Fast<T>::make4(T(0), T(0), T(0), T(0));
+            else if constexpr (kLarge) return sorted.vel[off + sorted_idx];
+            else return M.v.vel[sorted_idx];
+        };
+        auto orig_of = [&](int sorted_idx) -> int {          // wave-uniform index
+            if constexpr (kLarge) return uniform(sorted.aux[off + sorted_idx].x);
+            else return uniform(static_cast<int>(M.orig[sorted_idx]));
+        };
+        int c0 = 0;                                          // first centre of the wavefront's batch
+        auto row_bits_of = [&](int sorted_idx) -> unsigned long long {     // per-lane index inside the batch's range
+            if constexpr (kLarge) {
+                return M.row[wave][min(max(sorted_idx - c0, 0), 7)];
+            } else {
+                const int idx = min(sorted_idx, kMediumMaxAtoms - 1);
+                return (static_cast<unsigned long long>(M.row_hi[idx]) << 32) | M.row_lo[idx];
+            }
+        };
         auto row_of = [&](int sorted_idx) -> T* {            // wave-uniform index
-            const unsigned lo = static_cast<unsigned>(uniform(static_cast<int>(M.row_lo[sorted_idx])));
-            const unsigned hi = static_cast<unsigned>(uniform(static_cast<int>(M.row_hi[sorted_idx])));
+            const unsigned long long bits = row_bits_of(sorted_idx);
+            const unsigned lo = static_cast<unsigned>(uniform(static_cast<int>(bits & 0xffffffffull)));
+            const unsigned hi = static_cast<unsigned>(uniform(static_cast<int>(bits >> 32)));
             return reinterpret_cast<T*>((static_cast<unsigned long long>(hi) << 32) | lo);
         };
 
         // ------------------------------------------------------------ batches of kNB centres per wavefront
-        for (int c0 = wave * kNB; c0 < n; c0 += 4 * kNB) {
+        const int first_c0 = (kLarge ? static_cast<int>(blockIdx.y) * 4 + wave : wave) * kNB;
+        const int stride_c0 = (kLarge ? static_cast<int>(gridDim.y) : 1) * 4 * kNB;
+        for (c0 = first_c0; c0 < n; c0 += stride_c0) {
             const int nb = min(kNB, n - c0);
             unsigned overflow = 0;
+            if constexpr (kLarge) {
+                if (lane < nb) {
+                    const int type = static_cast<int>(sorted.atom[off + c0 + lane].w);
+                    T* const bucket = type == 0 ? out.p[0] : type == 1 ? out.p[1] : type == 2 ? out.p[2] : out.p[3];
+                    M.row[wave][lane] = reinterpret_cast<unsigned long long>(bucket + static_cast<size_t>(sorted.aux[off + c0 + lane].y) * kFeats);
+                }
+                wave_lds_fence();
+            }
 
             for (int b = 0; b < nb; ++b) {
                 const int i = c0 + b;
-                const vec4 ai = M.atom[i];
+                const vec4 ai = atom_at(i);
                 int posR = 0, posA = 0;                 // list lengths so far (wave-uniform)
                 int cR[4] = {0, 0, 0, 0}, cA[4] = {0, 0, 0, 0};
                 for (int jc = 0; jc < n; jc += 64) {
                     const int j = jc + lane;
-                    const int jj = min(j, kMediumMaxAtoms - 1);
-                    const vec4 aj = M.atom[jj];
+                    const int jj = min(j, last_atom);
+                    const vec4 aj = atom_at(jj);
                     const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
                     const T r = Fast<T>::sqrt_rn(dx * dx + dy * dy + dz * dz);
                     const bool valid = (j < n) && (j != i);
@@ -152,7 +197,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                             cA[a] += popc64(mA & ta);
                         }
                         const T inv = Fast<T>::rcp(r);
-                        const vec4 vi = M.v.vel[i], vjv = M.v.vel[jj];
+                        const vec4 vi = vel_at(i), vjv = vel_at(jj);
                         const T wx = vi.x - vjv.x, wy = vi.y - vjv.y, wz = vi.z - vjv.z;     // v_centre - v_partner
                         const T rd = (dx * wx + dy * wy + dz * wz) * inv;                    // d r along it
                         if (inR) {
@@ -260,17 +305,14 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
             }
 
             // ------------------------------------------------ segment table, phases 1 and 2, zero fill
-            fwd_angular_batch<false>(S, L, lane, nb, [&](int b) -> unsigned long long {
-                const int idx = min(c0 + b, kMediumMaxAtoms - 1);
-                return (static_cast<unsigned long long>(M.row_hi[idx]) << 32) | M.row_lo[idx];
-            });
+            fwd_angular_batch<false>(S, L, lane, nb, [&](int b) -> unsigned long long { return row_bits_of(c0 + b); });
 
             // ------------------------------------------------ centres whose lists overflowed
             if (overflow) {
                 __threadfence();
                 for (int b = 0; b < nb; ++b) {
                     if (overflow & (1u << b)) {
-                        const int i_orig = uniform(static_cast<int>(M.orig[c0 + b]));
+                        const int i_orig = orig_of(c0 + b);
                         if constexpr (kJvp)
                             jvp_center_generic<T>(L, lane, X, Y, Z, A, VX, VY, VZ, off, n, i_orig,
                                                   reinterpret_cast<T*>(S.rec), row_of(c0 + b));
@@ -299,7 +341,7 @@ hipError_t launch_fwd_medium(const T* X, const T* Y, const T* Z, const int32_t* 
     const int32_t cap = sizeof(T) == 4 ? 4096 : 1024;
     const unsigned blocks = static_cast<unsigned>(n_mols < cap ? n_mols : cap);
     aev_fwd_medium_kernel<T, false><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, nullptr, nullptr,
-                                                                        nullptr, out, min_atoms, order);
+                                                                        nullptr, out, min_atoms, order, SortedAtoms<T>{});
     return hipGetLastError();
 }
 
@@ -314,7 +356,37 @@ hipError_t launch_jvp_medium(const T* X, const T* Y, const T* Z, const int32_t* 
     const int32_t cap = sizeof(T) == 4 ? 1024 : 512;
     const unsigned blocks = static_cast<unsigned>(n_mols < cap ? n_mols : cap);
     aev_fwd_medium_kernel<T, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, VX, VY, VZ,
-                                                                       out, min_atoms, order);
+                                                                       out, min_atoms, order, SortedAtoms<T>{});
+    return hipGetLastError();
+}
+
+template <typename T>
+size_t large_scratch_bytes(int64_t n_atoms, int32_t n_mols, bool with_vectors)
+{
+    return sorted_atoms_bytes<T>(n_atoms, n_mols, with_vectors);
+}
+
+// Molecules of more than 256 atoms: the sort into `scratch` (large_scratch_bytes), then the kernel above with the
+// centres of a molecule spread over the workgroups of a grid column.
+template <typename T>
+hipError_t launch_fwd_large(const T* X, const T* Y, const T* Z, const int32_t* A,
+                            const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                            const int32_t* SIs, const T* VX, const T* VY, const T* VZ, Buckets<T> out,
+                            const int32_t* order, void* scratch, int64_t n_atoms, hipStream_t stream)
+{
+    if (n_mols <= 0) return hipSuccess;
+    const bool jvp = VX != nullptr;
+    const SortedAtoms<T> sorted = carve_sorted_atoms<T>(scratch, n_atoms, n_mols, jvp);
+    const hipError_t e = launch_large_sort<T>(X, Y, Z, A, MOs, MACs, n_mols, SIs, VX, VY, VZ, nullptr, nullptr, nullptr, order,
+                                              sorted, stream);
+    if (e != hipSuccess) return e;
+    const dim3 grid(static_cast<unsigned>(n_mols < kLargeColumns ? n_mols : kLargeColumns), kLargeParts);
+    if (jvp)
+        aev_fwd_medium_kernel<T, true, true><<<grid, dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, VX, VY, VZ, out,
+                                                                         kMediumMaxAtoms + 1, order, sorted);
+    else
+        aev_fwd_medium_kernel<T, false, true><<<grid, dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, nullptr, nullptr,
+                                                                          nullptr, out, kMediumMaxAtoms + 1, order, sorted);
     return hipGetLastError();
 }
 
@@ -323,5 +395,10 @@ template hipError_t launch_fwd_medium<double>(const double*, const double*, cons
 
 template hipError_t launch_jvp_medium<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const float*, const float*, const float*, Buckets<float>, int, const int32_t*, hipStream_t);
 template hipError_t launch_jvp_medium<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const double*, const double*, const double*, Buckets<double>, int, const int32_t*, hipStream_t);
+
+template size_t large_scratch_bytes<float>(int64_t, int32_t, bool);
+template size_t large_scratch_bytes<double>(int64_t, int32_t, bool);
+template hipError_t launch_fwd_large<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const float*, const float*, const float*, Buckets<float>, const int32_t*, void*, int64_t, hipStream_t);
+template hipError_t launch_fwd_large<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, const double*, const double*, const double*, Buckets<double>, const int32_t*, void*, int64_t, hipStream_t);
 
 }  // namespace khan

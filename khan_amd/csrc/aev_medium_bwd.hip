@@ -18,7 +18,10 @@
 // Forces go to the output arrays with global atomics (a molecule's atoms are shared by four wavefronts).
 // A centre with more than 64 angular partners is handled by the general per-centre routine.
 // Reference: gpu_featurizer/kernel_cpu.cpp:217-366.
+#include <type_traits>
+
 #include "aev_bwd_batch.h"
+#include "aev_large.h"
 
 namespace khan {
 
@@ -31,7 +34,7 @@ constexpr int kChunks = kMediumMaxAtoms / 64;
 // double 23 % faster than at one).
 template <typename T> constexpr int kMedBwdCentres = 4;
 
-template <typename T>
+template <typename T, bool kLarge = false>
 struct __align__(16) MedBwdShared {
     typename Fast<T>::vec4 atom[kMediumMaxAtoms];   // x, y, z, type (sorted order)
     unsigned row_lo[kMediumMaxAtoms];      // address of the atom's upstream row
@@ -40,18 +43,29 @@ struct __align__(16) MedBwdShared {
     int wcount[4][4];                      // atoms of each type held by each wavefront before the sort
     int next;                              // next centre (sorted position) to hand out
 };
-
+// above 256 atoms the sorted atoms are in device memory (aev_large.h); the list entries' sorted positions no
+// longer fit a byte and are kept here, one array per wavefront (the pool's byte array then holds the types)
 template <typename T>
+struct __align__(16) MedBwdShared<T, true> {
+    int pos[4][64];
+    int next;                              // centres handed out so far by this workgroup
+};
+
+// With kLarge the kernel takes the molecules of more than 256 atoms: the atoms come type-sorted from `sorted`, the
+// workgroups of one grid column (blockIdx.y = 0 .. gridDim.y - 1) share a molecule's centres, and the gradients were
+// zeroed by the kernel that sorted the atoms.
+template <typename T, bool kLarge = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 4 : 2, sizeof(T) == 4 ? 4 : 2)))
 void aev_bwd_medium_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
     const int32_t* __restrict__ MACs, int32_t n_mols, const int32_t* __restrict__ SIs,
     Buckets<const T> gin, T* __restrict__ gX, T* __restrict__ gY, T* __restrict__ gZ, int min_atoms,
-    const int32_t* __restrict__ order, bool walk_in_order)
+    const int32_t* __restrict__ order, bool walk_in_order, const SortedAtoms<T> sorted)
 {
     typedef typename Fast<T>::vec4 vec4;
-    __shared__ MedBwdShared<T> M;
+    typedef typename std::conditional<kLarge, int, unsigned short>::type idx_t;     // a sorted position in the radial queue
+    __shared__ MedBwdShared<T, kLarge> M;
     constexpr int kMB = kMedBwdCentres<T>;
     __shared__ BwdPool<T, kMB> pools[4];
     const int tid = threadIdx.x;
@@ -62,12 +76,21 @@ void aev_bwd_medium_kernel(
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
 
     __shared__ unsigned long long want[4];
-    for_each_molecule_in_range(MACs, n_mols, min_atoms, kMediumMaxAtoms, want, walk_in_order ? order : nullptr,
+    for_each_molecule_in_range(MACs, n_mols, min_atoms, kLarge ? INT32_MAX : kMediumMaxAtoms, want, walk_in_order ? order : nullptr,
                                order ? order + n_mols : nullptr, [&](int mol) {
         const int n = uniform(MACs[mol]);
         const int off = uniform(MOs[mol]);
+        int tb1, tb2, tb3;                     // sorted position of the first C, N, O atom
 
         // ------------------------------------------------------------ load, sort by type into LDS, zero outputs
+        if constexpr (kLarge) {
+            const int4 tb = sorted.tbase[mol];
+            tb1 = uniform(tb.y);
+            tb2 = uniform(tb.z);
+            tb3 = uniform(tb.w);
+            if (tid == 0) M.next = 0;
+            __syncthreads();
+        } else {
         const bool have = tid < n;
         T x = T(0), y = T(0), z = T(0);
         int type = 0;
@@ -108,15 +131,36 @@ void aev_bwd_medium_kernel(
             M.orig[dest] = static_cast<unsigned short>(tid);
         }
         __syncthreads();       // sorted arrays complete; the zeroed outputs are visible before any atomic add
-        const int tb1 = tbase[1], tb2 = tbase[2], tb3 = tbase[3];
+        tb1 = tbase[1];
+        tb2 = tbase[2];
+        tb3 = tbase[3];
+        }
         auto type_of = [&](int sorted_idx) { return (sorted_idx >= tb1) + (sorted_idx >= tb2) + (sorted_idx >= tb3); };
+        auto atom_at = [&](int sorted_idx) -> vec4 {
+            if constexpr (kLarge) return sorted.atom[off + sorted_idx];
+            else return M.atom[sorted_idx];
+        };
+        auto row_bits_of = [&](int sorted_idx) -> unsigned long long {     // per-lane index
+            if constexpr (kLarge) {
+                const int type = type_of(sorted_idx);
+                const T* const bucket = type == 0 ? gin.p[0] : type == 1 ? gin.p[1] : type == 2 ? gin.p[2] : gin.p[3];
+                return reinterpret_cast<unsigned long long>(bucket + static_cast<size_t>(sorted.aux[off + sorted_idx].y) * kFeats);
+            } else {
+                return (static_cast<unsigned long long>(M.row_hi[sorted_idx]) << 32) | M.row_lo[sorted_idx];
+            }
+        };
         auto row_of = [&](int sorted_idx) -> const T* {            // wave-uniform index
-            const unsigned lo = static_cast<unsigned>(uniform(static_cast<int>(M.row_lo[sorted_idx])));
-            const unsigned hi = static_cast<unsigned>(uniform(static_cast<int>(M.row_hi[sorted_idx])));
+            const unsigned long long bits = row_bits_of(sorted_idx);
+            const unsigned lo = static_cast<unsigned>(uniform(static_cast<int>(bits & 0xffffffffull)));
+            const unsigned hi = static_cast<unsigned>(uniform(static_cast<int>(bits >> 32)));
             return reinterpret_cast<const T*>((static_cast<unsigned long long>(hi) << 32) | lo);
         };
+        auto orig_of = [&](int sorted_idx) -> int {                // per-lane index
+            if constexpr (kLarge) return sorted.aux[off + sorted_idx].x;
+            else return M.orig[sorted_idx];
+        };
         auto add_force = [&](int sorted_idx, T fx, T fy, T fz) {   // per-lane target
-            const int g = off + M.orig[sorted_idx];
+            const int g = off + orig_of(sorted_idx);
             atomicAdd(&gX[g], fx);
             atomicAdd(&gY[g], fy);
             atomicAdd(&gZ[g], fz);
@@ -127,8 +171,8 @@ void aev_bwd_medium_kernel(
         // would leave most lanes idle.  The queue lives in the pool's staging area, which is free while a
         // batch is being collected; it is emptied before the batch's upstream rows are staged.
         vec4* const q_d = reinterpret_cast<vec4*>(P.gst);                          // 128 x (dx, dy, dz, r)
-        unsigned short* const q_j = reinterpret_cast<unsigned short*>(q_d + 128);  // partner (sorted position)
-        unsigned short* const q_c = q_j + 128;                                     // centre (sorted position)
+        idx_t* const q_j = reinterpret_cast<idx_t*>(q_d + 128);                    // partner (sorted position)
+        idx_t* const q_c = q_j + 128;                                              // centre (sorted position)
         int qn = 0;
         auto radial_work_off = [&](int count) {      // entries 0..count-1, count <= 64
             T fx = T(0), fy = T(0), fz = T(0);
@@ -137,8 +181,8 @@ void aev_bwd_medium_kernel(
                 const vec4 e = q_d[lane];
                 const int j = q_j[lane];
                 c = q_c[lane];
-                const T* grow_c = reinterpret_cast<const T*>((static_cast<unsigned long long>(M.row_hi[c]) << 32) | M.row_lo[c]);
-                const T* grow_j = reinterpret_cast<const T*>((static_cast<unsigned long long>(M.row_hi[j]) << 32) | M.row_lo[j]);
+                const T* grow_c = reinterpret_cast<const T*>(row_bits_of(c));
+                const T* grow_j = reinterpret_cast<const T*>(row_bits_of(j));
                 const T inv = Fast<T>::rcp(e.w);
                 // the pair's pull on the centre from both rows; the partner gets its share when it is the centre
                 const T sc = bwd_radial_pair_both<T>(grow_c, type_of(j), grow_j, type_of(c), e.w, inv);
@@ -172,7 +216,7 @@ void aev_bwd_medium_kernel(
                 radial_work_off(take);
                 const int rest = qn - take;
                 vec4 e = Fast<T>::make4(T(0), T(0), T(0), T(1));
-                unsigned short ej = 0, ec = 0;
+                idx_t ej = 0, ec = 0;
                 if (lane < rest) {
                     e = q_d[64 + lane];
                     ej = q_j[64 + lane];
@@ -188,8 +232,30 @@ void aev_bwd_medium_kernel(
                 qn = rest;
             }
         };
+        // a full wave of queued pairs: work it off, keep the rest
+        auto radial_work_off_full = [&]() {
+            wave_lds_fence();
+            radial_work_off(64);
+            const int rest = qn - 64;
+            vec4 e = Fast<T>::make4(T(0), T(0), T(0), T(1));
+            idx_t ej = 0, ec = 0;
+            if (lane < rest) {
+                e = q_d[64 + lane];
+                ej = q_j[64 + lane];
+                ec = q_c[64 + lane];
+            }
+            wave_lds_fence();
+            if (lane < rest) {
+                q_d[lane] = e;
+                q_j[lane] = ej;
+                q_c[lane] = ec;
+            }
+            wave_lds_fence();
+            qn = rest;
+        };
 
         int pending = -1;          // a centre that was drawn but did not fit the previous batch
+        int scanned = -1;          // (large molecules) the centre whose radial pairs were queued last
         for (;;) {
             // ------------------------------------------------ collect a batch of centres
             int nb = 0, used = 0;
@@ -202,13 +268,55 @@ void aev_bwd_medium_kernel(
                     int drawn = 0;
                     if (lane == 0) drawn = atomicAdd(&M.next, 1);
                     c = uniform(drawn);
+                    if constexpr (kLarge) c = static_cast<int>(blockIdx.y) + static_cast<int>(gridDim.y) * c;
                 }
                 if (c >= n) break;
-                const vec4 ai = M.atom[c];
+                const vec4 ai = atom_at(c);
+                int m_c = 0;
+                bool too_many;
+                if constexpr (kLarge) {
+                    // One pass over the partners, 64 at a time: list entries are written behind the batch's as they
+                    // are found (a centre that turns out not to fit leaves them there, unused, and opens the next
+                    // batch, where it is scanned again; its radial pairs are queued the first time only).
+                    const bool again = c == scanned;
+                    int pos = used;
+                    for (int jc = 0; jc < n; jc += 64) {
+                        const int j = jc + lane;
+                        const vec4 aj = atom_at(min(j, n - 1));
+                        const T ddx = ai.x - aj.x, ddy = ai.y - aj.y, ddz = ai.z - aj.z;
+                        const T rr = Fast<T>::sqrt_rn(ddx * ddx + ddy * ddy + ddz * ddz);
+                        const bool valid = (j < n) && (j != c);
+                        const unsigned long long mRb = wave_ballot(!kSkipRadial && !again && valid && (rr < kR_Rc_f) && (rr > T(0)));
+                        const unsigned long long mAb = wave_ballot(valid && (rr < kA_Rc_f) && (rr > T(0)));
+                        if ((mAb >> lane) & 1ull) {
+                            const int p = pos + popc64(mAb & lt_mask);
+                            if (p < 64) {
+                                P.nbr[p] = Fast<T>::make4(ddx, ddy, ddz, rr);
+                                P.nbr_idx[p] = static_cast<unsigned char>(static_cast<int>(aj.w));      // the partner's type
+                                M.pos[wave][p] = j;
+                            }
+                        }
+                        pos += popc64(mAb);
+                        m_c += popc64(mAb);
+                        if ((mRb >> lane) & 1ull) {
+                            const int p = qn + popc64(mRb & lt_mask);
+                            q_d[p] = Fast<T>::make4(ddx, ddy, ddz, rr);
+                            q_j[p] = static_cast<idx_t>(j);
+                            q_c[p] = static_cast<idx_t>(c);
+                        }
+                        qn += popc64(mRb);
+                        if (qn >= 64) radial_work_off_full();
+                    }
+                    scanned = c;
+                    too_many = m_c > 64;
+                    if (!too_many && nb > 0 && used + m_c > 64) {       // full: this centre opens the next batch
+                        pending = c;
+                        break;
+                    }
+                } else {
                 // first pass over the partners: who is inside the cutoffs
                 T dx[kChunks], dy[kChunks], dz[kChunks], r[kChunks];
                 unsigned long long mA[kChunks], mR[kChunks];
-                int m_c = 0;
 #pragma unroll
                 for (int ch = 0; ch < kChunks; ++ch) {
                     mA[ch] = 0ull;
@@ -228,7 +336,7 @@ void aev_bwd_medium_kernel(
                         m_c += popc64(mA[ch]);
                     }
                 }
-                const bool too_many = m_c > 64;        // more partners than a pool holds
+                too_many = m_c > 64;                   // more partners than a pool holds
                 if (!too_many && nb > 0 && used + m_c > 64) {       // full: this centre opens the next batch
                     pending = c;
                     break;
@@ -254,27 +362,9 @@ void aev_bwd_medium_kernel(
                             q_c[p] = static_cast<unsigned short>(c);
                         }
                         qn += popc64(mR[ch]);
-                        if (qn >= 64) {                  // a full wave of pairs: work it off, keep the rest
-                            wave_lds_fence();
-                            radial_work_off(64);
-                            const int rest = qn - 64;
-                            vec4 e = Fast<T>::make4(T(0), T(0), T(0), T(1));
-                            unsigned short ej = 0, ec = 0;
-                            if (lane < rest) {
-                                e = q_d[64 + lane];
-                                ej = q_j[64 + lane];
-                                ec = q_c[64 + lane];
-                            }
-                            wave_lds_fence();
-                            if (lane < rest) {
-                                q_d[lane] = e;
-                                q_j[lane] = ej;
-                                q_c[lane] = ec;
-                            }
-                            wave_lds_fence();
-                            qn = rest;
-                        }
+                        if (qn >= 64) radial_work_off_full();
                     }
+                }
                 }
                 if (!too_many) {
                     wave_lds_fence();
@@ -290,7 +380,7 @@ void aev_bwd_medium_kernel(
                 if (too_many) {
                     // the general per-centre routine does this centre's angular part alone (its radial pairs are
                     // in the queue like everyone's)
-                    const int i_orig = uniform(static_cast<int>(M.orig[c]));
+                    const int i_orig = uniform(orig_of(c));
                     radial_drain();                    // the routine uses the staging area as scratch
                     bwd_center_generic<T>(L, lane, X, Y, Z, A, off, n, i_orig, P.gst, row_of(c),
                                               [&](int atom, T fx, T fy, T fz) {
@@ -331,11 +421,16 @@ void aev_bwd_medium_kernel(
             const int bs = entry < total ? b : 0;
             const int pb = sel6(bs, 0, pf1, pf2, pf3, pf4, pf5);
             const int m = sel6(bs, pf1, pf2, pf3, pf4, pf5, pf6) - pb;
-            const vec4 f = bwd_angular_rounds<T>(P, entry, copy, copies, entry < total, bs, pb, m, type_of);
+            // (the byte per list entry: the partner's sorted position, or for large molecules its type)
+            const vec4 f = bwd_angular_rounds<T>(P, entry, copy, copies, entry < total, bs, pb, m,
+                                                 [&](int v) { if constexpr (kLarge) return v; else return type_of(v); });
             const bool live = lane < total;       // from here on one lane per entry again
 
             // ------------------------------------------------ gather
-            if (live) add_force(P.nbr_idx[lane], f.x, f.y, f.z);
+            if (live) {
+                if constexpr (kLarge) add_force(M.pos[wave][lane], f.x, f.y, f.z);
+                else add_force(P.nbr_idx[lane], f.x, f.y, f.z);
+            }
             {
                 // a centre's list is a run of lanes: its sum is the difference of two values of an add-scan,
                 // and lane b adds centre b's
@@ -374,11 +469,33 @@ hipError_t launch_bwd_medium(const T* X, const T* Y, const T* Z, const int32_t* 
     const int32_t cap = sizeof(T) == 4 ? 4096 : 1024;
     const unsigned blocks = static_cast<unsigned>(n_mols < cap ? n_mols : cap);
     aev_bwd_medium_kernel<T><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ, min_atoms,
-                                                                  order, walk_in_order);
+                                                                  order, walk_in_order, SortedAtoms<T>{});
+    return hipGetLastError();
+}
+
+// Molecules of more than 256 atoms: the sort into `scratch` (large_scratch_bytes), which also zeroes their gradients,
+// then the kernel above with the centres of a molecule spread over the workgroups of a grid column.
+template <typename T>
+hipError_t launch_bwd_large(const T* X, const T* Y, const T* Z, const int32_t* A,
+                            const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                            const int32_t* SIs, Buckets<const T> g, T* gX, T* gY, T* gZ,
+                            const int32_t* order, void* scratch, int64_t n_atoms, hipStream_t stream)
+{
+    if (n_mols <= 0) return hipSuccess;
+    const SortedAtoms<T> sorted = carve_sorted_atoms<T>(scratch, n_atoms, n_mols, false);
+    const hipError_t e = launch_large_sort<T>(X, Y, Z, A, MOs, MACs, n_mols, SIs, nullptr, nullptr, nullptr, gX, gY, gZ, order,
+                                              sorted, stream);
+    if (e != hipSuccess) return e;
+    const dim3 grid(static_cast<unsigned>(n_mols < kLargeColumns ? n_mols : kLargeColumns), kLargeParts);
+    aev_bwd_medium_kernel<T, true><<<grid, dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ,
+                                                                  kMediumMaxAtoms + 1, order, false, sorted);
     return hipGetLastError();
 }
 
 template hipError_t launch_bwd_medium<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const float>, float*, float*, float*, int, const int32_t*, bool, hipStream_t);
 template hipError_t launch_bwd_medium<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const double>, double*, double*, double*, int, const int32_t*, bool, hipStream_t);
+
+template hipError_t launch_bwd_large<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const float>, float*, float*, float*, const int32_t*, void*, int64_t, hipStream_t);
+template hipError_t launch_bwd_large<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const double>, double*, double*, double*, const int32_t*, void*, int64_t, hipStream_t);
 
 }  // namespace khan

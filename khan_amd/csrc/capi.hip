@@ -105,6 +105,37 @@ private:
     hipStream_t stream_;
 };
 
+// Stream-ordered scratch for the type-sorted copy of the molecules of more than 256 atoms.  None while the stream is
+// being captured into a graph, when the caller may not allocate, or when the allocation fails: those molecules then
+// go through the general-shape kernels, which need no scratch.
+class LargeScratch {
+public:
+    LargeScratch(size_t bytes, hipStream_t stream) : stream_(stream)
+    {
+        if (bytes == 0) return;
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return;
+        }
+        if (hipMallocAsync(&p_, bytes, stream) != hipSuccess) {
+            (void)hipGetLastError();
+            p_ = nullptr;
+        }
+    }
+    ~LargeScratch()
+    {
+        if (p_) (void)hipFreeAsync(p_, stream_);
+    }
+    LargeScratch(const LargeScratch&) = delete;
+    LargeScratch& operator=(const LargeScratch&) = delete;
+    void* get() const { return p_; }
+
+private:
+    void* p_ = nullptr;
+    hipStream_t stream_;
+};
+
 // Which kernels have work.  `classes` (host memory, null = not known: launch everything) holds the number of molecules
 // of up to 32 atoms, of 33..64, of 65..256 and of more, as khan_size_order leaves them behind the order.
 struct SizeClasses {
@@ -127,12 +158,13 @@ struct SizeClasses {
     }
 };
 
-// forward: one wavefront per molecule up to 32 atoms (float32; 64 in float64), one workgroup up to 256, the
-// general kernel above
+// forward: one wavefront per molecule up to 32 atoms (float32; 64 in float64), one workgroup up to 256, several
+// workgroups above (on a sorted copy of the atoms in scratch memory; without scratch, the general kernel)
 template <typename T>
 int forward_dispatch(const T* xs, const T* ys, const T* zs, const int32_t* as, const int32_t* mos,
                      const int32_t* macs, int32_t n_mols, const int32_t* sis, khan::Buckets<T> out,
-                     const int32_t* order, const int32_t* classes_host, hipStream_t stream)
+                     const int32_t* order, const int32_t* classes_host, int64_t n_atoms, bool may_allocate,
+                     hipStream_t stream)
 {
     if (force_generic())
         return hip_status(khan::launch_fwd_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out, 0, nullptr, stream));
@@ -143,9 +175,15 @@ int forward_dispatch(const T* xs, const T* ys, const T* zs, const int32_t* as, c
         st = hip_status(khan::launch_fwd_small<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out, small_max, order, stream));
     if (st == KHAN_OK && cls.any(small_max + 1, khan::kMediumMaxAtoms))
         st = hip_status(khan::launch_fwd_medium<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out, small_max + 1, order, stream));
-    if (st == KHAN_OK && cls.any(khan::kMediumMaxAtoms + 1, INT32_MAX))
-        st = hip_status(khan::launch_fwd_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
-                                                    khan::kMediumMaxAtoms + 1, order, stream));
+    if (st == KHAN_OK && n_atoms > khan::kMediumMaxAtoms && cls.any(khan::kMediumMaxAtoms + 1, INT32_MAX)) {      // (n_atoms: of the whole batch)
+        const LargeScratch scratch(may_allocate ? khan::large_scratch_bytes<T>(n_atoms, n_mols, false) : 0, stream);
+        if (scratch.get())
+            st = hip_status(khan::launch_fwd_large<T>(xs, ys, zs, as, mos, macs, n_mols, sis, nullptr, nullptr, nullptr, out,
+                                                      order, scratch.get(), n_atoms, stream));
+        else
+            st = hip_status(khan::launch_fwd_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out,
+                                                        khan::kMediumMaxAtoms + 1, order, stream));
+    }
     return st;
 }
 
@@ -164,9 +202,15 @@ int backward_dispatch(const T* xs, const T* ys, const T* zs, const int32_t* as, 
     constexpr int small_max = sizeof(T) == 4 ? khan::kSmallPreferredMax : khan::kSmallMaxAtoms;
     const SizeClasses cls(classes_host);
     int st = KHAN_OK;
-    if (cls.any(khan::kMediumMaxAtoms + 1, INT32_MAX))
-        st = hip_status(khan::launch_bwd_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                    n_atoms, khan::kMediumMaxAtoms + 1, order, stream));
+    if (n_atoms > khan::kMediumMaxAtoms && cls.any(khan::kMediumMaxAtoms + 1, INT32_MAX)) {
+        const LargeScratch scratch(khan::large_scratch_bytes<T>(n_atoms, n_mols, false), stream);
+        if (scratch.get())
+            st = hip_status(khan::launch_bwd_large<T>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, order,
+                                                      scratch.get(), n_atoms, stream));
+        else
+            st = hip_status(khan::launch_bwd_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
+                                                        n_atoms, khan::kMediumMaxAtoms + 1, order, stream));
+    }
     // (the workgroup-per-molecule backward kernel measures slower when it walks the molecules in size order)
     if (st == KHAN_OK && cls.any(small_max + 1, khan::kMediumMaxAtoms))
         st = hip_status(khan::launch_bwd_medium<T>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
@@ -222,10 +266,12 @@ int featurize_impl(const T* xs, const T* ys, const T* zs, const int32_t* as, con
     const int st = featurize_check(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, as_stream(stream), &run);
     if (st != KHAN_OK || !run) return st;
     khan::Buckets<T> out{{h, c, n, o}};
-    if (!own_order)       // the caller's size order (or none): nothing is allocated
-        return forward_dispatch<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out, caller_order, classes_host, as_stream(stream));
+    const int64_t n_atoms = static_cast<int64_t>(acs_host[0]) + acs_host[1] + acs_host[2] + acs_host[3];
+    if (!own_order)       // the caller's size order (or none)
+        return forward_dispatch<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out, caller_order, classes_host, n_atoms, true,
+                                   as_stream(stream));
     SizeOrder order(macs, n_mols, as_stream(stream));
-    return forward_dispatch<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out, order.get(), nullptr, as_stream(stream));
+    return forward_dispatch<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out, order.get(), nullptr, n_atoms, true, as_stream(stream));
 }
 
 template <typename T>
@@ -286,10 +332,17 @@ int featurize_grad_inverse_impl(const T* xs, const T* ys, const T* zs, const int
     if (st == KHAN_OK && cls.any(khan::kSmallMaxAtoms + 1, khan::kMediumMaxAtoms))
         st = hip_status(khan::launch_jvp_medium<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
                                                    khan::kSmallMaxAtoms + 1, order, as_stream(stream)));
-    const int generic_from = khan::kMediumMaxAtoms + 1;
-    if (st == KHAN_OK && cls.any(generic_from, INT32_MAX))
-        st = hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
-                                                    generic_from, order, as_stream(stream)));
+    if (st == KHAN_OK && cls.any(khan::kMediumMaxAtoms + 1, INT32_MAX)) {
+        const int64_t n_atoms = static_cast<int64_t>(acs_host[0]) + acs_host[1] + acs_host[2] + acs_host[3];
+        const LargeScratch scratch(n_atoms > khan::kMediumMaxAtoms ? khan::large_scratch_bytes<T>(n_atoms, n_mols, true) : 0,
+                                   as_stream(stream));
+        if (scratch.get())
+            st = hip_status(khan::launch_fwd_large<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, order,
+                                                      scratch.get(), n_atoms, as_stream(stream)));
+        else if (n_atoms > khan::kMediumMaxAtoms)
+            st = hip_status(khan::launch_jvp_generic<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out,
+                                                        khan::kMediumMaxAtoms + 1, order, as_stream(stream)));
+    }
     return st;
 }
 
@@ -445,7 +498,9 @@ int khan_featurize_f32_noalloc(const float* xs, const float* ys, const float* zs
     e = khan::launch_size_order(macs, n_mols, order, as_stream(stream));
     if (e != hipSuccess) return hip_status(e);
     khan::Buckets<float> out{{h, c, n, o}};
-    return forward_dispatch<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, order, nullptr, as_stream(stream));
+    // (molecules of more than 256 atoms go through the general-shape kernels here: the faster ones need scratch memory)
+    const int64_t n_atoms = static_cast<int64_t>(acs_host[0]) + acs_host[1] + acs_host[2] + acs_host[3];
+    return forward_dispatch<float>(xs, ys, zs, as, mos, macs, n_mols, sis, out, order, nullptr, n_atoms, false, as_stream(stream));
 }
 
 int khan_featurize_grad_f32(const float* xs, const float* ys, const float* zs, const int32_t* as,

@@ -53,6 +53,24 @@ hipError_t launch_jvp_medium(const T* X, const T* Y, const T* Z, const int32_t* 
                              const int32_t* SIs, const T* VX, const T* VY, const T* VZ,
                              Buckets<T> out, int min_atoms, const int32_t* order, hipStream_t stream);
 
+// ---- molecules of more than 256 atoms: the same kernels reading a type-sorted copy of the atoms from `scratch`
+// (large_scratch_bytes bytes of device memory, 256-byte aligned; with_vectors for the Jacobian-vector product) ----
+template <typename T>
+size_t large_scratch_bytes(int64_t n_atoms, int32_t n_mols, bool with_vectors);
+// forward, or with VX/VY/VZ the Jacobian-vector product
+template <typename T>
+hipError_t launch_fwd_large(const T* X, const T* Y, const T* Z, const int32_t* A,
+                            const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                            const int32_t* SIs, const T* VX, const T* VY, const T* VZ, Buckets<T> out,
+                            const int32_t* order, void* scratch, int64_t n_atoms, hipStream_t stream);
+
+// backward (the molecules' gradients need no zeroing beforehand)
+template <typename T>
+hipError_t launch_bwd_large(const T* X, const T* Y, const T* Z, const int32_t* A,
+                            const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
+                            const int32_t* SIs, Buckets<const T> g, T* gX, T* gY, T* gZ,
+                            const int32_t* order, void* scratch, int64_t n_atoms, hipStream_t stream);
+
 template <typename T>
 hipError_t launch_bwd_medium(const T* X, const T* Y, const T* Z, const int32_t* A,
                              const int32_t* MOs, const int32_t* MACs, int32_t n_mols,

@@ -667,6 +667,51 @@ def test_crowded_centres_take_the_fallback(ops):
     check_forward_backward(ops, c)
 
 
+def _sparse_box(rng, n, density, min_dist):
+    """n points in a cube at the given number density, no two closer than min_dist (cell by cell, so that thousands
+    of points take a moment and not minutes)."""
+    side = (n / density) ** (1 / 3)
+    pts = np.empty((0, 3))
+    while len(pts) < n:
+        cand = rng.uniform(0, side, (n, 3))
+        for p in cand:
+            if len(pts) == 0 or np.min(np.linalg.norm(pts - p, axis=1)) >= min_dist:
+                pts = np.vstack([pts, p])
+                if len(pts) == n:
+                    break
+    return pts
+
+
+def test_molecules_of_more_than_256_atoms(ops):
+    # above 256 atoms several workgroups share a molecule and read its atoms, sorted by type, from device memory:
+    # boxes of 257 to 1,500 atoms at the density of the dense-box workload, a crowded ball whose inner centres
+    # overflow the partner lists (more than 64 radial, more than 32 angular forward, more than 64 angular backward),
+    # a single-type box, ordinary molecules in between; features, gradients and the Jacobian-vector product
+    say("case: molecules of 257..1,500 atoms, one of them crowded")
+    rng = np.random.default_rng(41)
+    mols = []
+    small = datagen.make_batch("organic", 4, first_mol=11)
+    for m in range(4):
+        sl = slice(small.MOs[m], small.MOs[m] + small.MACs[m])
+        mols.append((small.A[sl], np.stack([small.X[sl], small.Y[sl], small.Z[sl]], axis=1)))
+    for n in (257, 700, 1500):
+        mols.append((rng.choice(4, n, p=[0.5, 0.3, 0.1, 0.1]), _sparse_box(rng, n, 0.1, 0.9)))
+    mols.append((rng.integers(0, 4, 420), _packed_ball(rng, 420, 5.0, 0.85)))
+    mols.append((np.full(300, 2), _sparse_box(rng, 300, 0.1, 0.9)))
+    box = datagen.make_batch("boxes", 1)
+    mols.append((box.A, np.stack([box.X, box.Y, box.Z], axis=1)))
+    mols = [mols[i] for i in rng.permutation(len(mols))]
+    p = max(mols, key=lambda m: len(m[0]) if len(m[0]) == 420 else 0)[1]
+    dm = np.linalg.norm(p[:, None] - p[None], axis=2)
+    assert int(((dm < 3.1) & (dm > 0)).sum(axis=1).max()) > 64 and int(((dm < 4.6) & (dm > 0)).sum(axis=1).max()) > 64
+    A = np.concatenate([m[0] for m in mols]).astype(np.int32)
+    xyz = np.concatenate([m[1] for m in mols]).astype(np.float32).astype(np.float64)
+    mi = np.concatenate([np.full(len(m[0]), k) for k, m in enumerate(mols)]).astype(np.int32)
+    c = Case(xyz[:, 0], xyz[:, 1], xyz[:, 2], A, mi, len(mols))
+    check_forward_backward(ops, c)
+    _check_grad_inverse(ops, c)
+
+
 def test_radial_lists_at_their_fullest(ops):
     # The one-wavefront forward kernel gives every partner type a place of its own in a centre's radial list, each
     # rounded up to a whole trip of the walk.  Fullest lists: molecules of exactly 16, 32 and 64 atoms (the three scan

@@ -60,6 +60,43 @@ def test_no_alloc_entry_point_matches_featurize_on_two_calls_in_a_row():
             assert np.all(np.abs(got - ref) <= 1e-6 + 1e-5 * np.abs(ref)), "no-alloc entry point vs the oracle"
 
 
+def test_no_alloc_entry_point_with_a_molecule_of_more_than_256_atoms():
+    # above 256 atoms khan_featurize_f32 works on a sorted copy of the atoms in scratch memory; the entry point that
+    # allocates nothing keeps to the kernels without scratch: the same features to float32 rounding, both checked
+    # against the oracle
+    from khan_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(9)
+    small = datagen.make_batch("organic", 3, first_mol=77)
+    n_big = 300
+    side = (n_big / 0.1) ** (1 / 3)
+    pts = np.empty((0, 3))
+    while len(pts) < n_big:
+        q = rng.uniform(0, side, 3)
+        if len(pts) == 0 or np.min(np.linalg.norm(pts - q, axis=1)) >= 0.9:
+            pts = np.vstack([pts, q])
+    X = np.concatenate([small.X, pts[:, 0]]).astype(np.float32)
+    Y = np.concatenate([small.Y, pts[:, 1]]).astype(np.float32)
+    Z = np.concatenate([small.Z, pts[:, 2]]).astype(np.float32)
+    A = np.concatenate([small.A, rng.integers(0, 4, n_big)]).astype(np.int32)
+    macs = np.concatenate([small.MACs, [n_big]]).astype(np.int32)
+    mos = np.concatenate([[0], np.cumsum(macs)[:-1]]).astype(np.int32)
+    sc, _, ac = ob.ani_sort(A)
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")
+    t = {"X": d(X), "Y": d(Y), "Z": d(Z), "A": d(A), "mos": d(mos), "macs": d(macs), "sc": d(sc)}
+    n = len(A)
+    say("   no-alloc entry point: 3 small molecules and one of %d atoms" % n_big)
+    ref_out = torch.full((n * 384,), -1.0, dtype=torch.float32, device="cuda:0")
+    new_out = torch.full((n * 384,), -2.0, dtype=torch.float32, device="cuda:0")
+    assert _call(lib, "khan_featurize_f32", t, ac, ref_out) == 0
+    assert _call(lib, "khan_featurize_f32_noalloc", t, ac, new_out) == 0
+    torch.cuda.synchronize()
+    ref = np.concatenate(ob.featurize(X, Y, Z, A, mos, macs, sc, ac, dtype=np.float64))
+    for name, got in (("khan_featurize_f32", ref_out), ("khan_featurize_f32_noalloc", new_out)):
+        g = got.cpu().numpy().astype(np.float64)
+        assert np.all(np.abs(g - ref) <= 1e-6 + 1e-5 * np.abs(ref)), name + " vs the oracle"
+
+
 def test_no_alloc_entry_point_rejects_what_its_scratch_cannot_hold():
     from khan_amd import _lib
     lib = _lib.load()
