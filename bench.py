@@ -222,7 +222,7 @@ def grad_inverse_bench(args, batch, w, kind):
     ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
     launch_ms = e0.elapsed_time(e1) / args.steps
     nbytes = N * (384 * w + 6 * w + 8) + 8 * n_mols
-    kernel = "aev_fwd_%s_kernel<%s, true>" % ("small" if kind == "organic" else "medium", tname)
+    kernel = "aev_fwd_%s_kernel<%s, true, false>" % ("small" if kind == "organic" else "medium", tname)
     print(json.dumps({
         "metric": "AEV grad-inverse (Jacobian-vector product) atoms/sec, fp%d, 1 MI355X" % (8 * w),
         "value": N / (ms_per_step * 1e-3), "unit": "atoms/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

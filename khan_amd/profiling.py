@@ -42,8 +42,8 @@ DOMINANT = {
     ("organic1024", "bwd"): "aev_bwd_small_kernel<float>",
     ("organic16384_f64", "fwd"): "aev_fwd_small_kernel<double, false, false>",
     ("organic16384_f64", "bwd"): "aev_bwd_small_kernel<double>",
-    ("boxes4096", "fwd"): "aev_fwd_medium_kernel<float, false>",
-    ("boxes4096", "bwd"): "aev_bwd_medium_kernel<float>",
+    ("boxes4096", "fwd"): "aev_fwd_medium_kernel<float, false, false>",
+    ("boxes4096", "bwd"): "aev_bwd_medium_kernel<float, false>",
 }
 
 
