@@ -1,8 +1,10 @@
 """KHAN_AEV_FORCE_GENERIC=1 (read once per process by libkhan_aev.so) routes every molecule through the general-shape
-kernels (workgroup per molecule, wavefront per centre), which otherwise only see molecules of more than 256 atoms and
-the centres whose lists overflow.  Features, gradients and the Jacobian-vector product of organic molecules and dense
-boxes from those kernels are checked against the float64 oracle at the tolerances of test_gpu_parity.py; the variable is
-read at the first launch, so the run is a child process."""
+kernels (workgroup per molecule, wavefront per centre), which otherwise only see the centres whose lists overflow and,
+when no scratch memory may be taken, molecules of more than 256 atoms.  KHAN_AEV_LARGE_SCRATCH=0 withholds that scratch
+memory, as a stream under graph capture or a failed allocation would: molecules of more than 256 atoms then go to the
+general-shape kernels while the others keep to theirs.  Features, gradients and the Jacobian-vector product from both
+variants are checked against the float64 oracle at the tolerances of test_gpu_parity.py; the variables are read at the
+first launch, so each run is a child process."""
 import os
 import subprocess
 import sys
@@ -22,9 +24,11 @@ CHILD = r"""
 import sys
 import numpy as np, torch
 sys.path.insert(0, sys.argv[1])
-from khan_amd import datagen, ops
-kind, n_mols, out = sys.argv[2], int(sys.argv[3]), sys.argv[4]
-b = datagen.make_batch(kind, n_mols)
+from types import SimpleNamespace
+from khan_amd import ops
+inp, out = np.load(sys.argv[2]), sys.argv[3]
+b = SimpleNamespace(X=inp["X"], Y=inp["Y"], Z=inp["Z"], A=inp["A"], mol_idxs=inp["mol_idxs"], n_mols=int(inp["n_mols"]),
+                    n_atoms=len(inp["A"]))
 d = "cuda:0"
 res = {}
 A = torch.from_numpy(b.A).to(d)
@@ -51,9 +55,35 @@ np.savez(out, **res)
 """
 
 
-@pytest.mark.parametrize("kind,n_mols", [("organic", 96), ("boxes", 2)])
-def test_general_shape_kernels_match_the_oracle(tmp_path, kind, n_mols):
-    b = datagen.make_batch(kind, n_mols)
+def _with_large_molecules():
+    """three organic molecules, a dense box, and boxes of 300 and 520 atoms at 0.1 atoms per cubic Angstrom"""
+    from types import SimpleNamespace
+    rng = np.random.default_rng(23)
+    parts = []
+    for kind, n in (("organic", 3), ("boxes", 1)):
+        s = datagen.make_batch(kind, n)
+        for m in range(n):
+            sl = slice(s.MOs[m], s.MOs[m] + s.MACs[m])
+            parts.append((s.A[sl], np.stack([s.X[sl], s.Y[sl], s.Z[sl]], 1)))
+    for n in (300, 520):
+        side = (n / 0.1) ** (1 / 3)
+        pts = np.empty((0, 3))
+        while len(pts) < n:
+            q = rng.uniform(0, side, 3)
+            if len(pts) == 0 or np.min(np.linalg.norm(pts - q, axis=1)) >= 0.9:
+                pts = np.vstack([pts, q])
+        parts.insert(1, (rng.integers(0, 4, n), pts))
+    A = np.concatenate([p[0] for p in parts]).astype(np.int32)
+    xyz = np.concatenate([p[1] for p in parts]).astype(np.float32)
+    mi = np.concatenate([np.full(len(p[0]), k) for k, p in enumerate(parts)]).astype(np.int32)
+    return SimpleNamespace(X=xyz[:, 0].copy(), Y=xyz[:, 1].copy(), Z=xyz[:, 2].copy(), A=A, mol_idxs=mi, n_mols=len(parts),
+                           n_atoms=len(A))
+
+
+@pytest.mark.parametrize("kind,n_mols,variable", [("organic", 96, "KHAN_AEV_FORCE_GENERIC=1"), ("boxes", 2, "KHAN_AEV_FORCE_GENERIC=1"),
+                                                  ("large", 6, "KHAN_AEV_LARGE_SCRATCH=0")])
+def test_general_shape_kernels_match_the_oracle(tmp_path, kind, n_mols, variable):
+    b = _with_large_molecules() if kind == "large" else datagen.make_batch(kind, n_mols)
     MACs, MOs = ob.mol_offsets(b.mol_idxs, b.n_mols)
     sc, ga, ac = ob.ani_sort(b.A)
     up = np.random.default_rng(11).standard_normal((b.n_atoms, 384))
@@ -62,11 +92,13 @@ def test_general_shape_kernels_match_the_oracle(tmp_path, kind, n_mols):
     upb = ob.scatter_rows(up, b.A, sc, ac)
     grad = np.stack(ob.featurize_grad(b.X, b.Y, b.Z, b.A, MOs, MACs, sc, ac, upb, dtype=np.float64), 1)
     jvp = np.concatenate(ob.featurize_grad_inverse(b.X, b.Y, b.Z, b.A, MOs, MACs, sc, ac, v[0], v[1], v[2], dtype=np.float64))
-    out = str(tmp_path / "generic.npz")
+    out, inp = str(tmp_path / "generic.npz"), str(tmp_path / "inputs.npz")
+    np.savez(inp, X=b.X, Y=b.Y, Z=b.Z, A=b.A, mol_idxs=b.mol_idxs, n_mols=b.n_mols)
     env = dict(os.environ)
-    env["KHAN_AEV_FORCE_GENERIC"] = "1"
-    print("child: KHAN_AEV_FORCE_GENERIC=1, %s %d molecules" % (kind, n_mols), flush=True)
-    subprocess.run([sys.executable, "-c", CHILD, ROOT, kind, str(n_mols), out], env=env, check=True, timeout=300)
+    name, value = variable.split("=")
+    env[name] = value
+    print("child: %s, %s, %d molecules, %d atoms" % (variable, kind, b.n_mols, b.n_atoms), flush=True)
+    subprocess.run([sys.executable, "-c", CHILD, ROOT, inp, out], env=env, check=True, timeout=300)
     got = np.load(out)
     gscale = np.zeros_like(grad)
     for m in range(b.n_mols):
