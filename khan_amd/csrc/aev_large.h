@@ -57,7 +57,13 @@ hipError_t launch_large_sort(const T* X, const T* Y, const T* Z, const int32_t* 
                              const T* VZ, T* gX, T* gY, T* gZ, const int32_t* order, SortedAtoms<T> sorted,
                              hipStream_t stream);
 
-constexpr int kLargeParts = 64;      // workgroups that share a large molecule's centres (grid's y extent)
-constexpr int kLargeColumns = 32;    // molecules in flight (grid's x extent)
+// Grid of the kernels for large molecules: x = molecules in flight (at most 32), y = workgroups that share a
+// molecule's centres (64; more when the batch has few molecules, so that one large molecule alone still fills the GPU).
+__host__ inline dim3 large_grid(int32_t n_mols)
+{
+    const unsigned columns = static_cast<unsigned>(n_mols < 32 ? n_mols : 32);
+    const unsigned parts = columns >= 32 ? 64u : (2048u / columns > 1024u ? 1024u : 2048u / columns);
+    return dim3(columns, parts);
+}
 
 }  // namespace khan

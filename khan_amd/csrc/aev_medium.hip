@@ -158,10 +158,13 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
         };
 
         // ------------------------------------------------------------ batches of kNB centres per wavefront
-        const int first_c0 = (kLarge ? static_cast<int>(blockIdx.y) * 4 + wave : wave) * kNB;
-        const int stride_c0 = (kLarge ? static_cast<int>(gridDim.y) : 1) * 4 * kNB;
+        // (a large molecule that has the grid column to itself: shorter batches, so that every wavefront gets centres)
+        const int waves_y = static_cast<int>(gridDim.y) * 4;
+        const int batch = kLarge ? max(1, min(kNB, (n + waves_y - 1) / waves_y)) : kNB;
+        const int first_c0 = (kLarge ? static_cast<int>(blockIdx.y) * 4 + wave : wave) * batch;
+        const int stride_c0 = (kLarge ? waves_y : 4) * batch;
         for (c0 = first_c0; c0 < n; c0 += stride_c0) {
-            const int nb = min(kNB, n - c0);
+            const int nb = min(batch, n - c0);
             unsigned overflow = 0;
             if constexpr (kLarge) {
                 if (lane < nb) {
@@ -177,10 +180,9 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                 const vec4 ai = atom_at(i);
                 int posR = 0, posA = 0;                 // list lengths so far (wave-uniform)
                 int cR[4] = {0, 0, 0, 0}, cA[4] = {0, 0, 0, 0};
-                for (int jc = 0; jc < n; jc += 64) {
+                // one chunk of 64 partners: aj (and with kJvp vjv) of the atom at sorted position jc + lane
+                auto scan_chunk = [&](int jc, const vec4 aj, const vec4 vjv) {
                     const int j = jc + lane;
-                    const int jj = min(j, last_atom);
-                    const vec4 aj = atom_at(jj);
                     const T dx = ai.x - aj.x, dy = ai.y - aj.y, dz = ai.z - aj.z;
                     const T r = Fast<T>::sqrt_rn(dx * dx + dy * dy + dz * dz);
                     const bool valid = (j < n) && (j != i);
@@ -197,7 +199,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                             cA[a] += popc64(mA & ta);
                         }
                         const T inv = Fast<T>::rcp(r);
-                        const vec4 vi = vel_at(i), vjv = vel_at(jj);
+                        const vec4 vi = vel_at(i);
                         const T wx = vi.x - vjv.x, wy = vi.y - vjv.y, wz = vi.z - vjv.z;     // v_centre - v_partner
                         const T rd = (dx * wx + dy * wy + dz * wz) * inv;                    // d r along it
                         if (inR) {
@@ -239,6 +241,26 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                     }
                     posR += popc64(mR);
                     posA += popc64(mA);
+                };
+                if constexpr (kLarge) {
+                    // from device memory: four chunks' loads in flight at a time
+                    for (int jt = 0; jt < n; jt += 256) {
+                        vec4 at[4], vt[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int jj = min(jt + u * 64 + lane, last_atom);
+                            at[u] = atom_at(jj);
+                            vt[u] = vel_at(jj);
+                        }
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+                            if (jt + u * 64 < n) scan_chunk(jt + u * 64, at[u], vt[u]);
+                    }
+                } else {
+                    for (int jc = 0; jc < n; jc += 64) {
+                        const int jj = min(jc + lane, last_atom);
+                        scan_chunk(jc, atom_at(jj), vel_at(jj));
+                    }
                 }
                 if constexpr (!kJvp) {
                     wave_lds_fence();
@@ -380,7 +402,7 @@ hipError_t launch_fwd_large(const T* X, const T* Y, const T* Z, const int32_t* A
     const hipError_t e = launch_large_sort<T>(X, Y, Z, A, MOs, MACs, n_mols, SIs, VX, VY, VZ, nullptr, nullptr, nullptr, order,
                                               sorted, stream);
     if (e != hipSuccess) return e;
-    const dim3 grid(static_cast<unsigned>(n_mols < kLargeColumns ? n_mols : kLargeColumns), kLargeParts);
+    const dim3 grid = large_grid(n_mols);
     if (jvp)
         aev_fwd_medium_kernel<T, true, true><<<grid, dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, VX, VY, VZ, out,
                                                                          kMediumMaxAtoms + 1, order, sorted);

@@ -280,9 +280,8 @@ void aev_bwd_medium_kernel(
                     // batch, where it is scanned again; its radial pairs are queued the first time only).
                     const bool again = c == scanned;
                     int pos = used;
-                    for (int jc = 0; jc < n; jc += 64) {
+                    auto scan_chunk = [&](int jc, const vec4 aj) {
                         const int j = jc + lane;
-                        const vec4 aj = atom_at(min(j, n - 1));
                         const T ddx = ai.x - aj.x, ddy = ai.y - aj.y, ddz = ai.z - aj.z;
                         const T rr = Fast<T>::sqrt_rn(ddx * ddx + ddy * ddy + ddz * ddz);
                         const bool valid = (j < n) && (j != c);
@@ -306,6 +305,14 @@ void aev_bwd_medium_kernel(
                         }
                         qn += popc64(mRb);
                         if (qn >= 64) radial_work_off_full();
+                    };
+                    for (int jt = 0; jt < n; jt += 256) {          // four chunks' loads in flight at a time
+                        vec4 at[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) at[u] = atom_at(min(jt + u * 64 + lane, n - 1));
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+                            if (jt + u * 64 < n) scan_chunk(jt + u * 64, at[u]);
                     }
                     scanned = c;
                     too_many = m_c > 64;
@@ -486,7 +493,7 @@ hipError_t launch_bwd_large(const T* X, const T* Y, const T* Z, const int32_t* A
     const hipError_t e = launch_large_sort<T>(X, Y, Z, A, MOs, MACs, n_mols, SIs, nullptr, nullptr, nullptr, gX, gY, gZ, order,
                                               sorted, stream);
     if (e != hipSuccess) return e;
-    const dim3 grid(static_cast<unsigned>(n_mols < kLargeColumns ? n_mols : kLargeColumns), kLargeParts);
+    const dim3 grid = large_grid(n_mols);
     aev_bwd_medium_kernel<T, true><<<grid, dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ,
                                                                   kMediumMaxAtoms + 1, order, false, sorted);
     return hipGetLastError();
