@@ -37,6 +37,9 @@ WORKLOADS = {
     "organic1024": ("organic", 1024, 4, False),
     "organic16384_f64": ("organic", 16384, 8, True),     # double precision forward + backward + ani_charge
     "boxes4096": ("boxes", 4096, 4, False),              # dense boxes of 64..256 atoms
+    # not a line of the headline metric: boxes of 1,024..4,096 atoms (several workgroups per molecule, the atoms read
+    # type-sorted from device memory)
+    "bigboxes64": ("bigboxes", 64, 4, False),
     # not a line of the headline metric: energies and coordinate gradients through the atomic networks
     # (384-128-128-64-1 per type, random weights), the caller either side of the hot path
     "inference65536": ("organic", 65536, 4, False),

@@ -15,6 +15,7 @@
  *  boxes    n ~ U{64..256} atoms in a cube of side (n/0.1)^(1/3) A (number density 0.1 / A^3), placed by
  *           dart throwing with minimum distance 0.9 A, open boundaries, types H/C/N/O with
  *           p = 0.5/0.3/0.1/0.1.  One box is one "molecule".
+ *  bigboxes the same with n ~ U{1024..4096} atoms (systems of more than 256 atoms).
  *
  * Every molecule has its own random stream keyed by (seed, stream tag, molecule index), so a batch of
  * M molecules is a prefix of any larger batch made with the same seed.  Coordinates are drawn in
@@ -85,6 +86,8 @@ static void rng_direction(rng_t *g, double *u)   /* uniform on the unit sphere *
 #define MAX_ORGANIC_ATOMS 26
 #define TAG_ORGANIC 1ULL
 #define TAG_BOX 2ULL
+#define TAG_BIGBOX 3ULL
+#define MAX_MOL_ATOMS 4096
 
 static int too_close(const double (*p)[3], int n, const double *q, double dmin)
 {
@@ -166,9 +169,9 @@ static int organic_molecule(rng_t *g, int32_t *type, double (*pos)[3])
     }
 }
 
-static int box_molecule(rng_t *g, int32_t *type, double (*pos)[3])
+static int box_molecule(rng_t *g, int32_t *type, double (*pos)[3], int n_min, int n_span)
 {
-    const int n = 64 + rng_below(g, 193);
+    const int n = n_min + rng_below(g, n_span);
     const double side = cbrt((double)n / 0.1);
     int placed = 0;
     while (placed < n) {
@@ -182,7 +185,7 @@ static int box_molecule(rng_t *g, int32_t *type, double (*pos)[3])
     return n;
 }
 
-/* Generates molecules [first_mol, first_mol+n_mols) of the batch `kind` (0 organic, 1 boxes).
+/* Generates molecules [first_mol, first_mol+n_mols) of the batch `kind` (0 organic, 1 boxes, 2 bigboxes).
  * mol_atom_counts[n_mols] is always written.  If X is non-NULL, coordinates/types/mol_idxs of up to
  * `capacity` atoms are written too (mol_idxs counts from 0 at first_mol).  Returns the total atom
  * count, or -1 if capacity was too small, -2 for an unknown kind. */
@@ -190,14 +193,16 @@ int64_t khan_gen_batch(int32_t kind, uint64_t seed, int64_t first_mol, int64_t n
                        int32_t *mol_atom_counts, float *X, float *Y, float *Z, int32_t *A,
                        int32_t *mol_idxs, int64_t capacity)
 {
-    if (kind != 0 && kind != 1) return -2;
+    if (kind < 0 || kind > 2) return -2;
     int64_t total = 0;
-    int32_t type[256];
-    double pos[256][3];
+    static _Thread_local int32_t type[MAX_MOL_ATOMS];
+    static _Thread_local double pos[MAX_MOL_ATOMS][3];
     for (int64_t m = 0; m < n_mols; ++m) {
         rng_t g;
-        rng_seed(&g, seed, kind == 0 ? TAG_ORGANIC : TAG_BOX, (uint64_t)(first_mol + m));
-        const int n = (kind == 0) ? organic_molecule(&g, type, pos) : box_molecule(&g, type, pos);
+        rng_seed(&g, seed, kind == 0 ? TAG_ORGANIC : kind == 1 ? TAG_BOX : TAG_BIGBOX, (uint64_t)(first_mol + m));
+        const int n = (kind == 0)   ? organic_molecule(&g, type, pos)
+                      : (kind == 1) ? box_molecule(&g, type, pos, 64, 193)
+                                    : box_molecule(&g, type, pos, 1024, 3073);
         mol_atom_counts[m] = n;
         if (X) {
             if (total + n > capacity) return -1;

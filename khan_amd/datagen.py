@@ -14,7 +14,8 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libkhan_datagen.so")
 DEFAULT_SEED = 0x4B48414E
-KINDS = {"organic": 0, "boxes": 1}
+KINDS = {"organic": 0, "boxes": 1, "bigboxes": 2}
+MAX_ATOMS = {0: 26, 1: 256, 2: 4096}     # atoms per molecule, by kind
 TAG_CHARGES = 1
 TAG_UPSTREAM = 2
 
@@ -73,7 +74,7 @@ def make_batch(kind="organic", n_mols=1024, seed=DEFAULT_SEED, first_mol=0):
     lib = _load()
     k = KINDS[kind]
     macs = np.zeros(n_mols, dtype=np.int32)
-    cap = n_mols * (26 if k == 0 else 256)
+    cap = n_mols * MAX_ATOMS[k]
     X = np.empty(cap, dtype=np.float32)
     Y = np.empty(cap, dtype=np.float32)
     Z = np.empty(cap, dtype=np.float32)
