@@ -77,7 +77,7 @@ int khan_ani_sort(const int32_t *atomic_numbers, int64_t n_atoms, int32_t *scatt
  * out: h_feat[acs[0]*384], c_feat[acs[1]*384], n_feat[acs[2]*384], o_feat[acs[3]*384], row-major;
  *      the row of atom g is bucket[as[g]] + sis[g]*384.
  * Scratch, from the stream-ordered allocator on every call: the molecule indices in order of decreasing size, and,
- * for molecules of more than 256 atoms, a sorted copy of the atoms (24 bytes per atom of the batch in float32, 40 in
+ * for molecules of more than 256 atoms, a sorted copy of the atoms (about 25 bytes per atom and 48 per molecule of the batch in float32, 41 per atom in
  * float64).  While the stream is being captured into a graph neither is taken: molecules then run in the order given,
  * and those of more than 256 atoms in slower kernels that need no scratch. */
 int khan_featurize_f32(const float *xs, const float *ys, const float *zs, const int32_t *as,

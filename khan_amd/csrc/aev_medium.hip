@@ -128,6 +128,8 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
         __syncthreads();
         }
         const int last_atom = (kLarge ? n : kMediumMaxAtoms) - 1;
+        const int n_chunks = (n + 63) >> 6;
+        const size_t chunk0 = kLarge ? chunk_base(off, mol) : 0;     // the molecule's first chunk box
         auto atom_at = [&](int sorted_idx) -> vec4 {
             if constexpr (kLarge) return sorted.atom[off + sorted_idx];
             else return M.atom[sorted_idx];
@@ -180,6 +182,62 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                 const vec4 ai = atom_at(i);
                 int posR = 0, posA = 0;                 // list lengths so far (wave-uniform)
                 int cR[4] = {0, 0, 0, 0}, cA[4] = {0, 0, 0, 0};
+                // adds the radial list's entries (cnt[a] of type a, laid end to end) to acc[a]: lanes = (slot of 4) x (shell)
+                auto radial_sums = [&](T (&acc)[4], const int (&cnt)[4]) {
+                    int obase = 0;
+#pragma unroll
+                    for (int a = 0; a < 4; ++a) {
+                        const int cnt_a = cnt[a];
+                        T acc_r = T(0);
+                        for (int q0 = 0; q0 < (kSkipRadial ? 0 : cnt_a); q0 += 4 * kMedRadTrip) {
+                            vec2 e[kMedRadTrip], ab[kMedRadTrip];
+#pragma unroll
+                            for (int u = 0; u < kMedRadTrip; ++u) {
+                                const int at = min(obase + q0 + u * 4 + rslot, kRadCap - 1);
+                                e[u] = S.rad[at];
+                                if constexpr (kJvp) ab[u] = S.jvp.rad_ab[at];
+                            }
+#pragma unroll
+                            for (int u = 0; u < kMedRadTrip; ++u) {
+                                const T dd = e[u].x - L.rrs;
+                                // forward: exp(-eta d^2) f_C; derivative: exp(-eta d^2) (f_C' - 2 eta d f_C) dr
+                                T v = Fast<T>::gauss(static_cast<T>(kR_eta_f), dd);
+                                if constexpr (kJvp) v *= fma(ab[u].y, dd, ab[u].x);
+                                else v *= e[u].y;
+                                acc_r += (q0 + u * 4 + rslot < cnt_a) ? v : T(0);   // entries of other types: select
+                            }
+                        }
+                        acc[a] += acc_r;
+                        obase += cnt_a;
+                    }
+                };
+                // Large molecules: a centre's radial list is worked off whenever the next chunk's entries would not fit
+                // (no limit on the number of radial partners); racc collects the sums, cRdone the counts at the last time.
+                T racc[4] = {T(0), T(0), T(0), T(0)};
+                int cRdone[4] = {0, 0, 0, 0};
+                auto radial_flush = [&](int count) {
+                    wave_lds_fence();
+                    int cnt[4];
+                    if constexpr (kJvp) {
+#pragma unroll
+                        for (int a = 0; a < 4; ++a) {
+                            cnt[a] = cR[a] - cRdone[a];
+                            cRdone[a] = cR[a];
+                        }
+                    } else {
+                        int tR = -1;
+                        if (lane < count) {
+                            const vec2 e = S.rad[lane];
+                            tR = static_cast<int>(e.y);
+                            S.rad[lane] = Fast<T>::make2(e.x, Fast<T>::cutoff(e.x, static_cast<T>(kR_Rc_f)));
+                        }
+#pragma unroll
+                        for (int a = 0; a < 4; ++a) cnt[a] = popc64(wave_ballot(tR == a));
+                        wave_lds_fence();
+                    }
+                    radial_sums(racc, cnt);
+                    wave_lds_fence();               // the list may be overwritten
+                };
                 // one chunk of 64 partners: aj (and with kJvp vjv) of the atom at sorted position jc + lane
                 auto scan_chunk = [&](int jc, const vec4 aj, const vec4 vjv) {
                     const int j = jc + lane;
@@ -190,6 +248,12 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                     const bool inR = valid && (r < kR_Rc_f) && (!kJvp || r > T(0));
                     const bool inA = valid && (r < kA_Rc_f) && (!kJvp || r > T(0));
                     const unsigned long long mR = wave_ballot(inR), mA = wave_ballot(inA);
+                    if constexpr (kLarge) {
+                        if (posR + popc64(mR) > kRadCap) {
+                            radial_flush(posR);
+                            posR = 0;
+                        }
+                    }
                     if constexpr (kJvp) {
                         const int tj = static_cast<int>(aj.w);
 #pragma unroll
@@ -243,18 +307,33 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                     posA += popc64(mA);
                 };
                 if constexpr (kLarge) {
-                    // from device memory: four chunks' loads in flight at a time
-                    for (int jt = 0; jt < n; jt += 256) {
-                        vec4 at[4], vt[4];
+                    // From device memory.  The atoms are sorted by type and, inside a type, along a space-filling
+                    // curve: 64 chunks' boxes are tested against the centre at a time (one per lane), and only the
+                    // chunks that reach into the radial cutoff are scanned, four chunks' loads in flight at a time.
+                    const float cx = static_cast<float>(ai.x), cy = static_cast<float>(ai.y), cz = static_cast<float>(ai.z);
+                    for (int ch0 = 0; ch0 < n_chunks; ch0 += 64) {
+                        unsigned long long near = wave_ballot(chunk_in_reach(sorted.box + 2 * chunk0, ch0 + lane, n_chunks, cx, cy, cz));
+                        while (near) {
+                            int ch[4];
 #pragma unroll
-                        for (int u = 0; u < 4; ++u) {
-                            const int jj = min(jt + u * 64 + lane, last_atom);
-                            at[u] = atom_at(jj);
-                            vt[u] = vel_at(jj);
+                            for (int u = 0; u < 4; ++u) {
+                                ch[u] = -1;
+                                if (near) {
+                                    ch[u] = ch0 + lowest_bit(near);
+                                    near &= near - 1;
+                                }
+                            }
+                            vec4 at[4], vt[4];
+#pragma unroll
+                            for (int u = 0; u < 4; ++u) {
+                                const int jj = min(max(ch[u], 0) * 64 + lane, last_atom);
+                                at[u] = atom_at(jj);
+                                vt[u] = vel_at(jj);
+                            }
+#pragma unroll
+                            for (int u = 0; u < 4; ++u)
+                                if (ch[u] >= 0) scan_chunk(ch[u] * 64, at[u], vt[u]);
                         }
-#pragma unroll
-                        for (int u = 0; u < 4; ++u)
-                            if (jt + u * 64 < n) scan_chunk(jt + u * 64, at[u], vt[u]);
                     }
                 } else {
                     for (int jc = 0; jc < n; jc += 64) {
@@ -262,9 +341,10 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                         scan_chunk(jc, atom_at(jj), vel_at(jj));
                     }
                 }
+                if constexpr (kLarge) radial_flush(posR);
                 if constexpr (!kJvp) {
                     wave_lds_fence();
-                    const bool haveR = lane < min(posR, kRadCap), haveA = lane < min(posA, kCapA);
+                    const bool haveR = !kLarge && lane < min(posR, kRadCap), haveA = lane < min(posA, kCapA);
                     int tR = -1, tA = -1;           // type of this lane's list entry
                     if (haveR) {
                         const vec2 e = S.rad[lane];
@@ -286,7 +366,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                         cA[a] = popc64(wave_ballot(tA == a));
                     }
                 }
-                const bool fits = (posR <= kRadCap) && (posA <= kCapA);
+                const bool fits = (kLarge || posR <= kRadCap) && (posA <= kCapA);
                 if (!fits) overflow |= 1u << b;
                 if (lane < 4) S.nA[b][lane] = fits ? sel4(lane, cA[0], cA[1], cA[2], cA[3]) : 0;
                 wave_lds_fence();
@@ -294,33 +374,14 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                 // ---- radial features of this centre: lanes = (slot of 4) x (shell)
                 if (fits) {
                     T* row = row_of(i);
-                    int obase = 0;
+                    T acc[4] = {racc[0], racc[1], racc[2], racc[3]};
+                    if constexpr (!kLarge) radial_sums(acc, cR);
 #pragma unroll
                     for (int a = 0; a < 4; ++a) {
-                        const int cnt_a = cR[a];
-                        T acc_r = T(0);
-                        for (int q0 = 0; q0 < (kSkipRadial ? 0 : cnt_a); q0 += 4 * kMedRadTrip) {
-                            vec2 e[kMedRadTrip], ab[kMedRadTrip];
-#pragma unroll
-                            for (int u = 0; u < kMedRadTrip; ++u) {
-                                const int at = min(obase + q0 + u * 4 + rslot, kRadCap - 1);
-                                e[u] = S.rad[at];
-                                if constexpr (kJvp) ab[u] = S.jvp.rad_ab[at];
-                            }
-#pragma unroll
-                            for (int u = 0; u < kMedRadTrip; ++u) {
-                                const T dd = e[u].x - L.rrs;
-                                // forward: exp(-eta d^2) f_C; derivative: exp(-eta d^2) (f_C' - 2 eta d f_C) dr
-                                T v = Fast<T>::gauss(static_cast<T>(kR_eta_f), dd);
-                                if constexpr (kJvp) v *= fma(ab[u].y, dd, ab[u].x);
-                                else v *= e[u].y;
-                                acc_r += (q0 + u * 4 + rslot < cnt_a) ? v : T(0);   // entries of other types: select
-                            }
-                        }
+                        T acc_r = acc[a];
                         acc_r += __shfl_xor(acc_r, 16, 64);
                         acc_r += __shfl_xor(acc_r, 32, 64);
                         if (rslot == 0) store_global(row + a * kNumRRs + (lane & 15), acc_r);
-                        obase += cnt_a;
                     }
                 }
                 wave_lds_fence();

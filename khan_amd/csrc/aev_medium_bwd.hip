@@ -306,13 +306,30 @@ void aev_bwd_medium_kernel(
                         qn += popc64(mRb);
                         if (qn >= 64) radial_work_off_full();
                     };
-                    for (int jt = 0; jt < n; jt += 256) {          // four chunks' loads in flight at a time
-                        vec4 at[4];
+                    // 64 chunks' boxes are tested against the centre at a time (one per lane); the chunks that reach into
+                    // the radial cutoff are scanned, four chunks' loads in flight at a time
+                    const float cx = static_cast<float>(ai.x), cy = static_cast<float>(ai.y), cz = static_cast<float>(ai.z);
+                    const int n_chunks = (n + 63) >> 6;
+                    const float4* const boxes = sorted.box + 2 * chunk_base(off, mol);
+                    for (int ch0 = 0; ch0 < n_chunks; ch0 += 64) {
+                        unsigned long long near = wave_ballot(chunk_in_reach(boxes, ch0 + lane, n_chunks, cx, cy, cz));
+                        while (near) {
+                            int ch[4];
 #pragma unroll
-                        for (int u = 0; u < 4; ++u) at[u] = atom_at(min(jt + u * 64 + lane, n - 1));
+                            for (int u = 0; u < 4; ++u) {
+                                ch[u] = -1;
+                                if (near) {
+                                    ch[u] = ch0 + lowest_bit(near);
+                                    near &= near - 1;
+                                }
+                            }
+                            vec4 at[4];
 #pragma unroll
-                        for (int u = 0; u < 4; ++u)
-                            if (jt + u * 64 < n) scan_chunk(jt + u * 64, at[u]);
+                            for (int u = 0; u < 4; ++u) at[u] = atom_at(min(max(ch[u], 0) * 64 + lane, n - 1));
+#pragma unroll
+                            for (int u = 0; u < 4; ++u)
+                                if (ch[u] >= 0) scan_chunk(ch[u] * 64, at[u]);
+                        }
                     }
                     scanned = c;
                     too_many = m_c > 64;

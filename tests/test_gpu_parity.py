@@ -698,6 +698,12 @@ def test_molecules_of_more_than_256_atoms(ops):
         mols.append((rng.choice(4, n, p=[0.5, 0.3, 0.1, 0.1]), _sparse_box(rng, n, 0.1, 0.9)))
     mols.append((rng.integers(0, 4, 420), _packed_ball(rng, 420, 5.0, 0.85)))
     mols.append((np.full(300, 2), _sparse_box(rng, 300, 0.1, 0.9)))
+    # denser: most centres have more than 64 radial partners (their lists are worked off in pieces), few more than 32 angular
+    dense = _sparse_box(rng, 500, 0.17, 0.9)
+    dd = np.linalg.norm(dense[:, None] - dense[None], axis=2)
+    crowd_r, crowd_a = ((dd < 4.6) & (dd > 0)).sum(axis=1), ((dd < 3.1) & (dd > 0)).sum(axis=1)
+    assert int(((crowd_r > 64) & (crowd_a <= 32)).sum()) >= 20, (np.sort(crowd_r)[-30:], np.sort(crowd_a)[-30:])
+    mols.append((rng.choice(4, 500, p=[0.5, 0.3, 0.1, 0.1]), dense))
     box = datagen.make_batch("boxes", 1)
     mols.append((box.A, np.stack([box.X, box.Y, box.Z], axis=1)))
     mols = [mols[i] for i in rng.permutation(len(mols))]
