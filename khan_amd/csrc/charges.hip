@@ -12,9 +12,10 @@
 // partners j for molecules of up to 16 atoms, 2 x 32 up to 32, 1 x 64 above -- with the partners' data
 // held in the lanes, and the sums over j are in-wave DPP reductions (a lane per atom i walking all j
 // would leave four fifths of the lanes idle on a 12-atom molecule).  Molecules of 65 to 256 atoms go to a
-// second kernel that tiles the molecule through LDS (charge_tile_kernel below).  Above 256 atoms a lane takes
-// the atoms i = lane, lane + 64, ... and walks all partners j, whose loads are wave-uniform.  Each output
-// element is written once: no atomics and no pre-zeroing.
+// second kernel that tiles the molecule through LDS (charge_tile_kernel below).  Above 256 atoms several
+// workgroups share a molecule: all pairs, the partners tiled through LDS (charge_large_kernel).  Each output
+// element is written once, no atomics and no pre-zeroing -- except the energy of a molecule of more than 256 atoms,
+// which is the sum of its workgroups' shares.
 #include "aev_small_common.h"
 
 namespace khan {
@@ -70,21 +71,8 @@ __global__ __launch_bounds__(256) void charge_energy_kernel(
         if (lane == 0) E[mol] = acc;
         return;
     }
-    for (int i0 = 0; i0 < n; i0 += 64) {
-        const int i = i0 + lane;
-        const bool active = i < n;
-        const T xi = active ? X[off + i] : T(0), yi = active ? Y[off + i] : T(0),
-                zi = active ? Z[off + i] : T(0), qi = active ? Q[off + i] : T(0);
-        for (int j = i0 + 1; j < n; ++j) {
-            if (active && j > i) {
-                T u, du;
-                pair_terms<T, kDamped>(xi - X[off + j], yi - Y[off + j], zi - Z[off + j], pi_rc, rc, u, du);
-                acc += K * qi * Q[off + j] * u;
-            }
-        }
-    }
-    acc = wave_sum(acc);
-    if (lane == 0) E[mol] = acc;
+    // more than 256 atoms: charge_large_kernel adds its workgroups' shares to the energy, which starts from zero here
+    if (lane == 0) E[mol] = T(0);
 }
 
 template <typename T, bool kDamped>
@@ -133,30 +121,8 @@ __global__ __launch_bounds__(256) void charge_grad_kernel(
         }
         return;
     }
-    for (int i = lane; i < n; i += 64) {
-        const T xi = X[off + i], yi = Y[off + i], zi = Z[off + i], qi = Q[off + i];
-        T dq = T(0), fx = T(0), fy = T(0), fz = T(0);
-        for (int j = 0; j < n; ++j) {
-            if (j == i) continue;
-            const T dx = xi - X[off + j], dy = yi - Y[off + j], dz = zi - Z[off + j];
-            T u, du;
-            pair_terms<T, kDamped>(dx, dy, dz, pi_rc, rc, u, du);
-            const T qj = Q[off + j];
-            dq += qj * u;
-            const T w = qj * du;
-            fx += w * dx;
-            fy += w * dy;
-            fz += w * dz;
-        }
-        if (q_grads) q_grads[off + i] = gK * dq;
-        if (gX) {
-            gX[off + i] = gK * qi * fx;
-            gY[off + i] = gK * qi * fy;
-            gZ[off + i] = gK * qi * fz;
-        }
-    }
+    // more than 256 atoms: charge_large_kernel's
 }
-
 
 // Molecules of 65 to 256 atoms: one wavefront per molecule, the molecule (x, y, z, q) tiled through LDS.
 // A lane owns the atoms i = lane, lane + 64, ... (at most four).  In round d it pairs each of them with atom
@@ -262,6 +228,85 @@ __global__ __launch_bounds__(64) void charge_tile_kernel(
     }
 }
 
+// Molecules of more than 256 atoms: all pairs, the partners tiled through LDS 256 at a time.  A thread owns one atom i
+// of a block of 256 and sums over every partner j (each pair is evaluated from both ends: no exchange between threads, and
+// every per-atom output is written once, by its owner); the workgroups of a grid column (blockIdx.y) share a molecule's
+// blocks.  The energy is half the sum over atoms of q_i times the atom's sum, added to E[mol] (zeroed by
+// charge_energy_kernel, which runs before on the same stream) by one floating-point atomic per workgroup and block: its
+// last bits depend on the order of those additions.
+template <typename T, bool kDamped, bool kGrad>
+__global__ __launch_bounds__(256) void charge_large_kernel(
+    const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
+    const T* __restrict__ Q, const int32_t* __restrict__ MOs, const int32_t* __restrict__ MACs,
+    int32_t n_mols, const T* __restrict__ grads, T K, T* __restrict__ E, T* __restrict__ q_grads,
+    T* __restrict__ gX, T* __restrict__ gY, T* __restrict__ gZ)
+{
+    typedef typename Fast<T>::vec4 vec4;
+    __shared__ vec4 tile[256];
+    __shared__ T wpart[4];
+    __shared__ unsigned long long want[4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const T rc = static_cast<T>(kR_Rc_f), pi_rc = static_cast<T>(kPi / static_cast<double>(kR_Rc_f));
+    for_each_molecule_in_range(MACs, n_mols, kMediumMaxAtoms + 1, INT32_MAX, want, nullptr, nullptr, [&](int mol) {
+        const int n = uniform(MACs[mol]);
+        const int off = uniform(MOs[mol]);
+        for (int i0 = static_cast<int>(blockIdx.y) * 256; i0 < n; i0 += static_cast<int>(gridDim.y) * 256) {
+            const int i = i0 + tid;
+            const bool have = i < n;
+            const T xi = have ? X[off + i] : T(0), yi = have ? Y[off + i] : T(0), zi = have ? Z[off + i] : T(0),
+                    qi = have ? Q[off + i] : T(0);
+            T su = T(0), fx = T(0), fy = T(0), fz = T(0);      // sums over j of q_j u and of q_j du (x_i - x_j)
+            for (int j0 = 0; j0 < n; j0 += 256) {
+                __syncthreads();                               // the previous tile has been used
+                const int j = j0 + tid;
+                // (places beyond the molecule: charge zero)
+                tile[tid] = j < n ? Fast<T>::make4(X[off + j], Y[off + j], Z[off + j], Q[off + j])
+                                  : Fast<T>::make4(T(0), T(0), T(0), T(0));
+                __syncthreads();
+                const int cnt = min(256, n - j0);
+#pragma unroll 4
+                for (int t = 0; t < cnt; ++t) {
+                    const vec4 aj = tile[t];                   // the same address in every lane
+                    const T dx = xi - aj.x, dy = yi - aj.y, dz = zi - aj.z;
+                    T u, du;
+                    pair_terms<T, kDamped>(dx, dy, dz, pi_rc, rc, u, du);      // zero for the atom itself (r = 0)
+                    su = fma(aj.w, u, su);
+                    if constexpr (kGrad) {
+                        const T w = aj.w * du;
+                        fx = fma(w, dx, fx);
+                        fy = fma(w, dy, fy);
+                        fz = fma(w, dz, fz);
+                    }
+                }
+            }
+            if constexpr (!kGrad) {
+                const T part = wave_sum(have ? qi * su : T(0));
+                __syncthreads();                               // wpart is free
+                if (lane == 0) wpart[wave] = part;
+                __syncthreads();
+                if (tid == 0) atomicAdd(&E[mol], T(0.5) * K * (wpart[0] + wpart[1] + wpart[2] + wpart[3]));
+            } else if (have) {
+                const T gK = grads[mol] * K;
+                if (q_grads) q_grads[off + i] = gK * su;
+                if (gX) {
+                    gX[off + i] = gK * qi * fx;
+                    gY[off + i] = gK * qi * fy;
+                    gZ[off + i] = gK * qi * fz;
+                }
+            }
+        }
+        __syncthreads();
+    });
+}
+
+// grid of charge_large_kernel: x = molecules in flight, y = workgroups that share a molecule's blocks of 256 atoms
+static dim3 charge_large_grid(int32_t n_mols)
+{
+    const unsigned columns = static_cast<unsigned>(n_mols < 256 ? n_mols : 256);
+    const unsigned parts = columns >= 256 ? 4u : (1024u / columns > 256u ? 256u : 1024u / columns);
+    return dim3(columns, parts);
+}
+
 }  // namespace
 
 template <typename T>
@@ -276,10 +321,14 @@ hipError_t launch_charge_energy(const T* X, const T* Y, const T* Z, const T* Q, 
         charge_energy_kernel<T, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, K, E);
         charge_tile_kernel<T, true, false><<<dim3(tile_blocks), dim3(64), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, nullptr, K, E,
                                                                                    nullptr, nullptr, nullptr, nullptr);
+        charge_large_kernel<T, true, false><<<charge_large_grid(n_mols), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, nullptr, K,
+                                                                                             E, nullptr, nullptr, nullptr, nullptr);
     } else {
         charge_energy_kernel<T, false><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, K, E);
         charge_tile_kernel<T, false, false><<<dim3(tile_blocks), dim3(64), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, nullptr, K, E,
                                                                                     nullptr, nullptr, nullptr, nullptr);
+        charge_large_kernel<T, false, false><<<charge_large_grid(n_mols), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, nullptr, K,
+                                                                                              E, nullptr, nullptr, nullptr, nullptr);
     }
     return hipGetLastError();
 }
@@ -296,10 +345,14 @@ hipError_t launch_charge_grad(const T* X, const T* Y, const T* Z, const T* Q, co
         charge_grad_kernel<T, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, q_grads, gX, gY, gZ);
         charge_tile_kernel<T, true, true><<<dim3(tile_blocks), dim3(64), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, nullptr,
                                                                                   q_grads, gX, gY, gZ);
+        charge_large_kernel<T, true, true><<<charge_large_grid(n_mols), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K,
+                                                                                            nullptr, q_grads, gX, gY, gZ);
     } else {
         charge_grad_kernel<T, false><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, q_grads, gX, gY, gZ);
         charge_tile_kernel<T, false, true><<<dim3(tile_blocks), dim3(64), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, nullptr,
                                                                                    q_grads, gX, gY, gZ);
+        charge_large_kernel<T, false, true><<<charge_large_grid(n_mols), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K,
+                                                                                             nullptr, q_grads, gX, gY, gZ);
     }
     return hipGetLastError();
 }

@@ -292,6 +292,11 @@ def test_size_class_boundaries(ops):
     c = _boundary_case()
     check_forward_backward(ops, c)
     _check_grad_inverse(ops, c)
+    _check_charges(ops, c)
+
+
+def _check_charges(ops, c):
+    """charge energies, dE/dq and dE/dxyz of a case in both precisions against the float64 oracle"""
     q = np.random.default_rng(3).normal(0.0, 0.3, c.N)
     gm = np.random.default_rng(4).standard_normal(c.n_mols)
     E64 = ob.ani_charge(c.X, c.Y, c.Z, q, c.MOs, c.MACs, dtype=np.float64)
@@ -716,6 +721,7 @@ def test_molecules_of_more_than_256_atoms(ops):
     c = Case(xyz[:, 0], xyz[:, 1], xyz[:, 2], A, mi, len(mols))
     check_forward_backward(ops, c)
     _check_grad_inverse(ops, c)
+    _check_charges(ops, c)
 
 
 def test_radial_lists_at_their_fullest(ops):
