@@ -724,6 +724,44 @@ def test_molecules_of_more_than_256_atoms(ops):
     _check_charges(ops, c)
 
 
+def _jittered_lattice(rng, n, spacing, jitter, shape=None):
+    """n points on a cubic lattice (or one of the given shape), each moved by up to `jitter` along every axis"""
+    if shape is None:
+        k = int(np.ceil(n ** (1 / 3)))
+        shape = (k, k, k)
+    grid = np.stack(np.meshgrid(*[np.arange(d) for d in shape], indexing="ij"), axis=-1).reshape(-1, 3).astype(np.float64)
+    pick = rng.permutation(len(grid))[:n]
+    return grid[pick] * spacing + rng.uniform(-jitter, jitter, (n, 3))
+
+
+def test_large_molecules_in_every_regime_of_their_sort(ops):
+    # The kernel that sorts the atoms of a molecule of more than 256 atoms takes 4, 8 or 16 cells per dimension by the
+    # molecule's size and ranks the atoms of a step in one of two ways; a chunk of 64 sorted atoms may be full, nearly
+    # empty, or span two types.  Shapes: 9,000 atoms (16 cells, few atoms share a bin within a step), 1,025 (8 cells), 320
+    # (five full chunks) and 321, a flat sheet and a chain (no extent along one or two axes), in input orders that are
+    # not spatial.  Features, gradients, Jacobian-vector product and charges against the oracle.
+    say("case: large molecules: 9,000 / 1,025 / 320 / 321 atoms, a sheet, a chain")
+    rng = np.random.default_rng(57)
+    types = lambda n: rng.choice(4, n, p=[0.5, 0.3, 0.1, 0.1])
+    mols = [(types(9000), _jittered_lattice(rng, 9000, 2.15, 0.5)),
+            (types(1025), _jittered_lattice(rng, 1025, 2.15, 0.5)),
+            (types(320), _jittered_lattice(rng, 320, 2.15, 0.5)),
+            (np.full(321, 1), _jittered_lattice(rng, 321, 2.15, 0.5)),
+            (types(400), _jittered_lattice(rng, 400, 1.6, 0.3, shape=(20, 20, 1))),
+            (types(300), _jittered_lattice(rng, 300, 1.3, 0.25, shape=(300, 1, 1)))]
+    small = datagen.make_batch("organic", 2, first_mol=21)
+    for m in range(2):
+        sl = slice(small.MOs[m], small.MOs[m] + small.MACs[m])
+        mols.insert(2 * m + 1, (small.A[sl], np.stack([small.X[sl], small.Y[sl], small.Z[sl]], axis=1)))
+    A = np.concatenate([m[0] for m in mols]).astype(np.int32)
+    xyz = np.concatenate([m[1] for m in mols]).astype(np.float32).astype(np.float64)
+    mi = np.concatenate([np.full(len(m[0]), k) for k, m in enumerate(mols)]).astype(np.int32)
+    c = Case(xyz[:, 0], xyz[:, 1], xyz[:, 2], A, mi, len(mols))
+    check_forward_backward(ops, c)
+    _check_grad_inverse(ops, c)
+    _check_charges(ops, c)
+
+
 def test_radial_lists_at_their_fullest(ops):
     # The one-wavefront forward kernel gives every partner type a place of its own in a centre's radial list, each
     # rounded up to a whole trip of the walk.  Fullest lists: molecules of exactly 16, 32 and 64 atoms (the three scan
