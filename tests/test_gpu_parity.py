@@ -762,6 +762,33 @@ def test_large_molecules_in_every_regime_of_their_sort(ops):
     _check_charges(ops, c)
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_large_molecules(ops, seed):
+    # batches of one to four molecules of up to 3,000 atoms, most of them above 256: cubes, slabs and rods at densities
+    # of 0.02 to 0.16 atoms per cubic Angstrom, even or skewed type mixes, in an input order that is not spatial
+    say("case: random large molecules, seed %d" % seed)
+    rng = np.random.default_rng(seed)
+    for _ in range(4):
+        mols = []
+        for _m in range(int(rng.integers(1, 5))):
+            n = int(rng.choice([rng.integers(257, 400), rng.integers(400, 1100), rng.integers(1100, 3000), rng.integers(1, 200)]))
+            side = (n / float(rng.uniform(0.02, 0.16))) ** (1 / 3)
+            ext = np.array({"cube": (side, side, side), "slab": (2 * side, 2 * side, side / 4),
+                            "rod": (4 * side, side / 2, side / 2)}[str(rng.choice(["cube", "slab", "rod"]))])
+            k = np.maximum(np.ceil(ext / 1.9).astype(int), 1)
+            while np.prod(k) < n:
+                k += 1
+            cell = ext / k
+            grid = np.stack(np.meshgrid(*[np.arange(d) for d in k], indexing="ij"), -1).reshape(-1, 3)
+            pos = grid[rng.permutation(len(grid))[:n]] * cell + rng.uniform(-0.4, 0.4, (n, 3)) * np.minimum(cell, 1.9) / 1.9
+            mols.append((rng.choice(4, n, p=rng.dirichlet(np.ones(4) * rng.choice([0.3, 3.0]))), pos))
+        A = np.concatenate([m[0] for m in mols]).astype(np.int32)
+        xyz = np.concatenate([m[1] for m in mols]).astype(np.float32).astype(np.float64)
+        mi = np.concatenate([np.full(len(m[0]), k) for k, m in enumerate(mols)]).astype(np.int32)
+        say("   sizes %s" % [len(m[0]) for m in mols])
+        check_forward_backward(ops, Case(xyz[:, 0], xyz[:, 1], xyz[:, 2], A, mi, len(mols)))
+
+
 def test_radial_lists_at_their_fullest(ops):
     # The one-wavefront forward kernel gives every partner type a place of its own in a centre's radial list, each
     # rounded up to a whole trip of the walk.  Fullest lists: molecules of exactly 16, 32 and 64 atoms (the three scan
