@@ -3,10 +3,10 @@
 //
 // Up to 256 atoms a workgroup sorts its molecule into LDS itself.  Above that the sorted atoms live in device
 // memory (a molecule of a few thousand atoms stays in L2), written once per call by large_sort_kernel, and several
-// workgroups share a molecule's centres.  The atoms are sorted by type and, inside a type, along a space-filling
-// curve, and every 64 consecutive ones have a box around them: a centre scans only the chunks whose box reaches into
-// its cutoff.  The partner lists, the segment tables and the angular phases are those of the smaller molecules; only
-// where an atom is read from differs.
+// workgroups share a molecule's centres.  The atoms are sorted along a space-filling curve (by type inside a cell),
+// and every 64 consecutive ones have a box around them: a centre scans only the chunks whose box reaches into its
+// cutoff, and puts the partners it finds in order of type afterwards.  The partner lists, the segment tables and the
+// angular phases are those of the smaller molecules; only where an atom is read from differs.
 #pragma once
 #include "aev_small_common.h"
 #include "khan_params.h"
@@ -18,12 +18,11 @@ struct SortedAtoms {
     typename Fast<T>::vec4* atom;   // x, y, z, type of the atom at MOs[mol] + sorted position
     typename Fast<T>::vec4* vel;    // its incoming vector (Jacobian-vector product only), else null
     int2* aux;                      // its index inside the molecule, and its scatter index (row inside its type's bucket)
-    int4* tbase;                    // per molecule: sorted position of the first atom of each type
     float4* box;                    // per chunk of 64 sorted atoms: lowest x, y, z and highest x, y, z (two entries)
 };
 
-// Inside a type the atoms are ordered along a space-filling curve (16 x 16 x 16 cells over the molecule's extent, Morton
-// order), so that 64 consecutive atoms sit close together and a centre can skip the chunks whose box lies beyond its
+// The atoms are ordered along a space-filling curve (up to 16 x 16 x 16 cells over the molecule's extent, Morton order;
+// by type inside a cell), so that 64 consecutive atoms sit close together and a centre can skip the chunks whose box lies beyond its
 // cutoff.  The boxes of molecule `mol` (atoms from offset `off`) start at entry 2 * chunk_base(off, mol).
 __host__ __device__ __forceinline__ size_t chunk_base(int off, int mol) { return static_cast<size_t>(off >> 6) + static_cast<size_t>(mol); }
 constexpr int kSortCellsPerDim = 16;
@@ -36,7 +35,6 @@ __host__ inline size_t sorted_atoms_bytes(int64_t n_atoms, int32_t n_mols, bool 
 {
     const size_t vec = round_up_256(sizeof(typename Fast<T>::vec4) * static_cast<size_t>(n_atoms));
     return vec * (with_vel ? 2 : 1) + round_up_256(sizeof(int2) * static_cast<size_t>(n_atoms)) +
-           round_up_256(sizeof(int4) * static_cast<size_t>(n_mols)) +
            round_up_256(2 * sizeof(float4) * (static_cast<size_t>(n_atoms) / 64 + static_cast<size_t>(n_mols) + 1));
 }
 
@@ -57,8 +55,6 @@ __host__ inline SortedAtoms<T> carve_sorted_atoms(void* scratch, int64_t n_atoms
     }
     s.aux = reinterpret_cast<int2*>(p);
     p += round_up_256(sizeof(int2) * static_cast<size_t>(n_atoms));
-    s.tbase = reinterpret_cast<int4*>(p);
-    p += round_up_256(sizeof(int4) * static_cast<size_t>(n_mols));
     s.box = reinterpret_cast<float4*>(p);
     return s;
 }

@@ -1,5 +1,5 @@
 // Sorted copies of the molecules of more than 256 atoms, for the workgroup-per-molecule AEV kernels (aev_large.h).
-// One workgroup per molecule: a counting sort by (atom type, cell along a space-filling curve) that keeps the atoms'
+// One workgroup per molecule: a counting sort by (cell along a space-filling curve, atom type) that keeps the atoms'
 // order inside a bin, 256 atoms per step, and the box around every 64 consecutive sorted atoms.
 #include "aev_large.h"
 #include "khan_params.h"
@@ -33,8 +33,8 @@ __global__ __launch_bounds__(256) void large_sort_kernel(
     T* __restrict__ gX, T* __restrict__ gY, T* __restrict__ gZ, const int32_t* __restrict__ order,
     SortedAtoms<T> sorted)
 {
-    __shared__ int hist[4 * kSortCells];       // atoms per (type, cell); after the scan each one's next free sorted position
-    __shared__ int in_step[4 * kSortCells];    // atoms per (type, cell) among the 256 of the current step (zero between steps)
+    __shared__ int hist[4 * kSortCells];       // atoms per (cell, type); after the scan each one's next free sorted position
+    __shared__ int in_step[4 * kSortCells];    // atoms per (cell, type) among the 256 of the current step (zero between steps)
     __shared__ int2 shared_bin[256];           // (key, thread) of the step's atoms that share their bin with another
     __shared__ int wshared[4];                 // how many of them each wavefront holds
     __shared__ int step_key[256];              // keys of the 256 atoms of the current step
@@ -84,16 +84,16 @@ __global__ __launch_bounds__(256) void large_sort_kernel(
             hi[k] = fmaxf(fmaxf(ext[0][3 + k], ext[1][3 + k]), fmaxf(ext[2][3 + k], ext[3][3 + k]));
             scale[k] = static_cast<float>(g) / fmaxf(hi[k] - lo[k], 1.0e-3f);
         }
-        // (type, cell) of atom j: the cell's index along the space-filling curve
+        // (cell, type) of atom j: the cell's index along the space-filling curve, then the type
         auto key_of = [&](int j) -> int {
             const float p[3] = {static_cast<float>(X[off + j]), static_cast<float>(Y[off + j]), static_cast<float>(Z[off + j])};
             int c[3];
 #pragma unroll
             for (int k = 0; k < 3; ++k) c[k] = min(max(static_cast<int>((p[k] - lo[k]) * scale[k]), 0), g - 1);
-            return fold_type(A[off + j]) * cells + (spread4(c[0]) | (spread4(c[1]) << 1) | (spread4(c[2]) << 2));
+            return (spread4(c[0]) | (spread4(c[1]) << 1) | (spread4(c[2]) << 2)) * 4 + fold_type(A[off + j]);
         };
 
-        // ---- atoms per (type, cell)
+        // ---- atoms per (cell, type)
         for (int b = tid; b < bins; b += 256) {
             hist[b] = 0;
             in_step[b] = 0;
@@ -123,9 +123,8 @@ __global__ __launch_bounds__(256) void large_sort_kernel(
             }
         }
         __syncthreads();
-        if (tid == 0) sorted.tbase[mol] = make_int4(hist[0], hist[cells], hist[2 * cells], hist[3 * cells]);
 
-        // ---- place the atoms, 256 per step, in index order inside a (type, cell): the result does not depend on timing.
+        // ---- place the atoms, 256 per step, in index order inside a (cell, type): the result does not depend on timing.
         // An atom's data are fetched one step ahead, so that the loads run under the previous step's ranking.
         struct Fetched {
             T x, y, z, vx, vy, vz;
@@ -162,7 +161,7 @@ __global__ __launch_bounds__(256) void large_sort_kernel(
                 int c[3];
 #pragma unroll
                 for (int k = 0; k < 3; ++k) c[k] = min(max(static_cast<int>((p[k] - lo[k]) * scale[k]), 0), g - 1);
-                key = cur.type * cells + (spread4(c[0]) | (spread4(c[1]) << 1) | (spread4(c[2]) << 2));
+                key = (spread4(c[0]) | (spread4(c[1]) << 1) | (spread4(c[2]) << 2)) * 4 + cur.type;
             }
             // Rank among the step's atoms of the same bin, by thread.  In a large molecule most atoms are alone in their
             // bin within a step: the atoms that are not are listed (in thread order) and only they compare keys, with

@@ -43,6 +43,10 @@ struct __align__(16) MedShared {
 template <typename T, bool kJvp>
 struct __align__(16) MedShared<T, kJvp, true> {
     unsigned long long row[4][8];
+    // partner types of the entries of each wavefront's radial list and of the angular list it is building (used by the
+    // Jacobian-vector product, whose list entries have no room for the type)
+    unsigned char rtype[4][kRadCap];
+    unsigned char atype[4][kCapA];
 };
 
 // With kJvp the kernel computes the Jacobian-vector product instead (featurize_grad_inverse), as the
@@ -212,29 +216,37 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                     }
                 };
                 // Large molecules: a centre's radial list is worked off whenever the next chunk's entries would not fit
-                // (no limit on the number of radial partners); racc collects the sums, cRdone the counts at the last time.
+                // (no limit on the number of radial partners); racc collects the sums.
                 T racc[4] = {T(0), T(0), T(0), T(0)};
-                int cRdone[4] = {0, 0, 0, 0};
                 auto radial_flush = [&](int count) {
                     wave_lds_fence();
-                    int cnt[4];
-                    if constexpr (kJvp) {
-#pragma unroll
-                        for (int a = 0; a < 4; ++a) {
-                            cnt[a] = cR[a] - cRdone[a];
-                            cRdone[a] = cR[a];
-                        }
-                    } else {
-                        int tR = -1;
-                        if (lane < count) {
-                            const vec2 e = S.rad[lane];
-                            tR = static_cast<int>(e.y);
-                            S.rad[lane] = Fast<T>::make2(e.x, Fast<T>::cutoff(e.x, static_cast<T>(kR_Rc_f)));
-                        }
-#pragma unroll
-                        for (int a = 0; a < 4; ++a) cnt[a] = popc64(wave_ballot(tR == a));
-                        wave_lds_fence();
+                    // the entries arrive in the order of the sorted atoms (by cell): put them in order of type
+                    int tR = -1;
+                    vec2 e = Fast<T>::make2(T(0), T(0)), ab = Fast<T>::make2(T(0), T(0));
+                    if (lane < count) {
+                        e = S.rad[lane];
+                        if constexpr (kJvp) ab = S.jvp.rad_ab[lane];
+                        if constexpr (kJvp && kLarge) tR = M.rtype[wave][lane];
+                        else tR = static_cast<int>(e.y);
                     }
+                    int cnt[4], dest = 0, before = 0;
+#pragma unroll
+                    for (int a = 0; a < 4; ++a) {
+                        const unsigned long long ma = wave_ballot(tR == a);
+                        cnt[a] = popc64(ma);
+                        if (tR == a) dest = before + popc64(ma & lt_mask);
+                        before += cnt[a];
+                    }
+                    wave_lds_fence();               // every entry has been read
+                    if (lane < count) {
+                        if constexpr (kJvp) {
+                            S.rad[dest] = e;
+                            S.jvp.rad_ab[dest] = ab;
+                        } else {
+                            S.rad[dest] = Fast<T>::make2(e.x, Fast<T>::cutoff(e.x, static_cast<T>(kR_Rc_f)));
+                        }
+                    }
+                    wave_lds_fence();
                     radial_sums(racc, cnt);
                     wave_lds_fence();               // the list may be overwritten
                 };
@@ -273,6 +285,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                                 Fast<T>::cutoff_grad(r, static_cast<T>(kR_Rc_f), fc, dfc);
                                 S.rad[p] = Fast<T>::make2(r, fc);
                                 S.jvp.rad_ab[p] = Fast<T>::make2(dfc * rd, T(-2) * static_cast<T>(kR_eta_f) * fc * rd);
+                                if constexpr (kLarge) M.rtype[wave][p] = static_cast<unsigned char>(tj);
                             }
                         }
                         if (inA) {
@@ -284,6 +297,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                                 S.nbr_fc[b][p] = fc;
                                 S.jvp.nbr_p[b][p] = Fast<T>::make4(wx * inv, wy * inv, wz * inv, rd * inv);
                                 S.jvp.nbr_d[b][p] = Fast<T>::make2(dfc * rd, rd);
+                                if constexpr (kLarge) M.atype[wave][p] = static_cast<unsigned char>(tj);
                             }
                         }
                     } else {
@@ -341,7 +355,42 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                         scan_chunk(jc, atom_at(jj), vel_at(jj));
                     }
                 }
-                if constexpr (kLarge) radial_flush(posR);
+                if constexpr (kLarge) {
+                    radial_flush(posR);
+                    // the angular list too arrives in the order of the sorted atoms: put it in order of type
+                    const bool haveE = lane < min(posA, kCapA);
+                    int tA = -1;
+                    vec4 nb = Fast<T>::make4(T(0), T(0), T(0), T(0)), np = nb;
+                    vec2 nd = Fast<T>::make2(T(0), T(0));
+                    T fc = T(0);
+                    if (haveE) {
+                        nb = S.nbr[b][lane];
+                        fc = S.nbr_fc[b][lane];
+                        if constexpr (kJvp) {
+                            np = S.jvp.nbr_p[b][lane];
+                            nd = S.jvp.nbr_d[b][lane];
+                            tA = M.atype[wave][lane];
+                        } else {
+                            tA = static_cast<int>(fc);
+                        }
+                    }
+                    int dest = 0, before = 0;
+#pragma unroll
+                    for (int a = 0; a < 4; ++a) {
+                        const unsigned long long ma = wave_ballot(tA == a);
+                        if (tA == a) dest = before + popc64(ma & lt_mask);
+                        before += popc64(ma);
+                    }
+                    wave_lds_fence();               // every entry has been read
+                    if (haveE) {
+                        S.nbr[b][dest] = nb;
+                        S.nbr_fc[b][dest] = fc;
+                        if constexpr (kJvp) {
+                            S.jvp.nbr_p[b][dest] = np;
+                            S.jvp.nbr_d[b][dest] = nd;
+                        }
+                    }
+                }
                 if constexpr (!kJvp) {
                     wave_lds_fence();
                     const bool haveR = !kLarge && lane < min(posR, kRadCap), haveA = lane < min(posA, kCapA);

@@ -28,6 +28,7 @@ namespace khan {
 namespace {
 
 constexpr int kChunks = kMediumMaxAtoms / 64;
+constexpr int kTypeShift = 28;     // large molecules: a radial queue entry is a sorted position with the atom's type above it
 // centres per batch: four, so that the pools of the four wavefronts leave room for four workgroups on a CU in float
 // (LDS 39.6 KB; 128 registers) and two in double (76 KB; 256 registers) -- the shorter batches fill fewer lanes, the
 // additional wavefronts per SIMD hide more (dense boxes: float 4 % faster than six-centre batches at three workgroups,
@@ -84,10 +85,7 @@ void aev_bwd_medium_kernel(
 
         // ------------------------------------------------------------ load, sort by type into LDS, zero outputs
         if constexpr (kLarge) {
-            const int4 tb = sorted.tbase[mol];
-            tb1 = uniform(tb.y);
-            tb2 = uniform(tb.z);
-            tb3 = uniform(tb.w);
+            tb1 = tb2 = tb3 = 0;               // (the sorted atoms are not in order of type: types come with the atoms)
             if (tid == 0) M.next = 0;
             __syncthreads();
         } else {
@@ -140,9 +138,8 @@ void aev_bwd_medium_kernel(
             if constexpr (kLarge) return sorted.atom[off + sorted_idx];
             else return M.atom[sorted_idx];
         };
-        auto row_bits_of = [&](int sorted_idx) -> unsigned long long {     // per-lane index
+        auto row_bits_of = [&](int sorted_idx, int type) -> unsigned long long {     // per-lane index, and that atom's type
             if constexpr (kLarge) {
-                const int type = type_of(sorted_idx);
                 const T* const bucket = type == 0 ? gin.p[0] : type == 1 ? gin.p[1] : type == 2 ? gin.p[2] : gin.p[3];
                 return reinterpret_cast<unsigned long long>(bucket + static_cast<size_t>(sorted.aux[off + sorted_idx].y) * kFeats);
             } else {
@@ -150,7 +147,9 @@ void aev_bwd_medium_kernel(
             }
         };
         auto row_of = [&](int sorted_idx) -> const T* {            // wave-uniform index
-            const unsigned long long bits = row_bits_of(sorted_idx);
+            int type = 0;
+            if constexpr (kLarge) type = static_cast<int>(sorted.atom[off + sorted_idx].w);
+            const unsigned long long bits = row_bits_of(sorted_idx, type);
             const unsigned lo = static_cast<unsigned>(uniform(static_cast<int>(bits & 0xffffffffull)));
             const unsigned hi = static_cast<unsigned>(uniform(static_cast<int>(bits >> 32)));
             return reinterpret_cast<const T*>((static_cast<unsigned long long>(hi) << 32) | lo);
@@ -179,13 +178,23 @@ void aev_bwd_medium_kernel(
             int c = -1;
             if (lane < count) {
                 const vec4 e = q_d[lane];
-                const int j = q_j[lane];
+                int j = q_j[lane];
                 c = q_c[lane];
-                const T* grow_c = reinterpret_cast<const T*>(row_bits_of(c));
-                const T* grow_j = reinterpret_cast<const T*>(row_bits_of(j));
+                int tj, tc;
+                if constexpr (kLarge) {            // the queue carries the types in the four high bits
+                    tj = j >> kTypeShift;
+                    tc = c >> kTypeShift;
+                    j &= (1 << kTypeShift) - 1;
+                    c &= (1 << kTypeShift) - 1;
+                } else {
+                    tj = type_of(j);
+                    tc = type_of(c);
+                }
+                const T* grow_c = reinterpret_cast<const T*>(row_bits_of(c, tc));
+                const T* grow_j = reinterpret_cast<const T*>(row_bits_of(j, tj));
                 const T inv = Fast<T>::rcp(e.w);
                 // the pair's pull on the centre from both rows; the partner gets its share when it is the centre
-                const T sc = bwd_radial_pair_both<T>(grow_c, type_of(j), grow_j, type_of(c), e.w, inv);
+                const T sc = bwd_radial_pair_both<T>(grow_c, tj, grow_j, tc, e.w, inv);
                 fx = sc * e.x;
                 fy = sc * e.y;
                 fz = sc * e.z;
@@ -300,8 +309,8 @@ void aev_bwd_medium_kernel(
                         if ((mRb >> lane) & 1ull) {
                             const int p = qn + popc64(mRb & lt_mask);
                             q_d[p] = Fast<T>::make4(ddx, ddy, ddz, rr);
-                            q_j[p] = static_cast<idx_t>(j);
-                            q_c[p] = static_cast<idx_t>(c);
+                            q_j[p] = static_cast<idx_t>(j | (static_cast<int>(aj.w) << kTypeShift));
+                            q_c[p] = static_cast<idx_t>(c | (static_cast<int>(ai.w) << kTypeShift));
                         }
                         qn += popc64(mRb);
                         if (qn >= 64) radial_work_off_full();

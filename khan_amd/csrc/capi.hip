@@ -141,6 +141,9 @@ private:
     hipStream_t stream_;
 };
 
+// (the kernels for large molecules keep an atom's position inside its molecule in 28 bits)
+constexpr int64_t kLargeAtomLimit = int64_t(1) << 28;
+
 // Which kernels have work.  `classes` (host memory, null = not known: launch everything) holds the number of molecules
 // of up to 32 atoms, of 33..64, of 65..256 and of more, as khan_size_order leaves them behind the order.
 struct SizeClasses {
@@ -181,7 +184,7 @@ int forward_dispatch(const T* xs, const T* ys, const T* zs, const int32_t* as, c
     if (st == KHAN_OK && cls.any(small_max + 1, khan::kMediumMaxAtoms))
         st = hip_status(khan::launch_fwd_medium<T>(xs, ys, zs, as, mos, macs, n_mols, sis, out, small_max + 1, order, stream));
     if (st == KHAN_OK && n_atoms > khan::kMediumMaxAtoms && cls.any(khan::kMediumMaxAtoms + 1, INT32_MAX)) {      // (n_atoms: of the whole batch)
-        const LargeScratch scratch(may_allocate ? khan::large_scratch_bytes<T>(n_atoms, n_mols, false) : 0, stream);
+        const LargeScratch scratch(may_allocate && n_atoms < kLargeAtomLimit ? khan::large_scratch_bytes<T>(n_atoms, n_mols, false) : 0, stream);
         if (scratch.get())
             st = hip_status(khan::launch_fwd_large<T>(xs, ys, zs, as, mos, macs, n_mols, sis, nullptr, nullptr, nullptr, out,
                                                       order, scratch.get(), n_atoms, stream));
@@ -208,7 +211,7 @@ int backward_dispatch(const T* xs, const T* ys, const T* zs, const int32_t* as, 
     const SizeClasses cls(classes_host);
     int st = KHAN_OK;
     if (n_atoms > khan::kMediumMaxAtoms && cls.any(khan::kMediumMaxAtoms + 1, INT32_MAX)) {
-        const LargeScratch scratch(khan::large_scratch_bytes<T>(n_atoms, n_mols, false), stream);
+        const LargeScratch scratch(n_atoms < kLargeAtomLimit ? khan::large_scratch_bytes<T>(n_atoms, n_mols, false) : 0, stream);
         if (scratch.get())
             st = hip_status(khan::launch_bwd_large<T>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz, order,
                                                       scratch.get(), n_atoms, stream));
@@ -339,7 +342,7 @@ int featurize_grad_inverse_impl(const T* xs, const T* ys, const T* zs, const int
                                                    khan::kSmallMaxAtoms + 1, order, as_stream(stream)));
     if (st == KHAN_OK && cls.any(khan::kMediumMaxAtoms + 1, INT32_MAX)) {
         const int64_t n_atoms = static_cast<int64_t>(acs_host[0]) + acs_host[1] + acs_host[2] + acs_host[3];
-        const LargeScratch scratch(n_atoms > khan::kMediumMaxAtoms ? khan::large_scratch_bytes<T>(n_atoms, n_mols, true) : 0,
+        const LargeScratch scratch(n_atoms > khan::kMediumMaxAtoms && n_atoms < kLargeAtomLimit ? khan::large_scratch_bytes<T>(n_atoms, n_mols, true) : 0,
                                    as_stream(stream));
         if (scratch.get())
             st = hip_status(khan::launch_fwd_large<T>(xs, ys, zs, as, mos, macs, n_mols, sis, vx, vy, vz, out, order,
