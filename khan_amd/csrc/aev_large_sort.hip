@@ -216,7 +216,6 @@ __global__ __launch_bounds__(256) void large_sort_kernel(
         __syncthreads();                        // the workgroup's stores to sorted.atom are visible to its loads
         const size_t cb = chunk_base(off, mol);
         const int n_chunks = (n + 63) >> 6;
-#pragma unroll 4
         for (int c = wave; c < n_chunks; c += 4) {
             const int j = 64 * c + lane;
             float p[3] = {0.0f, 0.0f, 0.0f};
