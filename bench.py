@@ -27,7 +27,7 @@ FP32_PEAK_TFLOPS = 157.3       # MI355X vector FP32, published
 FP64_PEAK_TFLOPS = 78.6
 
 # roofline.traffic (HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) comes from the record
-# profiles/hbm_traffic.json through khan_amd.profiling: an entry measured on other kernel sources than the ones in
+# profiles/hbm_traffic.json through bench_profiling: an entry measured on other kernel sources than the ones in
 # the tree is reported as stale (traffic null), never passed on.
 
 # name: (generator, molecules, float width in bytes, charges kernels in the step)
@@ -175,7 +175,7 @@ def inference_bench(args, batch):
     sizes = (384,) + tuple(model.DEFAULT_LAYERS)
     macs_per_atom = sum(x * y for x, y in zip(sizes[:-1], sizes[1:]))
     gemm_flops = 2 * macs_per_atom * N * 2            # forward, and the data gradient on the way back
-    print(json.dumps({
+    return ({
         "metric": "ANI-1 energy + coordinate-gradient inference atoms/sec, fp32, 1 MI355X",
         "value": N / (ms_per_step * 1e-3), "unit": "atoms/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
@@ -193,7 +193,7 @@ def inference_bench(args, batch):
                      "bound": "mfma", "achieved": gemm_flops / (ms_per_step * 1e-3) / 1e12,
                      "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": gemm_flops / (ms_per_step * 1e-3) / 1e12 / FP32_PEAK_TFLOPS, "traffic": None},
-    }))
+    })
 
 
 def grad_inverse_bench(args, batch, w, kind):
@@ -225,8 +225,8 @@ def grad_inverse_bench(args, batch, w, kind):
     ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
     launch_ms = e0.elapsed_time(e1) / args.steps
     nbytes = N * (384 * w + 6 * w + 8) + 8 * n_mols
-    kernel = "aev_fwd_%s_kernel<%s, true, false>" % ("small" if kind == "organic" else "medium", tname)
-    print(json.dumps({
+    kernel = "aev_fwd_%s_kernel<%s, true>" % ("small" if kind == "organic" else "medium", tname)
+    return ({
         "metric": "AEV grad-inverse (Jacobian-vector product) atoms/sec, fp%d, 1 MI355X" % (8 * w),
         "value": N / (ms_per_step * 1e-3), "unit": "atoms/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f%d" % (8 * w),
@@ -235,7 +235,7 @@ def grad_inverse_bench(args, batch, w, kind):
         "roofline": {"kernel": kernel, "bound": "hbm", "achieved": nbytes / (launch_ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (launch_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "traffic": None, "launch_ms": launch_ms, "algorithmic_bytes": nbytes},
-    }))
+    })
 
 
 def charges_bench(args, batch, w):
@@ -273,7 +273,8 @@ def charges_bench(args, batch, w):
     t_g = sum(m[1].elapsed_time(m[2]) for m in marks) / args.steps
     nbytes = N * 8 * w + n_mols * (w + 8)
     peak = FP32_PEAK_TFLOPS if w == 4 else FP64_PEAK_TFLOPS
-    print(json.dumps({
+    tflops = 45.0 * C / ((t_e + t_g) * 1e-3) / 1e12
+    return ({
         "metric": "ani_charge energy + gradients atoms/sec, fp%d, 1 MI355X" % (8 * w),
         "value": N / (ms_per_step * 1e-3), "unit": "atoms/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -281,11 +282,12 @@ def charges_bench(args, batch, w):
         "config": {"workload": "%s: ani_charge + ani_charge_grad_xyz, %d molecules, %d atoms, %d pairs" % (
             args.workload, n_mols, N, C)},
         "molecules_per_s": n_mols / (ms_per_step * 1e-3),
-        "roofline": {"kernel": "charge kernels", "bound": "hbm", "achieved": nbytes / ((t_e + t_g) * 1e-3) / 1e9,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / ((t_e + t_g) * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": None, "energy_ms": t_e, "gradients_ms": t_g, "algorithmic_bytes": nbytes,
-                     "valu_frac": 45.0 * C / ((t_e + t_g) * 1e-3) / 1e12 / peak, "valu_peak_tflops": peak},
-    }))
+        # all pairs of a molecule from a few bytes per atom: the vector ALUs bound these kernels, not HBM
+        "roofline": {"kernel": "charge kernels", "bound": "valu", "achieved": tflops, "peak": peak, "unit": "TFLOP/s",
+                     "frac": tflops / peak, "traffic": None, "energy_ms": t_e, "gradients_ms": t_g,
+                     "algorithmic_flops": 45.0 * C, "algorithmic_bytes": nbytes,
+                     "hbm_frac": nbytes / ((t_e + t_g) * 1e-3) / 1e9 / HBM_PEAK_GBS},
+    })
 
 
 def main():
@@ -295,26 +297,76 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="organic65536", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="with the default workload: leave out the shorter runs of the other configurations "
+                         "(`configs` in the printed line)")
     ap.add_argument("--traffic-probe", choices=("fwd", "bwd"), default=None,
                     help="counter-collection mode: launch that pass twice, then a plain 64 MiB device copy of "
                          "known traffic (scales FETCH_SIZE / WRITE_SIZE), print nothing else and exit")
     ap.add_argument("--phase2", choices=("vector", "matrix"), default="vector",
                     help="matrix: measure the variant of the small-molecule forward kernel that sums the angular "
-                         "records on the matrix cores (sets KHAN_AEV_PHASE2 before the library's first launch)")
+                         "records on the matrix cores (loads the check build of the library, which alone holds it, "
+                         "and sets KHAN_AEV_PHASE2 before its first launch)")
     args = ap.parse_args()
     if args.phase2 == "matrix":
+        from khan_amd import build as _build
+        os.environ["KHAN_AEV_LIBRARY"] = _build.CHECK_LIBRARY
         os.environ["KHAN_AEV_PHASE2"] = "matrix"
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; the path shards by molecule with no exchange, "
                  "but no multi-GPU launch is part of this run (got --gpus %d)" % args.gpus)
 
-    import numpy as np
     import torch
-    from khan_amd import datagen, ops, _lib
+    from khan_amd import datagen, _lib
 
     _lib.load()   # fails loudly if the HIP library is missing
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
+    result = run_workload(args, args.workload, args.steps, args.warmup, cpu=not args.no_cpu_baseline)
+    if result is None:
+        return
+    if args.workload == HEADLINE and not args.headline_only:
+        # the other configurations, each a shorter run of its own step, summarised in the same line
+        steps, warmup = max(10, args.steps // 3), max(5, args.warmup // 2)
+        result["configs"] = {}
+        for name in EXTRA_CONFIGS:
+            torch.cuda.empty_cache()
+            result["configs"][name] = summary(run_workload(args, name, steps, warmup, cpu=False), steps, warmup)
+    print(json.dumps(result))
+
+
+HEADLINE = "organic65536"
+# BASELINE.json's configurations 3 and 4 and grad-inverse, reported beside the headline configuration (1 + 2)
+EXTRA_CONFIGS = ("organic16384_f64", "boxes4096", "grad_inverse65536", "charges_boxes4096_f64")
+
+
+def summary(r, steps, warmup):
+    """The figures of one extra configuration that go into the headline line."""
+    rf = r["roofline"]
+    out = {"ms_per_step": r["ms_per_step"], "atoms_per_s": r["value"], "dtype": r["dtype"], "steps": steps, "warmup": warmup,
+           "workload": r["config"]["workload"]}
+    if "fwd" in rf:
+        out.update({"fwd_ms": rf["fwd"]["ms"], "bwd_ms": rf["bwd"]["ms"],
+                    "hbm_frac": {"fwd": rf["fwd"]["hbm_frac"], "bwd": rf["bwd"]["hbm_frac"]},
+                    "valu_frac": {"fwd": rf["fwd"]["valu_frac"], "bwd": rf["bwd"]["valu_frac"]}})
+        if "charges" in rf:
+            out["charges"] = rf["charges"]
+    elif rf["bound"] == "valu":
+        out.update({"energy_ms": rf["energy_ms"], "gradients_ms": rf["gradients_ms"], "valu_frac": rf["frac"],
+                    "hbm_frac": rf["hbm_frac"]})
+    else:
+        out.update({"launch_ms": rf["launch_ms"], "hbm_frac": rf["frac"]})
+    return out
+
+
+def run_workload(args, workload, steps, warmup, cpu):
+    """Times one workload; -> its result (the JSON object a run of that workload alone prints), or None in the
+    counter-collection mode."""
+    import numpy as np
+    import torch
+    from khan_amd import datagen, ops
+
+    args = argparse.Namespace(**dict(vars(args), workload=workload, steps=steps, warmup=warmup, no_cpu_baseline=not cpu))
     dev = torch.device("cuda:0")
     kind, n_mols, w, with_charges = WORKLOADS[args.workload]
     tdt = torch.float32 if w == 4 else torch.float64
@@ -359,7 +411,23 @@ def main():
         print("traffic probe: %s x2 on %s, then a 64 MiB device copy" % (args.traffic_probe, args.workload))
         return
 
-    ev = {k: [] for k in ("sort", "fwd", "bwd")}
+    ev = {k: [] for k in ("sort", "fwd", "bwd", "charges")}
+
+    def sort_alone_ms(reps=20):
+        """mol_offsets + ani_sort + size_order (nine launches) on an otherwise idle GPU, per batch."""
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for k in range(3 + reps):
+            if k == 3:
+                torch.cuda.synchronize()
+                e0.record()
+            macs_, _ = ops.mol_offsets(mol_idxs, n_mols)
+            ops.ani_sort(A)
+            ops.size_order(macs_)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    sort_ms_alone = sort_alone_ms()
 
     # atom_counts is a host-memory input of featurize (the reference's op reads it on the host), so every batch
     # needs one 16-byte device-to-host copy between its sort and its forward pass.  As the reference's staging
@@ -427,6 +495,10 @@ def main():
             e = ops.ani_charge(X, Y, Z, Q, mos, macs)
             qg = ops.ani_charge_grad_xyz(X, Y, Z, Q, mos, macs, ones_m)
             behind = None
+            if timed:
+                marks.append(torch.cuda.Event(enable_timing=True))
+                marks[3].record()
+                behind = marks[3]
         if behind is None:
             behind = torch.cuda.Event()
             behind.record()
@@ -451,7 +523,9 @@ def main():
         ev["sort"].append(sm[0].elapsed_time(sm[1]))
         ev["fwd"].append(m[0].elapsed_time(m[1]))
         ev["bwd"].append(m[1].elapsed_time(m[2]))
-    ms = {k: float(np.mean(v)) for k, v in ev.items()}      # event intervals on the launch stream
+        if with_charges:
+            ev["charges"].append(m[2].elapsed_time(m[3]))
+    ms = {k: float(np.mean(v)) for k, v in ev.items() if v}      # event intervals on the launch stream
     ms_per_step = elapsed / args.steps * 1e3
 
     # dominant kernel = the longer of forward / backward; both bound by HBM when the arithmetic is minimal
@@ -460,7 +534,7 @@ def main():
     dom_flops = work["flops_" + dom]
     achieved = dom_bytes / (ms[dom] * 1e-3) / 1e9
     valu_peak = FP32_PEAK_TFLOPS if w == 4 else FP64_PEAK_TFLOPS
-    from khan_amd import profiling
+    import bench_profiling as profiling
     traffic, traffic_stale, traffic_entry = profiling.measured_traffic(args.workload, dom)
     roofline = {
         "kernel": "aev_bwd" if dom == "bwd" else "aev_fwd",
@@ -481,9 +555,18 @@ def main():
                 "valu_frac": work["flops_fwd"] / (ms["fwd"] * 1e-3) / 1e12 / valu_peak},
         "bwd": {"ms": ms["bwd"], "hbm_frac": work["bytes_bwd"] / (ms["bwd"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
                 "valu_frac": work["flops_bwd"] / (ms["bwd"] * 1e-3) / 1e12 / valu_peak},
-        "sort_offsets_ms": ms["sort"],
+        # mol_offsets + ani_sort + size_order of one batch: the nine launches alone on an idle GPU, and the interval
+        # they span in the timed loop, where they ride on the feeder stream beside the passes of the batch before
+        # (both passes fill the GPU, so the small launches wait for free wave slots; the step does not wait for them)
+        "sort_offsets_ms": sort_ms_alone,
+        "sort_offsets_interval_beside_passes_ms": ms["sort"],
         "host_enqueue_ms_per_step": host_enqueue_s / args.steps * 1e3,
     }
+    if with_charges:
+        C = counts["C"]
+        peak = FP32_PEAK_TFLOPS if w == 4 else FP64_PEAK_TFLOPS
+        roofline["charges"] = {"ms": ms["charges"], "what": "ani_charge + ani_charge_grad_xyz (energy, dE/dq, dE/dxyz)",
+                               "valu_frac": 45.0 * C / (ms["charges"] * 1e-3) / 1e12 / peak}
 
     result = {
         "metric": "AEV fwd+grad atoms/sec, fp%d, 1 MI355X" % (8 * w),
@@ -511,7 +594,7 @@ def main():
         result["config"]["forward_phase2"] = args.phase2 + " cores (measurement variant, not the default kernel)"
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(batch, min(n_mols, 8192) if kind == "organic" else 32, min(n_mols, 4096) if kind == "organic" else 8, w)
-    print(json.dumps(result))
+    return result
 
 
 if __name__ == "__main__":

@@ -10,25 +10,25 @@ Refreshing an entry (on a GPU box; four counter passes, one counter each, each a
     rocprofv3 --pmc FETCH_SIZE --kernel-trace --output-format csv -d OUT/fwd_fetch -o p -- python3 bench.py --workload W --traffic-probe fwd
     rocprofv3 --pmc WRITE_SIZE --kernel-trace --output-format csv -d OUT/fwd_write -o p -- python3 bench.py --workload W --traffic-probe fwd
     (the same two with --traffic-probe bwd)
-    python3 -m khan_amd.profiling traffic --workload W --dir OUT
+    python3 bench_profiling.py traffic --workload W --dir OUT
 
 `bench.py --traffic-probe` launches the pass twice and then a plain 64 MiB device-to-device copy whose traffic is
 known; the counters of the pass are scaled by what they read for that copy.
 
-Time by stage (`python -m khan_amd.profiling stages --workload W`): the passes are timed on the default library and on
+Time by stage (`python bench_profiling.py stages --workload W`): the passes are timed on the default library and on
 three measurement builds with the angular part, the radial part or both compiled out
 (`python -m khan_amd.build --stage-variants`, built beforehand); differences of those times are the stages.
 """
 import csv
 import glob
-import hashlib
 import json
 import os
 import subprocess
 import sys
 
-HERE = os.path.dirname(os.path.abspath(__file__))
-ROOT = os.path.dirname(HERE)
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
 RECORD = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 COPY_BYTES = 64 * 1024 * 1024
 
@@ -47,28 +47,12 @@ DOMINANT = {
 }
 
 
-def _code_only(text):
-    """Source text without comments and with runs of white space collapsed: what the digest is taken over, so that
-    rewording a comment does not make a measurement stale."""
-    import re
-    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
-    text = re.sub(r"//[^\n]*", " ", text)
-    return " ".join(text.split())
-
-
 def kernel_sources_digest():
-    """sha256 over the code (comments left out) of the AEV kernels the record is about (csrc/aev_*.hip, csrc/aev_*.h,
-    the two shared headers) and the build flags, 16 hex digits."""
-    from . import build
-    h = hashlib.sha256()
-    csrc = os.path.join(HERE, "csrc")
-    for name in sorted(os.listdir(csrc)):
-        if (name.startswith("aev_") and name.endswith((".hip", ".h"))) or name in ("khan_internal.h", "khan_params.h"):
-            h.update(name.encode())
-            with open(os.path.join(csrc, name), "r") as f:
-                h.update(_code_only(f.read()).encode())
-    h.update(" ".join(build.HIPCC_FLAGS).encode())
-    return h.hexdigest()[:16]
+    """Digest of the code of the AEV kernels the record is about (csrc/aev_*.hip, csrc/aev_*.h and the two shared
+    headers; comments left out) and of the build flags, 16 hex digits."""
+    from khan_amd import build
+    names = [os.path.basename(n) for n in build.HIP_SOURCES + build.HIP_HEADERS]
+    return build.sources_digest([n for n in names if n.startswith("aev_") or n in ("khan_internal.h", "khan_params.h")])
 
 
 def load_records():
@@ -159,7 +143,7 @@ def time_passes(workload, repeats=20):
     """Average time of the forward and of the backward pass (ms) of a bench workload on the library this process
     loaded, each pass launched with the batch's size order and size classes as bench.py does."""
     import torch
-    from . import datagen, ops
+    from khan_amd import datagen, ops
     kind, n_mols = BENCH_SHAPES[workload[:-4] if workload.endswith("_f64") else workload]
     tdt = torch.float64 if workload.endswith("_f64") else torch.float32
     b = datagen.make_batch(kind, n_mols)
@@ -197,7 +181,7 @@ def time_passes(workload, repeats=20):
 def stage_times(workload):
     """Time of the passes with the angular part, the radial part or both compiled out (the measurement builds of
     khan_amd.build.build_stage_variants), each library in a process of its own.  Returns {build: {fwd, bwd}}."""
-    from . import build
+    from khan_amd import build
     res = {}
     for name, skip in (("full", 0), ("no angular part", 1), ("no radial part", 2), ("neither (skeleton)", 3)):
         env = dict(os.environ)
@@ -207,7 +191,7 @@ def stage_times(workload):
             if not os.path.exists(lib):
                 raise RuntimeError(lib + " is missing: python -m khan_amd.build --stage-variants")
             env["KHAN_AEV_LIBRARY"] = lib
-        r = subprocess.run([sys.executable, "-m", "khan_amd.profiling", "time", "--workload", workload],
+        r = subprocess.run([sys.executable, os.path.join(ROOT, "bench_profiling.py"), "time", "--workload", workload],
                            env=env, cwd=ROOT, capture_output=True, text=True, timeout=300)
         if r.returncode != 0:
             raise RuntimeError("timing %s failed: %s" % (name, r.stderr[-2000:]))

@@ -76,6 +76,37 @@ class _AniCharge(torch.autograd.Function):
         return None, None, None, ops.ani_charge_grad(*args), None, None
 
 
+
+def _library_layer_backward(ctx, xs, ws, bs, gouts, celu_act, alpha, head=None):
+    """The gradients of one dense layer of the four atomic networks (with `head`: followed by the output layer) formed
+    from library operations under autograd, so that they carry a graph of their own: what `_Dense.backward` and
+    `_DenseHead.backward` return when they are differentiated again.  -> the gradients in the order of the layer's
+    tensor inputs (inputs, weights, biases[, output weights, output biases]), None where none was asked for."""
+    groups = 5 if head is not None else 3
+    res = [[None] * 4 for _ in range(groups)]
+    with torch.enable_grad():
+        for t in range(4):
+            if gouts[t] is None:
+                continue
+            k = ws[t].shape[0]
+            x = xs[t].reshape(-1, k)
+            a = torch.addmm(bs[t], x, ws[t])
+            if celu_act:
+                a = torch.nn.functional.celu(a, alpha)
+            operands = [xs[t], ws[t], bs[t]]
+            if head is not None:
+                a = (a @ head[0][t].reshape(-1, 1)).reshape(-1) + head[1][t].reshape(-1)
+                operands += [head[0][t], head[1][t]]
+            asked = [j for j in range(groups) if ctx.needs_input_grad[3 + 4 * j + t] and operands[j].requires_grad]
+            if not asked or not a.requires_grad:
+                continue
+            gs = torch.autograd.grad(a, [operands[j] for j in asked], gouts[t].reshape(a.shape), create_graph=True,
+                                     allow_unused=True)
+            for j, g in zip(asked, gs):
+                res[j][t] = g
+    return tuple(g for group in res for g in group)
+
+
 class _Dense(torch.autograd.Function):
     """act(in_t . W_t + b_t) for the four atom types through `ops.dense` (float32; CELU or no activation), forward on
     the matrix-core kernel and the data gradient too: d/d in = (g .* act'(out)) . W^T, with the activation's derivative
@@ -88,7 +119,7 @@ class _Dense(torch.autograd.Function):
         if weights_t is None:
             weights_t = [w.detach().t().contiguous() for w in ws]
         outs = ops.dense([x.detach().reshape(-1, k) for x in xs], weights_t, [b.detach() for b in bs], activation, alpha)
-        ctx.save_for_backward(*xs, *ws, *outs)
+        ctx.save_for_backward(*xs, *ws, *outs, *bs)
         ctx.activation, ctx.alpha = activation, alpha
         return outs
 
@@ -98,6 +129,11 @@ class _Dense(torch.autograd.Function):
         xs, ws, outs = saved[0:4], saved[4:8], saved[8:12]
         k, n_out = ws[0].shape
         celu_act = ctx.activation == ops.ACT_CELU
+        if torch.is_grad_enabled():
+            # A graph of this gradient was asked for (create_graph: a loss on forces differentiated with respect to
+            # the weights).  The kernels record nothing, so the layer is formed again from library operations, which
+            # do, and differentiated by them.
+            return (None, None, None) + _library_layer_backward(ctx, xs, ws, saved[12:16], gouts, celu_act, ctx.alpha)
         gs = [torch.zeros_like(outs[t]) if gouts[t] is None else gouts[t].contiguous() for t in range(4)]
         gx = (None,) * 4
         if any(ctx.needs_input_grad[3:7]):
@@ -139,7 +175,7 @@ class _DenseHead(torch.autograd.Function):
             weights_t = [w.detach().t().contiguous() for w in ws]
         outs, heads = ops.dense_head([x.detach().reshape(-1, k) for x in xs], weights_t, [b.detach() for b in bs],
                                      [w.detach() for w in hws], [b.detach() for b in hbs], activation, alpha)
-        ctx.save_for_backward(*xs, *ws, *hws, *outs)
+        ctx.save_for_backward(*xs, *ws, *hws, *outs, *bs, *hbs)
         ctx.activation, ctx.alpha = activation, alpha
         return heads
 
@@ -149,6 +185,9 @@ class _DenseHead(torch.autograd.Function):
         xs, ws, hws, outs = saved[0:4], saved[4:8], saved[8:12], saved[12:16]
         k, n_out = ws[0].shape
         celu_act = ctx.activation == ops.ACT_CELU
+        if torch.is_grad_enabled():      # create_graph: see _Dense.backward
+            return (None, None, None) + _library_layer_backward(ctx, xs, ws, saved[16:20], gheads, celu_act, ctx.alpha,
+                                                                head=(hws, saved[20:24]))
         gs = [torch.zeros(outs[t].shape[0], dtype=outs[t].dtype, device=outs[t].device) if gheads[t] is None
               else gheads[t].contiguous() for t in range(4)]
         gx = (None,) * 4
@@ -197,8 +236,27 @@ class _MolEnergy(torch.autograd.Function):
     @staticmethod
     def backward(ctx, ge):
         atom_types, sis, mos, macs = ctx.saved_tensors
-        gs = ops.mol_energy_grad(ge.contiguous(), atom_types, sis, mos, macs, ctx.counts)
+        gs = _MolEnergyGrad.apply(atom_types, sis, mos, macs, tuple(ctx.counts), ge)
         return (None, None, None, None) + tuple(g.reshape(sh) for g, sh in zip(gs, ctx.shapes))
+
+
+class _MolEnergyGrad(torch.autograd.Function):
+    """Every atom's entry of the four per-type vectors takes its molecule's value (`ops.mol_energy_grad`), the
+    transpose of the sums by molecule -- whose own way back is therefore those sums again (`ops.mol_energy`).  Both
+    maps are linear, so the pair is differentiable to any order."""
+
+    @staticmethod
+    def forward(ctx, atom_types, sis, mos, macs, counts, ge):
+        ctx.save_for_backward(atom_types, sis, mos, macs)
+        ctx.counts, ctx.dt, ctx.dev = counts, ge.dtype, ge.device
+        return tuple(ops.mol_energy_grad(ge.detach().contiguous(), atom_types, sis, mos, macs, list(counts)))
+
+    @staticmethod
+    def backward(ctx, *dgs):
+        atom_types, sis, mos, macs = ctx.saved_tensors
+        dgs = [torch.zeros(c, dtype=ctx.dt, device=ctx.dev) if d is None else d.contiguous()
+               for d, c in zip(dgs, ctx.counts)]
+        return (None,) * 5 + (_MolEnergy.apply(atom_types, sis, mos, macs, *dgs),)
 
 
 def mol_energy(type_outputs, atom_types, sis, mos, macs):

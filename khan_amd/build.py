@@ -4,10 +4,19 @@
   khan_amd/csrc/libkhan_datagen.so  host-only synthetic batch generator (gcc)
   khan_amd/csrc/libkhan_host.so     host-only batch assembly (gcc, OpenMP)
 
+plus csrc/check_build/libkhan_aev.so, the same library with the check switches compiled in (`build_check_variant`),
+which only the tests of those switches load.
+
 Run as ``python -m khan_amd.build`` or through ``__graft_entry__.build()``.
 ``python -m khan_amd.build --stage-variants`` builds the three measurement libraries of `build_stage_variants`.
+
+Every libkhan_aev.so gets a stamp beside it (``libkhan_aev.so.digest``): the digest of the sources and flags it was
+built from, written after the generated code has passed `check_dpp_sources` and the link has succeeded.
+`library_is_current()` compares it with the sources in the tree.
 """
+import hashlib
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -39,17 +48,73 @@ def _hipcc():
     return exe
 
 
-def build_hip(jobs=4, defines=(), out_dir=None):
-    """Compile every HIP translation unit for gfx950 and link libkhan_aev.so (into `out_dir`, default csrc/)."""
+def _code_only(text):
+    """Source text without comments and with runs of white space collapsed: what a digest is taken over, so that
+    rewording a comment changes nothing."""
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", " ", text)
+    return " ".join(text.split())
+
+
+def sources_digest(names=None, defines=()):
+    """sha256 (16 hex digits) over the code of the HIP sources and headers (`names`: a subset of their file names;
+    default all of them), the compiler flags and the defines."""
+    h = hashlib.sha256()
+    paths = [os.path.join(CSRC, n) for n in HIP_SOURCES] + [n if os.path.isabs(n) else os.path.join(CSRC, n) for n in HIP_HEADERS]
+    for path in sorted(paths, key=os.path.basename):
+        name = os.path.basename(path)
+        if names is not None and name not in names:
+            continue
+        h.update(name.encode())
+        with open(path, "r") as f:
+            h.update(_code_only(f.read()).encode())
+    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join(sorted(defines)).encode())
+    return h.hexdigest()[:16]
+
+
+LIBRARY = os.path.join(CSRC, "libkhan_aev.so")
+
+
+def stamp_path(library=LIBRARY):
+    return library + ".digest"
+
+
+def library_stamp(library=LIBRARY):
+    """The digest written beside `library` when it was built, or None."""
+    try:
+        with open(stamp_path(library)) as f:
+            return f.read().strip()
+    except OSError:
+        return None
+
+
+def library_is_current(library=LIBRARY, defines=()):
+    """True if `library` exists and was built from the sources, flags and defines in the tree."""
+    return os.path.exists(library) and library_stamp(library) == sources_digest(defines=defines)
+
+
+def build_hip(jobs=4, defines=(), out_dir=None, sources=None):
+    """Compile the HIP translation units for gfx950 and link libkhan_aev.so (into `out_dir`, default csrc/).
+    `sources`: the translation units to compile with `defines`; the others' objects are taken from csrc/ as the
+    default build left them (for a variant whose defines touch only those files)."""
     hipcc = _hipcc()
     out_dir = out_dir or CSRC
     os.makedirs(out_dir, exist_ok=True)
+    stamp = stamp_path(os.path.join(out_dir, "libkhan_aev.so"))
+    if os.path.exists(stamp):
+        os.remove(stamp)                 # no stamp while the library and the sources may disagree
     objs = []
     procs = []
     for src in HIP_SOURCES:
+        shared = sources is not None and src not in sources
+        default_obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+        if shared and os.path.exists(default_obj) and os.path.getmtime(default_obj) >= os.path.getmtime(os.path.join(CSRC, src)):
+            objs.append(default_obj)
+            continue
         obj = os.path.join(out_dir, src.replace(".hip", ".o"))
         objs.append(obj)
-        cmd = [hipcc] + HIPCC_FLAGS + ["-D" + d for d in defines] + ["-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc] + HIPCC_FLAGS + ["-D" + d for d in (() if shared else defines)] + ["-c", os.path.join(CSRC, src), "-o", obj]
         print("+", " ".join(cmd), flush=True)
         procs.append(subprocess.Popen(cmd))
         if len(procs) >= jobs:
@@ -64,7 +129,25 @@ def build_hip(jobs=4, defines=(), out_dir=None):
     check_dpp_sources(defines)
     out = os.path.join(out_dir, "libkhan_aev.so")
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs)
+    with open(stamp, "w") as f:
+        f.write(sources_digest(defines=defines) + "\n")
     return out
+
+
+# The check switches (-DKHAN_CHECK_BUILD): environment variables, read once per process, that route every molecule
+# through the general-shape kernels (KHAN_AEV_FORCE_GENERIC=1), withhold the large molecules' scratch
+# (KHAN_AEV_LARGE_SCRATCH=0) or sum the forward kernel's angular records on the matrix cores (KHAN_AEV_PHASE2=matrix,
+# a measured-and-dropped variant).  They are compiled into csrc/check_build/libkhan_aev.so only, which the tests of
+# those paths name in KHAN_AEV_LIBRARY; the default library reads no such variable.
+CHECK_DEFINES = ("KHAN_CHECK_BUILD=1",)
+CHECK_SOURCES = ("capi.hip", "aev_small.hip")
+CHECK_LIBRARY = os.path.join(CSRC, "check_build", "libkhan_aev.so")
+
+
+def build_check_variant():
+    """csrc/check_build/libkhan_aev.so: the default build's objects, with the translation units that hold the check
+    switches compiled again with them.  Call after `build_hip()`."""
+    return build_hip(defines=CHECK_DEFINES, out_dir=os.path.dirname(CHECK_LIBRARY), sources=CHECK_SOURCES)
 
 
 STAGE_BUILDS = os.path.join(CSRC, "stage_builds")
@@ -76,7 +159,7 @@ def stage_variant_path(skip):
 
 def build_stage_variants():
     """Measurement builds of libkhan_aev.so with a stage of the AEV kernels compiled out (KHAN_PROFILE_SKIP = 1:
-    no angular part, 2: no radial part, 3: neither), for `python -m khan_amd.profiling stages`.  Their results are
+    no angular part, 2: no radial part, 3: neither), for `python bench_profiling.py stages`.  Their results are
     wrong by design; they are loaded only when KHAN_AEV_LIBRARY names them."""
     return [build_hip(defines=("KHAN_PROFILE_SKIP=%d" % k,), out_dir=os.path.dirname(stage_variant_path(k)))
             for k in (1, 2, 3)]
@@ -210,7 +293,7 @@ def build_host():
 
 
 def build_all():
-    return [build_hip(), build_datagen(), build_host()]
+    return [build_hip(), build_check_variant(), build_datagen(), build_host()]
 
 
 if __name__ == "__main__":

@@ -322,9 +322,10 @@ hipError_t launch_fwd_small(const T* X, const T* Y, const T* Z, const int32_t* A
 {
     if (n_mols <= 0) return hipSuccess;
     const unsigned blocks = (static_cast<unsigned>(n_mols) + kWavesPerBlock - 1u) / kWavesPerBlock;
+#ifdef KHAN_CHECK_BUILD
     if constexpr (sizeof(T) == 4) {
-        // KHAN_AEV_PHASE2=matrix (read once) selects the variant that sums the angular records on the matrix cores;
-        // it is slower than the default and kept for measurement
+        // check build only: KHAN_AEV_PHASE2=matrix (read once) selects the variant that sums the angular records on the
+        // matrix cores; it is slower than the default and kept for measurement
         static const bool matrix_phase2 = [] {
             const char* v = std::getenv("KHAN_AEV_PHASE2");
             return v != nullptr && std::strcmp(v, "matrix") == 0;
@@ -335,6 +336,7 @@ hipError_t launch_fwd_small(const T* X, const T* Y, const T* Z, const int32_t* A
             return hipGetLastError();
         }
     }
+#endif
     aev_fwd_small_kernel<T, false><<<dim3(blocks), dim3(64 * kWavesPerBlock), 0, stream>>>(
         X, Y, Z, A, MOs, MACs, n_mols, SIs, nullptr, nullptr, nullptr, out, max_atoms < 64 ? max_atoms : 64, order);
     return hipGetLastError();

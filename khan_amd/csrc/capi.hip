@@ -48,8 +48,11 @@ int hip_status(hipError_t e)
 
 inline hipStream_t as_stream(khan_stream_t s) { return static_cast<hipStream_t>(s); }
 
-// KHAN_AEV_FORCE_GENERIC=1 in the environment routes every molecule through the general-shape
-// kernels (read once; meant for A/B checks of the specialised kernels).
+// Check build only (-DKHAN_CHECK_BUILD, khan_amd/build.py: build_check_variant): KHAN_AEV_FORCE_GENERIC=1 in the
+// environment routes every molecule through the general-shape kernels, KHAN_AEV_LARGE_SCRATCH=0 withholds the large
+// molecules' scratch (both read once), so that tests reach those paths on ordinary inputs.  The default library
+// reads no environment variable here.
+#ifdef KHAN_CHECK_BUILD
 bool force_generic()
 {
     static const bool v = [] {
@@ -58,6 +61,18 @@ bool force_generic()
     }();
     return v;
 }
+bool large_scratch_withheld()
+{
+    static const bool v = [] {
+        const char* e = getenv("KHAN_AEV_LARGE_SCRATCH");
+        return e && e[0] == '0';
+    }();
+    return v;
+}
+#else
+constexpr bool force_generic() { return false; }
+constexpr bool large_scratch_withheld() { return false; }
+#endif
 
 template <typename T>
 bool aligned16(const khan::Buckets<const T>& g)
@@ -112,12 +127,7 @@ class LargeScratch {
 public:
     LargeScratch(size_t bytes, hipStream_t stream) : stream_(stream)
     {
-        // KHAN_AEV_LARGE_SCRATCH=0 in the environment (read once) withholds the scratch, for checks of the path without it
-        static const bool withheld = [] {
-            const char* e = getenv("KHAN_AEV_LARGE_SCRATCH");
-            return e && e[0] == '0';
-        }();
-        if (bytes == 0 || withheld) return;
+        if (bytes == 0 || large_scratch_withheld()) return;
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
             (void)hipGetLastError();

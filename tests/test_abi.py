@@ -169,7 +169,7 @@ def test_traffic_record_is_tied_to_the_kernel_sources(tmp_path, monkeypatch):
     """bench.py reports roofline.traffic from the record only while the record's digest matches the kernel sources in
     the tree; a record measured on other sources comes back as stale (bytes None), a missing one as absent."""
     import json
-    from khan_amd import profiling
+    import bench_profiling as profiling
     d = profiling.kernel_sources_digest()
     assert len(d) == 16 and d == profiling.kernel_sources_digest()
     rec = tmp_path / "hbm_traffic.json"
@@ -186,7 +186,7 @@ def test_traffic_record_is_tied_to_the_kernel_sources(tmp_path, monkeypatch):
 def test_the_committed_traffic_record_names_the_dominant_kernels():
     """Every entry of profiles/hbm_traffic.json belongs to a (workload, pass) whose dominant kernel is known, and
     carries the pieces its total is made of."""
-    from khan_amd import profiling
+    import bench_profiling as profiling
     rec = profiling.load_records()
     assert rec, "profiles/hbm_traffic.json is missing or empty"
     for key, e in rec.items():
@@ -210,3 +210,17 @@ def test_measurement_builds_are_not_the_default_library(monkeypatch):
     assert importlib.reload(_lib).LIB_PATH == build.stage_variant_path(3)
     monkeypatch.delenv("KHAN_AEV_LIBRARY")
     importlib.reload(_lib)
+
+
+def test_library_stamp_matches_the_sources():
+    """The libraries the tests load were built from the sources in the tree: the digest stamped beside each at build
+    time (after the generated code passed the lane-exchange check and the link succeeded) equals the digest of the
+    sources, flags and defines now.  tests/conftest.py builds again when it does not."""
+    from khan_amd import build
+    assert build.library_stamp() == build.sources_digest()
+    assert build.library_is_current()
+    assert build.library_stamp(build.CHECK_LIBRARY) == build.sources_digest(defines=build.CHECK_DEFINES)
+    assert build.library_stamp() != build.library_stamp(build.CHECK_LIBRARY)
+    # the digest follows the code, not the comments
+    assert build._code_only("a = 1; // note\n/* more */ b = 2;") == build._code_only("a = 1;\nb = 2;")
+    assert build.sources_digest(["capi.hip"]) != build.sources_digest(["charges.hip"])

@@ -1,4 +1,5 @@
-"""KHAN_AEV_FORCE_GENERIC=1 (read once per process by libkhan_aev.so) routes every molecule through the general-shape
+"""The check build of libkhan_aev.so (khan_amd/build.py: build_check_variant; the default library reads no environment
+variable) offers two switches.  KHAN_AEV_FORCE_GENERIC=1 (read once per process) routes every molecule through the general-shape
 kernels (workgroup per molecule, wavefront per centre), which otherwise only see the centres whose lists overflow and,
 when no scratch memory may be taken, molecules of more than 256 atoms.  KHAN_AEV_LARGE_SCRATCH=0 withholds that scratch
 memory, as a stream under graph capture or a failed allocation would: molecules of more than 256 atoms then go to the
@@ -94,7 +95,10 @@ def test_general_shape_kernels_match_the_oracle(tmp_path, kind, n_mols, variable
     jvp = np.concatenate(ob.featurize_grad_inverse(b.X, b.Y, b.Z, b.A, MOs, MACs, sc, ac, v[0], v[1], v[2], dtype=np.float64))
     out, inp = str(tmp_path / "generic.npz"), str(tmp_path / "inputs.npz")
     np.savez(inp, X=b.X, Y=b.Y, Z=b.Z, A=b.A, mol_idxs=b.mol_idxs, n_mols=b.n_mols)
+    from khan_amd import build
+    assert os.path.exists(build.CHECK_LIBRARY), "the check build is missing: python -m khan_amd.build"
     env = dict(os.environ)
+    env["KHAN_AEV_LIBRARY"] = build.CHECK_LIBRARY
     name, value = variable.split("=")
     env[name] = value
     print("child: %s, %s, %d molecules, %d atoms" % (variable, kind, b.n_mols, b.n_atoms), flush=True)

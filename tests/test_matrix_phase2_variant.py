@@ -1,5 +1,6 @@
 """The measurement variant of the small-molecule forward kernel that sums the angular records on the matrix cores
-(KHAN_AEV_PHASE2=matrix, read once per process by libkhan_aev.so) gives the same features as the default kernel:
+(KHAN_AEV_PHASE2=matrix, read once per process by the check build of libkhan_aev.so, which alone holds that kernel and
+that switch: khan_amd/build.py, build_check_variant) gives the same features as the default kernel:
 checked against the float64 oracle at the float32 tolerance of test_gpu_parity.py.  The variable is read when the
 first forward pass is launched, so the variant runs in a child process."""
 import os
@@ -38,7 +39,11 @@ def run_child(tmp_path, name, n_mols, variant):
     out = str(tmp_path / (name + ".npy"))
     env = dict(os.environ)
     env.pop("KHAN_AEV_PHASE2", None)
+    env.pop("KHAN_AEV_LIBRARY", None)
     if variant:
+        from khan_amd import build
+        assert os.path.exists(build.CHECK_LIBRARY), "the check build is missing: python -m khan_amd.build"
+        env["KHAN_AEV_LIBRARY"] = build.CHECK_LIBRARY
         env["KHAN_AEV_PHASE2"] = variant
     print("child: KHAN_AEV_PHASE2=%s, organic %d molecules" % (variant, n_mols), flush=True)
     subprocess.run([sys.executable, "-c", CHILD, ROOT, out, str(n_mols)], env=env, check=True, timeout=300)

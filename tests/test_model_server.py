@@ -515,3 +515,43 @@ def test_energy_server_round_trip_over_a_socket():
         server.close_connection(c)
     th.join(30)
     assert not th.is_alive()
+
+
+@pytest.mark.gpu
+def test_force_loss_reaches_the_weights_through_the_kernel_layers():
+    """A loss on forces (the coordinate gradient of the energy, taken with create_graph) differentiated with respect to
+    every weight and bias -- what force training does (khan/training/trainer_multi_tower.py:418-430) -- through the
+    kernel layers against the same model with library layers.  The kernel layers' own way back records no graph; asked
+    for one, they form the layer from library operations, and the force term must arrive in the weight gradients."""
+    from khan_amd.batching import DeviceBatch
+    b, _ = _molecules(n_mols=60, first=11)
+    dev = "cuda:0"
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    batch = DeviceBatch.from_device_arrays(d(b.X), d(b.Y), d(b.Z), d(b.A), d(b.mol_idxs), b.n_mols)
+    target = torch.from_numpy(np.random.default_rng(5).standard_normal((b.n_atoms, 3)).astype(np.float32)).to(dev)
+    grads, force_only = [], []
+    for kernel in (True, False):
+        m = model.AniModel(model.DEFAULT_LAYERS, model.celu, torch.float32, dev, seed=4, first_layer_kernel=kernel)
+        m.near.weights_need_grad = True
+        assert m.near.kernel_layers() == (3 if kernel else 0)
+        names = sorted(m.near.params)
+        xs, ys, zs = (t.detach().clone().requires_grad_(True) for t in (batch.xs, batch.ys, batch.zs))
+        feats = autograd.featurize(xs, ys, zs, batch.atom_types, batch.mol_offsets, batch.mol_atom_counts,
+                                   batch.scatter_idxs, batch.host_counts()[0])
+        energies = autograd.mol_energy(m.near.type_outputs(feats), batch.atom_types, batch.scatter_idxs,
+                                       batch.mol_offsets, batch.mol_atom_counts)
+        gx, gy, gz = torch.autograd.grad(energies.sum(), (xs, ys, zs), create_graph=True)
+        assert gx.requires_grad                               # the forces carry a graph back to the weights
+        force_loss = ((torch.stack((gx, gy, gz), dim=1) - target) ** 2).sum()
+        params = [m.near.params[k] for k in names]
+        gf = torch.autograd.grad(force_loss, params, retain_graph=True, allow_unused=True)
+        gs = torch.autograd.grad(energies.sum() + 0.1 * force_loss, params)
+        force_only.append([None if g is None else g.cpu().numpy().astype(np.float64) for g in gf])
+        grads.append([g.cpu().numpy().astype(np.float64) for g in gs])
+    for name, g1, g0, f1, f0 in zip(names, grads[0], grads[1], force_only[0], force_only[1]):
+        # the output layer's bias does not move the forces; every other parameter does
+        if f0 is None or np.abs(f0).max() == 0.0:
+            assert f1 is None or np.abs(f1).max() == 0.0, name
+        else:
+            assert f1 is not None and np.abs(f1 - f0).max() <= 5e-4 * np.abs(f0).max(), (name, np.abs(f1 - f0).max(), np.abs(f0).max())
+        assert np.abs(g1 - g0).max() <= 5e-4 * max(1e-6, np.abs(g0).max()), (name, np.abs(g1 - g0).max())
