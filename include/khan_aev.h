@@ -79,7 +79,12 @@ int khan_ani_sort(const int32_t *atomic_numbers, int64_t n_atoms, int32_t *scatt
  * Scratch, from the stream-ordered allocator on every call: the molecule indices in order of decreasing size, and,
  * for molecules of more than 256 atoms, a sorted copy of the atoms (about 25 bytes per atom and 48 per molecule of the batch in float32, 41 per atom in
  * float64).  While the stream is being captured into a graph neither is taken: molecules then run in the order given,
- * and those of more than 256 atoms in slower kernels that need no scratch. */
+ * and those of more than 256 atoms in slower kernels that need no scratch.
+ * Precondition for batches with molecules of more than 256 atoms: mos increases with the molecule index and the
+ * molecules do not overlap (mos[m+1] >= mos[m] + macs[m], as the exclusive prefix sum of macs gives).  The sorted copy
+ * keeps a molecule's boxes at a place derived from its offset and its index; with permuted offsets two such molecules
+ * could share box entries and their features would be wrong (every access stays in bounds).  Molecules of up to 256
+ * atoms accept any offsets, as the reference's kernels do. */
 int khan_featurize_f32(const float *xs, const float *ys, const float *zs, const int32_t *as,
                        const int32_t *mos, const int32_t *macs, int32_t n_mols, const int32_t *sis,
                        float *h_feat, float *c_feat, float *n_feat, float *o_feat,
@@ -150,8 +155,8 @@ int khan_featurize_grad_inverse_f64(const double *xs, const double *ys, const do
  * khan_size_order writes it into caller memory instead -- order[n_mols + KHAN_SIZE_ORDER_EXTRA] int32, device:
  * the molecule indices by decreasing atom count, then per-size counts, and in its last four elements the number
  * of molecules of up to 32 atoms, of 33..64, of 65..256 and of more -- and the *_ordered entry points take it as
- * an argument: the same results bit for bit, one order per batch instead of one per call, no allocation, and
- * usable under graph capture.  `order` may be NULL (molecules are then taken in batch order).
+ * an argument: the same results bit for bit, one order per batch instead of one per call, no allocation (but for
+ * the stream-ordered scratch of molecules of more than 256 atoms, see below), and usable under graph capture.  `order` may be NULL (molecules are then taken in batch order).
  * size_classes_host (HOST memory, may be NULL) is a copy of those last four elements: a caller that brings them
  * to the host anyway -- as it does the four atom counts of khan_ani_sort -- spares every pass the launches of
  * the kernels whose size class is empty in this batch (with NULL every kernel is launched and leaves by itself). */

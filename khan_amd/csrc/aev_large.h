@@ -23,7 +23,9 @@ struct SortedAtoms {
 
 // The atoms are ordered along a space-filling curve (up to 16 x 16 x 16 cells over the molecule's extent, Morton order;
 // by type inside a cell), so that 64 consecutive atoms sit close together and a centre can skip the chunks whose box lies beyond its
-// cutoff.  The boxes of molecule `mol` (atoms from offset `off`) start at entry 2 * chunk_base(off, mol).
+// cutoff.  The boxes of molecule `mol` (atoms from offset `off`) start at entry 2 * chunk_base(off, mol): molecule m has
+// at most macs[m] / 64 + 1 chunks, so these ranges are disjoint as long as the offsets increase with the molecule index
+// and the molecules do not overlap (the exclusive prefix sum of the atom counts; stated as a precondition in khan_aev.h).
 __host__ __device__ __forceinline__ size_t chunk_base(int off, int mol) { return static_cast<size_t>(off >> 6) + static_cast<size_t>(mol); }
 constexpr int kSortCellsPerDim = 16;
 constexpr int kSortCells = kSortCellsPerDim * kSortCellsPerDim * kSortCellsPerDim;

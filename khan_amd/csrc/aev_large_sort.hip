@@ -35,9 +35,9 @@ __global__ __launch_bounds__(256) void large_sort_kernel(
 {
     __shared__ int hist[4 * kSortCells];       // atoms per (cell, type); after the scan each one's next free sorted position
     __shared__ int in_step[4 * kSortCells];    // atoms per (cell, type) among the 256 of the current step (zero between steps)
-    __shared__ int2 shared_bin[256];           // (key, thread) of the step's atoms that share their bin with another
+    __shared__ __align__(16) int2 shared_bin[256];           // (key, thread) of the step's atoms that share their bin with another
     __shared__ int wshared[4];                 // how many of them each wavefront holds
-    __shared__ int step_key[256];              // keys of the 256 atoms of the current step
+    __shared__ __align__(16) int step_key[256];              // keys of the 256 atoms of the current step
     __shared__ float ext[4][6];                // each wavefront's share of the molecule's extent
     __shared__ int wsum[4];
     __shared__ unsigned long long want[4];

@@ -74,6 +74,9 @@ constexpr bool force_generic() { return false; }
 constexpr bool large_scratch_withheld() { return false; }
 #endif
 
+// below a few thousand molecules every wavefront of a launch is resident at once and the size order buys nothing
+constexpr int32_t kSizeOrderMinMols = 2048;
+
 template <typename T>
 bool aligned16(const khan::Buckets<const T>& g)
 {
@@ -89,8 +92,7 @@ class SizeOrder {
 public:
     SizeOrder(const int32_t* macs, int32_t n_mols, hipStream_t stream) : stream_(stream)
     {
-        // below a few thousand molecules every wavefront of the launch is resident at once and the order buys nothing
-        if (n_mols < 2048) return;
+        if (n_mols < kSizeOrderMinMols) return;
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
             (void)hipGetLastError();
@@ -511,10 +513,14 @@ int khan_featurize_f32_noalloc(const float* xs, const float* ys, const float* zs
     int32_t* order = nullptr;
     hipError_t e = noalloc_scratch(&order);
     if (e != hipSuccess) return hip_status(e);
-    // the class counts and cursors behind the indices keep the last call's values: launch_size_order clears them
-    // with a kernel first; the indices are all rewritten
-    e = khan::launch_size_order(macs, n_mols, order, as_stream(stream));
-    if (e != hipSuccess) return hip_status(e);
+    if (n_mols < kSizeOrderMinMols) {
+        order = nullptr;       // as khan_featurize_f32: every wavefront of so small a launch is resident at once
+    } else {
+        // the class counts and cursors behind the indices keep the last call's values: launch_size_order clears them
+        // with a kernel first; the indices are all rewritten
+        e = khan::launch_size_order(macs, n_mols, order, as_stream(stream));
+        if (e != hipSuccess) return hip_status(e);
+    }
     khan::Buckets<float> out{{h, c, n, o}};
     // (molecules of more than 256 atoms go through the general-shape kernels here: the faster ones need scratch memory)
     const int64_t n_atoms = static_cast<int64_t>(acs_host[0]) + acs_host[1] + acs_host[2] + acs_host[3];
@@ -746,7 +752,10 @@ int khan_coulomb_grad_f64(const double* xs, const double* ys, const double* zs, 
     return charge_grad_impl<double>(xs, ys, zs, qs, mos, macs, n_mols, grads, false, k, q_grads, gx, gy, gz, true, stream);
 }
 
-// The AEV passes on a size order that the caller computed once for the batch (khan_size_order): nothing is allocated.
+// The AEV passes on a size order that the caller computed once for the batch (khan_size_order).  They allocate nothing,
+// except for a batch that holds a molecule of more than 256 atoms: its sorted copy goes to stream-ordered scratch
+// (with the class counts unknown on the host, for any batch of more than 256 atoms), unless the stream is being
+// captured -- then those molecules take the general-shape kernels, which need none.
 int khan_featurize_ordered_f32(const float* xs, const float* ys, const float* zs, const int32_t* as,
                                const int32_t* mos, const int32_t* macs, int32_t n_mols, const int32_t* sis,
                                float* h, float* c, float* n, float* o, const int32_t* acs_host,

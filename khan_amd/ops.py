@@ -88,7 +88,8 @@ SIZE_ORDER_EXTRA = 520
 def size_order(macs):
     """-> int32[n_mols + 520]: the molecule indices by decreasing atom count and the per-size counts, to be
     passed as `order=` to featurize / featurize_grad / featurize_grad_inverse of the same batch (computed once
-    per batch instead of once per call; the calls then allocate nothing and can be captured into a graph).
+    per batch instead of once per call; the calls then allocate nothing -- except the sorted copy of molecules of more
+    than 256 atoms, where a batch holds any -- and can be captured into a graph).
     Its last four elements (`order[-4:]`) count the molecules of up to 32, 33..64, 65..256 and more atoms: copied
     to the host and passed as `size_classes=`, they spare the passes the launches of kernels without work."""
     lib = _lib.load()

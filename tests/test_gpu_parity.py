@@ -113,6 +113,35 @@ class Case:
                                           upb, dtype=np.float64), axis=1)
 
 
+
+def sample_case(c, mol_ids):
+    """The molecules `mol_ids` of case c as a case of their own, and the indices of their atoms in c."""
+    mol_ids = np.asarray(mol_ids, dtype=np.int64)
+    idx = np.concatenate([np.arange(c.MOs[m], c.MOs[m] + c.MACs[m]) for m in mol_ids]).astype(np.int64)
+    mi = np.repeat(np.arange(len(mol_ids)), c.MACs[mol_ids]).astype(np.int32)
+    return Case(c.X[idx], c.Y[idx], c.Z[idx], c.A[idx], mi, len(mol_ids)), idx
+
+
+def strided_molecules(n_mols, count, block=1):
+    """`count` molecule indices spread evenly over 0..n_mols-1, in runs of `block` consecutive molecules."""
+    starts = np.linspace(0, n_mols - block, count // block).astype(np.int64)
+    return np.unique((starts[:, None] + np.arange(block)[None, :]).reshape(-1))
+
+
+def check_sample_against_oracle(name, c, mol_ids, rows, g, up, rtol, atol, grad_atol):
+    """Rows (atom order) and gradients of a full-size launch against the float64 oracle on a sample of its molecules;
+    `up` are the upstream rows of that launch in atom order."""
+    sub, idx = sample_case(c, mol_ids)
+    it = torch.from_numpy(idx).to("cuda:0")
+    say("   %s: %d molecules, %d atoms against the float64 oracle" % (name, sub.n_mols, sub.N))
+    ref64 = ob.gather_rows(sub.oracle_feat(np.float64), sub.ga)
+    assert_close("rows, " + name, host(rows[it]), ref64, rtol, atol)
+    upb = ob.scatter_rows(host(up[it]).astype(np.float64), sub.A, sub.sc, sub.ac)
+    g64 = sub.oracle_grad(upb)
+    assert_close("gradient, " + name, host(g[it]), g64, rtol, grad_atol, scale=mol_scale(g64, sub.MOs, sub.MACs))
+    return sub, idx
+
+
 def gpu_sort_offsets(ops, c):
     macs, mos = ops.mol_offsets(dev(c.mol_idxs), c.n_mols)
     sc, ga, ac = ops.ani_sort(dev(c.A))
@@ -878,6 +907,13 @@ def test_full_size_batch_properties(ops):
         g64 = sc_.oracle_grad(upb)
         assert_close("gradient of molecules %d.. vs f64 oracle" % first, host(g[a0:a0 + sb.n_atoms]), g64,
                      F32_RTOL, F32_ATOL, scale=mol_scale(g64, sc_.MOs, sc_.MACs))
+    # the oracle on a sample taken at a stride through the whole batch (2,048 molecules in runs of 8), and on the
+    # 64 molecules with the most atoms
+    check_sample_against_oracle("2048 molecules at a stride", c, strided_molecules(M, 2048, block=8), rows, g, up,
+                                F32_RTOL, F32_ATOL, F32_ATOL)
+    largest = np.argsort(-c.MACs.astype(np.int64), kind="stable")[:64]
+    say("   the 64 largest molecules have %d..%d atoms" % (c.MACs[largest].min(), c.MACs[largest].max()))
+    check_sample_against_oracle("the 64 largest molecules", c, np.sort(largest), rows, g, up, F32_RTOL, F32_ATOL, F32_ATOL)
 
 
 # ----------------------------------------------------------------------------- autograd wiring
@@ -1077,6 +1113,23 @@ def test_full_size_double_precision_configuration(ops):
     E64 = ob.ani_charge(b.X[:n256], b.Y[:n256], b.Z[:n256], q[:n256], b.MOs[:256], b.MACs[:256], dtype=np.float64)
     Ea = host(Eabs)[:256]
     assert_close("charge energy, first 256 molecules", host(E)[:256], E64, F64_RTOL, 0.0, scale=Ea)
+    # the oracle on 1,024 molecules taken at a stride through the batch: features, gradients, and the charge
+    # energy with its derivatives by charge and by coordinate
+    ids = strided_molecules(M, 1024, block=4)
+    sub, idx = check_sample_against_oracle("1024 molecules at a stride, f64", c, ids, rows, g, up, F64_RTOL, F64_ATOL, 0.0)
+    qs = q[idx]
+    ones_s = np.ones(sub.n_mols)
+    E_ref = ob.ani_charge(sub.X, sub.Y, sub.Z, qs, sub.MOs, sub.MACs, dtype=np.float64)
+    dq_ref = ob.ani_charge_grad(sub.X, sub.Y, sub.Z, qs, sub.MOs, sub.MACs, ones_s, dtype=np.float64)
+    dxyz_ref = np.stack(ob.ani_charge_grad_xyz(sub.X, sub.Y, sub.Z, qs, sub.MOs, sub.MACs, ones_s, dtype=np.float64), axis=1)
+    # sums of terms of both signs, scaled as in test_charges: the energy by the same sum over |q|, the derivatives by
+    # their largest component in the molecule
+    Ea_s = ob.ani_charge(sub.X, sub.Y, sub.Z, np.abs(qs), sub.MOs, sub.MACs, dtype=np.float64)
+    it = torch.from_numpy(idx).to("cuda:0")
+    assert_close("charge energy, 1024 molecules at a stride", host(E)[ids], E_ref, F64_RTOL, 0.0, scale=Ea_s)
+    assert_close("dE/dq, 1024 molecules at a stride", host(qg[it]), dq_ref, F64_RTOL, 0.0, scale=mol_scale(dq_ref, sub.MOs, sub.MACs))
+    got_xyz = host(torch.stack([cx, cy, cz], 1)[it])
+    assert_close("dE/dxyz, 1024 molecules at a stride", got_xyz, dxyz_ref, F64_RTOL, 0.0, scale=mol_scale(dxyz_ref, sub.MOs, sub.MACs))
 
 
 def test_full_size_dense_boxes_configuration(ops):
@@ -1097,6 +1150,22 @@ def test_full_size_dense_boxes_configuration(ops):
         g64 = sc_.oracle_grad(upb)
         assert_close("gradient of boxes %d.. vs f64 oracle" % first, host(g[a0:a0 + sb.n_atoms]), g64,
                      F32_RTOL, F32_ATOL, scale=mol_scale(g64, sc_.MOs, sc_.MACs))
+    # the oracle on 128 boxes taken at a stride through the batch (float32 launch above), and 32 of them through the
+    # float64 kernels as a batch of their own
+    ids = strided_molecules(M, 128)
+    check_sample_against_oracle("128 boxes at a stride", c, ids, rows, g, up, F32_RTOL, F32_ATOL, F32_ATOL)
+    sub, _ = sample_case(c, ids[::4])
+    say("   32 boxes in float64: %d atoms" % sub.N)
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, sub)
+    acs = ac.cpu()
+    Xd, Yd, Zd = dev(sub.X, np.float64), dev(sub.Y, np.float64), dev(sub.Z, np.float64)
+    f = ops.featurize(Xd, Yd, Zd, dev(sub.A), mos, macs, sc, acs)
+    assert_close("features f64, 32 boxes", host(torch.cat(f)), np.concatenate(sub.oracle_feat(np.float64)), F64_RTOL, F64_ATOL)
+    upb = sub.upstream()
+    gx, gy, gz = ops.featurize_grad(Xd, Yd, Zd, dev(sub.A), mos, macs, sc, acs, *[dev(u) for u in upb])
+    g64 = sub.oracle_grad(upb)
+    assert_close("gradient f64, 32 boxes", host(torch.stack([gx, gy, gz], 1)), g64, F64_RTOL, 0.0,
+                 scale=mol_scale(g64, sub.MOs, sub.MACs))
 
 
 def test_gradient_against_central_differences_on_64_molecules(ops):
@@ -1232,9 +1301,10 @@ def test_gradient_error_per_element_beside_the_references_own_functor(ops):
     for k in range(5):
         assert q_hip32[k] <= q_ref32[k], ("float32 quantile", k, q_hip32, q_ref32)
         assert q_hip64[k] <= q_ref64[k], ("float64 quantile", k, q_hip64, q_ref64)
-    # worst per-element ratios as measured (13.1 in float32, 2.4 in float64: cancelling components); a regression
+    # worst per-element ratios: 1.5 times what was measured (13.1 in float32, 2.4 in float64 on 1,024 molecules; 10.8 and
+    # 1.2 on these 256: cancelling components); a regression
     # in the kernels moves these
-    assert q_hip32[4] <= 40.0 and q_hip64[4] <= 10.0, (q_hip32, q_hip64)
+    assert q_hip32[4] <= 20.0 and q_hip64[4] <= 4.0, (q_hip32, q_hip64)
 
 
 # ----------------------------------------------------------------------------- HIP graph capture

@@ -60,6 +60,49 @@ def test_no_alloc_entry_point_matches_featurize_on_two_calls_in_a_row():
             assert np.all(np.abs(got - ref) <= 1e-6 + 1e-5 * np.abs(ref)), "no-alloc entry point vs the oracle"
 
 
+def test_no_alloc_entry_point_replays_from_a_hip_graph():
+    """What sets the entry point apart: it can run where nothing may be allocated.  After one eager call (which looks
+    the scratch array's address up) it is captured into a HIP graph -- a capture fails on any allocation or memset on
+    the capturing stream -- and replayed on poisoned outputs, with eager work and synchronisations between the replays;
+    every replay must reproduce the eager result bit for bit.  4,096 molecules and two boxes: the size order (cleared by
+    a kernel of the graph, not by a memset node) and the kernels of the larger size classes are part of the graph."""
+    from khan_amd import _lib
+    lib = _lib.load()
+    b, sc, ac, t = _batch("organic", 4096, 20000)
+    big = datagen.make_batch("boxes", 2)
+    A = np.concatenate([b.A, big.A])
+    sc, _, ac = ob.ani_sort(A)
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")
+    macs = np.concatenate([b.MACs, big.MACs]).astype(np.int32)
+    mos = np.concatenate([[0], np.cumsum(macs)[:-1]]).astype(np.int32)
+    t = {"X": d(np.concatenate([b.X, big.X])), "Y": d(np.concatenate([b.Y, big.Y])), "Z": d(np.concatenate([b.Z, big.Z])),
+         "A": d(A), "mos": d(mos), "macs": d(macs), "sc": d(sc)}
+    n = len(A)
+    say("   no-alloc entry point under graph capture: %d molecules, %d atoms" % (len(macs), n))
+    eager = torch.full((n * 384,), -1.0, dtype=torch.float32, device="cuda:0")
+    assert _call(lib, "khan_featurize_f32_noalloc", t, ac, eager) == 0
+    torch.cuda.synchronize()
+    out = torch.full((n * 384,), -2.0, dtype=torch.float32, device="cuda:0")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        status = _call(lib, "khan_featurize_f32_noalloc", t, ac, out)     # on the capturing stream (the current one here)
+    assert status == 0
+    for replay in range(3):
+        out.fill_(-3.0 - replay)
+        scratch_user = torch.full((n * 384,), -1.0, dtype=torch.float32, device="cuda:0")
+        if replay == 1:     # an eager call on a smaller batch in between leaves other contents in the shared scratch
+            b2, sc2, ac2, t2 = _batch("organic", 2300, 100)
+            o2 = torch.empty(b2.n_atoms * 384, dtype=torch.float32, device="cuda:0")
+            assert _call(lib, "khan_featurize_f32_noalloc", t2, ac2, o2) == 0
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), "replay %d differs from the eager call" % replay
+        del scratch_user
+
+
 def test_no_alloc_entry_point_with_a_molecule_of_more_than_256_atoms():
     # above 256 atoms khan_featurize_f32 works on a sorted copy of the atoms in scratch memory; the entry point that
     # allocates nothing keeps to the kernels without scratch: the same features to float32 rounding, both checked
