@@ -236,6 +236,20 @@ int khan_ani_charge_grad_xyz_f64(const double *xs, const double *ys, const doubl
                                  double *x_grads, double *y_grads, double *z_grads,
                                  khan_stream_t stream);
 
+/* AniCharge and both gradients in one pass over the pairs: charge_energies[n_mols] as khan_ani_charge_* gives them
+ * (not multiplied by grads) and q_grads, x_grads, y_grads, z_grads [n_atoms] as khan_ani_charge_grad_xyz_* gives them
+ * (q_grads may be NULL).  No reference counterpart as one op: the reference runs AniCharge forward and AniChargeGrad on
+ * the way back, each a pass of its own over the pairs (ani_charges.cpp:81-119, 170-217); a caller that knows it will
+ * need the gradients (training, force evaluation) gets the energy from the same pair terms at no extra cost. */
+int khan_ani_charge_all_f32(const float *xs, const float *ys, const float *zs, const float *qs,
+                            const int32_t *mos, const int32_t *macs, int32_t n_mols, const float *grads,
+                            float *charge_energies, float *q_grads, float *x_grads, float *y_grads,
+                            float *z_grads, khan_stream_t stream);
+int khan_ani_charge_all_f64(const double *xs, const double *ys, const double *zs, const double *qs,
+                            const int32_t *mos, const int32_t *macs, int32_t n_mols, const double *grads,
+                            double *charge_energies, double *q_grads, double *x_grads, double *y_grads,
+                            double *z_grads, khan_stream_t stream);
+
 /* First dense layer of the per-type atomic networks, right behind the featurizer (khan/model/nn.py:38-68: matmul +
  * bias + activation per atom type; activation CELU, khan/model/activations.py:63-65, or none):
  *     out_t[r, :] = act(rows_t[r, :] . W_t + b_t),  t = H, C, N, O,  one launch for the four types.

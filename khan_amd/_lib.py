@@ -59,6 +59,8 @@ _SIGNATURES = {
     "khan_ani_charge_grad_f64": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32, _ptr, _ptr, _ptr]),
     "khan_ani_charge_grad_xyz_f32": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32] + [_ptr] * 6),
     "khan_ani_charge_grad_xyz_f64": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32] + [_ptr] * 6),
+    "khan_ani_charge_all_f32": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32] + [_ptr] * 7),
+    "khan_ani_charge_all_f64": (ctypes.c_int, [_ptr] * 6 + [ctypes.c_int32] + [_ptr] * 7),
     "khan_dense_first_f32": (ctypes.c_int, [ctypes.POINTER(_ptr), ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(_ptr),
                                             ctypes.POINTER(_ptr), ctypes.c_int32, ctypes.c_float, ctypes.POINTER(_ptr), _ptr]),
     "khan_dense_f32": (ctypes.c_int, [ctypes.POINTER(_ptr), ctypes.POINTER(ctypes.c_int32), ctypes.c_int32, ctypes.c_int32,

@@ -379,14 +379,14 @@ int charge_impl(const T* xs, const T* ys, const T* zs, const T* qs, const int32_
 template <typename T>
 int charge_grad_impl(const T* xs, const T* ys, const T* zs, const T* qs, const int32_t* mos,
                      const int32_t* macs, int32_t n_mols, const T* grads, bool damped, T k, T* qg, T* gx, T* gy, T* gz,
-                     bool want_xyz, khan_stream_t stream)
+                     bool want_xyz, khan_stream_t stream, T* energies = nullptr)
 {
     if (n_mols < 0) return KHAN_ERR_INVALID_ARG;
     if (n_mols == 0) return KHAN_OK;
     if (!xs || !ys || !zs || !qs || !mos || !macs || !grads) return KHAN_ERR_INVALID_ARG;
     if (want_xyz ? (!gx || !gy || !gz) : !qg) return KHAN_ERR_INVALID_ARG;
     return hip_status(khan::launch_charge_grad<T>(xs, ys, zs, qs, mos, macs, n_mols, grads, damped, k, qg,
-                                                  want_xyz ? gx : nullptr, gy, gz, as_stream(stream)));
+                                                  want_xyz ? gx : nullptr, gy, gz, energies, as_stream(stream)));
 }
 
 }  // namespace
@@ -599,6 +599,20 @@ int khan_ani_charge_grad_xyz_f32(const float* xs, const float* ys, const float* 
                                  khan_stream_t stream)
 {
     return charge_grad_impl<float>(xs, ys, zs, qs, mos, macs, n_mols, grads, true, khan::kChargeK_f, q_grads, gx, gy, gz, true, stream);
+}
+int khan_ani_charge_all_f32(const float* xs, const float* ys, const float* zs, const float* qs,
+                            const int32_t* mos, const int32_t* macs, int32_t n_mols, const float* grads,
+                            float* e, float* q_grads, float* gx, float* gy, float* gz, khan_stream_t stream)
+{
+    if (n_mols > 0 && !e) return KHAN_ERR_INVALID_ARG;
+    return charge_grad_impl<float>(xs, ys, zs, qs, mos, macs, n_mols, grads, true, khan::kChargeK_f, q_grads, gx, gy, gz, true, stream, e);
+}
+int khan_ani_charge_all_f64(const double* xs, const double* ys, const double* zs, const double* qs,
+                            const int32_t* mos, const int32_t* macs, int32_t n_mols, const double* grads,
+                            double* e, double* q_grads, double* gx, double* gy, double* gz, khan_stream_t stream)
+{
+    if (n_mols > 0 && !e) return KHAN_ERR_INVALID_ARG;
+    return charge_grad_impl<double>(xs, ys, zs, qs, mos, macs, n_mols, grads, true, static_cast<double>(khan::kChargeK_f), q_grads, gx, gy, gz, true, stream, e);
 }
 int khan_ani_charge_grad_xyz_f64(const double* xs, const double* ys, const double* zs,
                                  const double* qs, const int32_t* mos, const int32_t* macs,

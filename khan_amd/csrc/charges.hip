@@ -22,18 +22,89 @@ namespace khan {
 
 namespace {
 
+// Distance arithmetic per precision.  float: the hardware reciprocal square root with one Newton step, the hardware
+// reciprocal and the minimax cutoff polynomials of the AEV kernels.  double: no library call either -- the library's
+// sqrt, division, cos and sin come to some 250 instructions per pair, most of them range reduction and special cases
+// that cannot occur here, and made these kernels run at 2.6 % of the double-precision vector peak.
+template <typename T> struct ChargeMath;
+template <> struct ChargeMath<float> {
+    // r = sqrt(d2) and 1/r (0 for d2 = 0)
+    static __device__ __forceinline__ void dist(float d2, float& r, float& inv)
+    {
+        r = Fast<float>::sqrt_rn(d2);
+        inv = d2 > 0.0f ? Fast<float>::rcp(r) : 0.0f;
+    }
+    // f_C(r, R_Rc) and its derivative, for r <= R_Rc
+    static __device__ __forceinline__ void cutoff(float r, float& fc, float& dfc)
+    {
+        Fast<float>::cutoff_grad(r, kR_Rc_f, fc, dfc);
+    }
+};
+template <> struct ChargeMath<double> {
+    // v_rsq_f64 is good to 5e-8; one coupled Goldschmidt step (g -> sqrt, h -> 1/(2 sqrt)) squares that, the fused
+    // residual d2 - g^2 is exact and brings g to half an ulp, and one Newton step on the reciprocal of that g gives
+    // 1/r to an ulp: 10 instructions for both (measured against long double on 2^20 arguments: 1.1e-16 and 2.1e-16).
+    // Distances here are of order 1 A: no scaling for denormals is needed.
+    static __device__ __forceinline__ void dist(double d2, double& r, double& inv)
+    {
+        const double x = fmax(d2, 1e-300);
+        const double y = __builtin_amdgcn_rsq(x);
+        double g = x * y, h = 0.5 * y;
+        const double e = fma(-h, g, 0.5);
+        g = fma(g, e, g);
+        h = fma(h, e, h);
+        g = fma(fma(-g, g, x), h, g);
+        double v = h + h;
+        v = fma(v, fma(-g, v, 1.0), v);
+        r = d2 > 0.0 ? g : 0.0;
+        inv = d2 > 0.0 ? v : 0.0;
+    }
+    // f_C = 0.5 cos(pi r / rc) + 0.5 = cos^2(y), f_C' = -(pi / rc) sin(y) cos(y), y = pi r / (2 rc) in [0, pi/2]:
+    // y is folded onto [0, pi/4], where the Taylor polynomials to w^15 and w^16 are exact to 5e-17 and 2e-18
+    static __device__ __forceinline__ void cutoff(double r, double& fc, double& dfc)
+    {
+        constexpr double rc = static_cast<double>(kR_Rc_f);
+        const double y = (kPi / (2.0 * rc)) * r;
+        const bool fold = y > 0.25 * kPi;
+        const double w = fold ? 0.5 * kPi - y : y;
+        const double w2 = w * w;
+        double ps = -1.0 / 1307674368000.0;
+        ps = fma(ps, w2, 1.0 / 6227020800.0);
+        ps = fma(ps, w2, -1.0 / 39916800.0);
+        ps = fma(ps, w2, 1.0 / 362880.0);
+        ps = fma(ps, w2, -1.0 / 5040.0);
+        ps = fma(ps, w2, 1.0 / 120.0);
+        ps = fma(ps, w2, -1.0 / 6.0);
+        const double sw = fma(ps * w2, w, w);
+        double pc = 1.0 / 20922789888000.0;
+        pc = fma(pc, w2, -1.0 / 87178291200.0);
+        pc = fma(pc, w2, 1.0 / 479001600.0);
+        pc = fma(pc, w2, -1.0 / 3628800.0);
+        pc = fma(pc, w2, 1.0 / 40320.0);
+        pc = fma(pc, w2, -1.0 / 720.0);
+        pc = fma(pc, w2, 1.0 / 24.0);
+        pc = fma(pc, w2, -0.5);
+        const double cw = fma(pc, w2, 1.0);
+        const double sn = fold ? cw : sw, cs = fold ? sw : cw;
+        fc = cs * cs;
+        dfc = (-kPi / rc) * sn * cs;
+    }
+};
+
 // kDamped = false drops the cutoff function: plain Coulomb pairs q_i q_j / r (the reference's op is the damped form)
 template <typename T, bool kDamped>
-__device__ __forceinline__ void pair_terms(T dx, T dy, T dz, T pi_rc, T rc, T& u, T& dudr_over_r)
+__device__ __forceinline__ void pair_terms(T dx, T dy, T dz, T& u, T& dudr_over_r)
 {
-    const T r = Real<T>::sqrt_(dx * dx + dy * dy + dz * dz);
+    T r, inv;            // coincident atoms (r = 0): inv = 0, so that (1 - f_C)/r -> 0 there and the pair pulls nowhere
+    ChargeMath<T>::dist(dx * dx + dy * dy + dz * dz, r, inv);
     T fc = T(0), dfc = T(0);
-    if (kDamped && r <= rc) {
-        fc = cutoff_fn(r, pi_rc);
-        dfc = cutoff_dfn(r, pi_rc);
+    if constexpr (kDamped) {
+        // evaluated in every lane and selected: a branch would be taken by nearly every wavefront anyway
+        ChargeMath<T>::cutoff(r, fc, dfc);
+        const bool in = r <= static_cast<T>(kR_Rc_f);
+        fc = in ? fc : T(0);
+        dfc = in ? dfc : T(0);
     }
-    // coincident atoms (r = 0): (1 - f_C)/r -> 0 there, and the pair has no direction to pull along
-    const T inv = r > T(0) ? T(1) / r : T(0);
     u = (T(1) - fc) * inv;                            // (1 - f_C) / r
     dudr_over_r = (-dfc * inv - u * inv) * inv;       // d/dr[(1-f_C)/r] / r
 }
@@ -49,7 +120,6 @@ __global__ __launch_bounds__(256) void charge_energy_kernel(
     if (mol >= n_mols) return;
     const int n = MACs[mol], off = MOs[mol];
     if (n > kSmallMaxAtoms && n <= kMediumMaxAtoms) return;      // the tile kernel's
-    const T rc = static_cast<T>(kR_Rc_f), pi_rc = static_cast<T>(kPi / static_cast<double>(kR_Rc_f));
     T acc = T(0);
     if (n <= 64) {
         const int logW = n <= 16 ? 4 : n <= 32 ? 5 : 6;
@@ -64,7 +134,7 @@ __global__ __launch_bounds__(256) void charge_energy_kernel(
                     qi = __shfl(qj, i & 63, 64);
             const bool valid = (i < n) && jok && (jl > i);
             T u, du;
-            pair_terms<T, kDamped>(valid ? xi - xj : T(1), valid ? yi - yj : T(0), valid ? zi - zj : T(0), pi_rc, rc, u, du);
+            pair_terms<T, kDamped>(valid ? xi - xj : T(1), valid ? yi - yj : T(0), valid ? zi - zj : T(0), u, du);
             acc += valid ? K * qi * qj * u : T(0);
         }
         acc = wave_sum(acc);
@@ -80,15 +150,15 @@ __global__ __launch_bounds__(256) void charge_grad_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const T* __restrict__ Q, const int32_t* __restrict__ MOs, const int32_t* __restrict__ MACs,
     int32_t n_mols, const T* __restrict__ grads, T K, T* __restrict__ q_grads, T* __restrict__ gX,
-    T* __restrict__ gY, T* __restrict__ gZ)
+    T* __restrict__ gY, T* __restrict__ gZ, T* __restrict__ E)
 {
     const int lane = threadIdx.x & 63;
     const int64_t mol = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
     if (mol >= n_mols) return;
     const int n = MACs[mol], off = MOs[mol];
     if (n > kSmallMaxAtoms && n <= kMediumMaxAtoms) return;      // the tile kernel's
-    const T rc = static_cast<T>(kR_Rc_f), pi_rc = static_cast<T>(kPi / static_cast<double>(kR_Rc_f));
     const T gK = grads[mol] * K;
+    T e_acc = T(0);          // sum over atoms of q_i sum_j q_j u_ij = twice the energy / K
     if (n <= 64) {
         const int logW = n <= 16 ? 4 : n <= 32 ? 5 : 6;
         const int W = 1 << logW, G = 64 >> logW;
@@ -103,7 +173,7 @@ __global__ __launch_bounds__(256) void charge_grad_kernel(
             const bool valid = (i < n) && jok && (jl != i);
             const T dx = valid ? xi - xj : T(1), dy = valid ? yi - yj : T(0), dz = valid ? zi - zj : T(0);
             T u, du;
-            pair_terms<T, kDamped>(dx, dy, dz, pi_rc, rc, u, du);
+            pair_terms<T, kDamped>(dx, dy, dz, u, du);
             const T w = valid ? qj * du : T(0);
             // sums over the W partners of the group end up in its last lane
             const T dq = group_sum_to_last_lane(valid ? qj * u : T(0), logW);
@@ -111,6 +181,7 @@ __global__ __launch_bounds__(256) void charge_grad_kernel(
             const T fy = group_sum_to_last_lane(w * dy, logW);
             const T fz = group_sum_to_last_lane(w * dz, logW);
             if (jl == W - 1 && i < n) {
+                e_acc = fma(qi, dq, e_acc);
                 if (q_grads) q_grads[off + i] = gK * dq;
                 if (gX) {
                     gX[off + i] = gK * qi * fx;
@@ -119,112 +190,112 @@ __global__ __launch_bounds__(256) void charge_grad_kernel(
                 }
             }
         }
+        if (E) {
+            e_acc = wave_sum(e_acc);
+            if (lane == 0) E[mol] = T(0.5) * K * e_acc;
+        }
         return;
     }
-    // more than 256 atoms: charge_large_kernel's
+    // more than 256 atoms: charge_large_kernel's, which adds its workgroups' shares to an energy that starts from zero
+    if (E && lane == 0) E[mol] = T(0);
 }
 
-// Molecules of 65 to 256 atoms: one wavefront per molecule, the molecule (x, y, z, q) tiled through LDS.
-// A lane owns the atoms i = lane, lane + 64, ... (at most four).  In round d it pairs each of them with atom
-// j = (i + d) mod n, read from the tile: after (n-1)/2 rounds (plus half a round when n is even) every
-// unordered pair has been evaluated exactly once -- half the pair evaluations of a walk over all j != i, with all
-// lanes busy.  In a round the partners j of all atoms are distinct, so what a pair contributes to its partner
-// (dE/dq_j and the force on j) is added to the partner's slot in LDS by plain read-add-write, without atomics,
-// while the atom's own side stays in registers.  Every output element is written once.
+// Molecules of 65 to 256 atoms: one workgroup of four wavefronts per molecule, the molecule (x, y, z, q) in LDS, one
+// atom i per thread.  In round d a thread pairs its atom with atom j = (i + d) mod n, read from the tile: after
+// (n-1)/2 rounds (plus half a round when n is even) every unordered pair has been evaluated exactly once -- half the
+// pair evaluations of a walk over all j != i.  In a round the partners j of a wavefront's atoms are distinct, so what a
+// pair contributes to its partner (dE/dq_j and the force on j) is added to the partner's slot in LDS by plain
+// read-add-write, without atomics, while the atom's own side stays in registers.  Every wavefront adds into a copy of
+// its own of the partner slots, so the four never wait for each other inside the rounds (a barrier per round would be
+// the alternative); the copies are summed at the end.  A wavefront whose 64 atoms lie beyond the molecule sits the
+// rounds out.  Every output element is written once.
 template <typename T, bool kGrad> struct ChargeTile;
 template <typename T> struct __align__(16) ChargeTile<T, false> {
     typename Fast<T>::vec4 in[kMediumMaxAtoms];     // x, y, z, q
+    T wpart[4];
 };
 template <typename T> struct __align__(16) ChargeTile<T, true> {
     typename Fast<T>::vec4 in[kMediumMaxAtoms];     // x, y, z, q
-    typename Fast<T>::vec4 acc[kMediumMaxAtoms];    // partner side: force x, y, z and dE/dq
+    typename Fast<T>::vec4 acc[4][kMediumMaxAtoms]; // partner side, per wavefront: force x, y, z and dE/dq
+    T wpart[4];
 };
 
 template <typename T, bool kDamped, bool kGrad>
-__global__ __launch_bounds__(64) void charge_tile_kernel(
+__global__ __launch_bounds__(256) void charge_tile_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const T* __restrict__ Q, const int32_t* __restrict__ MOs, const int32_t* __restrict__ MACs,
     int32_t n_mols, const T* __restrict__ grads, T K, T* __restrict__ E, T* __restrict__ q_grads,
     T* __restrict__ gX, T* __restrict__ gY, T* __restrict__ gZ)
 {
     typedef typename Fast<T>::vec4 vec4;
-    constexpr int kOwn = kMediumMaxAtoms / 64;      // atoms per lane
+    static_assert(kMediumMaxAtoms == 256, "one atom per thread of a 256-thread workgroup");
     __shared__ ChargeTile<T, kGrad> S;
-    const int lane = threadIdx.x;
-    const T rc = static_cast<T>(kR_Rc_f), pi_rc = static_cast<T>(kPi / static_cast<double>(kR_Rc_f));
+    const int i = threadIdx.x, lane = i & 63, wave = uniform(i >> 6);
     for (int mol = blockIdx.x; mol < n_mols; mol += gridDim.x) {
         const int n = uniform(MACs[mol]);
         if (n <= kSmallMaxAtoms || n > kMediumMaxAtoms) continue;
         const int off = uniform(MOs[mol]);
-        vec4 own[kOwn];
-        T fx[kOwn], fy[kOwn], fz[kOwn], dq[kOwn];
-#pragma unroll
-        for (int k = 0; k < kOwn; ++k) {
-            const int i = lane + 64 * k;
-            own[k] = Fast<T>::make4(T(0), T(0), T(0), T(0));
-            fx[k] = fy[k] = fz[k] = dq[k] = T(0);
-            if (i < n) {
-                own[k] = Fast<T>::make4(X[off + i], Y[off + i], Z[off + i], Q[off + i]);
-                S.in[i] = own[k];
-                if constexpr (kGrad) S.acc[i] = Fast<T>::make4(T(0), T(0), T(0), T(0));
-            }
+        const bool have = i < n;
+        vec4 own = Fast<T>::make4(T(0), T(0), T(0), T(0));
+        if (have) {
+            own = Fast<T>::make4(X[off + i], Y[off + i], Z[off + i], Q[off + i]);
+            S.in[i] = own;
         }
-        wave_lds_fence();
+        if constexpr (kGrad) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) S.acc[w][i] = Fast<T>::make4(T(0), T(0), T(0), T(0));
+        }
+        __syncthreads();
         const int half = (n - 1) >> 1;
-        const int rounds = half + (((n & 1) == 0) ? 1 : 0);
-        T e_acc = T(0);
+        const int rounds = (wave * 64 < n) ? half + (((n & 1) == 0) ? 1 : 0) : 0;
+        T fx = T(0), fy = T(0), fz = T(0), dq = T(0), e_acc = T(0);
         for (int d = 1; d <= rounds; ++d) {
-#pragma unroll
-            for (int k = 0; k < kOwn; ++k) {
-                const int i = lane + 64 * k;
-                const bool act = (i < n) && (d <= half || i < (n >> 1));     // the half round: the lower half only
-                int j = i + d;
-                j -= (j >= n) ? n : 0;
-                const vec4 aj = S.in[act ? j : 0];
-                const T dx = act ? own[k].x - aj.x : T(1), dy = act ? own[k].y - aj.y : T(0), dz = act ? own[k].z - aj.z : T(0);
-                T u, du;
-                pair_terms<T, kDamped>(dx, dy, dz, pi_rc, rc, u, du);
-                if constexpr (!kGrad) {
-                    e_acc += act ? own[k].w * aj.w * u : T(0);
-                } else {
-                    if (act) {
-                        dq[k] = fma(aj.w, u, dq[k]);
-                        const T wq = own[k].w * aj.w * du;       // q_i q_j d/dr[(1-f_C)/r] / r
-                        fx[k] = fma(wq, dx, fx[k]);
-                        fy[k] = fma(wq, dy, fy[k]);
-                        fz[k] = fma(wq, dz, fz[k]);
-                        vec4 pa = S.acc[j];                      // distinct j across the lanes of this step
-                        pa.x = fma(-wq, dx, pa.x);
-                        pa.y = fma(-wq, dy, pa.y);
-                        pa.z = fma(-wq, dz, pa.z);
-                        pa.w = fma(own[k].w, u, pa.w);
-                        S.acc[j] = pa;
-                    }
-                    wave_lds_fence();                            // the next step may touch slots written here
+            const bool act = have && (d <= half || i < (n >> 1));     // the half round: the lower half only
+            int j = i + d;
+            j -= (j >= n) ? n : 0;
+            const vec4 aj = S.in[act ? j : 0];
+            const T dx = act ? own.x - aj.x : T(1), dy = act ? own.y - aj.y : T(0), dz = act ? own.z - aj.z : T(0);
+            T u, du;
+            pair_terms<T, kDamped>(dx, dy, dz, u, du);
+            const T qq = act ? own.w * aj.w : T(0);
+            e_acc = fma(qq, u, e_acc);
+            if constexpr (kGrad) {
+                if (act) {
+                    dq = fma(aj.w, u, dq);
+                    const T wq = qq * du;                    // q_i q_j d/dr[(1-f_C)/r] / r
+                    fx = fma(wq, dx, fx);
+                    fy = fma(wq, dy, fy);
+                    fz = fma(wq, dz, fz);
+                    vec4 pa = S.acc[wave][j];                // distinct j across the lanes of this wavefront
+                    pa.x = fma(-wq, dx, pa.x);
+                    pa.y = fma(-wq, dy, pa.y);
+                    pa.z = fma(-wq, dz, pa.z);
+                    pa.w = fma(own.w, u, pa.w);
+                    S.acc[wave][j] = pa;
                 }
+                wave_lds_fence();                            // the next round may touch slots written here
             }
         }
-        if constexpr (!kGrad) {
+        if (!kGrad || E) {
             e_acc = wave_sum(e_acc);
-            if (lane == 0) E[mol] = K * e_acc;
-        } else {
-            const T gK = grads[mol] * K;
-#pragma unroll
-            for (int k = 0; k < kOwn; ++k) {
-                const int i = lane + 64 * k;
-                if (i < n) {
-                    const vec4 pa = S.acc[i];
-                    if (q_grads) q_grads[off + i] = gK * (dq[k] + pa.w);
-                    if (gX) {
-                        // the force sums carry q_i already (wq = q_i q_j ...)
-                        gX[off + i] = gK * (fx[k] + pa.x);
-                        gY[off + i] = gK * (fy[k] + pa.y);
-                        gZ[off + i] = gK * (fz[k] + pa.z);
-                    }
+            if (lane == 0) S.wpart[wave] = e_acc;
+        }
+        __syncthreads();
+        if ((!kGrad || E) && i == 0) E[mol] = K * ((S.wpart[0] + S.wpart[1]) + (S.wpart[2] + S.wpart[3]));
+        if constexpr (kGrad) {
+            if (have) {
+                const T gK = grads[mol] * K;
+                const vec4 p0 = S.acc[0][i], p1 = S.acc[1][i], p2 = S.acc[2][i], p3 = S.acc[3][i];
+                if (q_grads) q_grads[off + i] = gK * (dq + ((p0.w + p1.w) + (p2.w + p3.w)));
+                if (gX) {
+                    // the force sums carry q_i already (wq = q_i q_j ...)
+                    gX[off + i] = gK * (fx + ((p0.x + p1.x) + (p2.x + p3.x)));
+                    gY[off + i] = gK * (fy + ((p0.y + p1.y) + (p2.y + p3.y)));
+                    gZ[off + i] = gK * (fz + ((p0.z + p1.z) + (p2.z + p3.z)));
                 }
             }
         }
-        wave_lds_fence();        // the next molecule reuses the tile
+        __syncthreads();         // the next molecule reuses the tile
     }
 }
 
@@ -232,7 +303,7 @@ __global__ __launch_bounds__(64) void charge_tile_kernel(
 // of a block of 256 and sums over every partner j (each pair is evaluated from both ends: no exchange between threads, and
 // every per-atom output is written once, by its owner); the workgroups of a grid column (blockIdx.y) share a molecule's
 // blocks.  The energy is half the sum over atoms of q_i times the atom's sum, added to E[mol] (zeroed by
-// charge_energy_kernel, which runs before on the same stream) by one floating-point atomic per workgroup and block: its
+// charge_energy_kernel or charge_grad_kernel, which runs before on the same stream) by one floating-point atomic per workgroup and block: its
 // last bits depend on the order of those additions.
 template <typename T, bool kDamped, bool kGrad>
 __global__ __launch_bounds__(256) void charge_large_kernel(
@@ -246,7 +317,6 @@ __global__ __launch_bounds__(256) void charge_large_kernel(
     __shared__ T wpart[4];
     __shared__ unsigned long long want[4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const T rc = static_cast<T>(kR_Rc_f), pi_rc = static_cast<T>(kPi / static_cast<double>(kR_Rc_f));
     for_each_molecule_in_range(MACs, n_mols, kMediumMaxAtoms + 1, INT32_MAX, want, nullptr, nullptr, [&](int mol) {
         const int n = uniform(MACs[mol]);
         const int off = uniform(MOs[mol]);
@@ -269,7 +339,7 @@ __global__ __launch_bounds__(256) void charge_large_kernel(
                     const vec4 aj = tile[t];                   // the same address in every lane
                     const T dx = xi - aj.x, dy = yi - aj.y, dz = zi - aj.z;
                     T u, du;
-                    pair_terms<T, kDamped>(dx, dy, dz, pi_rc, rc, u, du);      // zero for the atom itself (r = 0)
+                    pair_terms<T, kDamped>(dx, dy, dz, u, du);      // zero for the atom itself (r = 0)
                     su = fma(aj.w, u, su);
                     if constexpr (kGrad) {
                         const T w = aj.w * du;
@@ -279,13 +349,14 @@ __global__ __launch_bounds__(256) void charge_large_kernel(
                     }
                 }
             }
-            if constexpr (!kGrad) {
+            if (E) {                                           // (the same for every thread)
                 const T part = wave_sum(have ? qi * su : T(0));
                 __syncthreads();                               // wpart is free
                 if (lane == 0) wpart[wave] = part;
                 __syncthreads();
                 if (tid == 0) atomicAdd(&E[mol], T(0.5) * K * (wpart[0] + wpart[1] + wpart[2] + wpart[3]));
-            } else if (have) {
+            }
+            if (kGrad && have) {
                 const T gK = grads[mol] * K;
                 if (q_grads) q_grads[off + i] = gK * su;
                 if (gX) {
@@ -319,13 +390,13 @@ hipError_t launch_charge_energy(const T* X, const T* Y, const T* Z, const T* Q, 
     const unsigned tile_blocks = static_cast<unsigned>(n_mols < 8192 ? n_mols : 8192);
     if (damped) {
         charge_energy_kernel<T, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, K, E);
-        charge_tile_kernel<T, true, false><<<dim3(tile_blocks), dim3(64), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, nullptr, K, E,
+        charge_tile_kernel<T, true, false><<<dim3(tile_blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, nullptr, K, E,
                                                                                    nullptr, nullptr, nullptr, nullptr);
         charge_large_kernel<T, true, false><<<charge_large_grid(n_mols), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, nullptr, K,
                                                                                              E, nullptr, nullptr, nullptr, nullptr);
     } else {
         charge_energy_kernel<T, false><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, K, E);
-        charge_tile_kernel<T, false, false><<<dim3(tile_blocks), dim3(64), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, nullptr, K, E,
+        charge_tile_kernel<T, false, false><<<dim3(tile_blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, nullptr, K, E,
                                                                                     nullptr, nullptr, nullptr, nullptr);
         charge_large_kernel<T, false, false><<<charge_large_grid(n_mols), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, nullptr, K,
                                                                                               E, nullptr, nullptr, nullptr, nullptr);
@@ -336,30 +407,30 @@ hipError_t launch_charge_energy(const T* X, const T* Y, const T* Z, const T* Q, 
 template <typename T>
 hipError_t launch_charge_grad(const T* X, const T* Y, const T* Z, const T* Q, const int32_t* MOs,
                               const int32_t* MACs, int32_t n_mols, const T* grads, bool damped, T K, T* q_grads,
-                              T* gX, T* gY, T* gZ, hipStream_t stream)
+                              T* gX, T* gY, T* gZ, T* E, hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
     const unsigned blocks = (static_cast<unsigned>(n_mols) + 3u) / 4u;
     const unsigned tile_blocks = static_cast<unsigned>(n_mols < 8192 ? n_mols : 8192);
     if (damped) {
-        charge_grad_kernel<T, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, q_grads, gX, gY, gZ);
-        charge_tile_kernel<T, true, true><<<dim3(tile_blocks), dim3(64), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, nullptr,
+        charge_grad_kernel<T, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, q_grads, gX, gY, gZ, E);
+        charge_tile_kernel<T, true, true><<<dim3(tile_blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, E,
                                                                                   q_grads, gX, gY, gZ);
         charge_large_kernel<T, true, true><<<charge_large_grid(n_mols), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K,
-                                                                                            nullptr, q_grads, gX, gY, gZ);
+                                                                                            E, q_grads, gX, gY, gZ);
     } else {
-        charge_grad_kernel<T, false><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, q_grads, gX, gY, gZ);
-        charge_tile_kernel<T, false, true><<<dim3(tile_blocks), dim3(64), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, nullptr,
+        charge_grad_kernel<T, false><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, q_grads, gX, gY, gZ, E);
+        charge_tile_kernel<T, false, true><<<dim3(tile_blocks), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K, E,
                                                                                    q_grads, gX, gY, gZ);
         charge_large_kernel<T, false, true><<<charge_large_grid(n_mols), dim3(256), 0, stream>>>(X, Y, Z, Q, MOs, MACs, n_mols, grads, K,
-                                                                                             nullptr, q_grads, gX, gY, gZ);
+                                                                                             E, q_grads, gX, gY, gZ);
     }
     return hipGetLastError();
 }
 
 template hipError_t launch_charge_energy<float>(const float*, const float*, const float*, const float*, const int32_t*, const int32_t*, int32_t, bool, float, float*, hipStream_t);
 template hipError_t launch_charge_energy<double>(const double*, const double*, const double*, const double*, const int32_t*, const int32_t*, int32_t, bool, double, double*, hipStream_t);
-template hipError_t launch_charge_grad<float>(const float*, const float*, const float*, const float*, const int32_t*, const int32_t*, int32_t, const float*, bool, float, float*, float*, float*, float*, hipStream_t);
-template hipError_t launch_charge_grad<double>(const double*, const double*, const double*, const double*, const int32_t*, const int32_t*, int32_t, const double*, bool, double, double*, double*, double*, double*, hipStream_t);
+template hipError_t launch_charge_grad<float>(const float*, const float*, const float*, const float*, const int32_t*, const int32_t*, int32_t, const float*, bool, float, float*, float*, float*, float*, float*, hipStream_t);
+template hipError_t launch_charge_grad<double>(const double*, const double*, const double*, const double*, const int32_t*, const int32_t*, int32_t, const double*, bool, double, double*, double*, double*, double*, double*, hipStream_t);
 
 }  // namespace khan

@@ -147,7 +147,7 @@ hipError_t launch_charge_energy(const T* X, const T* Y, const T* Z, const T* Q, 
 template <typename T>
 hipError_t launch_charge_grad(const T* X, const T* Y, const T* Z, const T* Q, const int32_t* MOs,
                               const int32_t* MACs, int32_t n_mols, const T* grads, bool damped, T K, T* q_grads,
-                              T* gX, T* gY, T* gZ, hipStream_t stream);
+                              T* gX, T* gY, T* gZ, T* E, hipStream_t stream);     // E (may be null): the energies as well
 
 // ---- wavefront helpers (64 lanes) ----
 __device__ __forceinline__ unsigned long long wave_ballot(bool p) { return __ballot(p); }

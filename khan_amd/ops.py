@@ -262,6 +262,25 @@ def ani_charge_grad_xyz(xs, ys, zs, qs, mos, macs, grads):
     return qg, gx, gy, gz
 
 
+def ani_charge_all(xs, ys, zs, qs, mos, macs, grads):
+    """`ani_charge` and `ani_charge_grad_xyz` in one pass over the pairs
+    -> (charge_energies, q_grads, x_grads, y_grads, z_grads); the energies are not multiplied by `grads`."""
+    lib = _lib.load()
+    dt, n = _check_charge(xs, ys, zs, qs, mos, macs)
+    grads = _dev(grads, dt, "grads")
+    if grads.numel() != mos.numel():
+        raise ValueError("grads must have one element per molecule")
+    e = torch.zeros(mos.numel(), dtype=dt, device=xs.device)
+    qg = torch.zeros(n, dtype=dt, device=xs.device)
+    gx = torch.zeros(n, dtype=dt, device=xs.device)
+    gy = torch.zeros_like(gx)
+    gz = torch.zeros_like(gx)
+    fn = getattr(lib, "khan_ani_charge_all_" + _SUFFIX[dt])
+    _lib.check(fn(_p(xs), _p(ys), _p(zs), _p(qs), _p(mos), _p(macs), mos.numel(), _p(grads), _p(e), _p(qg),
+                  _p(gx), _p(gy), _p(gz), _stream()))
+    return e, qg, gx, gy, gz
+
+
 def mol_energy(type_outputs, atom_types, sis, mos, macs):
     """Per-molecule sums of the four per-type output vectors (`type_outputs[t]` is [acs[t]], float32 or float64; atom
     g's value is type_outputs[as[g]][sis[g]]) -> [n_mols]: the reference's gather to atom order + segment_sum by

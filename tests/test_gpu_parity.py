@@ -582,6 +582,11 @@ def test_charges(ops, kind, n_mols):
         assert np.array_equal(host(qg), dq)
         dxyz = host(torch.stack([gx, gy, gz], dim=1))
         assert_close("charge dE/dxyz %s" % ndt.__name__, dxyz, dx64, rtol, 0.0, scale=mol_scale(dx64, b.MOs, b.MACs))
+        # energy and both gradients from one pass over the pairs: the same gradients bit for bit, the energy (summed
+        # there as half the sum of q_i dE/dq_i) against the oracle
+        ea, qa, xa, ya, za = ops.ani_charge_all(X, Y, Z, Q, mos, macs, G)
+        assert_close("charge energy from the one-pass call %s" % ndt.__name__, host(ea), E64, rtol, 0.0, scale=Eabs)
+        assert torch.equal(qa, qg) and torch.equal(xa, gx) and torch.equal(ya, gy) and torch.equal(za, gz)
         # Euler: E is bilinear in q, so E = 1/2 sum_i q_i dE/dq_i (with unit upstream gradient)
         ones = torch.ones(n_mols, dtype=tdt, device="cuda:0")
         dq1 = host(ops.ani_charge_grad(X, Y, Z, Q, mos, macs, ones)).astype(np.float64)
