@@ -36,6 +36,7 @@ _SIGNATURES = {
     "khan_feature_size": (ctypes.c_int32, []),
     "khan_status_string": (ctypes.c_char_p, [ctypes.c_int]),
     "khan_last_hip_error": (ctypes.c_char_p, []),
+    "khan_set_reproducible_gradients": (ctypes.c_int, [ctypes.c_int]),
     "khan_get_parameters": (None, [ctypes.POINTER(ctypes.c_float)] * 4),
     "khan_mol_offsets": (ctypes.c_int, [_ptr, ctypes.c_int64, ctypes.c_int32, _ptr, _ptr, _ptr]),
     "khan_ani_sort": (ctypes.c_int, [_ptr, ctypes.c_int64, _ptr, _ptr, _ptr, _ptr]),

@@ -35,19 +35,38 @@ constexpr int kTypeShift = 28;     // large molecules: a radial queue entry is a
 // double 23 % faster than at one).
 template <typename T> constexpr int kMedBwdCentres = 4;
 
-template <typename T, bool kLarge = false>
+// Where a molecule's forces are summed.
+// kLocal = false: hardware atomics on the output arrays (zeroed by the workgroup first).  The fastest form, and the
+// only one for molecules of more than 256 atoms, which several workgroups share; the order of the additions, and with
+// it the last bits of the gradients, varies from run to run, and the output arrays must be in memory that supports
+// the atomics (ordinary device allocations).
+// kLocal = true (up to 256 atoms, on request: khan_set_reproducible_gradients): in LDS, one array per wavefront, by
+// plain read-add-write -- every instruction that adds is arranged so that its lanes hit distinct atoms -- the four
+// arrays added up in a fixed order at the end and every gradient stored once: no atomics, no pre-zeroed output, and,
+// with the centres dealt to the wavefronts by their position, the same result bit for bit on every run.  Each radial
+// pair is then evaluated once and pulls on both its atoms (with atomics it is evaluated from both ends, because
+// per-pair atomic adds to the partners cost more than the arithmetic they save).  The arrays take 12 KB (float), which
+// leaves three workgroups per CU instead of four: measured 9 % slower on dense boxes (0.90 -> 0.98 ms), with
+// the kernel's HBM traffic down from 2.14 to 1.07 times its algorithmic bytes.
+template <typename T, bool kOn> struct ForceLds {};
+template <typename T> struct ForceLds<T, true> {
+    T f[4][3][kMediumMaxAtoms];            // [wavefront][component][sorted position]
+};
+
+template <typename T, bool kLarge = false, bool kLocal = false>
 struct __align__(16) MedBwdShared {
+    ForceLds<T, kLocal> force;
     typename Fast<T>::vec4 atom[kMediumMaxAtoms];   // x, y, z, type (sorted order)
-    unsigned row_lo[kMediumMaxAtoms];      // address of the atom's upstream row
-    unsigned row_hi[kMediumMaxAtoms];
+    int row[kMediumMaxAtoms];              // the atom's row inside its type's bucket (its scatter index)
     unsigned short orig[kMediumMaxAtoms];  // sorted position -> index inside the molecule
+    unsigned short where[kMediumMaxAtoms]; // index inside the molecule -> sorted position
     int wcount[4][4];                      // atoms of each type held by each wavefront before the sort
     int next;                              // next centre (sorted position) to hand out
 };
 // above 256 atoms the sorted atoms are in device memory (aev_large.h); the list entries' sorted positions no
 // longer fit a byte and are kept here, one array per wavefront (the pool's byte array then holds the types)
 template <typename T>
-struct __align__(16) MedBwdShared<T, true> {
+struct __align__(16) MedBwdShared<T, true, false> {
     int pos[4][64];
     int next;                              // centres handed out so far by this workgroup
 };
@@ -55,8 +74,9 @@ struct __align__(16) MedBwdShared<T, true> {
 // With kLarge the kernel takes the molecules of more than 256 atoms: the atoms come type-sorted from `sorted`, the
 // workgroups of one grid column (blockIdx.y = 0 .. gridDim.y - 1) share a molecule's centres, and the gradients were
 // zeroed by the kernel that sorted the atoms.
-template <typename T, bool kLarge = false>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 4 : 2, sizeof(T) == 4 ? 4 : 2)))
+template <typename T, bool kLarge = false, bool kLocal = false>
+__global__ __launch_bounds__(256)
+__attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? (kLocal ? 3 : 4) : (kLocal ? 1 : 2), sizeof(T) == 4 ? (kLocal ? 3 : 4) : (kLocal ? 1 : 2))))
 void aev_bwd_medium_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
@@ -66,7 +86,8 @@ void aev_bwd_medium_kernel(
 {
     typedef typename Fast<T>::vec4 vec4;
     typedef typename std::conditional<kLarge, int, unsigned short>::type idx_t;     // a sorted position in the radial queue
-    __shared__ MedBwdShared<T, kLarge> M;
+    static_assert(!(kLarge && kLocal), "forces in LDS: molecules of up to 256 atoms only");
+    __shared__ MedBwdShared<T, kLarge, kLocal> M;
     constexpr int kMB = kMedBwdCentres<T>;
     __shared__ BwdPool<T, kMB> pools[4];
     const int tid = threadIdx.x;
@@ -92,16 +113,24 @@ void aev_bwd_medium_kernel(
         const bool have = tid < n;
         T x = T(0), y = T(0), z = T(0);
         int type = 0;
-        unsigned long long rowbits = 0;
+        int sis = 0;
         if (have) {
             x = X[off + tid];
             y = Y[off + tid];
             z = Z[off + tid];
             type = fold_type(A[off + tid]);
-            rowbits = reinterpret_cast<unsigned long long>(gin.p[type] + static_cast<size_t>(SIs[off + tid]) * kFeats);
-            gX[off + tid] = T(0);
-            gY[off + tid] = T(0);
-            gZ[off + tid] = T(0);
+            sis = SIs[off + tid];
+            if constexpr (!kLocal) {
+                gX[off + tid] = T(0);
+                gY[off + tid] = T(0);
+                gZ[off + tid] = T(0);
+            }
+        }
+        if constexpr (kLocal) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w)
+#pragma unroll
+                for (int k = 0; k < 3; ++k) M.force.f[w][k][tid] = T(0);
         }
         unsigned long long tmask[4];
 #pragma unroll
@@ -124,9 +153,9 @@ void aev_bwd_medium_kernel(
             const unsigned long long mine = type == 0 ? tmask[0] : type == 1 ? tmask[1] : type == 2 ? tmask[2] : tmask[3];
             const int dest = sel4(type, tbase[0], tbase[1], tbase[2], tbase[3]) + before + popc64(mine & lt_mask);
             M.atom[dest] = Fast<T>::make4(x, y, z, static_cast<T>(type));
-            M.row_lo[dest] = static_cast<unsigned>(rowbits & 0xffffffffull);
-            M.row_hi[dest] = static_cast<unsigned>(rowbits >> 32);
+            M.row[dest] = sis;
             M.orig[dest] = static_cast<unsigned short>(tid);
+            M.where[tid] = static_cast<unsigned short>(dest);
         }
         __syncthreads();       // sorted arrays complete; the zeroed outputs are visible before any atomic add
         tb1 = tbase[1];
@@ -139,16 +168,16 @@ void aev_bwd_medium_kernel(
             else return M.atom[sorted_idx];
         };
         auto row_bits_of = [&](int sorted_idx, int type) -> unsigned long long {     // per-lane index, and that atom's type
-            if constexpr (kLarge) {
-                const T* const bucket = type == 0 ? gin.p[0] : type == 1 ? gin.p[1] : type == 2 ? gin.p[2] : gin.p[3];
-                return reinterpret_cast<unsigned long long>(bucket + static_cast<size_t>(sorted.aux[off + sorted_idx].y) * kFeats);
-            } else {
-                return (static_cast<unsigned long long>(M.row_hi[sorted_idx]) << 32) | M.row_lo[sorted_idx];
-            }
+            const T* const bucket = type == 0 ? gin.p[0] : type == 1 ? gin.p[1] : type == 2 ? gin.p[2] : gin.p[3];
+            int sis;
+            if constexpr (kLarge) sis = sorted.aux[off + sorted_idx].y;
+            else sis = M.row[sorted_idx];
+            return reinterpret_cast<unsigned long long>(bucket + static_cast<size_t>(sis) * kFeats);
         };
         auto row_of = [&](int sorted_idx) -> const T* {            // wave-uniform index
-            int type = 0;
+            int type;
             if constexpr (kLarge) type = static_cast<int>(sorted.atom[off + sorted_idx].w);
+            else type = type_of(sorted_idx);
             const unsigned long long bits = row_bits_of(sorted_idx, type);
             const unsigned lo = static_cast<unsigned>(uniform(static_cast<int>(bits & 0xffffffffull)));
             const unsigned hi = static_cast<unsigned>(uniform(static_cast<int>(bits >> 32)));
@@ -158,11 +187,18 @@ void aev_bwd_medium_kernel(
             if constexpr (kLarge) return sorted.aux[off + sorted_idx].x;
             else return M.orig[sorted_idx];
         };
-        auto add_force = [&](int sorted_idx, T fx, T fy, T fz) {   // per-lane target
-            const int g = off + orig_of(sorted_idx);
-            atomicAdd(&gX[g], fx);
-            atomicAdd(&gY[g], fy);
-            atomicAdd(&gZ[g], fz);
+        // per-lane target; with forces in LDS the caller sees to it that the lanes of one call hit distinct atoms
+        auto add_force = [&](int sorted_idx, T fx, T fy, T fz) {
+            if constexpr (kLocal) {
+                M.force.f[wave][0][sorted_idx] += fx;
+                M.force.f[wave][1][sorted_idx] += fy;
+                M.force.f[wave][2][sorted_idx] += fz;
+            } else {
+                const int g = off + orig_of(sorted_idx);
+                atomicAdd(&gX[g], fx);
+                atomicAdd(&gY[g], fy);
+                atomicAdd(&gZ[g], fz);
+            }
         };
 
         // Radial pairs are queued and worked off 64 at a time: only about an eighth of the (centre, partner)
@@ -175,10 +211,10 @@ void aev_bwd_medium_kernel(
         int qn = 0;
         auto radial_work_off = [&](int count) {      // entries 0..count-1, count <= 64
             T fx = T(0), fy = T(0), fz = T(0);
-            int c = -1;
+            int c = -1, j = 0;
             if (lane < count) {
                 const vec4 e = q_d[lane];
-                int j = q_j[lane];
+                j = q_j[lane];
                 c = q_c[lane];
                 int tj, tc;
                 if constexpr (kLarge) {            // the queue carries the types in the four high bits
@@ -193,7 +229,9 @@ void aev_bwd_medium_kernel(
                 const T* grow_c = reinterpret_cast<const T*>(row_bits_of(c, tc));
                 const T* grow_j = reinterpret_cast<const T*>(row_bits_of(j, tj));
                 const T inv = Fast<T>::rcp(e.w);
-                // the pair's pull on the centre from both rows; the partner gets its share when it is the centre
+                // the pair's pull on the centre from both rows.  With forces in LDS the pair is queued once (by its
+                // centre of lower sorted position) and the partner gets minus this below; otherwise the partner gets
+                // its share when it is the centre
                 const T sc = bwd_radial_pair_both<T>(grow_c, tj, grow_j, tc, e.w, inv);
                 fx = sc * e.x;
                 fy = sc * e.y;
@@ -201,7 +239,7 @@ void aev_bwd_medium_kernel(
             }
             // The pairs of one centre are a run of lanes (the queue is filled centre after centre): one add-scan
             // per component, and the last lane of every run adds the difference of two prefix values to its
-            // centre -- one atomic per centre and component, issued for all centres of the step at once.
+            // centre -- one add per centre and component, issued for all centres of the step at once.
             const T px = group_sum_to_last_lane(fx, 6), py = group_sum_to_last_lane(fy, 6), pz = group_sum_to_last_lane(fz, 6);
             const int c_prev = __builtin_amdgcn_ds_bpermute(max(lane - 1, 0) << 2, c);
             const int c_next = __builtin_amdgcn_ds_bpermute(min(lane + 1, 63) << 2, c);
@@ -216,6 +254,18 @@ void aev_bwd_medium_kernel(
             if (run_end) {
                 const bool whole = first == 0;
                 add_force(c, whole ? px : px - qx, whole ? py : py - qy, whole ? pz : pz - qz);
+            }
+            if constexpr (kLocal) {
+                // the partners: run after run, because the partners of one centre are distinct atoms and those of two
+                // centres need not be
+                wave_lds_fence();
+                for (unsigned long long rs = starts; rs;) {
+                    const int b0 = lowest_bit(rs);
+                    rs &= rs - 1;
+                    const int b1 = rs ? lowest_bit(rs) : count;
+                    if (lane >= b0 && lane < b1) add_force(j, -fx, -fy, -fz);
+                    wave_lds_fence();
+                }
             }
         };
         auto radial_drain = [&]() {
@@ -263,6 +313,7 @@ void aev_bwd_medium_kernel(
             qn = rest;
         };
 
+        int dealt = 0;             // (forces in LDS) centres this wavefront has taken: it takes every fourth, by position
         int pending = -1;          // a centre that was drawn but did not fit the previous batch
         int scanned = -1;          // (large molecules) the centre whose radial pairs were queued last
         for (;;) {
@@ -274,10 +325,14 @@ void aev_bwd_medium_kernel(
                 int c = pending;
                 pending = -1;
                 if (c < 0) {
-                    int drawn = 0;
-                    if (lane == 0) drawn = atomicAdd(&M.next, 1);
-                    c = uniform(drawn);
-                    if constexpr (kLarge) c = static_cast<int>(blockIdx.y) + static_cast<int>(gridDim.y) * c;
+                    if constexpr (kLocal) {
+                        c = wave + 4 * dealt++;
+                    } else {
+                        int drawn = 0;
+                        if (lane == 0) drawn = atomicAdd(&M.next, 1);
+                        c = uniform(drawn);
+                        if constexpr (kLarge) c = static_cast<int>(blockIdx.y) + static_cast<int>(gridDim.y) * c;
+                    }
                 }
                 if (c >= n) break;
                 const vec4 ai = atom_at(c);
@@ -364,7 +419,8 @@ void aev_bwd_medium_kernel(
                         dz[ch] = ai.z - aj.z;
                         r[ch] = Fast<T>::sqrt_rn(dx[ch] * dx[ch] + dy[ch] * dy[ch] + dz[ch] * dz[ch]);
                         const bool valid = (j < n) && (j != c);
-                        mR[ch] = wave_ballot(!kSkipRadial && valid && (r[ch] < kR_Rc_f) && (r[ch] > T(0)));     // r = 0: a coincident atom exerts no force
+                        // r = 0: a coincident atom exerts no force; with forces in LDS a pair is queued by its lower centre only
+                        mR[ch] = wave_ballot(!kSkipRadial && valid && (r[ch] < kR_Rc_f) && (r[ch] > T(0)) && (!kLocal || j > c));
                         mA[ch] = wave_ballot(valid && (r[ch] < kA_Rc_f) && (r[ch] > T(0)));
                         m_c += popc64(mA[ch]);
                     }
@@ -417,11 +473,21 @@ void aev_bwd_medium_kernel(
                     radial_drain();                    // the routine uses the staging area as scratch
                     bwd_center_generic<T>(L, lane, X, Y, Z, A, off, n, i_orig, P.gst, row_of(c),
                                               [&](int atom, T fx, T fy, T fz) {
-                                                  atomicAdd(&gX[off + atom], fx);
-                                                  atomicAdd(&gY[off + atom], fy);
-                                                  atomicAdd(&gZ[off + atom], fz);
+                                                  if constexpr (kLocal) {
+                                                      // (lanes may meet on an atom here: LDS atomics, whose order within
+                                                      // an instruction is the hardware's)
+                                                      const int sp = M.where[atom];
+                                                      atomicAdd(&M.force.f[wave][0][sp], fx);
+                                                      atomicAdd(&M.force.f[wave][1][sp], fy);
+                                                      atomicAdd(&M.force.f[wave][2][sp], fz);
+                                                  } else {
+                                                      atomicAdd(&gX[off + atom], fx);
+                                                      atomicAdd(&gY[off + atom], fy);
+                                                      atomicAdd(&gZ[off + atom], fz);
+                                                  }
                                               },
                                               false);
+                    wave_lds_fence();
                     continue;
                 }
                 if (lane == nb) {
@@ -460,7 +526,14 @@ void aev_bwd_medium_kernel(
             const bool live = lane < total;       // from here on one lane per entry again
 
             // ------------------------------------------------ gather
-            if (live) {
+            if constexpr (kLocal) {
+                // centre after centre: the partners of one centre are distinct atoms
+                const int target = P.nbr_idx[live ? lane : 0];
+                for (int bb = 0; bb < nb; ++bb) {
+                    if (live && bs == bb) add_force(target, f.x, f.y, f.z);
+                    wave_lds_fence();
+                }
+            } else if (live) {
                 if constexpr (kLarge) add_force(M.pos[wave][lane], f.x, f.y, f.z);
                 else add_force(P.nbr_idx[lane], f.x, f.y, f.z);
             }
@@ -484,6 +557,15 @@ void aev_bwd_medium_kernel(
             }
             wave_lds_fence();
         }
+        if constexpr (kLocal) {
+            __syncthreads();  // every wavefront's forces are complete
+            if (tid < n) {
+                const int g = off + M.orig[tid];
+                gX[g] = (M.force.f[0][0][tid] + M.force.f[1][0][tid]) + (M.force.f[2][0][tid] + M.force.f[3][0][tid]);
+                gY[g] = (M.force.f[0][1][tid] + M.force.f[1][1][tid]) + (M.force.f[2][1][tid] + M.force.f[3][1][tid]);
+                gZ[g] = (M.force.f[0][2][tid] + M.force.f[1][2][tid]) + (M.force.f[2][2][tid] + M.force.f[3][2][tid]);
+            }
+        }
         __syncthreads();      // the next molecule reuses the sorted arrays
     });
 }
@@ -494,15 +576,20 @@ template <typename T>
 hipError_t launch_bwd_medium(const T* X, const T* Y, const T* Z, const int32_t* A,
                              const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
                              const int32_t* SIs, Buckets<const T> g, T* gX, T* gY,
-                             T* gZ, int min_atoms, const int32_t* order, bool walk_in_order, hipStream_t stream)
+                             T* gZ, int min_atoms, const int32_t* order, bool walk_in_order, bool reproducible,
+                             hipStream_t stream)
 {
     if (n_mols <= 0) return hipSuccess;
     // workgroups walk the molecules with the grid's stride and skip those of other sizes
     // (in float64 the working set lets one workgroup run per CU: a smaller grid costs less when it only skips)
     const int32_t cap = sizeof(T) == 4 ? 4096 : 1024;
     const unsigned blocks = static_cast<unsigned>(n_mols < cap ? n_mols : cap);
-    aev_bwd_medium_kernel<T><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ, min_atoms,
-                                                                  order, walk_in_order, SortedAtoms<T>{});
+    if (reproducible)
+        aev_bwd_medium_kernel<T, false, true><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ, min_atoms,
+                                                                                   order, walk_in_order, SortedAtoms<T>{});
+    else
+        aev_bwd_medium_kernel<T><<<dim3(blocks), dim3(256), 0, stream>>>(X, Y, Z, A, MOs, MACs, n_mols, SIs, g, gX, gY, gZ, min_atoms,
+                                                                      order, walk_in_order, SortedAtoms<T>{});
     return hipGetLastError();
 }
 
@@ -525,8 +612,8 @@ hipError_t launch_bwd_large(const T* X, const T* Y, const T* Z, const int32_t* A
     return hipGetLastError();
 }
 
-template hipError_t launch_bwd_medium<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const float>, float*, float*, float*, int, const int32_t*, bool, hipStream_t);
-template hipError_t launch_bwd_medium<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const double>, double*, double*, double*, int, const int32_t*, bool, hipStream_t);
+template hipError_t launch_bwd_medium<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const float>, float*, float*, float*, int, const int32_t*, bool, bool, hipStream_t);
+template hipError_t launch_bwd_medium<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const double>, double*, double*, double*, int, const int32_t*, bool, bool, hipStream_t);
 
 template hipError_t launch_bwd_large<float>(const float*, const float*, const float*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const float>, float*, float*, float*, const int32_t*, void*, int64_t, hipStream_t);
 template hipError_t launch_bwd_large<double>(const double*, const double*, const double*, const int32_t*, const int32_t*, const int32_t*, int32_t, const int32_t*, Buckets<const double>, double*, double*, double*, const int32_t*, void*, int64_t, hipStream_t);

@@ -1,4 +1,5 @@
 // extern "C" surface of libkhan_aev.so: argument checks and dispatch to the kernel launchers.
+#include <atomic>
 #include <cstdlib>
 #include <mutex>
 #include <string>
@@ -15,6 +16,9 @@ static __device__ __align__(256) int32_t scratch[KHAN_FEATURIZE_NOALLOC_MAX_MOLS
 namespace {
 
 thread_local std::string g_last_hip_error;
+
+// khan_set_reproducible_gradients: the one setting of the library (process-wide, read at every gradient call)
+std::atomic<int> g_reproducible{0};
 
 // Device address of `scratch` on the current device, looked up once per device with that device current.
 constexpr int kMaxDevices = 64;
@@ -234,7 +238,7 @@ int backward_dispatch(const T* xs, const T* ys, const T* zs, const int32_t* as, 
     // (the workgroup-per-molecule backward kernel measures slower when it walks the molecules in size order)
     if (st == KHAN_OK && cls.any(small_max + 1, khan::kMediumMaxAtoms))
         st = hip_status(khan::launch_bwd_medium<T>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
-                                                   small_max + 1, order, false, stream));
+                                                   small_max + 1, order, false, g_reproducible.load(std::memory_order_relaxed) != 0, stream));
     if (st == KHAN_OK && cls.any(0, small_max))
         st = hip_status(khan::launch_bwd_small<T>(xs, ys, zs, as, mos, macs, n_mols, sis, g, gx, gy, gz,
                                                   small_max, order, stream));
@@ -495,6 +499,11 @@ int khan_featurize_f64(const double* xs, const double* ys, const double* zs, con
                        khan_stream_t stream)
 {
     return featurize_impl<double>(xs, ys, zs, as, mos, macs, n_mols, sis, h, c, n, o, acs_host, stream);
+}
+
+int khan_set_reproducible_gradients(int on)
+{
+    return g_reproducible.exchange(on ? 1 : 0, std::memory_order_relaxed);
 }
 
 // khan_featurize_f32 without any allocation: the size order goes to the file-scope array above.

@@ -75,7 +75,8 @@ template <typename T>
 hipError_t launch_bwd_medium(const T* X, const T* Y, const T* Z, const int32_t* A,
                              const int32_t* MOs, const int32_t* MACs, int32_t n_mols,
                              const int32_t* SIs, Buckets<const T> g, T* gX, T* gY,
-                             T* gZ, int min_atoms, const int32_t* order, bool walk_in_order, hipStream_t stream);
+                             T* gZ, int min_atoms, const int32_t* order, bool walk_in_order, bool reproducible,
+                             hipStream_t stream);
 
 template <typename T>
 hipError_t launch_bwd_generic(const T* X, const T* Y, const T* Z, const int32_t* A,

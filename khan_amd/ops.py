@@ -85,6 +85,12 @@ def ani_sort(atomic_numbers):
 SIZE_ORDER_EXTRA = 520
 
 
+def set_reproducible_gradients(on):
+    """Process-wide: with True, `featurize_grad` sums the forces of molecules of up to 256 atoms in a fixed order (the
+    same bits on every run, no atomics) at some cost in speed; returns the previous setting."""
+    return bool(_lib.load().khan_set_reproducible_gradients(1 if on else 0))
+
+
 def size_order(macs):
     """-> int32[n_mols + 520]: the molecule indices by decreasing atom count and the per-size counts, to be
     passed as `order=` to featurize / featurize_grad / featurize_grad_inverse of the same batch (computed once

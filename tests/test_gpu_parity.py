@@ -706,6 +706,58 @@ def test_crowded_centres_take_the_fallback(ops):
     check_forward_backward(ops, c)
 
 
+
+def test_reproducible_gradients_setting(ops):
+    """khan_set_reproducible_gradients(1): the workgroup-per-molecule backward kernel sums a molecule's forces in LDS in
+    a fixed order instead of with hardware atomics.  Dense boxes (65..256 atoms), boxes of 40 and 60 atoms
+    (that kernel's in float32), small organic molecules and a ball with more than 64 angular partners per centre (its fallback inside the
+    kernel), in both precisions: against the float64 oracle at the usual tolerances, identical bits on repeated runs
+    (the outputs are fresh, uninitialised arrays every time: this form stores every gradient once and never reads
+    them), and, since the setting changes the order of the sums only, close to what the default gives."""
+    say("case: reproducible gradients (forces summed in LDS)")
+    rng = np.random.default_rng(77)
+    box = datagen.make_batch("boxes", 10, first_mol=100)
+    org = datagen.make_batch("organic", 400, first_mol=3000)
+    mols = []
+    for b in (box, org):
+        for m in range(b.n_mols):
+            sl = slice(b.MOs[m], b.MOs[m] + b.MACs[m])
+            mols.append((b.A[sl], np.stack([b.X[sl], b.Y[sl], b.Z[sl]], axis=1)))
+    mols.insert(3, (rng.integers(0, 4, 200), _packed_ball(rng, 200, 3.9, 0.85)))
+    for n_small in (40, 60):
+        mols.insert(5, (rng.integers(0, 4, n_small), _sparse_box(rng, n_small, 0.1, 0.9)))
+    A = np.concatenate([m[0] for m in mols]).astype(np.int32)
+    xyz = np.concatenate([m[1] for m in mols])
+    mi = np.concatenate([np.full(len(m[0]), k) for k, m in enumerate(mols)]).astype(np.int32)
+    c = Case(xyz[:, 0], xyz[:, 1], xyz[:, 2], A, mi, len(mols))
+    assert int((c.MACs > 64).sum()) >= 11 and int(((c.MACs > 32) & (c.MACs <= 64)).sum()) == 2, np.sort(c.MACs)[-20:]
+    macs, mos, sc, ga, ac = gpu_sort_offsets(ops, c)
+    acs = ac.cpu()
+    upb = c.upstream()
+    g64 = c.oracle_grad(upb)
+    S = mol_scale(g64, c.MOs, c.MACs)
+    Ad = dev(c.A)
+    previous = ops.set_reproducible_gradients(True)
+    try:
+        assert previous is False
+        for ndt, rtol, atol in ((np.float32, F32_RTOL, F32_ATOL), (np.float64, F64_RTOL, 0.0)):
+            X, Y, Z = dev(c.X, ndt), dev(c.Y, ndt), dev(c.Z, ndt)
+            gb = [dev(u, ndt) for u in upb]
+            runs = []
+            for k in range(3):
+                g = torch.stack(ops.featurize_grad(X, Y, Z, Ad, mos, macs, sc, acs, *gb), dim=1)
+                runs.append(g)
+                torch.zeros(1 << 22, device="cuda:0").sum()          # other work in between
+            assert_close("reproducible gradient %s vs f64 oracle" % ndt.__name__, host(runs[0]), g64, rtol, atol, scale=S)
+            assert torch.equal(runs[0], runs[1]) and torch.equal(runs[0], runs[2]), "gradients differ between runs"
+            assert ops.set_reproducible_gradients(False) is True
+            g_default = torch.stack(ops.featurize_grad(X, Y, Z, Ad, mos, macs, sc, acs, *gb), dim=1)
+            assert ops.set_reproducible_gradients(True) is False
+            assert_close("default gradient %s vs f64 oracle" % ndt.__name__, host(g_default), g64, rtol, atol, scale=S)
+            assert_close("reproducible vs default %s" % ndt.__name__, host(runs[0]), host(g_default).astype(np.float64), 4 * rtol, 4 * atol, scale=S)
+    finally:
+        ops.set_reproducible_gradients(False)
+
 def _sparse_box(rng, n, density, min_dist):
     """n points in a cube at the given number density, no two closer than min_dist (cell by cell, so that thousands
     of points take a moment and not minutes)."""
