@@ -373,16 +373,34 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB, kRadN
     }
 
     // ------------------------------------------------ segments without triples are zeros
-    // Each segment lane whose segment is empty clears its own 32 values: eight 16-byte stores per lane (or 32
-    // 4-byte ones if the row is not 16-byte aligned), for all centres of the batch at once.
-    if (lane < nb * kNumPairBlocks && cnt == 0) {
-        T* dst = reinterpret_cast<T*>((static_cast<unsigned long long>(seg_row_hi) << 32) | seg_row_lo);
-        if ((seg_row_lo & 15u) == 0u) {
-            constexpr int kPer = 16 / sizeof(T);
-#pragma unroll
-            for (int q = 0; q < kAngBlock / kPer; ++q) store_global16(dst + q * kPer);
-        } else {
-            for (int q = 0; q < kAngBlock; ++q) store_global(dst + q, T(0));
+    // The rows' addresses of the batch's empty segments are compacted into the (now free) table of row addresses, and
+    // the lanes clear them a line at a time: a segment's 32 values are 128 (float) or 256 (double) consecutive bytes,
+    // taken by 8 or 16 lanes with one 16-byte store each, so that one instruction writes 8 (4) whole segments and the
+    // memory system sees full lines.  (One segment per lane, eight 16-byte stores each, is the same bytes in eight
+    // times the write transactions, each a sixth of a line.)  Rows that are not 16-byte aligned: 4-byte stores.
+    {
+        const bool is_empty = lane < nb * kNumPairBlocks && cnt == 0;
+        const unsigned long long empties = wave_ballot(is_empty);
+        if (empties) {
+            const bool unaligned = wave_ballot(is_empty && (seg_row_lo & 15u) != 0u) != 0ull;
+            if (!unaligned) {
+                constexpr int kLanesPer = kAngBlock * static_cast<int>(sizeof(T)) / 16;      // lanes per segment: 8 or 16
+                constexpr int kPerStep = 64 / kLanesPer;
+                const int n_empty = popc64(empties);
+                if (is_empty) S.segrow[popc64(empties & lt_mask)] = (static_cast<unsigned long long>(seg_row_hi) << 32) | seg_row_lo;
+                wave_lds_fence();
+                for (int e0 = 0; e0 < n_empty; e0 += kPerStep) {
+                    const int e = e0 + lane / kLanesPer;
+                    if (e < n_empty) {
+                        char* dst = reinterpret_cast<char*>(S.segrow[e]) + (lane % kLanesPer) * 16;
+                        store_global16(dst);
+                    }
+                }
+                wave_lds_fence();
+            } else if (is_empty) {
+                T* dst = reinterpret_cast<T*>((static_cast<unsigned long long>(seg_row_hi) << 32) | seg_row_lo);
+                for (int q = 0; q < kAngBlock; ++q) store_global(dst + q, T(0));
+            }
         }
     }
 }

@@ -51,15 +51,16 @@ template <typename T> constexpr int kMedBwdCentres = 4;
 template <typename T, bool kOn> struct ForceLds {};
 template <typename T> struct ForceLds<T, true> {
     T f[4][3][kMediumMaxAtoms];            // [wavefront][component][sorted position]
+    unsigned short where[kMediumMaxAtoms]; // index inside the molecule -> sorted position
 };
 
 template <typename T, bool kLarge = false, bool kLocal = false>
 struct __align__(16) MedBwdShared {
     ForceLds<T, kLocal> force;
     typename Fast<T>::vec4 atom[kMediumMaxAtoms];   // x, y, z, type (sorted order)
-    int row[kMediumMaxAtoms];              // the atom's row inside its type's bucket (its scatter index)
+    unsigned row_lo[kMediumMaxAtoms];      // address of the atom's upstream row
+    unsigned row_hi[kMediumMaxAtoms];
     unsigned short orig[kMediumMaxAtoms];  // sorted position -> index inside the molecule
-    unsigned short where[kMediumMaxAtoms]; // index inside the molecule -> sorted position
     int wcount[4][4];                      // atoms of each type held by each wavefront before the sort
     int next;                              // next centre (sorted position) to hand out
 };
@@ -113,13 +114,13 @@ void aev_bwd_medium_kernel(
         const bool have = tid < n;
         T x = T(0), y = T(0), z = T(0);
         int type = 0;
-        int sis = 0;
+        unsigned long long rowbits = 0;
         if (have) {
             x = X[off + tid];
             y = Y[off + tid];
             z = Z[off + tid];
             type = fold_type(A[off + tid]);
-            sis = SIs[off + tid];
+            rowbits = reinterpret_cast<unsigned long long>(gin.p[type] + static_cast<size_t>(SIs[off + tid]) * kFeats);
             if constexpr (!kLocal) {
                 gX[off + tid] = T(0);
                 gY[off + tid] = T(0);
@@ -153,9 +154,10 @@ void aev_bwd_medium_kernel(
             const unsigned long long mine = type == 0 ? tmask[0] : type == 1 ? tmask[1] : type == 2 ? tmask[2] : tmask[3];
             const int dest = sel4(type, tbase[0], tbase[1], tbase[2], tbase[3]) + before + popc64(mine & lt_mask);
             M.atom[dest] = Fast<T>::make4(x, y, z, static_cast<T>(type));
-            M.row[dest] = sis;
+            M.row_lo[dest] = static_cast<unsigned>(rowbits & 0xffffffffull);
+            M.row_hi[dest] = static_cast<unsigned>(rowbits >> 32);
             M.orig[dest] = static_cast<unsigned short>(tid);
-            M.where[tid] = static_cast<unsigned short>(dest);
+            if constexpr (kLocal) M.force.where[tid] = static_cast<unsigned short>(dest);
         }
         __syncthreads();       // sorted arrays complete; the zeroed outputs are visible before any atomic add
         tb1 = tbase[1];
@@ -168,16 +170,16 @@ void aev_bwd_medium_kernel(
             else return M.atom[sorted_idx];
         };
         auto row_bits_of = [&](int sorted_idx, int type) -> unsigned long long {     // per-lane index, and that atom's type
-            const T* const bucket = type == 0 ? gin.p[0] : type == 1 ? gin.p[1] : type == 2 ? gin.p[2] : gin.p[3];
-            int sis;
-            if constexpr (kLarge) sis = sorted.aux[off + sorted_idx].y;
-            else sis = M.row[sorted_idx];
-            return reinterpret_cast<unsigned long long>(bucket + static_cast<size_t>(sis) * kFeats);
+            if constexpr (kLarge) {
+                const T* const bucket = type == 0 ? gin.p[0] : type == 1 ? gin.p[1] : type == 2 ? gin.p[2] : gin.p[3];
+                return reinterpret_cast<unsigned long long>(bucket + static_cast<size_t>(sorted.aux[off + sorted_idx].y) * kFeats);
+            } else {
+                return (static_cast<unsigned long long>(M.row_hi[sorted_idx]) << 32) | M.row_lo[sorted_idx];
+            }
         };
         auto row_of = [&](int sorted_idx) -> const T* {            // wave-uniform index
-            int type;
+            int type = 0;
             if constexpr (kLarge) type = static_cast<int>(sorted.atom[off + sorted_idx].w);
-            else type = type_of(sorted_idx);
             const unsigned long long bits = row_bits_of(sorted_idx, type);
             const unsigned lo = static_cast<unsigned>(uniform(static_cast<int>(bits & 0xffffffffull)));
             const unsigned hi = static_cast<unsigned>(uniform(static_cast<int>(bits >> 32)));
@@ -476,7 +478,7 @@ void aev_bwd_medium_kernel(
                                                   if constexpr (kLocal) {
                                                       // (lanes may meet on an atom here: LDS atomics, whose order within
                                                       // an instruction is the hardware's)
-                                                      const int sp = M.where[atom];
+                                                      const int sp = M.force.where[atom];
                                                       atomicAdd(&M.force.f[wave][0][sp], fx);
                                                       atomicAdd(&M.force.f[wave][1][sp], fy);
                                                       atomicAdd(&M.force.f[wave][2][sp], fz);
