@@ -45,7 +45,7 @@ struct __align__(16) BwdLds {
 
 // float: 4 wavefronts per SIMD (LDS 10.2 KB, 127 registers); double: 2 (LDS 20.4 KB, twice the registers)
 template <typename T>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 4 : 1, sizeof(T) == 4 ? 4 : 2)))
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 4 : 2, sizeof(T) == 4 ? 4 : 2)))
 void aev_bwd_small_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,

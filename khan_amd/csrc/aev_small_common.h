@@ -57,12 +57,14 @@ __device__ __forceinline__ double lane_push(int dest_lane, double v)
 typedef float __attribute__((address_space(1))) global_float;
 __device__ __forceinline__ void store_global(float* p, float v)
 {
-    *((global_float*)(p)) = v;
+    if constexpr (kSkipStores) asm volatile("" ::"v"(v), "v"(p));      // measurement build: the value is formed, not stored
+    else *((global_float*)(p)) = v;
 }
 typedef double __attribute__((address_space(1))) global_double;
 __device__ __forceinline__ void store_global(double* p, double v)
 {
-    *((global_double*)(p)) = v;
+    if constexpr (kSkipStores) asm volatile("" ::"v"(v), "v"(p));
+    else *((global_double*)(p)) = v;
 }
 // acc + a' * g, where a' is the value of `a` held by lane k of this lane's quad (k is a constant after unrolling).
 // The lane exchange is a modifier of the multiply-add, not an instruction of its own.  It reads `a` early: two
@@ -83,7 +85,8 @@ typedef float __attribute__((ext_vector_type(4))) zero_v4f;
 typedef zero_v4f __attribute__((address_space(1))) global_v4f_store;
 __device__ __forceinline__ void store_global16(void* p)
 {
-    *((global_v4f_store*)(p)) = zero_v4f{0.f, 0.f, 0.f, 0.f};
+    if constexpr (kSkipStores) asm volatile("" ::"v"(p));
+    else *((global_v4f_store*)(p)) = zero_v4f{0.f, 0.f, 0.f, 0.f};
 }
 // sum of the two half-waves, in every lane: swap the upper half of one copy with the lower half of
 // the other (one cross-lane VALU move, no LDS round trip), then add
@@ -289,21 +292,88 @@ template <> struct Fast<float> {
         cutoff_poly_grad(r * (1.0f / rc), 1.0f / rc, fc, dfc);
     }
 };
+// double-precision building blocks without library calls: the library's sqrt, division, cos and sin spend most of their
+// instructions on range reduction and special cases that cannot occur for distances of the order of an angstrom.
+// r = sqrt(x) and 1/r for x > 0: v_rsq_f64 is good to 5e-8; one coupled Goldschmidt step (g -> sqrt, h -> 1/(2 sqrt))
+// squares that, the fused residual x - g^2 is exact and brings g to half an ulp, and one Newton step on the reciprocal
+// of that g gives 1/r to an ulp (measured against long double on 2^20 arguments: 1.1e-16 and 2.1e-16).  x = 0 -> 0, 0.
+__device__ __forceinline__ void sqrt_and_rcp(double x0, double& r, double& inv)
+{
+    const double x = fmax(x0, 1e-300);
+    const double y = __builtin_amdgcn_rsq(x);
+    double g = x * y, h = 0.5 * y;
+    const double e = fma(-h, g, 0.5);
+    g = fma(g, e, g);
+    h = fma(h, e, h);
+    g = fma(fma(-g, g, x), h, g);
+    double v = h + h;
+    v = fma(v, fma(-g, v, 1.0), v);
+    r = x0 > 0.0 ? g : 0.0;
+    inv = x0 > 0.0 ? v : 0.0;
+}
+// 1/x for x of ordinary size: v_rcp_f64 and two Newton steps (no scaling, no fix-up of special cases)
+__device__ __forceinline__ double rcp_newton(double x)
+{
+    double v = __builtin_amdgcn_rcp(x);
+    v = fma(v, fma(-x, v, 1.0), v);
+    v = fma(v, fma(-x, v, 1.0), v);
+    return v;
+}
+// sin(y) and cos(y) for y in [0, pi/2] (for other y: finite values without meaning): y is folded onto [0, pi/4], where
+// the Taylor polynomials to w^15 and w^16 are exact to 5e-17 and 2e-18
+__device__ __forceinline__ void sincos_quarter(double y, double& sn, double& cs)
+{
+    const bool fold = y > 0.25 * kPi;
+    const double w = fold ? 0.5 * kPi - y : y;
+    const double w2 = w * w;
+    double ps = -1.0 / 1307674368000.0;
+    ps = fma(ps, w2, 1.0 / 6227020800.0);
+    ps = fma(ps, w2, -1.0 / 39916800.0);
+    ps = fma(ps, w2, 1.0 / 362880.0);
+    ps = fma(ps, w2, -1.0 / 5040.0);
+    ps = fma(ps, w2, 1.0 / 120.0);
+    ps = fma(ps, w2, -1.0 / 6.0);
+    const double sw = fma(ps * w2, w, w);
+    double pc = 1.0 / 20922789888000.0;
+    pc = fma(pc, w2, -1.0 / 87178291200.0);
+    pc = fma(pc, w2, 1.0 / 479001600.0);
+    pc = fma(pc, w2, -1.0 / 3628800.0);
+    pc = fma(pc, w2, 1.0 / 40320.0);
+    pc = fma(pc, w2, -1.0 / 720.0);
+    pc = fma(pc, w2, 1.0 / 24.0);
+    pc = fma(pc, w2, -0.5);
+    const double cw = fma(pc, w2, 1.0);
+    sn = fold ? cw : sw;
+    cs = fold ? sw : cw;
+}
+
 template <> struct Fast<double> {
     typedef double4 vec4;
     typedef double2 vec2;
     static __device__ __forceinline__ double4 make4(double a, double b, double c, double d) { return make_double4(a, b, c, d); }
     static __device__ __forceinline__ double2 make2(double a, double b) { return make_double2(a, b); }
-    static __device__ __forceinline__ double sqrt_(double x) { return sqrt(x); }
-    static __device__ __forceinline__ double sqrt_rn(double x) { return sqrt(x); }
-    static __device__ __forceinline__ double rcp(double x) { return 1.0 / x; }
+    static __device__ __forceinline__ double sqrt_(double x)
+    {
+        double r, inv;
+        sqrt_and_rcp(x, r, inv);
+        return r;
+    }
+    static __device__ __forceinline__ double sqrt_rn(double x) { return sqrt_(x); }
+    static __device__ __forceinline__ double rcp(double x) { return rcp_newton(x); }
     static __device__ __forceinline__ double gauss(double eta, double d) { return exp(-eta * d * d); }
-    static __device__ __forceinline__ double cutoff(double r, double rc) { return 0.5 * cos(kPi / rc * r) + 0.5; }
+    // f_C = 0.5 cos(pi r / rc) + 0.5 = cos^2(y), f_C' = -(pi / rc) sin(y) cos(y), y = pi r / (2 rc) in [0, pi/2] for r <= rc
+    static __device__ __forceinline__ double cutoff(double r, double rc)
+    {
+        double sn, cs;
+        sincos_quarter((kPi / (2.0 * rc)) * r, sn, cs);
+        return cs * cs;
+    }
     static __device__ __forceinline__ void cutoff_grad(double r, double rc, double& fc, double& dfc)
     {
-        const double w = kPi / rc;
-        fc = 0.5 * cos(w * r) + 0.5;
-        dfc = -0.5 * w * sin(w * r);
+        double sn, cs;
+        sincos_quarter((kPi / (2.0 * rc)) * r, sn, cs);
+        fc = cs * cs;
+        dfc = (-kPi / rc) * sn * cs;
     }
 };
 

@@ -23,9 +23,10 @@ namespace khan {
 namespace {
 
 // Distance arithmetic per precision.  float: the hardware reciprocal square root with one Newton step, the hardware
-// reciprocal and the minimax cutoff polynomials of the AEV kernels.  double: no library call either -- the library's
-// sqrt, division, cos and sin come to some 250 instructions per pair, most of them range reduction and special cases
-// that cannot occur here, and made these kernels run at 2.6 % of the double-precision vector peak.
+// reciprocal and the minimax cutoff polynomials of the AEV kernels.  double: no library call either (sqrt_and_rcp and
+// the Taylor cutoff of aev_small_common.h) -- the library's sqrt, division, cos and sin come to some 250 instructions
+// per pair, most of them range reduction and special cases that cannot occur here, and made these kernels run at
+// 2.6 % of the double-precision vector peak.
 template <typename T> struct ChargeMath;
 template <> struct ChargeMath<float> {
     // r = sqrt(d2) and 1/r (0 for d2 = 0)
@@ -41,53 +42,10 @@ template <> struct ChargeMath<float> {
     }
 };
 template <> struct ChargeMath<double> {
-    // v_rsq_f64 is good to 5e-8; one coupled Goldschmidt step (g -> sqrt, h -> 1/(2 sqrt)) squares that, the fused
-    // residual d2 - g^2 is exact and brings g to half an ulp, and one Newton step on the reciprocal of that g gives
-    // 1/r to an ulp: 10 instructions for both (measured against long double on 2^20 arguments: 1.1e-16 and 2.1e-16).
-    // Distances here are of order 1 A: no scaling for denormals is needed.
-    static __device__ __forceinline__ void dist(double d2, double& r, double& inv)
-    {
-        const double x = fmax(d2, 1e-300);
-        const double y = __builtin_amdgcn_rsq(x);
-        double g = x * y, h = 0.5 * y;
-        const double e = fma(-h, g, 0.5);
-        g = fma(g, e, g);
-        h = fma(h, e, h);
-        g = fma(fma(-g, g, x), h, g);
-        double v = h + h;
-        v = fma(v, fma(-g, v, 1.0), v);
-        r = d2 > 0.0 ? g : 0.0;
-        inv = d2 > 0.0 ? v : 0.0;
-    }
-    // f_C = 0.5 cos(pi r / rc) + 0.5 = cos^2(y), f_C' = -(pi / rc) sin(y) cos(y), y = pi r / (2 rc) in [0, pi/2]:
-    // y is folded onto [0, pi/4], where the Taylor polynomials to w^15 and w^16 are exact to 5e-17 and 2e-18
+    static __device__ __forceinline__ void dist(double d2, double& r, double& inv) { sqrt_and_rcp(d2, r, inv); }
     static __device__ __forceinline__ void cutoff(double r, double& fc, double& dfc)
     {
-        constexpr double rc = static_cast<double>(kR_Rc_f);
-        const double y = (kPi / (2.0 * rc)) * r;
-        const bool fold = y > 0.25 * kPi;
-        const double w = fold ? 0.5 * kPi - y : y;
-        const double w2 = w * w;
-        double ps = -1.0 / 1307674368000.0;
-        ps = fma(ps, w2, 1.0 / 6227020800.0);
-        ps = fma(ps, w2, -1.0 / 39916800.0);
-        ps = fma(ps, w2, 1.0 / 362880.0);
-        ps = fma(ps, w2, -1.0 / 5040.0);
-        ps = fma(ps, w2, 1.0 / 120.0);
-        ps = fma(ps, w2, -1.0 / 6.0);
-        const double sw = fma(ps * w2, w, w);
-        double pc = 1.0 / 20922789888000.0;
-        pc = fma(pc, w2, -1.0 / 87178291200.0);
-        pc = fma(pc, w2, 1.0 / 479001600.0);
-        pc = fma(pc, w2, -1.0 / 3628800.0);
-        pc = fma(pc, w2, 1.0 / 40320.0);
-        pc = fma(pc, w2, -1.0 / 720.0);
-        pc = fma(pc, w2, 1.0 / 24.0);
-        pc = fma(pc, w2, -0.5);
-        const double cw = fma(pc, w2, 1.0);
-        const double sn = fold ? cw : sw, cs = fold ? sw : cw;
-        fc = cs * cs;
-        dfc = (-kPi / rc) * sn * cs;
+        Fast<double>::cutoff_grad(r, static_cast<double>(kR_Rc_f), fc, dfc);
     }
 };
 
