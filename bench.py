@@ -158,8 +158,9 @@ def inference_bench(args, batch):
     xs, ys, zs = (torch.from_numpy(v).to(dev) for v in (batch.X, batch.Y, batch.Z))
     b = DeviceBatch.from_device_arrays(xs, ys, zs, torch.from_numpy(batch.A).to(dev),
                                        torch.from_numpy(batch.mol_idxs).to(dev), n_mols)
-    def timed(first_layer_kernel):
+    def timed(first_layer_kernel, whole_network=True):
         m = model.AniModel(model.DEFAULT_LAYERS, model.celu, torch.float32, dev, seed=1, first_layer_kernel=first_layer_kernel)
+        m.near.whole_network_kernel = whole_network
         for _ in range(args.warmup):
             m.batch_energies(b, need_grad=True)
         torch.cuda.synchronize()
@@ -170,8 +171,10 @@ def inference_bench(args, batch):
         return (time.perf_counter() - t0) / args.steps * 1e3, e, g
 
     ms_library, e_lib, g_lib = timed(False)      # every dense layer a library (rocBLAS) product
-    ms_per_step, e_k, g_k = timed(True)          # CELU layers, forward and backward, in this package's matrix-core kernel
+    ms_layers, e_l, g_l = timed(True, False)     # CELU layers, forward and backward, one launch per layer and direction
+    ms_per_step, e_k, g_k = timed(True)          # the whole network and its gradient back to the rows in one launch
     agree = float((e_k - e_lib).abs().max() / e_lib.abs().max())
+    agree_g = float((g_k - g_lib).abs().max() / g_lib.abs().max())
     sizes = (384,) + tuple(model.DEFAULT_LAYERS)
     macs_per_atom = sum(x * y for x, y in zip(sizes[:-1], sizes[1:]))
     gemm_flops = 2 * macs_per_atom * N * 2            # forward, and the data gradient on the way back
@@ -183,13 +186,14 @@ def inference_bench(args, batch):
         "config": {"workload": "inference65536: featurize + 4 atomic networks 384-128-128-64-1 (random weights) + "
                                "segment sum, gradient back to the coordinates; %d molecules, %d atoms" % (n_mols, N)},
         "molecules_per_s": n_mols / (ms_per_step * 1e-3),
-        "first_layer": {"kernel_ms_per_step": ms_per_step, "library_ms_per_step": ms_library,
-                        "max_relative_energy_difference": agree},
+        "networks": {"one_launch_ms_per_step": ms_per_step, "layer_by_layer_kernels_ms_per_step": ms_layers,
+                     "library_ms_per_step": ms_library, "max_relative_energy_difference_to_library": agree,
+                     "max_relative_gradient_difference_to_library": agree_g},
         "dense_products": "float32 operands split exactly into three bfloat16 parts, six partial products per pair on "
                           "v_mfma_f32_32x32x16_bf16, float32 accumulation (KHAN_DENSE_MATRIX=f32 selects "
                           "v_mfma_f32_32x32x2_f32)" if os.environ.get("KHAN_DENSE_MATRIX") != "f32" else "v_mfma_f32_32x32x2_f32",
-        "roofline": {"kernel": "dense layers, forward and data gradient (khan_dense_f32, khan_dense_head_f32, "
-                               "khan_dense_head_grad_f32): float32-equivalent flops of the whole step against the float32 matrix peak",
+        "roofline": {"kernel": "the atomic networks, forward and data gradient (khan_atomic_networks_f32): float32-equivalent "
+                               "flops of the whole step against the float32 matrix peak",
                      "bound": "mfma", "achieved": gemm_flops / (ms_per_step * 1e-3) / 1e12,
                      "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": gemm_flops / (ms_per_step * 1e-3) / 1e12 / FP32_PEAK_TFLOPS, "traffic": None},

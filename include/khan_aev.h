@@ -316,6 +316,30 @@ int khan_dense_head_grad_f32(const float *const *scale_host4, const float *const
                              float alpha, const float *const *deriv_of_host4, float *const *out_host4,
                              khan_stream_t stream);
 
+/* The whole atomic network of the reference's default size -- 384-128-128-64-1, CELU after all layers but the last
+ * (khan/model/nn.py:38-68; sizes khan/inference/energy_server.py:121) -- for the four atom types in ONE launch, and on
+ * request the gradient back to the feature rows in the same launch:
+ *     value_t[r] = (celu(celu(celu(rows_t[r] W1 + b1) W2 + b2) W3 + b3)) w4 + b4
+ *     grad_t[r, :] = scale_t[r] * d value_t[r] / d rows_t[r, :]            (grad_host4 non-NULL)
+ * A feature row is read once and its gradient written once; no activation of a hidden layer is written to memory
+ * (layer by layer, khan_dense_f32 and khan_dense_head_f32 write every activation and read it twice).  It is the pass of
+ * energy-and-force inference (energy_server.py:141-187): the values summed by molecule are the energies, and grad with
+ * scale = 1 is what khan_featurize_grad_f32 takes as its upstream rows.  Float32 matrix products as in khan_dense_f32.
+ *   rows_host4[t]          [n_t, 384] feature rows (the featurizer's buckets), 16-byte aligned
+ *   weights_t_host12[4l+t] layer l = 0, 1, 2 of type t TRANSPOSED: [128, 384], [128, 128], [64, 128]
+ *   weights_host12[4l+t]   the same layers as stored: [384, 128], [128, 128], [128, 64] (read for the gradient only;
+ *                          NULL when grad_host4 is NULL)
+ *   biases_host12[4l+t]    [128], [128], [64]
+ *   head_w_host4[t] [64], head_b_host4[t] one float (head_b_host4 or an entry may be NULL: no bias)
+ *   scale_host4[t]         [n_t] gradient with respect to each row's value, or NULL (the array or an entry): ones
+ *   value_host4[t] [n_t];  grad_host4[t] [n_t, 384], or grad_host4 = NULL: values only
+ * All are HOST arrays of DEVICE pointers; an empty type's pointers may be NULL. */
+int khan_atomic_networks_f32(const float *const *rows_host4, const int32_t *n_host4,
+                             const float *const *weights_t_host12, const float *const *weights_host12,
+                             const float *const *biases_host12, const float *const *head_w_host4,
+                             const float *const *head_b_host4, const float *const *scale_host4, float alpha,
+                             float *const *value_host4, float *const *grad_host4, khan_stream_t stream);
+
 /* Per-molecule sums of the atomic networks' outputs: e[m] = sum over the atoms g of molecule m of
  * out_{as[g]}[sis[g]] -- the gather to the batch's atom order and the segment sum by molecule of the reference
  * (khan/model/nn.py:165-177; trainer_multi_tower.py:350) in one launch, without the gathered copy, each molecule's

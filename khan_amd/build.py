@@ -25,7 +25,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 ROOT = os.path.dirname(HERE)
 
-HIP_SOURCES = ["capi.hip", "aev_generic.hip", "aev_small.hip", "aev_small_bwd.hip", "aev_medium.hip", "aev_medium_bwd.hip", "aev_large_sort.hip", "sort_offsets.hip", "charges.hip", "dense_first.hip", "mol_sum.hip"]
+HIP_SOURCES = ["capi.hip", "aev_generic.hip", "aev_small.hip", "aev_small_bwd.hip", "aev_medium.hip", "aev_medium_bwd.hip", "aev_large_sort.hip", "sort_offsets.hip", "charges.hip", "dense_first.hip", "dense_fused.hip", "mol_sum.hip"]
 HIP_HEADERS = ["khan_internal.h", "khan_params.h", "aev_generic_center.h", "aev_small_common.h", "aev_fwd_batch.h", "aev_bwd_batch.h", "aev_large.h", os.path.join(ROOT, "include", "khan_aev.h")]
 
 # packed-FP32 instruction selection is switched off on purpose (target feature -packed-fp32-ops)

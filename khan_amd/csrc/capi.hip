@@ -729,6 +729,42 @@ int khan_dense_head_grad_f32(const float* const* scale_host4, const float* const
                                                    out_host4, as_stream(stream)));
 }
 
+int khan_atomic_networks_f32(const float* const* rows_host4, const int32_t* n_host4, const float* const* weights_t_host12,
+                             const float* const* weights_host12, const float* const* biases_host12,
+                             const float* const* head_w_host4, const float* const* head_b_host4,
+                             const float* const* scale_host4, float alpha, float* const* value_host4,
+                             float* const* grad_host4, khan_stream_t stream)
+{
+    if (!rows_host4 || !n_host4 || !weights_t_host12 || !biases_host12 || !head_w_host4 || !value_host4) return KHAN_ERR_INVALID_ARG;
+    if (grad_host4 && !weights_host12) return KHAN_ERR_INVALID_ARG;
+    if (!(alpha > 0.0f)) return KHAN_ERR_INVALID_ARG;
+    int64_t total = 0;
+    for (int t = 0; t < 4; ++t) {
+        if (n_host4[t] < 0) return KHAN_ERR_INVALID_ARG;
+        if (n_host4[t] == 0) continue;
+        if (!rows_host4[t] || !head_w_host4[t] || !value_host4[t]) return KHAN_ERR_INVALID_ARG;
+        uintptr_t bits = reinterpret_cast<uintptr_t>(rows_host4[t]);        // 16-byte loads of rows and weights
+        for (int l = 0; l < 3; ++l) {
+            if (!weights_t_host12[4 * l + t] || !biases_host12[4 * l + t]) return KHAN_ERR_INVALID_ARG;
+            bits |= reinterpret_cast<uintptr_t>(weights_t_host12[4 * l + t]);
+            if (grad_host4) {
+                if (!weights_host12[4 * l + t]) return KHAN_ERR_INVALID_ARG;
+                bits |= reinterpret_cast<uintptr_t>(weights_host12[4 * l + t]);
+            }
+        }
+        if (grad_host4 && !grad_host4[t]) return KHAN_ERR_INVALID_ARG;
+        if (bits & 15u) return KHAN_ERR_INVALID_ARG;
+        total += n_host4[t];
+    }
+    if (total == 0) return KHAN_OK;
+    if (total > INT32_MAX) return KHAN_ERR_TOO_LARGE;
+    return hip_status(khan::launch_networks_fused(
+        rows_host4, n_host4, weights_t_host12, weights_t_host12 + 4, weights_t_host12 + 8,
+        weights_host12, weights_host12 ? weights_host12 + 4 : nullptr, weights_host12 ? weights_host12 + 8 : nullptr,
+        biases_host12, biases_host12 + 4, biases_host12 + 8, head_w_host4, head_b_host4, scale_host4, alpha, value_host4,
+        grad_host4, as_stream(stream)));
+}
+
 // Per-molecule sums of the per-type network outputs, and the way back.
 int khan_mol_energy_f32(const float* const* out_host4, const int32_t* as, const int32_t* sis, const int32_t* mos,
                         const int32_t* macs, int32_t n_mols, float* e, khan_stream_t stream)

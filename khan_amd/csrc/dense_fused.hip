@@ -1,0 +1,334 @@
+// The whole atomic network of the reference's default size, 384-128-128-64-1 with CELU (khan/model/nn.py:38-68,
+// khan/model/activations.py:63-65; sizes: khan/inference/energy_server.py:121), for the four atom types in ONE launch,
+// forward and -- on request -- back to the feature rows:
+//     a1 = celu(x W1 + b1), a2 = celu(a1 W2 + b2), a3 = celu(a2 W3 + b3), e = a3 w4 + b4          (per feature row x)
+//     g3 = s w4^T .* celu'(a3), g2 = (g3 W3^T) .* celu'(a2), g1 = (g2 W2^T) .* celu'(a1), dx = g1 W1^T
+// with s the gradient with respect to each row's value e (1 when none is given: the gradient of the sum of the values,
+// which is what forces need).  A feature row is read once and its gradient written once: the activations of a tile of
+// 128 rows never leave the compute unit.  Layer by layer the same pass moves 2.9 GB forward and 3.7 GB back per 767,292
+// rows (every activation written, read again by the next layer and once more on the way back); this one moves the rows
+// and their gradients, 2.4 GB, and the values.
+//
+// One workgroup of eight wavefronts owns 128 rows.  The products run on the bfloat16 matrix instructions with every
+// float32 operand split exactly into three bfloat16 parts and six partial products kept (dense_first.hip describes the
+// arithmetic: a float32 product to float32 accuracy).  A wavefront holds a 32 x 64 part of a layer's 128 x 128 output
+// (32 x 32 of the 128 x 64 one) in accumulator registers, and keeps its part of a1, a2 and a3 in registers for the way
+// back, where the gradients arrive in the same places.  Between layers the activations (gradients) go to LDS already
+// split, as three planes [row][k] of bfloat16: the next product's row operand, read straight from there.  The weights
+// stream from L2 in chunks of 16 k, split on the way into a double-buffered LDS stage, one barrier per chunk; layer 1
+// stages its feature rows the same way in the space the activation planes take later.  LDS: 139 KB, one workgroup per CU.
+#include "khan_internal.h"
+#include "khan_params.h"
+
+namespace khan {
+
+namespace {
+
+typedef float v4 __attribute__((ext_vector_type(4)));
+typedef float v16 __attribute__((ext_vector_type(16)));
+typedef unsigned u2v __attribute__((ext_vector_type(2)));
+typedef unsigned u4v __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f2v __attribute__((ext_vector_type(2)));
+
+constexpr int kRows = 128;          // rows per workgroup
+constexpr int kThreads = 512;
+constexpr int kK1 = 384, kN1 = 128, kN2 = 128, kN3 = 64;
+constexpr int kActStride = 136;     // bfloat16 elements between rows of the activation planes: 128 + 8 (16-byte reads without bank conflicts)
+constexpr int kKC = 16;             // k per staged chunk = one matrix instruction deep
+constexpr int kStStride = 24;       // bfloat16 elements between staged rows: 16 + 8
+
+struct FusedArgs {
+    const float* rows[4];           // [n_t, 384] feature rows per type
+    int n[4];
+    int tile_end[4];                // running sum of the per-type row tiles
+    const float* w1t[4];            // [128, 384]: layer 1's weights, the summed index contiguous (transposed)
+    const float* w2t[4];            // [128, 128]
+    const float* w3t[4];            // [64, 128]
+    const float* w1[4];             // [384, 128]: as stored -- the transposed operand of the way back
+    const float* w2[4];             // [128, 128]
+    const float* w3[4];             // [128, 64]
+    const float* b1[4];
+    const float* b2[4];
+    const float* b3[4];
+    const float* w4[4];             // [64]
+    const float* b4[4];             // one float
+    const float* scale[4];          // [n_t] gradient with respect to each row's value, or null (ones)
+    float* value[4];                // [n_t]
+    float* grad[4];                 // [n_t, 384], or null
+};
+
+struct __align__(16) FusedLds {
+    union {
+        unsigned short act[3][kRows][kActStride];        // a layer's activations or gradients, split: [part][row][k]
+        unsigned short astage[2][3][kRows][kStStride];   // layer 1: chunks of the feature rows
+    };
+    unsigned short bstage[2][3][128][kStStride];         // chunks of the weights: [buffer][part][column][k]
+    float rowval[2][kRows];                              // the output layer's partial sums; then the rows' upstream factors
+};
+
+// two floats -> their three bfloat16 parts, each pair packed into one register (first value in the low half)
+__device__ __forceinline__ void split_pair(float x0, float x1, unsigned& p1, unsigned& p2, unsigned& p3)
+{
+    p1 = __builtin_bit_cast(unsigned, __builtin_convertvector(f2v{x0, x1}, bf16x2));
+    const float r0 = x0 - __uint_as_float(p1 << 16), r1 = x1 - __uint_as_float(p1 & 0xffff0000u);
+    p2 = __builtin_bit_cast(unsigned, __builtin_convertvector(f2v{r0, r1}, bf16x2));
+    const float s0 = r0 - __uint_as_float(p2 << 16), s1 = r1 - __uint_as_float(p2 & 0xffff0000u);
+    p3 = __builtin_bit_cast(unsigned, __builtin_convertvector(f2v{s0, s1}, bf16x2));
+}
+
+// a chunk piece (four consecutive k of one row or column) split into the three planes of a stage buffer
+__device__ __forceinline__ void stage_piece(unsigned short (&dst)[3][128][kStStride], int r, int k4, const v4 x)
+{
+    unsigned lo[3], hi[3];
+    split_pair(x[0], x[1], lo[0], lo[1], lo[2]);
+    split_pair(x[2], x[3], hi[0], hi[1], hi[2]);
+#pragma unroll
+    for (int q = 0; q < 3; ++q) *reinterpret_cast<u2v*>(&dst[q][r][k4]) = u2v{lo[q], hi[q]};
+}
+
+__device__ __forceinline__ float celu_of(float v, float alpha, float inv_alpha)
+{
+    return v >= 0.f ? v : alpha * (__expf(v * inv_alpha) - 1.0f);
+}
+// CELU' from CELU's own value: 1 for h >= 0, exp(z / alpha) = h / alpha + 1 below
+__device__ __forceinline__ float celu_slope(float h, float inv_alpha) { return h >= 0.f ? 1.0f : fmaf(h, inv_alpha, 1.0f); }
+
+// sum over the 32 lanes of each half of the wavefront; lanes 16-31 and 48-63 hold the result
+__device__ __forceinline__ float half_sum_to_upper_row(float v)
+{
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));   // row_ror:8
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false));   // row_ror:4
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false));   // row_ror:2
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false));   // row_ror:1
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xa, 0xf, false));   // row_bcast:15
+    return v;
+}
+
+// Positions: accumulator e of a wavefront's block j is row wr*32 + 8 (e / 4) + 4 half + e % 4 of the tile and column
+// col0 + j*32 + l32, col0 = wc*64 for a 128-wide output (two blocks per wavefront), wc*32 for the 64-wide one (one).
+struct Place {
+    int tid, lane, wr, wc, l32, half;
+    __device__ __forceinline__ int row(int e) const { return wr * 32 + 8 * (e >> 2) + 4 * half + (e & 3); }
+};
+
+// One layer's product for this workgroup's 128 rows: acc = A . B^T, A = 128 x kK (rows), B = (kNB * 64) x kK
+// (`wt`, row-major: one row per output column), chunk by chunk of 16 k.  A comes from the activation planes, or
+// (kAGlobal) from `arows` in memory, staged like the weights.  Ends with a barrier: afterwards nobody reads the planes
+// or the stage any more.
+template <int kK, int kNB, bool kAGlobal>
+__device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (&acc)[2], const float* __restrict__ wt,
+                                              const float* __restrict__ arows, int row0, int n)
+{
+    constexpr int chunks = kK / kKC;
+    constexpr int kCols = kNB * 64;                      // 128 or 64 output columns
+    const int r = P.tid >> 2, k4 = (P.tid & 3) << 2;     // this thread's piece of a chunk: row or column r, k4..k4+3
+    const bool b_mine = r < kCols;                       // (the 64-column product: half of the threads stage weights)
+    const int arow = min(row0 + r, n - 1);               // rows past the end: the last row again, never stored
+    v4 rb = v4{0.f, 0.f, 0.f, 0.f}, ra = v4{0.f, 0.f, 0.f, 0.f};
+    auto fetch = [&](int c) {
+        if (b_mine) rb = *reinterpret_cast<const v4*>(wt + static_cast<size_t>(r) * kK + c * kKC + k4);
+        if constexpr (kAGlobal) ra = *reinterpret_cast<const v4*>(arows + static_cast<size_t>(arow) * kK + c * kKC + k4);
+    };
+    auto stage = [&](int buf) {
+        if (b_mine) stage_piece(S.bstage[buf], r, k4, rb);
+        if constexpr (kAGlobal) stage_piece(S.astage[buf], r, k4, ra);
+    };
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
+    fetch(0);
+    stage(0);
+    if (chunks > 1) fetch(1);
+    __syncthreads();             // chunk 0 is staged; the activation planes written before this call are complete
+    const int col0 = kNB == 2 ? P.wc * 64 : P.wc * 32;
+    for (int c = 0; c < chunks; ++c) {
+        if (c + 1 < chunks) {
+            stage((c + 1) & 1);                          // the other buffer: last read before the previous barrier
+            if (c + 2 < chunks) fetch(c + 2);            // in flight during the products
+        }
+        bf16x8 av[3];
+#pragma unroll
+        for (int m = 0; m < 3; ++m) {
+            if constexpr (kAGlobal)
+                av[m] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u4v*>(&S.astage[c & 1][m][P.wr * 32 + P.l32][P.half * 8]));
+            else
+                av[m] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u4v*>(&S.act[m][P.wr * 32 + P.l32][c * kKC + P.half * 8]));
+        }
+#pragma unroll
+        for (int j = 0; j < kNB; ++j) {
+            bf16x8 bv[3];
+#pragma unroll
+            for (int m = 0; m < 3; ++m)
+                bv[m] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u4v*>(&S.bstage[c & 1][m][col0 + j * 32 + P.l32][P.half * 8]));
+            // smallest partial products first
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[2], bv[0], acc[j], 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[2], acc[j], 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[1], acc[j], 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[0], acc[j], 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[1], acc[j], 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[0], acc[j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+}
+
+// a wavefront's values of a layer (kNB blocks) -> the activation planes, split; column = k of the next product
+template <int kNB>
+__device__ __forceinline__ void to_planes(FusedLds& S, const Place& P, const v16 (&v)[2])
+{
+    const int col0 = kNB == 2 ? P.wc * 64 : P.wc * 32;
+#pragma unroll
+    for (int j = 0; j < kNB; ++j) {
+        const int col = col0 + j * 32 + P.l32;
+#pragma unroll
+        for (int e = 0; e < 16; e += 2) {
+            unsigned p[3];
+            split_pair(v[j][e], v[j][e + 1], p[0], p[1], p[2]);
+            const int r0 = P.row(e), r1 = P.row(e + 1);
+#pragma unroll
+            for (int q = 0; q < 3; ++q) {
+                S.act[q][r0][col] = static_cast<unsigned short>(p[q] & 0xffffu);
+                S.act[q][r1][col] = static_cast<unsigned short>(p[q] >> 16);
+            }
+        }
+    }
+}
+
+template <bool kGrad>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
+{
+    __shared__ FusedLds S;
+    Place P;
+    P.tid = threadIdx.x;
+    P.lane = P.tid & 63;
+    const int wave = P.tid >> 6;
+    P.wr = wave >> 1;
+    P.wc = wave & 1;
+    P.l32 = P.lane & 31;
+    P.half = P.lane >> 5;
+    const int tile = blockIdx.x;
+    const int t = (tile >= args.tile_end[0]) + (tile >= args.tile_end[1]) + (tile >= args.tile_end[2]);
+    const int first = t == 0 ? 0 : args.tile_end[t - 1];
+    const int row0 = (tile - first) * kRows, n = args.n[t];
+
+    v16 acc[2], a1[2], a2[2], a3[2];
+    // ------------------------------------------------------------ layer 1: 384 -> 128
+    layer_product<kK1, 2, true>(S, P, acc, args.w1t[t], args.rows[t], row0, n);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const float b = args.b1[t][P.wc * 64 + j * 32 + P.l32];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) a1[j][e] = celu_of(acc[j][e] + b, alpha, inv_alpha);
+    }
+    to_planes<2>(S, P, a1);
+    // ------------------------------------------------------------ layer 2: 128 -> 128
+    layer_product<kN1, 2, false>(S, P, acc, args.w2t[t], nullptr, row0, n);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const float b = args.b2[t][P.wc * 64 + j * 32 + P.l32];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) a2[j][e] = celu_of(acc[j][e] + b, alpha, inv_alpha);
+    }
+    to_planes<2>(S, P, a2);
+    // ------------------------------------------------------------ layer 3: 128 -> 64, and the output layer 64 -> 1
+    layer_product<kN2, 1, false>(S, P, acc, args.w3t[t], nullptr, row0, n);
+    const int c3 = P.wc * 32 + P.l32;                    // this lane's column of the 64
+    const float w4 = args.w4[t][c3];
+    {
+        const float b = args.b3[t][c3];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            a3[0][e] = celu_of(acc[0][e] + b, alpha, inv_alpha);
+            const float tot = half_sum_to_upper_row(a3[0][e] * w4);      // over this wavefront's 32 of the 64 columns
+            if (P.l32 == 16 + e) S.rowval[P.wc][P.row(e)] = tot;
+        }
+    }
+    __syncthreads();
+    if (P.tid < kRows) {
+        const int gr = row0 + P.tid;
+        const float value = S.rowval[0][P.tid] + S.rowval[1][P.tid] + (args.b4[t] ? args.b4[t][0] : 0.f);
+        if (gr < n) args.value[t][gr] = value;
+    }
+    if constexpr (!kGrad) return;
+    // ------------------------------------------------------------ the way back
+    __syncthreads();             // the partial sums have been read
+    if (P.tid < kRows) S.rowval[0][P.tid] = args.scale[t] ? args.scale[t][min(row0 + P.tid, n - 1)] : 1.0f;
+    __syncthreads();
+    {
+        v16 g3[2];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) g3[0][e] = S.rowval[0][P.row(e)] * w4 * celu_slope(a3[0][e], inv_alpha);
+        to_planes<1>(S, P, g3);
+    }
+    // g2 = (g3 W3^T) .* celu'(a2): 64 -> 128
+    layer_product<kN3, 2, false>(S, P, acc, args.w3[t], nullptr, row0, n);
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[j][e] *= celu_slope(a2[j][e], inv_alpha);
+    to_planes<2>(S, P, acc);
+    // g1 = (g2 W2^T) .* celu'(a1): 128 -> 128
+    layer_product<kN2, 2, false>(S, P, acc, args.w2[t], nullptr, row0, n);
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[j][e] *= celu_slope(a1[j][e], inv_alpha);
+    to_planes<2>(S, P, acc);
+    // dx = g1 W1^T: 128 -> 384, three column tiles of 128
+    float* __restrict__ out = args.grad[t];
+    for (int ct = 0; ct < kK1 / 128; ++ct) {
+        layer_product<kN1, 2, false>(S, P, acc, args.w1[t] + static_cast<size_t>(ct) * 128 * kN1, nullptr, row0, n);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int col = ct * 128 + P.wc * 64 + j * 32 + P.l32;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int gr = row0 + P.row(e);
+                if (gr < n) out[static_cast<size_t>(gr) * kK1 + col] = acc[j][e];
+            }
+        }
+    }
+}
+
+}  // namespace
+
+// rows[t]: [n[t], 384]; w*t: transposed weights ([out, in]); w*: as stored ([in, out]); value[t]: [n[t]];
+// grad[t]: [n[t], 384] or null pointers (then only the values are formed; w1, w2, w3 and scale are not read).
+hipError_t launch_networks_fused(const float* const rows[4], const int32_t n[4],
+                                 const float* const w1t[4], const float* const w2t[4], const float* const w3t[4],
+                                 const float* const w1[4], const float* const w2[4], const float* const w3[4],
+                                 const float* const b1[4], const float* const b2[4], const float* const b3[4],
+                                 const float* const w4[4], const float* const b4[4], const float* const scale[4],
+                                 float alpha, float* const value[4], float* const grad[4], hipStream_t stream)
+{
+    FusedArgs a;
+    int tiles = 0;
+    bool want_grad = false;
+    for (int t = 0; t < 4; ++t) {
+        a.rows[t] = rows[t];
+        a.n[t] = n[t];
+        tiles += (n[t] + kRows - 1) / kRows;
+        a.tile_end[t] = tiles;
+        a.w1t[t] = w1t[t]; a.w2t[t] = w2t[t]; a.w3t[t] = w3t[t];
+        a.w1[t] = w1 ? w1[t] : nullptr; a.w2[t] = w2 ? w2[t] : nullptr; a.w3[t] = w3 ? w3[t] : nullptr;
+        a.b1[t] = b1[t]; a.b2[t] = b2[t]; a.b3[t] = b3[t];
+        a.w4[t] = w4[t];
+        a.b4[t] = b4 ? b4[t] : nullptr;
+        a.scale[t] = scale ? scale[t] : nullptr;
+        a.value[t] = value[t];
+        a.grad[t] = grad ? grad[t] : nullptr;
+        want_grad = want_grad || (grad && grad[t]);
+    }
+    if (tiles == 0) return hipSuccess;
+    if (want_grad)
+        networks_fused_kernel<true><<<dim3(static_cast<unsigned>(tiles)), dim3(kThreads), 0, stream>>>(a, alpha, 1.0f / alpha);
+    else
+        networks_fused_kernel<false><<<dim3(static_cast<unsigned>(tiles)), dim3(kThreads), 0, stream>>>(a, alpha, 1.0f / alpha);
+    return hipGetLastError();
+}
+
+}  // namespace khan

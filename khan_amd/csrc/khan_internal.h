@@ -137,6 +137,13 @@ hipError_t launch_dense_head(const float* const rows[4], const int32_t n[4], int
 hipError_t launch_dense_head_grad(const float* const scale[4], const float* const head_w[4], const int32_t n[4], int32_t k,
                                   int32_t n_out, const float* const wt[4], float alpha, const float* const deriv_of[4],
                                   float* const out[4], hipStream_t stream);
+// the whole 384-128-128-64-1 CELU network of the four types in one launch, forward and (grad non-null) back to the rows
+hipError_t launch_networks_fused(const float* const rows[4], const int32_t n[4],
+                                 const float* const w1t[4], const float* const w2t[4], const float* const w3t[4],
+                                 const float* const w1[4], const float* const w2[4], const float* const w3[4],
+                                 const float* const b1[4], const float* const b2[4], const float* const b3[4],
+                                 const float* const w4[4], const float* const b4[4], const float* const scale[4],
+                                 float alpha, float* const value[4], float* const grad[4], hipStream_t stream);
 hipError_t launch_dense_first(const float* const rows[4], const int32_t n[4], const float* const wt[4],
                               const float* const bias[4], bool celu, float alpha, float* const out[4],
                               hipStream_t stream);

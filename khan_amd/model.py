@@ -76,6 +76,7 @@ class MoleculeNN:
     def __init__(self, layer_sizes=DEFAULT_LAYERS, activation_fn=celu, dtype=torch.float32, device="cpu",
                  prefix="near_", seed=None, first_layer_kernel=True):
         self.first_layer_kernel = bool(first_layer_kernel)
+        self.whole_network_kernel = True    # the one-launch network where it applies (`one_launch`); False: layer by layer
         self.weights_need_grad = False      # set it to differentiate through the kernel layers' weights (training)
         layer_sizes = tuple(int(v) for v in layer_sizes)
         if layer_sizes[-1] != 1:
@@ -133,6 +134,22 @@ class MoleculeNN:
                 break
             n += 1
         return n
+
+    def one_launch(self):
+        """True if the whole network runs in `ops.atomic_networks` (one launch for the three CELU layers and the output
+        layer of the four types, and for the gradient back to the feature rows): the reference's default widths
+        384-128-128-64-1 in float32 on the GPU with CELU, the weights taken as constants (inference)."""
+        from . import ops
+        return (self.whole_network_kernel and self.kernel_layers() == 3 and self.layer_sizes == ops.NETWORK_WIDTHS + (1,)
+                and not self.weights_need_grad)
+
+    def one_launch_operands(self):
+        """-> (weights_t, weights, biases, head_weights, head_biases) as `ops.atomic_networks` takes them."""
+        rows = [[self.names[t][k] for t in TYPE_MAP] for k in range(4)]
+        weights_t = [self.layer_transposed(k) for k in range(3)]
+        weights = [[self.params[r[0]].detach() for r in rows[k]] for k in range(3)]
+        biases = [[self.params[r[1]].detach() for r in rows[k]] for k in range(3)]
+        return weights_t, weights, biases, [self.params[r[0]].detach() for r in rows[3]], [self.params[r[1]].detach() for r in rows[3]]
 
     def atom_outputs(self, atom_type_features, gather_idxs):
         """Per-type flat feature buckets -> one number per atom in the batch's atom order (nn.py:176-177)."""
@@ -215,11 +232,24 @@ class AniModel:
     # --------------------------------------------------------------------------------------- inference
     def batch_energies(self, b, need_grad=False):
         """DeviceBatch -> per-molecule energies [n_mols] (and d energy / d xyz when need_grad)."""
-        from . import autograd
+        from . import autograd, ops
         xs, ys, zs = b.xs, b.ys, b.zs
+        acs, order, classes = b.host_counts()
+        if self.charge is None and self.near.one_launch():
+            # featurize -> the four networks in one launch (values, and the gradient of their sum with respect to the
+            # feature rows) -> sums by molecule; the coordinate gradient is featurize_grad of those rows' gradients
+            feats = ops.featurize(xs, ys, zs, b.atom_types, b.mol_offsets, b.mol_atom_counts, b.scatter_idxs, acs,
+                                  order=order, size_classes=classes)
+            weights_t, weights, biases, head_w, head_b = self.near.one_launch_operands()
+            values, grads = ops.atomic_networks(feats, weights_t, biases, head_w, head_b, weights=weights, want_grad=need_grad)
+            energies = ops.mol_energy(values, b.atom_types, b.scatter_idxs, b.mol_offsets, b.mol_atom_counts)
+            if not need_grad:
+                return energies, None
+            gx, gy, gz = ops.featurize_grad(xs, ys, zs, b.atom_types, b.mol_offsets, b.mol_atom_counts, b.scatter_idxs, acs,
+                                            *[g.reshape(-1) for g in grads], order=order, size_classes=classes)
+            return energies, torch.stack((gx, gy, gz), dim=1)
         if need_grad:
             xs, ys, zs = (t.detach().clone().requires_grad_(True) for t in (xs, ys, zs))
-        acs, order, classes = b.host_counts()
         feats = autograd.featurize(xs, ys, zs, b.atom_types, b.mol_offsets, b.mol_atom_counts, b.scatter_idxs, acs,
                                    order=order, size_classes=classes)
         # the networks' outputs summed by molecule straight from the four per-type vectors (nn.py:165-177 in one launch)

@@ -466,6 +466,54 @@ def dense_head_grad(scales, head_weights, weights_nk, deriv_of, alpha=0.1):
     return tuple(outs)
 
 
+NETWORK_WIDTHS = (384, 128, 128, 64)      # the layer widths `atomic_networks` is built for (then 64 -> 1)
+
+
+def atomic_networks(rows, weights_t, biases, head_weights, head_biases=None, weights=None, scales=None, want_grad=False,
+                    alpha=0.1):
+    """The 384-128-128-64-1 CELU networks of the four atom types in one launch, float32: -> (values, grads).
+    values[t] is [n_t], the network's output for every feature row of rows[t] ([n_t, 384] or a flat bucket); with
+    `want_grad`, grads[t] ([n_t, 384]) is scales[t][:, None] * d values[t] / d rows[t] (scales None: ones), formed in
+    the same launch without any hidden layer's activations going to memory; otherwise grads is None.
+    weights_t[l][t]: layer l = 0, 1, 2 transposed ([128, 384], [128, 128], [64, 128]); weights[l][t]: the same layers as
+    stored ([384, 128], [128, 128], [128, 64]; needed with want_grad); biases[l][t]; head_weights[t] (64 values),
+    head_biases[t] (one value)."""
+    lib = _lib.load()
+    shapes_t = ((128, 384), (128, 128), (64, 128))
+    xs, ns, vals, grads = [], [], [], []
+    for t in range(4):
+        x = _dense_matrix(rows[t].reshape(-1, 384), 384, "rows[%d]" % t)
+        xs.append(x)
+        ns.append(int(x.shape[0]))
+        vals.append(torch.empty(x.shape[0], dtype=torch.float32, device=x.device))
+        if want_grad:
+            grads.append(torch.empty((x.shape[0], 384), dtype=torch.float32, device=x.device))
+    wts, ws, bs = [], [], []
+    for l in range(3):
+        for t in range(4):
+            wts.append(_dense_weights(weights_t[l][t], shapes_t[l][0], shapes_t[l][1], "weights_t[%d][%d]" % (l, t)))
+            bs.append(_dev(biases[l][t].reshape(-1), torch.float32, "biases"))
+            if bs[-1].numel() != shapes_t[l][0]:
+                raise ValueError("biases[%d][%d] must have %d elements" % (l, t, shapes_t[l][0]))
+            if want_grad:
+                ws.append(_dense_weights(weights[l][t], shapes_t[l][1], shapes_t[l][0], "weights[%d][%d]" % (l, t)))
+    hws = [_dev(h.reshape(-1), torch.float32, "head_weights") for h in head_weights]
+    if any(h.numel() != 64 for h in hws):
+        raise ValueError("head_weights must have 64 elements each")
+    hbs = None if head_biases is None else [_dev(h.reshape(-1), torch.float32, "head_biases") for h in head_biases]
+    scs = None
+    if scales is not None:
+        scs = [_dev(sc.reshape(-1), torch.float32, "scales") for sc in scales]
+        if any(sc.numel() != n for sc, n in zip(scs, ns)):
+            raise ValueError("scales[t] must have one element per row")
+    p12 = lambda ts: (ctypes.c_void_p * 12)(*[t.data_ptr() for t in ts])
+    _lib.check(lib.khan_atomic_networks_f32(_ptr4(xs), (ctypes.c_int32 * 4)(*ns), p12(wts), p12(ws) if want_grad else None,
+                                            p12(bs), _ptr4(hws), None if hbs is None else _ptr4(hbs),
+                                            None if scs is None else _ptr4(scs), float(alpha), _ptr4(vals),
+                                            _ptr4(grads) if want_grad else None, _stream()))
+    return tuple(vals), (tuple(grads) if want_grad else None)
+
+
 def dense_first(atom_type_features, acs, weights_t, biases, activation=ACT_CELU, alpha=0.1):
     """First dense layer of the four atomic networks on the featurizer's buckets, float32, one launch:
     -> four [acs[t], 128] tensors act(rows_t . W_t + b_t).  `weights_t[t]` is W_t TRANSPOSED, [128, 384]."""

@@ -555,3 +555,60 @@ def test_force_loss_reaches_the_weights_through_the_kernel_layers():
         else:
             assert f1 is not None and np.abs(f1 - f0).max() <= 5e-4 * np.abs(f0).max(), (name, np.abs(f1 - f0).max(), np.abs(f0).max())
         assert np.abs(g1 - g0).max() <= 5e-4 * max(1e-6, np.abs(g0).max()), (name, np.abs(g1 - g0).max())
+
+
+def _network_f64(x, Ws, bs, w4, b4, scale, alpha=0.1):
+    """The 384-128-128-64-1 CELU network and its gradient with respect to the rows in float64 numpy."""
+    acts, a = [], x
+    for W, b_ in zip(Ws, bs):
+        a = nn_ref._celu(a @ W + b_)
+        acts.append(a)
+    value = a @ w4 + b4
+    g = (scale[:, None] * w4[None, :]) * np.where(acts[2] >= 0, 1.0, acts[2] / alpha + 1.0)
+    g = (g @ Ws[2].T) * np.where(acts[1] >= 0, 1.0, acts[1] / alpha + 1.0)
+    g = (g @ Ws[1].T) * np.where(acts[0] >= 0, 1.0, acts[0] / alpha + 1.0)
+    return value, g @ Ws[0].T
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("with_scale", [False, True])
+def test_whole_network_in_one_launch_matches_float64(with_scale):
+    """khan_atomic_networks_f32 (the three CELU layers and the output layer of the four types in one launch, the
+    hidden activations never leaving the compute unit, and the gradient back to the rows in the same launch) against
+    float64 numpy on the same float32 operands: row counts on and off the 128-row tile, an empty type, one row; values
+    only (no gradient asked for) must equal the values of the launch that also forms the gradient."""
+    from khan_amd import ops
+    dev = "cuda:0"
+    f32 = lambda a: np.ascontiguousarray(a.astype(np.float32))
+    d = lambda a: torch.from_numpy(f32(a)).to(dev)
+    rng = np.random.default_rng(11)
+    ns = [0, 1, 300, 1024 + 77]
+    widths = (384, 128, 128, 64)
+    xs = [np.abs(rng.standard_normal((n, 384))) * 0.5 for n in ns]          # feature rows are non-negative
+    Ws = [[rng.standard_normal((widths[l], widths[l + 1])) * (2.0 / (widths[l] + widths[l + 1])) ** 0.5 for l in range(3)] for _ in range(4)]
+    bs = [[rng.standard_normal(widths[l + 1]) * 0.1 for l in range(3)] for _ in range(4)]
+    w4 = [rng.standard_normal(64) * 0.2 for _ in range(4)]
+    b4 = [rng.standard_normal(1) for _ in range(4)]
+    scales = [rng.standard_normal(n) for n in ns]
+    weights = [[d(Ws[t][l]) for t in range(4)] for l in range(3)]
+    weights_t = [[d(Ws[t][l].T) for t in range(4)] for l in range(3)]
+    biases = [[d(bs[t][l]) for t in range(4)] for l in range(3)]
+    rows = [d(x) for x in xs]
+    vals, grads = ops.atomic_networks(rows, weights_t, biases, [d(w) for w in w4], [d(b_) for b_ in b4], weights=weights,
+                                      scales=[d(sc) for sc in scales] if with_scale else None, want_grad=True)
+    vals_only, none = ops.atomic_networks(rows, weights_t, biases, [d(w) for w in w4], [d(b_) for b_ in b4])
+    assert none is None
+    for t in range(4):
+        up = lambda a: f32(a).astype(np.float64)
+        sc = up(scales[t]) if with_scale else np.ones(ns[t])
+        want_v, want_g = _network_f64(up(xs[t]), [up(W) for W in Ws[t]], [up(b_) for b_ in bs[t]], up(w4[t]), up(b4[t])[0], sc)
+        got_v, got_g = vals[t].cpu().numpy().astype(np.float64), grads[t].cpu().numpy().astype(np.float64)
+        assert got_v.shape == (ns[t],) and got_g.shape == (ns[t], 384)
+        assert torch.equal(vals[t], vals_only[t])
+        if ns[t] == 0:
+            continue
+        # float32 products through four layers: relative to the size of the values / of the largest gradient entry of the row
+        vscale = np.abs(want_v).max() + 1.0
+        assert np.all(np.isfinite(got_v)) and np.abs(got_v - want_v).max() <= 2e-5 * vscale, (t, np.abs(got_v - want_v).max(), vscale)
+        gscale = np.abs(want_g).max(axis=1, keepdims=True) + 1e-6
+        assert np.all(np.isfinite(got_g)) and np.all(np.abs(got_g - want_g) <= 5e-5 * gscale), (t, (np.abs(got_g - want_g) / gscale).max())
