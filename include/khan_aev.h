@@ -329,14 +329,22 @@ int khan_dense_head_grad_f32(const float *const *scale_host4, const float *const
  *   weights_t_host12[4l+t] layer l = 0, 1, 2 of type t TRANSPOSED: [128, 384], [128, 128], [64, 128]
  *   weights_host12[4l+t]   the same layers as stored: [384, 128], [128, 128], [128, 64] (read for the gradient only;
  *                          NULL when grad_host4 is NULL)
+ *   packed                 DEVICE buffer written by khan_atomic_networks_pack_f32 from the same 24 matrices, or NULL.
+ *                          With it neither weights array is read (both may be NULL) and the kernel copies the weights'
+ *                          three bfloat16 parts instead of splitting them again for every 128 rows: the same bits out,
+ *                          a tenth less time.  Pack once per set of weights (khan_atomic_networks_packed_bytes() bytes,
+ *                          16-byte aligned); pack again after the weights change.
  *   biases_host12[4l+t]    [128], [128], [64]
  *   head_w_host4[t] [64], head_b_host4[t] one float (head_b_host4 or an entry may be NULL: no bias)
  *   scale_host4[t]         [n_t] gradient with respect to each row's value, or NULL (the array or an entry): ones
  *   value_host4[t] [n_t];  grad_host4[t] [n_t, 384], or grad_host4 = NULL: values only
  * All are HOST arrays of DEVICE pointers; an empty type's pointers may be NULL. */
+int64_t khan_atomic_networks_packed_bytes(void);
+int khan_atomic_networks_pack_f32(const float *const *weights_t_host12, const float *const *weights_host12,
+                                  void *packed, khan_stream_t stream);
 int khan_atomic_networks_f32(const float *const *rows_host4, const int32_t *n_host4,
                              const float *const *weights_t_host12, const float *const *weights_host12,
-                             const float *const *biases_host12, const float *const *head_w_host4,
+                             const void *packed, const float *const *biases_host12, const float *const *head_w_host4,
                              const float *const *head_b_host4, const float *const *scale_host4, float alpha,
                              float *const *value_host4, float *const *grad_host4, khan_stream_t stream);
 

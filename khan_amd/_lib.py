@@ -74,7 +74,10 @@ _SIGNATURES = {
     "khan_dense_head_grad_f32": (ctypes.c_int, [ctypes.POINTER(_ptr), ctypes.POINTER(_ptr), ctypes.POINTER(ctypes.c_int32),
                                                 ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(_ptr), ctypes.c_float,
                                                 ctypes.POINTER(_ptr), ctypes.POINTER(_ptr), _ptr]),
-    "khan_atomic_networks_f32": (ctypes.c_int, [ctypes.POINTER(_ptr), ctypes.POINTER(ctypes.c_int32)] + [ctypes.POINTER(_ptr)] * 6
+    "khan_atomic_networks_packed_bytes": (ctypes.c_int64, []),
+    "khan_atomic_networks_pack_f32": (ctypes.c_int, [ctypes.POINTER(_ptr), ctypes.POINTER(_ptr), _ptr, _ptr]),
+    "khan_atomic_networks_f32": (ctypes.c_int, [ctypes.POINTER(_ptr), ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(_ptr),
+                                                ctypes.POINTER(_ptr), _ptr] + [ctypes.POINTER(_ptr)] * 4
                                  + [ctypes.c_float, ctypes.POINTER(_ptr), ctypes.POINTER(_ptr), _ptr]),
     "khan_mol_energy_f32": (ctypes.c_int, [ctypes.POINTER(_ptr)] + [_ptr] * 4 + [ctypes.c_int32, _ptr, _ptr]),
     "khan_mol_energy_f64": (ctypes.c_int, [ctypes.POINTER(_ptr)] + [_ptr] * 4 + [ctypes.c_int32, _ptr, _ptr]),

@@ -729,14 +729,28 @@ int khan_dense_head_grad_f32(const float* const* scale_host4, const float* const
                                                    out_host4, as_stream(stream)));
 }
 
+int64_t khan_atomic_networks_packed_bytes(void) { return static_cast<int64_t>(khan::networks_packed_bytes()); }
+
+int khan_atomic_networks_pack_f32(const float* const* weights_t_host12, const float* const* weights_host12, void* packed,
+                                  khan_stream_t stream)
+{
+    if (!weights_t_host12 || !weights_host12 || !packed) return KHAN_ERR_INVALID_ARG;
+    for (int k = 0; k < 12; ++k)
+        if (!weights_t_host12[k] || !weights_host12[k]) return KHAN_ERR_INVALID_ARG;
+    if (reinterpret_cast<uintptr_t>(packed) & 15u) return KHAN_ERR_INVALID_ARG;
+    return hip_status(khan::launch_networks_pack(weights_t_host12, weights_t_host12 + 4, weights_t_host12 + 8, weights_host12,
+                                                 weights_host12 + 4, weights_host12 + 8, packed, as_stream(stream)));
+}
+
 int khan_atomic_networks_f32(const float* const* rows_host4, const int32_t* n_host4, const float* const* weights_t_host12,
-                             const float* const* weights_host12, const float* const* biases_host12,
+                             const float* const* weights_host12, const void* packed, const float* const* biases_host12,
                              const float* const* head_w_host4, const float* const* head_b_host4,
                              const float* const* scale_host4, float alpha, float* const* value_host4,
                              float* const* grad_host4, khan_stream_t stream)
 {
-    if (!rows_host4 || !n_host4 || !weights_t_host12 || !biases_host12 || !head_w_host4 || !value_host4) return KHAN_ERR_INVALID_ARG;
-    if (grad_host4 && !weights_host12) return KHAN_ERR_INVALID_ARG;
+    if (!rows_host4 || !n_host4 || !biases_host12 || !head_w_host4 || !value_host4) return KHAN_ERR_INVALID_ARG;
+    if (!packed && (!weights_t_host12 || (grad_host4 && !weights_host12))) return KHAN_ERR_INVALID_ARG;
+    if (packed && (reinterpret_cast<uintptr_t>(packed) & 15u)) return KHAN_ERR_INVALID_ARG;
     if (!(alpha > 0.0f)) return KHAN_ERR_INVALID_ARG;
     int64_t total = 0;
     for (int t = 0; t < 4; ++t) {
@@ -745,7 +759,9 @@ int khan_atomic_networks_f32(const float* const* rows_host4, const int32_t* n_ho
         if (!rows_host4[t] || !head_w_host4[t] || !value_host4[t]) return KHAN_ERR_INVALID_ARG;
         uintptr_t bits = reinterpret_cast<uintptr_t>(rows_host4[t]);        // 16-byte loads of rows and weights
         for (int l = 0; l < 3; ++l) {
-            if (!weights_t_host12[4 * l + t] || !biases_host12[4 * l + t]) return KHAN_ERR_INVALID_ARG;
+            if (!biases_host12[4 * l + t]) return KHAN_ERR_INVALID_ARG;
+            if (packed) continue;
+            if (!weights_t_host12[4 * l + t]) return KHAN_ERR_INVALID_ARG;
             bits |= reinterpret_cast<uintptr_t>(weights_t_host12[4 * l + t]);
             if (grad_host4) {
                 if (!weights_host12[4 * l + t]) return KHAN_ERR_INVALID_ARG;
@@ -758,11 +774,13 @@ int khan_atomic_networks_f32(const float* const* rows_host4, const int32_t* n_ho
     }
     if (total == 0) return KHAN_OK;
     if (total > INT32_MAX) return KHAN_ERR_TOO_LARGE;
+    const bool plain = !packed;
     return hip_status(khan::launch_networks_fused(
-        rows_host4, n_host4, weights_t_host12, weights_t_host12 + 4, weights_t_host12 + 8,
-        weights_host12, weights_host12 ? weights_host12 + 4 : nullptr, weights_host12 ? weights_host12 + 8 : nullptr,
+        rows_host4, n_host4, plain ? weights_t_host12 : nullptr, plain ? weights_t_host12 + 4 : nullptr,
+        plain ? weights_t_host12 + 8 : nullptr, plain && weights_host12 ? weights_host12 : nullptr,
+        plain && weights_host12 ? weights_host12 + 4 : nullptr, plain && weights_host12 ? weights_host12 + 8 : nullptr,
         biases_host12, biases_host12 + 4, biases_host12 + 8, head_w_host4, head_b_host4, scale_host4, alpha, value_host4,
-        grad_host4, as_stream(stream)));
+        grad_host4, packed, as_stream(stream)));
 }
 
 // Per-molecule sums of the per-type network outputs, and the way back.

@@ -15,7 +15,9 @@
 // (32 x 32 of the 128 x 64 one) in accumulator registers, and keeps its part of a1, a2 and a3 in registers for the way
 // back, where the gradients arrive in the same places.  Between layers the activations (gradients) go to LDS already
 // split, as three planes [row][k] of bfloat16: the next product's row operand, read straight from there.  The weights
-// stream from L2 in chunks of 16 k, split on the way into a double-buffered LDS stage, one barrier per chunk; layer 1
+// stream from L2 in chunks of 16 k into a double-buffered LDS stage, one barrier per chunk -- split on the way, or, when
+// the caller has had them split once beforehand (launch_networks_pack: a quarter of the kernel's vector instructions
+// were the same weights being split again for every tile of rows), copied as they are; layer 1
 // stages its feature rows the same way in the space the activation planes take later.  LDS: 139 KB, one workgroup per CU.
 #include "khan_internal.h"
 #include "khan_params.h"
@@ -57,7 +59,20 @@ struct FusedArgs {
     const float* scale[4];          // [n_t] gradient with respect to each row's value, or null (ones)
     float* value[4];                // [n_t]
     float* grad[4];                 // [n_t, 384], or null
+    const unsigned short* packed;   // the six weight matrices of every type already split (pack_weights_kernel), or null
 };
+
+// Packed weights: per type the six matrices one after the other (layer 1 as stored as three matrices of 128 columns),
+// each chunk by chunk of 16 k as [chunk][part][column][16 k] of bfloat16 -- what a workgroup would otherwise split again
+// for every tile of rows it takes, laid out so that a chunk's part is one contiguous run that the workgroup's
+// threads copy 8 bytes each.
+constexpr int kPackF1 = 0;                              // layer 1 transposed: 128 columns x 384
+constexpr int kPackF2 = kPackF1 + 3 * kN1 * kK1;        // layer 2 transposed: 128 x 128
+constexpr int kPackF3 = kPackF2 + 3 * kN2 * kN1;        // layer 3 transposed: 64 x 128
+constexpr int kPackB1 = kPackF3 + 3 * kN3 * kN2;        // layer 1 as stored: 384 columns x 128
+constexpr int kPackB2 = kPackB1 + 3 * kK1 * kN1;        // layer 2 as stored: 128 x 128
+constexpr int kPackB3 = kPackB2 + 3 * kN1 * kN2;        // layer 3 as stored: 128 x 64
+constexpr int kPackPerType = kPackB3 + 3 * kN2 * kN3;   // 442,368 bfloat16 values
 
 struct __align__(16) FusedLds {
     union {
@@ -117,8 +132,10 @@ struct Place {
 // (`wt`, row-major: one row per output column), chunk by chunk of 16 k.  A comes from the activation planes, or
 // (kAGlobal) from `arows` in memory, staged like the weights.  Ends with a barrier: afterwards nobody reads the planes
 // or the stage any more.
-template <int kK, int kNB, bool kAGlobal>
-__device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (&acc)[2], const float* __restrict__ wt,
+// kPacked: `wt` points at the matrix's packed chunks (bfloat16) and a piece is copied as it is; otherwise at float32
+// weights, split while they are staged.
+template <int kK, int kNB, bool kAGlobal, bool kPacked>
+__device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (&acc)[2], const void* __restrict__ wt,
                                               const float* __restrict__ arows, int row0, int n)
 {
     constexpr int chunks = kK / kKC;
@@ -126,30 +143,59 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
     const int r = P.tid >> 2, k4 = (P.tid & 3) << 2;     // this thread's piece of a chunk: row or column r, k4..k4+3
     const bool b_mine = r < kCols;                       // (the 64-column product: half of the threads stage weights)
     const int arow = min(row0 + r, n - 1);               // rows past the end: the last row again, never stored
-    v4 rb = v4{0.f, 0.f, 0.f, 0.f}, ra = v4{0.f, 0.f, 0.f, 0.f};
-    auto fetch = [&](int c) {
-        if (b_mine) rb = *reinterpret_cast<const v4*>(wt + static_cast<size_t>(r) * kK + c * kKC + k4);
-        if constexpr (kAGlobal) ra = *reinterpret_cast<const v4*>(arows + static_cast<size_t>(arow) * kK + c * kKC + k4);
+    // Two sets of registers for the pieces on their way from memory: a piece is asked for two chunks before it is
+    // staged and three before it is multiplied (with one set, one chunk ahead, every chunk waited for its weights to
+    // arrive from L2: the kernel ran at the pace of that latency).
+    struct Piece {
+        v4 b, a;
+        u2v p[3];
     };
-    auto stage = [&](int buf) {
-        if (b_mine) stage_piece(S.bstage[buf], r, k4, rb);
-        if constexpr (kAGlobal) stage_piece(S.astage[buf], r, k4, ra);
+    Piece R[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+        R[s].b = v4{0.f, 0.f, 0.f, 0.f};
+        R[s].a = v4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < 3; ++q) R[s].p[q] = u2v{0u, 0u};
+    }
+    auto fetch = [&](int c, Piece& x) {
+        if (b_mine) {
+            if constexpr (kPacked) {
+                const unsigned short* w = static_cast<const unsigned short*>(wt) + (c * 3 * kCols + r) * kKC + k4;
+#pragma unroll
+                for (int q = 0; q < 3; ++q) x.p[q] = *reinterpret_cast<const u2v*>(w + q * kCols * kKC);
+            } else {
+                x.b = *reinterpret_cast<const v4*>(static_cast<const float*>(wt) + static_cast<size_t>(r) * kK + c * kKC + k4);
+            }
+        }
+        if constexpr (kAGlobal) x.a = *reinterpret_cast<const v4*>(arows + static_cast<size_t>(arow) * kK + c * kKC + k4);
+    };
+    auto stage = [&](int buf, const Piece& x) {
+        if (b_mine) {
+            if constexpr (kPacked) {
+#pragma unroll
+                for (int q = 0; q < 3; ++q) *reinterpret_cast<u2v*>(&S.bstage[buf][q][r][k4]) = x.p[q];
+            } else {
+                stage_piece(S.bstage[buf], r, k4, x.b);
+            }
+        }
+        if constexpr (kAGlobal) stage_piece(S.astage[buf], r, k4, x.a);
     };
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
-    fetch(0);
-    stage(0);
-    if (chunks > 1) fetch(1);
+    static_assert(chunks % 2 == 0 && chunks >= 4, "the chunk loop is unrolled by two");
+    fetch(0, R[0]);
+    fetch(1, R[1]);
+    stage(0, R[0]);
+    fetch(2, R[0]);
     __syncthreads();             // chunk 0 is staged; the activation planes written before this call are complete
     const int col0 = kNB == 2 ? P.wc * 64 : P.wc * 32;
-    for (int c = 0; c < chunks; ++c) {
-        if (c + 1 < chunks) {
-            stage((c + 1) & 1);                          // the other buffer: last read before the previous barrier
-            if (c + 2 < chunks) fetch(c + 2);            // in flight during the products
-        }
-        bf16x8 av[3];
+    // chunk c: stage chunk c + 1 (its piece is in `x`) into the other buffer, ask for chunk c + 3, multiply chunk c
+    auto step = [&](int c, Piece& x) {
+        // this chunk's operands are asked for first: they arrive from LDS while the next chunk's piece is split
+        bf16x8 av[3], bv[2][3];
 #pragma unroll
         for (int m = 0; m < 3; ++m) {
             if constexpr (kAGlobal)
@@ -158,20 +204,30 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
                 av[m] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u4v*>(&S.act[m][P.wr * 32 + P.l32][c * kKC + P.half * 8]));
         }
 #pragma unroll
-        for (int j = 0; j < kNB; ++j) {
-            bf16x8 bv[3];
+        for (int j = 0; j < kNB; ++j)
 #pragma unroll
             for (int m = 0; m < 3; ++m)
-                bv[m] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u4v*>(&S.bstage[c & 1][m][col0 + j * 32 + P.l32][P.half * 8]));
+                bv[j][m] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u4v*>(&S.bstage[c & 1][m][col0 + j * 32 + P.l32][P.half * 8]));
+        asm volatile("" ::: "memory");                   // the reads above stay ahead of the stage's writes
+        if (c + 1 < chunks) {
+            stage((c + 1) & 1, x);                       // the other buffer: last read before the previous barrier
+            if (c + 3 < chunks) fetch(c + 3, x);
+        }
+#pragma unroll
+        for (int j = 0; j < kNB; ++j) {
             // smallest partial products first
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[2], bv[0], acc[j], 0, 0, 0);
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[2], acc[j], 0, 0, 0);
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[1], acc[j], 0, 0, 0);
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[0], acc[j], 0, 0, 0);
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[1], acc[j], 0, 0, 0);
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[0], acc[j], 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[2], bv[j][0], acc[j], 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][2], acc[j], 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[j][1], acc[j], 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[j][0], acc[j], 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][1], acc[j], 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][0], acc[j], 0, 0, 0);
         }
         __syncthreads();
+    };
+    for (int c = 0; c < chunks; c += 2) {
+        step(c, R[1]);
+        step(c + 1, R[0]);
     }
 }
 
@@ -197,7 +253,7 @@ __device__ __forceinline__ void to_planes(FusedLds& S, const Place& P, const v16
     }
 }
 
-template <bool kGrad>
+template <bool kGrad, bool kPacked>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
 {
@@ -215,9 +271,16 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
     const int first = t == 0 ? 0 : args.tile_end[t - 1];
     const int row0 = (tile - first) * kRows, n = args.n[t];
 
+    // a layer's weights: split beforehand, or float32 as the caller holds them
+    const unsigned short* const pk = kPacked ? args.packed + static_cast<size_t>(t) * kPackPerType : nullptr;
+    auto weights = [&](const float* plain, int packed_at) -> const void* {
+        if constexpr (kPacked) return pk + packed_at;
+        else return plain;
+    };
+
     v16 acc[2], a1[2], a2[2], a3[2];
     // ------------------------------------------------------------ layer 1: 384 -> 128
-    layer_product<kK1, 2, true>(S, P, acc, args.w1t[t], args.rows[t], row0, n);
+    layer_product<kK1, 2, true, kPacked>(S, P, acc, weights(args.w1t[t], kPackF1), args.rows[t], row0, n);
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const float b = args.b1[t][P.wc * 64 + j * 32 + P.l32];
@@ -226,7 +289,7 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
     }
     to_planes<2>(S, P, a1);
     // ------------------------------------------------------------ layer 2: 128 -> 128
-    layer_product<kN1, 2, false>(S, P, acc, args.w2t[t], nullptr, row0, n);
+    layer_product<kN1, 2, false, kPacked>(S, P, acc, weights(args.w2t[t], kPackF2), nullptr, row0, n);
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const float b = args.b2[t][P.wc * 64 + j * 32 + P.l32];
@@ -235,7 +298,7 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
     }
     to_planes<2>(S, P, a2);
     // ------------------------------------------------------------ layer 3: 128 -> 64, and the output layer 64 -> 1
-    layer_product<kN2, 1, false>(S, P, acc, args.w3t[t], nullptr, row0, n);
+    layer_product<kN2, 1, false, kPacked>(S, P, acc, weights(args.w3t[t], kPackF3), nullptr, row0, n);
     const int c3 = P.wc * 32 + P.l32;                    // this lane's column of the 64
     const float w4 = args.w4[t][c3];
     {
@@ -265,14 +328,14 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
         to_planes<1>(S, P, g3);
     }
     // g2 = (g3 W3^T) .* celu'(a2): 64 -> 128
-    layer_product<kN3, 2, false>(S, P, acc, args.w3[t], nullptr, row0, n);
+    layer_product<kN3, 2, false, kPacked>(S, P, acc, weights(args.w3[t], kPackB3), nullptr, row0, n);
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[j][e] *= celu_slope(a2[j][e], inv_alpha);
     to_planes<2>(S, P, acc);
     // g1 = (g2 W2^T) .* celu'(a1): 128 -> 128
-    layer_product<kN2, 2, false>(S, P, acc, args.w2[t], nullptr, row0, n);
+    layer_product<kN2, 2, false, kPacked>(S, P, acc, weights(args.w2[t], kPackB2), nullptr, row0, n);
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -281,7 +344,10 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
     // dx = g1 W1^T: 128 -> 384, three column tiles of 128
     float* __restrict__ out = args.grad[t];
     for (int ct = 0; ct < kK1 / 128; ++ct) {
-        layer_product<kN1, 2, false>(S, P, acc, args.w1[t] + static_cast<size_t>(ct) * 128 * kN1, nullptr, row0, n);
+        const void* w;
+        if constexpr (kPacked) w = pk + kPackB1 + static_cast<size_t>(ct) * 3 * 128 * kN1;
+        else w = args.w1[t] + static_cast<size_t>(ct) * 128 * kN1;
+        layer_product<kN1, 2, false, kPacked>(S, P, acc, w, nullptr, row0, n);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int col = ct * 128 + P.wc * 64 + j * 32 + P.l32;
@@ -294,18 +360,70 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
     }
 }
 
+// one float32 weight -> its three bfloat16 parts in the packed buffer; a thread per weight of one type's six matrices
+__global__ __launch_bounds__(256) void pack_weights_kernel(FusedArgs args, unsigned short* __restrict__ packed)
+{
+    const int t = blockIdx.y;
+    const int i = blockIdx.x * 256 + threadIdx.x;           // index among the type's 147,456 weights
+    constexpr int n1 = kN1 * kK1, n2 = kN2 * kN1, n3 = kN3 * kN2;
+    if (i >= 2 * (n1 + n2 + n3)) return;
+    const float* src;
+    int at, cols, k_len, j = i;      // the matrix: where it starts in the packed buffer, its columns and its summed length
+    if (j < n1) { src = args.w1t[t]; at = kPackF1; cols = kN1; k_len = kK1; }
+    else if ((j -= n1) < n2) { src = args.w2t[t]; at = kPackF2; cols = kN2; k_len = kN1; }
+    else if ((j -= n2) < n3) { src = args.w3t[t]; at = kPackF3; cols = kN3; k_len = kN2; }
+    else if ((j -= n3) < n1) {       // layer 1 as stored, [384][128]: three matrices of 128 columns
+        src = args.w1[t];
+        const int ct = j / (128 * kN1);
+        src += ct * 128 * kN1;
+        j -= ct * 128 * kN1;
+        at = kPackB1 + ct * 3 * 128 * kN1;
+        cols = 128;
+        k_len = kN1;
+    }
+    else if ((j -= n1) < n2) { src = args.w2[t]; at = kPackB2; cols = kN1; k_len = kN2; }
+    else { j -= n2; src = args.w3[t]; at = kPackB3; cols = kN2; k_len = kN3; }
+    unsigned p1, p2, p3;
+    split_pair(src[j], 0.f, p1, p2, p3);
+    const int r = j / k_len, k = j - r * k_len;
+    unsigned short* dst = packed + static_cast<size_t>(t) * kPackPerType + at + ((k / kKC) * 3 * cols + r) * kKC + (k % kKC);
+    dst[0] = static_cast<unsigned short>(p1 & 0xffffu);
+    dst[cols * kKC] = static_cast<unsigned short>(p2 & 0xffffu);
+    dst[2 * cols * kKC] = static_cast<unsigned short>(p3 & 0xffffu);
+}
+
 }  // namespace
+
+size_t networks_packed_bytes() { return static_cast<size_t>(4) * kPackPerType * sizeof(unsigned short); }
+
+// the six weight matrices of each type (three transposed, three as stored) split into `packed` (networks_packed_bytes())
+hipError_t launch_networks_pack(const float* const w1t[4], const float* const w2t[4], const float* const w3t[4],
+                                const float* const w1[4], const float* const w2[4], const float* const w3[4],
+                                void* packed, hipStream_t stream)
+{
+    FusedArgs a = {};
+    for (int t = 0; t < 4; ++t) {
+        a.w1t[t] = w1t[t]; a.w2t[t] = w2t[t]; a.w3t[t] = w3t[t];
+        a.w1[t] = w1[t]; a.w2[t] = w2[t]; a.w3[t] = w3[t];
+    }
+    constexpr int per_type = 2 * (kN1 * kK1 + kN2 * kN1 + kN3 * kN2);
+    pack_weights_kernel<<<dim3((per_type + 255) / 256, 4), dim3(256), 0, stream>>>(a, static_cast<unsigned short*>(packed));
+    return hipGetLastError();
+}
 
 // rows[t]: [n[t], 384]; w*t: transposed weights ([out, in]); w*: as stored ([in, out]); value[t]: [n[t]];
 // grad[t]: [n[t], 384] or null pointers (then only the values are formed; w1, w2, w3 and scale are not read).
+// packed: the weights as launch_networks_pack left them (then w*t and w* are not read), or null.
 hipError_t launch_networks_fused(const float* const rows[4], const int32_t n[4],
                                  const float* const w1t[4], const float* const w2t[4], const float* const w3t[4],
                                  const float* const w1[4], const float* const w2[4], const float* const w3[4],
                                  const float* const b1[4], const float* const b2[4], const float* const b3[4],
                                  const float* const w4[4], const float* const b4[4], const float* const scale[4],
-                                 float alpha, float* const value[4], float* const grad[4], hipStream_t stream)
+                                 float alpha, float* const value[4], float* const grad[4], const void* packed,
+                                 hipStream_t stream)
 {
-    FusedArgs a;
+    FusedArgs a = {};
+    a.packed = static_cast<const unsigned short*>(packed);
     int tiles = 0;
     bool want_grad = false;
     for (int t = 0; t < 4; ++t) {
@@ -313,7 +431,7 @@ hipError_t launch_networks_fused(const float* const rows[4], const int32_t n[4],
         a.n[t] = n[t];
         tiles += (n[t] + kRows - 1) / kRows;
         a.tile_end[t] = tiles;
-        a.w1t[t] = w1t[t]; a.w2t[t] = w2t[t]; a.w3t[t] = w3t[t];
+        a.w1t[t] = w1t ? w1t[t] : nullptr; a.w2t[t] = w2t ? w2t[t] : nullptr; a.w3t[t] = w3t ? w3t[t] : nullptr;
         a.w1[t] = w1 ? w1[t] : nullptr; a.w2[t] = w2 ? w2[t] : nullptr; a.w3[t] = w3 ? w3[t] : nullptr;
         a.b1[t] = b1[t]; a.b2[t] = b2[t]; a.b3[t] = b3[t];
         a.w4[t] = w4[t];
@@ -324,10 +442,14 @@ hipError_t launch_networks_fused(const float* const rows[4], const int32_t n[4],
         want_grad = want_grad || (grad && grad[t]);
     }
     if (tiles == 0) return hipSuccess;
-    if (want_grad)
-        networks_fused_kernel<true><<<dim3(static_cast<unsigned>(tiles)), dim3(kThreads), 0, stream>>>(a, alpha, 1.0f / alpha);
-    else
-        networks_fused_kernel<false><<<dim3(static_cast<unsigned>(tiles)), dim3(kThreads), 0, stream>>>(a, alpha, 1.0f / alpha);
+    const dim3 grid(static_cast<unsigned>(tiles)), block(kThreads);
+    if (want_grad) {
+        if (packed) networks_fused_kernel<true, true><<<grid, block, 0, stream>>>(a, alpha, 1.0f / alpha);
+        else networks_fused_kernel<true, false><<<grid, block, 0, stream>>>(a, alpha, 1.0f / alpha);
+    } else {
+        if (packed) networks_fused_kernel<false, true><<<grid, block, 0, stream>>>(a, alpha, 1.0f / alpha);
+        else networks_fused_kernel<false, false><<<grid, block, 0, stream>>>(a, alpha, 1.0f / alpha);
+    }
     return hipGetLastError();
 }
 

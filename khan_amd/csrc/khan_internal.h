@@ -143,7 +143,12 @@ hipError_t launch_networks_fused(const float* const rows[4], const int32_t n[4],
                                  const float* const w1[4], const float* const w2[4], const float* const w3[4],
                                  const float* const b1[4], const float* const b2[4], const float* const b3[4],
                                  const float* const w4[4], const float* const b4[4], const float* const scale[4],
-                                 float alpha, float* const value[4], float* const grad[4], hipStream_t stream);
+                                 float alpha, float* const value[4], float* const grad[4], const void* packed,
+                                 hipStream_t stream);
+size_t networks_packed_bytes();
+hipError_t launch_networks_pack(const float* const w1t[4], const float* const w2t[4], const float* const w3t[4],
+                                const float* const w1[4], const float* const w2[4], const float* const w3[4],
+                                void* packed, hipStream_t stream);
 hipError_t launch_dense_first(const float* const rows[4], const int32_t n[4], const float* const wt[4],
                               const float* const bias[4], bool celu, float alpha, float* const out[4],
                               hipStream_t stream);

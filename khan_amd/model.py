@@ -144,12 +144,19 @@ class MoleculeNN:
                 and not self.weights_need_grad)
 
     def one_launch_operands(self):
-        """-> (weights_t, weights, biases, head_weights, head_biases) as `ops.atomic_networks` takes them."""
+        """-> (packed weights, biases, head_weights, head_biases) as `ops.atomic_networks` takes them; the weights are
+        split into their bfloat16 parts once and kept until a weight is written again."""
+        from . import ops
         rows = [[self.names[t][k] for t in TYPE_MAP] for k in range(4)]
-        weights_t = [self.layer_transposed(k) for k in range(3)]
-        weights = [[self.params[r[0]].detach() for r in rows[k]] for k in range(3)]
+        ws = [self.params[r[0]] for k in range(3) for r in rows[k]]
+        key = tuple((w.data_ptr(), w._version) for w in ws)
+        cache = self.__dict__.setdefault("_packed_cache", {})
+        if cache.get("key") != key:
+            weights_t = [self.layer_transposed(k) for k in range(3)]
+            weights = [[self.params[r[0]].detach() for r in rows[k]] for k in range(3)]
+            cache["key"], cache["packed"] = key, ops.pack_network_weights(weights_t, weights)
         biases = [[self.params[r[1]].detach() for r in rows[k]] for k in range(3)]
-        return weights_t, weights, biases, [self.params[r[0]].detach() for r in rows[3]], [self.params[r[1]].detach() for r in rows[3]]
+        return cache["packed"], biases, [self.params[r[0]].detach() for r in rows[3]], [self.params[r[1]].detach() for r in rows[3]]
 
     def atom_outputs(self, atom_type_features, gather_idxs):
         """Per-type flat feature buckets -> one number per atom in the batch's atom order (nn.py:176-177)."""
@@ -240,8 +247,8 @@ class AniModel:
             # feature rows) -> sums by molecule; the coordinate gradient is featurize_grad of those rows' gradients
             feats = ops.featurize(xs, ys, zs, b.atom_types, b.mol_offsets, b.mol_atom_counts, b.scatter_idxs, acs,
                                   order=order, size_classes=classes)
-            weights_t, weights, biases, head_w, head_b = self.near.one_launch_operands()
-            values, grads = ops.atomic_networks(feats, weights_t, biases, head_w, head_b, weights=weights, want_grad=need_grad)
+            packed, biases, head_w, head_b = self.near.one_launch_operands()
+            values, grads = ops.atomic_networks(feats, None, biases, head_w, head_b, want_grad=need_grad, packed=packed)
             energies = ops.mol_energy(values, b.atom_types, b.scatter_idxs, b.mol_offsets, b.mol_atom_counts)
             if not need_grad:
                 return energies, None

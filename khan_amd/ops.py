@@ -469,17 +469,36 @@ def dense_head_grad(scales, head_weights, weights_nk, deriv_of, alpha=0.1):
 NETWORK_WIDTHS = (384, 128, 128, 64)      # the layer widths `atomic_networks` is built for (then 64 -> 1)
 
 
+_NETWORK_SHAPES_T = ((128, 384), (128, 128), (64, 128))
+
+
+def pack_network_weights(weights_t, weights):
+    """The 24 weight matrices of `atomic_networks` (weights_t[l][t] transposed, weights[l][t] as stored) split once into
+    their bfloat16 parts: -> a uint8 device buffer to pass as `packed=`.  Pack again after the weights change."""
+    lib = _lib.load()
+    wts, ws = [], []
+    for l in range(3):
+        for t in range(4):
+            n_out, k = _NETWORK_SHAPES_T[l]
+            wts.append(_dense_weights(weights_t[l][t], n_out, k, "weights_t[%d][%d]" % (l, t)))
+            ws.append(_dense_weights(weights[l][t], k, n_out, "weights[%d][%d]" % (l, t)))
+    packed = torch.empty(int(lib.khan_atomic_networks_packed_bytes()), dtype=torch.uint8, device=wts[0].device)
+    p12 = lambda ts: (ctypes.c_void_p * 12)(*[t.data_ptr() for t in ts])
+    _lib.check(lib.khan_atomic_networks_pack_f32(p12(wts), p12(ws), _p(packed), _stream()))
+    return packed
+
+
 def atomic_networks(rows, weights_t, biases, head_weights, head_biases=None, weights=None, scales=None, want_grad=False,
-                    alpha=0.1):
+                    alpha=0.1, packed=None):
     """The 384-128-128-64-1 CELU networks of the four atom types in one launch, float32: -> (values, grads).
     values[t] is [n_t], the network's output for every feature row of rows[t] ([n_t, 384] or a flat bucket); with
     `want_grad`, grads[t] ([n_t, 384]) is scales[t][:, None] * d values[t] / d rows[t] (scales None: ones), formed in
     the same launch without any hidden layer's activations going to memory; otherwise grads is None.
     weights_t[l][t]: layer l = 0, 1, 2 transposed ([128, 384], [128, 128], [64, 128]); weights[l][t]: the same layers as
-    stored ([384, 128], [128, 128], [128, 64]; needed with want_grad); biases[l][t]; head_weights[t] (64 values),
+    stored ([384, 128], [128, 128], [128, 64]; needed with want_grad); or `packed` = pack_network_weights(...) of the
+    same matrices (then weights_t and weights may be None).  biases[l][t]; head_weights[t] (64 values),
     head_biases[t] (one value)."""
     lib = _lib.load()
-    shapes_t = ((128, 384), (128, 128), (64, 128))
     xs, ns, vals, grads = [], [], [], []
     for t in range(4):
         x = _dense_matrix(rows[t].reshape(-1, 384), 384, "rows[%d]" % t)
@@ -491,12 +510,17 @@ def atomic_networks(rows, weights_t, biases, head_weights, head_biases=None, wei
     wts, ws, bs = [], [], []
     for l in range(3):
         for t in range(4):
-            wts.append(_dense_weights(weights_t[l][t], shapes_t[l][0], shapes_t[l][1], "weights_t[%d][%d]" % (l, t)))
+            n_out, k = _NETWORK_SHAPES_T[l]
             bs.append(_dev(biases[l][t].reshape(-1), torch.float32, "biases"))
-            if bs[-1].numel() != shapes_t[l][0]:
-                raise ValueError("biases[%d][%d] must have %d elements" % (l, t, shapes_t[l][0]))
-            if want_grad:
-                ws.append(_dense_weights(weights[l][t], shapes_t[l][1], shapes_t[l][0], "weights[%d][%d]" % (l, t)))
+            if bs[-1].numel() != n_out:
+                raise ValueError("biases[%d][%d] must have %d elements" % (l, t, n_out))
+            if packed is None:
+                wts.append(_dense_weights(weights_t[l][t], n_out, k, "weights_t[%d][%d]" % (l, t)))
+                if want_grad:
+                    ws.append(_dense_weights(weights[l][t], k, n_out, "weights[%d][%d]" % (l, t)))
+    if packed is not None and (packed.dtype != torch.uint8 or not packed.is_cuda
+                               or packed.numel() != int(lib.khan_atomic_networks_packed_bytes())):
+        raise ValueError("packed must be the buffer pack_network_weights returned")
     hws = [_dev(h.reshape(-1), torch.float32, "head_weights") for h in head_weights]
     if any(h.numel() != 64 for h in hws):
         raise ValueError("head_weights must have 64 elements each")
@@ -507,7 +531,8 @@ def atomic_networks(rows, weights_t, biases, head_weights, head_biases=None, wei
         if any(sc.numel() != n for sc, n in zip(scs, ns)):
             raise ValueError("scales[t] must have one element per row")
     p12 = lambda ts: (ctypes.c_void_p * 12)(*[t.data_ptr() for t in ts])
-    _lib.check(lib.khan_atomic_networks_f32(_ptr4(xs), (ctypes.c_int32 * 4)(*ns), p12(wts), p12(ws) if want_grad else None,
+    _lib.check(lib.khan_atomic_networks_f32(_ptr4(xs), (ctypes.c_int32 * 4)(*ns), p12(wts) if wts else None,
+                                            p12(ws) if ws else None, None if packed is None else _p(packed),
                                             p12(bs), _ptr4(hws), None if hbs is None else _ptr4(hbs),
                                             None if scs is None else _ptr4(scs), float(alpha), _ptr4(vals),
                                             _ptr4(grads) if want_grad else None, _stream()))

@@ -598,6 +598,12 @@ def test_whole_network_in_one_launch_matches_float64(with_scale):
                                       scales=[d(sc) for sc in scales] if with_scale else None, want_grad=True)
     vals_only, none = ops.atomic_networks(rows, weights_t, biases, [d(w) for w in w4], [d(b_) for b_ in b4])
     assert none is None
+    # the weights split once beforehand: the same bits out
+    packed = ops.pack_network_weights(weights_t, weights)
+    vals_p, grads_p = ops.atomic_networks(rows, None, biases, [d(w) for w in w4], [d(b_) for b_ in b4], packed=packed,
+                                          scales=[d(sc) for sc in scales] if with_scale else None, want_grad=True)
+    for t in range(4):
+        assert torch.equal(vals_p[t], vals[t]) and torch.equal(grads_p[t], grads[t])
     for t in range(4):
         up = lambda a: f32(a).astype(np.float64)
         sc = up(scales[t]) if with_scale else np.ones(ns[t])
