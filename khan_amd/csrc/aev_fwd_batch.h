@@ -295,6 +295,9 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB, kRadN
             continue;
         }
 
+        // Phase 2 is a chain of short dependent steps (a test, a branch, one multiply-add), bound by their latency, where
+        // phase 1 is vector arithmetic: a wavefront in phase 2 goes first when both are ready (1.5 % of the kernel).
+        __builtin_amdgcn_s_setprio(1);
         // phase 2: lane = (half, theta_t, Rs_s); the halves take alternate records.  Records past
         // `total` in the last step are zeros, so whole groups of eight pairs can always be run.
         const int npairs = min(64, total - base) >> 1;
@@ -365,6 +368,7 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB, kRadN
                 run8(q0 + 8, v1);
             }
         }
+        __builtin_amdgcn_s_setprio(0);
         wave_lds_fence();
     }
     if (total > 0) {

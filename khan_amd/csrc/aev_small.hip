@@ -42,10 +42,10 @@ constexpr int kRadSlots = 96;
 // With kJvp the kernel computes the Jacobian-vector product instead (featurize_grad_inverse): every term of
 // the forward sums is replaced by its derivative along the per-atom vectors (VX, VY, VZ).
 // float: 4 wavefronts per SIMD (LDS 9.8 KB, <= 128 VGPRs; the kernel loses a fifth of its speed at three);
-// double or kJvp: 2 (LDS 19 KB); both: 1.
+// float kJvp: 3 (<= 168 VGPRs; its LDS, 16.2 KB, lets ten wavefronts share a CU); double: 2 (LDS 19 KB); double kJvp: 1.
 template <typename T, bool kJvp, bool kMatrixPhase2 = false>
 __global__ __launch_bounds__(64 * kWavesPerBlock)
-__attribute__((amdgpu_waves_per_eu((sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1), (sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1) + ((kJvp && sizeof(T) == 4) ? 1 : 0))))
+__attribute__((amdgpu_waves_per_eu((kJvp && sizeof(T) == 4) ? 3 : (sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1), (kJvp && sizeof(T) == 4) ? 3 : (sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1))))
 void aev_fwd_small_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const T* __restrict__ Z,
     const int32_t* __restrict__ A, const int32_t* __restrict__ MOs,
