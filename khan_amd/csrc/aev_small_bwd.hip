@@ -75,7 +75,7 @@ void aev_bwd_small_kernel(
         y = Y[off + lane];
         z = Z[off + lane];
         type = fold_type(A[off + lane]);
-        rowbits = reinterpret_cast<unsigned long long>(gin.p[type] + static_cast<size_t>(SIs[off + lane]) * kFeats);
+        rowbits = reinterpret_cast<unsigned long long>(gin.p[type] + (kOneUpstreamRow ? size_t(0) : static_cast<size_t>(SIs[off + lane]) * kFeats));
     }
     int tcount[4], tbase[4];
     int dest = lane;

@@ -12,7 +12,8 @@ namespace khan {
 
 // Measurement builds only (khan_amd/build.py: build_stage_variants): KHAN_PROFILE_SKIP compiles a stage of the AEV
 // kernels out, so that the time of the rest can be measured.  Bit 0: the angular part, bit 1: the radial part, bit 2: the
-// forward kernels' stores of feature rows (the values are still computed).
+// forward kernels' stores of feature rows (the values are still computed), bit 3: every atom reads the upstream row of
+// the first atom of its type (the small backward kernel: its loads then hit the caches).
 // Such a library gives wrong results by design and is never the one the package loads by default.
 #ifndef KHAN_PROFILE_SKIP
 #define KHAN_PROFILE_SKIP 0
@@ -20,6 +21,7 @@ namespace khan {
 constexpr bool kSkipAngular = (KHAN_PROFILE_SKIP & 1) != 0;
 constexpr bool kSkipRadial = (KHAN_PROFILE_SKIP & 2) != 0;
 constexpr bool kSkipStores = (KHAN_PROFILE_SKIP & 4) != 0;
+constexpr bool kOneUpstreamRow = (KHAN_PROFILE_SKIP & 8) != 0;
 
 constexpr int kNumTypes = 4;
 constexpr int kNumRRs = 16;
