@@ -178,6 +178,8 @@ def inference_bench(args, batch):
     sizes = (384,) + tuple(model.DEFAULT_LAYERS)
     macs_per_atom = sum(x * y for x, y in zip(sizes[:-1], sizes[1:]))
     gemm_flops = 2 * macs_per_atom * N * 2            # forward, and the data gradient on the way back
+    import bench_profiling as profiling
+    net_traffic, net_stale, _ = profiling.measured_traffic("organic%d" % n_mols, "networks")
     return ({
         "metric": "ANI-1 energy + coordinate-gradient inference atoms/sec, fp32, 1 MI355X",
         "value": N / (ms_per_step * 1e-3), "unit": "atoms/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -188,7 +190,10 @@ def inference_bench(args, batch):
         "molecules_per_s": n_mols / (ms_per_step * 1e-3),
         "networks": {"one_launch_ms_per_step": ms_per_step, "layer_by_layer_kernels_ms_per_step": ms_layers,
                      "library_ms_per_step": ms_library, "max_relative_energy_difference_to_library": agree,
-                     "max_relative_gradient_difference_to_library": agree_g},
+                     "max_relative_gradient_difference_to_library": agree_g,
+                     # khan_atomic_networks_f32 with the gradient: feature rows read, gradient rows written
+                     "algorithmic_bytes_per_launch": 2 * N * 384 * 4 + N * 4,
+                     "hbm_bytes_per_launch": net_traffic, "hbm_bytes_stale": net_stale},
         "dense_products": "float32 operands split exactly into three bfloat16 parts, six partial products per pair on "
                           "v_mfma_f32_32x32x16_bf16, float32 accumulation (KHAN_DENSE_MATRIX=f32 selects "
                           "v_mfma_f32_32x32x2_f32)" if os.environ.get("KHAN_DENSE_MATRIX") != "f32" else "v_mfma_f32_32x32x2_f32",
@@ -313,9 +318,14 @@ def main():
     ap.add_argument("--headline-only", action="store_true",
                     help="with the default workload: leave out the shorter runs of the other configurations "
                          "(`configs` in the printed line)")
-    ap.add_argument("--traffic-probe", choices=("fwd", "bwd"), default=None,
-                    help="counter-collection mode: launch that pass twice, then a plain 64 MiB device copy of "
-                         "known traffic (scales FETCH_SIZE / WRITE_SIZE), print nothing else and exit")
+    ap.add_argument("--traffic-probe", choices=("fwd", "bwd", "networks", "charges"), default=None,
+                    help="counter-collection mode: launch that pass twice (fwd, bwd: the AEV passes; networks: "
+                         "khan_atomic_networks_f32 with its gradient on the workload's feature rows; charges: "
+                         "khan_ani_charge_all), then a plain 64 MiB device copy of known traffic (scales FETCH_SIZE / "
+                         "WRITE_SIZE), print nothing else and exit")
+    ap.add_argument("--reproducible-gradients", action="store_true",
+                    help="time (or probe) the backward pass with khan_set_reproducible_gradients(1): forces of molecules "
+                         "of 33-256 atoms summed in a fixed order in LDS instead of by atomics")
     ap.add_argument("--phase2", choices=("vector", "matrix"), default="vector",
                     help="matrix: measure the variant of the small-molecule forward kernel that sums the angular "
                          "records on the matrix cores (loads the check build of the library, which alone holds it, "
@@ -335,6 +345,9 @@ def main():
     _lib.load()   # fails loudly if the HIP library is missing
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
+    if args.reproducible_gradients:
+        from khan_amd import ops as _ops
+        _ops.set_reproducible_gradients(True)
     result = run_workload(args, args.workload, args.steps, args.warmup, cpu=not args.no_cpu_baseline)
     if result is None:
         return
@@ -388,7 +401,7 @@ def run_workload(args, workload, steps, warmup, cpu):
         return inference_bench(args, batch)
     if args.workload.startswith("grad_inverse"):
         return grad_inverse_bench(args, batch, w, kind)
-    if args.workload.startswith("charges_"):
+    if args.workload.startswith("charges_") and not args.traffic_probe:
         return charges_bench(args, batch, w)
     N = batch.n_atoms
     counts = batch.work_counts()
@@ -412,11 +425,23 @@ def run_workload(args, workload, steps, warmup, cpu):
         for c in acs.tolist():
             grads.append(upstream[start * 384:(start + c) * 384])
             start += c
+        if args.traffic_probe == "networks":
+            from khan_amd import model
+            net = model.AniModel(model.DEFAULT_LAYERS, model.celu, torch.float32, dev, seed=1).near
+            feats = ops.featurize(X, Y, Z, A, mos, macs, sc, acs)
+            packed, biases, head_w, head_b = net.one_launch_operands()
+        if args.traffic_probe == "charges":
+            Qp = torch.from_numpy(datagen.charges(N)).to(dev).to(tdt)
+            ones_p = torch.ones(n_mols, dtype=tdt, device=dev)
         for _ in range(2):
             if args.traffic_probe == "fwd":
                 ops.featurize(X, Y, Z, A, mos, macs, sc, acs)
-            else:
+            elif args.traffic_probe == "bwd":
                 ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *grads)
+            elif args.traffic_probe == "networks":
+                ops.atomic_networks(feats, None, biases, head_w, head_b, want_grad=True, packed=packed)
+            else:
+                ops.ani_charge_all(X, Y, Z, Qp, mos, macs, ones_p)
         src = torch.empty(64 * 1024 * 1024 // 4, dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)
         dst.copy_(src)
@@ -602,6 +627,8 @@ def run_workload(args, workload, steps, warmup, cpu):
         "molecules_per_s": n_mols / (ms_per_step * 1e-3),
         "roofline": roofline,
     }
+    if args.reproducible_gradients:
+        result["config"]["backward"] = "khan_set_reproducible_gradients(1): not the default kernel for molecules of 33-256 atoms"
     if args.phase2 != "vector":
         result["config"]["forward_phase2"] = args.phase2 + " cores (measurement variant, not the default kernel)"
     if not args.no_cpu_baseline:

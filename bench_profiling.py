@@ -16,8 +16,13 @@ Refreshing an entry (on a GPU box; four counter passes, one counter each, each a
 known; the counters of the pass are scaled by what they read for that copy.
 
 Time by stage (`python bench_profiling.py stages --workload W`): the passes are timed on the default library and on
-three measurement builds with the angular part, the radial part or both compiled out
+measurement builds with the angular part, the radial part or both compiled out, with the forward kernels' stores of
+the feature rows compiled out, and with the backward kernels reading every upstream row from one cached row
 (`python -m khan_amd.build --stage-variants`, built beforehand); differences of those times are the stages.
+
+`--traffic-probe networks` (on an AEV workload, whose feature rows it takes) and `--traffic-probe charges` (on a
+charges workload) do the same for khan_atomic_networks_f32 and khan_ani_charge_all; `python3 bench_profiling.py
+traffic --workload W --dir OUT --passes networks` reads OUT/networks_fetch and OUT/networks_write.
 """
 import csv
 import glob
@@ -43,14 +48,21 @@ DOMINANT = {
     ("organic16384_f64", "fwd"): "aev_fwd_small_kernel<double, false, false>",
     ("organic16384_f64", "bwd"): "aev_bwd_small_kernel<double>",
     ("boxes4096", "fwd"): "aev_fwd_medium_kernel<float, false, false>",
-    ("boxes4096", "bwd"): "aev_bwd_medium_kernel<float, false>",
+    ("boxes4096", "bwd"): "aev_bwd_medium_kernel<float, false, false>",
+    ("organic65536", "networks"): "networks_fused_kernel<true, true>",
+    ("charges_boxes4096_f64", "charges"): "charge_tile_kernel<double",
 }
+# the sources an entry's digest covers, by pass
+_DIGEST_SOURCES = {"networks": ("dense_fused.hip", "khan_internal.h"), "charges": ("charges.hip", "khan_internal.h")}
 
 
-def kernel_sources_digest():
-    """Digest of the code of the AEV kernels the record is about (csrc/aev_*.hip, csrc/aev_*.h and the two shared
-    headers; comments left out) and of the build flags, 16 hex digits."""
+def kernel_sources_digest(which="fwd"):
+    """Digest of the code of the kernels the record is about (for the AEV passes csrc/aev_*.hip, csrc/aev_*.h and
+    the two shared headers; for `networks` and `charges` their translation unit; comments left out) and of the
+    build flags, 16 hex digits."""
     from khan_amd import build
+    if which in _DIGEST_SOURCES:
+        return build.sources_digest(list(_DIGEST_SOURCES[which]))
     names = [os.path.basename(n) for n in build.HIP_SOURCES + build.HIP_HEADERS]
     return build.sources_digest([n for n in names if n.startswith("aev_") or n in ("khan_internal.h", "khan_params.h")])
 
@@ -67,7 +79,7 @@ def measured_traffic(workload, which):
     e = load_records().get("%s/%s" % (workload, which))
     if e is None:
         return None, False, None
-    if e.get("sources_digest") != kernel_sources_digest():
+    if e.get("sources_digest") != kernel_sources_digest(which):
         return None, True, e
     return e["bytes"], False, e
 
@@ -96,18 +108,18 @@ def _last_value(rows, name_part):
     return best[1]
 
 
-def refresh(workload, directory):
-    """Reads the four counter passes under `directory` ({fwd,bwd}_{fetch,write}/) and rewrites the workload's
-    two entries of the record.  Returns the entries."""
+def refresh(workload, directory, passes=("fwd", "bwd")):
+    """Reads the counter passes under `directory` ({fwd,bwd}_{fetch,write}/, or those of `passes`) and rewrites the
+    workload's entries of the record.  Returns the entries."""
     rec = load_records()
-    digest = kernel_sources_digest()
     try:
         head = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip()
     except OSError:
         head = ""
     out = {}
-    for which in ("fwd", "bwd"):
+    for which in passes:
         kernel = DOMINANT[(workload, which)]
+        digest = kernel_sources_digest(which)
         vals = {}
         for counter, sub in (("FETCH_SIZE", "fetch"), ("WRITE_SIZE", "write")):
             rows = _counter_rows(os.path.join(directory, "%s_%s" % (which, sub)), counter)
@@ -183,7 +195,8 @@ def stage_times(workload):
     khan_amd.build.build_stage_variants), each library in a process of its own.  Returns {build: {fwd, bwd}}."""
     from khan_amd import build
     res = {}
-    for name, skip in (("full", 0), ("no angular part", 1), ("no radial part", 2), ("neither (skeleton)", 3)):
+    for name, skip in (("full", 0), ("no angular part", 1), ("no radial part", 2), ("neither (skeleton)", 3),
+                       ("forward stores nothing", 4), ("backward reads one cached upstream row", 8)):
         env = dict(os.environ)
         env.pop("KHAN_AEV_LIBRARY", None)
         if skip:
@@ -206,6 +219,11 @@ def print_stage_table(workload, res):
     print("|---|---|---|")
     for name, r in res.items():
         print("| %s | %.3f | %.3f |" % (name, r["fwd"], r["bwd"]))
+    print("| => forward: feature-row stores not hidden under the arithmetic | %.3f (%.0f %%) | |" % (
+        full["fwd"] - res["forward stores nothing"]["fwd"], 100 * (full["fwd"] - res["forward stores nothing"]["fwd"]) / full["fwd"]))
+    b1 = res["backward reads one cached upstream row"]["bwd"]
+    print("| => backward: upstream-row reads from HBM not hidden under the arithmetic | | %.3f (%.0f %%) |" % (
+        full["bwd"] - b1, 100 * (full["bwd"] - b1) / full["bwd"]))
     print("| => angular part (full - no angular) | %.3f (%.0f %%) | %.3f (%.0f %%) |" % tuple(
         x for w in ("fwd", "bwd") for x in (full[w] - res["no angular part"][w], 100 * (full[w] - res["no angular part"][w]) / full[w])))
     print("| => radial part (full - no radial) | %.3f (%.0f %%) | %.3f (%.0f %%) |" % tuple(
@@ -221,6 +239,7 @@ def main(argv=None):
     t = sub.add_parser("traffic", help="rewrite a workload's entries of profiles/hbm_traffic.json from counter runs")
     t.add_argument("--workload", required=True)
     t.add_argument("--dir", required=True, help="directory holding fwd_fetch/ fwd_write/ bwd_fetch/ bwd_write/")
+    t.add_argument("--passes", nargs="+", default=["fwd", "bwd"], choices=("fwd", "bwd", "networks", "charges"))
     sub.add_parser("digest", help="print the digest of the kernel sources in the tree")
     st = sub.add_parser("stages", help="time by stage of the AEV passes, from the measurement builds "
                                        "(python -m khan_amd.build --stage-variants)")
@@ -236,13 +255,12 @@ def main(argv=None):
     elif args.cmd == "stages":
         print_stage_table(args.workload, stage_times(args.workload))
     elif args.cmd == "show":
-        d = kernel_sources_digest()
         for k, e in sorted(load_records().items()):
             print("%-24s %-40s %8.1f MB  (fetch %.1f + write %.1f)  %s" % (
                 k, e["kernel"], e["bytes"] / 1e6, e["fetch_bytes"] / 1e6, e["write_bytes"] / 1e6,
-                "current" if e["sources_digest"] == d else "STALE (measured on %s)" % e["sources_digest"]))
+                "current" if e["sources_digest"] == kernel_sources_digest(e["pass"]) else "STALE (measured on %s)" % e["sources_digest"]))
     else:
-        for which, e in refresh(args.workload, args.dir).items():
+        for which, e in refresh(args.workload, args.dir, tuple(args.passes)).items():
             print("%s/%s  %s: fetch %.1f MB + write %.1f MB = %.1f MB per launch" % (
                 args.workload, which, e["kernel"], e["fetch_bytes"] / 1e6, e["write_bytes"] / 1e6, e["bytes"] / 1e6))
 

@@ -8,7 +8,7 @@ plus csrc/check_build/libkhan_aev.so, the same library with the check switches c
 which only the tests of those switches load.
 
 Run as ``python -m khan_amd.build`` or through ``__graft_entry__.build()``.
-``python -m khan_amd.build --stage-variants`` builds the three measurement libraries of `build_stage_variants`.
+``python -m khan_amd.build --stage-variants`` builds the measurement libraries of `build_stage_variants`.
 
 Every libkhan_aev.so gets a stamp beside it (``libkhan_aev.so.digest``): the digest of the sources and flags it was
 built from, written after the generated code has passed `check_dpp_sources` and the link has succeeded.
@@ -157,12 +157,17 @@ def stage_variant_path(skip):
     return os.path.join(STAGE_BUILDS, "skip%d" % skip, "libkhan_aev.so")
 
 
+STAGE_SKIPS = (1, 2, 3, 4, 8)
+STAGE_SOURCES = ("aev_small.hip", "aev_small_bwd.hip", "aev_medium.hip", "aev_medium_bwd.hip")
+
+
 def build_stage_variants():
     """Measurement builds of libkhan_aev.so with a stage of the AEV kernels compiled out (KHAN_PROFILE_SKIP = 1:
-    no angular part, 2: no radial part, 3: neither), for `python bench_profiling.py stages`.  Their results are
-    wrong by design; they are loaded only when KHAN_AEV_LIBRARY names them."""
-    return [build_hip(defines=("KHAN_PROFILE_SKIP=%d" % k,), out_dir=os.path.dirname(stage_variant_path(k)))
-            for k in (1, 2, 3)]
+    no angular part, 2: no radial part, 3: neither, 4: the forward kernels store no feature rows, 8: the backward
+    kernels read every upstream row from one cached row), for `python bench_profiling.py stages`.  Their results
+    are wrong by design; they are loaded only when KHAN_AEV_LIBRARY names them.  Call after `build_hip()`."""
+    return [build_hip(defines=("KHAN_PROFILE_SKIP=%d" % k,), out_dir=os.path.dirname(stage_variant_path(k)), sources=STAGE_SOURCES)
+            for k in STAGE_SKIPS]
 
 
 DPP_SOURCES = ["aev_small.hip", "aev_medium.hip"]     # translation units that use fma_quad (aev_small_common.h)
