@@ -116,7 +116,7 @@ __device__ __forceinline__ T bwd_radial_pair(const T* grow, int tj, T r, T inv)
 // partner c reads row j's block for c's type, and the two share r and with it every shell factor.  The result
 // times (x_c - x_j) is the whole radial force on c from this pair, so that nothing has to be added to j: j
 // receives the same when it is the centre.
-template <typename T>
+template <typename T, bool kLibraryCutoff = false>
 __device__ __forceinline__ T bwd_radial_pair_both(const T* grow_c, int tj, const T* grow_j, int tc, T r, T inv)
 {
     constexpr int kN = ShellWindow<T>::kShells;
@@ -125,7 +125,7 @@ __device__ __forceinline__ T bwd_radial_pair_both(const T* grow_c, int tj, const
     load_shell_window<T>(grow_c + tj * kNumRRs, q0, g, rs);
     load_shell_window<T>(grow_j + tc * kNumRRs, q0, w, rs);
     T fc, dfc;
-    Fast<T>::cutoff_grad(r, static_cast<T>(kR_Rc_f), fc, dfc);
+    cutoff_grad_as<T, kLibraryCutoff>(r, static_cast<T>(kR_Rc_f), fc, dfc);
 #pragma unroll
     for (int q = 0; q < kN; ++q) g[q] += w[q];
     return radial_shell_sum<T, kN>(g, rs, r, fc, dfc) * inv;

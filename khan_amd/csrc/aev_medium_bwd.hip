@@ -90,6 +90,9 @@ void aev_bwd_medium_kernel(
     static_assert(!(kLarge && kLocal), "forces in LDS: molecules of up to 256 atoms only");
     __shared__ MedBwdShared<T, kLarge, kLocal> M;
     constexpr int kMB = kMedBwdCentres<T>;
+    // the double kernel for 65-256 atoms runs at 256 registers (two workgroups per compute unit): with the cutoff's
+    // polynomial constants resident it spills 21 of them and is 8 % slower than with the library's cos and sin
+    constexpr bool kLibraryCutoff = sizeof(T) == 8 && !kLarge && !kLocal;
     __shared__ BwdPool<T, kMB> pools[4];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -234,7 +237,7 @@ void aev_bwd_medium_kernel(
                 // the pair's pull on the centre from both rows.  With forces in LDS the pair is queued once (by its
                 // centre of lower sorted position) and the partner gets minus this below; otherwise the partner gets
                 // its share when it is the centre
-                const T sc = bwd_radial_pair_both<T>(grow_c, tj, grow_j, tc, e.w, inv);
+                const T sc = bwd_radial_pair_both<T, kLibraryCutoff>(grow_c, tj, grow_j, tc, e.w, inv);
                 fx = sc * e.x;
                 fy = sc * e.y;
                 fz = sc * e.z;
@@ -463,7 +466,7 @@ void aev_bwd_medium_kernel(
                         const vec4 d = P.nbr[used + lane];
                         const T inv = Fast<T>::rcp(d.w);
                         T fc, dfc;
-                        Fast<T>::cutoff_grad(d.w, static_cast<T>(kA_Rc_f), fc, dfc);
+                        cutoff_grad_as<T, kLibraryCutoff>(d.w, static_cast<T>(kA_Rc_f), fc, dfc);
                         P.nbr[used + lane] = Fast<T>::make4(d.x * inv, d.y * inv, d.z * inv, d.w);
                         P.nbr_fc[used + lane] = Fast<T>::make2(fc, dfc);
                     }

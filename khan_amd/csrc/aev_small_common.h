@@ -358,10 +358,18 @@ template <> struct Fast<double> {
         sqrt_and_rcp(x, r, inv);
         return r;
     }
-    static __device__ __forceinline__ double sqrt_rn(double x) { return sqrt_(x); }
     static __device__ __forceinline__ double rcp(double x) { return rcp_newton(x); }
+    static __device__ __forceinline__ double sqrt_rn(double x) { return sqrt_(x); }
     static __device__ __forceinline__ double gauss(double eta, double d) { return exp(-eta * d * d); }
     // f_C = 0.5 cos(pi r / rc) + 0.5 = cos^2(y), f_C' = -(pi / rc) sin(y) cos(y), y = pi r / (2 rc) in [0, pi/2] for r <= rc
+    // the same from the library's cos and sin: three times the instructions, but no table of fifteen double constants
+    // kept in registers across the kernel (a kernel at its register limit takes this one)
+    static __device__ __forceinline__ void cutoff_grad_library(double r, double rc, double& fc, double& dfc)
+    {
+        const double w = kPi / rc;
+        fc = 0.5 * cos(w * r) + 0.5;
+        dfc = -0.5 * w * sin(w * r);
+    }
     static __device__ __forceinline__ double cutoff(double r, double rc)
     {
         double sn, cs;
@@ -376,5 +384,11 @@ template <> struct Fast<double> {
         dfc = (-kPi / rc) * sn * cs;
     }
 };
+// f_C and f_C' in the form a kernel asks for: `kLibrary` (double only) takes Fast<double>::cutoff_grad_library
+template <typename T, bool kLibrary> __device__ __forceinline__ void cutoff_grad_as(T r, T rc, T& fc, T& dfc)
+{
+    if constexpr (kLibrary && sizeof(T) == 8) Fast<T>::cutoff_grad_library(r, rc, fc, dfc);
+    else Fast<T>::cutoff_grad(r, rc, fc, dfc);
+}
 
 }  // namespace khan

@@ -9,16 +9,31 @@
 // rows (every activation written, read again by the next layer and once more on the way back); this one moves the rows
 // and their gradients, 2.4 GB, and the values.
 //
-// One workgroup of eight wavefronts owns 128 rows.  The products run on the bfloat16 matrix instructions with every
-// float32 operand split exactly into three bfloat16 parts and six partial products kept (dense_first.hip describes the
-// arithmetic: a float32 product to float32 accuracy).  A wavefront holds a 32 x 64 part of a layer's 128 x 128 output
+// One workgroup of eight wavefronts owns 128 rows.  The products run on the 16-bit matrix instructions
+// (v_mfma_f32_32x32x16_f16, sixteen times the rate of the float32 ones) with every float32 operand split into two
+// half-precision parts:
+//     x = h + 2^-11 l,   h = half(x),   l = half(2^11 (x - h))
+// h carries 11 significant bits, x - h is exact in float32 and at most 2^-12 |x|, and l carries its 11 leading bits:
+// |x - h - 2^-11 l| <= 2^-24 |x|, the rounding of float32 itself.  The residual is scaled by 2^11 so that it has
+// x's exponent and not one twelve binary orders below it, where half precision would run out of exponent for every
+// |x| < 0.25.  Of the four partial products of x w three are kept, each an exact 22-bit product accumulated in
+// float32, in two accumulators:
+//     hi += h_x h_w,   lo += h_x l_w + l_x h_w,   x w ~ hi + 2^-11 lo      (left out: l_x l_w 2^-22 <= 2^-24 |x w|)
+// which is a float32 product to float32 accuracy (three terms of 2^-24 |x w| each) from three matrix instructions;
+// the three-way bfloat16 split of dense_first.hip needs six.  What it costs is range: half precision ends at 65,504,
+// so an operand (feature, activation, weight) of that size or more gives NaN -- never a wrong finite number -- and an
+// |x| below 6e-5 keeps an absolute accuracy of 2^-36 instead of a relative one.  On the way back the gradient is
+// carried for a unit upstream factor and multiplied by the row's factor only when it is stored (the pass is linear
+// in it), so that the gradients' size inside the kernel does not depend on the caller's loss scale.
+// A wavefront holds a 32 x 64 part of a layer's 128 x 128 output
 // (32 x 32 of the 128 x 64 one) in accumulator registers, and keeps its part of a1, a2 and a3 in registers for the way
 // back, where the gradients arrive in the same places.  Between layers the activations (gradients) go to LDS already
-// split, as three planes [row][k] of bfloat16: the next product's row operand, read straight from there.  The weights
+// split, as two planes [row][k] of half precision: the next product's row operand, read straight from there.  The weights
 // stream from L2 in chunks of 16 k into a double-buffered LDS stage, one barrier per chunk -- split on the way, or, when
 // the caller has had them split once beforehand (launch_networks_pack: a quarter of the kernel's vector instructions
 // were the same weights being split again for every tile of rows), copied as they are; layer 1
-// stages its feature rows the same way in the space the activation planes take later.  LDS: 139 KB, one workgroup per CU.
+// stages its feature rows the same way in the space the activation planes take later.  LDS: 93 KB, one workgroup per CU
+// (the accumulators and the saved activations of eight more wavefronts would not fit the registers).
 #include "khan_internal.h"
 #include "khan_params.h"
 
@@ -30,16 +45,18 @@ typedef float v4 __attribute__((ext_vector_type(4)));
 typedef float v16 __attribute__((ext_vector_type(16)));
 typedef unsigned u2v __attribute__((ext_vector_type(2)));
 typedef unsigned u4v __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+typedef _Float16 h8v __attribute__((ext_vector_type(8)));
 typedef float f2v __attribute__((ext_vector_type(2)));
 
 constexpr int kRows = 128;          // rows per workgroup
 constexpr int kThreads = 512;
 constexpr int kK1 = 384, kN1 = 128, kN2 = 128, kN3 = 64;
-constexpr int kActStride = 136;     // bfloat16 elements between rows of the activation planes: 128 + 8 (16-byte reads without bank conflicts)
+constexpr int kActStride = 136;     // 16-bit elements between rows of the activation planes: 128 + 8 (16-byte reads without bank conflicts)
 constexpr int kKC = 16;             // k per staged chunk = one matrix instruction deep
-constexpr int kStStride = 24;       // bfloat16 elements between staged rows: 16 + 8
+constexpr int kStStride = 24;       // 16-bit elements between staged rows: 16 + 8
+constexpr int kParts = 2;           // half-precision parts per float32 operand
+constexpr float kResidualScale = 2048.0f, kResidualBack = 1.0f / 2048.0f;      // 2^11
 
 struct FusedArgs {
     const float* rows[4];           // [n_t, 384] feature rows per type
@@ -63,44 +80,46 @@ struct FusedArgs {
 };
 
 // Packed weights: per type the six matrices one after the other (layer 1 as stored as three matrices of 128 columns),
-// each chunk by chunk of 16 k as [chunk][part][column][16 k] of bfloat16 -- what a workgroup would otherwise split again
+// each chunk by chunk of 16 k as [chunk][part][column][16 k] of half precision -- what a workgroup would otherwise split again
 // for every tile of rows it takes, laid out so that a chunk's part is one contiguous run that the workgroup's
 // threads copy 8 bytes each.
 constexpr int kPackF1 = 0;                              // layer 1 transposed: 128 columns x 384
-constexpr int kPackF2 = kPackF1 + 3 * kN1 * kK1;        // layer 2 transposed: 128 x 128
-constexpr int kPackF3 = kPackF2 + 3 * kN2 * kN1;        // layer 3 transposed: 64 x 128
-constexpr int kPackB1 = kPackF3 + 3 * kN3 * kN2;        // layer 1 as stored: 384 columns x 128
-constexpr int kPackB2 = kPackB1 + 3 * kK1 * kN1;        // layer 2 as stored: 128 x 128
-constexpr int kPackB3 = kPackB2 + 3 * kN1 * kN2;        // layer 3 as stored: 128 x 64
-constexpr int kPackPerType = kPackB3 + 3 * kN2 * kN3;   // 442,368 bfloat16 values
+constexpr int kPackF2 = kPackF1 + kParts * kN1 * kK1;        // layer 2 transposed: 128 x 128
+constexpr int kPackF3 = kPackF2 + kParts * kN2 * kN1;        // layer 3 transposed: 64 x 128
+constexpr int kPackB1 = kPackF3 + kParts * kN3 * kN2;        // layer 1 as stored: 384 columns x 128
+constexpr int kPackB2 = kPackB1 + kParts * kK1 * kN1;        // layer 2 as stored: 128 x 128
+constexpr int kPackB3 = kPackB2 + kParts * kN1 * kN2;        // layer 3 as stored: 128 x 64
+constexpr int kPackPerType = kPackB3 + kParts * kN2 * kN3;   // 294,912 half-precision values
 
 struct __align__(16) FusedLds {
     union {
-        unsigned short act[3][kRows][kActStride];        // a layer's activations or gradients, split: [part][row][k]
-        unsigned short astage[2][3][kRows][kStStride];   // layer 1: chunks of the feature rows
+        unsigned short act[kParts][kRows][kActStride];        // a layer's activations or gradients, split: [part][row][k]
+        unsigned short astage[2][kParts][kRows][kStStride];   // layer 1: chunks of the feature rows
     };
-    unsigned short bstage[2][3][128][kStStride];         // chunks of the weights: [buffer][part][column][k]
+    unsigned short bstage[2][kParts][128][kStStride];         // chunks of the weights: [buffer][part][column][k]
     float rowval[2][kRows];                              // the output layer's partial sums; then the rows' upstream factors
 };
 
-// two floats -> their three bfloat16 parts, each pair packed into one register (first value in the low half)
-__device__ __forceinline__ void split_pair(float x0, float x1, unsigned& p1, unsigned& p2, unsigned& p3)
+// two floats -> their two half-precision parts (the value rounded, and 2^11 times what the rounding left), each pair
+// packed into one register (first value in the low half).  Both differences are exact in float32.
+__device__ __forceinline__ void split_pair(float x0, float x1, unsigned& p1, unsigned& p2)
 {
-    p1 = __builtin_bit_cast(unsigned, __builtin_convertvector(f2v{x0, x1}, bf16x2));
-    const float r0 = x0 - __uint_as_float(p1 << 16), r1 = x1 - __uint_as_float(p1 & 0xffff0000u);
-    p2 = __builtin_bit_cast(unsigned, __builtin_convertvector(f2v{r0, r1}, bf16x2));
-    const float s0 = r0 - __uint_as_float(p2 << 16), s1 = r1 - __uint_as_float(p2 & 0xffff0000u);
-    p3 = __builtin_bit_cast(unsigned, __builtin_convertvector(f2v{s0, s1}, bf16x2));
+    const h2v h = __builtin_convertvector(f2v{x0, x1}, h2v);
+    p1 = __builtin_bit_cast(unsigned, h);
+    // 2^11 x - 2^11 h in one fused multiply-add that reads h as it is (both products are exact, and so is the difference)
+    const float r0 = fmaf(static_cast<float>(h[0]), -kResidualScale, x0 * kResidualScale);
+    const float r1 = fmaf(static_cast<float>(h[1]), -kResidualScale, x1 * kResidualScale);
+    p2 = __builtin_bit_cast(unsigned, __builtin_convertvector(f2v{r0, r1}, h2v));
 }
 
-// a chunk piece (four consecutive k of one row or column) split into the three planes of a stage buffer
-__device__ __forceinline__ void stage_piece(unsigned short (&dst)[3][128][kStStride], int r, int k4, const v4 x)
+// a chunk piece (four consecutive k of one row or column) split into the planes of a stage buffer
+__device__ __forceinline__ void stage_piece(unsigned short (&dst)[kParts][128][kStStride], int r, int k4, const v4 x)
 {
-    unsigned lo[3], hi[3];
-    split_pair(x[0], x[1], lo[0], lo[1], lo[2]);
-    split_pair(x[2], x[3], hi[0], hi[1], hi[2]);
+    unsigned lo[kParts], hi[kParts];
+    split_pair(x[0], x[1], lo[0], lo[1]);
+    split_pair(x[2], x[3], hi[0], hi[1]);
 #pragma unroll
-    for (int q = 0; q < 3; ++q) *reinterpret_cast<u2v*>(&dst[q][r][k4]) = u2v{lo[q], hi[q]};
+    for (int q = 0; q < kParts; ++q) *reinterpret_cast<u2v*>(&dst[q][r][k4]) = u2v{lo[q], hi[q]};
 }
 
 __device__ __forceinline__ float celu_of(float v, float alpha, float inv_alpha)
@@ -132,7 +151,7 @@ struct Place {
 // (`wt`, row-major: one row per output column), chunk by chunk of 16 k.  A comes from the activation planes, or
 // (kAGlobal) from `arows` in memory, staged like the weights.  Ends with a barrier: afterwards nobody reads the planes
 // or the stage any more.
-// kPacked: `wt` points at the matrix's packed chunks (bfloat16) and a piece is copied as it is; otherwise at float32
+// kPacked: `wt` points at the matrix's packed chunks (half precision) and a piece is copied as it is; otherwise at float32
 // weights, split while they are staged.
 template <int kK, int kNB, bool kAGlobal, bool kPacked>
 __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (&acc)[2], const void* __restrict__ wt,
@@ -148,7 +167,7 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
     // arrive from L2: the kernel ran at the pace of that latency).
     struct Piece {
         v4 b, a;
-        u2v p[3];
+        u2v p[kParts];
     };
     Piece R[2];
 #pragma unroll
@@ -156,14 +175,14 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
         R[s].b = v4{0.f, 0.f, 0.f, 0.f};
         R[s].a = v4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int q = 0; q < 3; ++q) R[s].p[q] = u2v{0u, 0u};
+        for (int q = 0; q < kParts; ++q) R[s].p[q] = u2v{0u, 0u};
     }
     auto fetch = [&](int c, Piece& x) {
         if (b_mine) {
             if constexpr (kPacked) {
-                const unsigned short* w = static_cast<const unsigned short*>(wt) + (c * 3 * kCols + r) * kKC + k4;
+                const unsigned short* w = static_cast<const unsigned short*>(wt) + (c * kParts * kCols + r) * kKC + k4;
 #pragma unroll
-                for (int q = 0; q < 3; ++q) x.p[q] = *reinterpret_cast<const u2v*>(w + q * kCols * kKC);
+                for (int q = 0; q < kParts; ++q) x.p[q] = *reinterpret_cast<const u2v*>(w + q * kCols * kKC);
             } else {
                 x.b = *reinterpret_cast<const v4*>(static_cast<const float*>(wt) + static_cast<size_t>(r) * kK + c * kKC + k4);
             }
@@ -174,17 +193,21 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
         if (b_mine) {
             if constexpr (kPacked) {
 #pragma unroll
-                for (int q = 0; q < 3; ++q) *reinterpret_cast<u2v*>(&S.bstage[buf][q][r][k4]) = x.p[q];
+                for (int q = 0; q < kParts; ++q) *reinterpret_cast<u2v*>(&S.bstage[buf][q][r][k4]) = x.p[q];
             } else {
                 stage_piece(S.bstage[buf], r, k4, x.b);
             }
         }
         if constexpr (kAGlobal) stage_piece(S.astage[buf], r, k4, x.a);
     };
+    v16 lo[2];                   // the mixed partial products, 2^11 times their size
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
+        for (int e = 0; e < 16; ++e) {
+            acc[j][e] = 0.f;
+            lo[j][e] = 0.f;
+        }
     static_assert(chunks % 2 == 0 && chunks >= 4, "the chunk loop is unrolled by two");
     fetch(0, R[0]);
     fetch(1, R[1]);
@@ -195,40 +218,41 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
     // chunk c: stage chunk c + 1 (its piece is in `x`) into the other buffer, ask for chunk c + 3, multiply chunk c
     auto step = [&](int c, Piece& x) {
         // this chunk's operands are asked for first: they arrive from LDS while the next chunk's piece is split
-        bf16x8 av[3], bv[2][3];
+        h8v av[kParts], bv[2][kParts];
 #pragma unroll
-        for (int m = 0; m < 3; ++m) {
+        for (int m = 0; m < kParts; ++m) {
             if constexpr (kAGlobal)
-                av[m] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u4v*>(&S.astage[c & 1][m][P.wr * 32 + P.l32][P.half * 8]));
+                av[m] = __builtin_bit_cast(h8v, *reinterpret_cast<const u4v*>(&S.astage[c & 1][m][P.wr * 32 + P.l32][P.half * 8]));
             else
-                av[m] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u4v*>(&S.act[m][P.wr * 32 + P.l32][c * kKC + P.half * 8]));
+                av[m] = __builtin_bit_cast(h8v, *reinterpret_cast<const u4v*>(&S.act[m][P.wr * 32 + P.l32][c * kKC + P.half * 8]));
         }
 #pragma unroll
         for (int j = 0; j < kNB; ++j)
 #pragma unroll
-            for (int m = 0; m < 3; ++m)
-                bv[j][m] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u4v*>(&S.bstage[c & 1][m][col0 + j * 32 + P.l32][P.half * 8]));
+            for (int m = 0; m < kParts; ++m)
+                bv[j][m] = __builtin_bit_cast(h8v, *reinterpret_cast<const u4v*>(&S.bstage[c & 1][m][col0 + j * 32 + P.l32][P.half * 8]));
         asm volatile("" ::: "memory");                   // the reads above stay ahead of the stage's writes
         if (c + 1 < chunks) {
             stage((c + 1) & 1, x);                       // the other buffer: last read before the previous barrier
             if (c + 3 < chunks) fetch(c + 3, x);
         }
+        // independent accumulators alternate, so that no matrix instruction waits for the one before it
 #pragma unroll
-        for (int j = 0; j < kNB; ++j) {
-            // smallest partial products first
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[2], bv[j][0], acc[j], 0, 0, 0);
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][2], acc[j], 0, 0, 0);
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[j][1], acc[j], 0, 0, 0);
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[j][0], acc[j], 0, 0, 0);
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][1], acc[j], 0, 0, 0);
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][0], acc[j], 0, 0, 0);
-        }
+        for (int j = 0; j < kNB; ++j) lo[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[1], bv[j][0], lo[j], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < kNB; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[0], bv[j][0], acc[j], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < kNB; ++j) lo[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[0], bv[j][1], lo[j], 0, 0, 0);
         __syncthreads();
     };
     for (int c = 0; c < chunks; c += 2) {
         step(c, R[1]);
         step(c + 1, R[0]);
     }
+#pragma unroll
+    for (int j = 0; j < kNB; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[j][e] = fmaf(lo[j][e], kResidualBack, acc[j][e]);
 }
 
 // a wavefront's values of a layer (kNB blocks) -> the activation planes, split; column = k of the next product
@@ -241,11 +265,11 @@ __device__ __forceinline__ void to_planes(FusedLds& S, const Place& P, const v16
         const int col = col0 + j * 32 + P.l32;
 #pragma unroll
         for (int e = 0; e < 16; e += 2) {
-            unsigned p[3];
-            split_pair(v[j][e], v[j][e + 1], p[0], p[1], p[2]);
+            unsigned p[kParts];
+            split_pair(v[j][e], v[j][e + 1], p[0], p[1]);
             const int r0 = P.row(e), r1 = P.row(e + 1);
 #pragma unroll
-            for (int q = 0; q < 3; ++q) {
+            for (int q = 0; q < kParts; ++q) {
                 S.act[q][r0][col] = static_cast<unsigned short>(p[q] & 0xffffu);
                 S.act[q][r1][col] = static_cast<unsigned short>(p[q] >> 16);
             }
@@ -324,7 +348,7 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
     {
         v16 g3[2];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) g3[0][e] = S.rowval[0][P.row(e)] * w4 * celu_slope(a3[0][e], inv_alpha);
+        for (int e = 0; e < 16; ++e) g3[0][e] = w4 * celu_slope(a3[0][e], inv_alpha);     // for a unit upstream factor
         to_planes<1>(S, P, g3);
     }
     // g2 = (g3 W3^T) .* celu'(a2): 64 -> 128
@@ -343,9 +367,12 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
     to_planes<2>(S, P, acc);
     // dx = g1 W1^T: 128 -> 384, three column tiles of 128
     float* __restrict__ out = args.grad[t];
+    float upstream[16];          // the upstream factors of this lane's sixteen rows
+#pragma unroll
+    for (int e = 0; e < 16; ++e) upstream[e] = S.rowval[0][P.row(e)];
     for (int ct = 0; ct < kK1 / 128; ++ct) {
         const void* w;
-        if constexpr (kPacked) w = pk + kPackB1 + static_cast<size_t>(ct) * 3 * 128 * kN1;
+        if constexpr (kPacked) w = pk + kPackB1 + static_cast<size_t>(ct) * kParts * 128 * kN1;
         else w = args.w1[t] + static_cast<size_t>(ct) * 128 * kN1;
         layer_product<kN1, 2, false, kPacked>(S, P, acc, w, nullptr, row0, n);
 #pragma unroll
@@ -354,13 +381,13 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int gr = row0 + P.row(e);
-                if (gr < n) out[static_cast<size_t>(gr) * kK1 + col] = acc[j][e];
+                if (gr < n) out[static_cast<size_t>(gr) * kK1 + col] = acc[j][e] * upstream[e];
             }
         }
     }
 }
 
-// one float32 weight -> its three bfloat16 parts in the packed buffer; a thread per weight of one type's six matrices
+// one float32 weight -> its two half-precision parts in the packed buffer; a thread per weight of one type's six matrices
 __global__ __launch_bounds__(256) void pack_weights_kernel(FusedArgs args, unsigned short* __restrict__ packed)
 {
     const int t = blockIdx.y;
@@ -377,19 +404,18 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(FusedArgs args, unsig
         const int ct = j / (128 * kN1);
         src += ct * 128 * kN1;
         j -= ct * 128 * kN1;
-        at = kPackB1 + ct * 3 * 128 * kN1;
+        at = kPackB1 + ct * kParts * 128 * kN1;
         cols = 128;
         k_len = kN1;
     }
     else if ((j -= n1) < n2) { src = args.w2[t]; at = kPackB2; cols = kN1; k_len = kN2; }
     else { j -= n2; src = args.w3[t]; at = kPackB3; cols = kN2; k_len = kN3; }
-    unsigned p1, p2, p3;
-    split_pair(src[j], 0.f, p1, p2, p3);
+    unsigned p1, p2;
+    split_pair(src[j], 0.f, p1, p2);
     const int r = j / k_len, k = j - r * k_len;
-    unsigned short* dst = packed + static_cast<size_t>(t) * kPackPerType + at + ((k / kKC) * 3 * cols + r) * kKC + (k % kKC);
+    unsigned short* dst = packed + static_cast<size_t>(t) * kPackPerType + at + ((k / kKC) * kParts * cols + r) * kKC + (k % kKC);
     dst[0] = static_cast<unsigned short>(p1 & 0xffffu);
     dst[cols * kKC] = static_cast<unsigned short>(p2 & 0xffffu);
-    dst[2 * cols * kKC] = static_cast<unsigned short>(p3 & 0xffffu);
 }
 
 }  // namespace
