@@ -194,9 +194,10 @@ def inference_bench(args, batch):
                      # khan_atomic_networks_f32 with the gradient: feature rows read, gradient rows written
                      "algorithmic_bytes_per_launch": 2 * N * 384 * 4 + N * 4,
                      "hbm_bytes_per_launch": net_traffic, "hbm_bytes_stale": net_stale},
-        "dense_products": "float32 operands split exactly into three bfloat16 parts, six partial products per pair on "
-                          "v_mfma_f32_32x32x16_bf16, float32 accumulation (KHAN_DENSE_MATRIX=f32 selects "
-                          "v_mfma_f32_32x32x2_f32)" if os.environ.get("KHAN_DENSE_MATRIX") != "f32" else "v_mfma_f32_32x32x2_f32",
+        "dense_products": "one launch: float32 operands split into two half-precision parts (value rounded, 2^11 x residual), "
+                          "three partial products per pair on v_mfma_f32_32x32x16_f16, float32 accumulation; layer by layer: "
+                          + ("three bfloat16 parts, six partial products on v_mfma_f32_32x32x16_bf16"
+                             if os.environ.get("KHAN_DENSE_MATRIX") != "f32" else "v_mfma_f32_32x32x2_f32"),
         "roofline": {"kernel": "the atomic networks, forward and data gradient (khan_atomic_networks_f32): float32-equivalent "
                                "flops of the whole step against the float32 matrix peak",
                      "bound": "mfma", "achieved": gemm_flops / (ms_per_step * 1e-3) / 1e12,

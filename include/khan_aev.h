@@ -324,14 +324,22 @@ int khan_dense_head_grad_f32(const float *const *scale_host4, const float *const
  * A feature row is read once and its gradient written once; no activation of a hidden layer is written to memory
  * (layer by layer, khan_dense_f32 and khan_dense_head_f32 write every activation and read it twice).  It is the pass of
  * energy-and-force inference (energy_server.py:141-187): the values summed by molecule are the energies, and grad with
- * scale = 1 is what khan_featurize_grad_f32 takes as its upstream rows.  Float32 matrix products as in khan_dense_f32.
+ * scale = 1 is what khan_featurize_grad_f32 takes as its upstream rows.
+ * The products are float32 products to float32 accuracy, formed on the half-precision matrix instructions: every float32
+ * operand x is split into h = half(x) and l = half(2^11 (x - h)) (x - h - 2^-11 l is at most 2^-24 |x|), and three of
+ * the four partial products are accumulated in float32 (the fourth is below 2^-24 of the product).  OPERAND RANGE: a
+ * feature, activation or weight of 65,504 or more in size (half precision's largest number) makes that row's value and
+ * gradient NaN -- never a wrong finite number, and no other row's; an operand below 6e-5 in size keeps an absolute
+ * accuracy of 2^-36 instead of a relative one (it then no longer counts beside the row's other terms).  The gradient
+ * is carried through the layers for scale = 1 and multiplied by scale_t[r] when it is stored, so its accuracy does not
+ * depend on the size of scale.
  *   rows_host4[t]          [n_t, 384] feature rows (the featurizer's buckets), 16-byte aligned
  *   weights_t_host12[4l+t] layer l = 0, 1, 2 of type t TRANSPOSED: [128, 384], [128, 128], [64, 128]
  *   weights_host12[4l+t]   the same layers as stored: [384, 128], [128, 128], [128, 64] (read for the gradient only;
  *                          NULL when grad_host4 is NULL)
  *   packed                 DEVICE buffer written by khan_atomic_networks_pack_f32 from the same 24 matrices, or NULL.
  *                          With it neither weights array is read (both may be NULL) and the kernel copies the weights'
- *                          three bfloat16 parts instead of splitting them again for every 128 rows: the same bits out,
+ *                          two half-precision parts instead of splitting them again for every 128 rows: the same bits out,
  *                          a tenth less time.  Pack once per set of weights (khan_atomic_networks_packed_bytes() bytes,
  *                          16-byte aligned); pack again after the weights change.
  *   biases_host12[4l+t]    [128], [128], [64]

@@ -145,7 +145,7 @@ class MoleculeNN:
 
     def one_launch_operands(self):
         """-> (packed weights, biases, head_weights, head_biases) as `ops.atomic_networks` takes them; the weights are
-        split into their bfloat16 parts once and kept until a weight is written again."""
+        split into their half-precision parts once and kept until a weight is written again."""
         from . import ops
         rows = [[self.names[t][k] for t in TYPE_MAP] for k in range(4)]
         ws = [self.params[r[0]] for k in range(3) for r in rows[k]]

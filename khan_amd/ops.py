@@ -474,7 +474,7 @@ _NETWORK_SHAPES_T = ((128, 384), (128, 128), (64, 128))
 
 def pack_network_weights(weights_t, weights):
     """The 24 weight matrices of `atomic_networks` (weights_t[l][t] transposed, weights[l][t] as stored) split once into
-    their bfloat16 parts: -> a uint8 device buffer to pass as `packed=`.  Pack again after the weights change."""
+    their half-precision parts: -> a uint8 device buffer to pass as `packed=`.  Pack again after the weights change."""
     lib = _lib.load()
     wts, ws = [], []
     for l in range(3):
@@ -497,7 +497,9 @@ def atomic_networks(rows, weights_t, biases, head_weights, head_biases=None, wei
     weights_t[l][t]: layer l = 0, 1, 2 transposed ([128, 384], [128, 128], [64, 128]); weights[l][t]: the same layers as
     stored ([384, 128], [128, 128], [128, 64]; needed with want_grad); or `packed` = pack_network_weights(...) of the
     same matrices (then weights_t and weights may be None).  biases[l][t]; head_weights[t] (64 values),
-    head_biases[t] (one value)."""
+    head_biases[t] (one value).  The products are float32 products to float32 accuracy from two half-precision parts
+    per operand: features, activations and weights have to stay below 65,504 in size (beyond it the row's results are
+    NaN); the size of `scales` does not matter."""
     lib = _lib.load()
     xs, ns, vals, grads = [], [], [], []
     for t in range(4):

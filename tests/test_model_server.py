@@ -618,3 +618,56 @@ def test_whole_network_in_one_launch_matches_float64(with_scale):
         assert np.all(np.isfinite(got_v)) and np.abs(got_v - want_v).max() <= 2e-5 * vscale, (t, np.abs(got_v - want_v).max(), vscale)
         gscale = np.abs(want_g).max(axis=1, keepdims=True) + 1e-6
         assert np.all(np.isfinite(got_g)) and np.all(np.abs(got_g - want_g) <= 5e-5 * gscale), (t, (np.abs(got_g - want_g) / gscale).max())
+
+
+@pytest.mark.gpu
+def test_whole_network_operand_range():
+    """khan_atomic_networks_f32 forms its products from two half-precision parts per float32 operand.  Pinned here: the
+    accuracy does not depend on the size of the upstream factors (1e-8, 1e+6: the gradient is carried for a unit factor
+    and scaled when it is stored) nor degrade for small feature rows (1e-4), and a feature beyond half precision's
+    range (1e5 > 65,504) turns that row's value and gradient into NaN -- no wrong finite number -- and no other row's."""
+    from khan_amd import ops
+    dev = "cuda:0"
+    f32 = lambda a: np.ascontiguousarray(a.astype(np.float32))
+    d = lambda a: torch.from_numpy(f32(a)).to(dev)
+    up = lambda a: f32(a).astype(np.float64)
+    rng = np.random.default_rng(5)
+    widths = (384, 128, 128, 64)
+    n = 700
+    Ws = [rng.standard_normal((widths[l], widths[l + 1])) * (2.0 / (widths[l] + widths[l + 1])) ** 0.5 for l in range(3)]
+    bs = [rng.standard_normal(widths[l + 1]) * 0.1 for l in range(3)]
+    w4, b4 = rng.standard_normal(64) * 0.2, rng.standard_normal(1)
+    empty = torch.zeros((0, 384), device=dev)
+    none = torch.zeros(0, device=dev)
+    wt = [[d(Ws[l].T)] * 4 for l in range(3)]
+    w = [[d(Ws[l])] * 4 for l in range(3)]
+    bi = [[d(bs[l])] * 4 for l in range(3)]
+
+    def launch(x, sc):
+        vals, grads = ops.atomic_networks([empty, d(x), empty, empty], wt, bi, [d(w4)] * 4, [d(b4)] * 4, weights=w,
+                                          scales=[none, d(sc), none, none], want_grad=True)
+        return vals[1].cpu().numpy().astype(np.float64), grads[1].cpu().numpy().astype(np.float64)
+
+    worst = {}
+    for name, xscale, sscale in (("ordinary", 0.5, 1.0), ("features 1e-4", 1e-4, 1.0), ("upstream 1e-8", 0.5, 1e-8), ("upstream 1e+6", 0.5, 1e6)):
+        x = np.abs(rng.standard_normal((n, 384))) * xscale
+        sc = rng.standard_normal(n) * sscale
+        want_v, want_g = _network_f64(up(x), [up(W) for W in Ws], [up(b_) for b_ in bs], up(w4), up(b4)[0], up(sc))
+        got_v, got_g = launch(x, sc)
+        ev = np.abs(got_v - want_v).max() / (np.abs(want_v).max() + 1.0)
+        eg = (np.abs(got_g - want_g) / (np.abs(want_g).max(axis=1, keepdims=True) + 1e-300)).max()
+        worst[name] = (ev, eg)
+        assert np.isfinite(got_v).all() and np.isfinite(got_g).all(), name
+        assert ev <= 5e-6 and eg <= 2e-5, (name, ev, eg)
+    print("\none-launch networks, worst value / gradient error relative to the largest value / the row's largest entry:", worst)
+    # the same relative accuracy whatever the upstream factors' size
+    assert worst["upstream 1e-8"][1] <= 1.5 * worst["ordinary"][1] + 1e-6 and worst["upstream 1e+6"][1] <= 1.5 * worst["ordinary"][1] + 1e-6
+
+    x = np.abs(rng.standard_normal((n, 384))) * 0.5
+    sc = np.ones(n)
+    clean_v, clean_g = launch(x, sc)
+    x[300, 17] = 1.0e5
+    got_v, got_g = launch(x, sc)
+    assert not np.isfinite(got_v[300]) and not np.isfinite(got_g[300]).any()
+    keep = np.arange(n) != 300
+    assert np.array_equal(got_v[keep], clean_v[keep]) and np.array_equal(got_g[keep], clean_g[keep])
