@@ -49,8 +49,19 @@ typedef _Float16 h2v __attribute__((ext_vector_type(2)));
 typedef _Float16 h8v __attribute__((ext_vector_type(8)));
 typedef float f2v __attribute__((ext_vector_type(2)));
 
-constexpr int kRows = 128;          // rows per workgroup
-constexpr int kThreads = 512;
+#ifndef KHAN_FUSED_DEPTH1
+#define KHAN_FUSED_DEPTH1 4
+#endif
+#ifndef KHAN_FUSED_DEPTH
+#define KHAN_FUSED_DEPTH 4
+#endif
+constexpr int kDepthRows = KHAN_FUSED_DEPTH1;     // register sets of layer 1 (feature rows from HBM)
+constexpr int kDepthWeights = KHAN_FUSED_DEPTH;   // and of the other products (weights from L2)
+#ifndef KHAN_FUSED_ROWS
+#define KHAN_FUSED_ROWS 64
+#endif
+constexpr int kRows = KHAN_FUSED_ROWS;      // rows per workgroup: 64 (four wavefronts, two workgroups per CU) or 128 (eight, one)
+constexpr int kThreads = kRows * 4;         // a wavefront per 32 rows x 64 columns of a 128-wide output
 constexpr int kK1 = 384, kN1 = 128, kN2 = 128, kN3 = 64;
 constexpr int kActStride = 136;     // 16-bit elements between rows of the activation planes: 128 + 8 (16-byte reads without bank conflicts)
 constexpr int kKC = 16;             // k per staged chunk = one matrix instruction deep
@@ -96,7 +107,6 @@ struct __align__(16) FusedLds {
         unsigned short act[kParts][kRows][kActStride];        // a layer's activations or gradients, split: [part][row][k]
         unsigned short astage[2][kParts][kRows][kStStride];   // layer 1: chunks of the feature rows
     };
-    unsigned short bstage[2][kParts][128][kStStride];         // chunks of the weights: [buffer][part][column][k]
     float rowval[2][kRows];                              // the output layer's partial sums; then the rows' upstream factors
 };
 
@@ -113,7 +123,8 @@ __device__ __forceinline__ void split_pair(float x0, float x1, unsigned& p1, uns
 }
 
 // a chunk piece (four consecutive k of one row or column) split into the planes of a stage buffer
-__device__ __forceinline__ void stage_piece(unsigned short (&dst)[kParts][128][kStStride], int r, int k4, const v4 x)
+template <int kR>
+__device__ __forceinline__ void stage_piece(unsigned short (&dst)[kParts][kR][kStStride], int r, int k4, const v4 x)
 {
     unsigned lo[kParts], hi[kParts];
     split_pair(x[0], x[1], lo[0], lo[1]);
@@ -147,59 +158,75 @@ struct Place {
     __device__ __forceinline__ int row(int e) const { return wr * 32 + 8 * (e >> 2) + 4 * half + (e & 3); }
 };
 
-// One layer's product for this workgroup's 128 rows: acc = A . B^T, A = 128 x kK (rows), B = (kNB * 64) x kK
-// (`wt`, row-major: one row per output column), chunk by chunk of 16 k.  A comes from the activation planes, or
-// (kAGlobal) from `arows` in memory, staged like the weights.  Ends with a barrier: afterwards nobody reads the planes
-// or the stage any more.
-// kPacked: `wt` points at the matrix's packed chunks (half precision) and a piece is copied as it is; otherwise at float32
-// weights, split while they are staged.
-template <int kK, int kNB, bool kAGlobal, bool kPacked>
+// One layer's product for this workgroup's rows: acc = A . B^T, A = kRows x kK (rows), B = (kNB * 64) x kK (`wt`: one
+// row per output column), chunk by chunk of 16 k.
+// B never passes through LDS: a matrix instruction's operand is, per lane, eight consecutive k of one column -- 16
+// bytes of a packed chunk, and the 64 lanes' pieces are one contiguous kilobyte -- so every wavefront loads its own
+// operands straight into registers, kDepth chunks ahead (they come from L2, or from the compute unit's L1 when the
+// wavefront beside it has just asked for the same columns).  With the weights staged in LDS the kernel was bound by
+// LDS traffic: nine kilobytes read and written per wavefront and chunk for six matrix instructions, and a barrier
+// per chunk.  A comes from the activation planes, with no barrier inside the product; or (kAGlobal: layer 1) from
+// `arows` in memory through a double-buffered LDS stage (the rows are float32 and have to be split and regrouped), one
+// barrier per chunk.  Begins and ends with a barrier: the planes written before the call are complete, and afterwards
+// nobody reads the planes or the stage any more.
+// kPacked: `wt` points at the matrix's packed chunks (half precision); otherwise at float32 weights, of which a lane
+// loads its eight values and splits them itself.
+template <int kK, int kNB, bool kAGlobal, bool kPacked, int kDepth>
 __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (&acc)[2], const void* __restrict__ wt,
                                               const float* __restrict__ arows, int row0, int n)
 {
     constexpr int chunks = kK / kKC;
     constexpr int kCols = kNB * 64;                      // 128 or 64 output columns
-    const int r = P.tid >> 2, k4 = (P.tid & 3) << 2;     // this thread's piece of a chunk: row or column r, k4..k4+3
-    const bool b_mine = r < kCols;                       // (the 64-column product: half of the threads stage weights)
+    static_assert(chunks % kDepth == 0 && kDepth >= 2, "the chunk loop is unrolled by the number of register sets");
+    const int col0 = kNB == 2 ? P.wc * 64 : P.wc * 32;
+    // a chunk's operands for this wavefront's blocks, as loaded: the two parts (packed), or eight float32 weights
+    struct BSet {
+        u4v raw[kNB][2];
+    };
+    BSet B[kDepth];
+    auto bfetch = [&](int c, BSet& x) {
+#pragma unroll
+        for (int j = 0; j < kNB; ++j) {
+            const int col = col0 + j * 32 + P.l32;
+            if constexpr (kPacked) {
+                const unsigned short* w = static_cast<const unsigned short*>(wt) + (c * kParts * kCols + col) * kKC + P.half * 8;
+#pragma unroll
+                for (int m = 0; m < kParts; ++m) x.raw[j][m] = *reinterpret_cast<const u4v*>(w + m * kCols * kKC);
+            } else {
+                const float* w = static_cast<const float*>(wt) + static_cast<size_t>(col) * kK + c * kKC + P.half * 8;
+                x.raw[j][0] = *reinterpret_cast<const u4v*>(w);
+                x.raw[j][1] = *reinterpret_cast<const u4v*>(w + 4);
+            }
+        }
+    };
+    auto boperand = [&](const BSet& x, int j, h8v (&bv)[kParts]) {
+        if constexpr (kPacked) {
+#pragma unroll
+            for (int m = 0; m < kParts; ++m) bv[m] = __builtin_bit_cast(h8v, x.raw[j][m]);
+        } else {
+            u4v part[kParts];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const v4 f = __builtin_bit_cast(v4, x.raw[j][h]);
+                unsigned a[kParts], b[kParts];
+                split_pair(f[0], f[1], a[0], a[1]);
+                split_pair(f[2], f[3], b[0], b[1]);
+#pragma unroll
+                for (int m = 0; m < kParts; ++m) {
+                    part[m][2 * h] = a[m];
+                    part[m][2 * h + 1] = b[m];
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < kParts; ++m) bv[m] = __builtin_bit_cast(h8v, part[m]);
+        }
+    };
+    // layer 1: this thread's piece of a chunk of the feature rows: row r, k4..k4+3
+    const int r = P.tid >> 2, k4 = (P.tid & 3) << 2;
     const int arow = min(row0 + r, n - 1);               // rows past the end: the last row again, never stored
-    // Two sets of registers for the pieces on their way from memory: a piece is asked for two chunks before it is
-    // staged and three before it is multiplied (with one set, one chunk ahead, every chunk waited for its weights to
-    // arrive from L2: the kernel ran at the pace of that latency).
-    struct Piece {
-        v4 b, a;
-        u2v p[kParts];
-    };
-    Piece R[2];
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-        R[s].b = v4{0.f, 0.f, 0.f, 0.f};
-        R[s].a = v4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int q = 0; q < kParts; ++q) R[s].p[q] = u2v{0u, 0u};
-    }
-    auto fetch = [&](int c, Piece& x) {
-        if (b_mine) {
-            if constexpr (kPacked) {
-                const unsigned short* w = static_cast<const unsigned short*>(wt) + (c * kParts * kCols + r) * kKC + k4;
-#pragma unroll
-                for (int q = 0; q < kParts; ++q) x.p[q] = *reinterpret_cast<const u2v*>(w + q * kCols * kKC);
-            } else {
-                x.b = *reinterpret_cast<const v4*>(static_cast<const float*>(wt) + static_cast<size_t>(r) * kK + c * kKC + k4);
-            }
-        }
-        if constexpr (kAGlobal) x.a = *reinterpret_cast<const v4*>(arows + static_cast<size_t>(arow) * kK + c * kKC + k4);
-    };
-    auto stage = [&](int buf, const Piece& x) {
-        if (b_mine) {
-            if constexpr (kPacked) {
-#pragma unroll
-                for (int q = 0; q < kParts; ++q) *reinterpret_cast<u2v*>(&S.bstage[buf][q][r][k4]) = x.p[q];
-            } else {
-                stage_piece(S.bstage[buf], r, k4, x.b);
-            }
-        }
-        if constexpr (kAGlobal) stage_piece(S.astage[buf], r, k4, x.a);
-    };
+    v4 A[kAGlobal ? kDepth : 1];
+    auto afetch = [&](int c, v4& x) { x = *reinterpret_cast<const v4*>(arows + static_cast<size_t>(arow) * kK + c * kKC + k4); };
+
     v16 lo[2];                   // the mixed partial products, 2^11 times their size
 #pragma unroll
     for (int j = 0; j < 2; ++j)
@@ -208,17 +235,20 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
             acc[j][e] = 0.f;
             lo[j][e] = 0.f;
         }
-    static_assert(chunks % 2 == 0 && chunks >= 4, "the chunk loop is unrolled by two");
-    fetch(0, R[0]);
-    fetch(1, R[1]);
-    stage(0, R[0]);
-    fetch(2, R[0]);
-    __syncthreads();             // chunk 0 is staged; the activation planes written before this call are complete
-    const int col0 = kNB == 2 ? P.wc * 64 : P.wc * 32;
-    // chunk c: stage chunk c + 1 (its piece is in `x`) into the other buffer, ask for chunk c + 3, multiply chunk c
-    auto step = [&](int c, Piece& x) {
-        // this chunk's operands are asked for first: they arrive from LDS while the next chunk's piece is split
-        h8v av[kParts], bv[2][kParts];
+#pragma unroll
+    for (int s = 0; s < kDepth; ++s) {
+        bfetch(s, B[s]);
+        if constexpr (kAGlobal) afetch(s, A[s]);
+    }
+    if constexpr (kAGlobal) {
+        stage_piece(S.astage[0], r, k4, A[0]);
+        if (kDepth < chunks) afetch(kDepth, A[0]);
+    }
+    __syncthreads();             // chunk 0 of the rows is staged; the activation planes written before this call are complete
+    // chunk c: (layer 1: stage the rows' chunk c + 1 into the other buffer, ask for their chunk c + 1 + kDepth,) multiply
+    // chunk c, ask for the weights of chunk c + kDepth
+    auto step = [&](int c, BSet& b, v4& a_next) {
+        h8v av[kParts];
 #pragma unroll
         for (int m = 0; m < kParts; ++m) {
             if constexpr (kAGlobal)
@@ -226,16 +256,16 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
             else
                 av[m] = __builtin_bit_cast(h8v, *reinterpret_cast<const u4v*>(&S.act[m][P.wr * 32 + P.l32][c * kKC + P.half * 8]));
         }
-#pragma unroll
-        for (int j = 0; j < kNB; ++j)
-#pragma unroll
-            for (int m = 0; m < kParts; ++m)
-                bv[j][m] = __builtin_bit_cast(h8v, *reinterpret_cast<const u4v*>(&S.bstage[c & 1][m][col0 + j * 32 + P.l32][P.half * 8]));
-        asm volatile("" ::: "memory");                   // the reads above stay ahead of the stage's writes
-        if (c + 1 < chunks) {
-            stage((c + 1) & 1, x);                       // the other buffer: last read before the previous barrier
-            if (c + 3 < chunks) fetch(c + 3, x);
+        if constexpr (kAGlobal) {
+            asm volatile("" ::: "memory");               // the reads above stay ahead of the stage's writes
+            if (c + 1 < chunks) {
+                stage_piece(S.astage[(c + 1) & 1], r, k4, a_next);     // the other buffer: last read before the previous barrier
+                if (c + 1 + kDepth < chunks) afetch(c + 1 + kDepth, a_next);
+            }
         }
+        h8v bv[2][kParts];
+#pragma unroll
+        for (int j = 0; j < kNB; ++j) boperand(b, j, bv[j]);
         // independent accumulators alternate, so that no matrix instruction waits for the one before it
 #pragma unroll
         for (int j = 0; j < kNB; ++j) lo[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[1], bv[j][0], lo[j], 0, 0, 0);
@@ -243,12 +273,14 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
         for (int j = 0; j < kNB; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[0], bv[j][0], acc[j], 0, 0, 0);
 #pragma unroll
         for (int j = 0; j < kNB; ++j) lo[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[0], bv[j][1], lo[j], 0, 0, 0);
-        __syncthreads();
+        if (c + kDepth < chunks) bfetch(c + kDepth, b);
+        if constexpr (kAGlobal) __syncthreads();
     };
-    for (int c = 0; c < chunks; c += 2) {
-        step(c, R[1]);
-        step(c + 1, R[0]);
+    for (int c = 0; c < chunks; c += kDepth) {
+#pragma unroll
+        for (int u = 0; u < kDepth; ++u) step(c + u, B[u], A[kAGlobal ? (u + 1) % kDepth : 0]);
     }
+    if constexpr (!kAGlobal) __syncthreads();
 #pragma unroll
     for (int j = 0; j < kNB; ++j)
 #pragma unroll
@@ -304,7 +336,7 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
 
     v16 acc[2], a1[2], a2[2], a3[2];
     // ------------------------------------------------------------ layer 1: 384 -> 128
-    layer_product<kK1, 2, true, kPacked>(S, P, acc, weights(args.w1t[t], kPackF1), args.rows[t], row0, n);
+    layer_product<kK1, 2, true, kPacked, kDepthRows>(S, P, acc, weights(args.w1t[t], kPackF1), args.rows[t], row0, n);
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const float b = args.b1[t][P.wc * 64 + j * 32 + P.l32];
@@ -313,7 +345,7 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
     }
     to_planes<2>(S, P, a1);
     // ------------------------------------------------------------ layer 2: 128 -> 128
-    layer_product<kN1, 2, false, kPacked>(S, P, acc, weights(args.w2t[t], kPackF2), nullptr, row0, n);
+    layer_product<kN1, 2, false, kPacked, kDepthWeights>(S, P, acc, weights(args.w2t[t], kPackF2), nullptr, row0, n);
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const float b = args.b2[t][P.wc * 64 + j * 32 + P.l32];
@@ -322,7 +354,7 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
     }
     to_planes<2>(S, P, a2);
     // ------------------------------------------------------------ layer 3: 128 -> 64, and the output layer 64 -> 1
-    layer_product<kN2, 1, false, kPacked>(S, P, acc, weights(args.w3t[t], kPackF3), nullptr, row0, n);
+    layer_product<kN2, 1, false, kPacked, kDepthWeights>(S, P, acc, weights(args.w3t[t], kPackF3), nullptr, row0, n);
     const int c3 = P.wc * 32 + P.l32;                    // this lane's column of the 64
     const float w4 = args.w4[t][c3];
     {
@@ -352,14 +384,14 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
         to_planes<1>(S, P, g3);
     }
     // g2 = (g3 W3^T) .* celu'(a2): 64 -> 128
-    layer_product<kN3, 2, false, kPacked>(S, P, acc, weights(args.w3[t], kPackB3), nullptr, row0, n);
+    layer_product<kN3, 2, false, kPacked, kDepthWeights>(S, P, acc, weights(args.w3[t], kPackB3), nullptr, row0, n);
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[j][e] *= celu_slope(a2[j][e], inv_alpha);
     to_planes<2>(S, P, acc);
     // g1 = (g2 W2^T) .* celu'(a1): 128 -> 128
-    layer_product<kN2, 2, false, kPacked>(S, P, acc, weights(args.w2[t], kPackB2), nullptr, row0, n);
+    layer_product<kN2, 2, false, kPacked, kDepthWeights>(S, P, acc, weights(args.w2[t], kPackB2), nullptr, row0, n);
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -374,7 +406,7 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
         const void* w;
         if constexpr (kPacked) w = pk + kPackB1 + static_cast<size_t>(ct) * kParts * 128 * kN1;
         else w = args.w1[t] + static_cast<size_t>(ct) * 128 * kN1;
-        layer_product<kN1, 2, false, kPacked>(S, P, acc, w, nullptr, row0, n);
+        layer_product<kN1, 2, false, kPacked, kDepthWeights>(S, P, acc, w, nullptr, row0, n);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int col = ct * 128 + P.wc * 64 + j * 32 + P.l32;
