@@ -338,10 +338,10 @@ int khan_dense_head_grad_f32(const float *const *scale_host4, const float *const
  *   weights_host12[4l+t]   the same layers as stored: [384, 128], [128, 128], [128, 64] (read for the gradient only;
  *                          NULL when grad_host4 is NULL)
  *   packed                 DEVICE buffer written by khan_atomic_networks_pack_f32 from the same 24 matrices, or NULL.
- *                          With it neither weights array is read (both may be NULL) and the kernel copies the weights'
- *                          two half-precision parts instead of splitting them again for every 128 rows: the same bits out,
- *                          a tenth less time.  Pack once per set of weights (khan_atomic_networks_packed_bytes() bytes,
- *                          16-byte aligned); pack again after the weights change.
+ *                          With it neither weights array is read (both may be NULL) and the kernel loads the weights'
+ *                          two half-precision parts as they are instead of splitting the float32 weights again in every
+ *                          wavefront: the same bits out, less time.  Pack once per set of weights
+ *                          (khan_atomic_networks_packed_bytes() bytes, 16-byte aligned); pack again after the weights change.
  *   biases_host12[4l+t]    [128], [128], [64]
  *   head_w_host4[t] [64], head_b_host4[t] one float (head_b_host4 or an entry may be NULL: no bias)
  *   scale_host4[t]         [n_t] gradient with respect to each row's value, or NULL (the array or an entry): ones

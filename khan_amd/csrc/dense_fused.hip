@@ -5,11 +5,12 @@
 //     g3 = s w4^T .* celu'(a3), g2 = (g3 W3^T) .* celu'(a2), g1 = (g2 W2^T) .* celu'(a1), dx = g1 W1^T
 // with s the gradient with respect to each row's value e (1 when none is given: the gradient of the sum of the values,
 // which is what forces need).  A feature row is read once and its gradient written once: the activations of a tile of
-// 128 rows never leave the compute unit.  Layer by layer the same pass moves 2.9 GB forward and 3.7 GB back per 767,292
+// rows never leave the compute unit.  Layer by layer the same pass moves 2.9 GB forward and 3.7 GB back per 767,292
 // rows (every activation written, read again by the next layer and once more on the way back); this one moves the rows
 // and their gradients, 2.4 GB, and the values.
 //
-// One workgroup of eight wavefronts owns 128 rows.  The products run on the 16-bit matrix instructions
+// One workgroup of four wavefronts owns 64 rows; two workgroups share a compute unit and, having no barriers in common,
+// fill each other's waits.  The products run on the 16-bit matrix instructions
 // (v_mfma_f32_32x32x16_f16, sixteen times the rate of the float32 ones) with every float32 operand split into two
 // half-precision parts:
 //     x = h + 2^-11 l,   h = half(x),   l = half(2^11 (x - h))
@@ -29,11 +30,11 @@
 // (32 x 32 of the 128 x 64 one) in accumulator registers, and keeps its part of a1, a2 and a3 in registers for the way
 // back, where the gradients arrive in the same places.  Between layers the activations (gradients) go to LDS already
 // split, as two planes [row][k] of half precision: the next product's row operand, read straight from there.  The weights
-// stream from L2 in chunks of 16 k into a double-buffered LDS stage, one barrier per chunk -- split on the way, or, when
-// the caller has had them split once beforehand (launch_networks_pack: a quarter of the kernel's vector instructions
-// were the same weights being split again for every tile of rows), copied as they are; layer 1
-// stages its feature rows the same way in the space the activation planes take later.  LDS: 93 KB, one workgroup per CU
-// (the accumulators and the saved activations of eight more wavefronts would not fit the registers).
+// do not pass through LDS: every wavefront loads its operands of a chunk of 16 k straight into registers (layer_product)
+// -- from the chunks the caller has had split once beforehand (launch_networks_pack), or from the float32 weights, which
+// a lane then splits itself.  Layer 1's feature rows, float32 in memory, go through a double-buffered LDS stage in the
+// space the activation planes take later.  LDS: 35 KB per workgroup; 2 wavefronts per SIMD (the accumulators and the
+// saved activations take 200 registers).
 #include "khan_internal.h"
 #include "khan_params.h"
 
