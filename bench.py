@@ -236,6 +236,8 @@ def grad_inverse_bench(args, batch, w, kind):
     launch_ms = e0.elapsed_time(e1) / args.steps
     nbytes = N * (384 * w + 6 * w + 8) + 8 * n_mols
     kernel = "aev_fwd_%s_kernel<%s, true>" % ("small" if kind == "organic" else "medium", tname)
+    import bench_profiling as profiling
+    traffic, stale, _ = profiling.measured_traffic(args.workload.replace("grad_inverse", "organic") if kind == "organic" and w == 4 else args.workload, "jvp")
     return ({
         "metric": "AEV grad-inverse (Jacobian-vector product) atoms/sec, fp%d, 1 MI355X" % (8 * w),
         "value": N / (ms_per_step * 1e-3), "unit": "atoms/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -244,7 +246,7 @@ def grad_inverse_bench(args, batch, w, kind):
         "config": {"workload": "%s: featurize_grad_inverse, %d molecules, %d atoms" % (args.workload, n_mols, N)},
         "roofline": {"kernel": kernel, "bound": "hbm", "achieved": nbytes / (launch_ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (launch_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": None, "launch_ms": launch_ms, "algorithmic_bytes": nbytes},
+                     "traffic": traffic, "traffic_stale": stale, "launch_ms": launch_ms, "algorithmic_bytes": nbytes},
     })
 
 
@@ -319,8 +321,8 @@ def main():
     ap.add_argument("--headline-only", action="store_true",
                     help="with the default workload: leave out the shorter runs of the other configurations "
                          "(`configs` in the printed line)")
-    ap.add_argument("--traffic-probe", choices=("fwd", "bwd", "networks", "charges"), default=None,
-                    help="counter-collection mode: launch that pass twice (fwd, bwd: the AEV passes; networks: "
+    ap.add_argument("--traffic-probe", choices=("fwd", "bwd", "jvp", "networks", "charges"), default=None,
+                    help="counter-collection mode: launch that pass twice (fwd, bwd: the AEV passes; jvp: featurize_grad_inverse; networks: "
                          "khan_atomic_networks_f32 with its gradient on the workload's feature rows; charges: "
                          "khan_ani_charge_all), then a plain 64 MiB device copy of known traffic (scales FETCH_SIZE / "
                          "WRITE_SIZE), print nothing else and exit")
@@ -439,6 +441,8 @@ def run_workload(args, workload, steps, warmup, cpu):
                 ops.featurize(X, Y, Z, A, mos, macs, sc, acs)
             elif args.traffic_probe == "bwd":
                 ops.featurize_grad(X, Y, Z, A, mos, macs, sc, acs, *grads)
+            elif args.traffic_probe == "jvp":
+                ops.featurize_grad_inverse(X, Y, Z, A, mos, macs, sc, acs, *(upstream[k * N:(k + 1) * N] for k in range(3)))
             elif args.traffic_probe == "networks":
                 ops.atomic_networks(feats, None, biases, head_w, head_b, want_grad=True, packed=packed)
             else:

@@ -50,6 +50,7 @@ DOMINANT = {
     ("boxes4096", "fwd"): "aev_fwd_medium_kernel<float, false, false>",
     ("boxes4096", "bwd"): "aev_bwd_medium_kernel<float, false, false>",
     ("organic65536", "networks"): "networks_fused_kernel<true, true>",
+    ("organic65536", "jvp"): "aev_fwd_small_kernel<float, true, false>",
     ("charges_boxes4096_f64", "charges"): "charge_tile_kernel<double",
 }
 # the sources an entry's digest covers, by pass
@@ -239,7 +240,7 @@ def main(argv=None):
     t = sub.add_parser("traffic", help="rewrite a workload's entries of profiles/hbm_traffic.json from counter runs")
     t.add_argument("--workload", required=True)
     t.add_argument("--dir", required=True, help="directory holding fwd_fetch/ fwd_write/ bwd_fetch/ bwd_write/")
-    t.add_argument("--passes", nargs="+", default=["fwd", "bwd"], choices=("fwd", "bwd", "networks", "charges"))
+    t.add_argument("--passes", nargs="+", default=["fwd", "bwd"], choices=("fwd", "bwd", "jvp", "networks", "charges"))
     sub.add_parser("digest", help="print the digest of the kernel sources in the tree")
     st = sub.add_parser("stages", help="time by stage of the AEV passes, from the measurement builds "
                                        "(python -m khan_amd.build --stage-variants)")
