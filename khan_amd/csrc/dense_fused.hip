@@ -61,7 +61,7 @@ constexpr int kDepthWeights = KHAN_FUSED_DEPTH;   // and of the other products (
 #ifndef KHAN_FUSED_ROWS
 #define KHAN_FUSED_ROWS 64
 #endif
-constexpr int kRows = KHAN_FUSED_ROWS;      // rows per workgroup: 64 (four wavefronts, two workgroups per CU) or 128 (eight, one)
+constexpr int kRows = KHAN_FUSED_ROWS;      // rows per workgroup
 constexpr int kThreads = kRows * 4;         // a wavefront per 32 rows x 64 columns of a 128-wide output
 constexpr int kK1 = 384, kN1 = 128, kN2 = 128, kN3 = 64;
 constexpr int kActStride = 136;     // 16-bit elements between rows of the activation planes: 128 + 8 (16-byte reads without bank conflicts)
@@ -152,63 +152,66 @@ __device__ __forceinline__ float half_sum_to_upper_row(float v)
     return v;
 }
 
-// Positions: accumulator e of a wavefront's block j is row wr*32 + 8 (e / 4) + 4 half + e % 4 of the tile and column
-// col0 + j*32 + l32, col0 = wc*64 for a 128-wide output (two blocks per wavefront), wc*32 for the 64-wide one (one).
+// Positions.  A 128-wide output (kWide): the wavefront owns the tile's 64 rows x 32 columns, columns wave*32 + l32, as
+// two 32 x 32 blocks one above the other -- block j, accumulator e is row j*32 + 8 (e / 4) + 4 half + e % 4.  The
+// 64-wide output of layer 3: one block per wavefront, rows wr*32 + ..., columns wc*32 + l32.
 struct Place {
-    int tid, lane, wr, wc, l32, half;
-    __device__ __forceinline__ int row(int e) const { return wr * 32 + 8 * (e >> 2) + 4 * half + (e & 3); }
+    int tid, lane, wave, wr, wc, l32, half;
+    __device__ __forceinline__ int rib(int e) const { return 8 * (e >> 2) + 4 * half + (e & 3); }      // row in the block
+    template <bool kWide> __device__ __forceinline__ int row(int j, int e) const { return (kWide ? j * 32 : wr * 32) + rib(e); }
+    template <bool kWide> __device__ __forceinline__ int col() const { return (kWide ? wave * 32 : wc * 32) + l32; }
 };
 
-// One layer's product for this workgroup's rows: acc = A . B^T, A = kRows x kK (rows), B = (kNB * 64) x kK (`wt`: one
-// row per output column), chunk by chunk of 16 k.
+// One layer's product for this workgroup's 64 rows: acc = A . B^T, A = 64 x kK (rows), B = (kWide ? 128 : 64) x kK
+// (`wt`: one row per output column), chunk by chunk of 16 k.
 // B never passes through LDS: a matrix instruction's operand is, per lane, eight consecutive k of one column -- 16
 // bytes of a packed chunk, and the 64 lanes' pieces are one contiguous kilobyte -- so every wavefront loads its own
-// operands straight into registers, kDepth chunks ahead (they come from L2, or from the compute unit's L1 when the
-// wavefront beside it has just asked for the same columns).  With the weights staged in LDS the kernel was bound by
-// LDS traffic: nine kilobytes read and written per wavefront and chunk for six matrix instructions, and a barrier
-// per chunk.  A comes from the activation planes, with no barrier inside the product; or (kAGlobal: layer 1) from
-// `arows` in memory through a double-buffered LDS stage (the rows are float32 and have to be split and regrouped), one
-// barrier per chunk.  Begins and ends with a barrier: the planes written before the call are complete, and afterwards
-// nobody reads the planes or the stage any more.
+// operands straight into registers, kDepth chunks ahead.  In a 128-wide product a wavefront takes ALL 64 rows of 32
+// columns: its weight operand serves two matrix instructions' worth of rows, no other wavefront loads the same
+// columns, and the row operand -- from LDS, which has the bandwidth to spare -- is read twice as often instead.  (With
+// 32 rows x 64 columns per wavefront the two wavefronts of a column half loaded the same weights: the weights' loads,
+// 1.2 MB per tile through the compute unit's 64-byte-per-cycle load path, were the largest single part of the kernel.)
+// With the weights staged in LDS (the first version) the kernel was bound by LDS traffic: nine kilobytes read and
+// written per wavefront and chunk for six matrix instructions, and a barrier per chunk.  A comes from the activation
+// planes, with no barrier inside the product; or (kAGlobal: layer 1) from `arows` in memory through a double-buffered
+// LDS stage (the rows are float32 and have to be split and regrouped), one barrier per chunk.  Begins and ends with a
+// barrier: the planes written before the call are complete, and afterwards nobody reads the planes or the stage any more.
 // kPacked: `wt` points at the matrix's packed chunks (half precision); otherwise at float32 weights, of which a lane
 // loads its eight values and splits them itself.
-template <int kK, int kNB, bool kAGlobal, bool kPacked, int kDepth>
+template <int kK, bool kWide, bool kAGlobal, bool kPacked, int kDepth>
 __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (&acc)[2], const void* __restrict__ wt,
                                               const float* __restrict__ arows, int row0, int n)
 {
     constexpr int chunks = kK / kKC;
-    constexpr int kCols = kNB * 64;                      // 128 or 64 output columns
+    constexpr int kCols = kWide ? 128 : 64;              // output columns
+    constexpr int kNB = kWide ? 2 : 1;                   // blocks (accumulators) of this wavefront
     static_assert(chunks % kDepth == 0 && kDepth >= 2, "the chunk loop is unrolled by the number of register sets");
-    const int col0 = kNB == 2 ? P.wc * 64 : P.wc * 32;
-    // a chunk's operands for this wavefront's blocks, as loaded: the two parts (packed), or eight float32 weights
+    const int col = P.col<kWide>();
+    // a chunk's weight operand for this wavefront's columns, as loaded: the two parts (packed), or eight float32 weights
     struct BSet {
-        u4v raw[kNB][2];
+        u4v raw[2];
     };
     BSet B[kDepth];
     auto bfetch = [&](int c, BSet& x) {
+        if constexpr (kPacked) {
+            const unsigned short* w = static_cast<const unsigned short*>(wt) + (c * kParts * kCols + col) * kKC + P.half * 8;
 #pragma unroll
-        for (int j = 0; j < kNB; ++j) {
-            const int col = col0 + j * 32 + P.l32;
-            if constexpr (kPacked) {
-                const unsigned short* w = static_cast<const unsigned short*>(wt) + (c * kParts * kCols + col) * kKC + P.half * 8;
-#pragma unroll
-                for (int m = 0; m < kParts; ++m) x.raw[j][m] = *reinterpret_cast<const u4v*>(w + m * kCols * kKC);
-            } else {
-                const float* w = static_cast<const float*>(wt) + static_cast<size_t>(col) * kK + c * kKC + P.half * 8;
-                x.raw[j][0] = *reinterpret_cast<const u4v*>(w);
-                x.raw[j][1] = *reinterpret_cast<const u4v*>(w + 4);
-            }
+            for (int m = 0; m < kParts; ++m) x.raw[m] = *reinterpret_cast<const u4v*>(w + m * kCols * kKC);
+        } else {
+            const float* w = static_cast<const float*>(wt) + static_cast<size_t>(col) * kK + c * kKC + P.half * 8;
+            x.raw[0] = *reinterpret_cast<const u4v*>(w);
+            x.raw[1] = *reinterpret_cast<const u4v*>(w + 4);
         }
     };
-    auto boperand = [&](const BSet& x, int j, h8v (&bv)[kParts]) {
+    auto boperand = [&](const BSet& x, h8v (&bv)[kParts]) {
         if constexpr (kPacked) {
 #pragma unroll
-            for (int m = 0; m < kParts; ++m) bv[m] = __builtin_bit_cast(h8v, x.raw[j][m]);
+            for (int m = 0; m < kParts; ++m) bv[m] = __builtin_bit_cast(h8v, x.raw[m]);
         } else {
             u4v part[kParts];
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const v4 f = __builtin_bit_cast(v4, x.raw[j][h]);
+                const v4 f = __builtin_bit_cast(v4, x.raw[h]);
                 unsigned a[kParts], b[kParts];
                 split_pair(f[0], f[1], a[0], a[1]);
                 split_pair(f[2], f[3], b[0], b[1]);
@@ -249,13 +252,17 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
     // chunk c: (layer 1: stage the rows' chunk c + 1 into the other buffer, ask for their chunk c + 1 + kDepth,) multiply
     // chunk c, ask for the weights of chunk c + kDepth
     auto step = [&](int c, BSet& b, v4& a_next) {
-        h8v av[kParts];
+        h8v av[2][kParts];
 #pragma unroll
-        for (int m = 0; m < kParts; ++m) {
-            if constexpr (kAGlobal)
-                av[m] = __builtin_bit_cast(h8v, *reinterpret_cast<const u4v*>(&S.astage[c & 1][m][P.wr * 32 + P.l32][P.half * 8]));
-            else
-                av[m] = __builtin_bit_cast(h8v, *reinterpret_cast<const u4v*>(&S.act[m][P.wr * 32 + P.l32][c * kKC + P.half * 8]));
+        for (int j = 0; j < kNB; ++j) {
+            const int arow_l = (kWide ? j * 32 : P.wr * 32) + P.l32;
+#pragma unroll
+            for (int m = 0; m < kParts; ++m) {
+                if constexpr (kAGlobal)
+                    av[j][m] = __builtin_bit_cast(h8v, *reinterpret_cast<const u4v*>(&S.astage[c & 1][m][arow_l][P.half * 8]));
+                else
+                    av[j][m] = __builtin_bit_cast(h8v, *reinterpret_cast<const u4v*>(&S.act[m][arow_l][c * kKC + P.half * 8]));
+            }
         }
         if constexpr (kAGlobal) {
             asm volatile("" ::: "memory");               // the reads above stay ahead of the stage's writes
@@ -264,16 +271,15 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
                 if (c + 1 + kDepth < chunks) afetch(c + 1 + kDepth, a_next);
             }
         }
-        h8v bv[2][kParts];
-#pragma unroll
-        for (int j = 0; j < kNB; ++j) boperand(b, j, bv[j]);
+        h8v bv[kParts];
+        boperand(b, bv);
         // independent accumulators alternate, so that no matrix instruction waits for the one before it
 #pragma unroll
-        for (int j = 0; j < kNB; ++j) lo[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[1], bv[j][0], lo[j], 0, 0, 0);
+        for (int j = 0; j < kNB; ++j) lo[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[j][1], bv[0], lo[j], 0, 0, 0);
 #pragma unroll
-        for (int j = 0; j < kNB; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[0], bv[j][0], acc[j], 0, 0, 0);
+        for (int j = 0; j < kNB; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[j][0], bv[0], acc[j], 0, 0, 0);
 #pragma unroll
-        for (int j = 0; j < kNB; ++j) lo[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[0], bv[j][1], lo[j], 0, 0, 0);
+        for (int j = 0; j < kNB; ++j) lo[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[j][0], bv[1], lo[j], 0, 0, 0);
         if (c + kDepth < chunks) bfetch(c + kDepth, b);
         if constexpr (kAGlobal) __syncthreads();
     };
@@ -288,19 +294,18 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
         for (int e = 0; e < 16; ++e) acc[j][e] = fmaf(lo[j][e], kResidualBack, acc[j][e]);
 }
 
-// a wavefront's values of a layer (kNB blocks) -> the activation planes, split; column = k of the next product
-template <int kNB>
+// a wavefront's values of a layer -> the activation planes, split; column = k of the next product
+template <bool kWide>
 __device__ __forceinline__ void to_planes(FusedLds& S, const Place& P, const v16 (&v)[2])
 {
-    const int col0 = kNB == 2 ? P.wc * 64 : P.wc * 32;
+    const int col = P.col<kWide>();
 #pragma unroll
-    for (int j = 0; j < kNB; ++j) {
-        const int col = col0 + j * 32 + P.l32;
+    for (int j = 0; j < (kWide ? 2 : 1); ++j) {
 #pragma unroll
         for (int e = 0; e < 16; e += 2) {
             unsigned p[kParts];
             split_pair(v[j][e], v[j][e + 1], p[0], p[1]);
-            const int r0 = P.row(e), r1 = P.row(e + 1);
+            const int r0 = P.row<kWide>(j, e), r1 = P.row<kWide>(j, e + 1);
 #pragma unroll
             for (int q = 0; q < kParts; ++q) {
                 S.act[q][r0][col] = static_cast<unsigned short>(p[q] & 0xffffu);
@@ -314,13 +319,14 @@ template <bool kGrad, bool kPacked>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
 {
+    static_assert(kRows == 64 && kThreads == 256, "four wavefronts: 64 rows x 32 columns each of a 128-wide output");
     __shared__ FusedLds S;
     Place P;
     P.tid = threadIdx.x;
     P.lane = P.tid & 63;
-    const int wave = P.tid >> 6;
-    P.wr = wave >> 1;
-    P.wc = wave & 1;
+    P.wave = P.tid >> 6;
+    P.wr = P.wave >> 1;
+    P.wc = P.wave & 1;
     P.l32 = P.lane & 31;
     P.half = P.lane >> 5;
     const int tile = blockIdx.x;
@@ -334,29 +340,32 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
         if constexpr (kPacked) return pk + packed_at;
         else return plain;
     };
+    const int cw = P.col<true>();                        // this lane's column of a 128-wide layer
 
     v16 acc[2], a1[2], a2[2], a3[2];
     // ------------------------------------------------------------ layer 1: 384 -> 128
-    layer_product<kK1, 2, true, kPacked, kDepthRows>(S, P, acc, weights(args.w1t[t], kPackF1), args.rows[t], row0, n);
+    layer_product<kK1, true, true, kPacked, kDepthRows>(S, P, acc, weights(args.w1t[t], kPackF1), args.rows[t], row0, n);
+    {
+        const float b = args.b1[t][cw];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const float b = args.b1[t][P.wc * 64 + j * 32 + P.l32];
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) a1[j][e] = celu_of(acc[j][e] + b, alpha, inv_alpha);
+            for (int e = 0; e < 16; ++e) a1[j][e] = celu_of(acc[j][e] + b, alpha, inv_alpha);
     }
-    to_planes<2>(S, P, a1);
+    to_planes<true>(S, P, a1);
     // ------------------------------------------------------------ layer 2: 128 -> 128
-    layer_product<kN1, 2, false, kPacked, kDepthWeights>(S, P, acc, weights(args.w2t[t], kPackF2), nullptr, row0, n);
+    layer_product<kN1, true, false, kPacked, kDepthWeights>(S, P, acc, weights(args.w2t[t], kPackF2), nullptr, row0, n);
+    {
+        const float b = args.b2[t][cw];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const float b = args.b2[t][P.wc * 64 + j * 32 + P.l32];
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) a2[j][e] = celu_of(acc[j][e] + b, alpha, inv_alpha);
+            for (int e = 0; e < 16; ++e) a2[j][e] = celu_of(acc[j][e] + b, alpha, inv_alpha);
     }
-    to_planes<2>(S, P, a2);
+    to_planes<true>(S, P, a2);
     // ------------------------------------------------------------ layer 3: 128 -> 64, and the output layer 64 -> 1
-    layer_product<kN2, 1, false, kPacked, kDepthWeights>(S, P, acc, weights(args.w3t[t], kPackF3), nullptr, row0, n);
-    const int c3 = P.wc * 32 + P.l32;                    // this lane's column of the 64
+    layer_product<kN2, false, false, kPacked, kDepthWeights>(S, P, acc, weights(args.w3t[t], kPackF3), nullptr, row0, n);
+    const int c3 = P.col<false>();                       // this lane's column of the 64
     const float w4 = args.w4[t][c3];
     {
         const float b = args.b3[t][c3];
@@ -364,7 +373,7 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
         for (int e = 0; e < 16; ++e) {
             a3[0][e] = celu_of(acc[0][e] + b, alpha, inv_alpha);
             const float tot = half_sum_to_upper_row(a3[0][e] * w4);      // over this wavefront's 32 of the 64 columns
-            if (P.l32 == 16 + e) S.rowval[P.wc][P.row(e)] = tot;
+            if (P.l32 == 16 + e) S.rowval[P.wc][P.row<false>(0, e)] = tot;
         }
     }
     __syncthreads();
@@ -382,39 +391,40 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
         v16 g3[2];
 #pragma unroll
         for (int e = 0; e < 16; ++e) g3[0][e] = w4 * celu_slope(a3[0][e], inv_alpha);     // for a unit upstream factor
-        to_planes<1>(S, P, g3);
+        to_planes<false>(S, P, g3);
     }
     // g2 = (g3 W3^T) .* celu'(a2): 64 -> 128
-    layer_product<kN3, 2, false, kPacked, kDepthWeights>(S, P, acc, weights(args.w3[t], kPackB3), nullptr, row0, n);
+    layer_product<kN3, true, false, kPacked, (kDepthWeights > 4 ? 4 : kDepthWeights)>(S, P, acc, weights(args.w3[t], kPackB3), nullptr, row0, n);
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[j][e] *= celu_slope(a2[j][e], inv_alpha);
-    to_planes<2>(S, P, acc);
+    to_planes<true>(S, P, acc);
     // g1 = (g2 W2^T) .* celu'(a1): 128 -> 128
-    layer_product<kN2, 2, false, kPacked, kDepthWeights>(S, P, acc, weights(args.w2[t], kPackB2), nullptr, row0, n);
+    layer_product<kN2, true, false, kPacked, kDepthWeights>(S, P, acc, weights(args.w2[t], kPackB2), nullptr, row0, n);
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[j][e] *= celu_slope(a1[j][e], inv_alpha);
-    to_planes<2>(S, P, acc);
+    to_planes<true>(S, P, acc);
     // dx = g1 W1^T: 128 -> 384, three column tiles of 128
     float* __restrict__ out = args.grad[t];
-    float upstream[16];          // the upstream factors of this lane's sixteen rows
+    float upstream[2][16];       // the upstream factors of this lane's rows
 #pragma unroll
-    for (int e = 0; e < 16; ++e) upstream[e] = S.rowval[0][P.row(e)];
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) upstream[j][e] = S.rowval[0][P.row<true>(j, e)];
     for (int ct = 0; ct < kK1 / 128; ++ct) {
         const void* w;
         if constexpr (kPacked) w = pk + kPackB1 + static_cast<size_t>(ct) * kParts * 128 * kN1;
         else w = args.w1[t] + static_cast<size_t>(ct) * 128 * kN1;
-        layer_product<kN1, 2, false, kPacked, kDepthWeights>(S, P, acc, w, nullptr, row0, n);
+        layer_product<kN1, true, false, kPacked, kDepthWeights>(S, P, acc, w, nullptr, row0, n);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            const int col = ct * 128 + P.wc * 64 + j * 32 + P.l32;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int gr = row0 + P.row(e);
-                if (gr < n) out[static_cast<size_t>(gr) * kK1 + col] = acc[j][e] * upstream[e];
+                const int gr = row0 + P.row<true>(j, e);
+                if (gr < n) out[static_cast<size_t>(gr) * kK1 + ct * 128 + cw] = acc[j][e] * upstream[j][e];
             }
         }
     }
