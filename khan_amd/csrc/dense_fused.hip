@@ -26,8 +26,8 @@
 // |x| below 6e-5 keeps an absolute accuracy of 2^-36 instead of a relative one.  On the way back the gradient is
 // carried for a unit upstream factor and multiplied by the row's factor only when it is stored (the pass is linear
 // in it), so that the gradients' size inside the kernel does not depend on the caller's loss scale.
-// A wavefront holds a 32 x 64 part of a layer's 128 x 128 output
-// (32 x 32 of the 128 x 64 one) in accumulator registers, and keeps its part of a1, a2 and a3 in registers for the way
+// A wavefront holds all 64 rows of 32 columns of a layer's 64 x 128 output
+// (32 x 32 of the 64 x 64 one) in accumulator registers, and keeps its part of a1, a2 and a3 in registers for the way
 // back, where the gradients arrive in the same places.  Between layers the activations (gradients) go to LDS already
 // split, as two planes [row][k] of half precision: the next product's row operand, read straight from there.  The weights
 // do not pass through LDS: every wavefront loads its operands of a chunk of 16 k straight into registers (layer_product)
