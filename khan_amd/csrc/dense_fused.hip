@@ -66,7 +66,7 @@ constexpr int kThreads = kRows * 4;         // a wavefront per 32 rows x 64 colu
 constexpr int kK1 = 384, kN1 = 128, kN2 = 128, kN3 = 64;
 constexpr int kActStride = 136;     // 16-bit elements between rows of the activation planes: 128 + 8 (16-byte reads without bank conflicts)
 constexpr int kKC = 16;             // k per staged chunk = one matrix instruction deep
-constexpr int kStStride = 24;       // 16-bit elements between staged rows: 16 + 8
+constexpr int kStStride = 40;       // 16-bit elements between staged rows: a pair of chunks (32 k) + 8
 constexpr int kParts = 2;           // half-precision parts per float32 operand
 constexpr float kResidualScale = 2048.0f, kResidualBack = 1.0f / 2048.0f;      // 2^11
 
@@ -106,7 +106,7 @@ constexpr int kPackPerType = kPackB3 + kParts * kN2 * kN3;   // 294,912 half-pre
 struct __align__(16) FusedLds {
     union {
         unsigned short act[kParts][kRows][kActStride];        // a layer's activations or gradients, split: [part][row][k]
-        unsigned short astage[2][kParts][kRows][kStStride];   // layer 1: chunks of the feature rows
+        unsigned short astage[2][kParts][kRows][kStStride];   // layer 1: pairs of chunks of the feature rows
     };
     float rowval[2][kRows];                              // the output layer's partial sums; then the rows' upstream factors
 };
@@ -225,11 +225,25 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
             for (int m = 0; m < kParts; ++m) bv[m] = __builtin_bit_cast(h8v, part[m]);
         }
     };
-    // layer 1: this thread's piece of a chunk of the feature rows: row r, k4..k4+3
-    const int r = P.tid >> 2, k4 = (P.tid & 3) << 2;
-    const int arow = min(row0 + r, n - 1);               // rows past the end: the last row again, never stored
-    v4 A[kAGlobal ? kDepth : 1];
-    auto afetch = [&](int c, v4& x) { x = *reinterpret_cast<const v4*>(arows + static_cast<size_t>(arow) * kK + c * kKC + k4); };
+    // Layer 1: the feature rows go through LDS a PAIR of chunks (32 k = one 128-byte line per row) at a time: eight lanes
+    // fetch a row's line together, a thread two rows' pieces (rows r8 and r8 + 32, k8..k8+3 of the pair), and a barrier
+    // closes a pair, not a chunk.  kPairsAhead pairs are in flight in registers.
+    constexpr int kPairsAhead = 2;
+    static_assert(!kAGlobal || (kDepth == 2 * kPairsAhead && kRows == 64 && kThreads == 256), "the unrolled loop body is two pairs long");
+    const int r8 = P.tid >> 3, k8 = (P.tid & 7) << 2;
+    const int arow0 = min(row0 + r8, n - 1), arow1 = min(row0 + r8 + 32, n - 1);      // rows past the end: the last row again, never stored
+    struct APair {
+        v4 x[2];
+    };
+    APair A[kAGlobal ? kPairsAhead : 1];
+    auto afetch = [&](int q, APair& a) {
+        a.x[0] = *reinterpret_cast<const v4*>(arows + static_cast<size_t>(arow0) * kK + q * 2 * kKC + k8);
+        a.x[1] = *reinterpret_cast<const v4*>(arows + static_cast<size_t>(arow1) * kK + q * 2 * kKC + k8);
+    };
+    auto astage_pair = [&](int q, const APair& a) {
+        stage_piece(S.astage[q & 1], r8, k8, a.x[0]);
+        stage_piece(S.astage[q & 1], r8 + 32, k8, a.x[1]);
+    };
 
     v16 lo[2];                   // the mixed partial products, 2^11 times their size
 #pragma unroll
@@ -240,18 +254,17 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
             lo[j][e] = 0.f;
         }
 #pragma unroll
-    for (int s = 0; s < kDepth; ++s) {
-        bfetch(s, B[s]);
-        if constexpr (kAGlobal) afetch(s, A[s]);
-    }
+    for (int s = 0; s < kDepth; ++s) bfetch(s, B[s]);
     if constexpr (kAGlobal) {
-        stage_piece(S.astage[0], r, k4, A[0]);
-        if (kDepth < chunks) afetch(kDepth, A[0]);
+#pragma unroll
+        for (int q = 0; q < kPairsAhead; ++q) afetch(q, A[q]);
+        astage_pair(0, A[0]);
+        if (2 * kPairsAhead < chunks) afetch(kPairsAhead, A[0]);
     }
-    __syncthreads();             // chunk 0 of the rows is staged; the activation planes written before this call are complete
-    // chunk c: (layer 1: stage the rows' chunk c + 1 into the other buffer, ask for their chunk c + 1 + kDepth,) multiply
-    // chunk c, ask for the weights of chunk c + kDepth
-    auto step = [&](int c, BSet& b, v4& a_next) {
+    __syncthreads();             // pair 0 of the rows is staged; the activation planes written before this call are complete
+    // chunk c: (layer 1, first chunk of a pair: stage the rows' next pair into the other buffer, ask for the pair
+    // kPairsAhead further on,) multiply chunk c, ask for the weights of chunk c + kDepth
+    auto step = [&](int c, BSet& b, APair& a_next) {
         h8v av[2][kParts];
 #pragma unroll
         for (int j = 0; j < kNB; ++j) {
@@ -259,16 +272,17 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
 #pragma unroll
             for (int m = 0; m < kParts; ++m) {
                 if constexpr (kAGlobal)
-                    av[j][m] = __builtin_bit_cast(h8v, *reinterpret_cast<const u4v*>(&S.astage[c & 1][m][arow_l][P.half * 8]));
+                    av[j][m] = __builtin_bit_cast(h8v, *reinterpret_cast<const u4v*>(&S.astage[(c >> 1) & 1][m][arow_l][(c & 1) * kKC + P.half * 8]));
                 else
                     av[j][m] = __builtin_bit_cast(h8v, *reinterpret_cast<const u4v*>(&S.act[m][arow_l][c * kKC + P.half * 8]));
             }
         }
         if constexpr (kAGlobal) {
             asm volatile("" ::: "memory");               // the reads above stay ahead of the stage's writes
-            if (c + 1 < chunks) {
-                stage_piece(S.astage[(c + 1) & 1], r, k4, a_next);     // the other buffer: last read before the previous barrier
-                if (c + 1 + kDepth < chunks) afetch(c + 1 + kDepth, a_next);
+            const int q = c >> 1;
+            if ((c & 1) == 0 && 2 * (q + 1) < chunks) {
+                astage_pair(q + 1, a_next);              // the other buffer: last read before the previous barrier
+                if (2 * (q + 1 + kPairsAhead) < chunks) afetch(q + 1 + kPairsAhead, a_next);
             }
         }
         h8v bv[kParts];
@@ -281,11 +295,15 @@ __device__ __forceinline__ void layer_product(FusedLds& S, const Place& P, v16 (
 #pragma unroll
         for (int j = 0; j < kNB; ++j) lo[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[j][0], bv[1], lo[j], 0, 0, 0);
         if (c + kDepth < chunks) bfetch(c + kDepth, b);
-        if constexpr (kAGlobal) __syncthreads();
+        if constexpr (kAGlobal) {
+            if (c & 1) __syncthreads();                  // the pair has been read, the next one is staged
+        }
     };
     for (int c = 0; c < chunks; c += kDepth) {
+        // (layer 1: kDepth = 2 kPairsAhead chunks; chunk c + u belongs to pair c / 2 + u / 2, and the pair staged during
+        // it, one further on, sits in register set (u / 2 + 1) % kPairsAhead)
 #pragma unroll
-        for (int u = 0; u < kDepth; ++u) step(c + u, B[u], A[kAGlobal ? (u + 1) % kDepth : 0]);
+        for (int u = 0; u < kDepth; ++u) step(c + u, B[u], A[kAGlobal ? ((u >> 1) + 1) % kPairsAhead : 0]);
     }
     if constexpr (!kAGlobal) __syncthreads();
 #pragma unroll
