@@ -50,19 +50,10 @@ typedef _Float16 h2v __attribute__((ext_vector_type(2)));
 typedef _Float16 h8v __attribute__((ext_vector_type(8)));
 typedef float f2v __attribute__((ext_vector_type(2)));
 
-#ifndef KHAN_FUSED_DEPTH1
-#define KHAN_FUSED_DEPTH1 4
-#endif
-#ifndef KHAN_FUSED_DEPTH
-#define KHAN_FUSED_DEPTH 4
-#endif
-constexpr int kDepthRows = KHAN_FUSED_DEPTH1;     // register sets of layer 1 (feature rows from HBM)
-constexpr int kDepthWeights = KHAN_FUSED_DEPTH;   // and of the other products (weights from L2)
-#ifndef KHAN_FUSED_ROWS
-#define KHAN_FUSED_ROWS 64
-#endif
-constexpr int kRows = KHAN_FUSED_ROWS;      // rows per workgroup
-constexpr int kThreads = kRows * 4;         // a wavefront per 32 rows x 64 columns of a 128-wide output
+constexpr int kDepthRows = 4;       // chunks of weights in flight in layer 1 (= two pairs of chunks of the feature rows)
+constexpr int kDepthWeights = 4;    // and in the other products (2 measured 6 % slower, 8 the same)
+constexpr int kRows = 64;           // rows per workgroup
+constexpr int kThreads = 256;       // four wavefronts: 64 rows x 32 columns each of a 128-wide output
 constexpr int kK1 = 384, kN1 = 128, kN2 = 128, kN3 = 64;
 constexpr int kActStride = 136;     // 16-bit elements between rows of the activation planes: 128 + 8 (16-byte reads without bank conflicts)
 constexpr int kKC = 16;             // k per staged chunk = one matrix instruction deep
@@ -412,7 +403,7 @@ void networks_fused_kernel(FusedArgs args, float alpha, float inv_alpha)
         to_planes<false>(S, P, g3);
     }
     // g2 = (g3 W3^T) .* celu'(a2): 64 -> 128
-    layer_product<kN3, true, false, kPacked, (kDepthWeights > 4 ? 4 : kDepthWeights)>(S, P, acc, weights(args.w3[t], kPackB3), nullptr, row0, n);
+    layer_product<kN3, true, false, kPacked, kDepthWeights>(S, P, acc, weights(args.w3[t], kPackB3), nullptr, row0, n);
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
