@@ -202,7 +202,8 @@ def inference_bench(args, batch):
                                "flops of the whole step against the float32 matrix peak",
                      "bound": "mfma", "achieved": gemm_flops / (ms_per_step * 1e-3) / 1e12,
                      "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": gemm_flops / (ms_per_step * 1e-3) / 1e12 / FP32_PEAK_TFLOPS, "traffic": None},
+                     "frac": gemm_flops / (ms_per_step * 1e-3) / 1e12 / FP32_PEAK_TFLOPS,
+                     "traffic": net_traffic, "traffic_stale": net_stale},      # of the networks' one launch
     })
 
 
@@ -294,6 +295,8 @@ def charges_bench(args, batch, w):
     nbytes = N * 8 * w + n_mols * (w + 8)
     peak = FP32_PEAK_TFLOPS if w == 4 else FP64_PEAK_TFLOPS
     tflops = 45.0 * C / (t_all * 1e-3) / 1e12
+    import bench_profiling as profiling
+    traffic, stale, _ = profiling.measured_traffic(args.workload, "charges")
     return ({
         "metric": "ani_charge energy + gradients atoms/sec, fp%d, 1 MI355X" % (8 * w),
         "value": N / (ms_per_step * 1e-3), "unit": "atoms/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -304,7 +307,7 @@ def charges_bench(args, batch, w):
         "molecules_per_s": n_mols / (ms_per_step * 1e-3),
         # all pairs of a molecule from a few bytes per atom: the vector ALUs bound these kernels, not HBM
         "roofline": {"kernel": "charge kernels", "bound": "valu", "achieved": tflops, "peak": peak, "unit": "TFLOP/s",
-                     "frac": tflops / peak, "traffic": None, "launch_ms": t_all,
+                     "frac": tflops / peak, "traffic": traffic, "traffic_stale": stale, "launch_ms": t_all,
                      "energy_ms": t_e, "gradients_ms": t_g,       # ani_charge and ani_charge_grad_xyz as separate calls
                      "algorithmic_flops": 45.0 * C, "algorithmic_bytes": nbytes,
                      "hbm_frac": nbytes / (t_all * 1e-3) / 1e9 / HBM_PEAK_GBS},
