@@ -8,42 +8,43 @@ namespace khan {
 
 // LDS working set of one wavefront
 // what the Jacobian-vector variant keeps on top of the forward working set
-template <typename T, bool kJvp, int kNB, int kRadN> struct FwdJvpLds {};
-template <typename T, int kNB, int kRadN> struct __align__(16) FwdJvpLds<T, true, kNB, kRadN> {
-    typename Fast<T>::vec4 vel[64];               // the incoming vector of every atom (sorted order)
-    typename Fast<T>::vec4 nbr_p[kNB][kCapA];      // (v_centre - v_partner)/r, and its component along the unit vector
-    typename Fast<T>::vec2 nbr_d[kNB][kCapA];      // f_C'(r) dr, and dr = change of the distance along the vectors
+template <typename T, bool kJvp, int kNB, int kRadN, int kCap> struct FwdJvpLds {};
+template <typename T, int kNB, int kRadN, int kCap> struct __align__(16) FwdJvpLds<T, true, kNB, kRadN, kCap> {
+    typename Fast<T>::vec4 nbr_p[kNB][kCap];       // (v_centre - v_partner)/r, and its component along the unit vector: dr / r
+    T nbr_dfc[kNB][kCap];                          // f_C'(r) dr, dr = change of the distance along the vectors (= nbr_p.w r)
     typename Fast<T>::vec2 rad_ab[kRadN];         // radial entries: f_C' dr, and -2 eta f_C dr
     T rec2[64][12];                               // phase-1 records: dA_0..7, H_0..3
 };
 
-// LDS working set of one wavefront, for batches of kNB centres
-template <typename T, bool kJvp = false, int kNB = kFB, int kRadN = 64>
+// LDS working set of one wavefront, for batches of kNB centres with at most kCap angular partners each
+template <typename T, bool kJvp = false, int kNB = kFB, int kRadN = 64, int kCap = kCapA>
 struct __align__(16) FwdWaveLds {
     static constexpr int kCentres = kNB;
-    typename Fast<T>::vec4 nbr[kNB][kCapA];    // unit vector (centre minus partner)/r, and r
-    T nbr_fc[kNB][kCapA];                      // f_C(r, A_Rc)
+    static constexpr int kCapacity = kCap;
+    static constexpr int kSegments = kNB * kNumPairBlocks;      // a segment per (centre, type pair) at most
+    typename Fast<T>::vec4 nbr[kNB][kCap];     // unit vector (centre minus partner)/r, and r
+    T nbr_fc[kNB][kCap];                       // f_C(r, A_Rc)
     typename Fast<T>::vec2 rad[kRadN];        // (r, f_C(r, R_Rc)) of the radial partners of a scan step's centres
     T rec[64][12];                            // phase-1 records: A_0..7, G_0..3
-    SegDesc seg[64];                          // non-empty segments of the batch, in order
-    unsigned long long segrow[64];            // where each of them puts its 32 output values
+    SegDesc seg[kSegments];                   // non-empty segments of the batch, in order
+    unsigned long long segrow[kSegments];     // where each of them puts its 32 output values (then: the empty blocks' addresses)
     unsigned bits[bit_words(kNB)];            // bit per triple slot: a segment starts here
     int nA[kNB][4];                            // angular partners per type, per centre of the batch
-    FwdJvpLds<T, kJvp, kNB, kRadN> jvp;
+    FwdJvpLds<T, kJvp, kNB, kRadN, kCap> jvp;
 };
 
 // Padding slots of phase 1 read entry 0 of centre 0's list whatever it holds; their products are cancelled by a
 // zero radial factor, which needs every other factor finite.  Entry 0 is either a partner written by a scan or
 // what this writes once per wavefront before the first batch.
-template <typename T, bool kJvp, int kNB, int kRadN>
-__device__ __forceinline__ void fwd_lds_init(FwdWaveLds<T, kJvp, kNB, kRadN>& S, int lane)
+template <typename T, bool kJvp, int kNB, int kRadN, int kCap>
+__device__ __forceinline__ void fwd_lds_init(FwdWaveLds<T, kJvp, kNB, kRadN, kCap>& S, int lane)
 {
     if (lane == 0) {
         S.nbr[0][0] = Fast<T>::make4(T(0), T(0), T(0), T(0));
         S.nbr_fc[0][0] = T(0);
         if constexpr (kJvp) {
             S.jvp.nbr_p[0][0] = Fast<T>::make4(T(0), T(0), T(0), T(0));
-            S.jvp.nbr_d[0][0] = Fast<T>::make2(T(0), T(0));
+            S.jvp.nbr_dfc[0][0] = T(0);
         }
     }
 }
@@ -58,8 +59,8 @@ __device__ __forceinline__ void fwd_lds_init(FwdWaveLds<T, kJvp, kNB, kRadN>& S,
 // segment's records of A_t G_s is the product of an 8 x K by a K x 4 matrix, and v_mfma_f32_16x16x4_f32 takes four
 // records (K = 4) per instruction, using an 8 x 4 corner of its 16 x 16 result.  The variant exists to be measured
 // against the vector form; the launcher selects it on request only.
-template <bool kMatrixPhase2, typename T, bool kJvp, int kNB, int kRadN, typename RowOfCentre>
-__device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB, kRadN>& S, const LaneConsts<T>& L, int lane, int nb,
+template <bool kMatrixPhase2, typename T, bool kJvp, int kNB, int kRadN, int kCap, typename RowOfCentre>
+__device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB, kRadN, kCap>& S, const LaneConsts<T>& L, int lane, int nb,
                                                   RowOfCentre row_of_centre)
 {
     static_assert(kNB * kNumPairBlocks <= 64, "one segment-table lane per (centre, type pair)");
@@ -93,8 +94,8 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB, kRadN
         const int ob = sel4(seg_bt, 0, nn.x, nn.x + nn.y, nn.x + nn.y + nn.z);
         const bool same = seg_a == seg_bt;
         cnt = same ? (__mul24(na, na - 1) >> 1) : __mul24(na, nbt);
-        mine.aj = static_cast<unsigned>((seg_b * kCapA + oa) * static_cast<int>(sizeof(vec4)));
-        mine.ak = static_cast<unsigned>((seg_b * kCapA + ob) * static_cast<int>(sizeof(vec4)));
+        mine.aj = static_cast<unsigned>((seg_b * kCap + oa) * static_cast<int>(sizeof(vec4)));
+        mine.ak = static_cast<unsigned>((seg_b * kCap + ob) * static_cast<int>(sizeof(vec4)));
         // floor(2^15 / n_a) + 1 (the reciprocal is within an ulp, and 2^15 / n_a is never that close below an integer)
         const unsigned magic = static_cast<unsigned>(32768.0f * __builtin_amdgcn_rcpf(static_cast<float>(max(na, 1)))) + 1u;
         mine.div = magic | (static_cast<unsigned>(na) << 16) | (same ? (1u << 24) : 0u);
@@ -183,11 +184,14 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB, kRadN
         const T s = Fast<T>::sqrt_(fmin(fmax(cx * cx + cy * cy + cz * cz, T(0)), T(1)));
         T Af[8], dAf[8];
         T dc = T(0), cot = T(0);
+        T drj = T(0), drk = T(0);          // change of the two distances along the vectors
         if constexpr (kJvp) {
             // d cos = u_k.p_j + u_j.p_k - c (alpha_j + alpha_k), p = (v_i - v_partner)/r, alpha = u.p
             const char* const p_bytes = reinterpret_cast<const char*>(&S.jvp.nbr_p[0][0]);
             const vec4 pj = *reinterpret_cast<const vec4*>(p_bytes + bj), pk = *reinterpret_cast<const vec4*>(p_bytes + bk);
             dc = (vk.x * pj.x + vk.y * pj.y + vk.z * pj.z) + (vj.x * pk.x + vj.y * pk.y + vj.z * pk.z) - c * (pj.w + pk.w);
+            drj = pj.w * vj.w;
+            drk = pk.w * vk.w;
             cot = c * s * Fast<T>::rcp(s * s + Real<T>::kCotEps);     // c/s, zero on the line (cusp of the angle)
         }
         T bases[8];
@@ -213,10 +217,10 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB, kRadN
         T Gf[4], Hf[4];
         T dP = T(0), drho = T(0);
         if constexpr (kJvp) {
-            const char* const d_bytes = reinterpret_cast<const char*>(&S.jvp.nbr_d[0][0]);
-            const vec2 dj = *reinterpret_cast<const vec2*>(d_bytes + bj / 2u), dk = *reinterpret_cast<const vec2*>(d_bytes + bk / 2u);
-            dP = ok ? T(0.0078125) * (dj.x * fk + fj * dk.x) : T(0);
-            drho = T(0.5) * (dj.y + dk.y);
+            const char* const d_bytes = reinterpret_cast<const char*>(&S.jvp.nbr_dfc[0][0]);
+            const T dj = *reinterpret_cast<const T*>(d_bytes + bj / kPerT), dk = *reinterpret_cast<const T*>(d_bytes + bk / kPerT);
+            dP = ok ? T(0.0078125) * (dj * fk + fj * dk) : T(0);
+            drho = T(0.5) * (drj + drk);
         }
 #pragma unroll
         for (int sidx = 0; sidx < 4; ++sidx) {

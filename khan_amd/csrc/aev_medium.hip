@@ -296,7 +296,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                                 S.nbr[b][p] = Fast<T>::make4(dx * inv, dy * inv, dz * inv, r);
                                 S.nbr_fc[b][p] = fc;
                                 S.jvp.nbr_p[b][p] = Fast<T>::make4(wx * inv, wy * inv, wz * inv, rd * inv);
-                                S.jvp.nbr_d[b][p] = Fast<T>::make2(dfc * rd, rd);
+                                S.jvp.nbr_dfc[b][p] = dfc * rd;
                                 if constexpr (kLarge) M.atype[wave][p] = static_cast<unsigned char>(tj);
                             }
                         }
@@ -361,14 +361,14 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                     const bool haveE = lane < min(posA, kCapA);
                     int tA = -1;
                     vec4 nb = Fast<T>::make4(T(0), T(0), T(0), T(0)), np = nb;
-                    vec2 nd = Fast<T>::make2(T(0), T(0));
+                    T nd = T(0);
                     T fc = T(0);
                     if (haveE) {
                         nb = S.nbr[b][lane];
                         fc = S.nbr_fc[b][lane];
                         if constexpr (kJvp) {
                             np = S.jvp.nbr_p[b][lane];
-                            nd = S.jvp.nbr_d[b][lane];
+                            nd = S.jvp.nbr_dfc[b][lane];
                             tA = M.atype[wave][lane];
                         } else {
                             tA = static_cast<int>(fc);
@@ -387,7 +387,7 @@ __global__ __launch_bounds__(256) void aev_fwd_medium_kernel(
                         S.nbr_fc[b][dest] = fc;
                         if constexpr (kJvp) {
                             S.jvp.nbr_p[b][dest] = np;
-                            S.jvp.nbr_d[b][dest] = nd;
+                            S.jvp.nbr_dfc[b][dest] = nd;
                         }
                     }
                 }

@@ -57,7 +57,10 @@ void aev_fwd_small_kernel(
     typedef typename Fast<T>::vec2 vec2;
     // centres per batch: six; four in the float Jacobian-vector kernel, whose working set then lets ten wavefronts share a CU instead of eight
     constexpr int kNB = (kJvp && sizeof(T) == 4) ? 4 : kFB;
-    __shared__ FwdWaveLds<T, kJvp, kNB, kRadSlots> lds_all[kWavesPerBlock];
+    // angular partners kept per centre: 32; 28 in the float Jacobian-vector kernel, whose working set then is 13.4 KB
+    // and twelve wavefronts share a CU (a centre with more goes to the general routine, as above 32 elsewhere)
+    constexpr int kCap = (kJvp && sizeof(T) == 4) ? 28 : kCapA;
+    __shared__ FwdWaveLds<T, kJvp, kNB, kRadSlots, kCap> lds_all[kWavesPerBlock];
     const int lane = threadIdx.x & 63;
     const int wave = kWavesPerBlock == 1 ? 0 : uniform(threadIdx.x >> 6);    // a constant LDS base with one wavefront per workgroup
     const int slot = blockIdx.x * kWavesPerBlock + wave;
@@ -66,7 +69,7 @@ void aev_fwd_small_kernel(
     const int n = uniform(MACs[mol]);
     const int off = uniform(MOs[mol]);
     if (n <= 0 || n > max_atoms) return;          // larger molecules belong to other kernels (max_atoms <= 64)
-    FwdWaveLds<T, kJvp, kNB, kRadSlots>& S = lds_all[wave];
+    FwdWaveLds<T, kJvp, kNB, kRadSlots, kCap>& S = lds_all[wave];
     const LaneConsts<T> L = lane_consts<T>(lane);
     const unsigned long long lane_bit = 1ull << lane;
     const unsigned long long lt_mask = lane_bit - 1ull;
@@ -120,7 +123,6 @@ void aev_fwd_small_kernel(
         vx = lane_push(dest, vx);
         vy = lane_push(dest, vy);
         vz = lane_push(dest, vz);
-        S.jvp.vel[lane] = Fast<T>::make4(vx, vy, vz, T(0));
     }
     auto row_of = [&](int sorted_lane) -> T* {     // sorted_lane is wave-uniform
         const unsigned lo = static_cast<unsigned>(lane_read(rp_lo, sorted_lane));
@@ -166,6 +168,12 @@ void aev_fwd_small_kernel(
     // the sorted atoms stay in the lanes' registers: the partner this lane tests in every scan step, once; the
     // step's centres by lane exchange
     const T xj = lane_fetch(x, jl << 2), yj = lane_fetch(y, jl << 2), zj = lane_fetch(z, jl << 2);
+    T vxj = T(0), vyj = T(0), vzj = T(0);
+    if constexpr (kJvp) {
+        vxj = lane_fetch(vx, jl << 2);
+        vyj = lane_fetch(vy, jl << 2);
+        vzj = lane_fetch(vz, jl << 2);
+    }
 
     fwd_lds_init(S, lane);
     wave_lds_fence();
@@ -196,14 +204,14 @@ void aev_fwd_small_kernel(
             const bool inR = valid && (r < kR_Rc_f) && (!kJvp || r > T(0));
             const bool inA = valid && (r < kA_Rc_f) && (!kJvp || r > T(0));
             const unsigned long long mR = wave_ballot(inR), mA = wave_ballot(inA);
-            const bool fits = popc64(mA & sub_mask) <= kCapA;
+            const bool fits = popc64(mA & sub_mask) <= kCap;
             T wx = T(0), wy = T(0), wz = T(0), rd = T(0);        // v_centre - v_partner, and d r along it
             const T inv = Fast<T>::rcp(r);
             if constexpr (kJvp) {
-                const vec4 vi = S.jvp.vel[centre_ok ? i : 0], vjv = S.jvp.vel[jl];
-                wx = vi.x - vjv.x;
-                wy = vi.y - vjv.y;
-                wz = vi.z - vjv.z;
+                // the incoming vectors stay in the lanes like the positions: the partner's once, the centre's by lane exchange
+                wx = lane_fetch(vx, ci) - vxj;
+                wy = lane_fetch(vy, ci) - vyj;
+                wz = lane_fetch(vz, ci) - vzj;
                 rd = (dx * wx + dy * wy + dz * wz) * inv;
             }
             if (inR) {
@@ -226,7 +234,7 @@ void aev_fwd_small_kernel(
                     Fast<T>::cutoff_grad(r, static_cast<T>(kA_Rc_f), fc, dfc);
                     S.nbr_fc[cb][pos] = fc;
                     S.jvp.nbr_p[cb][pos] = Fast<T>::make4(wx * inv, wy * inv, wz * inv, rd * inv);
-                    S.jvp.nbr_d[cb][pos] = Fast<T>::make2(dfc * rd, rd);
+                    S.jvp.nbr_dfc[cb][pos] = dfc * rd;
                 } else {
                     S.nbr_fc[cb][pos] = Fast<T>::cutoff(r, static_cast<T>(kA_Rc_f));
                 }
@@ -240,7 +248,7 @@ void aev_fwd_small_kernel(
             if (cl_on) {
                 const int cb = b0 + cl_g;
                 cntR = popc64(mR & cl_mask);
-                if (cb < nb) S.nA[cb][cl_a] = (popc64(mA & cl_sub) <= kCapA) ? popc64(mA & cl_mask) : 0;
+                if (cb < nb) S.nA[cb][cl_a] = (popc64(mA & cl_sub) <= kCap) ? popc64(mA & cl_mask) : 0;
             }
             // largest radial count of each type over the groups of this step (lanes 0..15 hold them)
             int mx = cntR;
