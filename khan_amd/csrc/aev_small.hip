@@ -42,7 +42,7 @@ constexpr int kRadSlots = 96;
 // With kJvp the kernel computes the Jacobian-vector product instead (featurize_grad_inverse): every term of
 // the forward sums is replaced by its derivative along the per-atom vectors (VX, VY, VZ).
 // float: 4 wavefronts per SIMD (LDS 9.8 KB, <= 128 VGPRs; the kernel loses a fifth of its speed at three);
-// float kJvp: 3 (<= 168 VGPRs; its LDS, 16.2 KB, lets ten wavefronts share a CU); double: 2 (LDS 19 KB); double kJvp: 1.
+// float kJvp: 3 (<= 168 VGPRs; its LDS, 13.4 KB, lets twelve wavefronts share a CU); double: 2 (LDS 17 KB); double kJvp: 1.
 template <typename T, bool kJvp, bool kMatrixPhase2 = false>
 __global__ __launch_bounds__(64 * kWavesPerBlock)
 __attribute__((amdgpu_waves_per_eu((kJvp && sizeof(T) == 4) ? 3 : (sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1), (kJvp && sizeof(T) == 4) ? 3 : (sizeof(T) == 4 ? 4 : 2) / (kJvp ? 2 : 1))))
@@ -55,7 +55,7 @@ void aev_fwd_small_kernel(
 {
     typedef typename Fast<T>::vec4 vec4;
     typedef typename Fast<T>::vec2 vec2;
-    // centres per batch: six; four in the float Jacobian-vector kernel, whose working set then lets ten wavefronts share a CU instead of eight
+    // centres per batch: six; four in the float Jacobian-vector kernel (with kCap below: twelve wavefronts per CU)
     constexpr int kNB = (kJvp && sizeof(T) == 4) ? 4 : kFB;
     // angular partners kept per centre: 32; 28 in the float Jacobian-vector kernel, whose working set then is 13.4 KB
     // and twelve wavefronts share a CU (a centre with more goes to the general routine, as above 32 elsewhere)
