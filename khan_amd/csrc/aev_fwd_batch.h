@@ -314,9 +314,11 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB, kRadN
             ph = &S.jvp.rec2[L.half][8 + ang_s];
         }
         // float: the four lanes of a quad (same theta_t) each read A_t of one of four consecutive pairs, and the
-        // product takes it from the quad lane that holds it: one LDS read of A serves four pairs
-        constexpr bool kQuadA = sizeof(T) == 4 && !kJvp;
+        // product takes it from the quad lane that holds it: one LDS read of A (and of dA_t) serves four pairs
+        constexpr bool kQuadA = sizeof(T) == 4;
         const T* pa4 = &S.rec[L.half + 2 * ang_s][ang_t];
+        const T* pda4 = pa4;
+        if constexpr (kJvp) pda4 = &S.jvp.rec2[L.half + 2 * ang_s][ang_t];
         unsigned long long mm = starts;
         if (base == 0) {            // the batch's first segment opens here; nothing to close
             cur_lo = static_cast<unsigned>(lane_read(static_cast<int>(d_row_lo), 0));
@@ -324,19 +326,23 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB, kRadN
             mm &= ~1ull;
         }
         struct Group {
-            T a[8], g[8], da[kJvp ? 8 : 1], h[kJvp ? 8 : 1];
+            T a[kQuadA ? 2 : 8], g[8], da[!kJvp ? 1 : kQuadA ? 2 : 8], h[kJvp ? 8 : 1];
         };
         auto load8 = [&](int q0, Group& v) {
             if constexpr (kQuadA) {
                 v.a[0] = pa4[q0 * 24];
                 v.a[1] = pa4[(q0 + 4) * 24];
+                if constexpr (kJvp) {
+                    v.da[0] = pda4[q0 * 24];
+                    v.da[1] = pda4[(q0 + 4) * 24];
+                }
             }
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
                 if constexpr (!kQuadA) v.a[u] = pa[(q0 + u) * 24];
                 v.g[u] = pg[(q0 + u) * 24];
                 if constexpr (kJvp) {
-                    v.da[u] = pda[(q0 + u) * 24];
+                    if constexpr (!kQuadA) v.da[u] = pda[(q0 + u) * 24];
                     v.h[u] = ph[(q0 + u) * 24];
                 }
             }
@@ -355,7 +361,8 @@ __device__ __forceinline__ void fwd_angular_batch(FwdWaveLds<T, kJvp, kNB, kRadN
                     cur_hi = static_cast<unsigned>(lane_read(static_cast<int>(d_row_hi), first));
                     acc = T(0);
                 }
-                if constexpr (kJvp) acc = fma(v.da[u], v.g[u], fma(v.a[u], v.h[u], acc));
+                if constexpr (kJvp && kQuadA) acc = fma_quad(v.da[u >> 2], u & 3, v.g[u], fma_quad(v.a[u >> 2], u & 3, v.h[u], acc));
+                else if constexpr (kJvp) acc = fma(v.da[u], v.g[u], fma(v.a[u], v.h[u], acc));
                 else if constexpr (kQuadA) acc = fma_quad(v.a[u >> 2], u & 3, v.g[u], acc);
                 else acc = fma(v.a[u], v.g[u], acc);
             }
