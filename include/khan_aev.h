@@ -55,7 +55,7 @@ const char *khan_last_hip_error(void);
  * the reference's gradient runs on the CPU in a fixed order, kernel_cpu.cpp:217-366).  With 1, khan_featurize_grad_*
  * sums the forces of molecules of 33..256 atoms (float32; 65..256 in float64) in on-chip memory in a fixed order and
  * stores every gradient once: the same bits on every run, no atomics, and no requirement on the kind of memory the
- * gradient arrays live in.  Costs 9 % of that kernel's speed in float32 (it runs three workgroups per CU instead
+ * gradient arrays live in.  Costs 11 % of that kernel's speed in float32 (it runs three workgroups per CU instead
  * of four) and more in float64 (one instead of two).  Not covered: molecules of more than 256 atoms, centres with more than 64
  * partners inside the angular cutoff, and upstream buckets that are not 16-byte aligned (the general kernels, atomics). */
 int khan_set_reproducible_gradients(int on);
