@@ -172,10 +172,11 @@ template <typename T> struct __align__(16) ChargeTile<T, false> {
     typename Fast<T>::vec4 in[kMediumMaxAtoms];     // x, y, z, q
     T wpart[4];
 };
+// (in double these are 40,960 bytes, a quarter of a compute unit's LDS to the byte: the wavefronts' partial energies
+// go into the tile's first entry once the rounds are over, not into four words more that would cost the fourth workgroup)
 template <typename T> struct __align__(16) ChargeTile<T, true> {
     typename Fast<T>::vec4 in[kMediumMaxAtoms];     // x, y, z, q
     typename Fast<T>::vec4 acc[4][kMediumMaxAtoms]; // partner side, per wavefront: force x, y, z and dE/dq
-    T wpart[4];
 };
 
 template <typename T, bool kDamped, bool kGrad>
@@ -234,12 +235,19 @@ __global__ __launch_bounds__(256) void charge_tile_kernel(
                 wave_lds_fence();                            // the next round may touch slots written here
             }
         }
+        T* wpart;
+        if constexpr (kGrad) {
+            wpart = reinterpret_cast<T*>(&S.in[0]);
+            if (E) __syncthreads();          // every wavefront has finished its rounds: the tile is free
+        } else {
+            wpart = S.wpart;
+        }
         if (!kGrad || E) {
             e_acc = wave_sum(e_acc);
-            if (lane == 0) S.wpart[wave] = e_acc;
+            if (lane == 0) wpart[wave] = e_acc;
         }
         __syncthreads();
-        if ((!kGrad || E) && i == 0) E[mol] = K * ((S.wpart[0] + S.wpart[1]) + (S.wpart[2] + S.wpart[3]));
+        if ((!kGrad || E) && i == 0) E[mol] = K * ((wpart[0] + wpart[1]) + (wpart[2] + wpart[3]));
         if constexpr (kGrad) {
             if (have) {
                 const T gK = grads[mol] * K;
