@@ -368,7 +368,7 @@ def main():
 
 
 HEADLINE = "organic65536"
-# BASELINE.json's configurations 3 and 4 and grad-inverse, reported beside the headline configuration (1 + 2)
+# the float64 + charges, dense-box and grad-inverse configurations, reported beside the headline configuration
 EXTRA_CONFIGS = ("organic16384_f64", "boxes4096", "grad_inverse65536", "charges_boxes4096_f64")
 
 
